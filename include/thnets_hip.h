@@ -1,0 +1,429 @@
+/*
+ * thnets_hip.h -- C ABI of the MI355X (gfx950) engine for thnets.
+ *
+ * Three layers, all plain C (extern "C" when included from C++/HIP):
+ *
+ *  1. The thnets tensor / module / network structures, laid out field for
+ *     field like the reference's default (non -DLOWP, non -DOPENCL) build so
+ *     that a `struct module[]` built by an existing thnets caller can be
+ *     handed to this library unchanged (thnets.h:104-120, 122-130, 140-232,
+ *     250-336, 401-407, 571-580).
+ *  2. The high level calls a thnets user already knows (thnets.h:582-598)
+ *     plus the new constructors THCreateHipNetwork / THCreateHipLowpNetwork
+ *     that sit beside THCreateCudaNetwork / THCreateLowpNetwork
+ *     (thapi.c:730-742, 784-796).
+ *  3. The kernel level entry points (thhip_*): plain device pointers and
+ *     sizes, one per hand written HIP kernel.  These are what the module
+ *     glue calls and what a foreign-function binding would bind.
+ *
+ * Every entry point that touches the GPU aborts through THError when a HIP
+ * call fails; there is no CPU fallback in this library.
+ */
+#ifndef THNETS_HIP_H
+#define THNETS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ */
+/* 1. thnets ABI                                                       */
+/* ------------------------------------------------------------------ */
+
+/* thnets.h:16-22 */
+enum therror {
+	ERR_OPENFILE = -1,
+	ERR_READFILE = -2,
+	ERR_NOTIMPLEMENTED = -3,
+	ERR_CORRUPTED = -4,
+	ERR_WRONGOBJECT = -5
+};
+
+/* thnets.h:104-108.  mustfree: 0 borrowed, 1 free(), 2 cudaFree (unused
+ * here), 3 OpenCL (unused here), 4 = device memory owned by this engine. */
+typedef struct THFloatStorage {
+	float *data;
+	int nref, mustfree;
+} THFloatStorage;
+
+#define TH_MUSTFREE_HIP 4
+
+/* thnets.h:110-120 (default build: no sub/mult members). */
+typedef struct THFloatTensor {
+	long size[4];
+	long stride[4];
+	int nDimension;
+	THFloatStorage *storage;
+	long storageOffset;
+} THFloatTensor;
+
+/* Per-module parameter blocks, thnets.h:122-248.  Only the members of the
+ * union that this engine reads are spelled out; the union is padded to the
+ * reference's size so that modules[i] indexes identically. */
+struct SpatialConvolution {
+	THFloatTensor *bias, *weight, *finput;
+	int dW, dH, padW, padH, kW, kH, nInputPlane, nOutputPlane;
+	int refl_pad;
+	int padW2, padH2;
+	int autopad;
+	int dlH, dlW;
+};
+
+struct SpatialMaxPooling {
+	int padW, padH, dW, dH, kW, kH, ceil_mode;
+	int iwidth, iheight;
+	THFloatTensor *indices;
+	int padW2, padH2;
+};
+
+struct SpatialAveragePooling {
+	int padW, padH, dW, dH, kW, kH, ceil_mode;
+	int iwidth, iheight, count_include_pad;
+	int padW2, padH2;
+};
+
+struct Linear {
+	THFloatTensor *bias, *weight, *addBuffer;
+	int commute;
+};
+
+struct Threshold {
+	float threshold, val, alpha;
+	int inplace;
+};
+
+struct View {
+	int numElements, nDimension;
+	long size[4];
+};
+
+struct Dropout {
+	float p;
+	int inplace, v2;
+};
+
+struct SpatialBatchNormalization {
+	THFloatTensor *running_mean, *running_var, *weight, *bias;
+	double eps;
+};
+
+struct network;
+
+struct Sequential {
+	struct network *net;
+};
+
+struct Concat {
+	struct network *net;
+	int dimension;
+};
+
+/* thnets.h:250-288 -- numeric values are part of the ABI. */
+enum moduletype {
+	MT_Nil,
+	MT_SpatialConvolutionMM,
+	MT_SpatialConvolutionVirtMM,
+	MT_SpatialConvolution,
+	MT_SpatialMaxPooling,
+	MT_SpatialAveragePooling,
+	MT_Linear,
+	MT_SoftMax,
+	MT_Threshold,
+	MT_View,
+	MT_Dropout,
+	MT_SpatialZeroPadding,
+	MT_Reshape,
+	MT_Normalize,
+	MT_SpatialFullConvolution,
+	MT_SpatialMaxUnpooling,
+	MT_SpatialBatchNormalization,
+	MT_Sequential,
+	MT_Concat,
+	MT_ConcatTable,
+	MT_JoinTable,
+	MT_CAddTable,
+	MT_CSubTable,
+	MT_PReLU,
+	MT_Identity,
+	MT_Padding,
+	MT_LogSoftMax,
+	MT_Slice,
+	MT_Cmax,
+	MT_Upsample,
+	MT_LSTM,
+	MT_GRU,
+	MT_Squeeze,
+	MT_Unsqueeze,
+	MT_Sigmoid,
+	MT_Tanh,
+	MT_Transpose
+};
+
+#define MAXMODULEINPUTS 16
+#define TH_MODULE_UNION_BYTES 80
+
+/* thnets.h:292-336 */
+struct module {
+	int type;
+	THFloatTensor *(*updateOutput)(struct module *m, THFloatTensor *in);
+	void (*nnfree)(struct module *m);
+	THFloatTensor *output;
+	struct network *net;
+	void *nnmodule;			/* struct nnmodule * of the .t7 loader */
+	char *outputname;
+	int ninputs;
+	int inputs[MAXMODULEINPUTS];
+	union {
+		struct SpatialConvolution SpatialConvolution;
+		struct SpatialMaxPooling SpatialMaxPooling;
+		struct SpatialAveragePooling SpatialAveragePooling;
+		struct Linear Linear;
+		struct Threshold Threshold;
+		struct View View;
+		struct Dropout Dropout;
+		struct SpatialBatchNormalization SpatialBatchNormalization;
+		struct Sequential Sequential;
+		struct Concat Concat;
+		struct Sequential ConcatTable;
+		char abi_pad[TH_MODULE_UNION_BYTES];
+	};
+};
+
+/* thnets.h:401; the two HIP engines are appended. */
+enum {
+	ENGINE_CPU, ENGINE_CUDA, ENGINE_OPENCL, ENGINE_OPENCLINIT, ENGINE_LOWP,
+	ENGINE_HIP, ENGINE_HIPLOWP
+};
+
+/* thnets.h:403-407 */
+struct network {
+	int nelem, engine;
+	struct module *modules;
+};
+
+/* thnets.h:571-580 */
+typedef struct thnetwork {
+	void *netobj;			/* struct thobject * */
+	void *statobj;			/* struct thobject * */
+	struct network *net;
+	void *pynet;			/* struct pyelement * */
+	void **allpynodes;		/* struct pyelement ** */
+	THFloatTensor *out;
+	float mean[3], std[3];
+} THNETWORK;
+
+/* Tensor helpers with the reference's semantics (thbasic.c:17-460). */
+void THError(const char *fmt, ...);
+THFloatTensor *THFloatTensor_new(void);
+THFloatStorage *THFloatStorage_new(long size);
+THFloatStorage *THFloatStorage_newwithbuffer(void *buffer);
+THFloatTensor *THFloatTensor_newWithStorage1d(THFloatStorage *storage, long storageOffset, long size0, long stride0);
+THFloatTensor *THFloatTensor_newWithStorage2d(THFloatStorage *storage, long storageOffset, long size0, long stride0, long size1, long stride1);
+THFloatTensor *THFloatTensor_newWithTensor(THFloatTensor *tensor);
+float *THFloatTensor_data(THFloatTensor *tensor);
+long THFloatTensor_nElement(THFloatTensor *t);
+void THFloatTensor_resize(THFloatTensor *t, long *size, int nDimension);
+void THFloatTensor_resize4d(THFloatTensor *t, long size0, long size1, long size2, long size3);
+void THFloatTensor_resize3d(THFloatTensor *t, long size0, long size1, long size2);
+void THFloatTensor_resize2d(THFloatTensor *t, long size0, long size1);
+void THFloatTensor_resize1d(THFloatTensor *t, long size0);
+void THFloatTensor_set(THFloatTensor *tdst, THFloatTensor *tsrc);
+void THFloatTensor_free(THFloatTensor *t);
+
+/* ------------------------------------------------------------------ */
+/* 2. High level API                                                   */
+/* ------------------------------------------------------------------ */
+
+/* thapi.c:335-361 */
+void THInit(void);
+/* thapi.c:237-242.  `in` must live where the network's engine lives: a
+ * device tensor for ENGINE_HIP / ENGINE_HIPLOWP. */
+THFloatTensor *THForward(THNETWORK *net, THFloatTensor *in);
+/* thapi.c:363-450.  Normalises the caller's buffer in place with
+ * mean/std, uploads, runs, downloads; *result is library owned. */
+int THProcessFloat(THNETWORK *network, float *data, int batchsize, int width, int height, int nplanes,
+	float **result, int *outwidth, int *outheight);
+/* thapi.c:452-563.  8-bit HWC images; conversion + normalisation run on the
+ * device for the HIP engines. */
+int THProcessImages(THNETWORK *network, unsigned char **images, int batchsize, int width, int height, int stride,
+	float **result, int *outwidth, int *outheight, int bgr);
+/* thapi.c:642-690 */
+void THMakeSpatial(THNETWORK *network, int size);
+/* thapi.c:692-728.  Only switches the module type tag (MM <-> VirtMM);
+ * this library carries no direct-convolution path, mm_type 0 is refused. */
+int THUseSpatialConvolutionMM(THNETWORK *network, int mm_type);
+/* thapi.c:601-635 (engine networks only: frees device state). */
+void THFreeNetwork(THNETWORK *network);
+/* thapi.c:637-640 */
+int THLastError(void);
+/* thapi.c:12; th_profile makes forward() print per-module seconds. */
+extern int th_debug, th_profile, th_minmax;
+extern double th_convtot, th_convflops;
+
+/* New: the MI355X engine.  Same shape as THCreateCudaNetwork
+ * (thapi.c:730-742): returns a new THNETWORK whose modules own device
+ * copies of every weight; the source network may be freed afterwards.
+ * Conv+Threshold pairs are fused; Linear becomes a 1x1 convolution
+ * (cudnn_basic.c:244-265). */
+THNETWORK *THCreateHipNetwork(THNETWORK *net);
+/* New: counterpart of THCudaHalfFloat (thapi.c:744-755).  0 = fp32,
+ * 1 = fp16 storage + fp16 MFMA, 2 = bf16 storage + bf16 MFMA.  Read at
+ * engine creation.  Returns 0, or ERR_NOTIMPLEMENTED for other values. */
+int THHipHalfFloat(int enable);
+/* New: the uint8 engine on the GPU, counterpart of THCreateLowpNetwork
+ * (thapi.c:784-796, lowp_basic.c:133-212): activations quantised to
+ * [-range/2, range/2) in 255 steps, int8 MFMA GEMM with gemmlowp offsets
+ * and (multiplier, shift) requantisation (lowp_basic.c:299-321). */
+THNETWORK *THCreateHipLowpNetwork(THNETWORK *net, float range);
+/* Device <-> host tensors (cudnn_basic.c:64-97 are the CUDA analogues). */
+THFloatTensor *THHipTensor_newFromFloatTensor(THFloatTensor *t);
+THFloatTensor *THFloatTensor_newFromHipTensor(THFloatTensor *t);
+/* Copies module `idx`'s current output of an engine network to the host as
+ * float (half / uint8 activations are widened; uint8 codes are returned as
+ * code values, not de-quantised).  Returns element count; *dst is malloc'd. */
+long THHipNetwork_copyModuleOutput(THNETWORK *net, int idx, float **dst, long size[4], int *ndim);
+/* Quantisation (mult, sub) of module `idx`'s output in a HIPLOWP network. */
+int THHipNetwork_getModuleQuant(THNETWORK *net, int idx, float *mult, float *sub);
+
+/* Drop-in for the reference's only call into gemmlowp (gemm8.cc:4-17,
+ * declared lowp_basic.c:290-297): host pointers in and out, the GEMM and
+ * requantisation run on the GPU.  Only the all-"transposed" (row-major)
+ * form the reference uses is accepted. */
+void lowpgemm(const int is_a_transposed, const int is_b_transposed, const int is_c_transposed,
+	const int m, const int n, const int k,
+	const unsigned char *a, const unsigned char *b, unsigned char *c,
+	const int lda, const int ldb, const int ldc,
+	const int a_offset, const int b_offset, const int c_offset,
+	const int c_mult, const int c_shift);
+
+/* ------------------------------------------------------------------ */
+/* 3. Kernel level C ABI (device pointers unless stated)               */
+/* ------------------------------------------------------------------ */
+
+/* Element types of device activations / weights. */
+enum thhip_dtype { THHIP_F32 = 0, THHIP_F16 = 1, THHIP_BF16 = 2, THHIP_U8 = 3 };
+
+/* Runtime plumbing. */
+int thhip_device_count(void);
+void *thhip_malloc(size_t bytes);
+void thhip_free(void *p);
+void thhip_memcpy_h2d(void *dst, const void *src, size_t bytes);
+void thhip_memcpy_d2h(void *dst, const void *src, size_t bytes);
+void thhip_memcpy_d2d(void *dst, const void *src, size_t bytes);
+void thhip_memset(void *dst, int value, size_t bytes);
+void thhip_sync(void);
+/* Events on the engine's stream: slots 0..63. thhip_event_ms(a,b) syncs b. */
+void thhip_event_record(int slot);
+float thhip_event_ms(int slot_start, int slot_stop);
+/* Per-kernel-family accumulated time (ms) and launch count measured with
+ * events around every launch while profiling is on (family ids below). */
+enum thhip_family { THHIP_FAM_CONV = 0, THHIP_FAM_GEMV = 1, THHIP_FAM_CONV_I8 = 2, THHIP_FAM_OTHER = 3, THHIP_FAM_COUNT = 4 };
+void thhip_profile_enable(int on);
+void thhip_profile_reset(void);
+void thhip_profile_get(int family, double *ms, long *launches, double *work);
+
+/* Weight packing for the implicit-GEMM convolution: row-major
+ * [Co][K=Ci*kH*kW] (SpatialConvolutionMM.c:141-144) -> the K-chunked,
+ * M-interleaved layout the kernel streams.  Returns a device buffer. */
+void *thhip_conv_pack_weight(const float *w_host, int Co, int K, int dtype);
+size_t thhip_conv_packed_bytes(int Co, int K, int dtype);
+
+/* Replaces nn_SpatialConvolutionMM_updateOutput's per-image
+ * im2col + sgemm + bias (SpatialConvolutionMM.c:75-109, 126-225) and, when
+ * `act` != 0, the following nn_Threshold_updateOutput
+ * (Threshold.c:38-63): y = x > thr ? x : val applied to the sum.
+ * x: [B,Ci,H,W], y: [B,Co,oH,oW], both NCHW contiguous in `dtype`;
+ * wpacked from thhip_conv_pack_weight; bias fp32 [Co] or NULL. */
+void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype);
+
+/* Replaces nn_Linear_updateOutput's 1-D branch (Linear.c:86-90 ->
+ * thbasic.c:713-741 -> sgemv.c:48-105): y = bias + W x, W row-major
+ * [nOut][nIn] fp32/fp16/bf16, optional fused threshold. */
+void thhip_gemv(const void *x, const void *w, const float *bias, void *y,
+	int nIn, int nOut, int act, float thr, float val, int dtype);
+
+/* Replaces nn_Threshold_updateOutput (Threshold.c:38-63), out of place or
+ * in place (y == x).  alpha != 0 selects the LeakyReLU branch. */
+void thhip_threshold(const void *x, void *y, long n, float thr, float val, float alpha, int inplace, int dtype);
+
+/* Replaces nn_SpatialMaxPooling_updateOutput (SpatialMaxPooling.c:168-247)
+ * and Lowp_SpatialMaxPooling_updateOutput (lowp_SpatialMaxPooling.c:45-108);
+ * oH/oW come from thhip_pool_outsize. */
+void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype);
+void thhip_pool_outsize(int H, int W, int kH, int kW, int dH, int dW, int padH, int padW, int ceil_mode,
+	int *oH, int *oW);
+
+/* Replaces nn_SpatialAveragePooling_updateOutput
+ * (SpatialAveragePooling.c:71-207). */
+void thhip_avgpool(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int count_include_pad, int dtype);
+
+/* Replaces nn_SoftMax_updateOutput (SoftMax.c:24-90) with the reference's
+ * polynomial exp approximation (thbasic.c:462-491). */
+void thhip_softmax(const void *x, void *y, long nframe, long dim, long stride, int dtype);
+
+/* Replaces nn_SpatialBatchNormalization_updateOutput
+ * (SpatialBatchNormalization.c:57-116); scale/shift are fp32 device arrays
+ * holding mean, invstd, weight, bias per plane. */
+void thhip_batchnorm(const void *x, void *y, long B, long C, long HW,
+	const float *mean, const float *invstd, const float *weight, const float *bias, int dtype);
+
+/* Replaces nn_CAddTable_updateOutput's two-input branch
+ * (CAddTable.c:59-70): y[j] = a[j] + sign*b[j] for j < nb, y[j] = a[j]
+ * beyond; sign = -1 reproduces the reference's MT_CAddTable arithmetic. */
+void thhip_axpby2(const void *a, const void *b, void *y, long na, long nb, float sign, int act, int dtype);
+
+/* fp32 host-layout conversions on the device. */
+void thhip_convert(const void *src, int src_dtype, void *dst, int dst_dtype, long n);
+
+/* Replaces rgb2float / bgr2float (thapi.c:20-46; CUDA analogue
+ * cudnn_copy.cu:13-116): one interleaved 8-bit image (device copy, `stride`
+ * bytes per row, cp planes) -> normalised planar dst in `dtype`. */
+void thhip_rgb2float(void *dst, const unsigned char *src, int width, int height, int stride, int cp,
+	const float *mean, const float *std, int bgr, int dtype);
+
+/* ---- uint8 (LOWP) path ---- */
+
+/* Replaces THLowpTensor_newFromFloatTensor's arithmetic
+ * (lowp_basic.c:15-35) on the device: min/max (including 0) over n floats,
+ * then q = roundf(v*mult) - roundf(min*mult).  mult/sub returned to host. */
+void thhip_quantize(const float *x, unsigned char *q, long n, float *mult, float *sub);
+/* Replaces THFloatTensor_newFromLowpTensor (lowp_basic.c:40-58). */
+void thhip_dequantize(const unsigned char *q, float *x, long n, float mult, float sub);
+
+/* Weight packing for the int8 kernel: uint8 codes [Co][K] -> signed
+ * (code-128) K-chunked layout + per-row sums.  Returns a device buffer. */
+void *thhip_conv_pack_weight_u8(const unsigned char *w_host, int Co, int K);
+
+/* Replaces Lowp_SpatialConvolution_updateOutput's per-image
+ * uint8 im2col + THLowpTensor_mm/lowpgemm + lowpadd
+ * (lowp_SpatialConvolution.c:5-120, lowp_basic.c:299-321, gemm8.cc:13-16):
+ * acc = sum_k (w+a_off)(x+b_off) with x = `zero` in the padding,
+ * c = clamp(((acc+c_off)*c_mult + round) >> c_shift, 0, 255),
+ * then per-plane saturating add of addend[o] with the reference's
+ * unclamped-below tail for the last (oH*oW)%8 elements of each plane,
+ * then (act != 0) the uint8 threshold q > thr ? q : val. */
+void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
+	int act, int thr, int val);
+
+/* Replaces Lowp_Threshold_updateOutput (lowp_Threshold.c:3-28) on codes. */
+void thhip_threshold_u8(const unsigned char *x, unsigned char *y, long n, int thr, int val, int inplace);
+
+/* Replaces Lowp_SoftMax_updateOutput (lowp_SoftMax.c:3-89); returns the
+ * output (mult) it derives (sub is 0). */
+float thhip_softmax_u8(const unsigned char *x, unsigned char *y, long nframe, long dim, long stride,
+	float in_mult, float in_sub);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif
