@@ -287,6 +287,9 @@ THFloatTensor *THFloatTensor_newFromHipTensor(THFloatTensor *t);
 long THHipNetwork_copyModuleOutput(THNETWORK *net, int idx, float **dst, long size[4], int *ndim);
 /* Quantisation (mult, sub) of module `idx`'s output in a HIPLOWP network. */
 int THHipNetwork_getModuleQuant(THNETWORK *net, int idx, float *mult, float *sub);
+/* Declares the quantisation of the uint8 device tensor the next THForward of
+ * a HIPLOWP network will be given (THProcessFloat derives it by itself). */
+int THHipNetwork_setInputQuant(THNETWORK *net, float mult, float sub);
 
 /* Drop-in for the reference's only call into gemmlowp (gemm8.cc:4-17,
  * declared lowp_basic.c:290-297): host pointers in and out, the GEMM and
@@ -330,6 +333,8 @@ void thhip_profile_get(int family, double *ms, long *launches, double *work);
  * M-interleaved layout the kernel streams.  Returns a device buffer. */
 void *thhip_conv_pack_weight(const float *w_host, int Co, int K, int dtype);
 size_t thhip_conv_packed_bytes(int Co, int K, int dtype);
+/* The inverse: packed -> row-major [Co][K] in the same dtype (new device buffer). */
+void *thhip_conv_unpack_rows(const void *wpacked, int Co, int K, int dtype);
 
 /* Replaces nn_SpatialConvolutionMM_updateOutput's per-image
  * im2col + sgemm + bias (SpatialConvolutionMM.c:75-109, 126-225) and, when

@@ -454,3 +454,89 @@ class Reference:
     def module_output(self, hostnet, idx):
         from thnets_amd.netbuild import tensor_to_numpy
         return tensor_to_numpy(self.abi, hostnet.thnet.net.contents.modules[idx].output)
+
+    # ---- -DLOWP build only: the reference's uint8 helpers that do not need gemmlowp ----
+    def _lowp_tensor(self, hostnet, q, mult, sub):
+        """uint8 codes as the reference stores them: a THFloatTensor whose storage holds bytes."""
+        q = np.ascontiguousarray(q, np.uint8)
+        from thnets_amd.abi import THFloatStorage
+        st = THFloatStorage(q.ctypes.data, 1, 0)
+        t = self.abi.THFloatTensor()
+        t.nDimension = q.ndim
+        stride = 1
+        for i in range(q.ndim - 1, -1, -1):
+            t.size[i] = q.shape[i]
+            t.stride[i] = stride
+            stride *= q.shape[i]
+        t.storage = C.pointer(st)
+        t.mult, t.sub = mult, sub
+        hostnet._keep += [q, st, t]
+        return t
+
+    def _lowp_read(self, pt):
+        t = pt.contents
+        shape = tuple(t.size[i] for i in range(t.nDimension))
+        n = int(np.prod(shape))
+        buf = (C.c_ubyte * n).from_address(t.storage.contents.data + t.storageOffset)
+        return np.frombuffer(buf, np.uint8).reshape(shape).copy(), float(t.mult), float(t.sub)
+
+    def lowp_quantize(self, x):
+        """THLowpTensor_newFromFloatTensor (lowp_basic.c:5-38) run by the reference."""
+        assert self.lowp
+        from thnets_amd.netbuild import HostNetwork
+        hn = HostNetwork(self.lib, self.abi)
+        t = hn.tensor(np.ascontiguousarray(x, np.float32))
+        self.lib.THLowpTensor_newFromFloatTensor.restype = C.c_void_p
+        self.lib.THLowpTensor_newFromFloatTensor.argtypes = [C.c_void_p]
+        out = self.lib.THLowpTensor_newFromFloatTensor(C.addressof(t.contents))
+        return self._lowp_read(C.cast(out, self.abi.PTensor))
+
+    def lowp_dequantize(self, q, mult, sub):
+        """THFloatTensor_newFromLowpTensor (lowp_basic.c:40-58) run by the reference."""
+        from thnets_amd.netbuild import HostNetwork, tensor_to_numpy
+        hn = HostNetwork(self.lib, self.abi)
+        t = self._lowp_tensor(hn, q, mult, sub)
+        self.lib.THFloatTensor_newFromLowpTensor.restype = C.c_void_p
+        self.lib.THFloatTensor_newFromLowpTensor.argtypes = [C.c_void_p]
+        out = self.lib.THFloatTensor_newFromLowpTensor(C.addressof(t))
+        return tensor_to_numpy(self.abi, C.cast(out, self.abi.PTensor))
+
+    def lowp_scale_float(self, mult, sub, value):
+        from thnets_amd.netbuild import HostNetwork
+        hn = HostNetwork(self.lib, self.abi)
+        t = self._lowp_tensor(hn, np.zeros(1, np.uint8), mult, sub)
+        self.lib.THLowp_ScaleFloat.restype = C.c_ubyte
+        self.lib.THLowp_ScaleFloat.argtypes = [C.c_void_p, C.c_float]
+        return self.lib.THLowp_ScaleFloat(C.addressof(t), value)
+
+    def lowp_module(self, spec, q, mult, sub, out_mult=None, out_sub=None):
+        """Runs one of Lowp_Threshold / Lowp_SpatialMaxPooling / Lowp_SoftMax
+        _updateOutput (lowp/lowp_*.c) on codes q; OpenMP is pinned to one thread
+        (the shipped softmax shares a scratch row between threads)."""
+        from thnets_amd.netbuild import HostNetwork
+        fn = {"threshold": "Lowp_Threshold_updateOutput", "maxpool": "Lowp_SpatialMaxPooling_updateOutput",
+              "softmax": "Lowp_SoftMax_updateOutput"}[spec["type"]]
+        hn = HostNetwork(self.lib, self.abi).build([spec])
+        m = hn.thnet.net.contents.modules[0]
+        if out_mult is not None:
+            m.output.contents.mult, m.output.contents.sub = out_mult, out_sub
+        t = self._lowp_tensor(hn, np.array(q, np.uint8, copy=True), mult, sub)
+        self.set_threads(1)
+        f = getattr(self.lib, fn)
+        f.restype = C.c_void_p
+        f.argtypes = [C.c_void_p, C.c_void_p]
+        out = f(C.addressof(m), C.addressof(t))
+        return self._lowp_read(C.cast(out, self.abi.PTensor))
+
+    def lowp_load_images(self, images, mean, std, bgr=0):
+        """Lowp_LoadImages (lowp_basic.c:82-131) run by the reference."""
+        imgs = [np.ascontiguousarray(im, np.uint8) for im in images]
+        H, W = imgs[0].shape[:2]
+        ptrs = (C.c_void_p * len(imgs))(*[im.ctypes.data for im in imgs])
+        m = (C.c_float * 3)(*mean)
+        s = (C.c_float * 3)(*std)
+        self.lib.Lowp_LoadImages.restype = C.c_void_p
+        self.lib.Lowp_LoadImages.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int]
+        self.set_threads(1)
+        out = self.lib.Lowp_LoadImages(ptrs, len(imgs), W, H, W * 3, m, s, int(bgr))
+        return self._lowp_read(C.cast(out, self.abi.PTensor))

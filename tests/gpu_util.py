@@ -1,0 +1,82 @@
+"""Helpers for the GPU tests: call the kernel-level C ABI on numpy data."""
+import ctypes as C
+
+import numpy as np
+
+from thnets_amd import abi, api
+
+F32, F16, BF16, U8 = abi.THHIP_F32, abi.THHIP_F16, abi.THHIP_BF16, abi.THHIP_U8
+
+
+def note(msg):
+    print("[gpu-case] " + msg, flush=True)
+
+
+def conv2d(lib, x, w, bias, d=(1, 1), pad=(0, 0), act=0, thr=0.0, val=0.0, dtype=F32):
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    B, Ci, H, W = x.shape
+    Co, _, kH, kW = w.shape
+    K = Ci * kH * kW
+    oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
+    note("conv2d x%s w%s d%s pad%s dtype%d" % (x.shape, w.shape, d, pad, dtype))
+    wp = lib.thhip_conv_pack_weight(w.ctypes.data, Co, K, dtype)
+    dx = api.to_device_dtype(lib, x, dtype)
+    db = api.DeviceArray(lib, np.ascontiguousarray(bias, np.float32)) if bias is not None else None
+    dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW * (4 if dtype == F32 else 2))
+    lib.thhip_conv2d(dx.ptr, wp, db.ptr if db else None, dy.ptr, B, Ci, H, W, Co, kH, kW, d[0], d[1], pad[0], pad[1],
+                     act, thr, val, dtype)
+    lib.thhip_sync()
+    y = api.from_device_dtype(dy, (B, Co, oH, oW), dtype)
+    lib.thhip_free(wp)
+    return y
+
+
+def gemv(lib, x, w, bias, act=0, thr=0.0, val=0.0, dtype=F32):
+    nOut, nIn = w.shape
+    note("gemv %dx%d dtype%d" % (nOut, nIn, dtype))
+    dx = api.to_device_dtype(lib, x, dtype)
+    dw = api.to_device_dtype(lib, w, dtype)
+    db = api.DeviceArray(lib, np.ascontiguousarray(bias, np.float32)) if bias is not None else None
+    dy = api.DeviceArray(lib, nbytes=nOut * 4)
+    lib.thhip_gemv(dx.ptr, dw.ptr, db.ptr if db else None, dy.ptr, nIn, nOut, act, thr, val, dtype)
+    lib.thhip_sync()
+    return api.from_device_dtype(dy, (nOut,), dtype)
+
+
+def unary(lib, fn, x, out_shape, dtype, *args):
+    dx = api.to_device_dtype(lib, x, dtype) if dtype != U8 else api.DeviceArray(lib, np.ascontiguousarray(x, np.uint8))
+    n = int(np.prod(out_shape))
+    dy = api.DeviceArray(lib, nbytes=n * {F32: 4, F16: 2, BF16: 2, U8: 1}[dtype])
+    fn(dx.ptr, dy.ptr, *args)
+    lib.thhip_sync()
+    return api.from_device_dtype(dy, out_shape, dtype)
+
+
+def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0):
+    xq = np.ascontiguousarray(xq, np.uint8)
+    wq = np.ascontiguousarray(wq, np.uint8)
+    B, Ci, H, W = xq.shape
+    Co, _, kH, kW = wq.shape
+    K = Ci * kH * kW
+    oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
+    note("conv2d_u8 x%s w%s d%s pad%s prm%s" % (xq.shape, wq.shape, d, pad, prm))
+    wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, K)
+    dx = api.DeviceArray(lib, xq)
+    da = api.DeviceArray(lib, np.ascontiguousarray(addend, np.int32)) if addend is not None else None
+    dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW)
+    lib.thhip_conv2d_u8(dx.ptr, wp, da.ptr if da else None, dy.ptr, B, Ci, H, W, Co, kH, kW, d[0], d[1], pad[0], pad[1],
+                        zero, prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"], prm["c_shift"], act, thr, val)
+    lib.thhip_sync()
+    y = dy.get((B, Co, oH, oW), np.uint8)
+    lib.thhip_free(wp)
+    return y
+
+
+def assert_close(got, want, tol, what=""):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    assert got.shape == want.shape, (what, got.shape, want.shape)
+    err = np.abs(got - want).max()
+    ref = max(np.abs(want).max(), 1e-30)
+    assert err <= tol * ref, "%s: max|err| %.3g > %.3g * max|ref| %.3g" % (what, err, tol, ref)

@@ -1,0 +1,118 @@
+"""The C ABI: structure layout against the reference's header (golden numbers written
+by tests/golden/make_abi_layout.py from the reference's own thnets.h), and that the
+built library exports every symbol include/thnets_hip.h declares.  No GPU needed."""
+import ctypes as C
+import json
+import os
+import re
+import subprocess
+
+import pytest
+
+from thnets_amd import abi, api
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GOLDEN = json.load(open(os.path.join(ROOT, "tests", "golden", "abi_layout.json")))
+HEADER = os.path.join(ROOT, "include", "thnets_hip.h")
+
+
+@pytest.mark.parametrize("variant", ["default", "lowp"])
+def test_ctypes_mirror_matches_reference_layout(variant):
+    lay = (abi.ABI if variant == "default" else abi.ABI_LOWP).layout()
+    for k, v in lay.items():
+        assert GOLDEN[variant][k] == v, k
+
+
+def test_enum_values_match_reference():
+    g = GOLDEN["default"]
+    assert len(abi.MODULE_TYPES) == g["n_module_types"]
+    assert abi.MT["MT_Linear"] == g["MT_Linear"]
+    assert abi.MT["MT_CAddTable"] == g["MT_CAddTable"]
+    assert abi.MT["MT_SpatialBatchNormalization"] == g["MT_SpatialBatchNormalization"]
+    assert abi.ENGINE_LOWP == g["ENGINE_LOWP"]
+    assert abi.ENGINE_HIP == g["ENGINE_LOWP"] + 1
+
+
+PROBE = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "thnets_hip.h"
+int main(void)
+{
+	printf("{\"sizeof_THFloatStorage\": %zu, \"sizeof_THFloatTensor\": %zu, \"sizeof_module\": %zu,"
+		"\"off_module_union\": %zu, \"off_module_output\": %zu, \"off_module_net\": %zu,"
+		"\"off_module_inputs\": %zu, \"sizeof_SpatialConvolution\": %zu, \"off_conv_nOutputPlane\": %zu,"
+		"\"sizeof_SpatialMaxPooling\": %zu, \"off_maxpool_indices\": %zu, \"off_bn_eps\": %zu,"
+		"\"sizeof_network\": %zu, \"sizeof_THNETWORK\": %zu, \"off_thnetwork_net\": %zu,"
+		"\"off_thnetwork_out\": %zu, \"off_thnetwork_mean\": %zu, \"off_thnetwork_std\": %zu,"
+		"\"n_module_types\": %d, \"MT_Linear\": %d, \"MT_CAddTable\": %d, \"ENGINE_LOWP\": %d}\n",
+		sizeof(THFloatStorage), sizeof(THFloatTensor), sizeof(struct module),
+		offsetof(struct module, SpatialConvolution), offsetof(struct module, output), offsetof(struct module, net),
+		offsetof(struct module, inputs), sizeof(struct SpatialConvolution),
+		offsetof(struct SpatialConvolution, nOutputPlane), sizeof(struct SpatialMaxPooling),
+		offsetof(struct SpatialMaxPooling, indices), offsetof(struct SpatialBatchNormalization, eps),
+		sizeof(struct network), sizeof(THNETWORK), offsetof(THNETWORK, net), offsetof(THNETWORK, out),
+		offsetof(THNETWORK, mean), offsetof(THNETWORK, std), MT_Transpose + 1, MT_Linear, MT_CAddTable, ENGINE_LOWP);
+	return 0;
+}
+'''
+
+
+def test_c_header_matches_reference_layout(tmp_path):
+    src = tmp_path / "probe.c"
+    src.write_text(PROBE)
+    exe = tmp_path / "probe"
+    subprocess.check_call(["gcc", "-I", os.path.join(ROOT, "include"), "-o", str(exe), str(src)])
+    got = json.loads(subprocess.check_output([str(exe)]).decode())
+    for k, v in got.items():
+        assert GOLDEN["default"][k] == v, k
+
+
+def test_golden_layout_is_current_when_reference_is_mounted(tmp_path):
+    ref = "/root/reference"
+    if not os.path.exists(os.path.join(ref, "thnets.h")):
+        pytest.skip("reference tree not mounted")
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_abi_layout", os.path.join(ROOT, "tests", "golden",
+                                                                                  "make_abi_layout.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    assert mod.probe(ref, []) == GOLDEN["default"]
+    assert mod.probe(ref, ["-DLOWP"]) == GOLDEN["lowp"]
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = re.findall(r"^[A-Za-z_][A-Za-z0-9_ \*]*?\b([A-Za-z_][A-Za-z0-9_]*)\s*\([^;{]*\)\s*;", text, flags=re.M)
+    return sorted(set(n for n in names if not n.startswith("(")))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = api.load_library()
+    names = declared_functions()
+    assert "THCreateHipNetwork" in names and "thhip_conv2d" in names and "lowpgemm" in names
+    assert len(names) >= 55
+    for n in names:
+        assert hasattr(lib, n), "libthnets_hip.so does not export %s" % n
+    for v in ("th_debug", "th_profile", "th_minmax"):
+        C.c_int.in_dll(lib, v)
+    for n in names:
+        assert n in api.PROTOTYPES, "no ctypes prototype for %s" % n
+
+
+def test_thhip_half_float_switch_contract():
+    lib = api.load_library()
+    assert lib.THHipHalfFloat(1) == 0
+    assert lib.THHipHalfFloat(2) == 0
+    assert lib.THHipHalfFloat(3) == -3      # ERR_NOTIMPLEMENTED, like THCudaHalfFloat without fp16
+    assert lib.THHipHalfFloat(0) == 0
+
+
+def test_pool_outsize_is_host_only_and_follows_reference_rule(oracle):
+    lib = api.load_library()
+    for (H, W, k, d, p, ceil) in [(55, 55, 3, 2, 0, 0), (13, 13, 3, 2, 0, 1), (112, 112, 3, 2, 1, 0), (7, 9, 2, 2, 1, 1),
+                                  (6, 6, 3, 3, 1, 1), (5, 5, 2, 2, 1, 1)]:
+        oh, ow = C.c_int(), C.c_int()
+        lib.thhip_pool_outsize(H, W, k, k, d, d, p, p, ceil, C.byref(oh), C.byref(ow))
+        assert (oh.value, ow.value) == oracle.pool_outsize(H, W, k, k, d, d, p, p, ceil)

@@ -1,0 +1,126 @@
+"""Bit-exact parity of the uint8 (LOWP) kernels and engine against the CPU oracle."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import cases
+import gpu_util as G
+from thnets_amd import api, configs
+
+pytestmark = pytest.mark.gpu
+
+
+def test_quantize_dequantize_bit_exact(hiplib, oracle):
+    g = cases.rng(10)
+    for x in (g.standard_normal((2, 3, 5, 7), dtype=np.float32), g.uniform(0, 1, (4, 11)).astype(np.float32),
+              -g.uniform(0, 3, 50).astype(np.float32), np.zeros(9, np.float32),
+              g.standard_normal(300000, dtype=np.float32) * 100):
+        dx = api.DeviceArray(hiplib, x)
+        dq = api.DeviceArray(hiplib, nbytes=x.size)
+        m, s = C.c_float(), C.c_float()
+        hiplib.thhip_quantize(dx.ptr, dq.ptr, x.size, C.byref(m), C.byref(s))
+        hiplib.thhip_sync()
+        q, mo, so = oracle.lowp_quantize(x)
+        assert (m.value, s.value) == (mo, so)
+        assert np.array_equal(dq.get(x.shape, np.uint8), q)
+        dy = api.DeviceArray(hiplib, nbytes=x.nbytes)
+        hiplib.thhip_dequantize(dq.ptr, dy.ptr, x.size, mo, so)
+        hiplib.thhip_sync()
+        assert np.array_equal(dy.get(x.shape, np.float32), oracle.lowp_dequantize(q, mo, so))
+
+
+def _lowp_case(i, rngv=16.0, seed=0):
+    B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW = cases.CONV_CASES[i]
+    g = cases.rng(1000 + i + seed)
+    x = g.uniform(-3, 3, (B, Ci, H, W)).astype(np.float32)
+    w = g.standard_normal((Co, Ci, kH, kW), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * kH * kW)))
+    b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.5)
+    return x, w, b, (dH, dW), (pH, pW)
+
+
+@pytest.mark.parametrize("i", range(len(cases.CONV_CASES)))
+def test_conv_u8_bit_exact(hiplib, oracle, i):
+    x, w, b, d, p = _lowp_case(i)
+    rngv = 16.0
+    om, osub = float(np.float32(255) / np.float32(rngv)), -rngv / 2
+    xq, im, isub = oracle.lowp_quantize(x)
+    wq, wm, wsub = oracle.lowp_quantize(w)
+    bq, bm, bsub = oracle.lowp_quantize(b)
+    want = oracle.lowp_conv2d(xq, im, isub, wq, wm, wsub, bq, bm, bsub, om, osub, d, p)
+    prm = oracle.lowp_mm_params(wm, wsub, im, isub, om, osub)
+    zero = int(np.round(np.float32(-isub) * np.float32(im)))
+    addend = np.array([oracle.lowp_bias_addend(int(c), bm, bsub, om) for c in bq], np.int32)
+    got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm)
+    assert got.shape == want.shape
+    assert np.array_equal(got, want), "mismatching codes: %d of %d" % ((got != want).sum(), got.size)
+    # fused threshold on the codes
+    thr = oracle.lowp_scale_float(om, osub, 0.0)
+    got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, act=1, thr=thr, val=thr)
+    assert np.array_equal(got, oracle.lowp_threshold(want, thr, thr))
+
+
+def test_conv_u8_wrapping_requantisation_and_extreme_offsets(hiplib, oracle):
+    g = cases.rng(1100)
+    xq = g.integers(0, 256, (2, 5, 7, 6), dtype=np.uint8)
+    wq = g.integers(0, 256, (9, 5, 3, 3), dtype=np.uint8)
+    for prm in (dict(a_off=-128, b_off=-128, c_off=1000, c_mult=77, c_shift=12),
+                dict(a_off=0, b_off=0, c_off=0, c_mult=9000, c_shift=20),          # products beyond 2^31 wrap
+                dict(a_off=-255, b_off=3, c_off=-12345, c_mult=511, c_shift=18),
+                dict(a_off=-100, b_off=-7, c_off=5, c_mult=1, c_shift=0)):
+        col = np.stack([oracle.lowp_unfold(xq[t], (3, 3), (1, 1), (1, 1), 77) for t in range(2)])
+        want = np.stack([oracle.lowp_gemm(wq.reshape(9, 45), col[t], **prm) for t in range(2)]).reshape(2, 9, 7, 6)
+        got = G.conv2d_u8(hiplib, xq, wq, None, (1, 1), (1, 1), 77, prm)
+        assert np.array_equal(got, want), prm
+
+
+def test_lowpgemm_drop_in(hiplib, oracle):
+    g = cases.rng(1101)
+    for (m, n, k) in ((3, 5, 7), (64, 3025, 363), (100, 1, 900), (130, 77, 65)):
+        a = g.integers(0, 256, (m, k), dtype=np.uint8)
+        b = g.integers(0, 256, (k, n), dtype=np.uint8)
+        c = np.zeros((m, n), np.uint8)
+        G.note("lowpgemm %s" % ((m, n, k),))
+        hiplib.lowpgemm(1, 1, 1, m, n, k, a.ctypes.data, b.ctypes.data, c.ctypes.data, k, n, n, -117, -128, 32513, 1028, 18)
+        assert np.array_equal(c, oracle.lowp_gemm(a, b, -117, -128, 32513, 1028, 18))
+
+
+def test_threshold_and_softmax_u8_bit_exact(hiplib, oracle):
+    q = cases.rng(1102).integers(0, 256, (3, 1000), dtype=np.uint8)
+    y = G.unary(hiplib, hiplib.thhip_threshold_u8, q, q.shape, G.U8, q.size, 127, 127, 1)
+    assert np.array_equal(y, oracle.lowp_threshold(q, 127, 127, 1))
+    for shape in [(3, 1000), (1000,), (2, 21, 3, 3)]:
+        q = cases.rng(1103).integers(0, 256, shape, dtype=np.uint8)
+        nframe, dim, stride = {1: (1, shape[0], 1), 2: (shape[0], shape[-1], 1),
+                               4: (shape[0], shape[1], shape[2] * shape[3])}[len(shape)]
+        dx = api.DeviceArray(hiplib, q)
+        dy = api.DeviceArray(hiplib, nbytes=q.size)
+        hiplib.thhip_softmax_u8.restype = C.c_float
+        om = hiplib.thhip_softmax_u8(dx.ptr, dy.ptr, nframe, dim, stride, 7.96875, -16.0)
+        hiplib.thhip_sync()
+        want, wm, _ = oracle.lowp_softmax(q, 7.96875, -16.0)
+        assert np.array_equal(dy.get(shape, np.uint8), want)
+        assert om == np.float32(wm)
+
+
+def test_engine_small_network_bit_exact_every_layer(hiplib, oracle):
+    g = cases.rng(17)
+    w1 = g.standard_normal((6, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+    w2 = g.standard_normal((5, 6, 2, 2), dtype=np.float32) * np.float32(0.3)
+    layers = [configs.conv(w1, g.standard_normal(6, dtype=np.float32) * np.float32(0.1), 1, 1), configs.relu(),
+              configs.maxpool(2, 2),
+              configs.conv(w2, g.standard_normal(5, dtype=np.float32) * np.float32(0.1), 1, 0), configs.relu(),
+              {"type": "softmax"}]
+    x = g.uniform(-2, 2, (5, 3, 8, 8)).astype(np.float32)
+    net = api.HipNetwork(layers, lowp_range=16.0)
+    y = net.process_float(x)
+    xq, im, isub = oracle.lowp_quantize(x)
+    outs = []
+    q, m, s = oracle.lowp_run_layers(layers, xq, im, isub, 16.0, collect=outs)
+    for i in (1, 2, 4, 5):      # conv outputs hold the fused threshold, compare after it
+        assert np.array_equal(net.module_output(i).astype(np.uint8), outs[i][0]), i
+    assert np.array_equal(y, oracle.lowp_dequantize(q, m, s).ravel())
+    # a second forward on the same engine instance gives the same codes (the reference
+    # loses its quantisation parameters after the first)
+    assert np.array_equal(net.process_float(x), y)
+    net.free()

@@ -1,0 +1,129 @@
+"""Whole networks through the drop-in API (THCreateHipNetwork + THProcessFloat /
+THForward) against the CPU oracle layer by layer and against golden vectors written by
+the reference's own CPU library."""
+import os
+
+import numpy as np
+import pytest
+
+import cases
+import gpu_util as G
+from thnets_amd import api, configs
+
+pytestmark = pytest.mark.gpu
+
+GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fp32_golden.npz"))
+NET_TOL = 1e-4      # contract: 1e-3 * max|ref| per layer output
+
+
+def layerwise(net, oracle, cfg, tol):
+    x = oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])
+    outs = []
+    oracle.run_layers(cfg["layers"], x, collect=outs)
+    layers = cfg["layers"]
+    for i, o in enumerate(outs):
+        if isinstance(o, list):
+            continue
+        want = o
+        # a Threshold folded into its producer: the producer's buffer holds the thresholded values
+        if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold" and layers[i]["type"] in ("conv", "linear", "caddtable"):
+            want = outs[i + 1]
+        G.assert_close(net.module_output(i).ravel(), np.asarray(want).ravel(), tol, "module %d %s" % (i, layers[i]["type"]))
+
+
+@pytest.mark.parametrize("name", sorted(cases.small_networks().keys()))
+def test_small_networks_vs_oracle_and_golden(hiplib, oracle, name):
+    cfg = cases.small_networks()[name]
+    G.note("network " + name)
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    x0 = cfg["input"].copy()
+    y = net.process_float(cfg["input"])
+    assert np.array_equal(cfg["input"], x0)
+    G.assert_close(y, GOLD["net_" + name], NET_TOL, "golden")
+    layerwise(net, oracle, cfg, NET_TOL)
+    # repeated calls are stable
+    assert np.array_equal(net.process_float(cfg["input"]), y)
+    net.free()
+
+
+def test_process_float_normalises_callers_buffer_in_place(hiplib, oracle):
+    import ctypes as C
+    cfg = cases.small_networks()["tiny_cnn"]
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    x = np.array(cfg["input"], np.float32, copy=True)
+    res = api.c_fp()
+    ow, oh = C.c_int(), C.c_int()
+    B, Cn, H, W = x.shape
+    n = hiplib.THProcessFloat(net.handle, x.ctypes.data, B, W, H, Cn, C.byref(res), C.byref(ow), C.byref(oh))
+    assert n == 30 and (ow.value, oh.value) == (1, 1)
+    assert np.array_equal(x, oracle.normalize(cfg["input"], cfg["mean"], cfg["std"]))   # thapi.c:397-402
+    net.free()
+
+
+def test_config1_vs_golden_sample(hiplib, oracle):
+    cfg = configs.config1()
+    net = api.HipNetwork(cfg["layers"])
+    net.upload(cfg["input"])
+    net.forward()
+    y = net.module_output(1).ravel()
+    G.assert_close(y[cases.sample_indices(y.size)], GOLD["config1/sample"], 2e-5)
+    assert abs(y.astype(np.float64).sum() - GOLD["config1/sum"]) <= 1e-5 * abs(GOLD["config1/sum"])
+    G.assert_close(y, oracle.run_layers(cfg["layers"], cfg["input"]).ravel(), 2e-5)
+    net.free()
+
+
+def test_alexnet_b1_vs_golden_and_layerwise(hiplib, oracle):
+    cfg = configs.alexnet_owt()
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    y = net.process_float(cfg["input"])
+    G.assert_close(y, GOLD["alexnet_b1"], NET_TOL)
+    layerwise(net, oracle, cfg, NET_TOL)
+    net.free()
+    # the THMakeSpatial form gives the same logits
+    cfg2 = configs.alexnet_owt(softmax=False)
+    a = api.HipNetwork(cfg2["layers"], cfg2["mean"], cfg2["std"])
+    b = api.HipNetwork(cfg2["layers"], cfg2["mean"], cfg2["std"], make_spatial=224)
+    assert b.nelem == a.nelem - 1
+    G.assert_close(b.process_float(cfg2["input"]), a.process_float(cfg2["input"]), 1e-5)
+    a.free()
+    b.free()
+
+
+@pytest.mark.parametrize("half", [1, 2])
+def test_half_engine_small_vgg(hiplib, oracle, half):
+    cfg = cases.small_networks()["vgg16_small"]
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"], half=half)
+    y = net.process_float(cfg["input"])
+    G.assert_close(y, GOLD["net_vgg16_small"], 2e-2 if half == 1 else 6e-2, "half engine")
+    net.free()
+
+
+def test_process_images_matches_process_float(hiplib, oracle):
+    cfg = cases.small_networks()["tiny_cnn"]
+    g = cases.rng(1200)
+    imgs = [g.integers(0, 256, (8, 8, 3), dtype=np.uint8) for _ in range(3)]
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    y = net.process_images(imgs, bgr=0)
+    x = np.stack([oracle.rgb2float(im, cfg["mean"], cfg["std"], 0) for im in imgs])
+    want = oracle.run_layers(cfg["layers"], x)
+    G.assert_close(y, want.ravel(), 1e-5)
+    yb = net.process_images(imgs, bgr=1)
+    xb = np.stack([oracle.rgb2float(im, cfg["mean"], cfg["std"], 1) for im in imgs])
+    G.assert_close(yb, oracle.run_layers(cfg["layers"], xb).ravel(), 1e-5)
+    net.free()
+
+
+def test_vgg16_full_size_properties(hiplib, oracle):
+    """Full configuration 3 (batch 16, 224x224): too large for the CPU checker inside a
+    test, so check size-independent properties: batch == images one by one, and the
+    first convolution + pooling block against the oracle on one image."""
+    cfg = configs.vgg16(batch=4)
+    net = api.HipNetwork(cfg["layers"])
+    y = net.process_float(cfg["input"]).reshape(4, -1)
+    y1 = net.process_float(cfg["input"][2:3]).ravel()
+    G.assert_close(y1, y[2], 1e-5, "batch vs single image")
+    net.upload(cfg["input"][:1])
+    net.forward()
+    want = oracle.run_layers(cfg["layers"][:5], cfg["input"][:1])
+    G.assert_close(net.module_output(4), want, 2e-5, "first block")
+    net.free()

@@ -1,0 +1,677 @@
+/*
+ * Implicit-GEMM convolution for gfx950 on the matrix cores.
+ *
+ * Replaces the reference's per-image im2col + SGEMM + bias fill
+ * (modules/SpatialConvolutionMM.c:11-109, thbasic.c:601-711, 1073-1103,
+ * OpenBLAS-stripped/sgemm.c) and the Threshold module that usually follows
+ * (modules/Threshold.c:38-63) with one kernel:
+ *
+ *     C[M = Co][N = B*oH*oW] = Wp[M][K = Ci*kH*kW] * im2col(x)[K][N]
+ *
+ * The im2col matrix is never materialised: each workgroup gathers its
+ * K-tile x N-tile slab straight from the NCHW input (lanes run along the
+ * output row, so loads coalesce along W), zero-filling the padding, and
+ * stages it through LDS.  Weights are pre-packed once at engine creation
+ * into the exact order the LDS tile wants, so their loads are 16-byte,
+ * fully coalesced and written to LDS unchanged.
+ *
+ * Fragment layout.  K is cut into chunks (8 values for fp32, 16 for
+ * fp16/bf16); within a chunk, lane half h = lane/32 owns the contiguous
+ * sub-range [h*C/2, (h+1)*C/2) as ONE 16-byte vector, for row (A) or column
+ * (B) lane%32.  A 32x32x2 fp32 MFMA contracts the two lane halves, so step s
+ * of a chunk uses element s of every lane's vector; a 32x32x16 half MFMA
+ * consumes the whole vector.  The contraction order inside a chunk is thus
+ * permuted relative to k, which a sum does not care about.  Both LDS tiles
+ * are stored [chunk][32-row block][h][32][16 B]: every ds_read_b128 /
+ * ds_write_b128 of a wave touches 1 KiB contiguous, i.e. no bank conflicts.
+ */
+#include <stdlib.h>
+#include <string.h>
+#include <vector>
+#include "thhip_internal.h"
+
+#define CONV_THREADS 256
+
+struct ConvParams {
+	const void *x;
+	const void *wp;
+	const float *bias;
+	void *y;
+	int B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, oH, oW;
+	int K, KC, N, oHW, HW, kHW;
+	unsigned magic_khw, magic_kw;
+	int act;
+	float thr, val;
+	int tiles_m, tiles_n;
+	unsigned x_bytes;
+	/* uint8 path only */
+	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
+	const int *addend;	/* per-plane bias addend, or NULL */
+	int zero, offA, offB, c_off, c_mult, c_shift, ithr, ival;
+};
+
+/* floor(n / d) for n*d < 2^32, d > 1, with m = floor(2^32/d) + 1. */
+static inline unsigned conv_magic(unsigned d)
+{
+	return d <= 1 ? 0u : (unsigned)(((1ull << 32) / d) + 1);
+}
+
+template <int DT> struct ConvTraits;
+template <> struct ConvTraits<THHIP_F32> {
+	static constexpr int CHUNK = 8;		/* k values per chunk */
+	static constexpr int VEC = 4;		/* elements per 16-byte lane vector */
+	typedef float elem;
+};
+template <> struct ConvTraits<THHIP_F16> {
+	static constexpr int CHUNK = 16;
+	static constexpr int VEC = 8;
+	typedef _Float16 elem;
+};
+template <> struct ConvTraits<THHIP_BF16> {
+	static constexpr int CHUNK = 16;
+	static constexpr int VEC = 8;
+	typedef __bf16 elem;
+};
+
+template <> struct ConvTraits<THHIP_U8> {
+	static constexpr int CHUNK = 32;
+	static constexpr int VEC = 16;
+	typedef unsigned char elem;
+};
+
+template <int DT> struct ConvAcc { typedef floatx16 T; };
+template <> struct ConvAcc<THHIP_U8> { typedef intx16 T; };
+
+template <int DT>
+__device__ __forceinline__ void conv_mma(typename ConvAcc<DT>::T &acc, const floatx4 &a, const floatx4 &b);
+
+template <>
+__device__ __forceinline__ void conv_mma<THHIP_F32>(floatx16 &acc, const floatx4 &a, const floatx4 &b)
+{
+	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], acc, 0, 0, 0);
+	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
+}
+
+template <>
+__device__ __forceinline__ void conv_mma<THHIP_F16>(floatx16 &acc, const floatx4 &a, const floatx4 &b)
+{
+	acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
+}
+
+template <>
+__device__ __forceinline__ void conv_mma<THHIP_BF16>(floatx16 &acc, const floatx4 &a, const floatx4 &b)
+{
+	acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+
+template <>
+__device__ __forceinline__ void conv_mma<THHIP_U8>(intx16 &acc, const floatx4 &a, const floatx4 &b)
+{
+	acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), acc, 0, 0, 0);
+}
+
+/* gemmlowp's legacy output stage as the reference calls it (lowp/gemm8.cc:13-16):
+ * ((acc + c_off) * c_mult + rounding) >> c_shift in wrapping 32-bit arithmetic,
+ * arithmetic shift, saturated to a byte. */
+__device__ __forceinline__ int conv_requant(int acc, int c_off, int c_mult, int c_shift)
+{
+	unsigned u = ((unsigned)acc + (unsigned)c_off) * (unsigned)c_mult;
+	u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
+	int t = (int)u >> c_shift;
+	return t < 0 ? 0 : t > 255 ? 255 : t;
+}
+
+/* Scalar (wave-uniform) decode of k -> offset of tap (c,kh,kw) in the image. */
+struct KTap { int koff, kh, kw; };
+
+__device__ __forceinline__ KTap conv_ktap(const ConvParams &p, int k)
+{
+	KTap t;
+	unsigned c, rem, kh;
+	if (p.kHW == 1) {
+		c = k;
+		rem = 0;
+	} else {
+		c = __umulhi((unsigned)k, p.magic_khw);
+		rem = k - c * p.kHW;
+	}
+	if (p.kW == 1)
+		kh = rem;
+	else
+		kh = __umulhi(rem, p.magic_kw);
+	t.kh = kh;
+	t.kw = rem - kh * p.kW;
+	t.koff = c * p.HW + t.kh * p.W + t.kw;
+	if (k >= p.K)
+		t.kh = 0x40000000;	/* K padding: forces the bounds test to fail */
+	return t;
+}
+
+template <int DT, int BM, int BN, int WGM, int WGN>
+__global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
+{
+	typedef ConvTraits<DT> TR;
+	typedef typename TR::elem elem;
+	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC;
+	constexpr int MB = BM / 32, NB = BN / 32;		/* 32-row blocks per tile */
+	constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32;	/* MFMA tiles per wave */
+	constexpr int A_VECS = MB * 2 * 64;			/* 16-byte vectors per K-tile (2 chunks) */
+	constexpr int B_VECS = NB * 2 * 64;
+	constexpr int A_PER_WAVE = MB * 2 / 4;			/* 1 KiB blocks loaded per wave */
+	constexpr int B_PER_THREAD = BN / 64;			/* (chunk,h) vectors gathered per thread */
+	static_assert(WGM * WGN == 4, "four waves per workgroup");
+	static_assert(MB * 2 % 4 == 0 && BN % 64 == 0, "tile shape");
+
+	__shared__ floatx4 lds[2 * (A_VECS + B_VECS)];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wm = wave % WGM, wn = wave / WGM;
+
+	/* XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so
+	 * give each XCD a contiguous run of tiles (M fastest) and let neighbours
+	 * that share an input slab share an L2. */
+	int tile;
+	{
+		const int nblk = gridDim.x, bid = blockIdx.x;
+		const int xcd = bid & 7, local = bid >> 3;
+		const int q = nblk >> 3, r = nblk & 7;
+		tile = xcd * q + (xcd < r ? xcd : r) + local;
+	}
+	const int tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
+
+	/* ---- B gather role: one output position per thread ---- */
+	const int n_local = tid % BN;
+	const int slot = __builtin_amdgcn_readfirstlane(tid / BN);
+	const int n_glob = tile_n * BN + n_local;
+	const bool n_ok = n_glob < p.N;
+	int iy0, ix0, xoff;
+	{
+		int nn = n_ok ? n_glob : 0;
+		int b = nn / p.oHW, r = nn - b * p.oHW;
+		int oy = r / p.oW, ox = r - oy * p.oW;
+		iy0 = oy * p.dH - p.padH;
+		ix0 = ox * p.dW - p.padW;
+		xoff = b * p.Ci * p.HW + iy0 * p.W + ix0;
+	}
+	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
+
+	const floatx4 *wp = (const floatx4 *)p.wp;
+	floatx4 areg[A_PER_WAVE];
+	floatx4 breg[B_PER_THREAD];
+	int colsum = 0;		/* uint8 path: sum of this thread's gathered (code - 128) */
+
+	auto load_tile = [&](int kt) {
+#pragma unroll
+		for (int i = 0; i < A_PER_WAVE; i++) {
+			const int idx = wave + 4 * i;
+			const int mbi = idx % MB, kci = idx / MB;
+			areg[i] = wp[((size_t)(tile_m * MB + mbi) * p.KC + kt * 2 + kci) * 64 + lane];
+		}
+#pragma unroll
+		for (int j = 0; j < B_PER_THREAD; j++) {
+			const int pidx = slot * B_PER_THREAD + j;
+			const int kbase = (kt * 2 + (pidx >> 1)) * CHUNK + (pidx & 1) * VEC;
+			elem v[VEC];
+#pragma unroll
+			for (int e = 0; e < VEC; e++) {
+				const KTap t = conv_ktap(p, kbase + e);
+				const int iy = iy0 + t.kh, ix = ix0 + t.kw;
+				const bool ok = n_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+				/* an offset past the buffer's extent reads as zero */
+				const unsigned voff = ok ? (unsigned)(xoff + t.koff) * (unsigned)sizeof(elem) : 0xfffffff0u;
+				if constexpr (DT == THHIP_U8) {
+					/* padding is the code of 0.0 (lowp_SpatialConvolution.c:101);
+					 * columns past N and the K padding hold 128, which the
+					 * re-centring below turns into 0 */
+					const unsigned char ld = __builtin_amdgcn_raw_buffer_load_b8(xrsrc, voff, 0, 0);
+					v[e] = ok ? ld : (unsigned char)((n_ok && kbase + e < p.K) ? p.zero : 128);
+				} else if constexpr (sizeof(elem) == 4) {
+					v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, voff, 0, 0));
+				} else {
+					v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b16(xrsrc, voff, 0, 0));
+				}
+			}
+			floatx4 packed;
+			__builtin_memcpy(&packed, v, 16);
+			if constexpr (DT == THHIP_U8) {
+				/* code - 128 as a signed byte, and this thread's share of the
+				 * column sum of the re-centred codes */
+				intx4 q = __builtin_bit_cast(intx4, packed);
+#pragma unroll
+				for (int d = 0; d < 4; d++) {
+					q[d] ^= (int)0x80808080;
+					colsum = __builtin_amdgcn_sdot4(q[d], 0x01010101, colsum, false);
+				}
+				packed = __builtin_bit_cast(floatx4, q);
+			}
+			breg[j] = packed;
+		}
+	};
+
+	auto store_tile = [&](int buf) {
+		floatx4 *la = lds + buf * (A_VECS + B_VECS);
+		floatx4 *lb = la + A_VECS;
+#pragma unroll
+		for (int i = 0; i < A_PER_WAVE; i++) {
+			const int idx = wave + 4 * i;
+			const int mbi = idx % MB, kci = idx / MB;
+			la[(kci * MB + mbi) * 64 + lane] = areg[i];
+		}
+#pragma unroll
+		for (int j = 0; j < B_PER_THREAD; j++) {
+			const int pidx = slot * B_PER_THREAD + j;
+			const int kci = pidx >> 1, h = pidx & 1;
+			lb[((kci * NB + (n_local >> 5)) * 2 + h) * 32 + (n_local & 31)] = breg[j];
+		}
+	};
+
+	typename ConvAcc<DT>::T acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; i++)
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[i][j][r] = 0;
+
+	const int nkt = p.KC / 2;
+	load_tile(0);
+	store_tile(0);
+	__syncthreads();
+	for (int kt = 0; kt < nkt; kt++) {
+		const int cur = kt & 1;
+		if (kt + 1 < nkt)
+			load_tile(kt + 1);
+		const floatx4 *la = lds + cur * (A_VECS + B_VECS);
+		const floatx4 *lb = la + A_VECS;
+#pragma unroll
+		for (int kci = 0; kci < 2; kci++) {
+			floatx4 af[TM], bf[TN];
+#pragma unroll
+			for (int i = 0; i < TM; i++)
+				af[i] = la[(kci * MB + wm * TM + i) * 64 + lane];
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+				bf[j] = lb[(kci * NB + wn * TN + j) * 64 + lane];
+#pragma unroll
+			for (int i = 0; i < TM; i++)
+#pragma unroll
+				for (int j = 0; j < TN; j++)
+					conv_mma<DT>(acc[i][j], af[i], bf[j]);
+		}
+		if (kt + 1 < nkt)
+			store_tile(cur ^ 1);
+		__syncthreads();
+	}
+
+	/* ---- epilogue ---- */
+	elem *y = (elem *)p.y;
+	if constexpr (DT == THHIP_U8) {
+		/* Every (chunk, half) share of a column was gathered by one of the
+		 * 256/BN threads that own it: add the shares up in LDS. */
+		__shared__ int cs[BN];
+		if (tid < BN)
+			cs[tid] = 0;
+		__syncthreads();
+		atomicAdd(&cs[n_local], colsum);
+		__syncthreads();
+		/* sum (w+a_off)(x+b_off) with w = w'+128, x = x'+128:
+		 *   sum w'x' + (128+b_off) rowsum + (128+a_off) colsum + K (128+a_off)(128+b_off) */
+		const int tail0 = (p.oHW / 8) * 8;	/* lowpadd's unclamped tail starts here */
+#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			const int nl = (wn * TN + j) * 32 + (lane & 31);
+			const int n = tile_n * BN + nl;
+			if (n >= p.N)
+				continue;
+			const int b = n / p.oHW, rem = n - b * p.oHW;
+			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+			const int colterm = p.offA * cs[nl] + p.K * p.offA * p.offB;
+#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					const int m = m0 + 8 * (r >> 2) + (r & 3);
+					if (m < p.Co) {
+						const int a = acc[i][j][r] + p.offB * p.rowsum[m] + colterm;
+						int q = conv_requant(a, p.c_off, p.c_mult, p.c_shift);
+						if (p.addend) {
+							/* lowpadd, lowp_SpatialConvolution.c:71-88 */
+							const int sum = q + p.addend[m];
+							if (rem < tail0)
+								q = sum > 255 ? 255 : sum < 0 ? 0 : sum;
+							else
+								q = sum > 255 ? 255 : (sum & 255);
+						}
+						if (p.act)
+							q = q > p.ithr ? q : p.ival;
+						y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
+					}
+				}
+			}
+		}
+	} else {
+		/* bias, optional threshold, NCHW store */
+#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
+			if (n >= p.N)
+				continue;
+			const int b = n / p.oHW, rem = n - b * p.oHW;
+			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					const int m = m0 + 8 * (r >> 2) + (r & 3);
+					if (m < p.Co) {
+						float v = acc[i][j][r] + (p.bias ? p.bias[m] : 0.0f);
+						if (p.act)
+							v = v > p.thr ? v : p.val;
+						y[ybase + (size_t)m * p.oHW] = (elem)v;
+					}
+				}
+			}
+		}
+	}
+}
+
+/* ------------------------------------------------------------------ */
+/* host side                                                           */
+/* ------------------------------------------------------------------ */
+
+#define CONV_MPAD 128	/* packed rows are padded to the largest M tile */
+
+static inline int conv_chunk(int dtype) { return dtype == THHIP_F32 ? 8 : dtype == THHIP_U8 ? 32 : 16; }
+static inline int conv_kc(int K, int dtype)
+{
+	int c = conv_chunk(dtype);
+	int kc = (K + c - 1) / c;
+	return (kc + 1) & ~1;	/* whole K-tiles of two chunks */
+}
+
+extern "C" size_t thhip_conv_packed_bytes(int Co, int K, int dtype)
+{
+	size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
+	return mpad / 32 * conv_kc(K, dtype) * 1024;
+}
+
+static inline unsigned short f32_to_f16_bits(float f)
+{
+	_Float16 h = (_Float16)f;
+	unsigned short u;
+	memcpy(&u, &h, 2);
+	return u;
+}
+
+static inline unsigned short f32_to_bf16_bits(float f)
+{
+	unsigned u;
+	memcpy(&u, &f, 4);
+	if ((u & 0x7fffffffu) > 0x7f800000u)
+		return (unsigned short)((u >> 16) | 0x40);
+	u += 0x7fffu + ((u >> 16) & 1);	/* round to nearest even */
+	return (unsigned short)(u >> 16);
+}
+
+extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int K, int dtype)
+{
+	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
+		THError("thhip_conv_pack_weight: unsupported dtype %d", dtype);
+	const int chunk = conv_chunk(dtype), vec = chunk / 2, KC = conv_kc(K, dtype);
+	const size_t bytes = thhip_conv_packed_bytes(Co, K, dtype);
+	const int esize = thhip_esize(dtype);
+	unsigned char *host = (unsigned char *)calloc(1, bytes);
+	if (!host)
+		THError("thhip_conv_pack_weight: out of host memory (%zu bytes)", bytes);
+	for (int m = 0; m < Co; m++) {
+		const int mb = m >> 5, mi = m & 31;
+		for (int k = 0; k < K; k++) {
+			const int kc = k / chunk, h = (k % chunk) / vec, e = k % vec;
+			const size_t idx = ((((size_t)mb * KC + kc) * 2 + h) * 32 + mi) * vec + e;
+			const float v = w[(size_t)m * K + k];
+			if (dtype == THHIP_F32)
+				((float *)host)[idx] = v;
+			else if (dtype == THHIP_F16)
+				((unsigned short *)host)[idx] = f32_to_f16_bits(v);
+			else
+				((unsigned short *)host)[idx] = f32_to_bf16_bits(v);
+		}
+	}
+	(void)esize;
+	void *dev = thhip_malloc(bytes);
+	thhip_memcpy_h2d(dev, host, bytes);
+	free(host);
+	return dev;
+}
+
+template <int DT, int BM, int BN, int WGM, int WGN>
+static void conv_launch(ConvParams &p)
+{
+	p.tiles_m = (p.Co + BM - 1) / BM;
+	p.tiles_n = (p.N + BN - 1) / BN;
+	dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+	conv_mfma_kernel<DT, BM, BN, WGM, WGN><<<grid, dim3(CONV_THREADS), 0, thhip_stream()>>>(p);
+}
+
+template <int DT>
+static void conv_dispatch(ConvParams &p)
+{
+	/* Tile choice: the largest tile that still yields enough workgroups to
+	 * fill 256 CUs a couple of times over; Co <= 64 never needs BM = 128. */
+	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
+	const long t64n = (long)((p.Co + 127) / 128) * ((p.N + 63) / 64);
+	if (p.Co > 64 && t128 >= 512)
+		conv_launch<DT, 128, 128, 2, 2>(p);
+	else if (p.Co > 64 && t64n >= 384)
+		conv_launch<DT, 128, 64, 2, 2>(p);
+	else if (p.Co <= 64 && (long)((p.N + 127) / 128) >= 512)
+		conv_launch<DT, 64, 128, 2, 2>(p);
+	else
+		conv_launch<DT, 64, 64, 2, 2>(p);
+}
+
+struct ConvU8Args {
+	const int *addend;
+	int zero, a_off, b_off, c_off, c_mult, c_shift, ithr, ival;
+};
+
+static void conv_run(const void *x, const void *wpacked, const float *bias, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype, const ConvU8Args *u8)
+{
+	if (B < 1 || Ci < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
+		THError("thhip_conv2d: bad geometry");
+	const int oW = (W + 2 * padW - kW) / dW + 1;	/* SpatialConvolutionMM.c:159-160 */
+	const int oH = (H + 2 * padH - kH) / dH + 1;
+	if (oW < 1 || oH < 1)
+		THError("Given input size: (%dx%dx%d). Calculated output size: (%dx%dx%d). Output size is too small",
+			Ci, H, W, Co, oH, oW);
+	const int esize = thhip_esize(dtype);
+	const long K = (long)Ci * kH * kW;
+	if (K * kH * kW >= (1L << 32) || K > (1 << 30))
+		THError("thhip_conv2d: K = %ld too large", K);
+	/* 32-bit offsets inside the kernel: run the batch in slices whose input
+	 * and output stay below 2^31 bytes. */
+	const long in_img = (long)Ci * H * W, out_img = (long)Co * oH * oW;
+	long bmax = ((1L << 31) - 16) / (esize * (in_img > out_img ? in_img : out_img));
+	if (bmax < 1)
+		THError("thhip_conv2d: one image exceeds 2 GiB");
+	if ((long)oH * oW * bmax > (1L << 30))
+		bmax = (1L << 30) / ((long)oH * oW);
+	for (int b0 = 0; b0 < B; b0 += (int)bmax) {
+		const int bn = B - b0 < bmax ? B - b0 : (int)bmax;
+		ConvParams p;
+		memset(&p, 0, sizeof(p));
+		p.x = (const char *)x + (size_t)b0 * in_img * esize;
+		p.y = (char *)y + (size_t)b0 * out_img * esize;
+		p.wp = wpacked;
+		p.bias = bias;
+		p.B = bn; p.Ci = Ci; p.H = H; p.W = W; p.Co = Co; p.kH = kH; p.kW = kW;
+		p.dH = dH; p.dW = dW; p.padH = padH; p.padW = padW; p.oH = oH; p.oW = oW;
+		p.K = (int)K;
+		p.KC = conv_kc((int)K, dtype);
+		p.N = bn * oH * oW;
+		p.oHW = oH * oW;
+		p.HW = H * W;
+		p.kHW = kH * kW;
+		p.magic_khw = conv_magic(kH * kW);
+		p.magic_kw = conv_magic(kW);
+		p.act = act; p.thr = thr; p.val = val;
+		p.x_bytes = (unsigned)(bn * in_img * esize);
+		if (u8) {
+			p.rowsum = (const int *)((const char *)wpacked + thhip_conv_packed_bytes(Co, (int)K, THHIP_U8));
+			p.addend = u8->addend;
+			p.zero = u8->zero;
+			p.offA = 128 + u8->a_off;
+			p.offB = 128 + u8->b_off;
+			p.c_off = u8->c_off; p.c_mult = u8->c_mult; p.c_shift = u8->c_shift;
+			p.ithr = u8->ithr; p.ival = u8->ival;
+			ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * Co * (double)K * p.N);
+			conv_dispatch<THHIP_U8>(p);
+		} else {
+			ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N);
+			THHIP_DISPATCH_FLOAT(dtype, conv_dispatch<DT>(p));
+		}
+	}
+}
+
+extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype)
+{
+	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
+		THError("thhip_conv2d: unsupported dtype %d", dtype);
+	conv_run(x, wpacked, bias, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0);
+}
+
+/* uint8 codes [Co][K] -> (code - 128) as signed bytes in the packed layout,
+ * followed by the per-row sums of the re-centred codes. */
+extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int K)
+{
+	const int chunk = 32, vec = 16, KC = conv_kc(K, THHIP_U8);
+	const size_t bytes = thhip_conv_packed_bytes(Co, K, THHIP_U8);
+	const size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
+	const size_t total = bytes + mpad * sizeof(int);
+	unsigned char *host = (unsigned char *)calloc(1, total);
+	if (!host)
+		THError("thhip_conv_pack_weight_u8: out of host memory (%zu bytes)", total);
+	int *rowsum = (int *)(host + bytes);
+	for (int m = 0; m < Co; m++) {
+		const int mb = m >> 5, mi = m & 31;
+		int sum = 0;
+		for (int k = 0; k < K; k++) {
+			const int kc = k / chunk, h = (k % chunk) / vec, e = k % vec;
+			const size_t idx = ((((size_t)mb * KC + kc) * 2 + h) * 32 + mi) * vec + e;
+			const int c = (int)w[(size_t)m * K + k] - 128;
+			host[idx] = (unsigned char)(signed char)c;
+			sum += c;
+		}
+		rowsum[m] = sum;
+	}
+	void *dev = thhip_malloc(total);
+	thhip_memcpy_h2d(dev, host, total);
+	free(host);
+	return dev;
+}
+
+extern "C" void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
+	int act, int thr, int val)
+{
+	if (c_shift < 0 || c_shift > 31)
+		THError("thhip_conv2d_u8: shift %d out of range", c_shift);
+	ConvU8Args u8 = { addend, zero & 255, a_off, b_off, c_off, c_mult, c_shift, thr, val };
+	conv_run(x, wpacked, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
+}
+
+/* The reference's only entry into gemmlowp (lowp/gemm8.cc:4-17): host
+ * matrices, row-major A[m][k], B[k][n], C[m][n].  Run as a 1x1 "convolution"
+ * over an image of n positions (oH = 1, oW = n), without bias add. */
+extern "C" void lowpgemm(const int is_a_transposed, const int is_b_transposed, const int is_c_transposed,
+	const int m, const int n, const int k,
+	const unsigned char *a, const unsigned char *b, unsigned char *c,
+	const int lda, const int ldb, const int ldc,
+	const int a_offset, const int b_offset, const int c_offset,
+	const int c_mult, const int c_shift)
+{
+	if (!is_a_transposed || !is_b_transposed || !is_c_transposed)
+		THError("lowpgemm: only the all-transposed (row-major) form of lowp_basic.c:314-320 is implemented");
+	if (m < 1 || n < 1 || k < 1 || lda < k || ldb < n || ldc < n)
+		THError("lowpgemm: bad sizes");
+	unsigned char *wtmp = 0, *btmp = 0, *ctmp = 0;
+	const unsigned char *ap = a, *bp = b;
+	if (lda != k) {
+		wtmp = (unsigned char *)malloc((size_t)m * k);
+		for (int i = 0; i < m; i++)
+			memcpy(wtmp + (size_t)i * k, a + (size_t)i * lda, k);
+		ap = wtmp;
+	}
+	if (ldb != n) {
+		btmp = (unsigned char *)malloc((size_t)k * n);
+		for (int i = 0; i < k; i++)
+			memcpy(btmp + (size_t)i * n, b + (size_t)i * ldb, n);
+		bp = btmp;
+	}
+	void *wp = thhip_conv_pack_weight_u8(ap, m, k);
+	unsigned char *dx = (unsigned char *)thhip_malloc((size_t)k * n);
+	unsigned char *dy = (unsigned char *)thhip_malloc((size_t)m * n);
+	thhip_memcpy_h2d(dx, bp, (size_t)k * n);
+	thhip_conv2d_u8(dx, wp, 0, dy, 1, k, 1, n, m, 1, 1, 1, 1, 0, 0, 0, a_offset, b_offset, c_offset, c_mult, c_shift, 0, 0, 0);
+	if (ldc != n) {
+		ctmp = (unsigned char *)malloc((size_t)m * n);
+		thhip_memcpy_d2h(ctmp, dy, (size_t)m * n);
+		for (int i = 0; i < m; i++)
+			memcpy(c + (size_t)i * ldc, ctmp + (size_t)i * n, n);
+	} else
+		thhip_memcpy_d2h(c, dy, (size_t)m * n);
+	thhip_free(wp);
+	thhip_free(dx);
+	thhip_free(dy);
+	free(wtmp);
+	free(btmp);
+	free(ctmp);
+}
+
+/* Packed weights -> row-major [Co][K] in the same dtype, on the device; used
+ * when a layer turns out to be a matrix-vector product (one output position). */
+template <typename E, int CHUNK>
+__global__ void conv_unpack_rows_kernel(const E *wp, E *rows, int Co, int K, int KC)
+{
+	constexpr int VEC = CHUNK / 2;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long total = (long)Co * K, step = (long)gridDim.x * blockDim.x;
+	for (; i < total; i += step) {
+		const int m = (int)(i / K), k = (int)(i % K);
+		const int mb = m >> 5, mi = m & 31;
+		const int kc = k / CHUNK, h = (k % CHUNK) / VEC, e = k % VEC;
+		rows[i] = wp[((((size_t)mb * KC + kc) * 2 + h) * 32 + mi) * VEC + e];
+	}
+}
+
+extern "C" void *thhip_conv_unpack_rows(const void *wpacked, int Co, int K, int dtype)
+{
+	const int KC = conv_kc(K, dtype);
+	const long total = (long)Co * K;
+	void *rows = thhip_malloc((size_t)total * thhip_esize(dtype));
+	long blocks = (total + 255) / 256;
+	if (blocks > 65536)
+		blocks = 65536;
+	if (dtype == THHIP_F32)
+		conv_unpack_rows_kernel<float, 8><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
+			(const float *)wpacked, (float *)rows, Co, K, KC);
+	else if (dtype == THHIP_F16 || dtype == THHIP_BF16)
+		conv_unpack_rows_kernel<unsigned short, 16><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
+			(const unsigned short *)wpacked, (unsigned short *)rows, Co, K, KC);
+	else
+		THError("thhip_conv_unpack_rows: unsupported dtype %d", dtype);
+	hipcheck(hipGetLastError());
+	return rows;
+}

@@ -1,0 +1,534 @@
+/*
+ * The small HBM-bound kernels that keep activations on the device between
+ * the GEMM-shaped modules: Threshold, max / average pooling, SoftMax, batch
+ * normalisation, the two-input table add, dtype conversion, 8-bit image
+ * loading, and the uint8 (LOWP) counterparts.  Each one reads its input once
+ * and writes its output once; lanes run along the innermost (W) dimension.
+ */
+#include <float.h>
+#include <string.h>
+#include <math.h>
+#include "thhip_internal.h"
+
+#define EW_THREADS 256
+
+static inline dim3 ew_grid(long n, int per_thread = 1)
+{
+	long blocks = (n + (long)EW_THREADS * per_thread - 1) / ((long)EW_THREADS * per_thread);
+	if (blocks < 1)
+		blocks = 1;
+	if (blocks > 65536 * 16)
+		blocks = 65536 * 16;
+	return dim3((unsigned)blocks);
+}
+
+/* ---------------- Threshold (modules/Threshold.c:38-63) ---------------- */
+
+template <int DT>
+__global__ void threshold_kernel(const void *x, void *y, long n, float thr, float val, float alpha, int mode)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < n; i += step) {
+		const float v = ThhipElem<DT>::ld(x, i);
+		float r;
+		if (mode == 0)		/* in place: x <= thr -> val */
+			r = v <= thr ? val : v;
+		else if (mode == 1)	/* out of place, alpha != 0 */
+			r = v >= 0 ? v : v * alpha;
+		else			/* out of place */
+			r = v > thr ? v : val;
+		ThhipElem<DT>::st(y, i, r);
+	}
+}
+
+extern "C" void thhip_threshold(const void *x, void *y, long n, float thr, float val, float alpha, int inplace, int dtype)
+{
+	if (n <= 0)
+		return;
+	const int mode = inplace ? 0 : (alpha != 0 ? 1 : 2);
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * n * thhip_esize(dtype));
+	THHIP_DISPATCH_FLOAT(dtype, (threshold_kernel<DT><<<ew_grid(n, 4), dim3(EW_THREADS), 0, thhip_stream()>>>(
+		x, y, n, thr, val, alpha, mode)));
+}
+
+__global__ void threshold_u8_kernel(const unsigned char *x, unsigned char *y, long n, int thr, int val, int inplace)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < n; i += step) {
+		const int v = x[i];
+		/* lowp_Threshold.c:14-24: the two branches differ only in how they are
+		 * written; both give v > thr ? v : val */
+		y[i] = (unsigned char)((inplace ? !(v <= thr) : (v > thr)) ? v : val);
+	}
+}
+
+extern "C" void thhip_threshold_u8(const unsigned char *x, unsigned char *y, long n, int thr, int val, int inplace)
+{
+	if (n <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * n);
+	threshold_u8_kernel<<<ew_grid(n, 8), dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, n, thr, val, inplace);
+}
+
+/* ---------------- pooling ---------------- */
+
+/* Output extent: modules/SpatialMaxPooling.c:187-203 (float division, floor
+ * or ceil, drop a last window starting beyond the padded input). */
+extern "C" void thhip_pool_outsize(int H, int W, int kH, int kW, int dH, int dW, int padH, int padW, int ceil_mode,
+	int *oH, int *oW)
+{
+	long oh, ow;
+	if (ceil_mode) {
+		oh = (long)(ceilf((float)(H - kH + 2 * padH) / dH)) + 1;
+		ow = (long)(ceilf((float)(W - kW + 2 * padW) / dW)) + 1;
+	} else {
+		oh = (long)(floorf((float)(H - kH + 2 * padH) / dH)) + 1;
+		ow = (long)(floorf((float)(W - kW + 2 * padW) / dW)) + 1;
+	}
+	if (padW || padH) {
+		if ((oh - 1) * dH >= H + padH)
+			--oh;
+		if ((ow - 1) * dW >= W + padW)
+			--ow;
+	}
+	*oH = (int)oh;
+	*oW = (int)ow;
+}
+
+struct PoolParams {
+	int C, H, W, oH, oW, kH, kW, dH, dW, padH, padW;
+	long total;
+};
+
+template <int DT>
+__global__ void maxpool_kernel(const void *x, void *y, PoolParams p)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < p.total; i += step) {
+		const int ox = (int)(i % p.oW);
+		const long t = i / p.oW;
+		const int oy = (int)(t % p.oH);
+		const long plane = t / p.oH;
+		int hs = oy * p.dH - p.padH, ws = ox * p.dW - p.padW;
+		const int he = min(hs + p.kH, p.H), we = min(ws + p.kW, p.W);
+		hs = max(hs, 0);
+		ws = max(ws, 0);
+		const long base = plane * p.H * p.W;
+		if constexpr (DT == THHIP_U8) {
+			int m = 0;	/* lowp_SpatialMaxPooling.c:28 */
+			for (int yy = hs; yy < he; yy++)
+				for (int xx = ws; xx < we; xx++)
+					m = max(m, (int)((const unsigned char *)x)[base + (long)yy * p.W + xx]);
+			((unsigned char *)y)[i] = (unsigned char)m;
+		} else {
+			float m = -FLT_MAX;	/* SpatialMaxPooling.c:96 */
+			for (int yy = hs; yy < he; yy++)
+				for (int xx = ws; xx < we; xx++) {
+					const float v = ThhipElem<DT>::ld(x, base + (long)yy * p.W + xx);
+					if (v > m)
+						m = v;
+				}
+			ThhipElem<DT>::st(y, i, m);
+		}
+	}
+}
+
+extern "C" void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype)
+{
+	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * C * oH * oW };
+	if (p.total <= 0)
+		return;
+	const double esz = thhip_esize(dtype);
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, esz * ((double)B * C * H * W + (double)p.total));
+	const dim3 grid = ew_grid(p.total);
+	switch (dtype) {
+	case THHIP_F32: maxpool_kernel<THHIP_F32><<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, p); break;
+	case THHIP_F16: maxpool_kernel<THHIP_F16><<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, p); break;
+	case THHIP_BF16: maxpool_kernel<THHIP_BF16><<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, p); break;
+	case THHIP_U8: maxpool_kernel<THHIP_U8><<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, p); break;
+	default: THError("thhip_maxpool: unsupported dtype %d", dtype);
+	}
+}
+
+/* modules/SpatialAveragePooling.c:156-203 */
+template <int DT>
+__global__ void avgpool_kernel(const void *x, void *y, PoolParams p, int count_include_pad)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < p.total; i += step) {
+		const int ox = (int)(i % p.oW);
+		const long t = i / p.oW;
+		const int oy = (int)(t % p.oH);
+		const long plane = t / p.oH;
+		int hs = oy * p.dH - p.padH, ws = ox * p.dW - p.padW;
+		int he = min(hs + p.kH, p.H + p.padH), we = min(ws + p.kW, p.W + p.padW);
+		const int pool = (he - hs) * (we - ws);
+		hs = max(hs, 0);
+		ws = max(ws, 0);
+		he = min(he, p.H);
+		we = min(we, p.W);
+		const int div = count_include_pad ? pool : (he - hs) * (we - ws);
+		const long base = plane * p.H * p.W;
+		float sum = 0;
+		for (int yy = hs; yy < he; yy++)
+			for (int xx = ws; xx < we; xx++)
+				sum += ThhipElem<DT>::ld(x, base + (long)yy * p.W + xx);
+		ThhipElem<DT>::st(y, i, sum / (float)div);
+	}
+}
+
+extern "C" void thhip_avgpool(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int count_include_pad, int dtype)
+{
+	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * C * oH * oW };
+	if (p.total <= 0)
+		return;
+	const double esz = thhip_esize(dtype);
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, esz * ((double)B * C * H * W + (double)p.total));
+	THHIP_DISPATCH_FLOAT(dtype, (avgpool_kernel<DT><<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>(
+		x, y, p, count_include_pad)));
+}
+
+/* ---------------- SoftMax ---------------- */
+
+/* THExpMinusApprox, thbasic.c:462-491 */
+__device__ __forceinline__ double exp_minus_approx(double x)
+{
+	/* separately rounded steps, as a CPU build without fused multiply-add gives */
+#pragma clang fp contract(off)
+	if (x < 13.0) {
+		double y = 1.0 + x * (0.125 + x * (0.0078125 + x * (0.00032552083 + x * 1.0172526e-5)));
+		y *= y;
+		y *= y;
+		y *= y;
+		return 1 / y;
+	}
+	return 0;
+}
+
+/* modules/SoftMax.c:24-90: one wavefront per (frame, position). */
+template <int DT>
+__global__ __launch_bounds__(64) void softmax_kernel(const void *x, void *y, long dim, long stride)
+{
+	const long t = blockIdx.x;
+	const long base = (t / stride) * dim * stride + t % stride;
+	const int lane = threadIdx.x;
+	float m = -FLT_MAX;
+	for (long d = lane; d < dim; d += 64)
+		m = fmaxf(m, ThhipElem<DT>::ld(x, base + d * stride));
+	for (int off = 32; off > 0; off >>= 1)
+		m = fmaxf(m, __shfl_xor(m, off, 64));
+	float sum = 0;
+	for (long d = lane; d < dim; d += 64) {
+		const float z = (float)exp_minus_approx((double)(m - ThhipElem<DT>::ld(x, base + d * stride)));
+		sum += z;
+	}
+	for (int off = 32; off > 0; off >>= 1)
+		sum += __shfl_xor(sum, off, 64);
+	const float inv = 1 / sum;
+	for (long d = lane; d < dim; d += 64) {
+		const float z = (float)exp_minus_approx((double)(m - ThhipElem<DT>::ld(x, base + d * stride)));
+		ThhipElem<DT>::st(y, base + d * stride, z * inv);
+	}
+}
+
+extern "C" void thhip_softmax(const void *x, void *y, long nframe, long dim, long stride, int dtype)
+{
+	const long npos = nframe * stride;
+	if (npos <= 0 || dim <= 0)
+		return;
+	if (npos > 0x7fffffffL)
+		THError("thhip_softmax: too many positions");
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * npos * dim * thhip_esize(dtype));
+	THHIP_DISPATCH_FLOAT(dtype, (softmax_kernel<DT><<<dim3((unsigned)npos), dim3(64), 0, thhip_stream()>>>(
+		x, y, dim, stride)));
+}
+
+/* lowp/lowp_SoftMax.c:3-89.  The exponent argument keeps the tensor offset,
+ * and the float running sum is taken in index order by one lane so that the
+ * codes match a sequential evaluation bit for bit. */
+#define SOFTMAX_U8_MAXDIM 8192
+__global__ __launch_bounds__(64) void softmax_u8_kernel(const unsigned char *x, unsigned char *y, long dim, long stride,
+	float invmult, float sub, int single, float *max_out)
+{
+	__shared__ float tmp[SOFTMAX_U8_MAXDIM];
+	__shared__ float s_scale, s_max;
+	const long t = blockIdx.x;
+	const long base = (t / stride) * dim * stride + t % stride;
+	const int lane = threadIdx.x;
+	int qmax = 0;
+	for (long d = lane; d < dim; d += 64)
+		qmax = max(qmax, (int)x[base + d * stride]);
+	for (int off = 32; off > 0; off >>= 1)
+		qmax = max(qmax, __shfl_xor(qmax, off, 64));
+	for (long d = lane; d < dim; d += 64) {
+		const float arg = __fadd_rn(__fmul_rn((float)(qmax - (int)x[base + d * stride]), invmult), sub);
+		tmp[d] = (float)exp_minus_approx((double)arg);
+	}
+	__syncthreads();
+	if (lane == 0) {
+		float sum = 0;
+		for (long d = 0; d < dim; d++)
+			sum = __fadd_rn(sum, tmp[d]);
+		s_scale = 1 / sum;
+	}
+	__syncthreads();
+	const float scale = s_scale;
+	if (!single) {
+		for (long d = lane; d < dim; d += 64)
+			y[base + d * stride] = (unsigned char)(int)__fmul_rn(255.0f, __fmul_rn(tmp[d], scale));
+		return;
+	}
+	float mx = 0;
+	for (long d = lane; d < dim; d += 64) {
+		tmp[d] = __fmul_rn(tmp[d], scale);
+		mx = fmaxf(mx, tmp[d]);
+	}
+	for (int off = 32; off > 0; off >>= 1)
+		mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+	if (lane == 0) {
+		s_max = mx;
+		*max_out = mx;
+	}
+	__syncthreads();
+	const float rmax = 1 / s_max;
+	for (long d = lane; d < dim; d += 64)
+		y[base + d * stride] = (unsigned char)(int)__fmul_rn(__fmul_rn(255.0f, tmp[d]), rmax);
+}
+
+extern "C" float thhip_softmax_u8(const unsigned char *x, unsigned char *y, long nframe, long dim, long stride,
+	float in_mult, float in_sub)
+{
+	const long npos = nframe * stride;
+	if (npos <= 0 || dim <= 0)
+		return 0;
+	if (dim > SOFTMAX_U8_MAXDIM)
+		THError("thhip_softmax_u8: dim %ld exceeds %d", dim, SOFTMAX_U8_MAXDIM);
+	const float invmult = in_mult ? 1 / in_mult : 0;
+	const int single = npos == 1;
+	float *dmax = single ? (float *)thhip_malloc(4) : 0;
+	{
+		ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * npos * dim);
+		softmax_u8_kernel<<<dim3((unsigned)npos), dim3(64), 0, thhip_stream()>>>(x, y, dim, stride, invmult, in_sub,
+			single, dmax);
+	}
+	if (!single)
+		return 255;
+	float mx = 0;
+	thhip_memcpy_d2h(&mx, dmax, 4);
+	thhip_free(dmax);
+	return 255 / mx;
+}
+
+/* ---------------- batch normalisation ---------------- */
+
+/* modules/SpatialBatchNormalization.c:78-109: y = ((x - mean) * invstd) * w + b */
+template <int DT>
+__global__ void batchnorm_kernel(const void *x, void *y, long total, long C, long HW,
+	const float *mean, const float *invstd, const float *weight, const float *bias)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total; i += step) {
+		const long f = (i / HW) % C;
+		const float w = weight ? weight[f] : 1.0f, b = bias ? bias[f] : 0.0f;
+		const float v = ThhipElem<DT>::ld(x, i);
+		ThhipElem<DT>::st(y, i, ((v - mean[f]) * invstd[f]) * w + b);
+	}
+}
+
+extern "C" void thhip_batchnorm(const void *x, void *y, long B, long C, long HW,
+	const float *mean, const float *invstd, const float *weight, const float *bias, int dtype)
+{
+	const long total = B * C * HW;
+	if (total <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * total * thhip_esize(dtype));
+	THHIP_DISPATCH_FLOAT(dtype, (batchnorm_kernel<DT><<<ew_grid(total, 4), dim3(EW_THREADS), 0, thhip_stream()>>>(
+		x, y, total, C, HW, mean, invstd, weight, bias)));
+}
+
+/* ---------------- two-input table add (modules/CAddTable.c:59-70) ---------------- */
+
+template <int DT>
+__global__ void axpby2_kernel(const void *a, const void *b, void *y, long na, long nb, float sign, int act)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < na; i += step) {
+		float v = ThhipElem<DT>::ld(a, i);
+		if (i < nb)
+			v = v + sign * ThhipElem<DT>::ld(b, i);
+		if (act)
+			v = v > 0.0f ? v : 0.0f;
+		ThhipElem<DT>::st(y, i, v);
+	}
+}
+
+extern "C" void thhip_axpby2(const void *a, const void *b, void *y, long na, long nb, float sign, int act, int dtype)
+{
+	if (na <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, (2.0 * na + nb) * thhip_esize(dtype));
+	THHIP_DISPATCH_FLOAT(dtype, (axpby2_kernel<DT><<<ew_grid(na, 4), dim3(EW_THREADS), 0, thhip_stream()>>>(
+		a, b, y, na, nb, sign, act)));
+}
+
+/* ---------------- dtype conversion ---------------- */
+
+template <int SD, int DD>
+__global__ void convert_kernel(const void *src, void *dst, long n)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < n; i += step) {
+		float v;
+		if constexpr (SD == THHIP_U8)
+			v = (float)((const unsigned char *)src)[i];
+		else
+			v = ThhipElem<SD>::ld(src, i);
+		ThhipElem<DD>::st(dst, i, v);
+	}
+}
+
+extern "C" void thhip_convert(const void *src, int sd, void *dst, int dd, long n)
+{
+	if (n <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)n * (thhip_esize(sd) + thhip_esize(dd)));
+	const dim3 grid = ew_grid(n, 4), blk(EW_THREADS);
+	hipStream_t s = thhip_stream();
+#define CV(S, D) if (sd == S && dd == D) { convert_kernel<S, D><<<grid, blk, 0, s>>>(src, dst, n); return; }
+	CV(THHIP_F32, THHIP_F32) CV(THHIP_F32, THHIP_F16) CV(THHIP_F32, THHIP_BF16)
+	CV(THHIP_F16, THHIP_F32) CV(THHIP_BF16, THHIP_F32) CV(THHIP_U8, THHIP_F32)
+#undef CV
+	THError("thhip_convert: unsupported conversion %d -> %d", sd, dd);
+}
+
+/* ---------------- 8-bit image -> normalised planar float (thapi.c:20-46) ---------------- */
+
+template <int DT>
+__global__ void rgb2float_kernel(void *dst, const unsigned char *src, int width, int height, int stride, int cp,
+	floatx4 mean, floatx4 std1, int bgr)
+{
+	const long total = (long)cp * width * height;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total; i += step) {
+		const int j = (int)(i % width);
+		const long t = i / width;
+		const int r = (int)(t % height);
+		const int c = (int)(t / height);
+		const int sc = bgr ? cp - 1 - c : c;
+		const float byte = (float)src[sc + cp * j + (long)stride * r];
+		/* (byte * (1/255) - mean) * (1/std), three separately rounded steps */
+		const float v = __fmul_rn(__fsub_rn(__fmul_rn(byte, 0.003921568f), mean[c]), std1[c]);
+		ThhipElem<DT>::st(dst, i, v);
+	}
+}
+
+extern "C" void thhip_rgb2float(void *dst, const unsigned char *src, int width, int height, int stride, int cp,
+	const float *mean, const float *std, int bgr, int dtype)
+{
+	if (cp < 1 || cp > 3)
+		THError("thhip_rgb2float: %d colour planes", cp);
+	floatx4 m = { 0, 0, 0, 0 }, s = { 1, 1, 1, 1 };
+	for (int i = 0; i < cp; i++) {
+		m[i] = mean[i];
+		s[i] = 1 / std[i];
+	}
+	const long total = (long)cp * width * height;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)total * (1 + thhip_esize(dtype)));
+	THHIP_DISPATCH_FLOAT(dtype, (rgb2float_kernel<DT><<<ew_grid(total), dim3(EW_THREADS), 0, thhip_stream()>>>(
+		dst, src, width, height, stride, cp, m, s, bgr)));
+}
+
+/* ---------------- uint8 quantise / de-quantise (lowp/lowp_basic.c:5-58) ---------------- */
+
+__global__ void minmax_kernel(const float *x, long n, unsigned *out)
+{
+	/* out[0]: bits of the most negative value, out[1]: bits of the largest
+	 * positive value; both start at +0.0f, so zero is always in range
+	 * (lowp_basic.c:17).  Among same-sign floats the bit patterns order like
+	 * the magnitudes. */
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	float mn = 0, mx = 0;
+	for (; i < n; i += step) {
+		const float v = x[i];
+		if (v < mn)
+			mn = v;
+		if (v > mx)
+			mx = v;
+	}
+	for (int off = 32; off > 0; off >>= 1) {
+		mn = fminf(mn, __shfl_xor(mn, off, 64));
+		mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+	}
+	if ((threadIdx.x & 63) == 0) {
+		if (mn < 0)
+			atomicMax(&out[0], __float_as_uint(mn));
+		if (mx > 0)
+			atomicMax(&out[1], __float_as_uint(mx));
+	}
+}
+
+__global__ void quantize_kernel(const float *x, unsigned char *q, long n, float mult, float zero)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < n; i += step)
+		q[i] = (unsigned char)(int)__fsub_rn(roundf(__fmul_rn(x[i], mult)), zero);
+}
+
+extern "C" void thhip_quantize(const float *x, unsigned char *q, long n, float *mult_out, float *sub_out)
+{
+	unsigned bits[2] = { 0, 0 };
+	unsigned *d = (unsigned *)thhip_malloc(8);
+	thhip_memcpy_h2d(d, bits, 8);
+	if (n > 0) {
+		long blocks = (n + 255) / 256;
+		if (blocks > 2048)
+			blocks = 2048;
+		ThhipLaunchScope scope(THHIP_FAM_OTHER, 4.0 * n);
+		minmax_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(x, n, d);
+	}
+	thhip_memcpy_d2h(bits, d, 8);
+	thhip_free(d);
+	float mn, mx, mult;
+	memcpy(&mn, &bits[0], 4);
+	memcpy(&mx, &bits[1], 4);
+	if (mx - mn > 0)
+		mult = (float)(255.0 / (mx - mn));	/* lowp_basic.c:25-27 */
+	else
+		mult = 0;
+	const float zero = roundf(mn * mult);
+	if (n > 0) {
+		ThhipLaunchScope scope(THHIP_FAM_OTHER, 5.0 * n);
+		quantize_kernel<<<ew_grid(n, 4), dim3(EW_THREADS), 0, thhip_stream()>>>(x, q, n, mult, zero);
+	}
+	*mult_out = mult;
+	*sub_out = mn;
+}
+
+__global__ void dequantize_kernel(const unsigned char *q, float *x, long n, float invmult, float sub)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < n; i += step)
+		x[i] = __fadd_rn(__fmul_rn((float)q[i], invmult), sub);
+}
+
+extern "C" void thhip_dequantize(const unsigned char *q, float *x, long n, float mult, float sub)
+{
+	if (n <= 0)
+		return;
+	const float invmult = mult ? (float)(1.0 / mult) : 0;	/* lowp_basic.c:54 */
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 5.0 * n);
+	dequantize_kernel<<<ew_grid(n, 4), dim3(EW_THREADS), 0, thhip_stream()>>>(q, x, n, invmult, sub);
+}

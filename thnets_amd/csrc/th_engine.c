@@ -1,0 +1,882 @@
+/*
+ * The MI355X engine: turns a host `struct network` into one whose modules
+ * run on the GPU, the way THcudnn_ToCUDNN (cudnn/cudnn_basic.c:189-303) and
+ * THLowp_ToLowp (lowp/lowp_basic.c:133-212) re-target a network, and provides
+ * the updateOutput of every module type the convolution / Linear / LOWP path
+ * traverses.  Host code only: every number is produced by a kernel behind the
+ * thhip_* C ABI.
+ *
+ * Differences from the reference engines that a caller can observe:
+ *   - activations stay on the device between modules and module outputs are
+ *     kept (not freed per layer as thapi.c:205-209 does), so repeated forwards
+ *     allocate nothing once shapes are known;
+ *   - a Threshold that follows a convolution / Linear is folded into that
+ *     module's epilogue and becomes a pass-through;
+ *   - nested containers (Sequential, ConcatTable + CAddTable) are converted
+ *     recursively; the reference's GPU engines refuse them;
+ *   - the uint8 engine keeps each module's (mult, sub) with the module, works
+ *     at any batch size and for any number of forwards.
+ */
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+#include "th_engine.h"
+
+static int g_halfmode;	/* 0 fp32, 1 fp16, 2 bf16: THHipHalfFloat */
+
+int THHipHalfFloat(int enable)
+{
+	if (enable < 0 || enable > 2)
+		return ERR_NOTIMPLEMENTED;
+	g_halfmode = enable;
+	return 0;
+}
+
+int thhip_engine_dtype(void)
+{
+	return g_halfmode == 1 ? THHIP_F16 : g_halfmode == 2 ? THHIP_BF16 : THHIP_F32;
+}
+
+static int esize_of(int dtype)
+{
+	return dtype == THHIP_F32 ? 4 : dtype == THHIP_U8 ? 1 : 2;
+}
+
+struct hipnet *hipnet_of(struct module *m)
+{
+	return (struct hipnet *)m->net;
+}
+
+struct hipmod *hipmod_of(struct module *m)
+{
+	struct hipnet *hn = hipnet_of(m);
+	return &hn->hm[m - hn->pub.modules];
+}
+
+void *thhip_tensor_ptr(THFloatTensor *t, int dtype)
+{
+	if (!t || !t->storage || !t->storage->data)
+		THError("HIP engine: tensor without storage");
+	if (t->storage->mustfree != TH_MUSTFREE_HIP)
+		THError("HIP engine: module input is not a device tensor (create it with THHipTensor_newFromFloatTensor)");
+	return (char *)t->storage->data + t->storageOffset * esize_of(dtype);
+}
+
+/* Gives module m a contiguous device output of the given shape, reusing its
+ * allocation whenever it is large enough. */
+static void *out_resize(struct module *m, int dtype, int nd, const long *size)
+{
+	struct hipmod *hm = hipmod_of(m);
+	THFloatTensor *o = m->output;
+	long n = 1, stride = 1;
+	for (int i = 0; i < nd; i++)
+		n *= size[i];
+	size_t bytes = (size_t)n * esize_of(dtype);
+	if (!o->storage || o->storage->mustfree != TH_MUSTFREE_HIP || hm->cap < bytes || !hm->owns_output) {
+		THFloatStorage *s = malloc(sizeof(*s));
+		s->data = thhip_malloc(bytes);
+		s->nref = 1;
+		s->mustfree = TH_MUSTFREE_HIP;
+		if (o->storage)
+			thhip_storage_release(o->storage);
+		o->storage = s;
+		hm->cap = bytes;
+		hm->owns_output = 1;
+	}
+	o->storageOffset = 0;
+	o->nDimension = nd;
+	for (int i = nd - 1; i >= 0; i--) {
+		o->size[i] = size[i];
+		o->stride[i] = stride;
+		stride *= size[i];
+	}
+	return o->storage->data;
+}
+
+/* Output becomes another view of the input (in-place modules, View, Dropout). */
+static void out_alias(struct module *m, THFloatTensor *in)
+{
+	hipmod_of(m)->owns_output = 0;
+	THFloatTensor_set(m->output, in);
+}
+
+/* ------------------------------------------------------------------ */
+/* fp32 / fp16 / bf16 modules                                          */
+/* ------------------------------------------------------------------ */
+
+struct convshape { int B, H, W, outnd; };
+
+/* Input shapes a convolution accepts: 3-D (one image) and 4-D as
+ * SpatialConvolutionMM.c:146-152; vectors and matrices are taken as 1x1
+ * images the way the GPU engines run Linear (cudnn_SpatialConvolution.c:41-47,
+ * lowp_SpatialConvolution.c:138-147). */
+static struct convshape conv_input_shape(struct module *m, THFloatTensor *in)
+{
+	struct convshape s;
+	long planes;
+	switch (in->nDimension) {
+	case 1: s.B = 1; planes = in->size[0]; s.H = s.W = 1; break;
+	case 2: s.B = (int)in->size[0]; planes = in->size[1]; s.H = s.W = 1; break;
+	case 3: s.B = 1; planes = in->size[0]; s.H = (int)in->size[1]; s.W = (int)in->size[2]; break;
+	case 4: s.B = (int)in->size[0]; planes = in->size[1]; s.H = (int)in->size[2]; s.W = (int)in->size[3]; break;
+	default: THError("convolution input must have 1 to 4 dimensions"); planes = 0;
+	}
+	s.outnd = in->nDimension;
+	if (planes != m->SpatialConvolution.nInputPlane)
+		THError("nInputPlane %ld does not match input planes %ld", (long)m->SpatialConvolution.nInputPlane, planes);
+	return s;
+}
+
+static void *conv_out(struct module *m, int dtype, const struct convshape *s, int Co, int oH, int oW)
+{
+	long sz[4];
+	switch (s->outnd) {
+	case 1: sz[0] = Co; return out_resize(m, dtype, 1, sz);
+	case 2: sz[0] = s->B; sz[1] = Co; return out_resize(m, dtype, 2, sz);
+	case 3: sz[0] = Co; sz[1] = oH; sz[2] = oW; return out_resize(m, dtype, 3, sz);
+	default: sz[0] = s->B; sz[1] = Co; sz[2] = oH; sz[3] = oW; return out_resize(m, dtype, 4, sz);
+	}
+}
+
+static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	struct SpatialConvolution *c = &m->SpatialConvolution;
+	const int dt = hn->dtype;
+	struct convshape s = conv_input_shape(m, in);
+	const int oW = (s.W + 2 * c->padW - c->kW) / c->dW + 1;
+	const int oH = (s.H + 2 * c->padH - c->kH) / c->dH + 1;
+	if (oW < 1 || oH < 1)
+		THError("Given input size: (%dx%dx%d). Calculated output size: (%dx%dx%d). Output size is too small",
+			c->nInputPlane, s.H, s.W, c->nOutputPlane, oH, oW);
+	const void *x = thhip_tensor_ptr(in, dt);
+	void *y = conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
+	const int K = c->nInputPlane * c->kH * c->kW;
+	if (s.B == 1 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W) {
+		/* one output position: a matrix-vector product over the flattened
+		 * input, bound by reading the weights once */
+		if (!hm->wrow)
+			hm->wrow = thhip_conv_unpack_rows(hm->wpacked, c->nOutputPlane, K, dt);
+		thhip_gemv(x, hm->wrow, hm->bias, y, K, c->nOutputPlane, hm->fused_act, hm->thr, hm->val, dt);
+	} else
+		thhip_conv2d(x, hm->wpacked, hm->bias, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, hm->fused_act, hm->thr, hm->val, dt);
+	return m->output;
+}
+
+static THFloatTensor *Hip_Threshold_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	struct Threshold *t = &m->Threshold;
+	const int dt = hn->dtype;
+	if (hm->passthrough) {	/* already applied by the producer's epilogue */
+		out_alias(m, in);
+		return m->output;
+	}
+	const long n = THFloatTensor_nElement(in);
+	void *x = thhip_tensor_ptr(in, dt);
+	if (t->inplace == 1) {
+		thhip_threshold(x, x, n, t->threshold, t->val, t->alpha, 1, dt);
+		out_alias(m, in);
+	} else {
+		void *y = out_resize(m, dt, in->nDimension, in->size);
+		thhip_threshold(x, y, n, t->threshold, t->val, t->alpha, 0, dt);
+	}
+	return m->output;
+}
+
+struct planes { int B, C, H, W, nd; };
+
+static struct planes planes_of(THFloatTensor *in, const char *who)
+{
+	struct planes p;
+	if (in->nDimension == 3) {
+		p.B = 1; p.C = (int)in->size[0]; p.H = (int)in->size[1]; p.W = (int)in->size[2];
+	} else if (in->nDimension == 4) {
+		p.B = (int)in->size[0]; p.C = (int)in->size[1]; p.H = (int)in->size[2]; p.W = (int)in->size[3];
+	} else
+		THError("%s: 3D or 4D (batch mode) tensor expected", who);
+	p.nd = in->nDimension;
+	return p;
+}
+
+static void *planes_out(struct module *m, int dtype, const struct planes *p, int oH, int oW)
+{
+	long sz[4];
+	if (p->nd == 3) {
+		sz[0] = p->C; sz[1] = oH; sz[2] = oW;
+		return out_resize(m, dtype, 3, sz);
+	}
+	sz[0] = p->B; sz[1] = p->C; sz[2] = oH; sz[3] = oW;
+	return out_resize(m, dtype, 4, sz);
+}
+
+static THFloatTensor *Hip_SpatialMaxPooling_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct SpatialMaxPooling *q = &m->SpatialMaxPooling;
+	struct planes p = planes_of(in, "SpatialMaxPooling");
+	int oH, oW;
+	q->iwidth = p.W;
+	q->iheight = p.H;
+	thhip_pool_outsize(p.H, p.W, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, q->ceil_mode, &oH, &oW);
+	if (oH < 1 || oW < 1)
+		THError("SpatialMaxPooling: input %dx%d smaller than the window", p.H, p.W);
+	const void *x = thhip_tensor_ptr(in, hn->dtype);
+	void *y = planes_out(m, hn->dtype, &p, oH, oW);
+	thhip_maxpool(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, hn->dtype);
+	return m->output;
+}
+
+static THFloatTensor *Hip_SpatialAveragePooling_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct SpatialAveragePooling *q = &m->SpatialAveragePooling;
+	struct planes p = planes_of(in, "SpatialAveragePooling");
+	int kW = q->kW, kH = q->kH, oH, oW;
+	if (!(kW / 2 >= q->padW && kH / 2 >= q->padH))	/* SpatialAveragePooling.c:100-101 */
+		THError("pad should be smaller than half of kernel size");
+	if (kW == 0)
+		kW = p.W;	/* :116-119, global pooling */
+	if (kH == 0)
+		kH = p.H;
+	thhip_pool_outsize(p.H, p.W, kH, kW, q->dH, q->dW, q->padH, q->padW, q->ceil_mode, &oH, &oW);
+	if (!(p.W >= kW - 2 * q->padW && p.H >= kH - 2 * q->padH))
+		THError("input image smaller than kernel size");
+	const void *x = thhip_tensor_ptr(in, hn->dtype);
+	void *y = planes_out(m, hn->dtype, &p, oH, oW);
+	thhip_avgpool(x, y, p.B, p.C, p.H, p.W, oH, oW, kH, kW, q->dH, q->dW, q->padH, q->padW,
+		q->count_include_pad, hn->dtype);
+	return m->output;
+}
+
+/* frame / dim / stride rule of SoftMax.c:31-57 */
+static void softmax_shape(THFloatTensor *in, long *nframe, long *dim, long *stride)
+{
+	switch (in->nDimension) {
+	case 1: *nframe = 1; *dim = in->size[0]; *stride = 1; break;
+	case 2: *nframe = in->size[0]; *dim = in->size[1]; *stride = 1; break;
+	case 3: *nframe = 1; *dim = in->size[0]; *stride = in->size[1] * in->size[2]; break;
+	case 4: *nframe = in->size[0]; *dim = in->size[1]; *stride = in->size[2] * in->size[3]; break;
+	default: THError("1D, 2D, 3D or 4D tensor expected");
+	}
+}
+
+static THFloatTensor *Hip_SoftMax_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	long nframe, dim, stride;
+	softmax_shape(in, &nframe, &dim, &stride);
+	const void *x = thhip_tensor_ptr(in, hn->dtype);
+	void *y = out_resize(m, hn->dtype, in->nDimension, in->size);
+	thhip_softmax(x, y, nframe, dim, stride, hn->dtype);
+	return m->output;
+}
+
+static THFloatTensor *Hip_SpatialBatchNormalization_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	if (in->nDimension != 3 && in->nDimension != 4)
+		THError("SpatialBatchNormalization: 3D or 4D tensor expected");
+	const long B = in->nDimension == 4 ? in->size[0] : 1;
+	const long C = in->nDimension == 4 ? in->size[1] : in->size[0];
+	const long HW = THFloatTensor_nElement(in) / (B * C);
+	if (C != hm->bn_planes)
+		THError("SpatialBatchNormalization: %ld planes, module has %ld", C, hm->bn_planes);
+	const void *x = thhip_tensor_ptr(in, hn->dtype);
+	void *y = out_resize(m, hn->dtype, in->nDimension, in->size);
+	thhip_batchnorm(x, y, B, C, HW, hm->bn[0], hm->bn[1], hm->bn[2], hm->bn[3], hn->dtype);
+	return m->output;
+}
+
+/* View.c:48-100: pointer-only reshape. */
+static THFloatTensor *Hip_View_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct View *p = &m->View;
+	const long nElements = THFloatTensor_nElement(in);
+	out_alias(m, in);
+	THFloatTensor *o = m->output;
+	if (p->nDimension) {
+		long size[4], total = 1;
+		int ndim, i, j;
+		if (in->nDimension == 4) {
+			ndim = p->nDimension;
+			memcpy(size, p->size, sizeof(size));
+		} else {
+			ndim = p->nDimension - 1;
+			memcpy(size, p->size + 1, sizeof(size[0]) * 3);
+		}
+		for (i = 0; i < ndim; i++) {
+			if (size[i] == 0)
+				size[i] = in->size[i];
+			else if (size[i] < 0) {
+				size[i] = 1;
+				for (j = i; j < ndim; j++)
+					size[i] *= in->size[j];
+			}
+			total *= size[i];
+		}
+		if (total != nElements)
+			THError("Wrong number of elements in Reshape: %ld (input) vs %ld (reshaped)\n", nElements, total);
+		long stride = 1;
+		o->nDimension = ndim;
+		for (i = ndim - 1; i >= 0; i--) {
+			o->size[i] = size[i];
+			o->stride[i] = stride;
+			stride *= size[i];
+		}
+	} else {
+		long numElements = p->numElements;
+		long batch = in->nDimension == 4 ? in->size[0] : 1;
+		if (numElements == -1)
+			numElements = nElements / batch;
+		else
+			batch = nElements / numElements;
+		if (batch > 1) {
+			o->nDimension = 2;
+			o->size[0] = batch;
+			o->size[1] = numElements;
+			o->stride[0] = numElements;
+			o->stride[1] = 1;
+		} else {
+			o->nDimension = 1;
+			o->size[0] = numElements;
+			o->stride[0] = 1;
+		}
+	}
+	return o;
+}
+
+/* Dropout.c:37-53 at inference with v2 semantics is the identity. */
+static THFloatTensor *Hip_Identity_updateOutput(struct module *m, THFloatTensor *in)
+{
+	out_alias(m, in);
+	return m->output;
+}
+
+static THFloatTensor *run_network(struct network *net, THFloatTensor *in);
+
+/* Sequential.c:20-51 */
+static THFloatTensor *Hip_Sequential_updateOutput(struct module *m, THFloatTensor *in)
+{
+	in = run_network(m->Sequential.net, in);
+	out_alias(m, in);
+	return m->output;
+}
+
+/* ConcatTable.c:20-50: every branch sees the same input; the "table" handed
+ * on is the module itself. */
+static THFloatTensor *Hip_ConcatTable_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct network *net = m->ConcatTable.net;
+	for (int i = 0; i < net->nelem; i++)
+		net->modules[i].updateOutput(&net->modules[i], in);
+	return (THFloatTensor *)m;
+}
+
+/* CAddTable.c:32-86, arithmetic as shipped (see thhip_axpby2). */
+static THFloatTensor *Hip_CAddTable_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	struct module *table = (struct module *)in;
+	struct network *tn = table->ConcatTable.net;
+	const int nelem = tn->nelem, dt = hn->dtype;
+	struct module *mods = tn->modules;
+	const int sub = m->type == MT_CSubTable;
+	if (nelem < 1)
+		THError("CAddTable: empty table");
+	for (int i = 1; i < nelem; i++) {
+		if (mods[i].output->nDimension != mods[0].output->nDimension)
+			THError("Sum of tensors of different dimensionality");
+		for (int j = 0; j < mods[0].output->nDimension; j++)
+			if (mods[0].output->size[j] < mods[i].output->size[j])
+				THError("Sum of tensors of different sizes");
+	}
+	THFloatTensor *a = mods[0].output;
+	const long na = THFloatTensor_nElement(a);
+	void *y = out_resize(m, dt, a->nDimension, a->size);
+	if (nelem == 2) {
+		THFloatTensor *b = mods[1].output;
+		thhip_axpby2(thhip_tensor_ptr(a, dt), thhip_tensor_ptr(b, dt), y, na, THFloatTensor_nElement(b),
+			sub ? 1.0f : -1.0f, hm->fused_act, dt);
+	} else {
+		/* out = a, then every input including the first is added (subtracted) */
+		thhip_memcpy_d2d(y, thhip_tensor_ptr(a, dt), (size_t)na * esize_of(dt));
+		for (int i = 0; i < nelem; i++)
+			thhip_axpby2(y, thhip_tensor_ptr(mods[i].output, dt), y, na, THFloatTensor_nElement(mods[i].output),
+				sub ? -1.0f : 1.0f, (i == nelem - 1) ? hm->fused_act : 0, dt);
+	}
+	return m->output;
+}
+
+/* ------------------------------------------------------------------ */
+/* uint8 modules                                                       */
+/* ------------------------------------------------------------------ */
+
+/* THLowp_ScaleFloat, lowp_basic.c:214-222 */
+static int lowp_scale_float(float mult, float sub, float value)
+{
+	float scaled = (value - sub) * mult;
+	if (scaled < 0)
+		return 0;
+	if (scaled > 255)
+		return 255;
+	return (unsigned char)scaled;
+}
+
+static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	struct SpatialConvolution *c = &m->SpatialConvolution;
+	struct convshape s = conv_input_shape(m, in);
+	const int oW = (s.W + 2 * c->padW - c->kW) / c->dW + 1;
+	const int oH = (s.H + 2 * c->padH - c->kH) / c->dH + 1;
+	if (oW < 1 || oH < 1)
+		THError("Given input size: (%dx%dx%d). Calculated output size: (%dx%dx%d). Output size is too small",
+			c->nInputPlane, s.H, s.W, c->nOutputPlane, oH, oW);
+	/* THLowpTensor_mm, lowp_basic.c:309-320: the five integers gemmlowp gets */
+	const float im = hn->cur_mult, isub = hn->cur_sub;
+	const float om = hm->q_mult, osub = hm->q_sub;
+	float scaling = hm->wm * im / om;
+	int shift = roundf((log(scaling) / log(2))) + 10;
+	int mult = roundf((1 << shift) / scaling);
+	int offset = roundf(-osub * hm->wm * im);
+	int a_off = roundf(hm->wsub * hm->wm);
+	int b_off = roundf(isub * im);
+	int zero = roundf(-isub * im);	/* lowp_SpatialConvolution.c:101 */
+	int thr = 0, val = 0;
+	if (hm->fused_act) {	/* Lowp_Threshold on this module's output codes */
+		thr = lowp_scale_float(om, osub, hm->thr);
+		val = lowp_scale_float(om, osub, hm->val);
+	}
+	const void *x = thhip_tensor_ptr(in, THHIP_U8);
+	void *y = conv_out(m, THHIP_U8, &s, c->nOutputPlane, oH, oW);
+	thhip_conv2d_u8(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+		c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
+		hm->fused_act, thr, val);
+	hn->cur_mult = om;
+	hn->cur_sub = osub;
+	return m->output;
+}
+
+static THFloatTensor *HipLowp_Threshold_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	struct Threshold *t = &m->Threshold;
+	if (hm->passthrough) {
+		out_alias(m, in);
+		return m->output;
+	}
+	const int thr = lowp_scale_float(hn->cur_mult, hn->cur_sub, t->threshold);
+	const int val = lowp_scale_float(hn->cur_mult, hn->cur_sub, t->val);
+	const long n = THFloatTensor_nElement(in);
+	void *x = thhip_tensor_ptr(in, THHIP_U8);
+	if (t->inplace == 1) {
+		thhip_threshold_u8(x, x, n, thr, val, 1);
+		out_alias(m, in);
+	} else {
+		void *y = out_resize(m, THHIP_U8, in->nDimension, in->size);
+		thhip_threshold_u8(x, y, n, thr, val, 0);
+	}
+	hm->q_mult = hn->cur_mult;
+	hm->q_sub = hn->cur_sub;
+	return m->output;
+}
+
+static THFloatTensor *HipLowp_SpatialMaxPooling_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	struct SpatialMaxPooling *q = &m->SpatialMaxPooling;
+	struct planes p = planes_of(in, "SpatialMaxPooling");
+	int oH, oW;
+	thhip_pool_outsize(p.H, p.W, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, q->ceil_mode, &oH, &oW);
+	if (oH < 1 || oW < 1)
+		THError("SpatialMaxPooling: input %dx%d smaller than the window", p.H, p.W);
+	const void *x = thhip_tensor_ptr(in, THHIP_U8);
+	void *y = planes_out(m, THHIP_U8, &p, oH, oW);
+	thhip_maxpool(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, THHIP_U8);
+	hm->q_mult = hn->cur_mult;	/* lowp_SpatialMaxPooling.c:104-105 */
+	hm->q_sub = hn->cur_sub;
+	return m->output;
+}
+
+static THFloatTensor *HipLowp_SoftMax_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	long nframe, dim, stride;
+	softmax_shape(in, &nframe, &dim, &stride);
+	const void *x = thhip_tensor_ptr(in, THHIP_U8);
+	void *y = out_resize(m, THHIP_U8, in->nDimension, in->size);
+	hn->cur_mult = thhip_softmax_u8(x, y, nframe, dim, stride, hn->cur_mult, hn->cur_sub);
+	hn->cur_sub = 0;
+	hm->q_mult = hn->cur_mult;
+	hm->q_sub = 0;
+	return m->output;
+}
+
+static THFloatTensor *HipLowp_View_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	Hip_View_updateOutput(m, in);
+	hm->q_mult = hn->cur_mult;
+	hm->q_sub = hn->cur_sub;
+	return m->output;
+}
+
+static THFloatTensor *HipLowp_Identity_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	out_alias(m, in);
+	hm->q_mult = hn->cur_mult;
+	hm->q_sub = hn->cur_sub;
+	return m->output;
+}
+
+/* ------------------------------------------------------------------ */
+/* executor                                                            */
+/* ------------------------------------------------------------------ */
+
+int th_debug, th_profile, th_minmax;
+double th_convtot, th_convflops;
+
+static double seconds_now(void)
+{
+	struct timespec ts;
+	clock_gettime(CLOCK_MONOTONIC, &ts);
+	return ts.tv_sec + ts.tv_nsec * 1e-9;
+}
+
+static int is_conv_type(int type)
+{
+	return type == MT_SpatialConvolutionMM || type == MT_SpatialConvolutionVirtMM || type == MT_SpatialConvolution;
+}
+
+/* forward(), thapi.c:158-235, without the per-layer frees; with th_profile
+ * the stream is drained around each module the way the OpenCL engine calls
+ * clFinish (thapi.c:213-216), so the printed seconds are kernel time. */
+static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
+{
+	double t = 0;
+	for (int i = 0; i < net->nelem; i++) {
+		struct module *m = &net->modules[i];
+		if (th_profile) {
+			thhip_sync();
+			t = seconds_now();
+		}
+		in = m->updateOutput(m, in);
+		if (th_profile) {
+			thhip_sync();
+			t = seconds_now() - t;
+			if (is_conv_type(m->type) && m->type != MT_ConcatTable) {
+				double flops = 2.0 * THFloatTensor_nElement(in) * m->SpatialConvolution.nInputPlane *
+					m->SpatialConvolution.kW * m->SpatialConvolution.kH;
+				printf("%f seconds for module %d, %f Gflops/s\n", t, i + 1, flops * 1e-9 / t);
+				th_convtot += t;
+				th_convflops += flops;
+			} else
+				printf("%f seconds for module %d\n", t, i + 1);
+		}
+		if (th_debug > 1 && m->type != MT_ConcatTable)
+			printf("%d) %d %d %ld %ld %ld %ld\n", i + 1, m->type, in->nDimension, in->size[0], in->size[1],
+				in->size[2], in->size[3]);
+	}
+	return in;
+}
+
+THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in)
+{
+	if (net->engine != ENGINE_HIP && net->engine != ENGINE_HIPLOWP)
+		THError("This library only runs networks made by THCreateHipNetwork / THCreateHipLowpNetwork "
+			"(engine %d given); it carries no CPU path", net->engine);
+	th_convtot = 0;
+	th_convflops = 0;
+	THFloatTensor *out = run_network(net, in);
+	if (th_profile)
+		printf("%f seconds for convolutions %f Gflops/s\n", th_convtot, th_convflops * 1e-9 / th_convtot);
+	return out;
+}
+
+/* ------------------------------------------------------------------ */
+/* engine construction                                                 */
+/* ------------------------------------------------------------------ */
+
+static THFloatTensor *contiguous_host_floats(THFloatTensor *t, const char *what, long expect)
+{
+	if (!t || !t->storage || !t->storage->data)
+		return 0;
+	if (t->storage->mustfree == TH_MUSTFREE_HIP)
+		THError("%s already lives on the device: pass the host network to THCreateHipNetwork", what);
+	long stride = 1;
+	for (int i = t->nDimension - 1; i >= 0; i--) {
+		if (t->size[i] != 1 && t->stride[i] != stride)
+			THError("%s is not contiguous", what);
+		stride *= t->size[i];
+	}
+	if (expect >= 0 && THFloatTensor_nElement(t) != expect)
+		THError("%s has %ld elements, %ld expected", what, THFloatTensor_nElement(t), expect);
+	return t;
+}
+
+static float *upload_floats(THFloatTensor *t, const char *what, long expect)
+{
+	if (!contiguous_host_floats(t, what, expect))
+		return 0;
+	const long n = THFloatTensor_nElement(t);
+	float *d = thhip_malloc(sizeof(float) * n);
+	thhip_memcpy_h2d(d, THFloatTensor_data(t), sizeof(float) * n);
+	return d;
+}
+
+/* THLowpTensor_newFromFloatTensor's arithmetic on the host for the (small,
+ * one-off) weight and bias tensors: lowp_basic.c:15-35. */
+static unsigned char *quantize_host(const float *buf, long len, float *mult_out, float *sub_out)
+{
+	unsigned char *dst = malloc(len ? len : 1);
+	float min = 0, max = 0, mult;
+	long i;
+	for (i = 0; i < len; i++) {
+		if (buf[i] < min)
+			min = buf[i];
+		if (buf[i] > max)
+			max = buf[i];
+	}
+	if (max - min > 0)
+		mult = 255.0 / (max - min);
+	else
+		mult = 0;
+	const float zero = roundf(min * mult);
+	for (i = 0; i < len; i++)
+		dst[i] = (unsigned char)(int)(roundf(buf[i] * mult) - zero);
+	*mult_out = mult;
+	*sub_out = min;
+	return dst;
+}
+
+static struct network *to_hip(struct network *net, int engine, int dtype, float range);
+
+static void convert_module(struct hipnet *hn, struct network *src, int i, int engine, int dtype, float range)
+{
+	struct module *m = &hn->pub.modules[i];
+	struct module *sm = &src->modules[i];
+	struct hipmod *hm = &hn->hm[i];
+	const int lowp = engine == ENGINE_HIPLOWP;
+	m->output = THFloatTensor_new();
+	m->net = &hn->pub;
+	m->nnfree = 0;
+	hm->q_mult = 255 / range;	/* lowp_basic.c:135-136 */
+	hm->q_sub = -range / 2;
+	switch (sm->type) {
+	case MT_SpatialConvolution:
+	case MT_SpatialConvolutionMM:
+	case MT_SpatialConvolutionVirtMM:
+	case MT_Linear: {
+		THFloatTensor *w, *b;
+		int Co, K;
+		if (sm->type == MT_Linear) {
+			/* Linear runs as a 1x1 convolution (cudnn_basic.c:244-265) */
+			w = sm->Linear.weight;
+			b = sm->Linear.bias;
+			if (sm->Linear.commute)
+				THError("Linear with commute is not supported by the HIP engine");
+			if (!w || w->nDimension != 2)
+				THError("Linear weight must be a matrix");
+			Co = (int)w->size[0];
+			K = (int)w->size[1];
+			memset(&m->SpatialConvolution, 0, sizeof(m->SpatialConvolution));
+			m->type = MT_SpatialConvolutionMM;
+			m->SpatialConvolution.dW = m->SpatialConvolution.dH = 1;
+			m->SpatialConvolution.kW = m->SpatialConvolution.kH = 1;
+			m->SpatialConvolution.nOutputPlane = Co;
+			m->SpatialConvolution.nInputPlane = K;
+			hm->is_linear = 1;
+		} else {
+			struct SpatialConvolution *c = &sm->SpatialConvolution;
+			w = c->weight;
+			b = c->bias;
+			Co = c->nOutputPlane;
+			K = c->nInputPlane * c->kH * c->kW;
+		}
+		contiguous_host_floats(w, "convolution weight", (long)Co * K);
+		m->SpatialConvolution.weight = m->SpatialConvolution.bias = m->SpatialConvolution.finput = 0;
+		if (lowp) {
+			float bm = 0, bsub = 0;
+			unsigned char *wq = quantize_host(THFloatTensor_data(w), (long)Co * K, &hm->wm, &hm->wsub);
+			hm->wpacked = thhip_conv_pack_weight_u8(wq, Co, K);
+			free(wq);
+			if (!contiguous_host_floats(b, "convolution bias", Co))
+				THError("the uint8 engine needs a bias on every convolution (lowp_SpatialConvolution.c:111-120)");
+			unsigned char *bq = quantize_host(THFloatTensor_data(b), Co, &bm, &bsub);
+			int *addend = malloc(sizeof(int) * Co);
+			/* lowp_SpatialConvolution.c:112-119 */
+			float mult = hm->q_mult / bm;
+			int add = roundf(bsub * hm->q_mult);
+			for (int o = 0; o < Co; o++) {
+				int a = bq[o];
+				a = roundf(a * mult) + add;
+				addend[o] = a;
+			}
+			hm->addend = thhip_malloc(sizeof(int) * Co);
+			thhip_memcpy_h2d(hm->addend, addend, sizeof(int) * Co);
+			free(addend);
+			free(bq);
+			m->updateOutput = HipLowp_SpatialConvolution_updateOutput;
+		} else {
+			hm->wpacked = thhip_conv_pack_weight(THFloatTensor_data(w), Co, K, dtype);
+			hm->bias = upload_floats(b, "convolution bias", Co);
+			m->updateOutput = Hip_SpatialConvolution_updateOutput;
+		}
+		break;
+	}
+	case MT_Threshold:
+		m->updateOutput = lowp ? HipLowp_Threshold_updateOutput : Hip_Threshold_updateOutput;
+		break;
+	case MT_SpatialMaxPooling:
+		m->SpatialMaxPooling.indices = 0;	/* only SpatialMaxUnpooling reads them */
+		m->updateOutput = lowp ? HipLowp_SpatialMaxPooling_updateOutput : Hip_SpatialMaxPooling_updateOutput;
+		break;
+	case MT_SoftMax:
+		m->updateOutput = lowp ? HipLowp_SoftMax_updateOutput : Hip_SoftMax_updateOutput;
+		break;
+	case MT_Dropout:
+		if (!sm->Dropout.v2)
+			THError("Non v2 dropout not supported in the HIP engine");
+		m->Dropout.inplace = 1;
+		m->updateOutput = lowp ? HipLowp_Identity_updateOutput : Hip_Identity_updateOutput;
+		break;
+	case MT_Identity:
+		m->updateOutput = lowp ? HipLowp_Identity_updateOutput : Hip_Identity_updateOutput;
+		break;
+	case MT_View:
+		m->updateOutput = lowp ? HipLowp_View_updateOutput : Hip_View_updateOutput;
+		break;
+	case MT_SpatialAveragePooling:
+		if (lowp)
+			THError("MT_SpatialAveragePooling not supported in lowp");
+		m->updateOutput = Hip_SpatialAveragePooling_updateOutput;
+		break;
+	case MT_SpatialBatchNormalization: {
+		if (lowp)
+			THError("MT_SpatialBatchNormalization not supported in Lowp");
+		struct SpatialBatchNormalization *bn = &sm->SpatialBatchNormalization;
+		if (!contiguous_host_floats(bn->running_mean, "running_mean", -1) ||
+		    !contiguous_host_floats(bn->running_var, "running_var", -1))
+			THError("SpatialBatchNormalization needs running_mean and running_var");
+		const long C = THFloatTensor_nElement(bn->running_mean);
+		float *invstd = malloc(sizeof(float) * C);
+		const float *var = THFloatTensor_data(bn->running_var);
+		for (long f = 0; f < C; f++)
+			invstd[f] = 1 / sqrt(var[f] + bn->eps);	/* SpatialBatchNormalization.c:85 */
+		hm->bn_planes = C;
+		hm->bn[0] = upload_floats(bn->running_mean, "running_mean", C);
+		hm->bn[1] = thhip_malloc(sizeof(float) * C);
+		thhip_memcpy_h2d(hm->bn[1], invstd, sizeof(float) * C);
+		free(invstd);
+		hm->bn[2] = upload_floats(bn->weight, "batchnorm weight", C);
+		hm->bn[3] = upload_floats(bn->bias, "batchnorm bias", C);
+		memset(&m->SpatialBatchNormalization, 0, sizeof(m->SpatialBatchNormalization));
+		m->SpatialBatchNormalization.eps = bn->eps;
+		m->updateOutput = Hip_SpatialBatchNormalization_updateOutput;
+		break;
+	}
+	case MT_Sequential:
+		if (lowp)
+			THError("MT_Sequential not supported in lowp");
+		m->Sequential.net = to_hip(sm->Sequential.net, engine, dtype, range);
+		m->updateOutput = Hip_Sequential_updateOutput;
+		break;
+	case MT_ConcatTable:
+		if (lowp)
+			THError("MT_ConcatTable not supported in lowp");
+		m->ConcatTable.net = to_hip(sm->ConcatTable.net, engine, dtype, range);
+		m->updateOutput = Hip_ConcatTable_updateOutput;
+		break;
+	case MT_CAddTable:
+	case MT_CSubTable:
+		if (lowp)
+			THError("MT_CAddTable not supported in lowp");
+		m->updateOutput = Hip_CAddTable_updateOutput;
+		break;
+	default:
+		THError("module type %d is not supported by the HIP engine", sm->type);
+	}
+}
+
+static int foldable_threshold(struct module *t)
+{
+	return t->type == MT_Threshold && t->Threshold.alpha == 0;
+}
+
+static struct network *to_hip(struct network *net, int engine, int dtype, float range)
+{
+	struct hipnet *hn = calloc(1, sizeof(*hn));
+	hn->pub.nelem = net->nelem;
+	hn->pub.engine = engine;
+	hn->pub.modules = malloc(sizeof(struct module) * (net->nelem ? net->nelem : 1));
+	memcpy(hn->pub.modules, net->modules, sizeof(struct module) * net->nelem);
+	hn->hm = calloc(net->nelem ? net->nelem : 1, sizeof(struct hipmod));
+	hn->dtype = dtype;
+	hn->range = range;
+	for (int i = 0; i < net->nelem; i++)
+		convert_module(hn, net, i, engine, dtype, range);
+	/* fold a Threshold into the epilogue of the module that feeds it */
+	for (int i = 0; i + 1 < net->nelem; i++) {
+		struct module *m = &hn->pub.modules[i], *t = &hn->pub.modules[i + 1];
+		if (!foldable_threshold(t))
+			continue;
+		if (is_conv_type(m->type)) {
+			hn->hm[i].fused_act = 1;
+			hn->hm[i].thr = t->Threshold.threshold;
+			hn->hm[i].val = t->Threshold.val;
+			hn->hm[i + 1].passthrough = 1;
+		} else if ((m->type == MT_CAddTable || m->type == MT_CSubTable) &&
+			t->Threshold.threshold == 0 && t->Threshold.val == 0) {
+			hn->hm[i].fused_act = 1;
+			hn->hm[i + 1].passthrough = 1;
+		}
+	}
+	return &hn->pub;
+}
+
+struct network *THHip_ToHip(struct network *net, int lowp, float range)
+{
+	if (thhip_device_count() < 1)
+		THError("thnets HIP engine: no AMD GPU visible; this library has no CPU fallback");
+	if (lowp && !(range > 0))
+		THError("THCreateHipLowpNetwork: range must be positive");
+	return to_hip(net, lowp ? ENGINE_HIPLOWP : ENGINE_HIP, lowp ? THHIP_U8 : thhip_engine_dtype(), lowp ? range : 1);
+}
+
+void thhip_free_network(struct network *net)
+{
+	struct hipnet *hn = (struct hipnet *)net;
+	for (int i = 0; i < net->nelem; i++) {
+		struct module *m = &net->modules[i];
+		struct hipmod *hm = &hn->hm[i];
+		if (m->type == MT_Sequential && m->Sequential.net)
+			thhip_free_network(m->Sequential.net);
+		else if (m->type == MT_ConcatTable && m->ConcatTable.net)
+			thhip_free_network(m->ConcatTable.net);
+		THFloatTensor_free(m->output);
+		thhip_free(hm->wpacked);
+		thhip_free(hm->wrow);
+		thhip_free(hm->bias);
+		thhip_free(hm->addend);
+		for (int j = 0; j < 4; j++)
+			thhip_free(hm->bn[j]);
+	}
+	free(hn->hm);
+	free(net->modules);
+	free(hn);
+}

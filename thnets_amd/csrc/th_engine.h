@@ -1,0 +1,45 @@
+/* Engine-private declarations shared by the host C files (not installed). */
+#ifndef TH_ENGINE_H
+#define TH_ENGINE_H
+
+#include "../../include/thnets_hip.h"
+
+/* Per-module state the engine keeps beside `struct module` (index-parallel to
+ * network.modules), so that the public structure keeps the reference layout. */
+struct hipmod {
+	int fused_act;		/* the following Threshold is applied in this module's epilogue */
+	float thr, val;
+	int passthrough;	/* a Threshold whose work was folded into its producer */
+	int is_linear;		/* MT_Linear in the source network */
+	int owns_output;	/* output storage was allocated by this module */
+	size_t cap;		/* bytes allocated for the output */
+	void *wpacked;		/* convolution weights in the kernel's packed layout (device) */
+	void *wrow;		/* the same weights row-major, made on first matrix-vector use (device) */
+	float *bias;		/* fp32 bias (device) */
+	float *bn[4];		/* mean, invstd, weight, bias per plane (device) */
+	long bn_planes;
+	/* uint8 engine */
+	int *addend;		/* per-plane bias addend (device) */
+	float wm, wsub;		/* weight quantisation */
+	float q_mult, q_sub;	/* quantisation of this module's output */
+};
+
+/* A `struct network` with the engine's state behind it. */
+struct hipnet {
+	struct network pub;	/* must be first */
+	struct hipmod *hm;
+	int dtype;		/* enum thhip_dtype of activations */
+	float range;
+	float cur_mult, cur_sub;	/* uint8 engine: quantisation of the tensor in flight */
+};
+
+struct hipnet *hipnet_of(struct module *m);
+struct hipmod *hipmod_of(struct module *m);
+void *thhip_tensor_ptr(THFloatTensor *t, int dtype);
+int thhip_engine_dtype(void);
+struct network *THHip_ToHip(struct network *net, int lowp, float range);
+THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in);
+void thhip_free_network(struct network *net);
+void thhip_storage_release(THFloatStorage *s);
+
+#endif
