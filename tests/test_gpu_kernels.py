@@ -143,12 +143,21 @@ def test_pooling_bit_exact(hiplib, oracle, i):
     assert np.array_equal(yq, oracle.lowp_maxpool(q, kH, kW, dH, dW, pH, pW, ceil))
 
 
+def _softmax_dims(sh):
+    if len(sh) == 1:
+        return 1, sh[0], 1
+    if len(sh) == 2:
+        return sh[0], sh[1], 1
+    if len(sh) == 3:
+        return 1, sh[0], sh[1] * sh[2]
+    return sh[0], sh[1], sh[2] * sh[3]
+
+
 @pytest.mark.parametrize("i", range(len(cases.SOFTMAX_SHAPES)))
 def test_softmax(hiplib, oracle, i):
     x = cases.softmax_case(i)
     sh = x.shape
-    nframe, dim, stride = {1: (1, sh[0], 1), 2: (sh[0], sh[-1], 1), 3: (1, sh[0], int(np.prod(sh[1:]))),
-                           4: (sh[0], sh[1], int(np.prod(sh[2:])))}[x.ndim]
+    nframe, dim, stride = _softmax_dims(sh)
     y = G.unary(hiplib, hiplib.thhip_softmax, x, sh, G.F32, nframe, dim, stride, G.F32)
     G.assert_close(y, GOLD["softmax%d" % i], 1e-5)
 

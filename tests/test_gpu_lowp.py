@@ -91,8 +91,12 @@ def test_threshold_and_softmax_u8_bit_exact(hiplib, oracle):
     assert np.array_equal(y, oracle.lowp_threshold(q, 127, 127, 1))
     for shape in [(3, 1000), (1000,), (2, 21, 3, 3)]:
         q = cases.rng(1103).integers(0, 256, shape, dtype=np.uint8)
-        nframe, dim, stride = {1: (1, shape[0], 1), 2: (shape[0], shape[-1], 1),
-                               4: (shape[0], shape[1], shape[2] * shape[3])}[len(shape)]
+        if len(shape) == 1:
+            nframe, dim, stride = 1, shape[0], 1
+        elif len(shape) == 2:
+            nframe, dim, stride = shape[0], shape[1], 1
+        else:
+            nframe, dim, stride = shape[0], shape[1], shape[2] * shape[3]
         dx = api.DeviceArray(hiplib, q)
         dy = api.DeviceArray(hiplib, nbytes=q.size)
         hiplib.thhip_softmax_u8.restype = C.c_float

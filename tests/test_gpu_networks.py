@@ -26,7 +26,9 @@ def layerwise(net, oracle, cfg, tol):
             continue
         want = o
         # a Threshold folded into its producer: the producer's buffer holds the thresholded values
-        if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold" and layers[i]["type"] in ("conv", "linear", "caddtable"):
+        # (or applied in place on the producer's buffer)
+        if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold" and (
+                layers[i]["type"] in ("conv", "linear", "caddtable") or layers[i + 1].get("inplace", 1) == 1):
             want = outs[i + 1]
         G.assert_close(net.module_output(i).ravel(), np.asarray(want).ravel(), tol, "module %d %s" % (i, layers[i]["type"]))
 

@@ -12,6 +12,11 @@
 
 #define EW_THREADS 256
 
+/* Several of these kernels are held to bit-exact parity with a CPU evaluation
+ * that rounds after every operation, so nothing in this file may be fused
+ * into a multiply-add. */
+#pragma clang fp contract(off)
+
 static inline dim3 ew_grid(long n, int per_thread = 1)
 {
 	long blocks = (n + (long)EW_THREADS * per_thread - 1) / ((long)EW_THREADS * per_thread);
@@ -199,8 +204,6 @@ extern "C" void thhip_avgpool(const void *x, void *y, int B, int C, int H, int W
 /* THExpMinusApprox, thbasic.c:462-491 */
 __device__ __forceinline__ double exp_minus_approx(double x)
 {
-	/* separately rounded steps, as a CPU build without fused multiply-add gives */
-#pragma clang fp contract(off)
 	if (x < 13.0) {
 		double y = 1.0 + x * (0.125 + x * (0.0078125 + x * (0.00032552083 + x * 1.0172526e-5)));
 		y *= y;
@@ -267,26 +270,26 @@ __global__ __launch_bounds__(64) void softmax_u8_kernel(const unsigned char *x, 
 	for (int off = 32; off > 0; off >>= 1)
 		qmax = max(qmax, __shfl_xor(qmax, off, 64));
 	for (long d = lane; d < dim; d += 64) {
-		const float arg = __fadd_rn(__fmul_rn((float)(qmax - (int)x[base + d * stride]), invmult), sub);
+		const float arg = (float)(qmax - (int)x[base + d * stride]) * invmult + sub;
 		tmp[d] = (float)exp_minus_approx((double)arg);
 	}
 	__syncthreads();
 	if (lane == 0) {
 		float sum = 0;
 		for (long d = 0; d < dim; d++)
-			sum = __fadd_rn(sum, tmp[d]);
+			sum = sum + tmp[d];
 		s_scale = 1 / sum;
 	}
 	__syncthreads();
 	const float scale = s_scale;
 	if (!single) {
 		for (long d = lane; d < dim; d += 64)
-			y[base + d * stride] = (unsigned char)(int)__fmul_rn(255.0f, __fmul_rn(tmp[d], scale));
+			y[base + d * stride] = (unsigned char)(int)(255.0f * (tmp[d] * scale));
 		return;
 	}
 	float mx = 0;
 	for (long d = lane; d < dim; d += 64) {
-		tmp[d] = __fmul_rn(tmp[d], scale);
+		tmp[d] = tmp[d] * scale;
 		mx = fmaxf(mx, tmp[d]);
 	}
 	for (int off = 32; off > 0; off >>= 1)
@@ -298,7 +301,7 @@ __global__ __launch_bounds__(64) void softmax_u8_kernel(const unsigned char *x, 
 	__syncthreads();
 	const float rmax = 1 / s_max;
 	for (long d = lane; d < dim; d += 64)
-		y[base + d * stride] = (unsigned char)(int)__fmul_rn(__fmul_rn(255.0f, tmp[d]), rmax);
+		y[base + d * stride] = (unsigned char)(int)((255.0f * tmp[d]) * rmax);
 }
 
 extern "C" float thhip_softmax_u8(const unsigned char *x, unsigned char *y, long nframe, long dim, long stride,
@@ -427,7 +430,7 @@ __global__ void rgb2float_kernel(void *dst, const unsigned char *src, int width,
 		const int sc = bgr ? cp - 1 - c : c;
 		const float byte = (float)src[sc + cp * j + (long)stride * r];
 		/* (byte * (1/255) - mean) * (1/std), three separately rounded steps */
-		const float v = __fmul_rn(__fsub_rn(__fmul_rn(byte, 0.003921568f), mean[c]), std1[c]);
+		const float v = (byte * 0.003921568f - mean[c]) * std1[c];
 		ThhipElem<DT>::st(dst, i, v);
 	}
 }
@@ -483,7 +486,7 @@ __global__ void quantize_kernel(const float *x, unsigned char *q, long n, float 
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
 	const long step = (long)gridDim.x * blockDim.x;
 	for (; i < n; i += step)
-		q[i] = (unsigned char)(int)__fsub_rn(roundf(__fmul_rn(x[i], mult)), zero);
+		q[i] = (unsigned char)(int)(roundf(x[i] * mult) - zero);
 }
 
 extern "C" void thhip_quantize(const float *x, unsigned char *q, long n, float *mult_out, float *sub_out)
@@ -521,7 +524,7 @@ __global__ void dequantize_kernel(const unsigned char *q, float *x, long n, floa
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
 	const long step = (long)gridDim.x * blockDim.x;
 	for (; i < n; i += step)
-		x[i] = __fadd_rn(__fmul_rn((float)q[i], invmult), sub);
+		x[i] = (float)q[i] * invmult + sub;
 }
 
 extern "C" void thhip_dequantize(const unsigned char *q, float *x, long n, float mult, float sub)
