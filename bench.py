@@ -1,0 +1,168 @@
+"""Benchmark of the MI355X thnets engine on the reference's headline workloads.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One "step" is one THForward of the VGG-16-shape network (fp32, batch 16, 3x224x224,
+synthetic seeded input and weights) with the input already resident in HBM; the
+value is whole-job images/second.  The same run also times the uint8 AlexNet-OWT
+batch-64 network (reported under "extra"), measures the convolution kernel family
+with HIP events around every launch inside the timed region (-> "roofline"), and
+times the CPU baseline on the host cores (-> "cpu_baseline": the reference's own
+CPU library when oracle/_ref holds a build of it, else this repository's C
+restatement).  Prints one JSON line.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from thnets_amd import api, configs  # noqa: E402
+
+PEAK_TFLOPS_FP32_MFMA = 157.3
+PEAK_TOPS_INT8_MFMA = 5030.0
+
+
+def profile_get(lib, fam):
+    ms, n, work = C.c_double(), C.c_long(), C.c_double()
+    lib.thhip_profile_get(fam, C.byref(ms), C.byref(n), C.byref(work))
+    return ms.value, n.value, work.value
+
+
+def timed_forward(lib, net, steps, warmup, families):
+    """W untimed + K timed THForward calls; returns ms/step and per-family
+    (ms, launches, work) measured with events around each launch in the timed steps."""
+    for _ in range(warmup):
+        net.forward()
+    lib.thhip_sync()
+    lib.thhip_profile_reset()
+    lib.thhip_profile_enable(1)
+    t0 = time.perf_counter()
+    lib.thhip_event_record(0)
+    for _ in range(steps):
+        net.forward()
+    lib.thhip_event_record(1)
+    lib.thhip_sync()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    dev_ms = lib.thhip_event_ms(0, 1) / steps
+    fam = {f: profile_get(lib, f) for f in families}
+    lib.thhip_profile_enable(0)
+    return max(wall_ms, dev_ms), fam
+
+
+def cpu_baseline(cfg, seconds_budget=25.0):
+    """Times the CPU path on this host: THProcessFloat of the reference's own library
+    (kind "reference") or the C restatement (kind "port") on the same network."""
+    from oracle.oracle_py import Oracle, Reference
+    batch = cfg["input"].shape[0]
+    cores = os.cpu_count() or 1
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except AttributeError:
+        pass
+    if Reference.available():
+        ref = Reference()
+        threads = ref.set_threads(ref.threads_for_batch(batch, limit=min(cores, 16)))
+        hn = ref.host_network(cfg)
+        ref.process_float(hn, cfg["input"])          # warm-up
+        times = []
+        t_end = time.perf_counter() + seconds_budget
+        while len(times) < 5 and (not times or time.perf_counter() < t_end):
+            t0 = time.perf_counter()
+            ref.process_float(hn, cfg["input"])
+            times.append(time.perf_counter() - t0)
+        kind = "reference"
+    else:
+        orc = Oracle()
+        threads = min(orc.threads(), cores, 16)
+        orc.set_threads(threads)
+        x = orc.normalize(cfg["input"], cfg["mean"], cfg["std"])
+        times = []
+        t_end = time.perf_counter() + seconds_budget
+        while len(times) < 3 and (not times or time.perf_counter() < t_end):
+            t0 = time.perf_counter()
+            orc.run_layers(cfg["layers"], x)
+            times.append(time.perf_counter() - t0)
+        kind = "port"
+    best = min(times)
+    return {"value": round(batch / best, 3), "unit": "images/s", "cores": int(threads), "kind": kind,
+            "sample": "%d THProcessFloat calls of the same %s network (batch %d) after one warm-up; best of them"
+                      % (len(times), cfg["name"], batch),
+            "mean_value": round(batch / (sum(times) / len(times)), 3)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-int8", action="store_true", help="skip the uint8 AlexNet leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported (the path shards by batch, "
+              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    lib = api.load_library()
+    lib.THInit()
+
+    # ---- VGG-16 fp32 batch 16 (the headline) ----
+    cfg = configs.vgg16(batch=16)
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    net.upload(cfg["input"])
+    ms, fam = timed_forward(lib, net, args.steps, args.warmup, (0, 1, 3))
+    conv_ms, conv_n, conv_flops = fam[0]
+    value = 16.0 / (ms * 1e-3)
+    achieved = conv_flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
+    roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
+                "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4), "traffic": None,
+                "kernel": "conv_mfma_kernel<fp32> (implicit-GEMM convolution, all 13 conv + 3 batched FC launches per step)",
+                "launches_per_step": conv_n / args.steps, "avg_launch_ms": round(conv_ms / max(conv_n, 1), 5),
+                "flops_per_launch": conv_flops / max(conv_n, 1)}
+    extra = {"vgg16_conv_ms_per_step": round(conv_ms / args.steps, 4),
+             "vgg16_other_kernels_ms_per_step": round(fam[3][0] / args.steps, 4)}
+    net.free()
+
+    # ---- uint8 AlexNet-OWT batch 64 ----
+    if not args.no_int8:
+        c5 = configs.alexnet_lowp(batch=64)
+        x5 = c5["input"].copy()
+        for c in range(3):
+            x5[:, c] = (x5[:, c] - np.float32(c5["mean"][c])) / np.float32(c5["std"][c])
+        n5 = api.HipNetwork(c5["layers"], c5["mean"], c5["std"], lowp_range=c5["range"])
+        n5.upload(x5)
+        ms5, fam5 = timed_forward(lib, n5, args.steps, args.warmup, (2, 3))
+        i8_ms, i8_n, i8_ops = fam5[2]
+        i8_tops = i8_ops / (i8_ms * 1e-3) / 1e12 if i8_ms > 0 else 0.0
+        extra["int8_alexnet_owt_b64"] = {
+            "images_per_sec": round(64.0 / (ms5 * 1e-3), 1), "ms_per_step": round(ms5, 4),
+            "conv_i8_TOP/s": round(i8_tops, 2), "frac_of_int8_mfma_peak": round(i8_tops / PEAK_TOPS_INT8_MFMA, 4),
+            "dtype": "u8 x u8 -> i32", "workload": "AlexNet-OWT THMakeSpatial form, range 32 (BASELINE configs[4])"}
+        n5.free()
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(cfg)
+
+    line = {
+        "metric": "images/sec VGG-16 fp32 b16 (+ int8 AlexNet-OWT b64 under extra); % MFMA peak under roofline",
+        "value": round(value, 2), "unit": "images/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "VGG-16 shape, fp32, batch 16, 3x224x224, THForward with the input resident in HBM "
+                               "(BASELINE configs[2])", "batch": 16},
+        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -290,6 +290,10 @@ int THHipNetwork_getModuleQuant(THNETWORK *net, int idx, float *mult, float *sub
 /* Declares the quantisation of the uint8 device tensor the next THForward of
  * a HIPLOWP network will be given (THProcessFloat derives it by itself). */
 int THHipNetwork_setInputQuant(THNETWORK *net, float mult, float sub);
+/* Device counterpart of THLowpTensor_newFromFloatTensor (lowp_basic.c:5-38):
+ * upload, quantise with one min/max over the tensor, and record the result
+ * as the quantisation of `net`'s next input. */
+THFloatTensor *THHipLowpTensor_newFromFloatTensor(THNETWORK *net, THFloatTensor *t);
 
 /* Drop-in for the reference's only call into gemmlowp (gemm8.cc:4-17,
  * declared lowp_basic.c:290-297): host pointers in and out, the GEMM and
@@ -329,12 +333,13 @@ void thhip_profile_reset(void);
 void thhip_profile_get(int family, double *ms, long *launches, double *work);
 
 /* Weight packing for the implicit-GEMM convolution: row-major
- * [Co][K=Ci*kH*kW] (SpatialConvolutionMM.c:141-144) -> the K-chunked,
- * M-interleaved layout the kernel streams.  Returns a device buffer. */
-void *thhip_conv_pack_weight(const float *w_host, int Co, int K, int dtype);
-size_t thhip_conv_packed_bytes(int Co, int K, int dtype);
-/* The inverse: packed -> row-major [Co][K] in the same dtype (new device buffer). */
-void *thhip_conv_unpack_rows(const void *wpacked, int Co, int K, int dtype);
+ * [Co][Ci][kHW = kH*kW] (SpatialConvolutionMM.c:141-144) -> the K-chunked,
+ * M-interleaved layout the kernel streams (tap-major along K when Ci is a
+ * multiple of the kernel's plane block).  Returns a device buffer. */
+void *thhip_conv_pack_weight(const float *w_host, int Co, int Ci, int kHW, int dtype);
+size_t thhip_conv_packed_bytes(int Co, int Ci, int kHW, int dtype);
+/* The inverse: packed -> row-major [Co][Ci*kHW] in the same dtype (new device buffer). */
+void *thhip_conv_unpack_rows(const void *wpacked, int Co, int Ci, int kHW, int dtype);
 
 /* Replaces nn_SpatialConvolutionMM_updateOutput's per-image
  * im2col + sgemm + bias (SpatialConvolutionMM.c:75-109, 126-225) and, when
@@ -351,6 +356,16 @@ void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y
  * [nOut][nIn] fp32/fp16/bf16, optional fused threshold. */
 void thhip_gemv(const void *x, const void *w, const float *bias, void *y,
 	int nIn, int nOut, int act, float thr, float val, int dtype);
+
+/* Replaces nn_Linear_updateOutput's matrix branch for a small batch
+ * (Linear.c:92-108: addmm with beta 0, then the rank-1 bias update through
+ * addr / sger, thbasic.c:757-789): Y[b][o] = bias[o] + sum_k W[o][k] X[b][k],
+ * X [B][nIn], W row-major [nOut][nIn], Y [B][nOut].  thhip_linear_batched_supported
+ * says whether the shape is taken (fp32, B <= 32, nIn % 4 == 0); other shapes
+ * run as a 1x1 convolution through thhip_conv2d. */
+int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtype);
+void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
+	int B, int nIn, int nOut, int act, float thr, float val, int dtype);
 
 /* Replaces nn_Threshold_updateOutput (Threshold.c:38-63), out of place or
  * in place (y == x).  alpha != 0 selects the LeakyReLU branch. */
@@ -402,9 +417,9 @@ void thhip_quantize(const float *x, unsigned char *q, long n, float *mult, float
 /* Replaces THFloatTensor_newFromLowpTensor (lowp_basic.c:40-58). */
 void thhip_dequantize(const unsigned char *q, float *x, long n, float mult, float sub);
 
-/* Weight packing for the int8 kernel: uint8 codes [Co][K] -> signed
+/* Weight packing for the int8 kernel: uint8 codes [Co][Ci][kHW] -> signed
  * (code-128) K-chunked layout + per-row sums.  Returns a device buffer. */
-void *thhip_conv_pack_weight_u8(const unsigned char *w_host, int Co, int K);
+void *thhip_conv_pack_weight_u8(const unsigned char *w_host, int Co, int Ci, int kHW);
 
 /* Replaces Lowp_SpatialConvolution_updateOutput's per-image
  * uint8 im2col + THLowpTensor_mm/lowpgemm + lowpadd

@@ -20,7 +20,7 @@ def conv2d(lib, x, w, bias, d=(1, 1), pad=(0, 0), act=0, thr=0.0, val=0.0, dtype
     K = Ci * kH * kW
     oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
     note("conv2d x%s w%s d%s pad%s dtype%d" % (x.shape, w.shape, d, pad, dtype))
-    wp = lib.thhip_conv_pack_weight(w.ctypes.data, Co, K, dtype)
+    wp = lib.thhip_conv_pack_weight(w.ctypes.data, Co, Ci, kH * kW, dtype)
     dx = api.to_device_dtype(lib, x, dtype)
     db = api.DeviceArray(lib, np.ascontiguousarray(bias, np.float32)) if bias is not None else None
     dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW * (4 if dtype == F32 else 2))
@@ -61,7 +61,7 @@ def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0):
     K = Ci * kH * kW
     oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
     note("conv2d_u8 x%s w%s d%s pad%s prm%s" % (xq.shape, wq.shape, d, pad, prm))
-    wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, K)
+    wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, Ci, kH * kW)
     dx = api.DeviceArray(lib, xq)
     da = api.DeviceArray(lib, np.ascontiguousarray(addend, np.int32)) if addend is not None else None
     dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW)

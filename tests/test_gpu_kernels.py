@@ -81,10 +81,11 @@ def test_pack_unpack_roundtrip(hiplib):
     import ctypes as C
     from thnets_amd import api
     g = cases.rng(901)
-    for (Co, K) in [(5, 7), (64, 27), (130, 576), (33, 1000)]:
-        w = g.standard_normal((Co, K), dtype=np.float32)
-        wp = hiplib.thhip_conv_pack_weight(w.ctypes.data, Co, K, G.F32)
-        rows = hiplib.thhip_conv_unpack_rows(wp, Co, K, G.F32)
+    # plane counts that select the tap-major K order (multiples of 16) and the plain one
+    for (Co, Ci, kHW) in [(5, 7, 1), (64, 3, 9), (130, 64, 9), (33, 1000, 1), (40, 32, 25), (200, 256, 36)]:
+        w = g.standard_normal((Co, Ci * kHW), dtype=np.float32)
+        wp = hiplib.thhip_conv_pack_weight(w.ctypes.data, Co, Ci, kHW, G.F32)
+        rows = hiplib.thhip_conv_unpack_rows(wp, Co, Ci, kHW, G.F32)
         hiplib.thhip_sync()
         back = np.empty_like(w)
         hiplib.thhip_memcpy_d2h(back.ctypes.data, rows, back.nbytes)
@@ -114,6 +115,41 @@ def test_gemv_ragged_sizes(hiplib, oracle):
         w = g.standard_normal((nOut, nIn), dtype=np.float32)
         b = g.standard_normal(nOut, dtype=np.float32)
         G.assert_close(G.gemv(hiplib, x, w, b), oracle.linear(x, w, b), FP32_TOL, str((nOut, nIn)))
+
+
+def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
+    from thnets_amd import api
+    g = cases.rng(906)
+    shapes = [(4, 128, 64), (16, 512, 100), (2, 64, 17), (16, 4096, 1000), (32, 1028, 515), (17, 200, 33), (7, 25088, 48)]
+    for (B, nIn, nOut) in shapes:
+        assert hiplib.thhip_linear_batched_supported(B, nIn, nOut, G.F32)
+        x = g.standard_normal((B, nIn), dtype=np.float32)
+        w = g.standard_normal((nOut, nIn), dtype=np.float32) * np.float32(np.sqrt(2.0 / nIn))
+        b = g.standard_normal(nOut, dtype=np.float32)
+        G.note("linear_batched %s" % ((B, nIn, nOut),))
+        dx, dw, db = api.DeviceArray(hiplib, x), api.DeviceArray(hiplib, w), api.DeviceArray(hiplib, b)
+        dy = api.DeviceArray(hiplib, nbytes=B * nOut * 4)
+        hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 0, 0.0, 0.0, G.F32)
+        hiplib.thhip_sync()
+        y = dy.get((B, nOut), np.float32)
+        G.assert_close(y, oracle.linear(x, w, b), FP32_TOL, str((B, nIn, nOut)))
+        hiplib.thhip_linear_batched(dx.ptr, dw.ptr, None, dy.ptr, B, nIn, nOut, 1, 0.0, 0.0, G.F32)
+        hiplib.thhip_sync()
+        G.assert_close(dy.get((B, nOut), np.float32), np.maximum(oracle.linear(x, w, None), 0), FP32_TOL)
+    assert not hiplib.thhip_linear_batched_supported(33, 128, 64, G.F32)
+    assert not hiplib.thhip_linear_batched_supported(4, 130, 64, G.F32)
+    assert not hiplib.thhip_linear_batched_supported(4, 128, 64, G.F16)
+    for i in (2, 3):
+        x, s = cases.linear_case(i)
+        B, nIn = x.shape
+        nOut = s["weight"].shape[0]
+        dx, dw, db = api.DeviceArray(hiplib, x), api.DeviceArray(hiplib, s["weight"]), api.DeviceArray(hiplib, s["bias"])
+        dy = api.DeviceArray(hiplib, nbytes=B * nOut * 4)
+        if not hiplib.thhip_linear_batched_supported(B, nIn, nOut, G.F32):
+            continue
+        hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 0, 0.0, 0.0, G.F32)
+        hiplib.thhip_sync()
+        G.assert_close(dy.get((B, nOut), np.float32), GOLD["linear%d" % i], FP32_TOL)
 
 
 def test_threshold_bit_exact(hiplib, oracle):

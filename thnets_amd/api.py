@@ -58,6 +58,7 @@ PROTOTYPES = {
     "THHipNetwork_copyModuleOutput": (C.c_long, [vp, C.c_int, C.POINTER(c_fp), C.POINTER(C.c_long), c_ip]),
     "THHipNetwork_getModuleQuant": (C.c_int, [vp, C.c_int, c_fp, c_fp]),
     "THHipNetwork_setInputQuant": (C.c_int, [vp, C.c_float, C.c_float]),
+    "THHipLowpTensor_newFromFloatTensor": (vp, [vp, vp]),
     "lowpgemm": (None, [C.c_int] * 6 + [vp, vp, vp] + [C.c_int] * 8),
     "thhip_device_count": (C.c_int, []),
     "thhip_malloc": (vp, [C.c_size_t]),
@@ -72,11 +73,13 @@ PROTOTYPES = {
     "thhip_profile_enable": (None, [C.c_int]),
     "thhip_profile_reset": (None, []),
     "thhip_profile_get": (None, [C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_long), C.POINTER(C.c_double)]),
-    "thhip_conv_pack_weight": (vp, [vp, C.c_int, C.c_int, C.c_int]),
-    "thhip_conv_packed_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int]),
-    "thhip_conv_unpack_rows": (vp, [vp, C.c_int, C.c_int, C.c_int]),
+    "thhip_conv_pack_weight": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "thhip_conv_packed_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int]),
+    "thhip_conv_unpack_rows": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
+    "thhip_linear_batched_supported": (C.c_int, [C.c_int] * 4),
+    "thhip_linear_batched": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_threshold": (None, [vp, vp, C.c_long, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]),
     "thhip_maxpool": (None, [vp, vp] + [C.c_int] * 13),
     "thhip_pool_outsize": (None, [C.c_int] * 9 + [c_ip, c_ip]),
@@ -88,7 +91,7 @@ PROTOTYPES = {
     "thhip_rgb2float": (None, [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, C.c_int]),
     "thhip_quantize": (None, [vp, vp, C.c_long, c_fp, c_fp]),
     "thhip_dequantize": (None, [vp, vp, C.c_long, C.c_float, C.c_float]),
-    "thhip_conv_pack_weight_u8": (vp, [vp, C.c_int, C.c_int]),
+    "thhip_conv_pack_weight_u8": (vp, [vp, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d_u8": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3),
     "thhip_threshold_u8": (None, [vp, vp, C.c_long, C.c_int, C.c_int, C.c_int]),
     "thhip_softmax_u8": (C.c_float, [vp, vp, C.c_long, C.c_long, C.c_long, C.c_float, C.c_float]),
@@ -228,13 +231,17 @@ class HipNetwork:
         return np.ctypeslib.as_array(res, shape=(n,)).copy()
 
     def upload(self, x):
-        """Host float32 (already normalised) -> device tensor in the engine dtype;
-        kept alive by this object and reused by forward()."""
+        """Host float32 (already normalised) -> device tensor in the engine dtype
+        (quantised on the device for a uint8 network); kept alive by this object and
+        reused by forward()."""
         x = np.ascontiguousarray(x, np.float32)
         t = self.host.tensor(x)
-        self.lib.THHipHalfFloat(self.half)
-        dev = self.lib.THHipTensor_newFromFloatTensor(C.addressof(t.contents))
-        self.lib.THHipHalfFloat(0)
+        if self.lowp:
+            dev = self.lib.THHipLowpTensor_newFromFloatTensor(self.handle, C.addressof(t.contents))
+        else:
+            self.lib.THHipHalfFloat(self.half)
+            dev = self.lib.THHipTensor_newFromFloatTensor(C.addressof(t.contents))
+            self.lib.THHipHalfFloat(0)
         if self._dev_in:
             self.lib.THFloatTensor_free(self._dev_in)
         self._dev_in = dev

@@ -39,7 +39,8 @@ struct ConvParams {
 	void *y;
 	int B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, oH, oW;
 	int K, KC, N, oHW, HW, kHW;
-	unsigned magic_khw, magic_kw;
+	unsigned magic_khw, magic_kw;	/* low words of floor(2^32/d)+1 */
+	unsigned mhi_khw, mhi_kw;	/* their bit 32 (set only for d == 1) */
 	int act;
 	float thr, val;
 	int tiles_m, tiles_n;
@@ -50,10 +51,11 @@ struct ConvParams {
 	int zero, offA, offB, c_off, c_mult, c_shift, ithr, ival;
 };
 
-/* floor(n / d) for n*d < 2^32, d > 1, with m = floor(2^32/d) + 1. */
-static inline unsigned conv_magic(unsigned d)
+/* floor(n / d) = (n * m) >> 32 for n*d < 2^32 with the 33-bit m = floor(2^32/d) + 1,
+ * evaluated as n*m_hi + umulhi(n, m_lo); m_hi is 1 only for d == 1. */
+static inline unsigned long long conv_magic(unsigned d)
 {
-	return d <= 1 ? 0u : (unsigned)(((1ull << 32) / d) + 1);
+	return (1ull << 32) / d + 1;
 }
 
 template <int DT> struct ConvTraits;
@@ -129,27 +131,17 @@ struct KTap { int koff, kh, kw; };
 __device__ __forceinline__ KTap conv_ktap(const ConvParams &p, int k)
 {
 	KTap t;
-	unsigned c, rem, kh;
-	if (p.kHW == 1) {
-		c = k;
-		rem = 0;
-	} else {
-		c = __umulhi((unsigned)k, p.magic_khw);
-		rem = k - c * p.kHW;
-	}
-	if (p.kW == 1)
-		kh = rem;
-	else
-		kh = __umulhi(rem, p.magic_kw);
+	const unsigned c = (unsigned)k * p.mhi_khw + __umulhi((unsigned)k, p.magic_khw);
+	const unsigned rem = k - c * p.kHW;
+	const unsigned kh = rem * p.mhi_kw + __umulhi(rem, p.magic_kw);
 	t.kh = kh;
 	t.kw = rem - kh * p.kW;
 	t.koff = c * p.HW + t.kh * p.W + t.kw;
-	if (k >= p.K)
-		t.kh = 0x40000000;	/* K padding: forces the bounds test to fail */
+	t.kh = k < p.K ? t.kh : 0x40000000;	/* K padding: forces the bounds test to fail */
 	return t;
 }
 
-template <int DT, int BM, int BN, int WGM, int WGN>
+template <int DT, int BM, int BN, int WGM, int WGN, bool TAP>
 __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 {
 	typedef ConvTraits<DT> TR;
@@ -204,6 +196,14 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 	floatx4 breg[B_PER_THREAD];
 	int colsum = 0;		/* uint8 path: sum of this thread's gathered (code - 128) */
 
+	/* Tap-major K order (TAP): K-tile t covers one filter tap (kh, kw) and
+	 * CB = 2*CHUNK consecutive input planes, tiles ordered plane block outer,
+	 * tap inner.  Bounds test and in-plane offset are then one computation per
+	 * thread per K-tile and every element differs only by a wave-uniform plane
+	 * offset, which rides in the load's scalar offset. */
+	int t_cb = 0, t_kh = 0, t_kw = 0;
+	const int plane_bytes = p.HW * (int)sizeof(elem);
+
 	auto load_tile = [&](int kt) {
 #pragma unroll
 		for (int i = 0; i < A_PER_WAVE; i++) {
@@ -211,28 +211,51 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 			const int mbi = idx % MB, kci = idx / MB;
 			areg[i] = wp[((size_t)(tile_m * MB + mbi) * p.KC + kt * 2 + kci) * 64 + lane];
 		}
+		unsigned tap_voff = 0;
+		bool tap_ok = false;
+		if constexpr (TAP) {
+			const int iy = iy0 + t_kh, ix = ix0 + t_kw;
+			tap_ok = n_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			tap_voff = tap_ok ? (unsigned)(xoff + t_kh * p.W + t_kw) * (unsigned)sizeof(elem) : 0xfffffff0u;
+		}
 #pragma unroll
 		for (int j = 0; j < B_PER_THREAD; j++) {
 			const int pidx = slot * B_PER_THREAD + j;
-			const int kbase = (kt * 2 + (pidx >> 1)) * CHUNK + (pidx & 1) * VEC;
 			elem v[VEC];
+			if constexpr (TAP) {
+				const int cbase = t_cb * (2 * CHUNK) + (pidx >> 1) * CHUNK + (pidx & 1) * VEC;
 #pragma unroll
-			for (int e = 0; e < VEC; e++) {
-				const KTap t = conv_ktap(p, kbase + e);
-				const int iy = iy0 + t.kh, ix = ix0 + t.kw;
-				const bool ok = n_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-				/* an offset past the buffer's extent reads as zero */
-				const unsigned voff = ok ? (unsigned)(xoff + t.koff) * (unsigned)sizeof(elem) : 0xfffffff0u;
-				if constexpr (DT == THHIP_U8) {
-					/* padding is the code of 0.0 (lowp_SpatialConvolution.c:101);
-					 * columns past N and the K padding hold 128, which the
-					 * re-centring below turns into 0 */
-					const unsigned char ld = __builtin_amdgcn_raw_buffer_load_b8(xrsrc, voff, 0, 0);
-					v[e] = ok ? ld : (unsigned char)((n_ok && kbase + e < p.K) ? p.zero : 128);
-				} else if constexpr (sizeof(elem) == 4) {
-					v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, voff, 0, 0));
-				} else {
-					v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b16(xrsrc, voff, 0, 0));
+				for (int e = 0; e < VEC; e++) {
+					/* the scalar offset is not range checked: planes exist
+					 * because Ci is a multiple of the block */
+					const int soff = (cbase + e) * plane_bytes;
+					if constexpr (DT == THHIP_U8)
+						v[e] = __builtin_amdgcn_raw_buffer_load_b8(xrsrc, tap_voff, soff, 0);
+					else if constexpr (sizeof(elem) == 4)
+						v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, tap_voff, soff, 0));
+					else
+						v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b16(xrsrc, tap_voff, soff, 0));
+				}
+			} else {
+				const int kbase = (kt * 2 + (pidx >> 1)) * CHUNK + (pidx & 1) * VEC;
+#pragma unroll
+				for (int e = 0; e < VEC; e++) {
+					const KTap t = conv_ktap(p, kbase + e);
+					const int iy = iy0 + t.kh, ix = ix0 + t.kw;
+					const bool ok = n_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+					/* an offset past the buffer's extent reads as zero */
+					const unsigned voff = ok ? (unsigned)(xoff + t.koff) * (unsigned)sizeof(elem) : 0xfffffff0u;
+					if constexpr (DT == THHIP_U8) {
+						/* padding is the code of 0.0 (lowp_SpatialConvolution.c:101);
+						 * columns past N and the K padding hold 128, which the
+						 * re-centring below turns into 0 */
+						const unsigned char ld = __builtin_amdgcn_raw_buffer_load_b8(xrsrc, voff, 0, 0);
+						v[e] = ok ? ld : (unsigned char)((n_ok && kbase + e < p.K) ? p.zero : 128);
+					} else if constexpr (sizeof(elem) == 4) {
+						v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b32(xrsrc, voff, 0, 0));
+					} else {
+						v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b16(xrsrc, voff, 0, 0));
+					}
 				}
 			}
 			floatx4 packed;
@@ -241,6 +264,13 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 				/* code - 128 as a signed byte, and this thread's share of the
 				 * column sum of the re-centred codes */
 				intx4 q = __builtin_bit_cast(intx4, packed);
+				if constexpr (TAP) {
+					/* the whole vector shares one tap: fill it at once */
+					const int fill = (n_ok ? p.zero : 128) * 0x01010101;
+#pragma unroll
+					for (int d = 0; d < 4; d++)
+						q[d] = tap_ok ? q[d] : fill;
+				}
 #pragma unroll
 				for (int d = 0; d < 4; d++) {
 					q[d] ^= (int)0x80808080;
@@ -249,6 +279,15 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 				packed = __builtin_bit_cast(floatx4, q);
 			}
 			breg[j] = packed;
+		}
+		if constexpr (TAP) {
+			if (++t_kw == p.kW) {
+				t_kw = 0;
+				if (++t_kh == p.kH) {
+					t_kh = 0;
+					++t_cb;
+				}
+			}
 		}
 	};
 
@@ -389,17 +428,42 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 #define CONV_MPAD 128	/* packed rows are padded to the largest M tile */
 
 static inline int conv_chunk(int dtype) { return dtype == THHIP_F32 ? 8 : dtype == THHIP_U8 ? 32 : 16; }
-static inline int conv_kc(int K, int dtype)
+
+/* Tap-major K order needs whole blocks of 2*chunk input planes. */
+static inline bool conv_tap_major(int Ci, int dtype) { return Ci % (2 * conv_chunk(dtype)) == 0; }
+
+/* Number of K chunks (always whole K-tiles of two chunks). */
+static inline int conv_kc(int Ci, int kHW, int dtype)
 {
-	int c = conv_chunk(dtype);
-	int kc = (K + c - 1) / c;
-	return (kc + 1) & ~1;	/* whole K-tiles of two chunks */
+	const int c = conv_chunk(dtype);
+	if (conv_tap_major(Ci, dtype))
+		return Ci / c * kHW;
+	const int kc = (Ci * kHW + c - 1) / c;
+	return (kc + 1) & ~1;
 }
 
-extern "C" size_t thhip_conv_packed_bytes(int Co, int K, int dtype)
+/* Position of weight (plane c, tap) along the packed K axis. */
+static inline long conv_kpos(int c, int tap, int Ci, int kHW, int dtype)
+{
+	if (!conv_tap_major(Ci, dtype))
+		return (long)c * kHW + tap;
+	const int cb = 2 * conv_chunk(dtype);
+	return ((long)(c / cb) * kHW + tap) * cb + c % cb;
+}
+
+/* Element index of (row m, packed K position kp) in the packed buffer. */
+static inline size_t conv_pack_index(int m, long kp, int KC, int chunk)
+{
+	const int vec = chunk / 2;
+	const long kc = kp / chunk;
+	const int h = (int)(kp % chunk) / vec, e = (int)(kp % vec);
+	return ((((size_t)(m >> 5) * KC + kc) * 2 + h) * 32 + (m & 31)) * vec + e;
+}
+
+extern "C" size_t thhip_conv_packed_bytes(int Co, int Ci, int kHW, int dtype)
 {
 	size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
-	return mpad / 32 * conv_kc(K, dtype) * 1024;
+	return mpad / 32 * conv_kc(Ci, kHW, dtype) * 1024;
 }
 
 static inline unsigned short f32_to_f16_bits(float f)
@@ -420,31 +484,27 @@ static inline unsigned short f32_to_bf16_bits(float f)
 	return (unsigned short)(u >> 16);
 }
 
-extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int K, int dtype)
+extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW, int dtype)
 {
 	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
 		THError("thhip_conv_pack_weight: unsupported dtype %d", dtype);
-	const int chunk = conv_chunk(dtype), vec = chunk / 2, KC = conv_kc(K, dtype);
-	const size_t bytes = thhip_conv_packed_bytes(Co, K, dtype);
-	const int esize = thhip_esize(dtype);
+	const int chunk = conv_chunk(dtype), KC = conv_kc(Ci, kHW, dtype);
+	const size_t bytes = thhip_conv_packed_bytes(Co, Ci, kHW, dtype);
 	unsigned char *host = (unsigned char *)calloc(1, bytes);
 	if (!host)
 		THError("thhip_conv_pack_weight: out of host memory (%zu bytes)", bytes);
-	for (int m = 0; m < Co; m++) {
-		const int mb = m >> 5, mi = m & 31;
-		for (int k = 0; k < K; k++) {
-			const int kc = k / chunk, h = (k % chunk) / vec, e = k % vec;
-			const size_t idx = ((((size_t)mb * KC + kc) * 2 + h) * 32 + mi) * vec + e;
-			const float v = w[(size_t)m * K + k];
-			if (dtype == THHIP_F32)
-				((float *)host)[idx] = v;
-			else if (dtype == THHIP_F16)
-				((unsigned short *)host)[idx] = f32_to_f16_bits(v);
-			else
-				((unsigned short *)host)[idx] = f32_to_bf16_bits(v);
-		}
-	}
-	(void)esize;
+	for (int m = 0; m < Co; m++)
+		for (int c = 0; c < Ci; c++)
+			for (int tap = 0; tap < kHW; tap++) {
+				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, dtype), KC, chunk);
+				const float v = w[((size_t)m * Ci + c) * kHW + tap];
+				if (dtype == THHIP_F32)
+					((float *)host)[idx] = v;
+				else if (dtype == THHIP_F16)
+					((unsigned short *)host)[idx] = f32_to_f16_bits(v);
+				else
+					((unsigned short *)host)[idx] = f32_to_bf16_bits(v);
+			}
 	void *dev = thhip_malloc(bytes);
 	thhip_memcpy_h2d(dev, host, bytes);
 	free(host);
@@ -457,7 +517,10 @@ static void conv_launch(ConvParams &p)
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
 	dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
-	conv_mfma_kernel<DT, BM, BN, WGM, WGN><<<grid, dim3(CONV_THREADS), 0, thhip_stream()>>>(p);
+	if (conv_tap_major(p.Ci, DT))
+		conv_mfma_kernel<DT, BM, BN, WGM, WGN, true><<<grid, dim3(CONV_THREADS), 0, thhip_stream()>>>(p);
+	else
+		conv_mfma_kernel<DT, BM, BN, WGM, WGN, false><<<grid, dim3(CONV_THREADS), 0, thhip_stream()>>>(p);
 }
 
 template <int DT>
@@ -516,17 +579,19 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 		p.B = bn; p.Ci = Ci; p.H = H; p.W = W; p.Co = Co; p.kH = kH; p.kW = kW;
 		p.dH = dH; p.dW = dW; p.padH = padH; p.padW = padW; p.oH = oH; p.oW = oW;
 		p.K = (int)K;
-		p.KC = conv_kc((int)K, dtype);
+		p.KC = conv_kc(Ci, kH * kW, dtype);
 		p.N = bn * oH * oW;
 		p.oHW = oH * oW;
 		p.HW = H * W;
 		p.kHW = kH * kW;
-		p.magic_khw = conv_magic(kH * kW);
-		p.magic_kw = conv_magic(kW);
+		p.magic_khw = (unsigned)conv_magic(kH * kW);
+		p.mhi_khw = (unsigned)(conv_magic(kH * kW) >> 32);
+		p.magic_kw = (unsigned)conv_magic(kW);
+		p.mhi_kw = (unsigned)(conv_magic(kW) >> 32);
 		p.act = act; p.thr = thr; p.val = val;
 		p.x_bytes = (unsigned)(bn * in_img * esize);
 		if (u8) {
-			p.rowsum = (const int *)((const char *)wpacked + thhip_conv_packed_bytes(Co, (int)K, THHIP_U8));
+			p.rowsum = (const int *)((const char *)wpacked + thhip_conv_packed_bytes(Co, Ci, kH * kW, THHIP_U8));
 			p.addend = u8->addend;
 			p.zero = u8->zero;
 			p.offA = 128 + u8->a_off;
@@ -551,12 +616,12 @@ extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bi
 	conv_run(x, wpacked, bias, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0);
 }
 
-/* uint8 codes [Co][K] -> (code - 128) as signed bytes in the packed layout,
+/* uint8 codes [Co][Ci][kHW] -> (code - 128) as signed bytes in the packed layout,
  * followed by the per-row sums of the re-centred codes. */
-extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int K)
+extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int Ci, int kHW)
 {
-	const int chunk = 32, vec = 16, KC = conv_kc(K, THHIP_U8);
-	const size_t bytes = thhip_conv_packed_bytes(Co, K, THHIP_U8);
+	const int chunk = 32, KC = conv_kc(Ci, kHW, THHIP_U8);
+	const size_t bytes = thhip_conv_packed_bytes(Co, Ci, kHW, THHIP_U8);
 	const size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
 	const size_t total = bytes + mpad * sizeof(int);
 	unsigned char *host = (unsigned char *)calloc(1, total);
@@ -564,15 +629,14 @@ extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int K
 		THError("thhip_conv_pack_weight_u8: out of host memory (%zu bytes)", total);
 	int *rowsum = (int *)(host + bytes);
 	for (int m = 0; m < Co; m++) {
-		const int mb = m >> 5, mi = m & 31;
 		int sum = 0;
-		for (int k = 0; k < K; k++) {
-			const int kc = k / chunk, h = (k % chunk) / vec, e = k % vec;
-			const size_t idx = ((((size_t)mb * KC + kc) * 2 + h) * 32 + mi) * vec + e;
-			const int c = (int)w[(size_t)m * K + k] - 128;
-			host[idx] = (unsigned char)(signed char)c;
-			sum += c;
-		}
+		for (int c = 0; c < Ci; c++)
+			for (int tap = 0; tap < kHW; tap++) {
+				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, THHIP_U8), KC, chunk);
+				const int v = (int)w[((size_t)m * Ci + c) * kHW + tap] - 128;
+				host[idx] = (unsigned char)(signed char)v;
+				sum += v;
+			}
 		rowsum[m] = sum;
 	}
 	void *dev = thhip_malloc(total);
@@ -620,7 +684,7 @@ extern "C" void lowpgemm(const int is_a_transposed, const int is_b_transposed, c
 			memcpy(btmp + (size_t)i * n, b + (size_t)i * ldb, n);
 		bp = btmp;
 	}
-	void *wp = thhip_conv_pack_weight_u8(ap, m, k);
+	void *wp = thhip_conv_pack_weight_u8(ap, m, k, 1);
 	unsigned char *dx = (unsigned char *)thhip_malloc((size_t)k * n);
 	unsigned char *dy = (unsigned char *)thhip_malloc((size_t)m * n);
 	thhip_memcpy_h2d(dx, bp, (size_t)k * n);
@@ -640,36 +704,42 @@ extern "C" void lowpgemm(const int is_a_transposed, const int is_b_transposed, c
 	free(ctmp);
 }
 
-/* Packed weights -> row-major [Co][K] in the same dtype, on the device; used
- * when a layer turns out to be a matrix-vector product (one output position). */
-template <typename E, int CHUNK>
-__global__ void conv_unpack_rows_kernel(const E *wp, E *rows, int Co, int K, int KC)
+/* Packed weights -> row-major [Co][Ci*kHW] in the same dtype, on the device;
+ * used when a layer turns out to be a matrix-vector product (one output
+ * position). */
+template <typename E>
+__global__ void conv_unpack_rows_kernel(const E *wp, E *rows, int Co, int Ci, int kHW, int KC, int chunk, int tapmajor)
 {
-	constexpr int VEC = CHUNK / 2;
+	const int K = Ci * kHW, vec = chunk / 2, cb = 2 * chunk;
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
 	const long total = (long)Co * K, step = (long)gridDim.x * blockDim.x;
 	for (; i < total; i += step) {
 		const int m = (int)(i / K), k = (int)(i % K);
-		const int mb = m >> 5, mi = m & 31;
-		const int kc = k / CHUNK, h = (k % CHUNK) / VEC, e = k % VEC;
-		rows[i] = wp[((((size_t)mb * KC + kc) * 2 + h) * 32 + mi) * VEC + e];
+		long kp = k;
+		if (tapmajor) {
+			const int c = k / kHW, tap = k % kHW;
+			kp = ((long)(c / cb) * kHW + tap) * cb + c % cb;
+		}
+		const long kc = kp / chunk;
+		const int h = (int)(kp % chunk) / vec, e = (int)(kp % vec);
+		rows[i] = wp[((((size_t)(m >> 5) * KC + kc) * 2 + h) * 32 + (m & 31)) * vec + e];
 	}
 }
 
-extern "C" void *thhip_conv_unpack_rows(const void *wpacked, int Co, int K, int dtype)
+extern "C" void *thhip_conv_unpack_rows(const void *wpacked, int Co, int Ci, int kHW, int dtype)
 {
-	const int KC = conv_kc(K, dtype);
-	const long total = (long)Co * K;
+	const int KC = conv_kc(Ci, kHW, dtype), chunk = conv_chunk(dtype), tm = conv_tap_major(Ci, dtype);
+	const long total = (long)Co * Ci * kHW;
 	void *rows = thhip_malloc((size_t)total * thhip_esize(dtype));
 	long blocks = (total + 255) / 256;
 	if (blocks > 65536)
 		blocks = 65536;
 	if (dtype == THHIP_F32)
-		conv_unpack_rows_kernel<float, 8><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
-			(const float *)wpacked, (float *)rows, Co, K, KC);
+		conv_unpack_rows_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
+			(const float *)wpacked, (float *)rows, Co, Ci, kHW, KC, chunk, tm);
 	else if (dtype == THHIP_F16 || dtype == THHIP_BF16)
-		conv_unpack_rows_kernel<unsigned short, 16><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
-			(const unsigned short *)wpacked, (unsigned short *)rows, Co, K, KC);
+		conv_unpack_rows_kernel<unsigned short><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
+			(const unsigned short *)wpacked, (unsigned short *)rows, Co, Ci, kHW, KC, chunk, tm);
 	else
 		THError("thhip_conv_unpack_rows: unsupported dtype %d", dtype);
 	hipcheck(hipGetLastError());

@@ -378,3 +378,21 @@ int THHipNetwork_setInputQuant(THNETWORK *net, float mult, float sub)
 	hn->cur_sub = sub;
 	return 0;
 }
+
+/* Device counterpart of THLowpTensor_newFromFloatTensor (lowp_basic.c:5-38):
+ * uploads a host float tensor, quantises it on the device with one min/max
+ * over the whole tensor and records (mult, sub) as the quantisation of the
+ * network's next input. */
+THFloatTensor *THHipLowpTensor_newFromFloatTensor(THNETWORK *net, THFloatTensor *t)
+{
+	if (engine_of(net) != ENGINE_HIPLOWP)
+		THError("THHipLowpTensor_newFromFloatTensor needs a network made by THCreateHipLowpNetwork");
+	struct hipnet *hn = (struct hipnet *)net->net;
+	THFloatTensor *f = upload_as(t, THHIP_F32);
+	THFloatTensor *q = device_tensor_like(f, THHIP_U8);
+	thhip_quantize((const float *)f->storage->data, (unsigned char *)q->storage->data, THFloatTensor_nElement(f),
+		&hn->cur_mult, &hn->cur_sub);
+	thhip_sync();
+	THFloatTensor_free(f);
+	return q;
+}

@@ -155,12 +155,17 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 	const void *x = thhip_tensor_ptr(in, dt);
 	void *y = conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
 	const int K = c->nInputPlane * c->kH * c->kW;
-	if (s.B == 1 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W) {
-		/* one output position: a matrix-vector product over the flattened
-		 * input, bound by reading the weights once */
+	const int one_position = oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W;
+	if (one_position && (s.B == 1 || thhip_linear_batched_supported(s.B, K, c->nOutputPlane, dt))) {
+		/* one output position per image: a matrix-vector (or skinny matrix)
+		 * product over the flattened input, bound by reading the weights once */
 		if (!hm->wrow)
-			hm->wrow = thhip_conv_unpack_rows(hm->wpacked, c->nOutputPlane, K, dt);
-		thhip_gemv(x, hm->wrow, hm->bias, y, K, c->nOutputPlane, hm->fused_act, hm->thr, hm->val, dt);
+			hm->wrow = thhip_conv_unpack_rows(hm->wpacked, c->nOutputPlane, c->nInputPlane, c->kH * c->kW, dt);
+		if (s.B == 1)
+			thhip_gemv(x, hm->wrow, hm->bias, y, K, c->nOutputPlane, hm->fused_act, hm->thr, hm->val, dt);
+		else
+			thhip_linear_batched(x, hm->wrow, hm->bias, y, s.B, K, c->nOutputPlane, hm->fused_act, hm->thr,
+				hm->val, dt);
 	} else
 		thhip_conv2d(x, hm->wpacked, hm->bias, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
 			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, hm->fused_act, hm->thr, hm->val, dt);
@@ -683,7 +688,7 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 	case MT_SpatialConvolutionVirtMM:
 	case MT_Linear: {
 		THFloatTensor *w, *b;
-		int Co, K;
+		int Co, K, Ci, kHW;
 		if (sm->type == MT_Linear) {
 			/* Linear runs as a 1x1 convolution (cudnn_basic.c:244-265) */
 			w = sm->Linear.weight;
@@ -694,6 +699,8 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 				THError("Linear weight must be a matrix");
 			Co = (int)w->size[0];
 			K = (int)w->size[1];
+			Ci = K;
+			kHW = 1;
 			memset(&m->SpatialConvolution, 0, sizeof(m->SpatialConvolution));
 			m->type = MT_SpatialConvolutionMM;
 			m->SpatialConvolution.dW = m->SpatialConvolution.dH = 1;
@@ -706,14 +713,16 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 			w = c->weight;
 			b = c->bias;
 			Co = c->nOutputPlane;
-			K = c->nInputPlane * c->kH * c->kW;
+			Ci = c->nInputPlane;
+			kHW = c->kH * c->kW;
+			K = Ci * kHW;
 		}
 		contiguous_host_floats(w, "convolution weight", (long)Co * K);
 		m->SpatialConvolution.weight = m->SpatialConvolution.bias = m->SpatialConvolution.finput = 0;
 		if (lowp) {
 			float bm = 0, bsub = 0;
 			unsigned char *wq = quantize_host(THFloatTensor_data(w), (long)Co * K, &hm->wm, &hm->wsub);
-			hm->wpacked = thhip_conv_pack_weight_u8(wq, Co, K);
+			hm->wpacked = thhip_conv_pack_weight_u8(wq, Co, Ci, kHW);
 			free(wq);
 			if (!contiguous_host_floats(b, "convolution bias", Co))
 				THError("the uint8 engine needs a bias on every convolution (lowp_SpatialConvolution.c:111-120)");
@@ -733,7 +742,7 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 			free(bq);
 			m->updateOutput = HipLowp_SpatialConvolution_updateOutput;
 		} else {
-			hm->wpacked = thhip_conv_pack_weight(THFloatTensor_data(w), Co, K, dtype);
+			hm->wpacked = thhip_conv_pack_weight(THFloatTensor_data(w), Co, Ci, kHW, dtype);
 			hm->bias = upload_floats(b, "convolution bias", Co);
 			m->updateOutput = Hip_SpatialConvolution_updateOutput;
 		}
