@@ -351,6 +351,10 @@ void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype);
 
+/* Tuning override for experiments: force the convolution's workgroup tile
+ * (bm x bn in {64,128}) and split-K factor; 0 leaves a choice automatic. */
+void thhip_conv_set_tuning(int bm, int bn, int splitk);
+
 /* Replaces nn_Linear_updateOutput's 1-D branch (Linear.c:86-90 ->
  * thbasic.c:713-741 -> sgemv.c:48-105): y = bias + W x, W row-major
  * [nOut][nIn] fp32/fp16/bf16, optional fused threshold. */

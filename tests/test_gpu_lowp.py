@@ -74,6 +74,27 @@ def test_conv_u8_wrapping_requantisation_and_extreme_offsets(hiplib, oracle):
         assert np.array_equal(got, want), prm
 
 
+def test_conv_u8_split_k_bit_exact(hiplib, oracle):
+    rngv = 16.0
+    om, osub = float(np.float32(255) / np.float32(rngv)), -rngv / 2
+    try:
+        for (bm, bn, sk) in [(64, 64, 2), (64, 64, 5), (128, 128, 3), (128, 64, 4)]:
+            hiplib.thhip_conv_set_tuning(bm, bn, sk)
+            for i in (1, 5, 10):
+                x, w, b, d, p = _lowp_case(i, seed=50)
+                xq, im, isub = oracle.lowp_quantize(x)
+                wq, wm, wsub = oracle.lowp_quantize(w)
+                bq, bm_, bsub = oracle.lowp_quantize(b)
+                want = oracle.lowp_conv2d(xq, im, isub, wq, wm, wsub, bq, bm_, bsub, om, osub, d, p)
+                prm = oracle.lowp_mm_params(wm, wsub, im, isub, om, osub)
+                zero = int(np.round(np.float32(-isub) * np.float32(im)))
+                addend = np.array([oracle.lowp_bias_addend(int(c), bm_, bsub, om) for c in bq], np.int32)
+                got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm)
+                assert np.array_equal(got, want), (bm, bn, sk, i)
+    finally:
+        hiplib.thhip_conv_set_tuning(0, 0, 0)
+
+
 def test_lowpgemm_drop_in(hiplib, oracle):
     g = cases.rng(1101)
     for (m, n, k) in ((3, 5, 7), (64, 3025, 363), (100, 1, 900), (130, 77, 65)):

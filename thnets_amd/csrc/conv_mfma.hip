@@ -45,6 +45,10 @@ struct ConvParams {
 	float thr, val;
 	int tiles_m, tiles_n;
 	unsigned x_bytes;
+	/* split-K: S workgroups share an output tile, each over a K range */
+	int splitk;
+	int *ws;		/* [tile][S][BM*BN] partial accumulators (float or int bits) */
+	unsigned *cnt;		/* [tile] arrival counters, zero between launches */
 	/* uint8 path only */
 	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
 	const int *addend;	/* per-plane bias addend, or NULL */
@@ -173,6 +177,10 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		const int q = nblk >> 3, r = nblk & 7;
 		tile = xcd * q + (xcd < r ? xcd : r) + local;
 	}
+	/* split-K: the S parts of a tile are neighbours in the order */
+	const int split = p.splitk > 1 ? tile % p.splitk : 0;
+	if (p.splitk > 1)
+		tile /= p.splitk;
 	const int tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
 
 	/* ---- B gather role: one output position per thread ---- */
@@ -317,31 +325,42 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 			for (int r = 0; r < 16; r++)
 				acc[i][j][r] = 0;
 
-	const int nkt = p.KC / 2;
-	load_tile(0);
-	store_tile(0);
+	const int nkt_all = p.KC / 2;
+	const int kt0 = p.splitk > 1 ? (int)((long)nkt_all * split / p.splitk) : 0;
+	const int nkt = p.splitk > 1 ? (int)((long)nkt_all * (split + 1) / p.splitk) : nkt_all;
+	if constexpr (TAP) {
+		t_cb = kt0 / p.kHW;
+		const int tap = kt0 - t_cb * p.kHW;
+		t_kh = tap / p.kW;
+		t_kw = tap - t_kh * p.kW;
+	}
+	load_tile(kt0);
+	store_tile(kt0 & 1);
 	__syncthreads();
-	for (int kt = 0; kt < nkt; kt++) {
+	for (int kt = kt0; kt < nkt; kt++) {
 		const int cur = kt & 1;
 		if (kt + 1 < nkt)
 			load_tile(kt + 1);
 		const floatx4 *la = lds + cur * (A_VECS + B_VECS);
 		const floatx4 *lb = la + A_VECS;
+		/* both chunks' fragments first, then all MFMAs back to back */
+		floatx4 af[2][TM], bf[2][TN];
 #pragma unroll
 		for (int kci = 0; kci < 2; kci++) {
-			floatx4 af[TM], bf[TN];
 #pragma unroll
 			for (int i = 0; i < TM; i++)
-				af[i] = la[(kci * MB + wm * TM + i) * 64 + lane];
+				af[kci][i] = la[(kci * MB + wm * TM + i) * 64 + lane];
 #pragma unroll
 			for (int j = 0; j < TN; j++)
-				bf[j] = lb[(kci * NB + wn * TN + j) * 64 + lane];
+				bf[kci][j] = lb[(kci * NB + wn * TN + j) * 64 + lane];
+		}
+#pragma unroll
+		for (int kci = 0; kci < 2; kci++)
 #pragma unroll
 			for (int i = 0; i < TM; i++)
 #pragma unroll
 				for (int j = 0; j < TN; j++)
-					conv_mma<DT>(acc[i][j], af[i], bf[j]);
-		}
+					conv_mma<DT>(acc[i][j], af[kci][i], bf[kci][j]);
 		if (kt + 1 < nkt)
 			store_tile(cur ^ 1);
 		__syncthreads();
@@ -349,15 +368,75 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 
 	/* ---- epilogue ---- */
 	elem *y = (elem *)p.y;
+	__shared__ int cs[DT == THHIP_U8 ? BN : 1];
 	if constexpr (DT == THHIP_U8) {
 		/* Every (chunk, half) share of a column was gathered by one of the
 		 * 256/BN threads that own it: add the shares up in LDS. */
-		__shared__ int cs[BN];
 		if (tid < BN)
 			cs[tid] = 0;
 		__syncthreads();
 		atomicAdd(&cs[n_local], colsum);
 		__syncthreads();
+	}
+	if (p.splitk > 1) {
+		/* Each part stores its accumulators (for uint8 with its share of the
+		 * column-sum term folded in) in its own slice; the part that arrives
+		 * last adds the slices in a fixed order and finishes the tile, so the
+		 * result does not depend on timing. */
+		constexpr int TILE_WORDS = BM * BN;
+		int *mine = p.ws + ((size_t)tile * p.splitk + split) * TILE_WORDS;
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++) {
+				int colterm = 0;
+				if constexpr (DT == THHIP_U8)
+					colterm = p.offA * cs[(wn * TN + j) * 32 + (lane & 31)];
+#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					int word;
+					if constexpr (DT == THHIP_U8)
+						word = acc[i][j][r] + colterm;
+					else
+						word = __float_as_int(acc[i][j][r]);
+					mine[((i * TN + j) * 16 + r) * CONV_THREADS + tid] = word;
+				}
+			}
+		__threadfence();
+		__shared__ unsigned ticket;
+		__syncthreads();
+		if (tid == 0)
+			ticket = atomicAdd(&p.cnt[tile], 1u);
+		__syncthreads();
+		if (ticket != (unsigned)p.splitk - 1)
+			return;
+		__threadfence();
+		if (tid == 0)
+			p.cnt[tile] = 0;	/* ready for the next launch */
+		const int *all = p.ws + (size_t)tile * p.splitk * TILE_WORDS;
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					const int *src = all + ((i * TN + j) * 16 + r) * CONV_THREADS + tid;
+					if constexpr (DT == THHIP_U8) {
+						int sum = 0;
+						for (int q = 0; q < p.splitk; q++)
+							sum += __hip_atomic_load(src + (size_t)q * TILE_WORDS, __ATOMIC_RELAXED,
+								__HIP_MEMORY_SCOPE_AGENT);
+						acc[i][j][r] = sum;
+					} else {
+						float sum = 0;
+						for (int q = 0; q < p.splitk; q++)
+							sum += __int_as_float(__hip_atomic_load(src + (size_t)q * TILE_WORDS,
+								__ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+						acc[i][j][r] = sum;
+					}
+				}
+	}
+	if constexpr (DT == THHIP_U8) {
 		/* sum (w+a_off)(x+b_off) with w = w'+128, x = x'+128:
 		 *   sum w'x' + (128+b_off) rowsum + (128+a_off) colsum + K (128+a_off)(128+b_off) */
 		const int tail0 = (p.oHW / 8) * 8;	/* lowpadd's unclamped tail starts here */
@@ -369,7 +448,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 				continue;
 			const int b = n / p.oHW, rem = n - b * p.oHW;
 			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
-			const int colterm = p.offA * cs[nl] + p.K * p.offA * p.offB;
+			const int colterm = (p.splitk > 1 ? 0 : p.offA * cs[nl]) + p.K * p.offA * p.offB;
 #pragma unroll
 			for (int i = 0; i < TM; i++) {
 				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
@@ -511,12 +590,55 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 	return dev;
 }
 
+/* Experiment / tuning override: 0 = choose automatically. */
+static int g_force_bm, g_force_bn, g_force_splitk;
+
+extern "C" void thhip_conv_set_tuning(int bm, int bn, int splitk)
+{
+	g_force_bm = bm;
+	g_force_bn = bn;
+	g_force_splitk = splitk;
+}
+
+/* Split-K scratch: partial tiles and arrival counters (grow-only). */
+static int *g_ws;
+static size_t g_ws_bytes;
+static unsigned *g_cnt;
+static size_t g_cnt_n;
+
+static void conv_scratch(ConvParams &p, size_t tiles, size_t tile_words)
+{
+	const size_t need = tiles * p.splitk * tile_words * sizeof(int);
+	if (need > g_ws_bytes) {
+		hipcheck(hipStreamSynchronize(thhip_stream()));
+		thhip_free(g_ws);
+		g_ws = (int *)thhip_malloc(need);
+		g_ws_bytes = need;
+	}
+	if (tiles > g_cnt_n) {
+		hipcheck(hipStreamSynchronize(thhip_stream()));
+		thhip_free(g_cnt);
+		g_cnt_n = tiles < 4096 ? 4096 : tiles;
+		g_cnt = (unsigned *)thhip_malloc(g_cnt_n * sizeof(unsigned));
+		thhip_memset(g_cnt, 0, g_cnt_n * sizeof(unsigned));
+	}
+	p.ws = g_ws;
+	p.cnt = g_cnt;
+}
+
 template <int DT, int BM, int BN, int WGM, int WGN>
-static void conv_launch(ConvParams &p)
+static void conv_launch(ConvParams &p, int splitk)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
-	dim3 grid((unsigned)(p.tiles_m * p.tiles_n));
+	const int nkt = p.KC / 2;
+	if (splitk > nkt)
+		splitk = nkt;
+	p.splitk = splitk < 1 ? 1 : splitk;
+	const size_t tiles = (size_t)p.tiles_m * p.tiles_n;
+	if (p.splitk > 1)
+		conv_scratch(p, tiles, (size_t)BM * BN);
+	dim3 grid((unsigned)(tiles * p.splitk));
 	if (conv_tap_major(p.Ci, DT))
 		conv_mfma_kernel<DT, BM, BN, WGM, WGN, true><<<grid, dim3(CONV_THREADS), 0, thhip_stream()>>>(p);
 	else
@@ -527,17 +649,37 @@ template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
 	/* Tile choice: the largest tile that still yields enough workgroups to
-	 * fill 256 CUs a couple of times over; Co <= 64 never needs BM = 128. */
+	 * fill 256 CUs a couple of times over; Co <= 64 never needs BM = 128.
+	 * Splitting K is available (thhip_conv_set_tuning) but measured slower than
+	 * unsplit 64x64 tiles on every layer shape tried, so it is never chosen. */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	const long t64n = (long)((p.Co + 127) / 128) * ((p.N + 63) / 64);
-	if (p.Co > 64 && t128 >= 512)
-		conv_launch<DT, 128, 128, 2, 2>(p);
-	else if (p.Co > 64 && t64n >= 384)
-		conv_launch<DT, 128, 64, 2, 2>(p);
-	else if (p.Co <= 64 && (long)((p.N + 127) / 128) >= 512)
-		conv_launch<DT, 64, 128, 2, 2>(p);
+	int bm, bn, splitk = 1;
+	if (p.Co > 64 && t128 >= 512) {
+		bm = 128; bn = 128;
+	} else if (p.Co > 64 && t64n >= 384) {
+		bm = 128; bn = 64;
+	} else if (p.Co <= 64 && (long)((p.N + 127) / 128) >= 512) {
+		bm = 64; bn = 128;
+	} else {
+		bm = 64; bn = 64;
+	}
+	if (g_force_bm)
+		bm = g_force_bm;
+	if (g_force_bn)
+		bn = g_force_bn;
+	if (g_force_splitk)
+		splitk = g_force_splitk;
+	if (bm == 128 && bn == 128)
+		conv_launch<DT, 128, 128, 2, 2>(p, splitk);
+	else if (bm == 128 && bn == 64)
+		conv_launch<DT, 128, 64, 2, 2>(p, splitk);
+	else if (bm == 64 && bn == 128)
+		conv_launch<DT, 64, 128, 2, 2>(p, splitk);
+	else if (bm == 64 && bn == 64)
+		conv_launch<DT, 64, 64, 2, 2>(p, splitk);
 	else
-		conv_launch<DT, 64, 64, 2, 2>(p);
+		THError("thhip_conv2d: no %dx%d tile", bm, bn);
 }
 
 struct ConvU8Args {
