@@ -352,8 +352,9 @@ void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y
 	int act, float thr, float val, int dtype);
 
 /* Tuning override for experiments: force the convolution's workgroup tile
- * (bm x bn in {64,128}) and split-K factor; 0 leaves a choice automatic. */
-void thhip_conv_set_tuning(int bm, int bn, int splitk);
+ * (bm x bn in {64,128}), its split-K factor and the number of workgroups
+ * allowed to share a CU; 0 leaves a choice automatic. */
+void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);
 
 /* Replaces nn_Linear_updateOutput's 1-D branch (Linear.c:86-90 ->
  * thbasic.c:713-741 -> sgemv.c:48-105): y = bias + W x, W row-major

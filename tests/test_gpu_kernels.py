@@ -83,7 +83,7 @@ def test_conv_split_k_and_forced_tiles(hiplib, oracle):
     try:
         for (bm, bn) in [(64, 64), (128, 64), (64, 128), (128, 128)]:
             for sk in (1, 2, 3, 7):
-                hiplib.thhip_conv_set_tuning(bm, bn, sk)
+                hiplib.thhip_conv_set_tuning(bm, bn, sk, sk % 3)
                 for i in (4, 5, 10):
                     x, s = cases.conv_case(i)
                     d, p = (s["dH"], s["dW"]), (s["padH"], s["padW"])
@@ -91,12 +91,12 @@ def test_conv_split_k_and_forced_tiles(hiplib, oracle):
                     for rep in range(2):
                         y = G.conv2d(hiplib, x, s["weight"], s["bias"], d, p, act=1, thr=0.0, val=0.0)
                         G.assert_close(y, np.maximum(want, 0), FP32_TOL, "tile %dx%d splitk %d case %d" % (bm, bn, sk, i))
-        hiplib.thhip_conv_set_tuning(64, 64, 4)
+        hiplib.thhip_conv_set_tuning(64, 64, 4, 2)
         x, s = cases.conv_case(10)
         y = G.conv2d(hiplib, x, s["weight"], s["bias"], (1, 1), (1, 1), dtype=G.F16)
         G.assert_close(y, oracle.conv2d(x, s["weight"], s["bias"], (1, 1), (1, 1)), HALF_TOL)
     finally:
-        hiplib.thhip_conv_set_tuning(0, 0, 0)
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
 def test_pack_unpack_roundtrip(hiplib):

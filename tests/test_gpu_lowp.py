@@ -79,7 +79,7 @@ def test_conv_u8_split_k_bit_exact(hiplib, oracle):
     om, osub = float(np.float32(255) / np.float32(rngv)), -rngv / 2
     try:
         for (bm, bn, sk) in [(64, 64, 2), (64, 64, 5), (128, 128, 3), (128, 64, 4)]:
-            hiplib.thhip_conv_set_tuning(bm, bn, sk)
+            hiplib.thhip_conv_set_tuning(bm, bn, sk, sk % 3)
             for i in (1, 5, 10):
                 x, w, b, d, p = _lowp_case(i, seed=50)
                 xq, im, isub = oracle.lowp_quantize(x)
@@ -92,7 +92,7 @@ def test_conv_u8_split_k_bit_exact(hiplib, oracle):
                 got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm)
                 assert np.array_equal(got, want), (bm, bn, sk, i)
     finally:
-        hiplib.thhip_conv_set_tuning(0, 0, 0)
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
 def test_lowpgemm_drop_in(hiplib, oracle):

@@ -77,7 +77,7 @@ PROTOTYPES = {
     "thhip_conv_packed_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv_unpack_rows": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
-    "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int]),
+    "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_linear_batched_supported": (C.c_int, [C.c_int] * 4),
     "thhip_linear_batched": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),

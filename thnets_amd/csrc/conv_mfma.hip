@@ -591,13 +591,14 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 }
 
 /* Experiment / tuning override: 0 = choose automatically. */
-static int g_force_bm, g_force_bn, g_force_splitk;
+static int g_force_bm, g_force_bn, g_force_splitk, g_force_wgs;
 
-extern "C" void thhip_conv_set_tuning(int bm, int bn, int splitk)
+extern "C" void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu)
 {
 	g_force_bm = bm;
 	g_force_bn = bn;
 	g_force_splitk = splitk;
+	g_force_wgs = wgs_per_cu;
 }
 
 /* Split-K scratch: partial tiles and arrival counters (grow-only). */
@@ -626,8 +627,35 @@ static void conv_scratch(ConvParams &p, size_t tiles, size_t tile_words)
 	p.cnt = g_cnt;
 }
 
+#define CONV_LDS_PER_CU (160 * 1024)
+
+/* Launches kernel K with LDS padded so that at most `wgs` workgroups share a
+ * CU (0 = whatever registers and LDS allow).  The hardware hands left-over
+ * workgroups to as few CUs as it can fill, so fewer, faster residents per CU
+ * shorten the last, partially filled round of a grid. */
+template <typename K>
+static void conv_launch_kernel(K kernel, ConvParams &p, dim3 grid, int wgs)
+{
+	static int static_lds = -1, max_wgs;
+	if (static_lds < 0) {
+		hipFuncAttributes attr;
+		hipcheck(hipFuncGetAttributes(&attr, (const void *)kernel));
+		static_lds = (int)attr.sharedSizeBytes;
+		hipcheck(hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+			CONV_LDS_PER_CU - static_lds));
+		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&max_wgs, (const void *)kernel, CONV_THREADS, 0));
+	}
+	int dyn = 0;
+	if (wgs > 0 && wgs < max_wgs) {
+		dyn = CONV_LDS_PER_CU / (wgs + 1) + 512 - static_lds;
+		if (dyn < 0)
+			dyn = 0;
+	}
+	kernel<<<grid, dim3(CONV_THREADS), dyn, thhip_stream()>>>(p);
+}
+
 template <int DT, int BM, int BN, int WGM, int WGN>
-static void conv_launch(ConvParams &p, int splitk)
+static void conv_launch(ConvParams &p, int splitk, int wgs)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
@@ -640,27 +668,33 @@ static void conv_launch(ConvParams &p, int splitk)
 		conv_scratch(p, tiles, (size_t)BM * BN);
 	dim3 grid((unsigned)(tiles * p.splitk));
 	if (conv_tap_major(p.Ci, DT))
-		conv_mfma_kernel<DT, BM, BN, WGM, WGN, true><<<grid, dim3(CONV_THREADS), 0, thhip_stream()>>>(p);
+		conv_launch_kernel(conv_mfma_kernel<DT, BM, BN, WGM, WGN, true>, p, grid, wgs);
 	else
-		conv_mfma_kernel<DT, BM, BN, WGM, WGN, false><<<grid, dim3(CONV_THREADS), 0, thhip_stream()>>>(p);
+		conv_launch_kernel(conv_mfma_kernel<DT, BM, BN, WGM, WGN, false>, p, grid, wgs);
 }
 
 template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
-	/* Tile choice: the largest tile that still yields enough workgroups to
-	 * fill 256 CUs a couple of times over; Co <= 64 never needs BM = 128.
-	 * Splitting K is available (thhip_conv_set_tuning) but measured slower than
-	 * unsplit 64x64 tiles on every layer shape tried, so it is never chosen. */
+	/* Tile choice, from sweeps over the VGG / AlexNet / ResNet layer shapes on
+	 * a 256-CU part.  The hardware packs the workgroups of a grid's last,
+	 * partially filled round onto as few CUs as they fit, so a round costs
+	 * (residents per CU) x (tile time) even when nearly empty: with many tiles,
+	 * half-size tiles at four residents per CU waste the least; with few, the
+	 * big tile's better operand reuse wins; with very few, the smallest tile
+	 * spreads over the most CUs.  Splitting K is available
+	 * (thhip_conv_set_tuning) but measured slower than unsplit 64x64 tiles on
+	 * every layer shape tried, so it is never chosen. */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
-	const long t64n = (long)((p.Co + 127) / 128) * ((p.N + 63) / 64);
-	int bm, bn, splitk = 1;
-	if (p.Co > 64 && t128 >= 512) {
+	int bm, bn, splitk = 1, wgs = 0;
+	if (p.Co <= 64) {
+		bm = 64;
+		bn = (long)((p.N + 127) / 128) >= 512 ? 128 : 64;
+		wgs = 4;
+	} else if (t128 >= 700) {
+		bm = 128; bn = 64; wgs = 4;
+	} else if (t128 >= 300) {
 		bm = 128; bn = 128;
-	} else if (p.Co > 64 && t64n >= 384) {
-		bm = 128; bn = 64;
-	} else if (p.Co <= 64 && (long)((p.N + 127) / 128) >= 512) {
-		bm = 64; bn = 128;
 	} else {
 		bm = 64; bn = 64;
 	}
@@ -670,14 +704,16 @@ static void conv_dispatch(ConvParams &p)
 		bn = g_force_bn;
 	if (g_force_splitk)
 		splitk = g_force_splitk;
+	if (g_force_wgs)
+		wgs = g_force_wgs;
 	if (bm == 128 && bn == 128)
-		conv_launch<DT, 128, 128, 2, 2>(p, splitk);
+		conv_launch<DT, 128, 128, 2, 2>(p, splitk, wgs);
 	else if (bm == 128 && bn == 64)
-		conv_launch<DT, 128, 64, 2, 2>(p, splitk);
+		conv_launch<DT, 128, 64, 2, 2>(p, splitk, wgs);
 	else if (bm == 64 && bn == 128)
-		conv_launch<DT, 64, 128, 2, 2>(p, splitk);
+		conv_launch<DT, 64, 128, 2, 2>(p, splitk, wgs);
 	else if (bm == 64 && bn == 64)
-		conv_launch<DT, 64, 64, 2, 2>(p, splitk);
+		conv_launch<DT, 64, 64, 2, 2>(p, splitk, wgs);
 	else
 		THError("thhip_conv2d: no %dx%d tile", bm, bn);
 }
