@@ -28,6 +28,10 @@ from thnets_amd import api, configs  # noqa: E402
 
 PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_TOPS_INT8_MFMA = 5030.0
+# HBM bytes per conv_mfma_kernel launch in the VGG-16 b16 step (average of the 13), from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled against a 256 MiB copy
+# (profiles/conv_mfma_vgg16_fp32_b16_counters.md); algorithmic bytes are 115.9e6.
+CONV_HBM_BYTES_PER_LAUNCH = 163.2e6
 
 
 def profile_get(lib, fam):
@@ -114,6 +118,16 @@ def main():
     lib = api.load_library()
     lib.THInit()
 
+    # A plain device-to-device copy of known size: under `rocprofv3 --pmc FETCH_SIZE`
+    # / `WRITE_SIZE` its dispatch calibrates the counters (256 MiB read, 256 MiB written).
+    cal_bytes = 256 << 20
+    ca, cb = api.DeviceArray(lib, nbytes=cal_bytes), api.DeviceArray(lib, nbytes=cal_bytes)
+    lib.thhip_memset(ca.ptr, 1, cal_bytes)
+    lib.thhip_memcpy_d2d(cb.ptr, ca.ptr, cal_bytes)
+    lib.thhip_sync()
+    ca.free()
+    cb.free()
+
     # ---- VGG-16 fp32 batch 16 (the headline) ----
     cfg = configs.vgg16(batch=16)
     net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
@@ -123,13 +137,36 @@ def main():
     value = 16.0 / (ms * 1e-3)
     achieved = conv_flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4), "traffic": None,
+                "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4), "traffic": CONV_HBM_BYTES_PER_LAUNCH,
                 "kernel": "conv_mfma_kernel<fp32> (implicit-GEMM convolution, all 13 conv + 3 batched FC launches per step)",
                 "launches_per_step": conv_n / args.steps, "avg_launch_ms": round(conv_ms / max(conv_n, 1), 5),
                 "flops_per_launch": conv_flops / max(conv_n, 1)}
     extra = {"vgg16_conv_ms_per_step": round(conv_ms / args.steps, 4),
+             "vgg16_batched_fc_ms_per_step": round(fam[1][0] / args.steps, 4),
              "vgg16_other_kernels_ms_per_step": round(fam[3][0] / args.steps, 4)}
+    # the same step through the drop-in call: host normalisation + H2D + kernels + D2H
+    net.process_float(cfg["input"])
+    t0 = time.perf_counter()
+    for _ in range(5):
+        net.process_float(cfg["input"])
+    extra["vgg16_THProcessFloat_images_per_sec_pcie_inclusive"] = round(16 * 5 / (time.perf_counter() - t0), 1)
     net.free()
+
+    # ---- AlexNet-OWT fp32 batch 1 (GEMV-bound Linear layers) ----
+    c2 = configs.alexnet_owt()
+    n2 = api.HipNetwork(c2["layers"], c2["mean"], c2["std"])
+    x2 = c2["input"].copy()
+    for c in range(3):
+        x2[:, c] = (x2[:, c] - np.float32(c2["mean"][c])) / np.float32(c2["std"][c])
+    n2.upload(x2)
+    ms2, fam2 = timed_forward(lib, n2, max(args.steps, 20), args.warmup, (0, 1, 3))
+    gv_ms, gv_n, gv_bytes = fam2[1]
+    extra["alexnet_owt_fp32_b1"] = {
+        "images_per_sec": round(1e3 / ms2, 1), "ms_per_step": round(ms2, 4),
+        "gemv_GB/s": round(gv_bytes / (gv_ms * 1e-3) / 1e9, 1) if gv_ms > 0 else None,
+        "gemv_frac_of_hbm_peak": round(gv_bytes / (gv_ms * 1e-3) / 8e12, 4) if gv_ms > 0 else None,
+        "workload": "AlexNet-OWT fp32 batch 1 (BASELINE configs[1])"}
+    n2.free()
 
     # ---- uint8 AlexNet-OWT batch 64 ----
     if not args.no_int8:

@@ -149,3 +149,59 @@ def test_engine_small_network_bit_exact_every_layer(hiplib, oracle):
     # loses its quantisation parameters after the first)
     assert np.array_equal(net.process_float(x), y)
     net.free()
+
+
+def _device_codes(hiplib, net, q):
+    """uint8 codes -> a device tensor struct the engine accepts (test-side construction:
+    storage marked as engine-owned device memory, extra reference so it is never freed
+    by the library)."""
+    from thnets_amd import abi
+    dev = api.DeviceArray(hiplib, np.ascontiguousarray(q, np.uint8))
+    st = abi.THFloatStorage(dev.ptr, 2, 4)
+    t = abi.ABI.THFloatTensor()
+    t.nDimension = q.ndim
+    stride = 1
+    for i in range(q.ndim - 1, -1, -1):
+        t.size[i] = q.shape[i]
+        t.stride[i] = stride
+        stride *= q.shape[i]
+    t.storage = C.pointer(st)
+    return t, (dev, st)
+
+
+def test_alexnet_lowp_full_size_bit_exact_and_batch_property(hiplib, oracle):
+    """Configuration 5 at its real layer shapes.  Two images go through the CPU oracle
+    layer by layer (every code must match); then a batch of 64 must equal the same
+    images run in small batches with the batch's quantisation (the reference itself
+    can only run batch 1)."""
+    cfg = configs.alexnet_lowp(batch=64)
+    x = oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])
+    net = api.HipNetwork(cfg["layers"], lowp_range=cfg["range"])
+    xq, im, isub = oracle.lowp_quantize(x)              # one min/max over the whole batch
+    G.note("alexnet lowp b64 forward")
+    t, keep = _device_codes(hiplib, net, xq)
+    assert hiplib.THHipNetwork_setInputQuant(net.handle, im, isub) == 0
+    hiplib.THForward(net.handle, C.addressof(t))
+    last = net.nelem - 1
+    full = net.module_output(last).astype(np.uint8)
+    assert full.shape == (64, 1000, 1, 1)
+    # oracle on images 3 and 40
+    sel = [3, 40]
+    outs = []
+    q, m, s = oracle.lowp_run_layers(cfg["layers"], xq[sel], im, isub, cfg["range"], collect=outs)
+    assert np.array_equal(full[sel], q)
+    G.note("alexnet lowp b2 forward")
+    t2, keep2 = _device_codes(hiplib, net, xq[sel])
+    hiplib.THHipNetwork_setInputQuant(net.handle, im, isub)
+    hiplib.THForward(net.handle, C.addressof(t2))
+    layers = cfg["layers"]
+    for i, (qo, mo, so) in enumerate(outs):
+        want = qo
+        if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold":
+            want = outs[i + 1][0]
+        got = net.module_output(i).astype(np.uint8)
+        assert np.array_equal(got, want), "module %d (%s): %d codes differ" % (i, layers[i]["type"], (got != want).sum())
+        assert net.module_quant(i) == (np.float32(mo), np.float32(so))
+    # the logits carry information (not saturated everywhere)
+    assert len(np.unique(q)) > 20
+    net.free()
