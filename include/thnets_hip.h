@@ -439,6 +439,21 @@ void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *add
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
 	int act, int thr, int val);
 
+/* The same arithmetic as thhip_conv2d_u8 for layers with one output position
+ * per image (Linear, or a window covering its whole input): x [B][K] codes,
+ * wrow from thhip_linear_pack_weight_u8 (row-major [nOut][K] host codes ->
+ * device copy re-centred to signed bytes), rowsum from thhip_u8_rowsums,
+ * y [B][nOut].  Replaces the same reference lines; B <= 64, K % 16 == 0.
+ * thhip_linear_batched_u8_set_tuning forces the K split and the 32-row groups
+ * per wavefront (tests, tuning); zeros restore the heuristic. */
+int thhip_linear_batched_u8_supported(int B, int K, int nOut);
+unsigned char *thhip_linear_pack_weight_u8(const unsigned char *w_host, int nOut, int K);
+int *thhip_u8_rowsums(const unsigned char *w_host, int nOut, int K);
+void thhip_linear_batched_u8_set_tuning(int ksplit, int rg);
+void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wrow, const int *rowsum,
+	const int *addend, unsigned char *y, int B, int K, int nOut,
+	int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val);
+
 /* Replaces Lowp_Threshold_updateOutput (lowp_Threshold.c:3-28) on codes. */
 void thhip_threshold_u8(const unsigned char *x, unsigned char *y, long n, int thr, int val, int inplace);
 

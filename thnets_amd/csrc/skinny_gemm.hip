@@ -16,6 +16,7 @@
  * through LDS) and over gridDim.y workgroups (partials in a scratch buffer,
  * summed by a second tiny kernel that also applies bias and Threshold).
  */
+#include <stdlib.h>
 #include "thhip_internal.h"
 
 #define SK_THREADS 256
@@ -154,5 +155,315 @@ extern "C" void thhip_linear_batched(const void *x, const void *wrow, const floa
 		long blocks = (total + 255) / 256;
 		skinny_finish_kernel<THHIP_F32><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(part, bias, y, B, nOut,
 			ksplit, act, thr, val);
+	}
+}
+
+/* ------------------------------------------------------------------ */
+/* uint8 (LOWP) variant                                                */
+/* ------------------------------------------------------------------ */
+
+/*
+ * One output position per image in the uint8 engine (Linear layers, or a
+ * convolution whose window covers its whole input): C[b][o] over K codes.
+ * Both operands are K-contiguous in memory -- weights row-major [nOut][K],
+ * activations [B][K] -- and v_mfma_i32_32x32x32_i8 wants 16 consecutive k per
+ * lane (lane = row or column lane%32, k half lane/32), so operands go from
+ * global memory to the matrix core through registers only.  A K-step is 128
+ * codes: lane (m, h) reads the 64 contiguous bytes k0 + 64h .. +63 of its row
+ * as four 16-byte loads, and MFMA j contracts the 16-byte pieces j of both
+ * halves; the order of k inside a dot product is free as long as both
+ * operands use the same one.  Weights are stored re-centred (code - 128, done
+ * once at pack time), activations are re-centred on the fly (x ^ 0x80).
+ *
+ * The four wavefronts of a workgroup own the same RG*32 rows and every fourth
+ * K-step of the workgroup's slice; their int32 tiles are summed through LDS
+ * and written as one partial per (K slice, row, batch column).  A finishing
+ * kernel sums the slices, applies the expanded offset terms, gemmlowp's output
+ * stage, the saturating bias add (a plane of one element is all "tail": no
+ * lower clamp, lowp_SpatialConvolution.c:86-87) and the threshold.  Integer
+ * sums are exact, so the split changes nothing in the result.
+ */
+#define SKU_KSTEP 128
+#define SKU_BPAD 64	/* batch columns per partial row */
+
+template <int RG, int NB>	/* RG 32-row groups per wavefront; NB 32-column groups: batch <= 32 * NB */
+__global__ __launch_bounds__(SK_THREADS) void skinny_u8_kernel(const unsigned char *x, const unsigned char *w,
+	int *part, int *cspart, int B, int K, int nOut, int ksplit)
+{
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int m = lane & 31, h = lane >> 5;
+	const int row0 = blockIdx.x * (32 * RG);
+	const int nsteps = (K + SKU_KSTEP - 1) / SKU_KSTEP;
+	const int stride = ksplit * 4;
+	const bool want_cs = blockIdx.x == 0;
+	const unsigned char *wr[RG], *xr[NB];
+#pragma unroll
+	for (int rg = 0; rg < RG; rg++)
+		wr[rg] = w + (size_t)min(row0 + rg * 32 + m, nOut - 1) * K + h * 64;
+#pragma unroll
+	for (int g = 0; g < NB; g++)
+		xr[g] = x + (size_t)min(g * 32 + m, B - 1) * K + h * 64;
+	intx16 acc[RG][NB];
+	int cs[NB];
+#pragma unroll
+	for (int g = 0; g < NB; g++) {
+		cs[g] = 0;
+#pragma unroll
+		for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[rg][g][r] = 0;
+	}
+	const intx4 zero_a = { 0, 0, 0, 0 };
+	const intx4 zero_b = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
+	intx4 a[RG][4], b[NB][4], an[RG][4], bn[NB][4];
+
+	/* K % 16 == 0: a 16-byte piece is all inside the row or all outside */
+#define SKU_LOAD(A_, B_, ST_)                                                                  \
+	do {                                                                                   \
+		const int kk_ = (ST_) * SKU_KSTEP;                                             \
+		_Pragma("unroll") for (int j = 0; j < 4; j++) {                                \
+			const bool ok_ = kk_ + h * 64 + j * 16 < K;                            \
+			_Pragma("unroll") for (int rg = 0; rg < RG; rg++)                      \
+				A_[rg][j] = ok_ ? *(const intx4 *)(wr[rg] + kk_ + j * 16) : zero_a; \
+			_Pragma("unroll") for (int g = 0; g < NB; g++)                         \
+				B_[g][j] = ok_ ? *(const intx4 *)(xr[g] + kk_ + j * 16) : zero_b;  \
+		}                                                                              \
+	} while (0)
+
+	int st = blockIdx.y * 4 + wave;
+	if (st < nsteps)
+		SKU_LOAD(a, b, st);
+	for (; st < nsteps; st += stride) {
+		const int sn = st + stride;
+		if (sn < nsteps)
+			SKU_LOAD(an, bn, sn);
+#pragma unroll
+		for (int j = 0; j < 4; j++) {
+#pragma unroll
+			for (int g = 0; g < NB; g++) {
+#pragma unroll
+				for (int d = 0; d < 4; d++)
+					b[g][j][d] ^= (int)0x80808080;
+				if (want_cs) {
+#pragma unroll
+					for (int d = 0; d < 4; d++)
+						cs[g] = __builtin_amdgcn_sdot4(b[g][j][d], 0x01010101, cs[g], false);
+				}
+#pragma unroll
+				for (int rg = 0; rg < RG; rg++)
+					acc[rg][g] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[rg][j], b[g][j], acc[rg][g], 0, 0, 0);
+			}
+		}
+		if (sn < nsteps) {
+#pragma unroll
+			for (int j = 0; j < 4; j++) {
+#pragma unroll
+				for (int rg = 0; rg < RG; rg++)
+					a[rg][j] = an[rg][j];
+#pragma unroll
+				for (int g = 0; g < NB; g++)
+					b[g][j] = bn[g][j];
+			}
+		}
+	}
+#undef SKU_LOAD
+
+	/* D layout: lane holds column n = lane%32, rows 8*(r/4) + 4*(lane/32) + r%4 */
+	__shared__ int red[4][16][65];
+	__shared__ int csred[4][NB][64];
+#pragma unroll
+	for (int rg = 0; rg < RG; rg++)
+#pragma unroll
+		for (int g = 0; g < NB; g++) {
+			if (rg + g)
+				__syncthreads();
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				red[wave][r][lane] = acc[rg][g][r];
+			__syncthreads();
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				const int idx = tid + i * SK_THREADS;
+				const int n = idx & 31, o = idx >> 5;
+				const int r = 4 * (o >> 3) + (o & 3), ln = n + 32 * ((o >> 2) & 1);
+				const int s = (red[0][r][ln] + red[1][r][ln]) + (red[2][r][ln] + red[3][r][ln]);
+				const int bcol = g * 32 + n, orow = row0 + rg * 32 + o;
+				if (orow < nOut && bcol < B)
+					part[((size_t)blockIdx.y * nOut + orow) * SKU_BPAD + bcol] = s;
+			}
+		}
+	if (want_cs) {
+#pragma unroll
+		for (int g = 0; g < NB; g++)
+			csred[wave][g][lane] = cs[g];
+		__syncthreads();
+		if (tid < 32 * NB) {
+			const int g = tid >> 5, n = tid & 31;
+			int s = 0;
+#pragma unroll
+			for (int wv = 0; wv < 4; wv++)
+				s += csred[wv][g][n] + csred[wv][g][n + 32];
+			cspart[blockIdx.y * SKU_BPAD + tid] = s;
+		}
+	}
+}
+
+/* One workgroup per 32 output rows: sums the K slices, requantises and
+ * transposes [row][batch] partials into y [B][nOut] through LDS. */
+__global__ __launch_bounds__(256) void skinny_u8_finish_kernel(const int *part, const int *cspart, const int *rowsum,
+	const int *addend, unsigned char *y, int B, int K, int nOut, int ksplit, int offA, int offB,
+	int c_off, int c_mult, int c_shift, int act, int thr, int val)
+{
+	__shared__ int t[32][65];
+	__shared__ int csum[SKU_BPAD];
+	const int tid = threadIdx.x, o0 = blockIdx.x * 32;
+	if (tid < SKU_BPAD) {
+		int s = 0;
+		for (int p = 0; p < ksplit; p++)
+			s += cspart[p * SKU_BPAD + tid];
+		csum[tid] = s;
+	}
+	{
+		const int b = tid & 63, oo = tid >> 6;
+#pragma unroll
+		for (int i = 0; i < 8; i++) {
+			const int ol = oo + 4 * i, o = o0 + ol;
+			int s = 0;
+			if (o < nOut && b < B)
+				for (int p = 0; p < ksplit; p++)
+					s += part[((size_t)p * nOut + o) * SKU_BPAD + b];
+			t[ol][b] = s;
+		}
+	}
+	__syncthreads();
+	const int ol = tid & 31, o = o0 + ol, bb = tid >> 5;
+	if (o >= nOut)
+		return;
+	const int rs = offB * rowsum[o] + K * offA * offB;
+	const int add = addend ? addend[o] : 0;
+#pragma unroll
+	for (int i = 0; i < 8; i++) {
+		const int b = bb + 8 * i;
+		if (b >= B)
+			break;
+		const int a = t[ol][b] + rs + offA * csum[b];
+		unsigned u = ((unsigned)a + (unsigned)c_off) * (unsigned)c_mult;
+		u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
+		int q = (int)u >> c_shift;
+		q = q < 0 ? 0 : q > 255 ? 255 : q;
+		if (addend) {
+			const int sum = q + add;
+			q = sum > 255 ? 255 : (sum & 255);
+		}
+		if (act)
+			q = q > thr ? q : val;
+		y[(size_t)b * nOut + o] = (unsigned char)q;
+	}
+}
+
+static int *g_u8_scratch;
+static size_t g_u8_scratch_words;
+static int g_u8_ksplit, g_u8_rg;
+
+extern "C" int thhip_linear_batched_u8_supported(int B, int K, int nOut)
+{
+	return B >= 1 && B <= 64 && K % 16 == 0 && K >= 16 && nOut >= 1;
+}
+
+/* Test and tuning hook: force the K split (1..64) and the row groups per
+ * wavefront (1 or 2) of thhip_linear_batched_u8; 0 restores the heuristic. */
+extern "C" void thhip_linear_batched_u8_set_tuning(int ksplit, int rg)
+{
+	if (ksplit < 0 || ksplit > 64 || rg < 0 || rg > 2)
+		THError("thhip_linear_batched_u8_set_tuning(%d, %d): out of range", ksplit, rg);
+	g_u8_ksplit = ksplit;
+	g_u8_rg = rg;
+}
+
+/* Device copy of row-major weight codes [nOut][K], re-centred to signed bytes. */
+extern "C" unsigned char *thhip_linear_pack_weight_u8(const unsigned char *w_host, int nOut, int K)
+{
+	const size_t n = (size_t)nOut * K;
+	unsigned char *h = (unsigned char *)malloc(n);
+	for (size_t i = 0; i < n; i++)
+		h[i] = w_host[i] ^ 0x80;
+	unsigned char *d = (unsigned char *)thhip_malloc(n);
+	thhip_memcpy_h2d(d, h, n);
+	free(h);
+	return d;
+}
+
+/* Row sums of the re-centred weight codes, as a device array (made once per layer). */
+extern "C" int *thhip_u8_rowsums(const unsigned char *w_host, int nOut, int K)
+{
+	int *h = (int *)malloc(sizeof(int) * (size_t)nOut);
+	for (int o = 0; o < nOut; o++) {
+		int s = 0;
+		for (int k = 0; k < K; k++)
+			s += (int)w_host[(size_t)o * K + k] - 128;
+		h[o] = s;
+	}
+	int *d = (int *)thhip_malloc(sizeof(int) * (size_t)nOut);
+	thhip_memcpy_h2d(d, h, sizeof(int) * (size_t)nOut);
+	free(h);
+	return d;
+}
+
+template <int RG, int NB>
+static void skinny_u8_launch(dim3 grid, const unsigned char *x, const unsigned char *wrow, int *part, int *cspart,
+	int B, int K, int nOut, int ksplit)
+{
+	skinny_u8_kernel<RG, NB><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, cspart, B, K, nOut, ksplit);
+}
+
+extern "C" void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wrow, const int *rowsum,
+	const int *addend, unsigned char *y, int B, int K, int nOut,
+	int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val)
+{
+	if (!thhip_linear_batched_u8_supported(B, K, nOut))
+		THError("thhip_linear_batched_u8: unsupported shape B=%d K=%d nOut=%d", B, K, nOut);
+	if (c_shift < 0 || c_shift > 31)
+		THError("thhip_linear_batched_u8: shift %d out of range", c_shift);
+	const int rg = g_u8_rg ? g_u8_rg : nOut >= 2048 ? 2 : 1;
+	const int groups = (nOut + 32 * rg - 1) / (32 * rg);
+	const int nsteps = (K + SKU_KSTEP - 1) / SKU_KSTEP;
+	/* aim at ~1024 wavefronts with at least two K-steps each */
+	int ksplit = (256 + groups - 1) / groups;
+	if (ksplit > nsteps / 8)
+		ksplit = nsteps / 8;
+	if (g_u8_ksplit)
+		ksplit = g_u8_ksplit;
+	if (ksplit < 1)
+		ksplit = 1;
+	if (ksplit > 64)
+		ksplit = 64;
+	const size_t words = (size_t)ksplit * SKU_BPAD * ((size_t)nOut + 1);
+	if (words > g_u8_scratch_words) {
+		if (g_u8_scratch) {
+			hipcheck(hipStreamSynchronize(thhip_stream()));
+			thhip_free(g_u8_scratch);
+		}
+		g_u8_scratch_words = words < (1u << 20) ? (1u << 20) : words;
+		g_u8_scratch = (int *)thhip_malloc(g_u8_scratch_words * sizeof(int));
+	}
+	int *cspart = g_u8_scratch, *part = g_u8_scratch + (size_t)ksplit * SKU_BPAD;
+	{
+		ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * nOut * (double)K * B);
+		dim3 grid(groups, ksplit);
+		if (rg == 1 && B <= 32)
+			skinny_u8_launch<1, 1>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
+		else if (rg == 1)
+			skinny_u8_launch<1, 2>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
+		else if (B <= 32)
+			skinny_u8_launch<2, 1>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
+		else
+			skinny_u8_launch<2, 2>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
+	}
+	{
+		ThhipLaunchScope scope(THHIP_FAM_OTHER, (4.0 * ksplit + 1.0) * B * nOut);
+		skinny_u8_finish_kernel<<<dim3((nOut + 31) / 32), dim3(256), 0, thhip_stream()>>>(part, cspart, rowsum, addend, y,
+			B, K, nOut, ksplit, 128 + a_off, 128 + b_off, c_off, c_mult, c_shift, act, thr, val);
 	}
 }

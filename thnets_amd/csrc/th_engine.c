@@ -463,9 +463,15 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 	}
 	const void *x = thhip_tensor_ptr(in, THHIP_U8);
 	void *y = conv_out(m, THHIP_U8, &s, c->nOutputPlane, oH, oW);
-	thhip_conv2d_u8(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
-		c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
-		hm->fused_act, thr, val);
+	const int K = c->nInputPlane * c->kH * c->kW;
+	if (hm->wrow_u8 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
+	    thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
+		thhip_linear_batched_u8(x, hm->wrow_u8, hm->rowsum_u8, hm->addend, y, s.B, K, c->nOutputPlane,
+			a_off, b_off, offset, mult, shift, hm->fused_act, thr, val);
+	else
+		thhip_conv2d_u8(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
+			hm->fused_act, thr, val);
 	hn->cur_mult = om;
 	hn->cur_sub = osub;
 	return m->output;
@@ -723,6 +729,11 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 			float bm = 0, bsub = 0;
 			unsigned char *wq = quantize_host(THFloatTensor_data(w), (long)Co * K, &hm->wm, &hm->wsub);
 			hm->wpacked = thhip_conv_pack_weight_u8(wq, Co, Ci, kHW);
+			if (K % 16 == 0 && K >= 512) {
+				/* a candidate for the one-position (matrix) path: keep the codes row-major too */
+				hm->wrow_u8 = thhip_linear_pack_weight_u8(wq, Co, K);
+				hm->rowsum_u8 = thhip_u8_rowsums(wq, Co, K);
+			}
 			free(wq);
 			if (!contiguous_host_floats(b, "convolution bias", Co))
 				THError("the uint8 engine needs a bias on every convolution (lowp_SpatialConvolution.c:111-120)");
@@ -882,6 +893,8 @@ void thhip_free_network(struct network *net)
 		thhip_free(hm->wrow);
 		thhip_free(hm->bias);
 		thhip_free(hm->addend);
+		thhip_free(hm->wrow_u8);
+		thhip_free(hm->rowsum_u8);
 		for (int j = 0; j < 4; j++)
 			thhip_free(hm->bn[j]);
 	}

@@ -20,6 +20,8 @@ struct hipmod {
 	long bn_planes;
 	/* uint8 engine */
 	int *addend;		/* per-plane bias addend (device) */
+	unsigned char *wrow_u8;	/* row-major weight codes for one-position layers (device) */
+	int *rowsum_u8;		/* their re-centred row sums (device) */
 	float wm, wsub;		/* weight quantisation */
 	float q_mult, q_sub;	/* quantisation of this module's output */
 };
