@@ -439,6 +439,27 @@ void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *add
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
 	int act, int thr, int val);
 
+/* thhip_conv2d_u8 on tensors whose memory order is chosen per side: 0 = the
+ * reference's [B][C][H][W], 1 = channels-last [B][H][W][C], the order the
+ * uint8 engine keeps between convolutions so that the 16 codes of one MFMA
+ * operand vector are one 16-byte load.  Same arithmetic and the same
+ * reference lines; the tail rule of lowpadd still goes by the position inside
+ * the plane.  Channels-last x needs Ci % 64 == 0, channels-last y Co % 4 == 0. */
+void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
+	int act, int thr, int val, int x_channels_last, int y_channels_last);
+
+/* Lowp_SpatialMaxPooling_updateOutput (lowp_SpatialMaxPooling.c:45-108) on
+ * channels-last codes, C % 4 == 0. */
+void thhip_maxpool_u8_cl(const unsigned char *x, unsigned char *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW);
+
+/* Codes from [B][C][HW] to [B][HW][C] memory order (to_channels_last = 1) or
+ * back (0).  No counterpart in the reference, whose tensors are always
+ * plane-major; used where the engine's internal order meets the API. */
+void thhip_relayout_u8(const unsigned char *x, unsigned char *y, int B, int C, int HW, int to_channels_last);
+
 /* The same arithmetic as thhip_conv2d_u8 for layers with one output position
  * per image (Linear, or a window covering its whole input): x [B][K] codes,
  * wrow from thhip_linear_pack_weight_u8 (row-major [nOut][K] host codes ->

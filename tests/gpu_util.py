@@ -53,7 +53,9 @@ def unary(lib, fn, x, out_shape, dtype, *args):
     return api.from_device_dtype(dy, out_shape, dtype)
 
 
-def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0):
+def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0, x_cl=0, y_cl=0):
+    """xq and the result are [B][C][H][W] arrays; x_cl / y_cl make the device copies
+    channels-last ([B][H][W][C]) and call the layout entry point."""
     xq = np.ascontiguousarray(xq, np.uint8)
     wq = np.ascontiguousarray(wq, np.uint8)
     B, Ci, H, W = xq.shape
@@ -62,13 +64,22 @@ def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0):
     oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
     note("conv2d_u8 x%s w%s d%s pad%s prm%s" % (xq.shape, wq.shape, d, pad, prm))
     wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, Ci, kH * kW)
-    dx = api.DeviceArray(lib, xq)
+    dx = api.DeviceArray(lib, np.ascontiguousarray(xq.transpose(0, 2, 3, 1)) if x_cl else xq)
     da = api.DeviceArray(lib, np.ascontiguousarray(addend, np.int32)) if addend is not None else None
     dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW)
-    lib.thhip_conv2d_u8(dx.ptr, wp, da.ptr if da else None, dy.ptr, B, Ci, H, W, Co, kH, kW, d[0], d[1], pad[0], pad[1],
-                        zero, prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"], prm["c_shift"], act, thr, val)
+    if x_cl or y_cl:
+        lib.thhip_conv2d_u8_layout(dx.ptr, wp, da.ptr if da else None, dy.ptr, B, Ci, H, W, Co, kH, kW, d[0], d[1],
+                                   pad[0], pad[1], zero, prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"],
+                                   prm["c_shift"], act, thr, val, x_cl, y_cl)
+    else:
+        lib.thhip_conv2d_u8(dx.ptr, wp, da.ptr if da else None, dy.ptr, B, Ci, H, W, Co, kH, kW, d[0], d[1], pad[0],
+                            pad[1], zero, prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"], prm["c_shift"], act,
+                            thr, val)
     lib.thhip_sync()
-    y = dy.get((B, Co, oH, oW), np.uint8)
+    if y_cl:
+        y = np.ascontiguousarray(dy.get((B, oH, oW, Co), np.uint8).transpose(0, 3, 1, 2))
+    else:
+        y = dy.get((B, Co, oH, oW), np.uint8)
     lib.thhip_free(wp)
     return y
 

@@ -106,6 +106,75 @@ def test_lowpgemm_drop_in(hiplib, oracle):
         assert np.array_equal(c, oracle.lowp_gemm(a, b, -117, -128, 32513, 1028, 18))
 
 
+# (B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW): shapes for the channels-last memory order
+CL_CASES = [
+    (2, 64, 9, 11, 36, 3, 3, 1, 1, 1, 1),
+    (3, 128, 7, 7, 200, 5, 5, 2, 2, 2, 2),
+    (1, 192, 13, 13, 68, 1, 1, 1, 1, 0, 0),
+    (5, 64, 6, 6, 132, 6, 6, 1, 1, 0, 0),
+    (2, 3, 21, 19, 64, 7, 7, 2, 2, 3, 3),       # plane-major in (generic K order), channels-last out
+    (2, 32, 10, 10, 8, 3, 3, 1, 1, 1, 1),       # plane-major in (tap-major K order needs 64), channels-last out
+]
+
+
+@pytest.mark.parametrize("i", range(len(CL_CASES)))
+def test_conv_u8_channels_last_bit_exact(hiplib, oracle, i):
+    """Every combination of memory orders gives the codes of the plane-major restatement,
+    including the bias add's tail rule (which goes by the position inside the plane),
+    the fused threshold, forced tiles and a K split."""
+    B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW = CL_CASES[i]
+    g = cases.rng(1300 + i)
+    x = g.uniform(-3, 3, (B, Ci, H, W)).astype(np.float32)
+    w = g.standard_normal((Co, Ci, kH, kW), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * kH * kW)))
+    b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.5)
+    d, p = (dH, dW), (pH, pW)
+    rngv = 16.0
+    om, osub = float(np.float32(255) / np.float32(rngv)), -rngv / 2
+    xq, im, isub = oracle.lowp_quantize(x)
+    wq, wm, wsub = oracle.lowp_quantize(w)
+    bq, bm, bsub = oracle.lowp_quantize(b)
+    want = oracle.lowp_conv2d(xq, im, isub, wq, wm, wsub, bq, bm, bsub, om, osub, d, p)
+    prm = oracle.lowp_mm_params(wm, wsub, im, isub, om, osub)
+    zero = int(np.round(np.float32(-isub) * np.float32(im)))
+    addend = np.array([oracle.lowp_bias_addend(int(c), bm, bsub, om) for c in bq], np.int32)
+    thr = oracle.lowp_scale_float(om, osub, 0.0)
+    orders = [(0, 1)] + ([(1, 0), (1, 1)] if Ci % 64 == 0 else [])
+    try:
+        for tune in ((0, 0, 0, 0), (64, 64, 3, 2), (128, 128, 1, 0), (64, 128, 2, 1), (128, 64, 1, 4)):
+            hiplib.thhip_conv_set_tuning(*tune)
+            for (x_cl, y_cl) in orders:
+                got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, x_cl=x_cl, y_cl=y_cl)
+                assert np.array_equal(got, want), (tune, x_cl, y_cl, int((got != want).sum()))
+                got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, act=1, thr=thr, val=thr, x_cl=x_cl, y_cl=y_cl)
+                assert np.array_equal(got, oracle.lowp_threshold(want, thr, thr)), (tune, x_cl, y_cl)
+    finally:
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+
+
+def test_maxpool_and_relayout_channels_last(hiplib, oracle):
+    g = cases.rng(1400)
+    for (B, Cn, H, W, kH, kW, dH, dW, pH, pW, ceil) in ((2, 8, 13, 13, 3, 3, 2, 2, 0, 0, 0), (3, 64, 27, 27, 3, 3, 2, 2, 0, 0, 0),
+                                                       (1, 12, 7, 9, 2, 2, 2, 2, 1, 1, 1), (2, 4, 10, 8, 2, 3, 1, 2, 0, 1, 0)):
+        q = g.integers(0, 256, (B, Cn, H, W), dtype=np.uint8)
+        G.note("relayout/maxpool_u8_cl %s" % ((B, Cn, H, W, kH, kW, dH, dW, pH, pW, ceil),))
+        dq = api.DeviceArray(hiplib, q)
+        dcl = api.DeviceArray(hiplib, nbytes=q.size)
+        hiplib.thhip_relayout_u8(dq.ptr, dcl.ptr, B, Cn, H * W, 1)
+        hiplib.thhip_sync()
+        cl = dcl.get((B, H, W, Cn), np.uint8)
+        assert np.array_equal(cl, q.transpose(0, 2, 3, 1))
+        dback = api.DeviceArray(hiplib, nbytes=q.size)
+        hiplib.thhip_relayout_u8(dcl.ptr, dback.ptr, B, Cn, H * W, 0)
+        hiplib.thhip_sync()
+        assert np.array_equal(dback.get(q.shape, np.uint8), q)
+        want = oracle.lowp_maxpool(q, kH, kW, dH, dW, pH, pW, ceil)
+        oH, oW = want.shape[2:]
+        dy = api.DeviceArray(hiplib, nbytes=want.size)
+        hiplib.thhip_maxpool_u8_cl(dcl.ptr, dy.ptr, B, Cn, H, W, oH, oW, kH, kW, dH, dW, pH, pW)
+        hiplib.thhip_sync()
+        assert np.array_equal(dy.get((B, oH, oW, Cn), np.uint8).transpose(0, 3, 1, 2), want)
+
+
 def _linear_u8(hiplib, xq, wq, addend, prm, act=0, thr=0, val=0):
     B, K = xq.shape
     nOut = wq.shape[0]

@@ -53,6 +53,8 @@ struct ConvParams {
 	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
 	const int *addend;	/* per-plane bias addend, or NULL */
 	int zero, offA, offB, c_off, c_mult, c_shift, ithr, ival;
+	/* host side only: memory order of x and y, 0 = [B][C][H][W], 1 = [B][H][W][C] */
+	int x_cl, y_cl;
 };
 
 /* floor(n / d) = (n * m) >> 32 for n*d < 2^32 with the 33-bit m = floor(2^32/d) + 1,
@@ -145,9 +147,10 @@ __device__ __forceinline__ KTap conv_ktap(const ConvParams &p, int k)
 	return t;
 }
 
-template <int DT, int BM, int BN, int WGM, int WGN, bool TAP>
+template <int DT, int BM, int BN, int WGM, int WGN, bool TAP, bool CLI, bool CLO>
 __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 {
+	static_assert(TAP || !CLI, "channels-last input needs the tap-major K order");
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
 	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC;
@@ -195,7 +198,10 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		int oy = r / p.oW, ox = r - oy * p.oW;
 		iy0 = oy * p.dH - p.padH;
 		ix0 = ox * p.dW - p.padW;
-		xoff = b * p.Ci * p.HW + iy0 * p.W + ix0;
+		if constexpr (CLI)
+			xoff = ((b * p.H + iy0) * p.W + ix0) * p.Ci;
+		else
+			xoff = b * p.Ci * p.HW + iy0 * p.W + ix0;
 	}
 	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
 
@@ -224,13 +230,23 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		if constexpr (TAP) {
 			const int iy = iy0 + t_kh, ix = ix0 + t_kw;
 			tap_ok = n_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-			tap_voff = tap_ok ? (unsigned)(xoff + t_kh * p.W + t_kw) * (unsigned)sizeof(elem) : 0xfffffff0u;
+			if constexpr (CLI)
+				/* (the buffer is shorter than 2^31 bytes: this offset is out of
+				 * range, reads as zero, and adding 16 bytes cannot wrap) */
+				tap_voff = tap_ok ? (unsigned)(xoff + (t_kh * p.W + t_kw) * p.Ci + t_cb * (2 * CHUNK)) *
+					(unsigned)sizeof(elem) : 0x80000000u;
+			else
+				tap_voff = tap_ok ? (unsigned)(xoff + t_kh * p.W + t_kw) * (unsigned)sizeof(elem) : 0xfffffff0u;
 		}
 #pragma unroll
 		for (int j = 0; j < B_PER_THREAD; j++) {
 			const int pidx = slot * B_PER_THREAD + j;
 			elem v[VEC];
-			if constexpr (TAP) {
+			if constexpr (CLI) {
+				/* the VEC planes of this vector are adjacent in memory */
+				const uintx4 ld = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, tap_voff, pidx * 16, 0);
+				__builtin_memcpy(v, &ld, 16);
+			} else if constexpr (TAP) {
 				const int cbase = t_cb * (2 * CHUNK) + (pidx >> 1) * CHUNK + (pidx & 1) * VEC;
 #pragma unroll
 				for (int e = 0; e < VEC; e++) {
@@ -453,22 +469,34 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 			for (int i = 0; i < TM; i++) {
 				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
 #pragma unroll
-				for (int r = 0; r < 16; r++) {
-					const int m = m0 + 8 * (r >> 2) + (r & 3);
-					if (m < p.Co) {
-						const int a = acc[i][j][r] + p.offB * p.rowsum[m] + colterm;
-						int q = conv_requant(a, p.c_off, p.c_mult, p.c_shift);
-						if (p.addend) {
-							/* lowpadd, lowp_SpatialConvolution.c:71-88 */
-							const int sum = q + p.addend[m];
-							if (rem < tail0)
-								q = sum > 255 ? 255 : sum < 0 ? 0 : sum;
+				for (int g = 0; g < 4; g++) {
+					unsigned packed = 0;
+#pragma unroll
+					for (int e = 0; e < 4; e++) {
+						const int r = 4 * g + e, m = m0 + 8 * g + e;
+						if (m < p.Co) {
+							const int a = acc[i][j][r] + p.offB * p.rowsum[m] + colterm;
+							int q = conv_requant(a, p.c_off, p.c_mult, p.c_shift);
+							if (p.addend) {
+								/* lowpadd, lowp_SpatialConvolution.c:71-88 */
+								const int sum = q + p.addend[m];
+								if (rem < tail0)
+									q = sum > 255 ? 255 : sum < 0 ? 0 : sum;
+								else
+									q = sum > 255 ? 255 : (sum & 255);
+							}
+							if (p.act)
+								q = q > p.ithr ? q : p.ival;
+							if constexpr (CLO)
+								packed |= (unsigned)q << (8 * e);
 							else
-								q = sum > 255 ? 255 : (sum & 255);
+								y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
 						}
-						if (p.act)
-							q = q > p.ithr ? q : p.ival;
-						y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
+					}
+					if constexpr (CLO) {
+						/* Co % 4 == 0: the four planes are one aligned word */
+						if (m0 + 8 * g < p.Co)
+							*(unsigned *)(y + (size_t)n * p.Co + m0 + 8 * g) = packed;
 					}
 				}
 			}
@@ -486,13 +514,24 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 			for (int i = 0; i < TM; i++) {
 				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
 #pragma unroll
-				for (int r = 0; r < 16; r++) {
-					const int m = m0 + 8 * (r >> 2) + (r & 3);
-					if (m < p.Co) {
-						float v = acc[i][j][r] + (p.bias ? p.bias[m] : 0.0f);
-						if (p.act)
-							v = v > p.thr ? v : p.val;
-						y[ybase + (size_t)m * p.oHW] = (elem)v;
+				for (int g = 0; g < 4; g++) {
+					struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+#pragma unroll
+					for (int e = 0; e < 4; e++) {
+						const int r = 4 * g + e, m = m0 + 8 * g + e;
+						float v = 0;
+						if (m < p.Co) {
+							v = acc[i][j][r] + (p.bias ? p.bias[m] : 0.0f);
+							if (p.act)
+								v = v > p.thr ? v : p.val;
+							if constexpr (!CLO)
+								y[ybase + (size_t)m * p.oHW] = (elem)v;
+						}
+						quad.v[e] = (elem)v;
+					}
+					if constexpr (CLO) {
+						if (m0 + 8 * g < p.Co)
+							*(Quad *)(y + (size_t)n * p.Co + m0 + 8 * g) = quad;
 					}
 				}
 			}
@@ -633,10 +672,10 @@ static void conv_scratch(ConvParams &p, size_t tiles, size_t tile_words)
  * CU (0 = whatever registers and LDS allow).  The hardware hands left-over
  * workgroups to as few CUs as it can fill, so fewer, faster residents per CU
  * shorten the last, partially filled round of a grid. */
-template <typename K>
-static void conv_launch_kernel(K kernel, ConvParams &p, dim3 grid, int wgs)
+template <void (*kernel)(ConvParams)>
+static void conv_launch_kernel(ConvParams &p, dim3 grid, int wgs)
 {
-	static int static_lds = -1, max_wgs;
+	static int static_lds = -1, max_wgs;	/* per kernel: one instance of this function each */
 	if (static_lds < 0) {
 		hipFuncAttributes attr;
 		hipcheck(hipFuncGetAttributes(&attr, (const void *)kernel));
@@ -667,10 +706,27 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 	if (p.splitk > 1)
 		conv_scratch(p, tiles, (size_t)BM * BN);
 	dim3 grid((unsigned)(tiles * p.splitk));
-	if (conv_tap_major(p.Ci, DT))
-		conv_launch_kernel(conv_mfma_kernel<DT, BM, BN, WGM, WGN, true>, p, grid, wgs);
+	const bool tap = conv_tap_major(p.Ci, DT);
+	if (p.x_cl && !tap)
+		THError("thhip_conv2d: channels-last input needs Ci %% %d == 0 (Ci = %d)", 2 * conv_chunk(DT), p.Ci);
+	if (p.y_cl && p.Co % 4)
+		THError("thhip_conv2d: channels-last output needs Co %% 4 == 0 (Co = %d)", p.Co);
+	if constexpr (DT == THHIP_U8) {
+		/* the uint8 engine keeps its activations channels-last between convolutions */
+		if (p.x_cl && p.y_cl)
+			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, true, true>>(p, grid, wgs);
+		if (p.x_cl)
+			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, true, false>>(p, grid, wgs);
+		if (p.y_cl && tap)
+			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, false, true>>(p, grid, wgs);
+		if (p.y_cl)
+			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, false, true>>(p, grid, wgs);
+	} else if (p.x_cl || p.y_cl)
+		THError("thhip_conv2d: channels-last tensors are a uint8 feature");
+	if (tap)
+		conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, false, false>>(p, grid, wgs);
 	else
-		conv_launch_kernel(conv_mfma_kernel<DT, BM, BN, WGM, WGN, false>, p, grid, wgs);
+		conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, false, false>>(p, grid, wgs);
 }
 
 template <int DT>
@@ -720,7 +776,7 @@ static void conv_dispatch(ConvParams &p)
 
 struct ConvU8Args {
 	const int *addend;
-	int zero, a_off, b_off, c_off, c_mult, c_shift, ithr, ival;
+	int zero, a_off, b_off, c_off, c_mult, c_shift, ithr, ival, x_cl, y_cl;
 };
 
 static void conv_run(const void *x, const void *wpacked, const float *bias, void *y,
@@ -776,6 +832,7 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 			p.offB = 128 + u8->b_off;
 			p.c_off = u8->c_off; p.c_mult = u8->c_mult; p.c_shift = u8->c_shift;
 			p.ithr = u8->ithr; p.ival = u8->ival;
+			p.x_cl = u8->x_cl; p.y_cl = u8->y_cl;
 			ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * Co * (double)K * p.N);
 			conv_dispatch<THHIP_U8>(p);
 		} else {
@@ -823,15 +880,25 @@ extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int C
 	return dev;
 }
 
+extern "C" void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
+	int act, int thr, int val, int x_channels_last, int y_channels_last)
+{
+	if (c_shift < 0 || c_shift > 31)
+		THError("thhip_conv2d_u8: shift %d out of range", c_shift);
+	ConvU8Args u8 = { addend, zero & 255, a_off, b_off, c_off, c_mult, c_shift, thr, val,
+		x_channels_last != 0, y_channels_last != 0 };
+	conv_run(x, wpacked, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
+}
+
 extern "C" void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
 	int act, int thr, int val)
 {
-	if (c_shift < 0 || c_shift > 31)
-		THError("thhip_conv2d_u8: shift %d out of range", c_shift);
-	ConvU8Args u8 = { addend, zero & 255, a_off, b_off, c_off, c_mult, c_shift, thr, val };
-	conv_run(x, wpacked, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
+	thhip_conv2d_u8_layout(x, wpacked, addend, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW,
+		zero, a_off, b_off, c_off, c_mult, c_shift, act, thr, val, 0, 0);
 }
 
 /* The reference's only entry into gemmlowp (lowp/gemm8.cc:4-17): host

@@ -159,6 +159,81 @@ extern "C" void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W
 	}
 }
 
+/* The same pooling on channels-last codes [B][H][W][C], C % 4 == 0: a thread
+ * owns four adjacent planes of one output position and reads them as one word
+ * per window element (lowp_SpatialMaxPooling.c:20-50 per plane). */
+__global__ void maxpool_u8_cl_kernel(const unsigned *x, unsigned *y, PoolParams p)
+{
+	const int C4 = p.C / 4;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < p.total; i += step) {
+		const int c4 = (int)(i % C4);
+		long t = i / C4;
+		const int ox = (int)(t % p.oW);
+		t /= p.oW;
+		const int oy = (int)(t % p.oH);
+		const long b = t / p.oH;
+		int hs = oy * p.dH - p.padH, ws = ox * p.dW - p.padW;
+		const int he = min(hs + p.kH, p.H), we = min(ws + p.kW, p.W);
+		hs = max(hs, 0);
+		ws = max(ws, 0);
+		unsigned m0 = 0, m1 = 0, m2 = 0, m3 = 0;
+		for (int yy = hs; yy < he; yy++)
+			for (int xx = ws; xx < we; xx++) {
+				const unsigned v = x[((b * p.H + yy) * p.W + xx) * C4 + c4];
+				m0 = max(m0, v & 255u);
+				m1 = max(m1, (v >> 8) & 255u);
+				m2 = max(m2, (v >> 16) & 255u);
+				m3 = max(m3, v >> 24);
+			}
+		y[i] = m0 | (m1 << 8) | (m2 << 16) | (m3 << 24);
+	}
+}
+
+extern "C" void thhip_maxpool_u8_cl(const unsigned char *x, unsigned char *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW)
+{
+	if (C % 4)
+		THError("thhip_maxpool_u8_cl: C = %d is not a multiple of 4", C);
+	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * oH * oW * (C / 4) };
+	if (p.total <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)B * C * H * W + 4.0 * p.total);
+	maxpool_u8_cl_kernel<<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>((const unsigned *)x, (unsigned *)y, p);
+}
+
+/* Codes between plane-major [B][C][HW] and channels-last [B][HW][C] memory
+ * order (to_cl = 1: the former to the latter), through a 32 x 32 LDS tile. */
+__global__ void relayout_u8_kernel(const unsigned char *x, unsigned char *y, int C, int HW, int to_cl)
+{
+	__shared__ unsigned char t[32][33];
+	/* source [R][S] -> destination [S][R] per image */
+	const int R = to_cl ? C : HW, S = to_cl ? HW : C;
+	const size_t img = (size_t)blockIdx.z * C * HW;
+	const int r0 = blockIdx.y * 32, s0 = blockIdx.x * 32;
+	const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+	for (int k = ty; k < 32; k += 8)
+		if (r0 + k < R && s0 + tx < S)
+			t[k][tx] = x[img + (size_t)(r0 + k) * S + s0 + tx];
+	__syncthreads();
+	for (int k = ty; k < 32; k += 8)
+		if (s0 + k < S && r0 + tx < R)
+			y[img + (size_t)(s0 + k) * R + r0 + tx] = t[tx][k];
+}
+
+extern "C" void thhip_relayout_u8(const unsigned char *x, unsigned char *y, int B, int C, int HW, int to_channels_last)
+{
+	if (B < 1 || C < 1 || HW < 1)
+		return;
+	if (B > 65535)
+		THError("thhip_relayout_u8: batch %d too large", B);
+	const int R = to_channels_last ? C : HW, S = to_channels_last ? HW : C;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * B * C * HW);
+	relayout_u8_kernel<<<dim3((S + 31) / 32, (R + 31) / 32, B), dim3(256), 0, thhip_stream()>>>(x, y, C, HW,
+		to_channels_last != 0);
+}
+
 /* modules/SpatialAveragePooling.c:156-203 */
 template <int DT>
 __global__ void avgpool_kernel(const void *x, void *y, PoolParams p, int count_include_pad)

@@ -348,7 +348,17 @@ long THHipNetwork_copyModuleOutput(THNETWORK *net, int idx, float **dst, long si
 	if (net->net->modules[idx].type == MT_ConcatTable || !o || !o->storage)
 		THError("THHipNetwork_copyModuleOutput: module %d has no tensor output", idx);
 	thhip_sync();
-	THFloatTensor *h = download_as_float(o, hn->dtype);
+	THFloatTensor *h;
+	const int nd = o->nDimension;
+	if (hn->hm[idx].out_cl && nd >= 3 && o->size[nd - 1] * o->size[nd - 2] > 1) {
+		/* kept channels-last inside the uint8 engine: hand out the reference's order */
+		THFloatTensor *pm = device_tensor_like(o, THHIP_U8);
+		thhip_relayout_u8(thhip_tensor_ptr(o, THHIP_U8), (unsigned char *)pm->storage->data, nd == 4 ? (int)o->size[0] : 1,
+			(int)o->size[nd - 3], (int)(o->size[nd - 1] * o->size[nd - 2]), 0);
+		h = download_as_float(pm, hn->dtype);
+		THFloatTensor_free(pm);
+	} else
+		h = download_as_float(o, hn->dtype);
 	const long n = THFloatTensor_nElement(h);
 	*ndim = h->nDimension;
 	for (int i = 0; i < 4; i++)

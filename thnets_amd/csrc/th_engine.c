@@ -464,14 +464,19 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 	const void *x = thhip_tensor_ptr(in, THHIP_U8);
 	void *y = conv_out(m, THHIP_U8, &s, c->nOutputPlane, oH, oW);
 	const int K = c->nInputPlane * c->kH * c->kW;
+	/* with one position per plane both memory orders coincide */
+	const int x_cl = hn->cur_cl && s.H * s.W > 1;
+	if (x_cl && !hm->in_cl)
+		THError("uint8 engine: channels-last codes reached a convolution that was not planned for them");
 	if (hm->wrow_u8 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
-	    thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
+	    (x_cl == hm->in_cl || s.H * s.W == 1) && thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
 		thhip_linear_batched_u8(x, hm->wrow_u8, hm->rowsum_u8, hm->addend, y, s.B, K, c->nOutputPlane,
 			a_off, b_off, offset, mult, shift, hm->fused_act, thr, val);
 	else
-		thhip_conv2d_u8(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+		thhip_conv2d_u8_layout(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
 			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
-			hm->fused_act, thr, val);
+			hm->fused_act, thr, val, x_cl, hm->out_cl);
+	hn->cur_cl = hm->out_cl;
 	hn->cur_mult = om;
 	hn->cur_sub = osub;
 	return m->output;
@@ -514,7 +519,10 @@ static THFloatTensor *HipLowp_SpatialMaxPooling_updateOutput(struct module *m, T
 		THError("SpatialMaxPooling: input %dx%d smaller than the window", p.H, p.W);
 	const void *x = thhip_tensor_ptr(in, THHIP_U8);
 	void *y = planes_out(m, THHIP_U8, &p, oH, oW);
-	thhip_maxpool(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, THHIP_U8);
+	if (hn->cur_cl)
+		thhip_maxpool_u8_cl(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW);
+	else
+		thhip_maxpool(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, THHIP_U8);
 	hm->q_mult = hn->cur_mult;	/* lowp_SpatialMaxPooling.c:104-105 */
 	hm->q_sub = hn->cur_sub;
 	return m->output;
@@ -526,6 +534,9 @@ static THFloatTensor *HipLowp_SoftMax_updateOutput(struct module *m, THFloatTens
 	struct hipmod *hm = hipmod_of(m);
 	long nframe, dim, stride;
 	softmax_shape(in, &nframe, &dim, &stride);
+	if (hn->cur_cl && stride > 1)
+		THError("uint8 engine: channels-last codes reached SoftMax");
+	hn->cur_cl = 0;
 	const void *x = thhip_tensor_ptr(in, THHIP_U8);
 	void *y = out_resize(m, THHIP_U8, in->nDimension, in->size);
 	hn->cur_mult = thhip_softmax_u8(x, y, nframe, dim, stride, hn->cur_mult, hn->cur_sub);
@@ -539,6 +550,10 @@ static THFloatTensor *HipLowp_View_updateOutput(struct module *m, THFloatTensor 
 {
 	struct hipnet *hn = hipnet_of(m);
 	struct hipmod *hm = hipmod_of(m);
+	if (hn->cur_cl && THFloatTensor_nElement(in) != in->size[0] * (in->nDimension > 1 ? in->size[1] : 1) &&
+	    !(in->nDimension == 3 && in->size[1] * in->size[2] == 1))
+		THError("uint8 engine: channels-last codes reached View");
+	hn->cur_cl = 0;
 	Hip_View_updateOutput(m, in);
 	hm->q_mult = hn->cur_mult;
 	hm->q_sub = hn->cur_sub;
@@ -613,6 +628,7 @@ THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in)
 			"(engine %d given); it carries no CPU path", net->engine);
 	th_convtot = 0;
 	th_convflops = 0;
+	((struct hipnet *)net)->cur_cl = 0;	/* inputs arrive in the reference's plane-major order */
 	THFloatTensor *out = run_network(net, in);
 	if (th_profile)
 		printf("%f seconds for convolutions %f Gflops/s\n", th_convtot, th_convflops * 1e-9 / th_convtot);
@@ -729,12 +745,7 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 			float bm = 0, bsub = 0;
 			unsigned char *wq = quantize_host(THFloatTensor_data(w), (long)Co * K, &hm->wm, &hm->wsub);
 			hm->wpacked = thhip_conv_pack_weight_u8(wq, Co, Ci, kHW);
-			if (K % 16 == 0 && K >= 512) {
-				/* a candidate for the one-position (matrix) path: keep the codes row-major too */
-				hm->wrow_u8 = thhip_linear_pack_weight_u8(wq, Co, K);
-				hm->rowsum_u8 = thhip_u8_rowsums(wq, Co, K);
-			}
-			free(wq);
+			hm->wq_host = wq;	/* plan_channels_last() makes the row-major copy */
 			if (!contiguous_host_floats(b, "convolution bias", Co))
 				THError("the uint8 engine needs a bias on every convolution (lowp_SpatialConvolution.c:111-120)");
 			unsigned char *bq = quantize_host(THFloatTensor_data(b), Co, &bm, &bsub);
@@ -833,6 +844,60 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 	}
 }
 
+/* uint8 engine: decides which tensors live channels-last ([B][H][W][C]) in
+ * memory.  A convolution reads 16 adjacent planes of one pixel per operand
+ * vector, so it takes channels-last input whenever its planes come in whole
+ * blocks of 64 and the producer is another convolution reached only through
+ * modules that work in either order (Threshold, pooling, Dropout, Identity).
+ * Network inputs and every tensor a View or SoftMax sees stay plane-major.
+ * Also makes the row-major weight copies of the one-position (matrix) path,
+ * whose K order follows the input's memory order. */
+static void plan_channels_last(struct hipnet *hn)
+{
+	int prev = -1;
+	for (int i = 0; i < hn->pub.nelem; i++) {
+		struct module *m = &hn->pub.modules[i];
+		struct hipmod *hm = &hn->hm[i];
+		if (is_conv_type(m->type)) {
+			if (prev >= 0 && m->SpatialConvolution.nInputPlane % 64 == 0) {
+				for (int j = prev; j < i; j++)
+					hn->hm[j].out_cl = 1;
+				hm->in_cl = 1;
+			}
+			prev = i;
+		} else if (m->type != MT_Threshold && m->type != MT_SpatialMaxPooling && m->type != MT_Dropout &&
+			m->type != MT_Identity)
+			prev = -1;
+	}
+	for (int i = 0; i < hn->pub.nelem; i++) {
+		struct module *m = &hn->pub.modules[i];
+		struct hipmod *hm = &hn->hm[i];
+		if (!hm->wq_host)
+			continue;
+		const struct SpatialConvolution *c = &m->SpatialConvolution;
+		const int Co = c->nOutputPlane, Ci = c->nInputPlane, kHW = c->kH * c->kW;
+		const long K = (long)Ci * kHW;
+		if (K % 16 == 0 && K >= 512) {
+			unsigned char *rows = hm->wq_host;
+			if (hm->in_cl && kHW > 1) {
+				/* k = (tap, plane) instead of (plane, tap) */
+				rows = malloc((size_t)Co * K);
+				for (int o = 0; o < Co; o++)
+					for (int ci = 0; ci < Ci; ci++)
+						for (int t = 0; t < kHW; t++)
+							rows[(size_t)o * K + (size_t)t * Ci + ci] =
+								hm->wq_host[(size_t)o * K + (size_t)ci * kHW + t];
+			}
+			hm->wrow_u8 = thhip_linear_pack_weight_u8(rows, Co, (int)K);
+			hm->rowsum_u8 = thhip_u8_rowsums(rows, Co, (int)K);
+			if (rows != hm->wq_host)
+				free(rows);
+		}
+		free(hm->wq_host);
+		hm->wq_host = 0;
+	}
+}
+
 static int foldable_threshold(struct module *t)
 {
 	return t->type == MT_Threshold && t->Threshold.alpha == 0;
@@ -866,6 +931,8 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			hn->hm[i + 1].passthrough = 1;
 		}
 	}
+	if (engine == ENGINE_HIPLOWP)
+		plan_channels_last(hn);
 	return &hn->pub;
 }
 

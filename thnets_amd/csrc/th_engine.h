@@ -22,6 +22,8 @@ struct hipmod {
 	int *addend;		/* per-plane bias addend (device) */
 	unsigned char *wrow_u8;	/* row-major weight codes for one-position layers (device) */
 	int *rowsum_u8;		/* their re-centred row sums (device) */
+	unsigned char *wq_host;	/* weight codes on the host, only while the network is being built */
+	int in_cl, out_cl;	/* input / output codes are channels-last [B][H][W][C] in memory */
 	float wm, wsub;		/* weight quantisation */
 	float q_mult, q_sub;	/* quantisation of this module's output */
 };
@@ -33,6 +35,7 @@ struct hipnet {
 	int dtype;		/* enum thhip_dtype of activations */
 	float range;
 	float cur_mult, cur_sub;	/* uint8 engine: quantisation of the tensor in flight */
+	int cur_cl;		/* uint8 engine: the tensor in flight is channels-last in memory */
 };
 
 struct hipnet *hipnet_of(struct module *m);
