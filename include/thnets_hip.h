@@ -425,6 +425,11 @@ void thhip_dequantize(const unsigned char *q, float *x, long n, float mult, floa
 /* Weight packing for the int8 kernel: uint8 codes [Co][Ci][kHW] -> signed
  * (code-128) K-chunked layout + per-row sums.  Returns a device buffer. */
 void *thhip_conv_pack_weight_u8(const unsigned char *w_host, int Co, int Ci, int kHW);
+/* The same for a convolution whose input will be channels-last in memory
+ * (x_channels_last = 1: K runs tap-major, k = tap * Ci + plane; Ci % 16 == 0);
+ * 0 is thhip_conv_pack_weight_u8.  The packed buffer is only valid for calls
+ * with the same x_channels_last. */
+void *thhip_conv_pack_weight_u8_layout(const unsigned char *w_host, int Co, int Ci, int kHW, int x_channels_last);
 
 /* Replaces Lowp_SpatialConvolution_updateOutput's per-image
  * uint8 im2col + THLowpTensor_mm/lowpgemm + lowpadd
@@ -444,7 +449,8 @@ void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *add
  * uint8 engine keeps between convolutions so that the 16 codes of one MFMA
  * operand vector are one 16-byte load.  Same arithmetic and the same
  * reference lines; the tail rule of lowpadd still goes by the position inside
- * the plane.  Channels-last x needs Ci % 64 == 0, channels-last y Co % 4 == 0. */
+ * the plane.  Channels-last x needs Ci % 16 == 0 and weights packed for it,
+ * channels-last y Co % 4 == 0. */
 void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,

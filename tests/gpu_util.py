@@ -63,7 +63,10 @@ def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0, x_cl=
     K = Ci * kH * kW
     oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
     note("conv2d_u8 x%s w%s d%s pad%s prm%s" % (xq.shape, wq.shape, d, pad, prm))
-    wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, Ci, kH * kW)
+    if x_cl:
+        wp = lib.thhip_conv_pack_weight_u8_layout(wq.ctypes.data, Co, Ci, kH * kW, 1)
+    else:
+        wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, Ci, kH * kW)
     dx = api.DeviceArray(lib, np.ascontiguousarray(xq.transpose(0, 2, 3, 1)) if x_cl else xq)
     da = api.DeviceArray(lib, np.ascontiguousarray(addend, np.int32)) if addend is not None else None
     dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW)

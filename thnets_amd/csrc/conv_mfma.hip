@@ -39,8 +39,8 @@ struct ConvParams {
 	void *y;
 	int B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, oH, oW;
 	int K, KC, N, oHW, HW, kHW;
-	unsigned magic_khw, magic_kw;	/* low words of floor(2^32/d)+1 */
-	unsigned mhi_khw, mhi_kw;	/* their bit 32 (set only for d == 1) */
+	unsigned magic_khw, magic_kw, magic_ci;	/* low words of floor(2^32/d)+1 */
+	unsigned mhi_khw, mhi_kw, mhi_ci;	/* their bit 32 (set only for d == 1) */
 	int act;
 	float thr, val;
 	int tiles_m, tiles_n;
@@ -68,22 +68,32 @@ template <int DT> struct ConvTraits;
 template <> struct ConvTraits<THHIP_F32> {
 	static constexpr int CHUNK = 8;		/* k values per chunk */
 	static constexpr int VEC = 4;		/* elements per 16-byte lane vector */
+	static constexpr int KCH = 2;		/* chunks per K-tile (one LDS stage) */
+	static constexpr int PF = 1;		/* K-tiles prefetched into registers */
 	typedef float elem;
 };
 template <> struct ConvTraits<THHIP_F16> {
 	static constexpr int CHUNK = 16;
 	static constexpr int VEC = 8;
+	static constexpr int KCH = 2;
+	static constexpr int PF = 1;
 	typedef _Float16 elem;
 };
 template <> struct ConvTraits<THHIP_BF16> {
 	static constexpr int CHUNK = 16;
 	static constexpr int VEC = 8;
+	static constexpr int KCH = 2;
+	static constexpr int PF = 1;
 	typedef __bf16 elem;
 };
 
 template <> struct ConvTraits<THHIP_U8> {
 	static constexpr int CHUNK = 32;
 	static constexpr int VEC = 16;
+	/* an int8 MFMA retires 32 k in the time an fp32 one retires 1: deeper
+	 * K-tiles keep the work per barrier and per load round-trip up */
+	static constexpr int KCH = 4;
+	static constexpr int PF = 1;
 	typedef unsigned char elem;
 };
 
@@ -150,18 +160,18 @@ __device__ __forceinline__ KTap conv_ktap(const ConvParams &p, int k)
 template <int DT, int BM, int BN, int WGM, int WGN, bool TAP, bool CLI, bool CLO>
 __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 {
-	static_assert(TAP || !CLI, "channels-last input needs the tap-major K order");
+	static_assert(!(TAP && CLI), "tap-major K order is for plane-major input");
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
-	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC;
+	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC, KCH = TR::KCH, PF = TR::PF;
 	constexpr int MB = BM / 32, NB = BN / 32;		/* 32-row blocks per tile */
 	constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32;	/* MFMA tiles per wave */
-	constexpr int A_VECS = MB * 2 * 64;			/* 16-byte vectors per K-tile (2 chunks) */
-	constexpr int B_VECS = NB * 2 * 64;
-	constexpr int A_PER_WAVE = MB * 2 / 4;			/* 1 KiB blocks loaded per wave */
-	constexpr int B_PER_THREAD = BN / 64;			/* (chunk,h) vectors gathered per thread */
+	constexpr int A_VECS = MB * KCH * 64;			/* 16-byte vectors per K-tile (KCH chunks) */
+	constexpr int B_VECS = NB * KCH * 64;
+	constexpr int A_PER_WAVE = MB * KCH / 4;		/* 1 KiB blocks loaded per wave */
+	constexpr int B_PER_THREAD = BN * KCH / 128;		/* (chunk,h) vectors gathered per thread */
 	static_assert(WGM * WGN == 4, "four waves per workgroup");
-	static_assert(MB * 2 % 4 == 0 && BN % 64 == 0, "tile shape");
+	static_assert(MB * KCH % 4 == 0 && BN % 64 == 0, "tile shape");
 
 	__shared__ floatx4 lds[2 * (A_VECS + B_VECS)];
 
@@ -186,68 +196,105 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		tile /= p.splitk;
 	const int tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
 
-	/* ---- B gather role: one output position per thread ---- */
-	const int n_local = tid % BN;
+	/* ---- B gather role ----
+	 * Plane-major input: one output position per thread (lanes run along the
+	 * output row, so element loads coalesce along W); the 256/BN threads of a
+	 * position take different (chunk, half) vectors.
+	 * Channels-last input: the 2*KCH vectors of a position's K-tile slice are
+	 * adjacent in memory (whole runs of Ci bytes per tap), so eight
+	 * neighbouring lanes take the eight vectors of one position and a wave's
+	 * load touches few cache lines; a thread then serves B_PER_THREAD positions. */
+	constexpr int VPP = 2 * KCH;			/* vectors per position per K-tile */
+	constexpr int PPI = CONV_THREADS / VPP;		/* positions per pass (CLI) */
+	constexpr int NPOS = CLI ? B_PER_THREAD : 1;
+	static_assert(!CLI || BN % PPI == 0, "tile shape");
+	const int n_local = CLI ? tid / VPP : tid % BN;
 	const int slot = __builtin_amdgcn_readfirstlane(tid / BN);
-	const int n_glob = tile_n * BN + n_local;
-	const bool n_ok = n_glob < p.N;
-	int iy0, ix0, xoff;
-	{
-		int nn = n_ok ? n_glob : 0;
+	const int pv = tid % VPP;			/* (CLI) this thread's vector */
+	bool n_ok_[NPOS];
+	int iy0_[NPOS], ix0_[NPOS], xoff_[NPOS];
+#pragma unroll
+	for (int q = 0; q < NPOS; q++) {
+		const int n_glob = tile_n * BN + n_local + q * PPI;
+		n_ok_[q] = n_glob < p.N;
+		int nn = n_ok_[q] ? n_glob : 0;
 		int b = nn / p.oHW, r = nn - b * p.oHW;
 		int oy = r / p.oW, ox = r - oy * p.oW;
-		iy0 = oy * p.dH - p.padH;
-		ix0 = ox * p.dW - p.padW;
+		iy0_[q] = oy * p.dH - p.padH;
+		ix0_[q] = ox * p.dW - p.padW;
 		if constexpr (CLI)
-			xoff = ((b * p.H + iy0) * p.W + ix0) * p.Ci;
+			xoff_[q] = ((b * p.H + iy0_[q]) * p.W + ix0_[q]) * p.Ci;
 		else
-			xoff = b * p.Ci * p.HW + iy0 * p.W + ix0;
+			xoff_[q] = b * p.Ci * p.HW + iy0_[q] * p.W + ix0_[q];
 	}
+	const bool n_ok = n_ok_[0];
+	const int iy0 = iy0_[0], ix0 = ix0_[0], xoff = xoff_[0];
 	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
 
 	const floatx4 *wp = (const floatx4 *)p.wp;
-	floatx4 areg[A_PER_WAVE];
-	floatx4 breg[B_PER_THREAD];
-	int colsum = 0;		/* uint8 path: sum of this thread's gathered (code - 128) */
+	/* PF K-tiles are in flight from global memory to registers at any time */
+	floatx4 areg_[PF][A_PER_WAVE];
+	floatx4 breg_[PF][B_PER_THREAD];
+	int colsum[NPOS];	/* uint8 path: sums of this thread's gathered (code - 128) */
+#pragma unroll
+	for (int q = 0; q < NPOS; q++)
+		colsum[q] = 0;
 
-	/* Tap-major K order (TAP): K-tile t covers one filter tap (kh, kw) and
-	 * CB = 2*CHUNK consecutive input planes, tiles ordered plane block outer,
-	 * tap inner.  Bounds test and in-plane offset are then one computation per
-	 * thread per K-tile and every element differs only by a wave-uniform plane
-	 * offset, which rides in the load's scalar offset. */
+	/* Tap-major K order (TAP, plane-major input): K-tile t covers one filter tap
+	 * (kh, kw) and CB = KCH*CHUNK consecutive input planes, tiles ordered plane
+	 * block outer, tap inner.  Bounds test and in-plane offset are then one
+	 * computation per thread per K-tile and every element differs only by a
+	 * wave-uniform plane offset, which rides in the load's scalar offset.
+	 *
+	 * Channels-last input (CLI): k = tap * Ci + plane, so the VEC planes of a
+	 * lane vector are 16 adjacent bytes of one pixel.  Which tap a vector
+	 * belongs to is wave-uniform and decoded on the scalar unit. */
 	int t_cb = 0, t_kh = 0, t_kw = 0;
 	const int plane_bytes = p.HW * (int)sizeof(elem);
 
-	auto load_tile = [&](int kt) {
+	auto load_tile = [&](int kt, floatx4 (&areg)[A_PER_WAVE], floatx4 (&breg)[B_PER_THREAD]) {
 #pragma unroll
 		for (int i = 0; i < A_PER_WAVE; i++) {
 			const int idx = wave + 4 * i;
 			const int mbi = idx % MB, kci = idx / MB;
-			areg[i] = wp[((size_t)(tile_m * MB + mbi) * p.KC + kt * 2 + kci) * 64 + lane];
+			areg[i] = wp[((size_t)(tile_m * MB + mbi) * p.KC + kt * KCH + kci) * 64 + lane];
 		}
 		unsigned tap_voff = 0;
 		bool tap_ok = false;
 		if constexpr (TAP) {
 			const int iy = iy0 + t_kh, ix = ix0 + t_kw;
 			tap_ok = n_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-			if constexpr (CLI)
-				/* (the buffer is shorter than 2^31 bytes: this offset is out of
-				 * range, reads as zero, and adding 16 bytes cannot wrap) */
-				tap_voff = tap_ok ? (unsigned)(xoff + (t_kh * p.W + t_kw) * p.Ci + t_cb * (2 * CHUNK)) *
-					(unsigned)sizeof(elem) : 0x80000000u;
-			else
-				tap_voff = tap_ok ? (unsigned)(xoff + t_kh * p.W + t_kw) * (unsigned)sizeof(elem) : 0xfffffff0u;
+			tap_voff = tap_ok ? (unsigned)(xoff + t_kh * p.W + t_kw) * (unsigned)sizeof(elem) : 0xfffffff0u;
+		}
+		/* (CLI) decode of this thread's vector: the same for all its positions */
+		int cl_kh = 0, cl_kw = 0, cl_off = 0;
+		bool k_ok = true;		/* (CLI) the vector lies inside K */
+		if constexpr (CLI) {
+			const int kv = (kt * VPP + pv) * VEC;
+			const unsigned tap = (unsigned)kv * p.mhi_ci + __umulhi((unsigned)kv, p.magic_ci);
+			const int c = kv - tap * p.Ci;
+			const unsigned kh = tap * p.mhi_kw + __umulhi(tap, p.magic_kw);
+			cl_kh = (int)kh;
+			cl_kw = (int)(tap - kh * p.kW);
+			cl_off = (cl_kh * p.W + cl_kw) * p.Ci + c;
+			k_ok = kv < p.K;
 		}
 #pragma unroll
 		for (int j = 0; j < B_PER_THREAD; j++) {
-			const int pidx = slot * B_PER_THREAD + j;
+			const int pidx = CLI ? pv : slot * B_PER_THREAD + j;
+			const int q = CLI ? j : 0;	/* which of the thread's positions */
 			elem v[VEC];
+			bool vec_ok = tap_ok;		/* (TAP, CLI) the vector lies inside the image */
 			if constexpr (CLI) {
-				/* the VEC planes of this vector are adjacent in memory */
-				const uintx4 ld = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, tap_voff, pidx * 16, 0);
+				const int iy = iy0_[q] + cl_kh, ix = ix0_[q] + cl_kw;
+				vec_ok = n_ok_[q] && k_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+				/* the buffer is shorter than 2^31 bytes: the second offset is
+				 * out of range, reads as zero, and adding 16 cannot wrap */
+				const unsigned voff = vec_ok ? (unsigned)(xoff_[q] + cl_off) * (unsigned)sizeof(elem) : 0x80000000u;
+				const uintx4 ld = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, voff, 0, 0);
 				__builtin_memcpy(v, &ld, 16);
 			} else if constexpr (TAP) {
-				const int cbase = t_cb * (2 * CHUNK) + (pidx >> 1) * CHUNK + (pidx & 1) * VEC;
+				const int cbase = t_cb * (KCH * CHUNK) + (pidx >> 1) * CHUNK + (pidx & 1) * VEC;
 #pragma unroll
 				for (int e = 0; e < VEC; e++) {
 					/* the scalar offset is not range checked: planes exist
@@ -261,7 +308,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 						v[e] = __builtin_bit_cast(elem, __builtin_amdgcn_raw_buffer_load_b16(xrsrc, tap_voff, soff, 0));
 				}
 			} else {
-				const int kbase = (kt * 2 + (pidx >> 1)) * CHUNK + (pidx & 1) * VEC;
+				const int kbase = (kt * KCH + (pidx >> 1)) * CHUNK + (pidx & 1) * VEC;
 #pragma unroll
 				for (int e = 0; e < VEC; e++) {
 					const KTap t = conv_ktap(p, kbase + e);
@@ -287,20 +334,20 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 			if constexpr (DT == THHIP_U8) {
 				/* code - 128 as a signed byte, and this thread's share of the
 				 * column sum of the re-centred codes */
-				intx4 q = __builtin_bit_cast(intx4, packed);
-				if constexpr (TAP) {
+				intx4 cw = __builtin_bit_cast(intx4, packed);
+				if constexpr (TAP || CLI) {
 					/* the whole vector shares one tap: fill it at once */
-					const int fill = (n_ok ? p.zero : 128) * 0x01010101;
+					const int fill = ((n_ok_[q] && k_ok) ? p.zero : 128) * 0x01010101;
 #pragma unroll
 					for (int d = 0; d < 4; d++)
-						q[d] = tap_ok ? q[d] : fill;
+						cw[d] = vec_ok ? cw[d] : fill;
 				}
 #pragma unroll
 				for (int d = 0; d < 4; d++) {
-					q[d] ^= (int)0x80808080;
-					colsum = __builtin_amdgcn_sdot4(q[d], 0x01010101, colsum, false);
+					cw[d] ^= (int)0x80808080;
+					colsum[q] = __builtin_amdgcn_sdot4(cw[d], 0x01010101, colsum[q], false);
 				}
-				packed = __builtin_bit_cast(floatx4, q);
+				packed = __builtin_bit_cast(floatx4, cw);
 			}
 			breg[j] = packed;
 		}
@@ -315,7 +362,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		}
 	};
 
-	auto store_tile = [&](int buf) {
+	auto store_tile = [&](int buf, const floatx4 (&areg)[A_PER_WAVE], const floatx4 (&breg)[B_PER_THREAD]) {
 		floatx4 *la = lds + buf * (A_VECS + B_VECS);
 		floatx4 *lb = la + A_VECS;
 #pragma unroll
@@ -326,9 +373,19 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		}
 #pragma unroll
 		for (int j = 0; j < B_PER_THREAD; j++) {
-			const int pidx = slot * B_PER_THREAD + j;
-			const int kci = pidx >> 1, h = pidx & 1;
-			lb[((kci * NB + (n_local >> 5)) * 2 + h) * 32 + (n_local & 31)] = breg[j];
+			if constexpr (CLI) {
+				/* eight neighbouring lanes write the eight vectors of one
+				 * position, 512 bytes apart: rotate the position inside its
+				 * group of eight by the vector index to spread them over
+				 * the banks (the fragment reads undo it) */
+				const int nl = n_local + j * PPI;
+				const int kci = pv >> 1, h = pv & 1;
+				lb[((kci * NB + (nl >> 5)) * 2 + h) * 32 + ((nl & 31) ^ (pv & 7))] = breg[j];
+			} else {
+				const int pidx = slot * B_PER_THREAD + j;
+				const int kci = pidx >> 1, h = pidx & 1;
+				lb[((kci * NB + (n_local >> 5)) * 2 + h) * 32 + (n_local & 31)] = breg[j];
+			}
 		}
 	};
 
@@ -341,7 +398,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 			for (int r = 0; r < 16; r++)
 				acc[i][j][r] = 0;
 
-	const int nkt_all = p.KC / 2;
+	const int nkt_all = p.KC / KCH;
 	const int kt0 = p.splitk > 1 ? (int)((long)nkt_all * split / p.splitk) : 0;
 	const int nkt = p.splitk > 1 ? (int)((long)nkt_all * (split + 1) / p.splitk) : nkt_all;
 	if constexpr (TAP) {
@@ -350,48 +407,83 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		t_kh = tap / p.kW;
 		t_kw = tap - t_kh * p.kW;
 	}
-	load_tile(kt0);
-	store_tile(kt0 & 1);
+	/* Software pipeline: tiles kt+1 .. kt+PF are in registers or on their way
+	 * while tile kt is multiplied out of LDS; the register sets rotate, so the
+	 * loop is unrolled PF times to keep their indices constant. */
+#pragma unroll
+	for (int s = 0; s < PF; s++)
+		if (kt0 + s < nkt)
+			load_tile(kt0 + s, areg_[s], breg_[s]);
+	store_tile(0, areg_[0], breg_[0]);
 	__syncthreads();
-	for (int kt = kt0; kt < nkt; kt++) {
-		const int cur = kt & 1;
-		if (kt + 1 < nkt)
-			load_tile(kt + 1);
-		const floatx4 *la = lds + cur * (A_VECS + B_VECS);
-		const floatx4 *lb = la + A_VECS;
-		/* both chunks' fragments first, then all MFMAs back to back */
-		floatx4 af[2][TM], bf[2][TN];
+	for (int ktb = kt0; ktb < nkt; ktb += PF) {
 #pragma unroll
-		for (int kci = 0; kci < 2; kci++) {
+		for (int s = 0; s < PF; s++) {
+			const int kt = ktb + s;
+			if (kt >= nkt)
+				break;
+			const int cur = (kt - kt0) & 1;
+			/* set s held tile kt, which is in LDS by now: refill it */
+			if (kt + PF < nkt)
+				load_tile(kt + PF, areg_[s], breg_[s]);
+			const floatx4 *la = lds + cur * (A_VECS + B_VECS);
+			const floatx4 *lb = la + A_VECS;
+			/* two chunks' fragments first, then their MFMAs back to back */
 #pragma unroll
-			for (int i = 0; i < TM; i++)
-				af[kci][i] = la[(kci * MB + wm * TM + i) * 64 + lane];
+			for (int k2 = 0; k2 < KCH; k2 += 2) {
+				floatx4 af[2][TM], bf[2][TN];
 #pragma unroll
-			for (int j = 0; j < TN; j++)
-				bf[kci][j] = lb[(kci * NB + wn * TN + j) * 64 + lane];
+				for (int kci = 0; kci < 2; kci++) {
+#pragma unroll
+					for (int i = 0; i < TM; i++)
+						af[kci][i] = la[((k2 + kci) * MB + wm * TM + i) * 64 + lane];
+#pragma unroll
+					for (int j = 0; j < TN; j++) {
+						const int bl = CLI ? lane ^ ((((k2 + kci) << 1) | (lane >> 5)) & 7) : lane;
+						bf[kci][j] = lb[((k2 + kci) * NB + wn * TN + j) * 64 + bl];
+					}
+				}
+#pragma unroll
+				for (int kci = 0; kci < 2; kci++)
+#pragma unroll
+					for (int i = 0; i < TM; i++)
+#pragma unroll
+						for (int j = 0; j < TN; j++)
+							conv_mma<DT>(acc[i][j], af[kci][i], bf[kci][j]);
+			}
+			if (kt + 1 < nkt)
+				store_tile(cur ^ 1, areg_[(s + 1) % PF], breg_[(s + 1) % PF]);
+			__syncthreads();
 		}
-#pragma unroll
-		for (int kci = 0; kci < 2; kci++)
-#pragma unroll
-			for (int i = 0; i < TM; i++)
-#pragma unroll
-				for (int j = 0; j < TN; j++)
-					conv_mma<DT>(acc[i][j], af[kci][i], bf[kci][j]);
-		if (kt + 1 < nkt)
-			store_tile(cur ^ 1);
-		__syncthreads();
 	}
 
 	/* ---- epilogue ---- */
 	elem *y = (elem *)p.y;
 	__shared__ int cs[DT == THHIP_U8 ? BN : 1];
+	/* Per-row constants go through LDS (the tiles are done with it): loads from
+	 * global memory inside the store loops would each wait out a round trip,
+	 * and registers are what limits how many workgroups share a CU. */
+	int *lrow = (int *)lds;		/* [BM] bias bits, or uint8 row term; [BM..2BM) uint8 addend */
+	if (tid < BM) {
+		const int mc = min(tile_m * BM + tid, p.Co - 1);
+		if constexpr (DT == THHIP_U8) {
+			/* (128+b_off) rowsum + K (128+a_off)(128+b_off) */
+			lrow[tid] = p.offB * p.rowsum[mc] + p.K * p.offA * p.offB;
+			lrow[BM + tid] = p.addend ? p.addend[mc] : 0;
+		} else
+			lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+	}
+	if constexpr (DT != THHIP_U8)
+		__syncthreads();
 	if constexpr (DT == THHIP_U8) {
 		/* Every (chunk, half) share of a column was gathered by one of the
 		 * 256/BN threads that own it: add the shares up in LDS. */
 		if (tid < BN)
 			cs[tid] = 0;
 		__syncthreads();
-		atomicAdd(&cs[n_local], colsum);
+#pragma unroll
+		for (int q = 0; q < NPOS; q++)
+			atomicAdd(&cs[n_local + q * PPI], colsum[q]);
 		__syncthreads();
 	}
 	if (p.splitk > 1) {
@@ -429,33 +521,41 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		__threadfence();
 		if (tid == 0)
 			p.cnt[tile] = 0;	/* ready for the next launch */
-		const int *all = p.ws + (size_t)tile * p.splitk * TILE_WORDS;
+		const int *all = p.ws + (size_t)tile * p.splitk * TILE_WORDS + tid;
 #pragma unroll
 		for (int i = 0; i < TM; i++)
 #pragma unroll
 			for (int j = 0; j < TN; j++)
 #pragma unroll
-				for (int r = 0; r < 16; r++) {
-					const int *src = all + ((i * TN + j) * 16 + r) * CONV_THREADS + tid;
-					if constexpr (DT == THHIP_U8) {
-						int sum = 0;
-						for (int q = 0; q < p.splitk; q++)
-							sum += __hip_atomic_load(src + (size_t)q * TILE_WORDS, __ATOMIC_RELAXED,
-								__HIP_MEMORY_SCOPE_AGENT);
-						acc[i][j][r] = sum;
-					} else {
-						float sum = 0;
-						for (int q = 0; q < p.splitk; q++)
-							sum += __int_as_float(__hip_atomic_load(src + (size_t)q * TILE_WORDS,
-								__ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-						acc[i][j][r] = sum;
+				for (int r = 0; r < 16; r++)
+					acc[i][j][r] = 0;
+		/* one slice at a time, sixteen of its words in flight together */
+		for (int q = 0; q < p.splitk; q++) {
+			const int *src = all + (size_t)q * TILE_WORDS;
+#pragma unroll
+			for (int i = 0; i < TM; i++)
+#pragma unroll
+				for (int j = 0; j < TN; j++) {
+					int part[16];
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						part[r] = __hip_atomic_load(src + ((i * TN + j) * 16 + r) * CONV_THREADS,
+							__ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+					for (int r = 0; r < 16; r++) {
+						if constexpr (DT == THHIP_U8)
+							acc[i][j][r] += part[r];
+						else
+							acc[i][j][r] += __int_as_float(part[r]);
 					}
 				}
+		}
 	}
 	if constexpr (DT == THHIP_U8) {
 		/* sum (w+a_off)(x+b_off) with w = w'+128, x = x'+128:
 		 *   sum w'x' + (128+b_off) rowsum + (128+a_off) colsum + K (128+a_off)(128+b_off) */
 		const int tail0 = (p.oHW / 8) * 8;	/* lowpadd's unclamped tail starts here */
+		const bool has_add = p.addend != 0;
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
 			const int nl = (wn * TN + j) * 32 + (lane & 31);
@@ -464,34 +564,33 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 				continue;
 			const int b = n / p.oHW, rem = n - b * p.oHW;
 			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
-			const int colterm = (p.splitk > 1 ? 0 : p.offA * cs[nl]) + p.K * p.offA * p.offB;
+			const int colterm = p.splitk > 1 ? 0 : p.offA * cs[nl];
+			const bool tail = rem >= tail0;
 #pragma unroll
 			for (int i = 0; i < TM; i++) {
 				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
 #pragma unroll
 				for (int g = 0; g < 4; g++) {
 					unsigned packed = 0;
+					const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
+					const intx4 rowterm = *(const intx4 *)(lrow + ml);
+					const intx4 rowadd = *(const intx4 *)(lrow + BM + ml);
 #pragma unroll
 					for (int e = 0; e < 4; e++) {
 						const int r = 4 * g + e, m = m0 + 8 * g + e;
-						if (m < p.Co) {
-							const int a = acc[i][j][r] + p.offB * p.rowsum[m] + colterm;
-							int q = conv_requant(a, p.c_off, p.c_mult, p.c_shift);
-							if (p.addend) {
-								/* lowpadd, lowp_SpatialConvolution.c:71-88 */
-								const int sum = q + p.addend[m];
-								if (rem < tail0)
-									q = sum > 255 ? 255 : sum < 0 ? 0 : sum;
-								else
-									q = sum > 255 ? 255 : (sum & 255);
-							}
-							if (p.act)
-								q = q > p.ithr ? q : p.ival;
-							if constexpr (CLO)
-								packed |= (unsigned)q << (8 * e);
-							else
-								y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
+						const int a = acc[i][j][r] + rowterm[e] + colterm;
+						int q = conv_requant(a, p.c_off, p.c_mult, p.c_shift);
+						if (has_add) {
+							/* lowpadd, lowp_SpatialConvolution.c:71-88 */
+							const int sum = q + rowadd[e];
+							q = sum > 255 ? 255 : (tail ? (sum & 255) : (sum < 0 ? 0 : sum));
 						}
+						if (p.act)
+							q = q > p.ithr ? q : p.ival;
+						if constexpr (CLO)
+							packed |= (unsigned)q << (8 * e);
+						else if (m < p.Co)
+							y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
 					}
 					if constexpr (CLO) {
 						/* Co % 4 == 0: the four planes are one aligned word */
@@ -502,7 +601,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 			}
 		}
 	} else {
-		/* bias, optional threshold, NCHW store */
+		/* bias, optional threshold, store */
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
 			const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
@@ -516,15 +615,15 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 #pragma unroll
 				for (int g = 0; g < 4; g++) {
 					struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+					const floatx4 rowbias = *(const floatx4 *)(lrow + (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g);
 #pragma unroll
 					for (int e = 0; e < 4; e++) {
 						const int r = 4 * g + e, m = m0 + 8 * g + e;
-						float v = 0;
-						if (m < p.Co) {
-							v = acc[i][j][r] + (p.bias ? p.bias[m] : 0.0f);
-							if (p.act)
-								v = v > p.thr ? v : p.val;
-							if constexpr (!CLO)
+						float v = acc[i][j][r] + rowbias[e];
+						if (p.act)
+							v = v > p.thr ? v : p.val;
+						if constexpr (!CLO) {
+							if (m < p.Co)
 								y[ybase + (size_t)m * p.oHW] = (elem)v;
 						}
 						quad.v[e] = (elem)v;
@@ -547,26 +646,49 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 
 static inline int conv_chunk(int dtype) { return dtype == THHIP_F32 ? 8 : dtype == THHIP_U8 ? 32 : 16; }
 
-/* Tap-major K order needs whole blocks of 2*chunk input planes. */
-static inline bool conv_tap_major(int Ci, int dtype) { return Ci % (2 * conv_chunk(dtype)) == 0; }
+/* Chunks per K-tile: ConvTraits<DT>::KCH. */
+static inline int conv_kch(int dtype) { return dtype == THHIP_U8 ? ConvTraits<THHIP_U8>::KCH : 2; }
 
-/* Number of K chunks (always whole K-tiles of two chunks). */
-static inline int conv_kc(int Ci, int kHW, int dtype)
+/* Order of (plane c, tap) along the packed K axis; follows the input's memory
+ * order, so weights are packed for one of them. */
+enum { KORD_PLANE_TAP, KORD_TAP_MAJOR, KORD_CHANNELS_LAST };
+
+/* Tap-major K order needs whole blocks of KCH*chunk input planes. */
+static inline bool conv_tap_major(int Ci, int dtype) { return Ci % (conv_kch(dtype) * conv_chunk(dtype)) == 0; }
+
+static inline int conv_korder(int Ci, int dtype, int x_cl)
 {
-	const int c = conv_chunk(dtype);
-	if (conv_tap_major(Ci, dtype))
+	if (x_cl) {
+		if (Ci % (conv_chunk(dtype) / 2))
+			THError("thhip_conv2d: channels-last input needs Ci %% %d == 0 (Ci = %d)", conv_chunk(dtype) / 2, Ci);
+		return KORD_CHANNELS_LAST;
+	}
+	return conv_tap_major(Ci, dtype) ? KORD_TAP_MAJOR : KORD_PLANE_TAP;
+}
+
+/* Number of K chunks (always whole K-tiles). */
+static inline int conv_kc(int Ci, int kHW, int dtype, int x_cl)
+{
+	const int c = conv_chunk(dtype), kch = conv_kch(dtype);
+	if (conv_korder(Ci, dtype, x_cl) == KORD_TAP_MAJOR)
 		return Ci / c * kHW;
 	const int kc = (Ci * kHW + c - 1) / c;
-	return (kc + 1) & ~1;
+	return (kc + kch - 1) / kch * kch;
 }
 
 /* Position of weight (plane c, tap) along the packed K axis. */
-static inline long conv_kpos(int c, int tap, int Ci, int kHW, int dtype)
+static inline long conv_kpos(int c, int tap, int Ci, int kHW, int dtype, int x_cl)
 {
-	if (!conv_tap_major(Ci, dtype))
+	switch (conv_korder(Ci, dtype, x_cl)) {
+	case KORD_CHANNELS_LAST:
+		return (long)tap * Ci + c;
+	case KORD_TAP_MAJOR: {
+		const int cb = conv_kch(dtype) * conv_chunk(dtype);
+		return ((long)(c / cb) * kHW + tap) * cb + c % cb;
+	}
+	default:
 		return (long)c * kHW + tap;
-	const int cb = 2 * conv_chunk(dtype);
-	return ((long)(c / cb) * kHW + tap) * cb + c % cb;
+	}
 }
 
 /* Element index of (row m, packed K position kp) in the packed buffer. */
@@ -578,10 +700,15 @@ static inline size_t conv_pack_index(int m, long kp, int KC, int chunk)
 	return ((((size_t)(m >> 5) * KC + kc) * 2 + h) * 32 + (m & 31)) * vec + e;
 }
 
-extern "C" size_t thhip_conv_packed_bytes(int Co, int Ci, int kHW, int dtype)
+static size_t conv_packed_bytes(int Co, int Ci, int kHW, int dtype, int x_cl)
 {
 	size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
-	return mpad / 32 * conv_kc(Ci, kHW, dtype) * 1024;
+	return mpad / 32 * conv_kc(Ci, kHW, dtype, x_cl) * 1024;
+}
+
+extern "C" size_t thhip_conv_packed_bytes(int Co, int Ci, int kHW, int dtype)
+{
+	return conv_packed_bytes(Co, Ci, kHW, dtype, 0);
 }
 
 static inline unsigned short f32_to_f16_bits(float f)
@@ -606,7 +733,7 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 {
 	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
 		THError("thhip_conv_pack_weight: unsupported dtype %d", dtype);
-	const int chunk = conv_chunk(dtype), KC = conv_kc(Ci, kHW, dtype);
+	const int chunk = conv_chunk(dtype), KC = conv_kc(Ci, kHW, dtype, 0);
 	const size_t bytes = thhip_conv_packed_bytes(Co, Ci, kHW, dtype);
 	unsigned char *host = (unsigned char *)calloc(1, bytes);
 	if (!host)
@@ -614,7 +741,7 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 	for (int m = 0; m < Co; m++)
 		for (int c = 0; c < Ci; c++)
 			for (int tap = 0; tap < kHW; tap++) {
-				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, dtype), KC, chunk);
+				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, dtype, 0), KC, chunk);
 				const float v = w[((size_t)m * Ci + c) * kHW + tap];
 				if (dtype == THHIP_F32)
 					((float *)host)[idx] = v;
@@ -698,7 +825,7 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
-	const int nkt = p.KC / 2;
+	const int nkt = p.KC / ConvTraits<DT>::KCH;
 	if (splitk > nkt)
 		splitk = nkt;
 	p.splitk = splitk < 1 ? 1 : splitk;
@@ -707,16 +834,14 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 		conv_scratch(p, tiles, (size_t)BM * BN);
 	dim3 grid((unsigned)(tiles * p.splitk));
 	const bool tap = conv_tap_major(p.Ci, DT);
-	if (p.x_cl && !tap)
-		THError("thhip_conv2d: channels-last input needs Ci %% %d == 0 (Ci = %d)", 2 * conv_chunk(DT), p.Ci);
 	if (p.y_cl && p.Co % 4)
 		THError("thhip_conv2d: channels-last output needs Co %% 4 == 0 (Co = %d)", p.Co);
 	if constexpr (DT == THHIP_U8) {
 		/* the uint8 engine keeps its activations channels-last between convolutions */
 		if (p.x_cl && p.y_cl)
-			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, true, true>>(p, grid, wgs);
+			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, true, true>>(p, grid, wgs);
 		if (p.x_cl)
-			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, true, false>>(p, grid, wgs);
+			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, true, false>>(p, grid, wgs);
 		if (p.y_cl && tap)
 			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, false, true>>(p, grid, wgs);
 		if (p.y_cl)
@@ -813,7 +938,7 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 		p.B = bn; p.Ci = Ci; p.H = H; p.W = W; p.Co = Co; p.kH = kH; p.kW = kW;
 		p.dH = dH; p.dW = dW; p.padH = padH; p.padW = padW; p.oH = oH; p.oW = oW;
 		p.K = (int)K;
-		p.KC = conv_kc(Ci, kH * kW, dtype);
+		p.KC = conv_kc(Ci, kH * kW, dtype, u8 && u8->x_cl);
 		p.N = bn * oH * oW;
 		p.oHW = oH * oW;
 		p.HW = H * W;
@@ -822,10 +947,12 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 		p.mhi_khw = (unsigned)(conv_magic(kH * kW) >> 32);
 		p.magic_kw = (unsigned)conv_magic(kW);
 		p.mhi_kw = (unsigned)(conv_magic(kW) >> 32);
+		p.magic_ci = (unsigned)conv_magic(Ci);
+		p.mhi_ci = (unsigned)(conv_magic(Ci) >> 32);
 		p.act = act; p.thr = thr; p.val = val;
 		p.x_bytes = (unsigned)(bn * in_img * esize);
 		if (u8) {
-			p.rowsum = (const int *)((const char *)wpacked + thhip_conv_packed_bytes(Co, Ci, kH * kW, THHIP_U8));
+			p.rowsum = (const int *)((const char *)wpacked + conv_packed_bytes(Co, Ci, kH * kW, THHIP_U8, u8->x_cl));
 			p.addend = u8->addend;
 			p.zero = u8->zero;
 			p.offA = 128 + u8->a_off;
@@ -853,10 +980,11 @@ extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bi
 
 /* uint8 codes [Co][Ci][kHW] -> (code - 128) as signed bytes in the packed layout,
  * followed by the per-row sums of the re-centred codes. */
-extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int Ci, int kHW)
+extern "C" void *thhip_conv_pack_weight_u8_layout(const unsigned char *w, int Co, int Ci, int kHW, int x_channels_last)
 {
-	const int chunk = 32, KC = conv_kc(Ci, kHW, THHIP_U8);
-	const size_t bytes = thhip_conv_packed_bytes(Co, Ci, kHW, THHIP_U8);
+	const int x_cl = x_channels_last != 0;
+	const int chunk = 32, KC = conv_kc(Ci, kHW, THHIP_U8, x_cl);
+	const size_t bytes = conv_packed_bytes(Co, Ci, kHW, THHIP_U8, x_cl);
 	const size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
 	const size_t total = bytes + mpad * sizeof(int);
 	unsigned char *host = (unsigned char *)calloc(1, total);
@@ -867,7 +995,7 @@ extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int C
 		int sum = 0;
 		for (int c = 0; c < Ci; c++)
 			for (int tap = 0; tap < kHW; tap++) {
-				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, THHIP_U8), KC, chunk);
+				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, THHIP_U8, x_cl), KC, chunk);
 				const int v = (int)w[((size_t)m * Ci + c) * kHW + tap] - 128;
 				host[idx] = (unsigned char)(signed char)v;
 				sum += v;
@@ -878,6 +1006,11 @@ extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int C
 	thhip_memcpy_h2d(dev, host, total);
 	free(host);
 	return dev;
+}
+
+extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int Ci, int kHW)
+{
+	return thhip_conv_pack_weight_u8_layout(w, Co, Ci, kHW, 0);
 }
 
 extern "C" void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
@@ -973,7 +1106,7 @@ __global__ void conv_unpack_rows_kernel(const E *wp, E *rows, int Co, int Ci, in
 
 extern "C" void *thhip_conv_unpack_rows(const void *wpacked, int Co, int Ci, int kHW, int dtype)
 {
-	const int KC = conv_kc(Ci, kHW, dtype), chunk = conv_chunk(dtype), tm = conv_tap_major(Ci, dtype);
+	const int KC = conv_kc(Ci, kHW, dtype, 0), chunk = conv_chunk(dtype), tm = conv_tap_major(Ci, dtype);
 	const long total = (long)Co * Ci * kHW;
 	void *rows = thhip_malloc((size_t)total * thhip_esize(dtype));
 	long blocks = (total + 255) / 256;

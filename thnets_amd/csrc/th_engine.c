@@ -464,12 +464,14 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 	const void *x = thhip_tensor_ptr(in, THHIP_U8);
 	void *y = conv_out(m, THHIP_U8, &s, c->nOutputPlane, oH, oW);
 	const int K = c->nInputPlane * c->kH * c->kW;
-	/* with one position per plane both memory orders coincide */
-	const int x_cl = hn->cur_cl && s.H * s.W > 1;
-	if (x_cl && !hm->in_cl)
-		THError("uint8 engine: channels-last codes reached a convolution that was not planned for them");
+	/* the weights were packed for the planned memory order of the input; with
+	 * one pixel per plane both orders coincide */
+	if (s.H * s.W > 1 && hn->cur_cl != hm->in_cl)
+		THError("uint8 engine: a convolution planned for %s input got the other memory order",
+			hm->in_cl ? "channels-last" : "plane-major");
+	const int x_cl = hm->in_cl;
 	if (hm->wrow_u8 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
-	    (x_cl == hm->in_cl || s.H * s.W == 1) && thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
+	    thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
 		thhip_linear_batched_u8(x, hm->wrow_u8, hm->rowsum_u8, hm->addend, y, s.B, K, c->nOutputPlane,
 			a_off, b_off, offset, mult, shift, hm->fused_act, thr, val);
 	else
@@ -744,8 +746,7 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 		if (lowp) {
 			float bm = 0, bsub = 0;
 			unsigned char *wq = quantize_host(THFloatTensor_data(w), (long)Co * K, &hm->wm, &hm->wsub);
-			hm->wpacked = thhip_conv_pack_weight_u8(wq, Co, Ci, kHW);
-			hm->wq_host = wq;	/* plan_channels_last() makes the row-major copy */
+			hm->wq_host = wq;	/* plan_channels_last() packs them once the input's order is known */
 			if (!contiguous_host_floats(b, "convolution bias", Co))
 				THError("the uint8 engine needs a bias on every convolution (lowp_SpatialConvolution.c:111-120)");
 			unsigned char *bq = quantize_host(THFloatTensor_data(b), Co, &bm, &bsub);
@@ -847,7 +848,7 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 /* uint8 engine: decides which tensors live channels-last ([B][H][W][C]) in
  * memory.  A convolution reads 16 adjacent planes of one pixel per operand
  * vector, so it takes channels-last input whenever its planes come in whole
- * blocks of 64 and the producer is another convolution reached only through
+ * blocks of 16 and the producer is another convolution reached only through
  * modules that work in either order (Threshold, pooling, Dropout, Identity).
  * Network inputs and every tensor a View or SoftMax sees stay plane-major.
  * Also makes the row-major weight copies of the one-position (matrix) path,
@@ -859,7 +860,7 @@ static void plan_channels_last(struct hipnet *hn)
 		struct module *m = &hn->pub.modules[i];
 		struct hipmod *hm = &hn->hm[i];
 		if (is_conv_type(m->type)) {
-			if (prev >= 0 && m->SpatialConvolution.nInputPlane % 64 == 0) {
+			if (prev >= 0 && m->SpatialConvolution.nInputPlane % 16 == 0) {
 				for (int j = prev; j < i; j++)
 					hn->hm[j].out_cl = 1;
 				hm->in_cl = 1;
@@ -877,6 +878,7 @@ static void plan_channels_last(struct hipnet *hn)
 		const struct SpatialConvolution *c = &m->SpatialConvolution;
 		const int Co = c->nOutputPlane, Ci = c->nInputPlane, kHW = c->kH * c->kW;
 		const long K = (long)Ci * kHW;
+		hm->wpacked = thhip_conv_pack_weight_u8_layout(hm->wq_host, Co, Ci, kHW, hm->in_cl);
 		if (K % 16 == 0 && K >= 512) {
 			unsigned char *rows = hm->wq_host;
 			if (hm->in_cl && kHW > 1) {
