@@ -27,6 +27,7 @@
  */
 #include <stdlib.h>
 #include <string.h>
+#include <type_traits>
 #include <vector>
 #include "thhip_internal.h"
 
@@ -64,36 +65,32 @@ static inline unsigned long long conv_magic(unsigned d)
 	return (1ull << 32) / d + 1;
 }
 
+/* Chunks per K-tile (one LDS stage).  An int8 MFMA retires 32 k in the time
+ * an fp32 one retires 1, so where the gather is cheap (channels-last codes)
+ * deeper K-tiles keep the work per barrier up. */
+#define CONV_KCH_U8_CL 4
+__host__ __device__ constexpr int conv_kch(int dtype, bool x_cl) { return dtype == THHIP_U8 && x_cl ? CONV_KCH_U8_CL : 2; }
+
 template <int DT> struct ConvTraits;
 template <> struct ConvTraits<THHIP_F32> {
 	static constexpr int CHUNK = 8;		/* k values per chunk */
 	static constexpr int VEC = 4;		/* elements per 16-byte lane vector */
-	static constexpr int KCH = 2;		/* chunks per K-tile (one LDS stage) */
-	static constexpr int PF = 1;		/* K-tiles prefetched into registers */
 	typedef float elem;
 };
 template <> struct ConvTraits<THHIP_F16> {
 	static constexpr int CHUNK = 16;
 	static constexpr int VEC = 8;
-	static constexpr int KCH = 2;
-	static constexpr int PF = 1;
 	typedef _Float16 elem;
 };
 template <> struct ConvTraits<THHIP_BF16> {
 	static constexpr int CHUNK = 16;
 	static constexpr int VEC = 8;
-	static constexpr int KCH = 2;
-	static constexpr int PF = 1;
 	typedef __bf16 elem;
 };
 
 template <> struct ConvTraits<THHIP_U8> {
 	static constexpr int CHUNK = 32;
 	static constexpr int VEC = 16;
-	/* an int8 MFMA retires 32 k in the time an fp32 one retires 1: deeper
-	 * K-tiles keep the work per barrier and per load round-trip up */
-	static constexpr int KCH = 4;
-	static constexpr int PF = 1;
 	typedef unsigned char elem;
 };
 
@@ -158,12 +155,16 @@ __device__ __forceinline__ KTap conv_ktap(const ConvParams &p, int k)
 }
 
 template <int DT, int BM, int BN, int WGM, int WGN, bool TAP, bool CLI, bool CLO>
-__global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
+__global__ __launch_bounds__(CONV_THREADS)
+/* ask for four waves per SIMD where the tile allows it: without the hint the
+ * compiler spreads the accumulators over AGPRs plus a generous VGPR budget and
+ * halves the number of workgroups a CU can hold */
+__attribute__((amdgpu_waves_per_eu((TAP || CLI) ? 4 : 1, 8))) void conv_mfma_kernel(ConvParams p)
 {
 	static_assert(!(TAP && CLI), "tap-major K order is for plane-major input");
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
-	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC, KCH = TR::KCH, PF = TR::PF;
+	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC, KCH = conv_kch(DT, CLI);
 	constexpr int MB = BM / 32, NB = BN / 32;		/* 32-row blocks per tile */
 	constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32;	/* MFMA tiles per wave */
 	constexpr int A_VECS = MB * KCH * 64;			/* 16-byte vectors per K-tile (KCH chunks) */
@@ -173,7 +174,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 	static_assert(WGM * WGN == 4, "four waves per workgroup");
 	static_assert(MB * KCH % 4 == 0 && BN % 64 == 0, "tile shape");
 
-	__shared__ floatx4 lds[2 * (A_VECS + B_VECS)];
+	constexpr int STAGE_VECS = A_VECS + B_VECS;
+	__shared__ floatx4 lds[3 * STAGE_VECS];		/* three K-tile stages */
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -232,9 +234,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
 
 	const floatx4 *wp = (const floatx4 *)p.wp;
-	/* PF K-tiles are in flight from global memory to registers at any time */
-	floatx4 areg_[PF][A_PER_WAVE];
-	floatx4 breg_[PF][B_PER_THREAD];
+	floatx4 areg[A_PER_WAVE];		/* one K-tile on its way from global memory to LDS */
+	floatx4 breg[B_PER_THREAD];
 	int colsum[NPOS];	/* uint8 path: sums of this thread's gathered (code - 128) */
 #pragma unroll
 	for (int q = 0; q < NPOS; q++)
@@ -252,7 +253,7 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 	int t_cb = 0, t_kh = 0, t_kw = 0;
 	const int plane_bytes = p.HW * (int)sizeof(elem);
 
-	auto load_tile = [&](int kt, floatx4 (&areg)[A_PER_WAVE], floatx4 (&breg)[B_PER_THREAD]) {
+	auto load_tile = [&](int kt) {
 #pragma unroll
 		for (int i = 0; i < A_PER_WAVE; i++) {
 			const int idx = wave + 4 * i;
@@ -362,8 +363,8 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		}
 	};
 
-	auto store_tile = [&](int buf, const floatx4 (&areg)[A_PER_WAVE], const floatx4 (&breg)[B_PER_THREAD]) {
-		floatx4 *la = lds + buf * (A_VECS + B_VECS);
+	auto store_tile = [&](int stage) {
+		floatx4 *la = lds + stage * STAGE_VECS;
 		floatx4 *lb = la + A_VECS;
 #pragma unroll
 		for (int i = 0; i < A_PER_WAVE; i++) {
@@ -374,13 +375,13 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 #pragma unroll
 		for (int j = 0; j < B_PER_THREAD; j++) {
 			if constexpr (CLI) {
-				/* eight neighbouring lanes write the eight vectors of one
-				 * position, 512 bytes apart: rotate the position inside its
-				 * group of eight by the vector index to spread them over
-				 * the banks (the fragment reads undo it) */
+				/* neighbouring lanes write the VPP vectors of one position,
+				 * 512 bytes apart: move the position inside its group of
+				 * eight by the vector index to spread them over the banks
+				 * (the fragment reads undo it) */
 				const int nl = n_local + j * PPI;
 				const int kci = pv >> 1, h = pv & 1;
-				lb[((kci * NB + (nl >> 5)) * 2 + h) * 32 + ((nl & 31) ^ (pv & 7))] = breg[j];
+				lb[((kci * NB + (nl >> 5)) * 2 + h) * 32 + ((nl & 31) ^ ((pv * (8 / VPP)) & 7))] = breg[j];
 			} else {
 				const int pidx = slot * B_PER_THREAD + j;
 				const int kci = pidx >> 1, h = pidx & 1;
@@ -407,53 +408,75 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 		t_kh = tap / p.kW;
 		t_kw = tap - t_kh * p.kW;
 	}
-	/* Software pipeline: tiles kt+1 .. kt+PF are in registers or on their way
-	 * while tile kt is multiplied out of LDS; the register sets rotate, so the
-	 * loop is unrolled PF times to keep their indices constant. */
+	/* Software pipeline over three LDS stages.  While tile kt is multiplied,
+	 * tile kt+1 is already complete in LDS and tile kt+2 travels global memory
+	 * -> registers -> LDS, so fragments are read one chunk ahead of their
+	 * MFMAs, across the tile boundary too, and a wave's matrix core never
+	 * waits on LDS latency; one barrier per K-tile. */
+	floatx4 af[2][TM], bf[2][TN];
+	auto read_frags = [&](int stage, int kci, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
+		const floatx4 *la = lds + stage * STAGE_VECS;
+		const floatx4 *lb = la + A_VECS;
+		const int bl = CLI ? lane ^ ((((kci << 1) | (lane >> 5)) * (8 / VPP)) & 7) : lane;
 #pragma unroll
-	for (int s = 0; s < PF; s++)
-		if (kt0 + s < nkt)
-			load_tile(kt0 + s, areg_[s], breg_[s]);
-	store_tile(0, areg_[0], breg_[0]);
+		for (int i = 0; i < TM; i++)
+			a[i] = la[(kci * MB + wm * TM + i) * 64 + lane];
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+			b[j] = lb[(kci * NB + wn * TN + j) * 64 + bl];
+	};
+	load_tile(kt0);
+	store_tile(0);
+	if (kt0 + 1 < nkt) {
+		load_tile(kt0 + 1);
+		store_tile(1);
+	}
 	__syncthreads();
-	for (int ktb = kt0; ktb < nkt; ktb += PF) {
+	read_frags(0, 0, af[0], bf[0]);
+	static_assert(KCH % 2 == 0, "fragment sets alternate by chunk parity");
+	/* tile kt is in stage st, tile kt+1 in st1, and tile kt+2 goes to st2 */
+	auto step = [&](int kt, auto st, auto st1, auto st2) {
+		if (kt + 2 < nkt)
+			load_tile(kt + 2);
 #pragma unroll
-		for (int s = 0; s < PF; s++) {
-			const int kt = ktb + s;
-			if (kt >= nkt)
-				break;
-			const int cur = (kt - kt0) & 1;
-			/* set s held tile kt, which is in LDS by now: refill it */
-			if (kt + PF < nkt)
-				load_tile(kt + PF, areg_[s], breg_[s]);
-			const floatx4 *la = lds + cur * (A_VECS + B_VECS);
-			const floatx4 *lb = la + A_VECS;
-			/* two chunks' fragments first, then their MFMAs back to back */
+		for (int c = 0; c < KCH; c++) {
+			if (c + 1 < KCH)
+				read_frags(st, c + 1, af[(c + 1) & 1], bf[(c + 1) & 1]);
+			else if (kt + 1 < nkt)
+				read_frags(st1, 0, af[0], bf[0]);
 #pragma unroll
-			for (int k2 = 0; k2 < KCH; k2 += 2) {
-				floatx4 af[2][TM], bf[2][TN];
+			for (int i = 0; i < TM; i++)
 #pragma unroll
-				for (int kci = 0; kci < 2; kci++) {
-#pragma unroll
-					for (int i = 0; i < TM; i++)
-						af[kci][i] = la[((k2 + kci) * MB + wm * TM + i) * 64 + lane];
-#pragma unroll
-					for (int j = 0; j < TN; j++) {
-						const int bl = CLI ? lane ^ ((((k2 + kci) << 1) | (lane >> 5)) & 7) : lane;
-						bf[kci][j] = lb[((k2 + kci) * NB + wn * TN + j) * 64 + bl];
-					}
-				}
-#pragma unroll
-				for (int kci = 0; kci < 2; kci++)
-#pragma unroll
-					for (int i = 0; i < TM; i++)
-#pragma unroll
-						for (int j = 0; j < TN; j++)
-							conv_mma<DT>(acc[i][j], af[kci][i], bf[kci][j]);
-			}
+				for (int j = 0; j < TN; j++)
+					conv_mma<DT>(acc[i][j], af[c & 1][i], bf[c & 1][j]);
+		}
+		if (kt + 2 < nkt)
+			store_tile(st2);
+		__syncthreads();
+	};
+	if constexpr (TAP || CLI) {
+		/* small gather code: unroll three times so every stage is a constant */
+		typedef std::integral_constant<int, 0> S0;
+		typedef std::integral_constant<int, 1> S1;
+		typedef std::integral_constant<int, 2> S2;
+		int kt = kt0;
+		for (; kt + 2 < nkt; kt += 3) {
+			step(kt, S0{}, S1{}, S2{});
+			step(kt + 1, S1{}, S2{}, S0{});
+			step(kt + 2, S2{}, S0{}, S1{});
+		}
+		if (kt < nkt) {
+			step(kt, S0{}, S1{}, S2{});
 			if (kt + 1 < nkt)
-				store_tile(cur ^ 1, areg_[(s + 1) % PF], breg_[(s + 1) % PF]);
-			__syncthreads();
+				step(kt + 1, S1{}, S2{}, S0{});
+		}
+	} else {
+		/* the element-wise gather is long: one copy, stages rotate at run time */
+		int st = 0;
+		for (int kt = kt0; kt < nkt; kt++) {
+			const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
+			step(kt, st, st1, st2);
+			st = st1;
 		}
 	}
 
@@ -646,15 +669,12 @@ __global__ __launch_bounds__(CONV_THREADS) void conv_mfma_kernel(ConvParams p)
 
 static inline int conv_chunk(int dtype) { return dtype == THHIP_F32 ? 8 : dtype == THHIP_U8 ? 32 : 16; }
 
-/* Chunks per K-tile: ConvTraits<DT>::KCH. */
-static inline int conv_kch(int dtype) { return dtype == THHIP_U8 ? ConvTraits<THHIP_U8>::KCH : 2; }
-
 /* Order of (plane c, tap) along the packed K axis; follows the input's memory
  * order, so weights are packed for one of them. */
 enum { KORD_PLANE_TAP, KORD_TAP_MAJOR, KORD_CHANNELS_LAST };
 
 /* Tap-major K order needs whole blocks of KCH*chunk input planes. */
-static inline bool conv_tap_major(int Ci, int dtype) { return Ci % (conv_kch(dtype) * conv_chunk(dtype)) == 0; }
+static inline bool conv_tap_major(int Ci, int dtype) { return Ci % (conv_kch(dtype, false) * conv_chunk(dtype)) == 0; }
 
 static inline int conv_korder(int Ci, int dtype, int x_cl)
 {
@@ -669,7 +689,7 @@ static inline int conv_korder(int Ci, int dtype, int x_cl)
 /* Number of K chunks (always whole K-tiles). */
 static inline int conv_kc(int Ci, int kHW, int dtype, int x_cl)
 {
-	const int c = conv_chunk(dtype), kch = conv_kch(dtype);
+	const int c = conv_chunk(dtype), kch = conv_kch(dtype, x_cl);
 	if (conv_korder(Ci, dtype, x_cl) == KORD_TAP_MAJOR)
 		return Ci / c * kHW;
 	const int kc = (Ci * kHW + c - 1) / c;
@@ -683,7 +703,7 @@ static inline long conv_kpos(int c, int tap, int Ci, int kHW, int dtype, int x_c
 	case KORD_CHANNELS_LAST:
 		return (long)tap * Ci + c;
 	case KORD_TAP_MAJOR: {
-		const int cb = conv_kch(dtype) * conv_chunk(dtype);
+		const int cb = conv_kch(dtype, false) * conv_chunk(dtype);
 		return ((long)(c / cb) * kHW + tap) * cb + c % cb;
 	}
 	default:
@@ -825,7 +845,7 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
-	const int nkt = p.KC / ConvTraits<DT>::KCH;
+	const int nkt = p.KC / conv_kch(DT, p.x_cl);
 	if (splitk > nkt)
 		splitk = nkt;
 	p.splitk = splitk < 1 ? 1 : splitk;
