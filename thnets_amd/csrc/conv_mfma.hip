@@ -878,26 +878,22 @@ template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
 	/* Tile choice, from sweeps over the VGG / AlexNet / ResNet layer shapes on
-	 * a 256-CU part.  The hardware packs the workgroups of a grid's last,
+	 * a 256-CU part.  With fragments prefetched across K-tiles a 64x64 tile
+	 * keeps its four matrix cores nearly as busy as a bigger one, and small
+	 * tiles quantise best: the hardware packs the workgroups of a grid's last,
 	 * partially filled round onto as few CUs as they fit, so a round costs
-	 * (residents per CU) x (tile time) even when nearly empty: with many tiles,
-	 * half-size tiles at four residents per CU waste the least; with few, the
-	 * big tile's better operand reuse wins; with very few, the smallest tile
-	 * spreads over the most CUs.  Splitting K is available
-	 * (thhip_conv_set_tuning) but measured slower than unsplit 64x64 tiles on
-	 * every layer shape tried, so it is never chosen. */
+	 * (residents per CU) x (tile time) even when nearly empty.  Only the
+	 * widest layers (>= 700 tiles of 128x128) gain from the 128-row tile's
+	 * operand reuse.  Splitting K is available (thhip_conv_set_tuning) but
+	 * measured slower than unsplit 64x64 tiles on every layer shape tried, so
+	 * it is never chosen. */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	int bm, bn, splitk = 1, wgs = 0;
-	if (p.Co <= 64) {
-		bm = 64;
-		bn = (long)((p.N + 127) / 128) >= 512 ? 128 : 64;
-		wgs = 4;
-	} else if (t128 >= 700) {
-		bm = 128; bn = 64; wgs = 4;
-	} else if (t128 >= 300) {
-		bm = 128; bn = 128;
+	if (p.Co > 64 && t128 >= 700) {
+		bm = 128; bn = 64;
 	} else {
 		bm = 64; bn = 64;
+		wgs = p.Co <= 64 ? 0 : 4;
 	}
 	if (g_force_bm)
 		bm = g_force_bm;
