@@ -425,11 +425,15 @@ void thhip_dequantize(const unsigned char *q, float *x, long n, float mult, floa
 /* Weight packing for the int8 kernel: uint8 codes [Co][Ci][kHW] -> signed
  * (code-128) K-chunked layout + per-row sums.  Returns a device buffer. */
 void *thhip_conv_pack_weight_u8(const unsigned char *w_host, int Co, int Ci, int kHW);
-/* The same for a convolution whose input will be channels-last in memory
- * (x_channels_last = 1: K runs tap-major, k = tap * Ci + plane; Ci % 16 == 0);
- * 0 is thhip_conv_pack_weight_u8.  The packed buffer is only valid for calls
- * with the same x_channels_last. */
-void *thhip_conv_pack_weight_u8_layout(const unsigned char *w_host, int Co, int Ci, int kHW, int x_channels_last);
+/* The same for a stated way of reading the input (codes [Co][Ci][kH][kW]):
+ *   x_layout 0  plane-major [B][C][H][W], as thhip_conv_pack_weight_u8;
+ *   x_layout 1  channels-last [B][H][W][C] in memory (K runs tap-major,
+ *               k = tap * Ci + plane; Ci % 16 == 0);
+ *   x_layout 2  plane-major in memory with Ci <= 4 (the image layer): the
+ *               convolution first copies it to [B][H][W][4] so that four
+ *               neighbouring pixels of a kernel row are one operand vector.
+ * The packed buffer is only valid for calls with the same x_layout. */
+void *thhip_conv_pack_weight_u8_layout(const unsigned char *w_host, int Co, int Ci, int kH, int kW, int x_layout);
 
 /* Replaces Lowp_SpatialConvolution_updateOutput's per-image
  * uint8 im2col + THLowpTensor_mm/lowpgemm + lowpadd
@@ -444,17 +448,17 @@ void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *add
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
 	int act, int thr, int val);
 
-/* thhip_conv2d_u8 on tensors whose memory order is chosen per side: 0 = the
- * reference's [B][C][H][W], 1 = channels-last [B][H][W][C], the order the
- * uint8 engine keeps between convolutions so that the 16 codes of one MFMA
- * operand vector are one 16-byte load.  Same arithmetic and the same
+/* thhip_conv2d_u8 with the memory order chosen per side.  x_layout as in
+ * thhip_conv_pack_weight_u8_layout (and the weights packed for it);
+ * y_channels_last 0 = the reference's [B][C][H][W], 1 = [B][H][W][C], the
+ * order the uint8 engine keeps between convolutions so that the 16 codes of
+ * one MFMA operand vector are one 16-byte load.  Same arithmetic and the same
  * reference lines; the tail rule of lowpadd still goes by the position inside
- * the plane.  Channels-last x needs Ci % 16 == 0 and weights packed for it,
- * channels-last y Co % 4 == 0. */
+ * the plane.  Channels-last y needs Co % 4 == 0. */
 void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
-	int act, int thr, int val, int x_channels_last, int y_channels_last);
+	int act, int thr, int val, int x_layout, int y_channels_last);
 
 /* Lowp_SpatialMaxPooling_updateOutput (lowp_SpatialMaxPooling.c:45-108) on
  * channels-last codes, C % 4 == 0. */

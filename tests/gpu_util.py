@@ -54,8 +54,9 @@ def unary(lib, fn, x, out_shape, dtype, *args):
 
 
 def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0, x_cl=0, y_cl=0):
-    """xq and the result are [B][C][H][W] arrays; x_cl / y_cl make the device copies
-    channels-last ([B][H][W][C]) and call the layout entry point."""
+    """xq and the result are [B][C][H][W] arrays; x_cl = 1 / y_cl = 1 make the device
+    copies channels-last ([B][H][W][C]), x_cl = 2 asks for the four-plane pixel path
+    (plane-major in memory); both call the layout entry point."""
     xq = np.ascontiguousarray(xq, np.uint8)
     wq = np.ascontiguousarray(wq, np.uint8)
     B, Ci, H, W = xq.shape
@@ -64,10 +65,10 @@ def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0, x_cl=
     oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
     note("conv2d_u8 x%s w%s d%s pad%s prm%s" % (xq.shape, wq.shape, d, pad, prm))
     if x_cl:
-        wp = lib.thhip_conv_pack_weight_u8_layout(wq.ctypes.data, Co, Ci, kH * kW, 1)
+        wp = lib.thhip_conv_pack_weight_u8_layout(wq.ctypes.data, Co, Ci, kH, kW, x_cl)
     else:
         wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, Ci, kH * kW)
-    dx = api.DeviceArray(lib, np.ascontiguousarray(xq.transpose(0, 2, 3, 1)) if x_cl else xq)
+    dx = api.DeviceArray(lib, np.ascontiguousarray(xq.transpose(0, 2, 3, 1)) if x_cl == 1 else xq)
     da = api.DeviceArray(lib, np.ascontiguousarray(addend, np.int32)) if addend is not None else None
     dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW)
     if x_cl or y_cl:

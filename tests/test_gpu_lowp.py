@@ -115,6 +115,10 @@ CL_CASES = [
     (2, 16, 10, 10, 8, 3, 3, 1, 1, 1, 1),       # K = 144 ends inside a K-tile
     (2, 48, 5, 6, 40, 2, 3, 1, 1, 0, 1),
     (2, 3, 21, 19, 64, 7, 7, 2, 2, 3, 3),       # plane-major in only (generic K order), channels-last out
+    (3, 3, 35, 35, 64, 11, 11, 4, 4, 2, 2),     # the image layer: also through the four-plane pixel copy
+    (2, 1, 9, 12, 12, 3, 3, 1, 1, 1, 1),
+    (2, 4, 8, 7, 20, 5, 2, 2, 1, 2, 0),
+    (1, 2, 6, 30, 8, 1, 9, 1, 3, 0, 4),
 ]
 
 
@@ -139,7 +143,7 @@ def test_conv_u8_channels_last_bit_exact(hiplib, oracle, i):
     zero = int(np.round(np.float32(-isub) * np.float32(im)))
     addend = np.array([oracle.lowp_bias_addend(int(c), bm, bsub, om) for c in bq], np.int32)
     thr = oracle.lowp_scale_float(om, osub, 0.0)
-    orders = [(0, 1)] + ([(1, 0), (1, 1)] if Ci % 16 == 0 else [])
+    orders = [(0, 1)] + ([(1, 0), (1, 1)] if Ci % 16 == 0 else []) + ([(2, 0), (2, 1)] if Ci <= 4 else [])
     try:
         for tune in ((0, 0, 0, 0), (64, 64, 3, 2), (128, 128, 1, 0), (64, 128, 2, 1), (128, 64, 1, 4)):
             hiplib.thhip_conv_set_tuning(*tune)

@@ -32,6 +32,7 @@
 #include "thhip_internal.h"
 
 #define CONV_THREADS 256
+#define CONV_C4_SLACK 16	/* bytes before and after the four-plane pixel copy of an input */
 
 struct ConvParams {
 	const void *x;
@@ -54,6 +55,8 @@ struct ConvParams {
 	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
 	const int *addend;	/* per-plane bias addend, or NULL */
 	int zero, offA, offB, c_off, c_mult, c_shift, ithr, ival;
+	int kwv;		/* GM_PIXELS4: vectors (four pixels) per kernel row; magic_kw divides by it */
+	unsigned c4_fill;	/* GM_PIXELS4: one pixel outside the image */
 	/* host side only: memory order of x and y, 0 = [B][C][H][W], 1 = [B][H][W][C] */
 	int x_cl, y_cl;
 };
@@ -68,7 +71,7 @@ static inline unsigned long long conv_magic(unsigned d)
 /* Chunks per K-tile (one LDS stage).  An int8 MFMA retires 32 k in the time
  * an fp32 one retires 1, so where the gather is cheap (channels-last codes)
  * deeper K-tiles keep the work per barrier up. */
-#define CONV_KCH_U8_CL 4
+#define CONV_KCH_U8_CL 2
 __host__ __device__ constexpr int conv_kch(int dtype, bool x_cl) { return dtype == THHIP_U8 && x_cl ? CONV_KCH_U8_CL : 2; }
 
 template <int DT> struct ConvTraits;
@@ -154,14 +157,20 @@ __device__ __forceinline__ KTap conv_ktap(const ConvParams &p, int k)
 	return t;
 }
 
-template <int DT, int BM, int BN, int WGM, int WGN, bool TAP, bool CLI, bool CLO>
+/* GM, how the B operand is gathered: */
+enum { GM_PLANE_TAP, GM_TAP_MAJOR, GM_CHANNELS_LAST, GM_PIXELS4 };
+
+template <int DT, int BM, int BN, int WGM, int WGN, int GM, bool CLO>
 __global__ __launch_bounds__(CONV_THREADS)
 /* ask for four waves per SIMD where the tile allows it: without the hint the
  * compiler spreads the accumulators over AGPRs plus a generous VGPR budget and
  * halves the number of workgroups a CU can hold */
-__attribute__((amdgpu_waves_per_eu((TAP || CLI) ? 4 : 1, 8))) void conv_mfma_kernel(ConvParams p)
+__attribute__((amdgpu_waves_per_eu(GM != GM_PLANE_TAP ? 4 : 1, 8))) void conv_mfma_kernel(ConvParams p)
 {
-	static_assert(!(TAP && CLI), "tap-major K order is for plane-major input");
+	constexpr bool TAP = GM == GM_TAP_MAJOR;
+	constexpr bool C4 = GM == GM_PIXELS4;		/* uint8, <= 4 planes, re-laid out as [B][H][W][4] */
+	constexpr bool CLI = GM == GM_CHANNELS_LAST || C4;
+	static_assert(!C4 || DT == THHIP_U8, "the four-plane pixel layout is a uint8 path");
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
 	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC, KCH = conv_kch(DT, CLI);
@@ -224,7 +233,9 @@ __attribute__((amdgpu_waves_per_eu((TAP || CLI) ? 4 : 1, 8))) void conv_mfma_ker
 		int oy = r / p.oW, ox = r - oy * p.oW;
 		iy0_[q] = oy * p.dH - p.padH;
 		ix0_[q] = ox * p.dW - p.padW;
-		if constexpr (CLI)
+		if constexpr (C4)
+			xoff_[q] = ((b * p.H + iy0_[q]) * p.W + ix0_[q]) * 4 + CONV_C4_SLACK;
+		else if constexpr (CLI)
 			xoff_[q] = ((b * p.H + iy0_[q]) * p.W + ix0_[q]) * p.Ci;
 		else
 			xoff_[q] = b * p.Ci * p.HW + iy0_[q] * p.W + ix0_[q];
@@ -270,7 +281,15 @@ __attribute__((amdgpu_waves_per_eu((TAP || CLI) ? 4 : 1, 8))) void conv_mfma_ker
 		/* (CLI) decode of this thread's vector: the same for all its positions */
 		int cl_kh = 0, cl_kw = 0, cl_off = 0;
 		bool k_ok = true;		/* (CLI) the vector lies inside K */
-		if constexpr (CLI) {
+		if constexpr (C4) {
+			/* vector = four pixels of one kernel row: K runs (kh, kw4, pixel, plane) */
+			const unsigned vi = kt * VPP + pv;
+			const unsigned kh = vi * p.mhi_kw + __umulhi(vi, p.magic_kw);	/* / vectors per kernel row */
+			cl_kh = (int)kh;
+			cl_kw = (int)(vi - kh * p.kwv) * 4;
+			cl_off = (cl_kh * p.W + cl_kw) * 4;
+			k_ok = cl_kh < p.kH;
+		} else if constexpr (CLI) {
 			const int kv = (kt * VPP + pv) * VEC;
 			const unsigned tap = (unsigned)kv * p.mhi_ci + __umulhi((unsigned)kv, p.magic_ci);
 			const int c = kv - tap * p.Ci;
@@ -286,7 +305,26 @@ __attribute__((amdgpu_waves_per_eu((TAP || CLI) ? 4 : 1, 8))) void conv_mfma_ker
 			const int q = CLI ? j : 0;	/* which of the thread's positions */
 			elem v[VEC];
 			bool vec_ok = tap_ok;		/* (TAP, CLI) the vector lies inside the image */
-			if constexpr (CLI) {
+			if constexpr (C4) {
+				const int iy = iy0_[q] + cl_kh, ix = ix0_[q] + cl_kw;
+				const bool row_ok = n_ok_[q] && k_ok && (unsigned)iy < (unsigned)p.H;
+				/* the copy has slack on both sides, so a vector that sticks
+				 * out of its row still lies inside the buffer */
+				const unsigned voff = row_ok ? (unsigned)(xoff_[q] + cl_off) : 0x80000000u;
+				uintx4 ld = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, voff, 0, 0);
+				/* per pixel: a tap past the kernel row or a column past N is
+				 * code 128 (0 once re-centred, and its weight is 0 too); a
+				 * pixel outside the image is the code of 0.0 in the real
+				 * planes and 128 in the padding planes */
+				const unsigned fillpix = p.c4_fill;
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const bool live = n_ok_[q] && k_ok && cl_kw + e < p.kW;
+					const bool inside = row_ok && (unsigned)(ix + e) < (unsigned)p.W;
+					ld[e] = !live ? 0x80808080u : inside ? ld[e] : fillpix;
+				}
+				__builtin_memcpy(v, &ld, 16);
+			} else if constexpr (CLI) {
 				const int iy = iy0_[q] + cl_kh, ix = ix0_[q] + cl_kw;
 				vec_ok = n_ok_[q] && k_ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
 				/* the buffer is shorter than 2^31 bytes: the second offset is
@@ -336,7 +374,7 @@ __attribute__((amdgpu_waves_per_eu((TAP || CLI) ? 4 : 1, 8))) void conv_mfma_ker
 				/* code - 128 as a signed byte, and this thread's share of the
 				 * column sum of the re-centred codes */
 				intx4 cw = __builtin_bit_cast(intx4, packed);
-				if constexpr (TAP || CLI) {
+				if constexpr (TAP || (CLI && !C4)) {
 					/* the whole vector shares one tap: fill it at once */
 					const int fill = ((n_ok_[q] && k_ok) ? p.zero : 128) * 0x01010101;
 #pragma unroll
@@ -669,39 +707,53 @@ __attribute__((amdgpu_waves_per_eu((TAP || CLI) ? 4 : 1, 8))) void conv_mfma_ker
 
 static inline int conv_chunk(int dtype) { return dtype == THHIP_F32 ? 8 : dtype == THHIP_U8 ? 32 : 16; }
 
-/* Order of (plane c, tap) along the packed K axis; follows the input's memory
- * order, so weights are packed for one of them. */
-enum { KORD_PLANE_TAP, KORD_TAP_MAJOR, KORD_CHANNELS_LAST };
+/* Order of (plane c, tap) along the packed K axis; follows how the input is
+ * read (xl: 0 plane-major, 1 channels-last, 2 plane-major read through a
+ * four-plane pixel copy), so weights are packed for one of them. */
+enum { KORD_PLANE_TAP, KORD_TAP_MAJOR, KORD_CHANNELS_LAST, KORD_PIXELS4 };
 
 /* Tap-major K order needs whole blocks of KCH*chunk input planes. */
 static inline bool conv_tap_major(int Ci, int dtype) { return Ci % (conv_kch(dtype, false) * conv_chunk(dtype)) == 0; }
 
-static inline int conv_korder(int Ci, int dtype, int x_cl)
+static inline int conv_korder(int Ci, int dtype, int xl)
 {
-	if (x_cl) {
+	if (xl == 1) {
 		if (Ci % (conv_chunk(dtype) / 2))
 			THError("thhip_conv2d: channels-last input needs Ci %% %d == 0 (Ci = %d)", conv_chunk(dtype) / 2, Ci);
 		return KORD_CHANNELS_LAST;
 	}
+	if (xl == 2) {
+		if (dtype != THHIP_U8 || Ci > 4)
+			THError("thhip_conv2d: the four-plane pixel path is for uint8 inputs of at most 4 planes (Ci = %d)", Ci);
+		return KORD_PIXELS4;
+	}
+	if (xl)
+		THError("thhip_conv2d: unknown input layout %d", xl);
 	return conv_tap_major(Ci, dtype) ? KORD_TAP_MAJOR : KORD_PLANE_TAP;
 }
 
 /* Number of K chunks (always whole K-tiles). */
-static inline int conv_kc(int Ci, int kHW, int dtype, int x_cl)
+static inline int conv_kc(int Ci, int kH, int kW, int dtype, int xl)
 {
-	const int c = conv_chunk(dtype), kch = conv_kch(dtype, x_cl);
-	if (conv_korder(Ci, dtype, x_cl) == KORD_TAP_MAJOR)
-		return Ci / c * kHW;
-	const int kc = (Ci * kHW + c - 1) / c;
+	const int c = conv_chunk(dtype), kch = conv_kch(dtype, xl != 0);
+	const int ord = conv_korder(Ci, dtype, xl);
+	if (ord == KORD_TAP_MAJOR)
+		return Ci / c * kH * kW;
+	/* four-plane pixels: a kernel row is (kW+3)/4 vectors of 4 pixels x 4 planes */
+	const long K = ord == KORD_PIXELS4 ? (long)kH * ((kW + 3) / 4) * 16 : (long)Ci * kH * kW;
+	const int kc = (int)((K + c - 1) / c);
 	return (kc + kch - 1) / kch * kch;
 }
 
-/* Position of weight (plane c, tap) along the packed K axis. */
-static inline long conv_kpos(int c, int tap, int Ci, int kHW, int dtype, int x_cl)
+/* Position of weight (plane c, tap (kh, kw)) along the packed K axis. */
+static inline long conv_kpos(int c, int kh, int kw, int Ci, int kH, int kW, int dtype, int xl)
 {
-	switch (conv_korder(Ci, dtype, x_cl)) {
+	const int tap = kh * kW + kw, kHW = kH * kW;
+	switch (conv_korder(Ci, dtype, xl)) {
 	case KORD_CHANNELS_LAST:
 		return (long)tap * Ci + c;
+	case KORD_PIXELS4:
+		return (((long)kh * ((kW + 3) / 4) + kw / 4) * 4 + kw % 4) * 4 + c;
 	case KORD_TAP_MAJOR: {
 		const int cb = conv_kch(dtype, false) * conv_chunk(dtype);
 		return ((long)(c / cb) * kHW + tap) * cb + c % cb;
@@ -720,15 +772,16 @@ static inline size_t conv_pack_index(int m, long kp, int KC, int chunk)
 	return ((((size_t)(m >> 5) * KC + kc) * 2 + h) * 32 + (m & 31)) * vec + e;
 }
 
-static size_t conv_packed_bytes(int Co, int Ci, int kHW, int dtype, int x_cl)
+static size_t conv_packed_bytes(int Co, int Ci, int kH, int kW, int dtype, int xl)
 {
 	size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
-	return mpad / 32 * conv_kc(Ci, kHW, dtype, x_cl) * 1024;
+	return mpad / 32 * conv_kc(Ci, kH, kW, dtype, xl) * 1024;
 }
 
+/* (for plane-major input the packed size depends on kH * kW only) */
 extern "C" size_t thhip_conv_packed_bytes(int Co, int Ci, int kHW, int dtype)
 {
-	return conv_packed_bytes(Co, Ci, kHW, dtype, 0);
+	return conv_packed_bytes(Co, Ci, 1, kHW, dtype, 0);
 }
 
 static inline unsigned short f32_to_f16_bits(float f)
@@ -753,7 +806,7 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 {
 	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
 		THError("thhip_conv_pack_weight: unsupported dtype %d", dtype);
-	const int chunk = conv_chunk(dtype), KC = conv_kc(Ci, kHW, dtype, 0);
+	const int chunk = conv_chunk(dtype), KC = conv_kc(Ci, 1, kHW, dtype, 0);
 	const size_t bytes = thhip_conv_packed_bytes(Co, Ci, kHW, dtype);
 	unsigned char *host = (unsigned char *)calloc(1, bytes);
 	if (!host)
@@ -761,7 +814,7 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 	for (int m = 0; m < Co; m++)
 		for (int c = 0; c < Ci; c++)
 			for (int tap = 0; tap < kHW; tap++) {
-				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, dtype, 0), KC, chunk);
+				const size_t idx = conv_pack_index(m, conv_kpos(c, 0, tap, Ci, 1, kHW, dtype, 0), KC, chunk);
 				const float v = w[((size_t)m * Ci + c) * kHW + tap];
 				if (dtype == THHIP_F32)
 					((float *)host)[idx] = v;
@@ -845,7 +898,7 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
-	const int nkt = p.KC / conv_kch(DT, p.x_cl);
+	const int nkt = p.KC / conv_kch(DT, p.x_cl != 0);
 	if (splitk > nkt)
 		splitk = nkt;
 	p.splitk = splitk < 1 ? 1 : splitk;
@@ -856,22 +909,30 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 	const bool tap = conv_tap_major(p.Ci, DT);
 	if (p.y_cl && p.Co % 4)
 		THError("thhip_conv2d: channels-last output needs Co %% 4 == 0 (Co = %d)", p.Co);
+#define CONV_GO(GM, CLO) return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, GM, CLO>>(p, grid, wgs)
 	if constexpr (DT == THHIP_U8) {
 		/* the uint8 engine keeps its activations channels-last between convolutions */
-		if (p.x_cl && p.y_cl)
-			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, true, true>>(p, grid, wgs);
-		if (p.x_cl)
-			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, true, false>>(p, grid, wgs);
-		if (p.y_cl && tap)
-			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, false, true>>(p, grid, wgs);
-		if (p.y_cl)
-			return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, false, true>>(p, grid, wgs);
+		if (p.x_cl == 2) {
+			if (p.y_cl)
+				CONV_GO(GM_PIXELS4, true);
+			CONV_GO(GM_PIXELS4, false);
+		}
+		if (p.x_cl) {
+			if (p.y_cl)
+				CONV_GO(GM_CHANNELS_LAST, true);
+			CONV_GO(GM_CHANNELS_LAST, false);
+		}
+		if (p.y_cl) {
+			if (tap)
+				CONV_GO(GM_TAP_MAJOR, true);
+			CONV_GO(GM_PLANE_TAP, true);
+		}
 	} else if (p.x_cl || p.y_cl)
 		THError("thhip_conv2d: channels-last tensors are a uint8 feature");
 	if (tap)
-		conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, true, false, false>>(p, grid, wgs);
-	else
-		conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, false, false, false>>(p, grid, wgs);
+		CONV_GO(GM_TAP_MAJOR, false);
+	CONV_GO(GM_PLANE_TAP, false);
+#undef CONV_GO
 }
 
 template <int DT>
@@ -889,7 +950,11 @@ static void conv_dispatch(ConvParams &p)
 	 * it is never chosen. */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	int bm, bn, splitk = 1, wgs = 0;
-	if (p.Co > 64 && t128 >= 700) {
+	if (DT == THHIP_U8) {
+		/* int8 MFMAs outrun LDS at any of these tile sizes; the smallest
+		 * tile has the most workgroups in flight and measured fastest */
+		bm = 64; bn = 64;
+	} else if (p.Co > 64 && t128 >= 700) {
 		bm = 128; bn = 64;
 	} else {
 		bm = 64; bn = 64;
@@ -917,8 +982,41 @@ static void conv_dispatch(ConvParams &p)
 
 struct ConvU8Args {
 	const int *addend;
-	int zero, a_off, b_off, c_off, c_mult, c_shift, ithr, ival, x_cl, y_cl;
+	int zero, a_off, b_off, c_off, c_mult, c_shift, ithr, ival;
+	int x_cl;	/* 0 plane-major, 1 channels-last, 2 plane-major read through a four-plane pixel copy */
+	int y_cl;
 };
+
+/* Codes [B][C][HW], C <= 4 -> [B][HW][4] with code 128 (0 once re-centred) in
+ * the planes that do not exist: one word per pixel, so that four neighbouring
+ * pixels of a kernel row are one 16-byte operand vector. */
+__global__ void conv_pixels4_kernel(const unsigned char *x, unsigned *y, int C, long HW, long total)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total; i += step) {
+		const long b = i / HW, r = i - b * HW;
+		const unsigned char *src = x + b * C * HW + r;
+		unsigned w = 0x80808080u;
+		for (int c = 0; c < C; c++)
+			w = (w & ~(255u << (8 * c))) | ((unsigned)src[c * HW] << (8 * c));
+		y[i] = w;
+	}
+}
+
+static unsigned char *g_c4;
+static size_t g_c4_bytes;
+
+static unsigned char *conv_pixels4_scratch(size_t bytes)
+{
+	if (bytes > g_c4_bytes) {
+		hipcheck(hipStreamSynchronize(thhip_stream()));
+		thhip_free(g_c4);
+		g_c4 = (unsigned char *)thhip_malloc(bytes);
+		g_c4_bytes = bytes;
+	}
+	return g_c4;
+}
 
 static void conv_run(const void *x, const void *wpacked, const float *bias, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
@@ -937,8 +1035,10 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 		THError("thhip_conv2d: K = %ld too large", K);
 	/* 32-bit offsets inside the kernel: run the batch in slices whose input
 	 * and output stay below 2^31 bytes. */
+	const int xl = u8 ? u8->x_cl : 0;
 	const long in_img = (long)Ci * H * W, out_img = (long)Co * oH * oW;
-	long bmax = ((1L << 31) - 16) / (esize * (in_img > out_img ? in_img : out_img));
+	const long in_eff = xl == 2 ? 4L * H * W : in_img;	/* bytes the kernel addresses per image */
+	long bmax = ((1L << 31) - 64) / (esize * (in_eff > out_img ? in_eff : out_img));
 	if (bmax < 1)
 		THError("thhip_conv2d: one image exceeds 2 GiB");
 	if ((long)oH * oW * bmax > (1L << 30))
@@ -954,7 +1054,7 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 		p.B = bn; p.Ci = Ci; p.H = H; p.W = W; p.Co = Co; p.kH = kH; p.kW = kW;
 		p.dH = dH; p.dW = dW; p.padH = padH; p.padW = padW; p.oH = oH; p.oW = oW;
 		p.K = (int)K;
-		p.KC = conv_kc(Ci, kH * kW, dtype, u8 && u8->x_cl);
+		p.KC = conv_kc(Ci, kH, kW, dtype, xl);
 		p.N = bn * oH * oW;
 		p.oHW = oH * oW;
 		p.HW = H * W;
@@ -968,14 +1068,37 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 		p.act = act; p.thr = thr; p.val = val;
 		p.x_bytes = (unsigned)(bn * in_img * esize);
 		if (u8) {
-			p.rowsum = (const int *)((const char *)wpacked + conv_packed_bytes(Co, Ci, kH * kW, THHIP_U8, u8->x_cl));
+			p.rowsum = (const int *)((const char *)wpacked + conv_packed_bytes(Co, Ci, kH, kW, THHIP_U8, xl));
 			p.addend = u8->addend;
 			p.zero = u8->zero;
 			p.offA = 128 + u8->a_off;
 			p.offB = 128 + u8->b_off;
 			p.c_off = u8->c_off; p.c_mult = u8->c_mult; p.c_shift = u8->c_shift;
 			p.ithr = u8->ithr; p.ival = u8->ival;
-			p.x_cl = u8->x_cl; p.y_cl = u8->y_cl;
+			p.x_cl = xl; p.y_cl = u8->y_cl;
+			if (xl == 2) {
+				/* the kernel reads a [B][H][W][4] copy with slack on both sides */
+				const long pixels = (long)bn * H * W;
+				const size_t bytes = (size_t)pixels * 4 + 2 * CONV_C4_SLACK;
+				unsigned char *c4 = conv_pixels4_scratch(bytes);
+				{
+					ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)bn * in_img + 4.0 * pixels);
+					long blocks = (pixels + 255) / 256;
+					if (blocks > 65536 * 16)
+						blocks = 65536 * 16;
+					conv_pixels4_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
+						(const unsigned char *)p.x, (unsigned *)(c4 + CONV_C4_SLACK), Ci, (long)H * W, pixels);
+				}
+				p.x = c4;
+				p.x_bytes = (unsigned)bytes;
+				p.kwv = (kW + 3) / 4;
+				p.magic_kw = (unsigned)conv_magic(p.kwv);
+				p.mhi_kw = (unsigned)(conv_magic(p.kwv) >> 32);
+				unsigned fill = 0x80808080u;
+				for (int c = 0; c < Ci; c++)
+					fill = (fill & ~(255u << (8 * c))) | ((unsigned)p.zero << (8 * c));
+				p.c4_fill = fill;
+			}
 			ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * Co * (double)K * p.N);
 			conv_dispatch<THHIP_U8>(p);
 		} else {
@@ -994,13 +1117,13 @@ extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bi
 	conv_run(x, wpacked, bias, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0);
 }
 
-/* uint8 codes [Co][Ci][kHW] -> (code - 128) as signed bytes in the packed layout,
- * followed by the per-row sums of the re-centred codes. */
-extern "C" void *thhip_conv_pack_weight_u8_layout(const unsigned char *w, int Co, int Ci, int kHW, int x_channels_last)
+/* uint8 codes [Co][Ci][kH][kW] -> (code - 128) as signed bytes in the packed
+ * layout for input layout xl, followed by the per-row sums of the re-centred codes. */
+extern "C" void *thhip_conv_pack_weight_u8_layout(const unsigned char *w, int Co, int Ci, int kH, int kW, int x_layout)
 {
-	const int x_cl = x_channels_last != 0;
-	const int chunk = 32, KC = conv_kc(Ci, kHW, THHIP_U8, x_cl);
-	const size_t bytes = conv_packed_bytes(Co, Ci, kHW, THHIP_U8, x_cl);
+	const int xl = x_layout;
+	const int chunk = 32, KC = conv_kc(Ci, kH, kW, THHIP_U8, xl);
+	const size_t bytes = conv_packed_bytes(Co, Ci, kH, kW, THHIP_U8, xl);
 	const size_t mpad = (size_t)(Co + CONV_MPAD - 1) / CONV_MPAD * CONV_MPAD;
 	const size_t total = bytes + mpad * sizeof(int);
 	unsigned char *host = (unsigned char *)calloc(1, total);
@@ -1010,12 +1133,13 @@ extern "C" void *thhip_conv_pack_weight_u8_layout(const unsigned char *w, int Co
 	for (int m = 0; m < Co; m++) {
 		int sum = 0;
 		for (int c = 0; c < Ci; c++)
-			for (int tap = 0; tap < kHW; tap++) {
-				const size_t idx = conv_pack_index(m, conv_kpos(c, tap, Ci, kHW, THHIP_U8, x_cl), KC, chunk);
-				const int v = (int)w[((size_t)m * Ci + c) * kHW + tap] - 128;
-				host[idx] = (unsigned char)(signed char)v;
-				sum += v;
-			}
+			for (int kh = 0; kh < kH; kh++)
+				for (int kw = 0; kw < kW; kw++) {
+					const size_t idx = conv_pack_index(m, conv_kpos(c, kh, kw, Ci, kH, kW, THHIP_U8, xl), KC, chunk);
+					const int v = (int)w[(((size_t)m * Ci + c) * kH + kh) * kW + kw] - 128;
+					host[idx] = (unsigned char)(signed char)v;
+					sum += v;
+				}
 		rowsum[m] = sum;
 	}
 	void *dev = thhip_malloc(total);
@@ -1026,18 +1150,18 @@ extern "C" void *thhip_conv_pack_weight_u8_layout(const unsigned char *w, int Co
 
 extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int Ci, int kHW)
 {
-	return thhip_conv_pack_weight_u8_layout(w, Co, Ci, kHW, 0);
+	return thhip_conv_pack_weight_u8_layout(w, Co, Ci, 1, kHW, 0);
 }
 
 extern "C" void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
-	int act, int thr, int val, int x_channels_last, int y_channels_last)
+	int act, int thr, int val, int x_layout, int y_channels_last)
 {
 	if (c_shift < 0 || c_shift > 31)
 		THError("thhip_conv2d_u8: shift %d out of range", c_shift);
 	ConvU8Args u8 = { addend, zero & 255, a_off, b_off, c_off, c_mult, c_shift, thr, val,
-		x_channels_last != 0, y_channels_last != 0 };
+		x_layout, y_channels_last != 0 };
 	conv_run(x, wpacked, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
 }
 
@@ -1122,7 +1246,7 @@ __global__ void conv_unpack_rows_kernel(const E *wp, E *rows, int Co, int Ci, in
 
 extern "C" void *thhip_conv_unpack_rows(const void *wpacked, int Co, int Ci, int kHW, int dtype)
 {
-	const int KC = conv_kc(Ci, kHW, dtype, 0), chunk = conv_chunk(dtype), tm = conv_tap_major(Ci, dtype);
+	const int KC = conv_kc(Ci, 1, kHW, dtype, 0), chunk = conv_chunk(dtype), tm = conv_tap_major(Ci, dtype);
 	const long total = (long)Co * Ci * kHW;
 	void *rows = thhip_malloc((size_t)total * thhip_esize(dtype));
 	long blocks = (total + 255) / 256;

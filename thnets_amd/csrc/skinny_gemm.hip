@@ -310,31 +310,31 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_u8_kernel(const unsigned ch
 	}
 }
 
-/* One workgroup per 32 output rows: sums the K slices, requantises and
- * transposes [row][batch] partials into y [B][nOut] through LDS. */
+/* One workgroup per 32 output rows x 16 batch columns: sums the K slices,
+ * requantises and transposes [row][batch] partials into y [B][nOut] through LDS. */
 __global__ __launch_bounds__(256) void skinny_u8_finish_kernel(const int *part, const int *cspart, const int *rowsum,
 	const int *addend, unsigned char *y, int B, int K, int nOut, int ksplit, int offA, int offB,
 	int c_off, int c_mult, int c_shift, int act, int thr, int val)
 {
-	__shared__ int t[32][65];
-	__shared__ int csum[SKU_BPAD];
-	const int tid = threadIdx.x, o0 = blockIdx.x * 32;
-	if (tid < SKU_BPAD) {
+	__shared__ int t[32][17];
+	__shared__ int csum[16];
+	const int tid = threadIdx.x, o0 = blockIdx.x * 32, b0 = blockIdx.y * 16;
+	if (tid < 16) {
 		int s = 0;
 		for (int p = 0; p < ksplit; p++)
-			s += cspart[p * SKU_BPAD + tid];
+			s += cspart[p * SKU_BPAD + b0 + tid];
 		csum[tid] = s;
 	}
 	{
-		const int b = tid & 63, oo = tid >> 6;
+		const int bl = tid & 15, oo = tid >> 4;
 #pragma unroll
-		for (int i = 0; i < 8; i++) {
-			const int ol = oo + 4 * i, o = o0 + ol;
+		for (int i = 0; i < 2; i++) {
+			const int ol = oo + 16 * i, o = o0 + ol;
 			int s = 0;
-			if (o < nOut && b < B)
+			if (o < nOut && b0 + bl < B)
 				for (int p = 0; p < ksplit; p++)
-					s += part[((size_t)p * nOut + o) * SKU_BPAD + b];
-			t[ol][b] = s;
+					s += part[((size_t)p * nOut + o) * SKU_BPAD + b0 + bl];
+			t[ol][bl] = s;
 		}
 	}
 	__syncthreads();
@@ -344,11 +344,11 @@ __global__ __launch_bounds__(256) void skinny_u8_finish_kernel(const int *part, 
 	const int rs = offB * rowsum[o] + K * offA * offB;
 	const int add = addend ? addend[o] : 0;
 #pragma unroll
-	for (int i = 0; i < 8; i++) {
-		const int b = bb + 8 * i;
+	for (int i = 0; i < 2; i++) {
+		const int bl = bb + 8 * i, b = b0 + bl;
 		if (b >= B)
 			break;
-		const int a = t[ol][b] + rs + offA * csum[b];
+		const int a = t[ol][bl] + rs + offA * csum[bl];
 		unsigned u = ((unsigned)a + (unsigned)c_off) * (unsigned)c_mult;
 		u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
 		int q = (int)u >> c_shift;
@@ -463,7 +463,7 @@ extern "C" void thhip_linear_batched_u8(const unsigned char *x, const unsigned c
 	}
 	{
 		ThhipLaunchScope scope(THHIP_FAM_OTHER, (4.0 * ksplit + 1.0) * B * nOut);
-		skinny_u8_finish_kernel<<<dim3((nOut + 31) / 32), dim3(256), 0, thhip_stream()>>>(part, cspart, rowsum, addend, y,
+		skinny_u8_finish_kernel<<<dim3((nOut + 31) / 32, (B + 15) / 16), dim3(256), 0, thhip_stream()>>>(part, cspart, rowsum, addend, y,
 			B, K, nOut, ksplit, 128 + a_off, 128 + b_off, c_off, c_mult, c_shift, act, thr, val);
 	}
 }

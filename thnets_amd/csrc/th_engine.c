@@ -469,7 +469,7 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 	if (s.H * s.W > 1 && hn->cur_cl != hm->in_cl)
 		THError("uint8 engine: a convolution planned for %s input got the other memory order",
 			hm->in_cl ? "channels-last" : "plane-major");
-	const int x_cl = hm->in_cl;
+	const int x_cl = hm->x_layout;
 	if (hm->wrow_u8 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
 	    thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
 		thhip_linear_batched_u8(x, hm->wrow_u8, hm->rowsum_u8, hm->addend, y, s.B, K, c->nOutputPlane,
@@ -878,7 +878,9 @@ static void plan_channels_last(struct hipnet *hn)
 		const struct SpatialConvolution *c = &m->SpatialConvolution;
 		const int Co = c->nOutputPlane, Ci = c->nInputPlane, kHW = c->kH * c->kW;
 		const long K = (long)Ci * kHW;
-		hm->wpacked = thhip_conv_pack_weight_u8_layout(hm->wq_host, Co, Ci, kHW, hm->in_cl);
+		/* the image layer (<= 4 planes, plane-major) goes through the four-plane pixel copy */
+		hm->x_layout = hm->in_cl ? 1 : Ci <= 4 ? 2 : 0;
+		hm->wpacked = thhip_conv_pack_weight_u8_layout(hm->wq_host, Co, Ci, c->kH, c->kW, hm->x_layout);
 		if (K % 16 == 0 && K >= 512) {
 			unsigned char *rows = hm->wq_host;
 			if (hm->in_cl && kHW > 1) {

@@ -24,6 +24,7 @@ struct hipmod {
 	int *rowsum_u8;		/* their re-centred row sums (device) */
 	unsigned char *wq_host;	/* weight codes on the host, only while the network is being built */
 	int in_cl, out_cl;	/* input / output codes are channels-last [B][H][W][C] in memory */
+	int x_layout;		/* how the convolution reads its input: thhip_conv_pack_weight_u8_layout */
 	float wm, wsub;		/* weight quantisation */
 	float q_mult, q_sub;	/* quantisation of this module's output */
 };
