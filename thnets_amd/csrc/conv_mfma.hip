@@ -490,6 +490,22 @@ __attribute__((amdgpu_waves_per_eu(GM != GM_PLANE_TAP ? 4 : 1, 8))) void conv_mf
 		}
 		if (kt + 2 < nkt)
 			store_tile(st2);
+		if constexpr (DT == THHIP_F32 && GM != GM_PLANE_TAP) {
+			/* Ask the scheduler to spread the K-tile's loads, LDS traffic and
+			 * address arithmetic between the MFMAs instead of bunching them
+			 * before and after: the matrix core then works while they issue
+			 * (measured: +2.5 % on fp32, nothing on the shorter half and
+			 * int8 MFMAs). */
+			constexpr int NM = KCH * TM * TN * 4;
+#pragma unroll
+			for (int m = 0; m < NM; m++) {
+				__builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+				__builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+				__builtin_amdgcn_sched_group_barrier(0x006, 6, 0);
+				__builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+			}
+		}
 		__syncthreads();
 	};
 	if constexpr (TAP || CLI) {
