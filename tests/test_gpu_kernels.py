@@ -160,7 +160,8 @@ def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
         G.assert_close(dy.get((B, nOut), np.float32), np.maximum(oracle.linear(x, w, None), 0), FP32_TOL)
     assert not hiplib.thhip_linear_batched_supported(33, 128, 64, G.F32)
     assert not hiplib.thhip_linear_batched_supported(4, 130, 64, G.F32)
-    assert not hiplib.thhip_linear_batched_supported(4, 128, 64, G.F16)
+    assert hiplib.thhip_linear_batched_supported(4, 128, 64, G.F16)
+    assert not hiplib.thhip_linear_batched_supported(4, 132, 64, G.F16)        # half rows come in 16-byte vectors
     for i in (2, 3):
         x, s = cases.linear_case(i)
         B, nIn = x.shape
@@ -172,6 +173,28 @@ def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
         hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 0, 0.0, 0.0, G.F32)
         hiplib.thhip_sync()
         G.assert_close(dy.get((B, nOut), np.float32), GOLD["linear%d" % i], FP32_TOL)
+
+
+@pytest.mark.parametrize("dt", [G.F16, G.BF16])
+def test_linear_batched_half_types(hiplib, oracle, dt):
+    """fp16 / bf16 storage and MFMA, fp32 accumulation: against the fp32 restatement on
+    the rounded operands at the half tolerance (2e-2 of the largest reference value)."""
+    from thnets_amd import api
+    g = cases.rng(907)
+    for (B, nIn, nOut) in [(4, 128, 64), (16, 4096, 1000), (32, 1032, 515), (17, 200, 33), (3, 25088, 40)]:
+        x = g.standard_normal((B, nIn), dtype=np.float32)
+        w = g.standard_normal((nOut, nIn), dtype=np.float32) * np.float32(np.sqrt(2.0 / nIn))
+        b = g.standard_normal(nOut, dtype=np.float32)
+        G.note("linear_batched half dt%d %s" % (dt, (B, nIn, nOut)))
+        dx, dw = api.to_device_dtype(hiplib, x, dt), api.to_device_dtype(hiplib, w, dt)
+        db = api.DeviceArray(hiplib, b)
+        dy = api.DeviceArray(hiplib, nbytes=B * nOut * 2)
+        hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 1, 0.0, 0.0, dt)
+        hiplib.thhip_sync()
+        xr = api.from_device_dtype(dx, x.shape, dt)
+        wr = api.from_device_dtype(dw, w.shape, dt)
+        want = np.maximum(oracle.linear(xr, wr, b), 0)
+        G.assert_close(api.from_device_dtype(dy, (B, nOut), dt), want, HALF_TOL, str((B, nIn, nOut)))
 
 
 def test_threshold_bit_exact(hiplib, oracle):

@@ -447,8 +447,10 @@ __attribute__((amdgpu_waves_per_eu(GM != GM_PLANE_TAP ? 4 : 1, 8))) void conv_mf
 		t_kw = tap - t_kh * p.kW;
 	}
 	/* Software pipeline over three LDS stages.  While tile kt is multiplied,
-	 * tile kt+1 is already complete in LDS and tile kt+2 travels global memory
-	 * -> registers -> LDS, so fragments are read one chunk ahead of their
+	 * tile kt+1 is already complete in LDS, tile kt+2 moves from registers to
+	 * LDS and tile kt+3 is on its way from global memory to registers, so a
+	 * load has a whole K-tile of MFMAs to arrive and fragments are read one
+	 * chunk ahead of their
 	 * MFMAs, across the tile boundary too, and a wave's matrix core never
 	 * waits on LDS latency; one barrier per K-tile. */
 	floatx4 af[2][TM], bf[2][TN];
@@ -469,13 +471,19 @@ __attribute__((amdgpu_waves_per_eu(GM != GM_PLANE_TAP ? 4 : 1, 8))) void conv_mf
 		load_tile(kt0 + 1);
 		store_tile(1);
 	}
+	if (kt0 + 2 < nkt)
+		load_tile(kt0 + 2);
 	__syncthreads();
 	read_frags(0, 0, af[0], bf[0]);
 	static_assert(KCH % 2 == 0, "fragment sets alternate by chunk parity");
 	/* tile kt is in stage st, tile kt+1 in st1, and tile kt+2 goes to st2 */
 	auto step = [&](int kt, auto st, auto st1, auto st2) {
+		/* tile kt+2 was requested a whole step ago: it has had the time to
+		 * arrive, so parking it in LDS does not stall the MFMAs */
 		if (kt + 2 < nkt)
-			load_tile(kt + 2);
+			store_tile(st2);
+		if (kt + 3 < nkt)
+			load_tile(kt + 3);
 #pragma unroll
 		for (int c = 0; c < KCH; c++) {
 			if (c + 1 < KCH)
@@ -488,8 +496,6 @@ __attribute__((amdgpu_waves_per_eu(GM != GM_PLANE_TAP ? 4 : 1, 8))) void conv_mf
 				for (int j = 0; j < TN; j++)
 					conv_mma<DT>(acc[i][j], af[c & 1][i], bf[c & 1][j]);
 		}
-		if (kt + 2 < nkt)
-			store_tile(st2);
 		if constexpr (DT == THHIP_F32 && GM != GM_PLANE_TAP) {
 			/* Ask the scheduler to spread the K-tile's loads, LDS traffic and
 			 * address arithmetic between the MFMAs instead of bunching them
@@ -1020,6 +1026,26 @@ __global__ void conv_pixels4_kernel(const unsigned char *x, unsigned *y, int C, 
 	}
 }
 
+/* The same, four pixels per thread (HW % 4 == 0): one word per plane in, 16 bytes out. */
+__global__ void conv_pixels4x4_kernel(const unsigned *x, uintx4 *y, int C, long HW4, long total4)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total4; i += step) {
+		const long b = i / HW4, r = i - b * HW4;
+		const unsigned *src = x + b * C * HW4 + r;
+		unsigned pl[4] = { 0x80808080u, 0x80808080u, 0x80808080u, 0x80808080u };
+		for (int c = 0; c < C; c++)
+			pl[c] = src[c * HW4];
+		uintx4 o;
+#pragma unroll
+		for (int e = 0; e < 4; e++)	/* pixel e: byte e of every plane word */
+			o[e] = ((pl[0] >> (8 * e)) & 255u) | (((pl[1] >> (8 * e)) & 255u) << 8) |
+				(((pl[2] >> (8 * e)) & 255u) << 16) | (((pl[3] >> (8 * e)) & 255u) << 24);
+		y[i] = o;
+	}
+}
+
 static unsigned char *g_c4;
 static size_t g_c4_bytes;
 
@@ -1099,11 +1125,17 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 				unsigned char *c4 = conv_pixels4_scratch(bytes);
 				{
 					ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)bn * in_img + 4.0 * pixels);
-					long blocks = (pixels + 255) / 256;
+					const bool quads = ((long)H * W) % 4 == 0 && ((size_t)p.x & 3) == 0;
+					const long work = quads ? pixels / 4 : pixels;
+					long blocks = (work + 255) / 256;
 					if (blocks > 65536 * 16)
 						blocks = 65536 * 16;
-					conv_pixels4_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
-						(const unsigned char *)p.x, (unsigned *)(c4 + CONV_C4_SLACK), Ci, (long)H * W, pixels);
+					if (quads)
+						conv_pixels4x4_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
+							(const unsigned *)p.x, (uintx4 *)(c4 + CONV_C4_SLACK), Ci, (long)H * W / 4, work);
+					else
+						conv_pixels4_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
+							(const unsigned char *)p.x, (unsigned *)(c4 + CONV_C4_SLACK), Ci, (long)H * W, pixels);
 				}
 				p.x = c4;
 				p.x_bytes = (unsigned)bytes;

@@ -191,16 +191,60 @@ __global__ void maxpool_u8_cl_kernel(const unsigned *x, unsigned *y, PoolParams 
 	}
 }
 
+/* Sixteen planes per thread (C % 16 == 0): 16-byte loads and stores. */
+__global__ void maxpool_u8_cl16_kernel(const uintx4 *x, uintx4 *y, PoolParams p)
+{
+	const int C16 = p.C / 16;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < p.total; i += step) {
+		const int c16 = (int)(i % C16);
+		long t = i / C16;
+		const int ox = (int)(t % p.oW);
+		t /= p.oW;
+		const int oy = (int)(t % p.oH);
+		const long b = t / p.oH;
+		int hs = oy * p.dH - p.padH, ws = ox * p.dW - p.padW;
+		const int he = min(hs + p.kH, p.H), we = min(ws + p.kW, p.W);
+		hs = max(hs, 0);
+		ws = max(ws, 0);
+		unsigned m[16];
+#pragma unroll
+		for (int k = 0; k < 16; k++)
+			m[k] = 0;
+		for (int yy = hs; yy < he; yy++)
+			for (int xx = ws; xx < we; xx++) {
+				const uintx4 v = x[((b * p.H + yy) * p.W + xx) * C16 + c16];
+#pragma unroll
+				for (int d = 0; d < 4; d++) {
+					m[4 * d] = max(m[4 * d], v[d] & 255u);
+					m[4 * d + 1] = max(m[4 * d + 1], (v[d] >> 8) & 255u);
+					m[4 * d + 2] = max(m[4 * d + 2], (v[d] >> 16) & 255u);
+					m[4 * d + 3] = max(m[4 * d + 3], v[d] >> 24);
+				}
+			}
+		uintx4 o;
+#pragma unroll
+		for (int d = 0; d < 4; d++)
+			o[d] = m[4 * d] | (m[4 * d + 1] << 8) | (m[4 * d + 2] << 16) | (m[4 * d + 3] << 24);
+		y[i] = o;
+	}
+}
+
 extern "C" void thhip_maxpool_u8_cl(const unsigned char *x, unsigned char *y, int B, int C, int H, int W, int oH, int oW,
 	int kH, int kW, int dH, int dW, int padH, int padW)
 {
 	if (C % 4)
 		THError("thhip_maxpool_u8_cl: C = %d is not a multiple of 4", C);
-	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * oH * oW * (C / 4) };
+	const int per = C % 16 == 0 && ((size_t)x & 15) == 0 && ((size_t)y & 15) == 0 ? 16 : 4;
+	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * oH * oW * (C / per) };
 	if (p.total <= 0)
 		return;
-	ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)B * C * H * W + 4.0 * p.total);
-	maxpool_u8_cl_kernel<<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>((const unsigned *)x, (unsigned *)y, p);
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)B * C * H * W + (double)per * p.total);
+	if (per == 16)
+		maxpool_u8_cl16_kernel<<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>((const uintx4 *)x, (uintx4 *)y, p);
+	else
+		maxpool_u8_cl_kernel<<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>((const unsigned *)x, (unsigned *)y, p);
 }
 
 /* Codes between plane-major [B][C][HW] and channels-last [B][HW][C] memory

@@ -8,11 +8,12 @@
  * With so few columns the product is bound by reading W once from HBM, like
  * the batch-1 matrix-vector kernel, but every weight is used B times, which is
  * exactly one 16x16x4 fp32 MFMA per 16 rows x 16 batch columns x 4 k.  A
- * wavefront owns 16 output rows and a slice of K: lane (m = lane%16,
- * q = lane/16) streams 64 contiguous bytes of row m per step (four 16-byte
- * loads, k = k0 + 16q + 4j + s), the matching lane of the B operand reads the
- * same k of batch row n = lane%16 (X is small and stays in L2), and 16 MFMAs
- * contract them.  K is split over the four wavefronts of a workgroup (summed
+ * wavefront owns 16 output rows and a slice of K: per step lane (m = lane%16,
+ * q = lane/16) issues four 16-byte loads of row m (k = k0 + 16j + 4q + s, so
+ * the four quarters of a load cover 64 adjacent bytes), the matching lane of
+ * the B operand reads the same k of batch row n = lane%16 (X is small and
+ * stays in L2), and 16 MFMAs contract them; the order of k inside a dot
+ * product is free as long as both operands use the same one.  K is split over the four wavefronts of a workgroup (summed
  * through LDS) and over gridDim.y workgroups (partials in a scratch buffer,
  * summed by a second tiny kernel that also applies bias and Threshold).
  */
@@ -20,22 +21,44 @@
 #include "thhip_internal.h"
 
 #define SK_THREADS 256
-#define SK_KSTEP 64
+#define SK_KBYTES 256	/* bytes of a weight row one K-step covers: 64 per lane quarter */
 
-template <int NB>	/* NB 16-column groups: batch <= 16 * NB */
-__global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const float *x, const float *w, float *part,
+/* One 16-byte vector of both operands -> MFMAs.  fp32: four 16x16x4 steps;
+ * half types: one 16x16x32, whose lane quarter q holds 8 consecutive k. */
+template <int DT> __device__ __forceinline__ void skinny_mma(floatx4 &acc, const floatx4 &a, const floatx4 &b);
+template <> __device__ __forceinline__ void skinny_mma<THHIP_F32>(floatx4 &acc, const floatx4 &a, const floatx4 &b)
+{
+#pragma unroll
+	for (int s = 0; s < 4; s++)
+		acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s], b[s], acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void skinny_mma<THHIP_F16>(floatx4 &acc, const floatx4 &a, const floatx4 &b)
+{
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
+}
+template <> __device__ __forceinline__ void skinny_mma<THHIP_BF16>(floatx4 &acc, const floatx4 &a, const floatx4 &b)
+{
+	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+
+template <int DT, int NB>	/* NB 16-column groups: batch <= 16 * NB */
+__global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const void *xv, const void *wv, float *part,
 	int B, int nIn, int nOut, int ksplit)
 {
+	typedef typename ThhipElem<DT>::T elem;
+	constexpr int VEC = 16 / (int)sizeof(elem);		/* elements per 16-byte vector */
+	constexpr int KSTEP = SK_KBYTES / (int)sizeof(elem);	/* k per step */
+	const elem *x = (const elem *)xv, *w = (const elem *)wv;
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int m = lane & 15, q = lane >> 4;
 	const int row0 = blockIdx.x * 16;
 	const int row = min(row0 + m, nOut - 1);
-	/* K-steps of 64 are dealt round-robin to (workgroup slice, wave) */
-	const int nsteps = (nIn + SK_KSTEP - 1) / SK_KSTEP;
+	/* K-steps are dealt round-robin to (workgroup slice, wave) */
+	const int nsteps = (nIn + KSTEP - 1) / KSTEP;
 	const int stride = ksplit * 4;
-	const float *wr = w + (size_t)row * nIn;
-	const float *xr[NB];
+	const elem *wr = w + (size_t)row * nIn;
+	const elem *xr[NB];
 #pragma unroll
 	for (int g = 0; g < NB; g++)
 		xr[g] = x + (size_t)min(g * 16 + m, B - 1) * nIn;
@@ -46,12 +69,13 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const float *x, cons
 		acc[g] = floatx4{ 0, 0, 0, 0 };
 
 	for (int st = blockIdx.y * 4 + wave; st < nsteps; st += stride) {
-		const int kb = st * SK_KSTEP + q * 16;
+		/* load j of the four lane quarters covers 64 adjacent bytes of a row */
+		const int kb = st * KSTEP + q * VEC;
 		floatx4 a[4], b[NB][4];
 #pragma unroll
 		for (int j = 0; j < 4; j++) {
-			const int k = kb + j * 4;
-			const bool ok = k < nIn;	/* nIn % 4 == 0: a vector is all in or all out */
+			const int k = kb + j * (4 * VEC);
+			const bool ok = k < nIn;	/* nIn % VEC == 0: a vector is all in or all out */
 			a[j] = ok ? *(const floatx4 *)(wr + k) : floatx4{ 0, 0, 0, 0 };
 #pragma unroll
 			for (int g = 0; g < NB; g++)
@@ -60,10 +84,8 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const float *x, cons
 #pragma unroll
 		for (int j = 0; j < 4; j++)
 #pragma unroll
-			for (int s = 0; s < 4; s++)
-#pragma unroll
-				for (int g = 0; g < NB; g++)
-					acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[j][s], b[g][j][s], acc[g], 0, 0, 0);
+			for (int g = 0; g < NB; g++)
+				skinny_mma<DT>(acc[g], a[j], b[g][j]);
 	}
 
 	/* D layout: lane holds column n = lane%16, rows 4*(lane/16) + r */
@@ -119,7 +141,32 @@ static float *skinny_scratch(size_t bytes)
 
 extern "C" int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtype)
 {
-	return dtype == THHIP_F32 && B >= 1 && B <= 32 && nIn % 4 == 0 && nIn >= 4 && nOut >= 1;
+	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
+		return 0;
+	const int vec = dtype == THHIP_F32 ? 4 : 8;
+	return B >= 1 && B <= 32 && nIn % vec == 0 && nIn >= vec && nOut >= 1;
+}
+
+template <int DT>
+static void skinny_launch(const void *x, const void *wrow, const float *bias, void *y, float *part,
+	int B, int nIn, int nOut, int groups, int ksplit, int act, float thr, float val)
+{
+	{
+		/* algorithmic bytes: W once, X once, Y once */
+		ThhipLaunchScope scope(THHIP_FAM_GEMV, (double)thhip_esize(DT) * ((double)nOut * nIn + (double)B * nIn + (double)B * nOut));
+		dim3 grid(groups, ksplit);
+		if (B <= 16)
+			skinny_kernel<DT, 1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+		else
+			skinny_kernel<DT, 2><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+	}
+	{
+		ThhipLaunchScope scope(THHIP_FAM_OTHER, 4.0 * (ksplit + 1.0) * B * nOut);
+		long total = (long)B * nOut;
+		long blocks = (total + 255) / 256;
+		skinny_finish_kernel<DT><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(part, bias, y, B, nOut,
+			ksplit, act, thr, val);
+	}
 }
 
 extern "C" void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
@@ -128,7 +175,8 @@ extern "C" void thhip_linear_batched(const void *x, const void *wrow, const floa
 	if (!thhip_linear_batched_supported(B, nIn, nOut, dtype))
 		THError("thhip_linear_batched: unsupported shape B=%d nIn=%d nOut=%d dtype=%d", B, nIn, nOut, dtype);
 	const int groups = (nOut + 15) / 16;
-	const int nsteps = (nIn + SK_KSTEP - 1) / SK_KSTEP;
+	const int kstep = SK_KBYTES / thhip_esize(dtype);
+	const int nsteps = (nIn + kstep - 1) / kstep;
 	/* aim at ~4096 wavefronts, at least two K-steps per wavefront */
 	int ksplit = (1024 + groups - 1) / groups;
 	if (ksplit > nsteps / 8)
@@ -138,24 +186,7 @@ extern "C" void thhip_linear_batched(const void *x, const void *wrow, const floa
 	if (ksplit > 64)
 		ksplit = 64;
 	float *part = skinny_scratch((size_t)ksplit * B * nOut * sizeof(float));
-	{
-		/* algorithmic bytes: W once, X once, Y once */
-		ThhipLaunchScope scope(THHIP_FAM_GEMV, 4.0 * ((double)nOut * nIn + (double)B * nIn + (double)B * nOut));
-		dim3 grid(groups, ksplit);
-		if (B <= 16)
-			skinny_kernel<1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>((const float *)x, (const float *)wrow, part,
-				B, nIn, nOut, ksplit);
-		else
-			skinny_kernel<2><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>((const float *)x, (const float *)wrow, part,
-				B, nIn, nOut, ksplit);
-	}
-	{
-		ThhipLaunchScope scope(THHIP_FAM_OTHER, 4.0 * (ksplit + 1.0) * B * nOut);
-		long total = (long)B * nOut;
-		long blocks = (total + 255) / 256;
-		skinny_finish_kernel<THHIP_F32><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(part, bias, y, B, nOut,
-			ksplit, act, thr, val);
-	}
+	THHIP_DISPATCH_FLOAT(dtype, skinny_launch<DT>(x, wrow, bias, y, part, B, nIn, nOut, groups, ksplit, act, thr, val));
 }
 
 /* ------------------------------------------------------------------ */
@@ -169,10 +200,9 @@ extern "C" void thhip_linear_batched(const void *x, const void *wrow, const floa
  * activations [B][K] -- and v_mfma_i32_32x32x32_i8 wants 16 consecutive k per
  * lane (lane = row or column lane%32, k half lane/32), so operands go from
  * global memory to the matrix core through registers only.  A K-step is 128
- * codes: lane (m, h) reads the 64 contiguous bytes k0 + 64h .. +63 of its row
- * as four 16-byte loads, and MFMA j contracts the 16-byte pieces j of both
- * halves; the order of k inside a dot product is free as long as both
- * operands use the same one.  Weights are stored re-centred (code - 128, done
+ * codes, four MFMAs of 32: for MFMA j lane (m, h) reads the 16 bytes
+ * k0 + 32j + 16h .. +15 of its row, so the two halves of a load are adjacent
+ * in memory.  Weights are stored re-centred (code - 128, done
  * once at pack time), activations are re-centred on the fly (x ^ 0x80).
  *
  * The four wavefronts of a workgroup own the same RG*32 rows and every fourth
@@ -200,10 +230,10 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_u8_kernel(const unsigned ch
 	const unsigned char *wr[RG], *xr[NB];
 #pragma unroll
 	for (int rg = 0; rg < RG; rg++)
-		wr[rg] = w + (size_t)min(row0 + rg * 32 + m, nOut - 1) * K + h * 64;
+		wr[rg] = w + (size_t)min(row0 + rg * 32 + m, nOut - 1) * K + h * 16;
 #pragma unroll
 	for (int g = 0; g < NB; g++)
-		xr[g] = x + (size_t)min(g * 32 + m, B - 1) * K + h * 64;
+		xr[g] = x + (size_t)min(g * 32 + m, B - 1) * K + h * 16;
 	intx16 acc[RG][NB];
 	int cs[NB];
 #pragma unroll
@@ -224,11 +254,11 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_u8_kernel(const unsigned ch
 	do {                                                                                   \
 		const int kk_ = (ST_) * SKU_KSTEP;                                             \
 		_Pragma("unroll") for (int j = 0; j < 4; j++) {                                \
-			const bool ok_ = kk_ + h * 64 + j * 16 < K;                            \
+			const bool ok_ = kk_ + j * 32 + h * 16 < K;                            \
 			_Pragma("unroll") for (int rg = 0; rg < RG; rg++)                      \
-				A_[rg][j] = ok_ ? *(const intx4 *)(wr[rg] + kk_ + j * 16) : zero_a; \
+				A_[rg][j] = ok_ ? *(const intx4 *)(wr[rg] + kk_ + j * 32) : zero_a; \
 			_Pragma("unroll") for (int g = 0; g < NB; g++)                         \
-				B_[g][j] = ok_ ? *(const intx4 *)(xr[g] + kk_ + j * 16) : zero_b;  \
+				B_[g][j] = ok_ ? *(const intx4 *)(xr[g] + kk_ + j * 32) : zero_b;  \
 		}                                                                              \
 	} while (0)
 
