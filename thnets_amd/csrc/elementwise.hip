@@ -592,7 +592,16 @@ __global__ void minmax_kernel(const float *x, long n, unsigned *out)
 		mn = fminf(mn, __shfl_xor(mn, off, 64));
 		mx = fmaxf(mx, __shfl_xor(mx, off, 64));
 	}
+	/* one pair of atomics per workgroup: they all hit the same two words */
+	__shared__ float smn[4], smx[4];
 	if ((threadIdx.x & 63) == 0) {
+		smn[threadIdx.x >> 6] = mn;
+		smx[threadIdx.x >> 6] = mx;
+	}
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		mn = fminf(fminf(smn[0], smn[1]), fminf(smn[2], smn[3]));
+		mx = fmaxf(fmaxf(smx[0], smx[1]), fmaxf(smx[2], smx[3]));
 		if (mn < 0)
 			atomicMax(&out[0], __float_as_uint(mn));
 		if (mx > 0)
@@ -615,8 +624,8 @@ extern "C" void thhip_quantize(const float *x, unsigned char *q, long n, float *
 	thhip_memcpy_h2d(d, bits, 8);
 	if (n > 0) {
 		long blocks = (n + 255) / 256;
-		if (blocks > 2048)
-			blocks = 2048;
+		if (blocks > 1024)
+			blocks = 1024;
 		ThhipLaunchScope scope(THHIP_FAM_OTHER, 4.0 * n);
 		minmax_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(x, n, d);
 	}
