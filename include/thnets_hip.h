@@ -485,6 +485,13 @@ void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wrow, 
 	const int *addend, unsigned char *y, int B, int K, int nOut,
 	int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val);
 
+/* Replaces Lowp_LoadImages (lowp_basic.c:60-131) for one image: interleaved
+ * 8-bit pixels (device copy, `stride` bytes per row, 3 planes) -> planar uint8
+ * codes [3][height][width] in the fixed input range the reference derives from
+ * mean / std; (*mult, *sub) receive that range's quantisation. */
+void thhip_rgb2code(unsigned char *dst, const unsigned char *src_dev, int width, int height, int stride,
+	const float *mean, const float *std, int bgr, float *mult, float *sub);
+
 /* Replaces Lowp_Threshold_updateOutput (lowp_Threshold.c:3-28) on codes. */
 void thhip_threshold_u8(const unsigned char *x, unsigned char *y, long n, int thr, int val, int inplace);
 

@@ -274,6 +274,51 @@ def test_engine_small_network_bit_exact_every_layer(hiplib, oracle):
     net.free()
 
 
+def _oracle_load_images(oracle, imgs, mean, std, bgr):
+    n, (H, W) = len(imgs), imgs[0].shape[:2]
+    dst = np.empty((n, 3, H, W), np.uint8)
+    ptrs = (C.c_void_p * n)(*[im.ctypes.data for im in imgs])
+    m, s = C.c_float(), C.c_float()
+    oracle.lib.orc_lowp_load_images(dst.ctypes.data_as(C.POINTER(C.c_ubyte)), ptrs, n, W, H, W * 3,
+                                    (C.c_float * 3)(*mean), (C.c_float * 3)(*std), bgr, C.byref(m), C.byref(s))
+    return dst, m.value, s.value
+
+
+def test_process_images_uint8_engine(hiplib, oracle):
+    """THProcessImages on the uint8 engine: the image loader's codes (fixed range from
+    mean / std, values outside 0..255 wrapping like the reference's build) bit for bit,
+    then the same network codes and de-quantised result as the restatement."""
+    g = cases.rng(1500)
+    mean, std = (0.485, 0.456, 0.406), (0.229, 0.224, 0.225)
+    imgs = [np.ascontiguousarray(g.integers(0, 256, (9, 11, 3), dtype=np.uint8)) for _ in range(3)]
+    for bgr in (0, 1):
+        want, wm, ws = _oracle_load_images(oracle, imgs, mean, std, bgr)
+        m, s_ = C.c_float(), C.c_float()
+        for i, im in enumerate(imgs):
+            dsrc = api.DeviceArray(hiplib, im)
+            ddst = api.DeviceArray(hiplib, nbytes=3 * 9 * 11)
+            hiplib.thhip_rgb2code(ddst.ptr, dsrc.ptr, 11, 9, 33, (C.c_float * 3)(*mean), (C.c_float * 3)(*std), bgr,
+                                  C.byref(m), C.byref(s_))
+            hiplib.thhip_sync()
+            assert np.array_equal(ddst.get((3, 9, 11), np.uint8), want[i]), (bgr, i)
+        assert (m.value, s_.value) == (wm, ws)
+    w1 = g.standard_normal((8, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+    w2 = g.standard_normal((5, 8, 2, 2), dtype=np.float32) * np.float32(0.3)
+    layers = [configs.conv(w1, g.standard_normal(8, dtype=np.float32) * np.float32(0.1), 1, 1), configs.relu(),
+              configs.maxpool(2, 2),
+              configs.conv(w2, g.standard_normal(5, dtype=np.float32) * np.float32(0.1), 1, 0), configs.relu()]
+    imgs = [np.ascontiguousarray(g.integers(0, 256, (8, 10, 3), dtype=np.uint8)) for _ in range(4)]
+    net = api.HipNetwork(layers, mean, std, lowp_range=16.0)
+    for bgr in (0, 1):
+        y = net.process_images(imgs, bgr=bgr)
+        xq, im_, isub = _oracle_load_images(oracle, imgs, mean, std, bgr)
+        outs = []
+        q, mo, so = oracle.lowp_run_layers(layers, xq, im_, isub, 16.0, collect=outs)
+        assert np.array_equal(net.module_output(4).astype(np.uint8), outs[4][0]), bgr
+        assert np.array_equal(y, oracle.lowp_dequantize(q, mo, so).ravel()), bgr
+    net.free()
+
+
 def _device_codes(hiplib, net, q):
     """uint8 codes -> a device tensor struct the engine accepts (test-side construction:
     storage marked as engine-owned device memory, extra reference so it is never freed

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(CONV_THREADS)
 /* ask for four waves per SIMD where the tile allows it: without the hint the
  * compiler spreads the accumulators over AGPRs plus a generous VGPR budget and
  * halves the number of workgroups a CU can hold */
-__attribute__((amdgpu_waves_per_eu(GM != GM_PLANE_TAP ? 4 : 1, 8))) void conv_mfma_kernel(ConvParams p)
+__attribute__((amdgpu_waves_per_eu(GM == GM_PLANE_TAP ? 1 : BM * BN >= 128 * 128 ? 2 : 4, 8))) void conv_mfma_kernel(ConvParams p)
 {
 	constexpr bool TAP = GM == GM_TAP_MAJOR;
 	constexpr bool C4 = GM == GM_PIXELS4;		/* uint8, <= 4 planes, re-laid out as [B][H][W][4] */

@@ -570,6 +570,60 @@ extern "C" void thhip_rgb2float(void *dst, const unsigned char *src, int width, 
 		dst, src, width, height, stride, cp, m, s, bgr)));
 }
 
+/* ---------------- 8-bit image -> planar uint8 codes (lowp/lowp_basic.c:60-131) ---------------- */
+
+__global__ void rgb2code_kernel(unsigned char *dst, const unsigned char *src, int width, int height, int stride,
+	int sub0, int sub1, int sub2, float mult0, float mult1, float mult2, int bgr)
+{
+	const long total = 3L * width * height;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total; i += step) {
+		const int j = (int)(i % width);
+		const long t = i / width;
+		const int r = (int)(t % height);
+		const int c = (int)(t / height);
+		const int sc = bgr ? 2 - c : c;
+		const int sub = c == 0 ? sub0 : c == 1 ? sub1 : sub2;
+		const float mult = c == 0 ? mult0 : c == 1 ? mult1 : mult2;
+		/* rgb2tensord, lowp_basic.c:68: integer difference, one float product,
+		 * roundf, then the conversion to a byte of the reference's x86 build
+		 * (through int, so values outside 0..255 wrap) */
+		const float v = roundf((float)((int)src[sc + 3 * j + (long)stride * r] - sub) * mult);
+		dst[i] = (unsigned char)(int)v;
+	}
+}
+
+/* One image of Lowp_LoadImages (lowp_basic.c:82-131): the fixed input range
+ * derived from mean / std gives the tensor's (mult, sub), returned through the
+ * pointers, and per-plane integer offsets and factors.  src is a device copy
+ * of the interleaved 8-bit image. */
+extern "C" void thhip_rgb2code(unsigned char *dst, const unsigned char *src, int width, int height, int stride,
+	const float *mean, const float *std, int bgr, float *mult_out, float *sub_out)
+{
+	int sub[3];
+	float mult[3], mn = 1e30, mx = -1e30, tmult;
+	for (int i = 0; i < 3; i++) {
+		if (-mean[i] / std[i] < mn)
+			mn = -mean[i] / std[i];
+		if ((1 - mean[i]) / std[i] > mx)
+			mx = (1 - mean[i]) / std[i];
+	}
+	tmult = (mx - mn) ? 255 / (mx - mn) : 0;
+	for (int i = 0; i < 3; i++) {
+		sub[i] = roundf(255 * (mean[i] + std[i] * mn));
+		mult[i] = tmult / (255 * std[i]);
+	}
+	const long total = 3L * width * height;
+	if (total > 0) {
+		ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * total);
+		rgb2code_kernel<<<ew_grid(total), dim3(EW_THREADS), 0, thhip_stream()>>>(dst, src, width, height, stride,
+			sub[0], sub[1], sub[2], mult[0], mult[1], mult[2], bgr);
+	}
+	*mult_out = tmult;
+	*sub_out = mn;
+}
+
 /* ---------------- uint8 quantise / de-quantise (lowp/lowp_basic.c:5-58) ---------------- */
 
 __global__ void minmax_kernel(const float *x, long n, unsigned *out)

@@ -173,6 +173,23 @@ static int finish(THNETWORK *network, THFloatTensor *out, float **result, int *o
 	return (int)THFloatTensor_nElement(out);
 }
 
+/* uint8 engine: runs a device tensor of codes whose quantisation is in
+ * hn->cur_mult / cur_sub, de-quantises the result (lowp_basic.c:40-58) and
+ * leaves it in network->out. */
+static THFloatTensor *run_codes(THNETWORK *network, THFloatTensor *q)
+{
+	struct hipnet *hn = (struct hipnet *)network->net;
+	THFloatTensor *out = thhip_forward(network->net, q);
+	THFloatTensor *f = device_tensor_like(out, THHIP_F32);
+	thhip_dequantize(thhip_tensor_ptr(out, THHIP_U8), f->storage->data, THFloatTensor_nElement(out),
+		hn->cur_mult, hn->cur_sub);
+	if (network->out)
+		THFloatTensor_free(network->out);
+	network->out = download_as_float(f, THHIP_F32);
+	THFloatTensor_free(f);
+	return network->out;
+}
+
 /* Runs a device tensor of floats (engine dtype for ENGINE_HIP, fp32 for the
  * uint8 engine, which quantises it first) and leaves the float result in
  * network->out. */
@@ -182,19 +199,12 @@ static THFloatTensor *run_float_input(THNETWORK *network, THFloatTensor *dev_in)
 	THFloatTensor *out;
 	if (network->net->engine == ENGINE_HIPLOWP) {
 		/* THLowpTensor_newFromFloatTensor on the whole batch (one min/max),
-		 * lowp_basic.c:15-35, then de-quantise the result, :40-58 */
+		 * lowp_basic.c:15-35 */
 		const long cnt = THFloatTensor_nElement(dev_in);
 		THFloatTensor *q = device_tensor_like(dev_in, THHIP_U8);
 		thhip_quantize((const float *)thhip_tensor_ptr(dev_in, THHIP_F32), (unsigned char *)q->storage->data, cnt,
 			&hn->cur_mult, &hn->cur_sub);
-		out = thhip_forward(network->net, q);
-		THFloatTensor *f = device_tensor_like(out, THHIP_F32);
-		thhip_dequantize(thhip_tensor_ptr(out, THHIP_U8), f->storage->data, THFloatTensor_nElement(out),
-			hn->cur_mult, hn->cur_sub);
-		if (network->out)
-			THFloatTensor_free(network->out);
-		network->out = download_as_float(f, THHIP_F32);
-		THFloatTensor_free(f);
+		run_codes(network, q);
 		THFloatTensor_free(q);
 	} else {
 		out = thhip_forward(network->net, dev_in);
@@ -243,8 +253,33 @@ int THProcessImages(THNETWORK *network, unsigned char **images, int batchsize, i
 	int cp = 3;
 	if (stride < width * 3)
 		cp = 1;	/* thapi.c:458-459 */
-	if (engine == ENGINE_HIPLOWP)
-		THError("THProcessImages is not implemented for the uint8 HIP engine; use THProcessFloat");
+	if (engine == ENGINE_HIPLOWP) {
+		/* thapi.c:485-487, 551-558: Lowp_LoadImages (always three planes, always
+		 * 4-D), forward, de-quantise */
+		THFloatTensor *q = THFloatTensor_new();
+		q->storage = malloc(sizeof(*q->storage));
+		q->storage->nref = 1;
+		q->storage->mustfree = TH_MUSTFREE_HIP;
+		q->storage->data = thhip_malloc((size_t)batchsize * 3 * width * height);
+		unsigned char *staging = thhip_malloc((size_t)stride * height);
+		for (int i = 0; i < batchsize; i++) {
+			thhip_memcpy_h2d(staging, images[i], (size_t)stride * height);
+			thhip_rgb2code((unsigned char *)q->storage->data + (size_t)i * 3 * width * height, staging, width, height,
+				stride, network->mean, network->std, bgr, &hn->cur_mult, &hn->cur_sub);
+		}
+		thhip_sync();
+		thhip_free(staging);
+		long s4[4] = { batchsize, 3, height, width };
+		q->nDimension = 4;
+		long st = 1;
+		for (int i = 3; i >= 0; st *= s4[i], i--) {
+			q->size[i] = s4[i];
+			q->stride[i] = st;
+		}
+		THFloatTensor *out = run_codes(network, q);
+		THFloatTensor_free(q);
+		return finish(network, out, results, outwidth, outheight);
+	}
 	const int dt = hn->dtype;
 	const size_t esz = dt == THHIP_F32 ? 4 : 2;
 	THFloatTensor *t = THFloatTensor_new();
