@@ -177,6 +177,21 @@ def main():
         "workload": "AlexNet-OWT fp32 batch 1 (BASELINE configs[1])"}
     n2.free()
 
+    # ---- ResNet-18 fp32 batch 32 (1x1 projections, batch norm folded into the conv epilogue) ----
+    c4 = configs.resnet18(batch=32)
+    n4 = api.HipNetwork(c4["layers"], c4["mean"], c4["std"])
+    x4 = c4["input"].copy()
+    for c in range(3):
+        x4[:, c] = (x4[:, c] - np.float32(c4["mean"][c])) / np.float32(c4["std"][c])
+    n4.upload(x4)
+    ms4, fam4 = timed_forward(lib, n4, max(args.steps, 20), args.warmup, (0, 1, 3), profiled=False)
+    cv_ms, cv_n, cv_fl = fam4[0]
+    extra["resnet18_fp32_b32"] = {
+        "images_per_sec": round(32.0 / (ms4 * 1e-3), 1), "ms_per_step": round(ms4, 4),
+        "conv_TFLOP/s": round(cv_fl / (cv_ms * 1e-3) / 1e12, 2) if cv_ms > 0 else None,
+        "workload": "ResNet-18 shape fp32 batch 32 (BASELINE configs[3]), residual add with the reference's a - b arithmetic"}
+    n4.free()
+
     # ---- uint8 AlexNet-OWT batch 64 ----
     if not args.no_int8:
         c5 = configs.alexnet_lowp(batch=64)

@@ -273,6 +273,12 @@ THNETWORK *THCreateHipNetwork(THNETWORK *net);
  * 1 = fp16 storage + fp16 MFMA, 2 = bf16 storage + bf16 MFMA.  Read at
  * engine creation.  Returns 0, or ERR_NOTIMPLEMENTED for other values. */
 int THHipHalfFloat(int enable);
+/* 1 (default): SpatialBatchNormalization directly after a convolution is folded
+ * into the convolution's epilogue at engine creation (the reference folds at
+ * load time, absorb_bn, onnx.cc:472-570); 0: it runs as its own kernel like
+ * nn_SpatialBatchNormalization_updateOutput.  Applies to engines created
+ * afterwards; returns the previous setting. */
+int THHipFoldBatchNorm(int enable);
 /* New: the uint8 engine on the GPU, counterpart of THCreateLowpNetwork
  * (thapi.c:784-796, lowp_basic.c:133-212): activations quantised to
  * [-range/2, range/2) in 255 steps, int8 MFMA GEMM with gemmlowp offsets
@@ -348,6 +354,16 @@ void *thhip_conv_unpack_rows(const void *wpacked, int Co, int Ci, int kHW, int d
  * x: [B,Ci,H,W], y: [B,Co,oH,oW], both NCHW contiguous in `dtype`;
  * wpacked from thhip_conv_pack_weight; bias fp32 [Co] or NULL. */
 void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype);
+
+/* The same convolution with a per-plane factor before the bias:
+ *     y = act(scale[o] * sum + shift[o]),
+ * which is a convolution followed by SpatialBatchNormalization with
+ * scale = invstd * weight and shift = (bias - mean) * scale + bn_bias
+ * (SpatialBatchNormalization.c:57-116; the reference's own folding is
+ * absorb_bn, onnx.cc:529-557).  scale == NULL is thhip_conv2d. */
+void thhip_conv2d_affine(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype);
 

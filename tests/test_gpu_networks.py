@@ -16,7 +16,7 @@ GOLD = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"
 NET_TOL = 1e-4      # contract: 1e-3 * max|ref| per layer output
 
 
-def layerwise(net, oracle, cfg, tol):
+def layerwise(net, oracle, cfg, tol, folded_bn=True):
     x = oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])
     outs = []
     oracle.run_layers(cfg["layers"], x, collect=outs)
@@ -27,7 +27,13 @@ def layerwise(net, oracle, cfg, tol):
         want = o
         # a Threshold folded into its producer: the producer's buffer holds the thresholded values
         # (or applied in place on the producer's buffer)
-        if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold" and (
+        # a batch norm folded into the convolution before it: the convolution's buffer holds the
+        # normalised values (and the threshold's, if one follows the batch norm)
+        if folded_bn and layers[i]["type"] == "conv" and i + 1 < len(layers) and layers[i + 1]["type"] == "bn":
+            want = outs[i + 1]
+            if i + 2 < len(layers) and layers[i + 2]["type"] == "threshold":
+                want = outs[i + 2]
+        elif i + 1 < len(layers) and layers[i + 1]["type"] == "threshold" and (
                 layers[i]["type"] in ("conv", "linear", "caddtable") or layers[i + 1].get("inplace", 1) == 1):
             want = outs[i + 1]
         G.assert_close(net.module_output(i).ravel(), np.asarray(want).ravel(), tol, "module %d %s" % (i, layers[i]["type"]))
@@ -46,6 +52,30 @@ def test_small_networks_vs_oracle_and_golden(hiplib, oracle, name):
     # repeated calls are stable
     assert np.array_equal(net.process_float(cfg["input"]), y)
     net.free()
+
+
+def test_batchnorm_folding_on_and_off(hiplib, oracle):
+    """A batch norm after a convolution runs in the convolution's epilogue by default
+    and as its own kernel with THHipFoldBatchNorm(0); both match the restatement layer
+    by layer, the unfolded one as closely as any other fp32 path."""
+    cfg = cases.small_networks()["resnet18_small"]
+    for fold in (True, False):
+        net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"], fold_bn=fold)
+        y = net.process_float(cfg["input"])
+        G.assert_close(y, GOLD["net_resnet18_small"], NET_TOL, "golden fold=%s" % fold)
+        layerwise(net, oracle, cfg, NET_TOL, folded_bn=fold)
+        net.free()
+    # a stand-alone conv -> bn -> relu chain with awkward planes, against the double-checked layers
+    g = cases.rng(1600)
+    w = g.standard_normal((70, 5, 3, 3), dtype=np.float32) * np.float32(0.2)
+    layers = [configs.conv(w, g.standard_normal(70, dtype=np.float32), 1, 1), configs._bn(g, 70), configs.relu(),
+              configs.maxpool(2, 2)]
+    x = g.standard_normal((3, 5, 10, 12), dtype=np.float32)
+    want = oracle.run_layers(layers, x)
+    for fold in (True, False):
+        net = api.HipNetwork(layers, fold_bn=fold)
+        G.assert_close(net.process_float(x), want.ravel(), NET_TOL, "conv-bn-relu fold=%s" % fold)
+        net.free()
 
 
 def test_process_float_normalises_callers_buffer_in_place(hiplib, oracle):

@@ -52,6 +52,7 @@ PROTOTYPES = {
     "THLastError": (C.c_int, []),
     "THCreateHipNetwork": (vp, [vp]),
     "THHipHalfFloat": (C.c_int, [C.c_int]),
+    "THHipFoldBatchNorm": (C.c_int, [C.c_int]),
     "THCreateHipLowpNetwork": (vp, [vp, C.c_float]),
     "THHipTensor_newFromFloatTensor": (vp, [vp]),
     "THFloatTensor_newFromHipTensor": (vp, [vp]),
@@ -77,6 +78,7 @@ PROTOTYPES = {
     "thhip_conv_packed_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv_unpack_rows": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
+    "thhip_conv2d_affine": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_linear_batched_supported": (C.c_int, [C.c_int] * 4),
@@ -196,7 +198,7 @@ class HipNetwork:
     """A network on the engine, made from a layer list (see netbuild)."""
 
     def __init__(self, layers, mean=(0.0, 0.0, 0.0), std=(1.0, 1.0, 1.0), half=0, lowp_range=None,
-                 make_spatial=None):
+                 make_spatial=None, fold_bn=True):
         self.lib = lib = load_library()
         lib.THInit()
         self.host = HostNetwork(lib, abi.ABI, resolve_cpu=False).build(layers, mean, std)
@@ -210,7 +212,9 @@ class HipNetwork:
         else:
             if lib.THHipHalfFloat(half) != 0:
                 raise ValueError("THHipHalfFloat(%r) refused" % half)
+            old_fold = lib.THHipFoldBatchNorm(1 if fold_bn else 0)
             self.handle = lib.THCreateHipNetwork(C.addressof(self.host.thnet))
+            lib.THHipFoldBatchNorm(old_fold)
             lib.THHipHalfFloat(0)
             self.dtype = (abi.THHIP_F32, abi.THHIP_F16, abi.THHIP_BF16)[half]
         self.thnet = C.cast(self.handle, C.POINTER(abi.ABI.THNETWORK)).contents

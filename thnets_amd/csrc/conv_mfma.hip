@@ -38,6 +38,7 @@ struct ConvParams {
 	const void *x;
 	const void *wp;
 	const float *bias;
+	const float *scale;	/* float types: per-plane factor applied before the bias (folded batch norm), or NULL */
 	void *y;
 	int B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, oH, oW;
 	int K, KC, N, oHW, HW, kHW;
@@ -553,8 +554,11 @@ __attribute__((amdgpu_waves_per_eu(GM == GM_PLANE_TAP ? 1 : BM * BN >= 128 * 128
 			/* (128+b_off) rowsum + K (128+a_off)(128+b_off) */
 			lrow[tid] = p.offB * p.rowsum[mc] + p.K * p.offA * p.offB;
 			lrow[BM + tid] = p.addend ? p.addend[mc] : 0;
-		} else
+		} else {
 			lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+			if (p.scale)
+				lrow[BM + tid] = __float_as_int(p.scale[mc]);
+		}
 	}
 	if constexpr (DT != THHIP_U8)
 		__syncthreads();
@@ -684,7 +688,8 @@ __attribute__((amdgpu_waves_per_eu(GM == GM_PLANE_TAP ? 1 : BM * BN >= 128 * 128
 			}
 		}
 	} else {
-		/* bias, optional threshold, store */
+		/* (folded batch norm factor,) bias, optional threshold, store */
+		const bool has_scale = p.scale != 0;
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
 			const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
@@ -698,11 +703,15 @@ __attribute__((amdgpu_waves_per_eu(GM == GM_PLANE_TAP ? 1 : BM * BN >= 128 * 128
 #pragma unroll
 				for (int g = 0; g < 4; g++) {
 					struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
-					const floatx4 rowbias = *(const floatx4 *)(lrow + (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g);
+					const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
+					const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+					floatx4 rowscale = { 1, 1, 1, 1 };
+					if (has_scale)
+						rowscale = *(const floatx4 *)(lrow + BM + ml);
 #pragma unroll
 					for (int e = 0; e < 4; e++) {
 						const int r = 4 * g + e, m = m0 + 8 * g + e;
-						float v = acc[i][j][r] + rowbias[e];
+						float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
 						if (p.act)
 							v = v > p.thr ? v : p.val;
 						if constexpr (!CLO) {
@@ -1060,7 +1069,7 @@ static unsigned char *conv_pixels4_scratch(size_t bytes)
 	return g_c4;
 }
 
-static void conv_run(const void *x, const void *wpacked, const float *bias, void *y,
+static void conv_run(const void *x, const void *wpacked, const float *scale, const float *bias, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, const ConvU8Args *u8)
 {
@@ -1093,6 +1102,7 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 		p.y = (char *)y + (size_t)b0 * out_img * esize;
 		p.wp = wpacked;
 		p.bias = bias;
+		p.scale = scale;
 		p.B = bn; p.Ci = Ci; p.H = H; p.W = W; p.Co = Co; p.kH = kH; p.kW = kW;
 		p.dH = dH; p.dW = dW; p.padH = padH; p.padW = padW; p.oH = oH; p.oW = oW;
 		p.K = (int)K;
@@ -1156,13 +1166,20 @@ static void conv_run(const void *x, const void *wpacked, const float *bias, void
 	}
 }
 
-extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,
+extern "C" void thhip_conv2d_affine(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype)
 {
 	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
 		THError("thhip_conv2d: unsupported dtype %d", dtype);
-	conv_run(x, wpacked, bias, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0);
+	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0);
+}
+
+extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype)
+{
+	thhip_conv2d_affine(x, wpacked, 0, bias, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype);
 }
 
 /* uint8 codes [Co][Ci][kH][kW] -> (code - 128) as signed bytes in the packed
@@ -1210,7 +1227,7 @@ extern "C" void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpack
 		THError("thhip_conv2d_u8: shift %d out of range", c_shift);
 	ConvU8Args u8 = { addend, zero & 255, a_off, b_off, c_off, c_mult, c_shift, thr, val,
 		x_layout, y_channels_last != 0 };
-	conv_run(x, wpacked, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
+	conv_run(x, wpacked, 0, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
 }
 
 extern "C" void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,

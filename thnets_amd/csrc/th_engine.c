@@ -34,6 +34,19 @@ int THHipHalfFloat(int enable)
 	return 0;
 }
 
+static int g_fold_bn = 1;
+
+/* 1 (default): a SpatialBatchNormalization that directly follows a convolution
+ * is folded into that convolution's epilogue when the engine is created;
+ * 0: it runs as its own kernel, as in the reference's CPU path.  Returns the
+ * previous setting. */
+int THHipFoldBatchNorm(int enable)
+{
+	const int old = g_fold_bn;
+	g_fold_bn = enable != 0;
+	return old;
+}
+
 int thhip_engine_dtype(void)
 {
 	return g_halfmode == 1 ? THHIP_F16 : g_halfmode == 2 ? THHIP_BF16 : THHIP_F32;
@@ -156,7 +169,7 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 	void *y = conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
 	const int K = c->nInputPlane * c->kH * c->kW;
 	const int one_position = oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W;
-	if (one_position && (s.B == 1 || thhip_linear_batched_supported(s.B, K, c->nOutputPlane, dt))) {
+	if (one_position && !hm->scale && (s.B == 1 || thhip_linear_batched_supported(s.B, K, c->nOutputPlane, dt))) {
 		/* one output position per image: a matrix-vector (or skinny matrix)
 		 * product over the flattened input, bound by reading the weights once */
 		if (!hm->wrow)
@@ -167,7 +180,7 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 			thhip_linear_batched(x, hm->wrow, hm->bias, y, s.B, K, c->nOutputPlane, hm->fused_act, hm->thr,
 				hm->val, dt);
 	} else
-		thhip_conv2d(x, hm->wpacked, hm->bias, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+		thhip_conv2d_affine(x, hm->wpacked, hm->scale, hm->bias, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
 			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, hm->fused_act, hm->thr, hm->val, dt);
 	return m->output;
 }
@@ -286,6 +299,10 @@ static THFloatTensor *Hip_SpatialBatchNormalization_updateOutput(struct module *
 {
 	struct hipnet *hn = hipnet_of(m);
 	struct hipmod *hm = hipmod_of(m);
+	if (hm->passthrough) {	/* folded into the convolution before it */
+		out_alias(m, in);
+		return m->output;
+	}
 	if (in->nDimension != 3 && in->nDimension != 4)
 		THError("SpatialBatchNormalization: 3D or 4D tensor expected");
 	const long B = in->nDimension == 4 ? in->size[0] : 1;
@@ -919,16 +936,53 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 	hn->range = range;
 	for (int i = 0; i < net->nelem; i++)
 		convert_module(hn, net, i, engine, dtype, range);
+	/* fold a SpatialBatchNormalization into the convolution that feeds it:
+	 * ((sum + cb - mean) * invstd) * w + b  =  sum * s + ((cb - mean) * s + b),  s = invstd * w
+	 * (SpatialBatchNormalization.c:57-116; the reference's loader-side folding is absorb_bn, onnx.cc:529-557) */
+	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIP && g_fold_bn; i++) {
+		struct module *m = &hn->pub.modules[i], *sb = &net->modules[i + 1];
+		if (!is_conv_type(m->type) || hn->hm[i].is_linear || sb->type != MT_SpatialBatchNormalization)
+			continue;
+		struct SpatialBatchNormalization *bn = &sb->SpatialBatchNormalization;
+		const int Co = m->SpatialConvolution.nOutputPlane;
+		if (THFloatTensor_nElement(bn->running_mean) != Co)
+			continue;	/* the mismatch is reported when the network runs */
+		const float *mean = THFloatTensor_data(bn->running_mean), *var = THFloatTensor_data(bn->running_var);
+		const float *w = contiguous_host_floats(bn->weight, "batchnorm weight", Co) ? THFloatTensor_data(bn->weight) : 0;
+		const float *b = contiguous_host_floats(bn->bias, "batchnorm bias", Co) ? THFloatTensor_data(bn->bias) : 0;
+		THFloatTensor *cbt = net->modules[i].SpatialConvolution.bias;
+		const float *cb = contiguous_host_floats(cbt, "convolution bias", Co) ? THFloatTensor_data(cbt) : 0;
+		float *scale = malloc(sizeof(float) * Co), *shift = malloc(sizeof(float) * Co);
+		for (int o = 0; o < Co; o++) {
+			const float invstd = 1 / sqrt(var[o] + bn->eps);
+			scale[o] = w ? invstd * w[o] : invstd;
+			shift[o] = ((cb ? cb[o] : 0) - mean[o]) * scale[o] + (b ? b[o] : 0);
+		}
+		thhip_free(hn->hm[i].bias);
+		hn->hm[i].scale = thhip_malloc(sizeof(float) * Co);
+		hn->hm[i].bias = thhip_malloc(sizeof(float) * Co);
+		thhip_memcpy_h2d(hn->hm[i].scale, scale, sizeof(float) * Co);
+		thhip_memcpy_h2d(hn->hm[i].bias, shift, sizeof(float) * Co);
+		free(scale);
+		free(shift);
+		hn->hm[i + 1].passthrough = 1;
+	}
 	/* fold a Threshold into the epilogue of the module that feeds it */
 	for (int i = 0; i + 1 < net->nelem; i++) {
-		struct module *m = &hn->pub.modules[i], *t = &hn->pub.modules[i + 1];
+		struct module *m = &hn->pub.modules[i];
+		int ti = i + 1;
+		if (hn->hm[ti].passthrough && hn->pub.modules[ti].type == MT_SpatialBatchNormalization && ti + 1 < net->nelem)
+			ti++;	/* conv -> (folded BN) -> Threshold */
+		struct module *t = &hn->pub.modules[ti];
 		if (!foldable_threshold(t))
 			continue;
 		if (is_conv_type(m->type)) {
 			hn->hm[i].fused_act = 1;
 			hn->hm[i].thr = t->Threshold.threshold;
 			hn->hm[i].val = t->Threshold.val;
-			hn->hm[i + 1].passthrough = 1;
+			hn->hm[ti].passthrough = 1;
+		} else if (ti != i + 1) {
+			continue;
 		} else if ((m->type == MT_CAddTable || m->type == MT_CSubTable) &&
 			t->Threshold.threshold == 0 && t->Threshold.val == 0) {
 			hn->hm[i].fused_act = 1;
@@ -963,6 +1017,7 @@ void thhip_free_network(struct network *net)
 		thhip_free(hm->wpacked);
 		thhip_free(hm->wrow);
 		thhip_free(hm->bias);
+		thhip_free(hm->scale);
 		thhip_free(hm->addend);
 		thhip_free(hm->wrow_u8);
 		thhip_free(hm->rowsum_u8);

@@ -16,6 +16,7 @@ struct hipmod {
 	void *wpacked;		/* convolution weights in the kernel's packed layout (device) */
 	void *wrow;		/* the same weights row-major, made on first matrix-vector use (device) */
 	float *bias;		/* fp32 bias (device) */
+	float *scale;		/* fp32 per-plane factor of a folded batch norm, applied before the bias (device), or NULL */
 	float *bn[4];		/* mean, invstd, weight, bias per plane (device) */
 	long bn_planes;
 	/* uint8 engine */
