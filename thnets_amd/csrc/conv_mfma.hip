@@ -73,7 +73,21 @@ static inline unsigned long long conv_magic(unsigned d)
  * an fp32 one retires 1, so where the gather is cheap (channels-last codes)
  * deeper K-tiles keep the work per barrier up. */
 #define CONV_KCH_U8_CL 2
-__host__ __device__ constexpr int conv_kch(int dtype, bool x_cl) { return dtype == THHIP_U8 && x_cl ? CONV_KCH_U8_CL : 2; }
+#define CONV_KCH_F32 4
+__host__ __device__ constexpr int conv_kch(int dtype, bool x_cl)
+{
+	return dtype == THHIP_U8 && x_cl ? CONV_KCH_U8_CL : dtype == THHIP_F32 ? CONV_KCH_F32 : 2;
+}
+
+/* Waves per SIMD to ask the register allocator for (what each tile reaches
+ * without spilling): more for the small tiles, whose residency matters most. */
+__host__ __device__ constexpr int conv_min_waves(int dtype, int tile_elems, bool generic_gather)
+{
+	return generic_gather ? 1
+		: tile_elems <= 64 * 64 ? (dtype == THHIP_F32 ? 3 : 4)
+		: tile_elems <= 128 * 64 ? (dtype == THHIP_F32 ? 2 : 4)
+		: (dtype == THHIP_F32 ? 1 : 2);
+}
 
 template <int DT> struct ConvTraits;
 template <> struct ConvTraits<THHIP_F32> {
@@ -166,7 +180,7 @@ __global__ __launch_bounds__(CONV_THREADS)
 /* ask for four waves per SIMD where the tile allows it: without the hint the
  * compiler spreads the accumulators over AGPRs plus a generous VGPR budget and
  * halves the number of workgroups a CU can hold */
-__attribute__((amdgpu_waves_per_eu(GM == GM_PLANE_TAP ? 1 : BM * BN >= 128 * 128 ? 2 : 4, 8))) void conv_mfma_kernel(ConvParams p)
+__attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) void conv_mfma_kernel(ConvParams p)
 {
 	constexpr bool TAP = GM == GM_TAP_MAJOR;
 	constexpr bool C4 = GM == GM_PIXELS4;		/* uint8, <= 4 planes, re-laid out as [B][H][W][4] */
@@ -974,23 +988,17 @@ static void conv_dispatch(ConvParams &p)
 	 * keeps its four matrix cores nearly as busy as a bigger one, and small
 	 * tiles quantise best: the hardware packs the workgroups of a grid's last,
 	 * partially filled round onto as few CUs as they fit, so a round costs
-	 * (residents per CU) x (tile time) even when nearly empty.  Only the
-	 * widest layers (>= 700 tiles of 128x128) gain from the 128-row tile's
-	 * operand reuse.  Splitting K is available (thhip_conv_set_tuning) but
-	 * measured slower than unsplit 64x64 tiles on every layer shape tried, so
-	 * it is never chosen. */
+	 * (residents per CU) x (tile time) even when nearly empty.  fp32 (K-tiles
+	 * of 32) and uint8 (int8 MFMAs outrun LDS at any of these sizes, so the
+	 * tile with the most workgroups in flight wins) always take 64x64; the
+	 * half types take 128x64 on the widest layers (>= 700 tiles of 128x128)
+	 * for its operand reuse.  Splitting K is available (thhip_conv_set_tuning)
+	 * but measured slower than unsplit 64x64 tiles on every layer shape tried,
+	 * so it is never chosen; so is a cap on the workgroups per CU. */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
-	int bm, bn, splitk = 1, wgs = 0;
-	if (DT == THHIP_U8) {
-		/* int8 MFMAs outrun LDS at any of these tile sizes; the smallest
-		 * tile has the most workgroups in flight and measured fastest */
-		bm = 64; bn = 64;
-	} else if (p.Co > 64 && t128 >= 700) {
-		bm = 128; bn = 64;
-	} else {
-		bm = 64; bn = 64;
-		wgs = p.Co <= 64 ? 0 : 4;
-	}
+	int bm = 64, bn = 64, splitk = 1, wgs = 0;
+	if ((DT == THHIP_F16 || DT == THHIP_BF16) && p.Co > 64 && t128 >= 700)
+		bm = 128;
 	if (g_force_bm)
 		bm = g_force_bm;
 	if (g_force_bn)
@@ -1291,9 +1299,9 @@ extern "C" void lowpgemm(const int is_a_transposed, const int is_b_transposed, c
  * used when a layer turns out to be a matrix-vector product (one output
  * position). */
 template <typename E>
-__global__ void conv_unpack_rows_kernel(const E *wp, E *rows, int Co, int Ci, int kHW, int KC, int chunk, int tapmajor)
+__global__ void conv_unpack_rows_kernel(const E *wp, E *rows, int Co, int Ci, int kHW, int KC, int chunk, int kch, int tapmajor)
 {
-	const int K = Ci * kHW, vec = chunk / 2, cb = 2 * chunk;
+	const int K = Ci * kHW, vec = chunk / 2, cb = kch * chunk;
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
 	const long total = (long)Co * K, step = (long)gridDim.x * blockDim.x;
 	for (; i < total; i += step) {
@@ -1319,10 +1327,10 @@ extern "C" void *thhip_conv_unpack_rows(const void *wpacked, int Co, int Ci, int
 		blocks = 65536;
 	if (dtype == THHIP_F32)
 		conv_unpack_rows_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
-			(const float *)wpacked, (float *)rows, Co, Ci, kHW, KC, chunk, tm);
+			(const float *)wpacked, (float *)rows, Co, Ci, kHW, KC, chunk, conv_kch(dtype, false), tm);
 	else if (dtype == THHIP_F16 || dtype == THHIP_BF16)
 		conv_unpack_rows_kernel<unsigned short><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(
-			(const unsigned short *)wpacked, (unsigned short *)rows, Co, Ci, kHW, KC, chunk, tm);
+			(const unsigned short *)wpacked, (unsigned short *)rows, Co, Ci, kHW, KC, chunk, conv_kch(dtype, false), tm);
 	else
 		THError("thhip_conv_unpack_rows: unsupported dtype %d", dtype);
 	hipcheck(hipGetLastError());
