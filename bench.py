@@ -161,6 +161,18 @@ def main():
     extra["vgg16_THProcessFloat_images_per_sec_pcie_inclusive"] = round(16 * 5 / (time.perf_counter() - t0), 1)
     net.free()
 
+    # ---- VGG-16 fp16 batch 16 (THHipHalfFloat(1): fp16 storage and MFMA, fp32 accumulation) ----
+    nh = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"], half=1)
+    nh.upload(cfg["input"])
+    msh, famh = timed_forward(lib, nh, args.steps, args.warmup, (0, 1, 3), profiled=False)
+    hc_ms, hc_n, hc_fl = famh[0]
+    extra["vgg16_fp16_b16"] = {
+        "images_per_sec": round(16.0 / (msh * 1e-3), 1), "ms_per_step": round(msh, 4),
+        "conv_TFLOP/s": round(hc_fl / (hc_ms * 1e-3) / 1e12, 1) if hc_ms > 0 else None,
+        "frac_of_fp16_mfma_peak": round(hc_fl / (hc_ms * 1e-3) / 1e12 / 2500.0, 4) if hc_ms > 0 else None,
+        "workload": "VGG-16 shape, fp16 storage and MFMA, batch 16 (BASELINE configs[2], fp16 leg)"}
+    nh.free()
+
     # ---- AlexNet-OWT fp32 batch 1 (GEMV-bound Linear layers) ----
     c2 = configs.alexnet_owt()
     n2 = api.HipNetwork(c2["layers"], c2["mean"], c2["std"])
