@@ -367,6 +367,18 @@ void thhip_conv2d_affine(const void *x, const void *wpacked, const float *scale,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype);
 
+/* Half types (fp16 / bf16) with the memory order chosen per side, as for the
+ * uint8 entry points below: x_layout 0 = the reference's [B][C][H][W],
+ * 1 = channels-last [B][H][W][C] (Ci % 8 == 0; weights packed with
+ * thhip_conv_pack_weight_layout for it); y_channels_last likewise (Co % 4 == 0).
+ * The half engines keep activations channels-last between convolutions so
+ * that the eight values of one MFMA operand vector are one 16-byte load.
+ * Same arithmetic and reference lines as thhip_conv2d_affine. */
+void *thhip_conv_pack_weight_layout(const float *w_host, int Co, int Ci, int kH, int kW, int dtype, int x_layout);
+void thhip_conv2d_layout(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype, int x_layout, int y_channels_last);
+
 /* Tuning override for experiments: force the convolution's workgroup tile
  * (bm x bn in {64,128}), its split-K factor and the number of workgroups
  * allowed to share a CU; 0 leaves a choice automatic. */
@@ -485,6 +497,12 @@ void thhip_maxpool_u8_cl(const unsigned char *x, unsigned char *y, int B, int C,
  * back (0).  No counterpart in the reference, whose tensors are always
  * plane-major; used where the engine's internal order meets the API. */
 void thhip_relayout_u8(const unsigned char *x, unsigned char *y, int B, int C, int HW, int to_channels_last);
+/* The same for any element type of the engine (dtype gives the element size),
+ * and max pooling on channels-last tensors of the half types (C % 8 == 0) or
+ * codes (SpatialMaxPooling.c:168-247 / lowp_SpatialMaxPooling.c:45-108). */
+void thhip_relayout(const void *x, void *y, int B, int C, int HW, int to_channels_last, int dtype);
+void thhip_maxpool_cl(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype);
 
 /* The same arithmetic as thhip_conv2d_u8 for layers with one output position
  * per image (Linear, or a window covering its whole input): x [B][K] codes,

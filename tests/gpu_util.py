@@ -32,6 +32,31 @@ def conv2d(lib, x, w, bias, d=(1, 1), pad=(0, 0), act=0, thr=0.0, val=0.0, dtype
     return y
 
 
+def conv2d_layout(lib, x, w, bias, d=(1, 1), pad=(0, 0), act=0, thr=0.0, val=0.0, dtype=F16, x_cl=0, y_cl=0, scale=None):
+    """Half-type convolution with the device tensors channels-last on either side;
+    x and the result are [B][C][H][W] arrays."""
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    B, Ci, H, W = x.shape
+    Co, _, kH, kW = w.shape
+    oH, oW = (H + 2 * pad[0] - kH) // d[0] + 1, (W + 2 * pad[1] - kW) // d[1] + 1
+    note("conv2d_layout x%s w%s d%s pad%s dtype%d x_cl%d y_cl%d" % (x.shape, w.shape, d, pad, dtype, x_cl, y_cl))
+    wp = lib.thhip_conv_pack_weight_layout(w.ctypes.data, Co, Ci, kH, kW, dtype, x_cl)
+    dx = api.to_device_dtype(lib, np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if x_cl else x, dtype)
+    db = api.DeviceArray(lib, np.ascontiguousarray(bias, np.float32)) if bias is not None else None
+    ds = api.DeviceArray(lib, np.ascontiguousarray(scale, np.float32)) if scale is not None else None
+    dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW * 2)
+    lib.thhip_conv2d_layout(dx.ptr, wp, ds.ptr if ds else None, db.ptr if db else None, dy.ptr, B, Ci, H, W, Co, kH, kW,
+                            d[0], d[1], pad[0], pad[1], act, thr, val, dtype, x_cl, y_cl)
+    lib.thhip_sync()
+    if y_cl:
+        y = np.ascontiguousarray(api.from_device_dtype(dy, (B, oH, oW, Co), dtype).transpose(0, 3, 1, 2))
+    else:
+        y = api.from_device_dtype(dy, (B, Co, oH, oW), dtype)
+    lib.thhip_free(wp)
+    return y
+
+
 def gemv(lib, x, w, bias, act=0, thr=0.0, val=0.0, dtype=F32):
     nOut, nIn = w.shape
     note("gemv %dx%d dtype%d" % (nOut, nIn, dtype))

@@ -176,6 +176,59 @@ def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
 
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
+def test_conv_half_channels_last(hiplib, oracle, dt):
+    """fp16 / bf16 convolution with channels-last tensors on either side, the folded
+    batch-norm factor and the fused threshold: against the fp32 restatement on the
+    rounded operands, and against the same kernel on plane-major tensors."""
+    from thnets_amd import api
+    g = cases.rng(908)
+    shapes = [(2, 8, 9, 11, 36, 3, 3, 1, 1, 1, 1), (3, 64, 7, 7, 200, 5, 5, 2, 2, 2, 2), (1, 24, 13, 13, 68, 1, 1, 1, 1, 0, 0),
+              (5, 16, 6, 6, 132, 6, 6, 1, 1, 0, 0), (2, 3, 21, 19, 64, 7, 7, 2, 2, 3, 3), (2, 128, 8, 8, 64, 3, 3, 1, 1, 1, 1)]
+    for (B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW) in shapes:
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, kH, kW), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * kH * kW)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
+        wr = api.from_device_dtype(api.to_device_dtype(hiplib, w, dt), w.shape, dt)
+        raw = oracle.conv2d(xr, wr, None, (dH, dW), (pH, pW))
+        want = np.maximum(raw * sc[None, :, None, None] + b[None, :, None, None], 0)
+        base = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, scale=sc)
+        G.assert_close(base, want, HALF_TOL, "plane-major")
+        orders = [(0, 1)] + ([(1, 0), (1, 1)] if Ci % 8 == 0 else [])
+        for (x_cl, y_cl) in orders:
+            got = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=x_cl, y_cl=y_cl, scale=sc)
+            G.assert_close(got, want, HALF_TOL, str((x_cl, y_cl)))
+            G.assert_close(got, base, 1e-2, "vs plane-major " + str((x_cl, y_cl)))
+
+
+@pytest.mark.parametrize("dt", [G.F16, G.BF16])
+def test_maxpool_and_relayout_half_channels_last(hiplib, oracle, dt):
+    from thnets_amd import api
+    g = cases.rng(909)
+    for (B, Cn, H, W, kH, kW, dH, dW, pH, pW, ceil) in ((2, 8, 13, 13, 3, 3, 2, 2, 0, 0, 0), (3, 64, 14, 14, 2, 2, 2, 2, 0, 0, 0),
+                                                       (1, 16, 7, 9, 2, 2, 2, 2, 1, 1, 1), (2, 24, 10, 8, 2, 3, 1, 2, 0, 1, 0)):
+        x = g.standard_normal((B, Cn, H, W), dtype=np.float32)
+        dx = api.to_device_dtype(hiplib, x, dt)
+        xr = api.from_device_dtype(dx, x.shape, dt)
+        dcl = api.DeviceArray(hiplib, nbytes=x.size * 2)
+        hiplib.thhip_relayout(dx.ptr, dcl.ptr, B, Cn, H * W, 1, dt)
+        hiplib.thhip_sync()
+        assert np.array_equal(api.from_device_dtype(dcl, (B, H, W, Cn), dt), xr.transpose(0, 2, 3, 1))
+        dback = api.DeviceArray(hiplib, nbytes=x.size * 2)
+        hiplib.thhip_relayout(dcl.ptr, dback.ptr, B, Cn, H * W, 0, dt)
+        hiplib.thhip_sync()
+        assert np.array_equal(api.from_device_dtype(dback, x.shape, dt), xr)
+        spec = {"type": "maxpool", "kW": kW, "kH": kH, "dW": dW, "dH": dH, "padW": pW, "padH": pH, "ceil_mode": ceil}
+        want = oracle.run_layers([spec], xr)
+        oH, oW = want.shape[2:]
+        dy = api.DeviceArray(hiplib, nbytes=want.size * 2)
+        hiplib.thhip_maxpool_cl(dcl.ptr, dy.ptr, B, Cn, H, W, oH, oW, kH, kW, dH, dW, pH, pW, dt)
+        hiplib.thhip_sync()
+        assert np.array_equal(api.from_device_dtype(dy, (B, oH, oW, Cn), dt).transpose(0, 3, 1, 2), want)
+
+
+@pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_linear_batched_half_types(hiplib, oracle, dt):
     """fp16 / bf16 storage and MFMA, fp32 accumulation: against the fp32 restatement on
     the rounded operands at the half tolerance (2e-2 of the largest reference value)."""

@@ -127,7 +127,18 @@ def test_half_engine_small_vgg(hiplib, oracle, half):
     net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"], half=half)
     y = net.process_float(cfg["input"])
     G.assert_close(y, GOLD["net_vgg16_small"], 2e-2 if half == 1 else 6e-2, "half engine")
+    # every module output, read back in the reference's order although the engine keeps the
+    # tensors between convolutions channels-last
+    layerwise(net, oracle, cfg, 2e-2 if half == 1 else 6e-2)
     net.free()
+    # the same with batch norm (folded) and residual branches, and AlexNet's 11x11 / 5x5 layers
+    for name, tol in (("resnet18_small", 4e-2 if half == 1 else 1.5e-1), ("alexnet_small", 2e-2 if half == 1 else 6e-2)):
+        if name not in cases.small_networks():
+            continue
+        c2 = cases.small_networks()[name]
+        n2 = api.HipNetwork(c2["layers"], c2["mean"], c2["std"], half=half)
+        G.assert_close(n2.process_float(c2["input"]), GOLD["net_" + name], tol, name)
+        n2.free()
 
 
 def test_process_images_matches_process_float(hiplib, oracle):

@@ -78,6 +78,10 @@ PROTOTYPES = {
     "thhip_conv_packed_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv_unpack_rows": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
+    "thhip_conv_pack_weight_layout": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "thhip_conv2d_layout": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]),
+    "thhip_relayout": (None, [vp, vp] + [C.c_int] * 5),
+    "thhip_maxpool_cl": (None, [vp, vp] + [C.c_int] * 13),
     "thhip_conv2d_affine": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),

@@ -847,19 +847,22 @@ static inline unsigned short f32_to_bf16_bits(float f)
 	return (unsigned short)(u >> 16);
 }
 
-extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW, int dtype)
+extern "C" void *thhip_conv_pack_weight_layout(const float *w, int Co, int Ci, int kH, int kW, int dtype, int x_layout)
 {
 	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
 		THError("thhip_conv_pack_weight: unsupported dtype %d", dtype);
-	const int chunk = conv_chunk(dtype), KC = conv_kc(Ci, 1, kHW, dtype, 0);
-	const size_t bytes = thhip_conv_packed_bytes(Co, Ci, kHW, dtype);
+	if (x_layout != 0 && !(x_layout == 1 && dtype != THHIP_F32))
+		THError("thhip_conv_pack_weight: input layout %d with dtype %d", x_layout, dtype);
+	const int kHW = kH * kW;
+	const int chunk = conv_chunk(dtype), KC = conv_kc(Ci, kH, kW, dtype, x_layout);
+	const size_t bytes = conv_packed_bytes(Co, Ci, kH, kW, dtype, x_layout);
 	unsigned char *host = (unsigned char *)calloc(1, bytes);
 	if (!host)
 		THError("thhip_conv_pack_weight: out of host memory (%zu bytes)", bytes);
 	for (int m = 0; m < Co; m++)
 		for (int c = 0; c < Ci; c++)
 			for (int tap = 0; tap < kHW; tap++) {
-				const size_t idx = conv_pack_index(m, conv_kpos(c, 0, tap, Ci, 1, kHW, dtype, 0), KC, chunk);
+				const size_t idx = conv_pack_index(m, conv_kpos(c, tap / kW, tap % kW, Ci, kH, kW, dtype, x_layout), KC, chunk);
 				const float v = w[((size_t)m * Ci + c) * kHW + tap];
 				if (dtype == THHIP_F32)
 					((float *)host)[idx] = v;
@@ -872,6 +875,11 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 	thhip_memcpy_h2d(dev, host, bytes);
 	free(host);
 	return dev;
+}
+
+extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW, int dtype)
+{
+	return thhip_conv_pack_weight_layout(w, Co, Ci, 1, kHW, dtype, 0);
 }
 
 /* Experiment / tuning override: 0 = choose automatically. */
@@ -972,8 +980,22 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 				CONV_GO(GM_TAP_MAJOR, true);
 			CONV_GO(GM_PLANE_TAP, true);
 		}
+	} else if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
+		/* the half engines do the same: a 16-byte gather is eight planes of one pixel */
+		if (p.x_cl == 1) {
+			if (p.y_cl)
+				CONV_GO(GM_CHANNELS_LAST, true);
+			CONV_GO(GM_CHANNELS_LAST, false);
+		}
+		if (p.x_cl)
+			THError("thhip_conv2d: input layout %d is a uint8 feature", p.x_cl);
+		if (p.y_cl) {
+			if (tap)
+				CONV_GO(GM_TAP_MAJOR, true);
+			CONV_GO(GM_PLANE_TAP, true);
+		}
 	} else if (p.x_cl || p.y_cl)
-		THError("thhip_conv2d: channels-last tensors are a uint8 feature");
+		THError("thhip_conv2d: channels-last tensors are for the uint8 and half types");
 	if (tap)
 		CONV_GO(GM_TAP_MAJOR, false);
 	CONV_GO(GM_PLANE_TAP, false);
@@ -1079,7 +1101,7 @@ static unsigned char *conv_pixels4_scratch(size_t bytes)
 
 static void conv_run(const void *x, const void *wpacked, const float *scale, const float *bias, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
-	int act, float thr, float val, int dtype, const ConvU8Args *u8)
+	int act, float thr, float val, int dtype, const ConvU8Args *u8, int f_x_layout = 0, int f_y_cl = 0)
 {
 	if (B < 1 || Ci < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
 		THError("thhip_conv2d: bad geometry");
@@ -1094,7 +1116,7 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 		THError("thhip_conv2d: K = %ld too large", K);
 	/* 32-bit offsets inside the kernel: run the batch in slices whose input
 	 * and output stay below 2^31 bytes. */
-	const int xl = u8 ? u8->x_cl : 0;
+	const int xl = u8 ? u8->x_cl : f_x_layout;
 	const long in_img = (long)Ci * H * W, out_img = (long)Co * oH * oW;
 	const long in_eff = xl == 2 ? 4L * H * W : in_img;	/* bytes the kernel addresses per image */
 	long bmax = ((1L << 31) - 64) / (esize * (in_eff > out_img ? in_eff : out_img));
@@ -1168,6 +1190,8 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 			ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * Co * (double)K * p.N);
 			conv_dispatch<THHIP_U8>(p);
 		} else {
+			p.x_cl = xl;
+			p.y_cl = f_y_cl;
 			ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N);
 			THHIP_DISPATCH_FLOAT(dtype, conv_dispatch<DT>(p));
 		}
@@ -1181,6 +1205,18 @@ extern "C" void thhip_conv2d_affine(const void *x, const void *wpacked, const fl
 	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
 		THError("thhip_conv2d: unsupported dtype %d", dtype);
 	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0);
+}
+
+extern "C" void thhip_conv2d_layout(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype, int x_layout, int y_channels_last)
+{
+	if (dtype != THHIP_F16 && dtype != THHIP_BF16 && (x_layout || y_channels_last))
+		THError("thhip_conv2d_layout: channels-last tensors need a half dtype (got %d)", dtype);
+	if (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_BF16)
+		THError("thhip_conv2d: unsupported dtype %d", dtype);
+	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0,
+		x_layout, y_channels_last != 0);
 }
 
 extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,

@@ -247,11 +247,80 @@ extern "C" void thhip_maxpool_u8_cl(const unsigned char *x, unsigned char *y, in
 		maxpool_u8_cl_kernel<<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>((const unsigned *)x, (unsigned *)y, p);
 }
 
+/* SpatialMaxPooling (SpatialMaxPooling.c:168-247) on channels-last half tensors
+ * [B][H][W][C], C % 8 == 0: a thread owns eight adjacent planes of one output
+ * position and reads them as one 16-byte vector per window element. */
+template <int DT>
+__global__ void maxpool_half_cl_kernel(const uintx4 *x, uintx4 *y, PoolParams p)
+{
+	typedef typename ThhipElem<DT>::T elem;
+	const int C8 = p.C / 8;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < p.total; i += step) {
+		const int c8 = (int)(i % C8);
+		long t = i / C8;
+		const int ox = (int)(t % p.oW);
+		t /= p.oW;
+		const int oy = (int)(t % p.oH);
+		const long b = t / p.oH;
+		int hs = oy * p.dH - p.padH, ws = ox * p.dW - p.padW;
+		const int he = min(hs + p.kH, p.H), we = min(ws + p.kW, p.W);
+		hs = max(hs, 0);
+		ws = max(ws, 0);
+		float m[8];
+#pragma unroll
+		for (int k = 0; k < 8; k++)
+			m[k] = -FLT_MAX;
+		for (int yy = hs; yy < he; yy++)
+			for (int xx = ws; xx < we; xx++) {
+				const uintx4 raw = x[((b * p.H + yy) * p.W + xx) * C8 + c8];
+				elem v[8];
+				__builtin_memcpy(v, &raw, 16);
+#pragma unroll
+				for (int k = 0; k < 8; k++) {
+					const float f = (float)v[k];
+					if (f > m[k])
+						m[k] = f;
+				}
+			}
+		elem o[8];
+#pragma unroll
+		for (int k = 0; k < 8; k++)
+			o[k] = (elem)m[k];
+		uintx4 raw;
+		__builtin_memcpy(&raw, o, 16);
+		y[i] = raw;
+	}
+}
+
+extern "C" void thhip_maxpool_cl(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype)
+{
+	if (dtype == THHIP_U8) {
+		thhip_maxpool_u8_cl((const unsigned char *)x, (unsigned char *)y, B, C, H, W, oH, oW, kH, kW, dH, dW, padH, padW);
+		return;
+	}
+	if (dtype != THHIP_F16 && dtype != THHIP_BF16)
+		THError("thhip_maxpool_cl: dtype %d has no channels-last form", dtype);
+	if (C % 8)
+		THError("thhip_maxpool_cl: C = %d is not a multiple of 8", C);
+	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * oH * oW * (C / 8) };
+	if (p.total <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * B * C * H * W + 16.0 * p.total);
+	if (dtype == THHIP_F16)
+		maxpool_half_cl_kernel<THHIP_F16><<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>((const uintx4 *)x, (uintx4 *)y, p);
+	else
+		maxpool_half_cl_kernel<THHIP_BF16><<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>((const uintx4 *)x, (uintx4 *)y, p);
+}
+
 /* Codes between plane-major [B][C][HW] and channels-last [B][HW][C] memory
  * order (to_cl = 1: the former to the latter), through a 32 x 32 LDS tile. */
-__global__ void relayout_u8_kernel(const unsigned char *x, unsigned char *y, int C, int HW, int to_cl)
+template <typename E>
+__global__ void relayout_kernel(const E *x, E *y, int C, int HW, int to_cl)
 {
-	__shared__ unsigned char t[32][33];
+	__shared__ E t[32][33];
 	/* source [R][S] -> destination [S][R] per image */
 	const int R = to_cl ? C : HW, S = to_cl ? HW : C;
 	const size_t img = (size_t)blockIdx.z * C * HW;
@@ -266,16 +335,30 @@ __global__ void relayout_u8_kernel(const unsigned char *x, unsigned char *y, int
 			y[img + (size_t)(s0 + k) * R + r0 + tx] = t[tx][k];
 }
 
-extern "C" void thhip_relayout_u8(const unsigned char *x, unsigned char *y, int B, int C, int HW, int to_channels_last)
+extern "C" void thhip_relayout(const void *x, void *y, int B, int C, int HW, int to_channels_last, int dtype)
 {
 	if (B < 1 || C < 1 || HW < 1)
 		return;
 	if (B > 65535)
-		THError("thhip_relayout_u8: batch %d too large", B);
+		THError("thhip_relayout: batch %d too large", B);
 	const int R = to_channels_last ? C : HW, S = to_channels_last ? HW : C;
-	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * B * C * HW);
-	relayout_u8_kernel<<<dim3((S + 31) / 32, (R + 31) / 32, B), dim3(256), 0, thhip_stream()>>>(x, y, C, HW,
-		to_channels_last != 0);
+	const int esz = thhip_esize(dtype);
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * esz * B * C * HW);
+	const dim3 grid((S + 31) / 32, (R + 31) / 32, B);
+	if (esz == 1)
+		relayout_kernel<unsigned char><<<grid, dim3(256), 0, thhip_stream()>>>((const unsigned char *)x,
+			(unsigned char *)y, C, HW, to_channels_last != 0);
+	else if (esz == 2)
+		relayout_kernel<unsigned short><<<grid, dim3(256), 0, thhip_stream()>>>((const unsigned short *)x,
+			(unsigned short *)y, C, HW, to_channels_last != 0);
+	else
+		relayout_kernel<float><<<grid, dim3(256), 0, thhip_stream()>>>((const float *)x, (float *)y, C, HW,
+			to_channels_last != 0);
+}
+
+extern "C" void thhip_relayout_u8(const unsigned char *x, unsigned char *y, int B, int C, int HW, int to_channels_last)
+{
+	thhip_relayout(x, y, B, C, HW, to_channels_last, THHIP_U8);
 }
 
 /* modules/SpatialAveragePooling.c:156-203 */

@@ -386,10 +386,10 @@ long THHipNetwork_copyModuleOutput(THNETWORK *net, int idx, float **dst, long si
 	THFloatTensor *h;
 	const int nd = o->nDimension;
 	if (hn->hm[idx].out_cl && nd >= 3 && o->size[nd - 1] * o->size[nd - 2] > 1) {
-		/* kept channels-last inside the uint8 engine: hand out the reference's order */
-		THFloatTensor *pm = device_tensor_like(o, THHIP_U8);
-		thhip_relayout_u8(thhip_tensor_ptr(o, THHIP_U8), (unsigned char *)pm->storage->data, nd == 4 ? (int)o->size[0] : 1,
-			(int)o->size[nd - 3], (int)(o->size[nd - 1] * o->size[nd - 2]), 0);
+		/* kept channels-last inside the engine: hand out the reference's order */
+		THFloatTensor *pm = device_tensor_like(o, hn->dtype);
+		thhip_relayout(thhip_tensor_ptr(o, hn->dtype), pm->storage->data, nd == 4 ? (int)o->size[0] : 1,
+			(int)o->size[nd - 3], (int)(o->size[nd - 1] * o->size[nd - 2]), 0, hn->dtype);
 		h = download_as_float(pm, hn->dtype);
 		THFloatTensor_free(pm);
 	} else

@@ -168,7 +168,14 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 	const void *x = thhip_tensor_ptr(in, dt);
 	void *y = conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
 	const int K = c->nInputPlane * c->kH * c->kW;
-	const int one_position = oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W;
+	/* the weights were packed for the planned memory order of the input; with
+	 * one pixel per plane both orders coincide */
+	if (s.H * s.W > 1 && hn->cur_cl != hm->in_cl)
+		THError("HIP engine: a convolution planned for %s input got the other memory order",
+			hm->in_cl ? "channels-last" : "plane-major");
+	hn->cur_cl = hm->out_cl && oH * oW > 1;
+	const int one_position = oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
+		!hm->x_layout;	/* the row-major copy is made from plane-major packing */
 	if (one_position && !hm->scale && (s.B == 1 || thhip_linear_batched_supported(s.B, K, c->nOutputPlane, dt))) {
 		/* one output position per image: a matrix-vector (or skinny matrix)
 		 * product over the flattened input, bound by reading the weights once */
@@ -180,8 +187,9 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 			thhip_linear_batched(x, hm->wrow, hm->bias, y, s.B, K, c->nOutputPlane, hm->fused_act, hm->thr,
 				hm->val, dt);
 	} else
-		thhip_conv2d_affine(x, hm->wpacked, hm->scale, hm->bias, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
-			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, hm->fused_act, hm->thr, hm->val, dt);
+		thhip_conv2d_layout(x, hm->wpacked, hm->scale, hm->bias, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, hm->fused_act, hm->thr, hm->val, dt, hm->x_layout,
+			hm->out_cl);
 	return m->output;
 }
 
@@ -246,7 +254,12 @@ static THFloatTensor *Hip_SpatialMaxPooling_updateOutput(struct module *m, THFlo
 		THError("SpatialMaxPooling: input %dx%d smaller than the window", p.H, p.W);
 	const void *x = thhip_tensor_ptr(in, hn->dtype);
 	void *y = planes_out(m, hn->dtype, &p, oH, oW);
-	thhip_maxpool(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, hn->dtype);
+	if (hn->cur_cl)
+		thhip_maxpool_cl(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, hn->dtype);
+	else
+		thhip_maxpool(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, hn->dtype);
+	if (oH * oW == 1)
+		hn->cur_cl = 0;		/* one pixel per plane: both orders coincide */
 	return m->output;
 }
 
@@ -614,6 +627,7 @@ static int is_conv_type(int type)
 static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
 {
 	double t = 0;
+	((struct hipnet *)net)->cur_cl = 0;	/* inputs arrive in the reference's plane-major order */
 	for (int i = 0; i < net->nelem; i++) {
 		struct module *m = &net->modules[i];
 		if (th_profile) {
@@ -647,7 +661,6 @@ THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in)
 			"(engine %d given); it carries no CPU path", net->engine);
 	th_convtot = 0;
 	th_convflops = 0;
-	((struct hipnet *)net)->cur_cl = 0;	/* inputs arrive in the reference's plane-major order */
 	THFloatTensor *out = run_network(net, in);
 	if (th_profile)
 		printf("%f seconds for convolutions %f Gflops/s\n", th_convtot, th_convflops * 1e-9 / th_convtot);
@@ -862,30 +875,49 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 	}
 }
 
-/* uint8 engine: decides which tensors live channels-last ([B][H][W][C]) in
- * memory.  A convolution reads 16 adjacent planes of one pixel per operand
- * vector, so it takes channels-last input whenever its planes come in whole
- * blocks of 16 and the producer is another convolution reached only through
- * modules that work in either order (Threshold, pooling, Dropout, Identity).
- * Network inputs and every tensor a View or SoftMax sees stay plane-major.
- * Also makes the row-major weight copies of the one-position (matrix) path,
- * whose K order follows the input's memory order. */
-static void plan_channels_last(struct hipnet *hn)
+/* uint8 and half engines: decides which tensors live channels-last
+ * ([B][H][W][C]) in memory.  A convolution reads 16 bytes of adjacent planes of
+ * one pixel per operand vector (16 codes, 8 halfs), so it takes channels-last
+ * input whenever its planes come in whole vectors and the producer is another
+ * convolution reached only through modules that work in either order
+ * (Threshold, max pooling, Dropout, Identity, a batch norm folded away).
+ * Network inputs and every tensor another module sees stay plane-major.
+ * Weights are (re-)packed here, because their K order follows how the input
+ * is read; so are the row-major copies of the uint8 one-position (matrix) path. */
+static void plan_channels_last(struct hipnet *hn, struct network *src)
 {
+	const int lowp = hn->pub.engine == ENGINE_HIPLOWP;
+	const int vec = lowp ? 16 : 8;
 	int prev = -1;
+	if (!lowp && hn->dtype == THHIP_F32)
+		return;		/* fp32 gathers element-wise at full speed; it stays plane-major */
 	for (int i = 0; i < hn->pub.nelem; i++) {
 		struct module *m = &hn->pub.modules[i];
 		struct hipmod *hm = &hn->hm[i];
 		if (is_conv_type(m->type)) {
-			if (prev >= 0 && m->SpatialConvolution.nInputPlane % 16 == 0) {
+			if (prev >= 0 && m->SpatialConvolution.nInputPlane % vec == 0) {
 				for (int j = prev; j < i; j++)
 					hn->hm[j].out_cl = 1;
 				hm->in_cl = 1;
 			}
 			prev = i;
 		} else if (m->type != MT_Threshold && m->type != MT_SpatialMaxPooling && m->type != MT_Dropout &&
-			m->type != MT_Identity)
+			m->type != MT_Identity && !(m->type == MT_SpatialBatchNormalization && hm->passthrough))
 			prev = -1;
+	}
+	for (int i = 0; i < hn->pub.nelem && !lowp; i++) {
+		struct module *m = &hn->pub.modules[i];
+		struct hipmod *hm = &hn->hm[i];
+		if (!is_conv_type(m->type) || !hm->in_cl)
+			continue;
+		/* packed plane-major by convert_module: pack again for channels-last input */
+		const struct SpatialConvolution *c = &m->SpatialConvolution;
+		THFloatTensor *w = src->modules[i].type == MT_Linear ? src->modules[i].Linear.weight :
+			src->modules[i].SpatialConvolution.weight;
+		thhip_free(hm->wpacked);
+		hm->x_layout = 1;
+		hm->wpacked = thhip_conv_pack_weight_layout(THFloatTensor_data(w), c->nOutputPlane, c->nInputPlane, c->kH, c->kW,
+			hn->dtype, 1);
 	}
 	for (int i = 0; i < hn->pub.nelem; i++) {
 		struct module *m = &hn->pub.modules[i];
@@ -989,8 +1021,7 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			hn->hm[i + 1].passthrough = 1;
 		}
 	}
-	if (engine == ENGINE_HIPLOWP)
-		plan_channels_last(hn);
+	plan_channels_last(hn, net);
 	return &hn->pub;
 }
 
