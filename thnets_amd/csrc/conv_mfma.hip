@@ -1013,14 +1013,19 @@ static void conv_dispatch(ConvParams &p)
 	 * (residents per CU) x (tile time) even when nearly empty.  fp32 (K-tiles
 	 * of 32) and uint8 (int8 MFMAs outrun LDS at any of these sizes, so the
 	 * tile with the most workgroups in flight wins) always take 64x64; the
-	 * half types take 128x64 on the widest layers (>= 700 tiles of 128x128)
-	 * for its operand reuse.  Splitting K is available (thhip_conv_set_tuning)
+	 * half types, whose MFMAs are LDS-bound on layers large enough to fill the
+	 * machine, take 128x128 (64x128 for <= 64 planes) from 200 such tiles up
+	 * for the operand reuse.  Splitting K is available (thhip_conv_set_tuning)
 	 * but measured slower than unsplit 64x64 tiles on every layer shape tried,
 	 * so it is never chosen; so is a cap on the workgroups per CU. */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	int bm = 64, bn = 64, splitk = 1, wgs = 0;
-	if ((DT == THHIP_F16 || DT == THHIP_BF16) && p.Co > 64 && t128 >= 700)
-		bm = 128;
+	if (DT == THHIP_F16 || DT == THHIP_BF16) {
+		if (p.Co <= 64)
+			bn = 128;
+		else if (t128 >= 200)
+			bm = bn = 128;
+	}
 	if (g_force_bm)
 		bm = g_force_bm;
 	if (g_force_bn)
