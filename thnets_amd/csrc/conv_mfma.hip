@@ -74,9 +74,10 @@ static inline unsigned long long conv_magic(unsigned d)
  * deeper K-tiles keep the work per barrier up. */
 #define CONV_KCH_U8_CL 2
 #define CONV_KCH_F32 4
+#define CONV_KCH_HALF_CL 2
 __host__ __device__ constexpr int conv_kch(int dtype, bool x_cl)
 {
-	return dtype == THHIP_U8 && x_cl ? CONV_KCH_U8_CL : dtype == THHIP_F32 ? CONV_KCH_F32 : 2;
+	return dtype == THHIP_U8 ? (x_cl ? CONV_KCH_U8_CL : 2) : dtype == THHIP_F32 ? CONV_KCH_F32 : (x_cl ? CONV_KCH_HALF_CL : 2);
 }
 
 /* Waves per SIMD to ask the register allocator for (what each tile reaches
