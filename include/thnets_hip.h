@@ -383,6 +383,9 @@ void thhip_conv2d_layout(const void *x, const void *wpacked, const float *scale,
  * (bm x bn in {64,128}), its split-K factor and the number of workgroups
  * allowed to share a CU; 0 leaves a choice automatic. */
 void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);
+/* fp32 only: force K-tiles of 16 values (chunks = 2) or 32 (4); 0 restores the
+ * per-layer choice.  Tests and tuning, like thhip_conv_set_tuning. */
+void thhip_conv_set_ktile(int chunks);
 
 /* Replaces nn_Linear_updateOutput's 1-D branch (Linear.c:86-90 ->
  * thbasic.c:713-741 -> sgemv.c:48-105): y = bias + W x, W row-major

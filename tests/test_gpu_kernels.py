@@ -33,6 +33,33 @@ def test_conv_f32_vs_oracle_and_golden(hiplib, oracle, i):
     assert np.array_equal(ya, np.where(y > np.float32(0.1), y, np.float32(-0.5)))
     # no bias
     G.assert_close(G.conv2d(hiplib, x, s["weight"], None, d, p), oracle.conv2d(x, s["weight"], None, d, p), FP32_TOL)
+    # both K-tile depths of the fp32 kernel (the launcher picks one by layer width)
+    try:
+        for chunks in (2, 4):
+            hiplib.thhip_conv_set_ktile(chunks)
+            G.assert_close(G.conv2d(hiplib, x, s["weight"], s["bias"], d, p), GOLD["conv%d" % i], FP32_TOL, "ktile %d" % chunks)
+    finally:
+        hiplib.thhip_conv_set_ktile(0)
+
+
+def test_conv_f32_ktile_depths_tap_major_and_split(hiplib, oracle):
+    """Tap-major fp32 layers (planes in blocks of 32) at both K-tile depths, with forced
+    tiles and K splits that start inside a block."""
+    g = cases.rng(910)
+    for (B, Ci, H, W, Co, k, dd, pp) in ((2, 32, 9, 10, 70, 3, 1, 1), (1, 96, 7, 7, 130, 3, 2, 1), (3, 64, 6, 5, 64, 1, 1, 0)):
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        want = oracle.conv2d(x, w, b, (dd, dd), (pp, pp))
+        try:
+            for chunks in (2, 4):
+                hiplib.thhip_conv_set_ktile(chunks)
+                for tune in ((0, 0, 0, 0), (64, 64, 3, 0), (128, 64, 2, 2), (128, 128, 5, 0), (64, 128, 1, 1)):
+                    hiplib.thhip_conv_set_tuning(*tune)
+                    G.assert_close(G.conv2d(hiplib, x, w, b, (dd, dd), (pp, pp)), want, FP32_TOL, str((chunks, tune)))
+        finally:
+            hiplib.thhip_conv_set_ktile(0)
+            hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
 @pytest.mark.parametrize("dtype", [G.F16, G.BF16])

@@ -82,12 +82,13 @@ __host__ __device__ constexpr int conv_kch(int dtype, bool x_cl)
 
 /* Waves per SIMD to ask the register allocator for (what each tile reaches
  * without spilling): more for the small tiles, whose residency matters most. */
-__host__ __device__ constexpr int conv_min_waves(int dtype, int tile_elems, bool generic_gather)
+__host__ __device__ constexpr int conv_min_waves(int dtype, int tile_elems, bool generic_gather, int kch)
 {
+	const bool deep = dtype == THHIP_F32 && kch > 2;	/* fp32 K-tiles of 32: LDS limits first */
 	return generic_gather ? 1
-		: tile_elems <= 64 * 64 ? (dtype == THHIP_F32 ? 3 : 4)
-		: tile_elems <= 128 * 64 ? (dtype == THHIP_F32 ? 2 : 4)
-		: (dtype == THHIP_F32 ? 1 : 2);
+		: tile_elems <= 64 * 64 ? (deep ? 3 : 4)
+		: tile_elems <= 128 * 64 ? (deep ? 2 : 4)
+		: (deep ? 1 : 2);
 }
 
 template <int DT> struct ConvTraits;
@@ -176,12 +177,12 @@ __device__ __forceinline__ KTap conv_ktap(const ConvParams &p, int k)
 /* GM, how the B operand is gathered: */
 enum { GM_PLANE_TAP, GM_TAP_MAJOR, GM_CHANNELS_LAST, GM_PIXELS4 };
 
-template <int DT, int BM, int BN, int WGM, int WGN, int GM, bool CLO>
+template <int DT, int BM, int BN, int WGM, int WGN, int GM, bool CLO, int KCH>
 __global__ __launch_bounds__(CONV_THREADS)
 /* ask for four waves per SIMD where the tile allows it: without the hint the
  * compiler spreads the accumulators over AGPRs plus a generous VGPR budget and
  * halves the number of workgroups a CU can hold */
-__attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) void conv_mfma_kernel(ConvParams p)
+__attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8))) void conv_mfma_kernel(ConvParams p)
 {
 	constexpr bool TAP = GM == GM_TAP_MAJOR;
 	constexpr bool C4 = GM == GM_PIXELS4;		/* uint8, <= 4 planes, re-laid out as [B][H][W][4] */
@@ -189,7 +190,12 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) vo
 	static_assert(!C4 || DT == THHIP_U8, "the four-plane pixel layout is a uint8 path");
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
-	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC, KCH = conv_kch(DT, CLI);
+	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC;
+	/* KCH chunks per K-tile (one LDS stage).  Weights are packed in blocks of
+	 * PKCH chunks; a shallower K-tile walks a block in SUB steps (more, smaller
+	 * stages: more workgroups per CU, which the widest layers prefer). */
+	constexpr int PKCH = conv_kch(DT, CLI), SUB = PKCH / KCH;
+	static_assert(PKCH % KCH == 0 && KCH % 2 == 0, "K-tile depth");
 	constexpr int MB = BM / 32, NB = BN / 32;		/* 32-row blocks per tile */
 	constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32;	/* MFMA tiles per wave */
 	constexpr int A_VECS = MB * KCH * 64;			/* 16-byte vectors per K-tile (KCH chunks) */
@@ -269,7 +275,7 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) vo
 		colsum[q] = 0;
 
 	/* Tap-major K order (TAP, plane-major input): K-tile t covers one filter tap
-	 * (kh, kw) and CB = KCH*CHUNK consecutive input planes, tiles ordered plane
+	 * (kh, kw) and KCH*CHUNK consecutive input planes, tiles ordered plane
 	 * block outer, tap inner.  Bounds test and in-plane offset are then one
 	 * computation per thread per K-tile and every element differs only by a
 	 * wave-uniform plane offset, which rides in the load's scalar offset.
@@ -277,7 +283,7 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) vo
 	 * Channels-last input (CLI): k = tap * Ci + plane, so the VEC planes of a
 	 * lane vector are 16 adjacent bytes of one pixel.  Which tap a vector
 	 * belongs to is wave-uniform and decoded on the scalar unit. */
-	int t_cb = 0, t_kh = 0, t_kw = 0;
+	int t_cb = 0, t_kh = 0, t_kw = 0, t_sub = 0;
 	const int plane_bytes = p.HW * (int)sizeof(elem);
 
 	auto load_tile = [&](int kt) {
@@ -349,7 +355,7 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) vo
 				const uintx4 ld = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, voff, 0, 0);
 				__builtin_memcpy(v, &ld, 16);
 			} else if constexpr (TAP) {
-				const int cbase = t_cb * (KCH * CHUNK) + (pidx >> 1) * CHUNK + (pidx & 1) * VEC;
+				const int cbase = (t_cb * SUB + t_sub) * (KCH * CHUNK) + (pidx >> 1) * CHUNK + (pidx & 1) * VEC;
 #pragma unroll
 				for (int e = 0; e < VEC; e++) {
 					/* the scalar offset is not range checked: planes exist
@@ -407,7 +413,9 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) vo
 			breg[j] = packed;
 		}
 		if constexpr (TAP) {
-			if (++t_kw == p.kW) {
+			if (++t_sub < SUB) {
+				/* same tap, next planes of the block */
+			} else if (t_sub = 0, ++t_kw == p.kW) {
 				t_kw = 0;
 				if (++t_kh == p.kH) {
 					t_kh = 0;
@@ -457,8 +465,10 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0), 8))) vo
 	const int kt0 = p.splitk > 1 ? (int)((long)nkt_all * split / p.splitk) : 0;
 	const int nkt = p.splitk > 1 ? (int)((long)nkt_all * (split + 1) / p.splitk) : nkt_all;
 	if constexpr (TAP) {
-		t_cb = kt0 / p.kHW;
-		const int tap = kt0 - t_cb * p.kHW;
+		const int blk = kt0 / SUB;
+		t_sub = kt0 - blk * SUB;
+		t_cb = blk / p.kHW;
+		const int tap = blk - t_cb * p.kHW;
 		t_kh = tap / p.kW;
 		t_kw = tap - t_kh * p.kW;
 	}
@@ -884,7 +894,15 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 }
 
 /* Experiment / tuning override: 0 = choose automatically. */
-static int g_force_bm, g_force_bn, g_force_splitk, g_force_wgs;
+static int g_force_bm, g_force_bn, g_force_splitk, g_force_wgs, g_force_kch;
+
+/* fp32 only: force K-tiles of 16 (chunks = 2) or 32 (4); 0 = choose automatically. */
+extern "C" void thhip_conv_set_ktile(int chunks)
+{
+	if (chunks != 0 && chunks != 2 && chunks != CONV_KCH_F32)
+		THError("thhip_conv_set_ktile(%d): 0, 2 or %d", chunks, CONV_KCH_F32);
+	g_force_kch = chunks;
+}
 
 extern "C" void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu)
 {
@@ -947,12 +965,12 @@ static void conv_launch_kernel(ConvParams &p, dim3 grid, int wgs)
 	kernel<<<grid, dim3(CONV_THREADS), dyn, thhip_stream()>>>(p);
 }
 
-template <int DT, int BM, int BN, int WGM, int WGN>
+template <int DT, int BM, int BN, int WGM, int WGN, int KCH>
 static void conv_launch(ConvParams &p, int splitk, int wgs)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
-	const int nkt = p.KC / conv_kch(DT, p.x_cl != 0);
+	const int nkt = p.KC / KCH;
 	if (splitk > nkt)
 		splitk = nkt;
 	p.splitk = splitk < 1 ? 1 : splitk;
@@ -963,7 +981,7 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 	const bool tap = conv_tap_major(p.Ci, DT);
 	if (p.y_cl && p.Co % 4)
 		THError("thhip_conv2d: channels-last output needs Co %% 4 == 0 (Co = %d)", p.Co);
-#define CONV_GO(GM, CLO) return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, GM, CLO>>(p, grid, wgs)
+#define CONV_GO(GM, CLO) return conv_launch_kernel<conv_mfma_kernel<DT, BM, BN, WGM, WGN, GM, CLO, KCH>>(p, grid, wgs)
 	if constexpr (DT == THHIP_U8) {
 		/* the uint8 engine keeps its activations channels-last between convolutions */
 		if (p.x_cl == 2) {
@@ -1011,21 +1029,32 @@ static void conv_dispatch(ConvParams &p)
 	 * keeps its four matrix cores nearly as busy as a bigger one, and small
 	 * tiles quantise best: the hardware packs the workgroups of a grid's last,
 	 * partially filled round onto as few CUs as they fit, so a round costs
-	 * (residents per CU) x (tile time) even when nearly empty.  fp32 (K-tiles
-	 * of 32) and uint8 (int8 MFMAs outrun LDS at any of these sizes, so the
-	 * tile with the most workgroups in flight wins) always take 64x64; the
-	 * half types, whose MFMAs are LDS-bound on layers large enough to fill the
-	 * machine, take 128x128 (64x128 for <= 64 planes) from 200 such tiles up
-	 * for the operand reuse.  Splitting K is available (thhip_conv_set_tuning)
-	 * but measured slower than unsplit 64x64 tiles on every layer shape tried,
-	 * so it is never chosen; so is a cap on the workgroups per CU. */
+	 * (residents per CU) x (tile time) even when nearly empty.
+	 *   fp32: layers wide enough to keep every CU supplied (>= 300 tiles of
+	 * 128x128) run K-tiles of 16 (small LDS stages, up to six workgroups per
+	 * CU; 128x64 tiles from 700 such tiles up for the operand reuse); narrower
+	 * layers run 64x64 tiles with K-tiles of 32, which halve the barriers per
+	 * MFMA of the few workgroups each CU gets.
+	 *   uint8: int8 MFMAs outrun everything else at any of these sizes, so the
+	 * tile with the most workgroups in flight, 64x64, wins.
+	 *   half types: 128x128 (64x128 for <= 64 planes) from 200 such tiles up
+	 * for the operand reuse, 64x64 below.
+	 * Splitting K is available (thhip_conv_set_tuning) but measured slower
+	 * than unsplit 64x64 tiles on every layer shape tried, so it is never
+	 * chosen; so is a cap on the workgroups per CU. */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
-	int bm = 64, bn = 64, splitk = 1, wgs = 0;
+	int bm = 64, bn = 64, splitk = 1, wgs = 0, kch = conv_kch(DT, p.x_cl != 0);
 	if (DT == THHIP_F16 || DT == THHIP_BF16) {
 		if (p.Co <= 64)
 			bn = 128;
 		else if (t128 >= 200)
 			bm = bn = 128;
+	} else if (DT == THHIP_F32 && t128 >= 300) {
+		kch = 2;
+		if (p.Co > 64 && t128 >= 700)
+			bm = 128;
+		else if (p.Co > 64)
+			wgs = 4;
 	}
 	if (g_force_bm)
 		bm = g_force_bm;
@@ -1035,16 +1064,34 @@ static void conv_dispatch(ConvParams &p)
 		splitk = g_force_splitk;
 	if (g_force_wgs)
 		wgs = g_force_wgs;
-	if (bm == 128 && bn == 128)
-		conv_launch<DT, 128, 128, 2, 2>(p, splitk, wgs);
-	else if (bm == 128 && bn == 64)
-		conv_launch<DT, 128, 64, 2, 2>(p, splitk, wgs);
-	else if (bm == 64 && bn == 128)
-		conv_launch<DT, 64, 128, 2, 2>(p, splitk, wgs);
-	else if (bm == 64 && bn == 64)
-		conv_launch<DT, 64, 64, 2, 2>(p, splitk, wgs);
-	else
-		THError("thhip_conv2d: no %dx%d tile", bm, bn);
+	if (DT == THHIP_F32 && g_force_kch)
+		kch = g_force_kch;
+#define CONV_TILES(KCH)                                                      \
+	do {                                                                 \
+		if (bm == 128 && bn == 128)                                  \
+			conv_launch<DT, 128, 128, 2, 2, KCH>(p, splitk, wgs); \
+		else if (bm == 128 && bn == 64)                              \
+			conv_launch<DT, 128, 64, 2, 2, KCH>(p, splitk, wgs);  \
+		else if (bm == 64 && bn == 128)                              \
+			conv_launch<DT, 64, 128, 2, 2, KCH>(p, splitk, wgs);  \
+		else if (bm == 64 && bn == 64)                               \
+			conv_launch<DT, 64, 64, 2, 2, KCH>(p, splitk, wgs);   \
+		else                                                         \
+			THError("thhip_conv2d: no %dx%d tile", bm, bn);      \
+	} while (0)
+	if constexpr (DT == THHIP_F32) {
+		if (kch == 2)
+			CONV_TILES(2);
+		else
+			CONV_TILES(CONV_KCH_F32);
+	} else {
+		/* one depth per dtype and input layout */
+		if (p.x_cl)
+			CONV_TILES(conv_kch(DT, true));
+		else
+			CONV_TILES(conv_kch(DT, false));
+	}
+#undef CONV_TILES
 }
 
 struct ConvU8Args {
