@@ -386,6 +386,10 @@ void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);
 /* fp32 only: force K-tiles of 16 values (chunks = 2) or 32 (4); 0 restores the
  * per-layer choice.  Tests and tuning, like thhip_conv_set_tuning. */
 void thhip_conv_set_ktile(int chunks);
+/* Force how the tile grid is cut over the eight XCDs: the M tiles into
+ * mparts (1, 2, 4, 8) groups, the N tiles into 8 / mparts ranges; 0 restores
+ * the choice by weight size.  Tests and tuning. */
+void thhip_conv_set_xcd_parts(int mparts);
 
 /* Replaces nn_Linear_updateOutput's 1-D branch (Linear.c:86-90 ->
  * thbasic.c:713-741 -> sgemv.c:48-105): y = bias + W x, W row-major

@@ -46,7 +46,8 @@ def test_conv_f32_ktile_depths_tap_major_and_split(hiplib, oracle):
     """Tap-major fp32 layers (planes in blocks of 32) at both K-tile depths, with forced
     tiles and K splits that start inside a block."""
     g = cases.rng(910)
-    for (B, Ci, H, W, Co, k, dd, pp) in ((2, 32, 9, 10, 70, 3, 1, 1), (1, 96, 7, 7, 130, 3, 2, 1), (3, 64, 6, 5, 64, 1, 1, 0)):
+    for (B, Ci, H, W, Co, k, dd, pp) in ((2, 32, 9, 10, 70, 3, 1, 1), (1, 96, 7, 7, 130, 3, 2, 1), (3, 64, 6, 5, 64, 1, 1, 0),
+                                         (2, 32, 23, 17, 300, 3, 1, 1)):
         x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
         w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
         b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
@@ -57,8 +58,16 @@ def test_conv_f32_ktile_depths_tap_major_and_split(hiplib, oracle):
                 for tune in ((0, 0, 0, 0), (64, 64, 3, 0), (128, 64, 2, 2), (128, 128, 5, 0), (64, 128, 1, 1)):
                     hiplib.thhip_conv_set_tuning(*tune)
                     G.assert_close(G.conv2d(hiplib, x, w, b, (dd, dd), (pp, pp)), want, FP32_TOL, str((chunks, tune)))
+            # every way of cutting the tile grid over the XCDs, with ragged rectangles and a K split
+            hiplib.thhip_conv_set_ktile(0)
+            for parts in (1, 2, 4, 8):
+                hiplib.thhip_conv_set_xcd_parts(parts)
+                for tune in ((64, 64, 0, 0), (64, 64, 2, 0)):
+                    hiplib.thhip_conv_set_tuning(*tune)
+                    G.assert_close(G.conv2d(hiplib, x, w, b, (dd, dd), (pp, pp)), want, FP32_TOL, str((parts, tune)))
         finally:
             hiplib.thhip_conv_set_ktile(0)
+            hiplib.thhip_conv_set_xcd_parts(0)
             hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 

@@ -47,6 +47,7 @@ struct ConvParams {
 	int act;
 	float thr, val;
 	int tiles_m, tiles_n;
+	int mparts;		/* the tile grid is cut mparts x (8 / mparts) over the XCDs */
 	unsigned x_bytes;
 	/* split-K: S workgroups share an output tile, each over a K range */
 	int splitk;
@@ -213,21 +214,33 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wm = wave % WGM, wn = wave / WGM;
 
-	/* XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so
-	 * give each XCD a contiguous run of tiles (M fastest) and let neighbours
-	 * that share an input slab share an L2. */
-	int tile;
+	/* XCD-aware tile order.  Workgroups are dealt round-robin to the 8 XCDs,
+	 * each with its own L2, so every XCD gets one rectangle of the tile grid:
+	 * the M tiles are cut into p.mparts groups and the N tiles into 8 / mparts
+	 * ranges.  One part along M (every XCD: all weight rows, an eighth of the
+	 * positions) reads the least in total, but an XCD's workgroups all run at
+	 * once and sweep every weight row they own, so the launcher raises mparts
+	 * until an XCD's share of the weights fits its L2.  Inside the rectangle
+	 * M runs fastest: neighbours share an input slab. */
+	int tile_m, tile_n, split = 0;
 	{
-		const int nblk = gridDim.x, bid = blockIdx.x;
-		const int xcd = bid & 7, local = bid >> 3;
-		const int q = nblk >> 3, r = nblk & 7;
-		tile = xcd * q + (xcd < r ? xcd : r) + local;
+		const int bid = blockIdx.x;
+		const int xcd = bid & 7;
+		int local = bid >> 3;
+		if (p.splitk > 1) {	/* the S parts of a tile are neighbours in the order */
+			split = local % p.splitk;
+			local /= p.splitk;
+		}
+		const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
+		const int m0 = p.tiles_m * mp / p.mparts, m1 = p.tiles_m * (mp + 1) / p.mparts;
+		const int n0 = p.tiles_n * np / nparts, n1 = p.tiles_n * (np + 1) / nparts;
+		const int mw = m1 - m0;
+		if (local >= mw * (n1 - n0))
+			return;		/* the rectangles differ by a row or column: this slot is empty */
+		tile_m = m0 + local % mw;
+		tile_n = n0 + local / mw;
 	}
-	/* split-K: the S parts of a tile are neighbours in the order */
-	const int split = p.splitk > 1 ? tile % p.splitk : 0;
-	if (p.splitk > 1)
-		tile /= p.splitk;
-	const int tile_m = tile % p.tiles_m, tile_n = tile / p.tiles_m;
+	const int tile = tile_n * p.tiles_m + tile_m;	/* names the tile's split-K scratch */
 
 	/* ---- B gather role ----
 	 * Plane-major input: one output position per thread (lanes run along the
@@ -894,7 +907,15 @@ extern "C" void *thhip_conv_pack_weight(const float *w, int Co, int Ci, int kHW,
 }
 
 /* Experiment / tuning override: 0 = choose automatically. */
-static int g_force_bm, g_force_bn, g_force_splitk, g_force_wgs, g_force_kch;
+static int g_force_bm, g_force_bn, g_force_splitk, g_force_wgs, g_force_kch, g_force_mparts;
+
+/* Force the number of parts the M tiles are cut into over the XCDs (1, 2, 4 or 8); 0 = choose automatically. */
+extern "C" void thhip_conv_set_xcd_parts(int mparts)
+{
+	if (mparts != 0 && mparts != 1 && mparts != 2 && mparts != 4 && mparts != 8)
+		THError("thhip_conv_set_xcd_parts(%d): 0, 1, 2, 4 or 8", mparts);
+	g_force_mparts = mparts;
+}
 
 /* fp32 only: force K-tiles of 16 (chunks = 2) or 32 (4); 0 = choose automatically. */
 extern "C" void thhip_conv_set_ktile(int chunks)
@@ -977,7 +998,23 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 	const size_t tiles = (size_t)p.tiles_m * p.tiles_n;
 	if (p.splitk > 1)
 		conv_scratch(p, tiles, (size_t)BM * BN);
-	dim3 grid((unsigned)(tiles * p.splitk));
+	/* XCD rectangles: as few parts along M as keep an XCD's weight rows within
+	 * about half of its 4 MB L2 */
+	const double wbytes = (double)p.Co * p.K * thhip_esize(DT);
+	p.mparts = 1;
+	while (p.mparts < 8 && p.mparts * 2 <= p.tiles_m && wbytes / p.mparts > 2.5e6)
+		p.mparts *= 2;
+	if (g_force_mparts)
+		p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
+	size_t maxcnt = 0;
+	for (int x = 0; x < 8; x++) {
+		const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
+		const size_t cnt = (size_t)(p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
+			(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
+		if (cnt > maxcnt)
+			maxcnt = cnt;
+	}
+	dim3 grid((unsigned)(8 * maxcnt * p.splitk));
 	const bool tap = conv_tap_major(p.Ci, DT);
 	if (p.y_cl && p.Co % 4)
 		THError("thhip_conv2d: channels-last output needs Co %% 4 == 0 (Co = %d)", p.Co);
