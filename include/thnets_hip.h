@@ -390,6 +390,10 @@ void thhip_conv_set_ktile(int chunks);
  * mparts (1, 2, 4, 8) groups, the N tiles into 8 / mparts ranges; 0 restores
  * the choice by weight size.  Tests and tuning. */
 void thhip_conv_set_xcd_parts(int mparts);
+/* Channels-last inputs whose plane count is a multiple of the K-tile are
+ * gathered with the filter tap tracked on the scalar unit; on = 1 forces the
+ * per-thread tap decode that serves every plane count.  Tests and tuning. */
+void thhip_conv_set_generic_cl(int on);
 
 /* Replaces nn_Linear_updateOutput's 1-D branch (Linear.c:86-90 ->
  * thbasic.c:713-741 -> sgemv.c:48-105): y = bias + W x, W row-major

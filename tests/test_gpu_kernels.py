@@ -232,10 +232,19 @@ def test_conv_half_channels_last(hiplib, oracle, dt):
         base = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, scale=sc)
         G.assert_close(base, want, HALF_TOL, "plane-major")
         orders = [(0, 1)] + ([(1, 0), (1, 1)] if Ci % 8 == 0 else [])
-        for (x_cl, y_cl) in orders:
-            got = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=x_cl, y_cl=y_cl, scale=sc)
-            G.assert_close(got, want, HALF_TOL, str((x_cl, y_cl)))
-            G.assert_close(got, base, 1e-2, "vs plane-major " + str((x_cl, y_cl)))
+        try:
+            for (x_cl, y_cl) in orders:
+                # Ci a multiple of the K-tile: the scalar tap walk, then the per-thread decode
+                for generic in ((0, 1) if x_cl == 1 and Ci % 32 == 0 else (0,)):
+                    hiplib.thhip_conv_set_generic_cl(generic)
+                    for tune in ((0, 0, 0, 0), (128, 128, 2, 0)):
+                        hiplib.thhip_conv_set_tuning(*tune)
+                        got = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=x_cl, y_cl=y_cl, scale=sc)
+                        G.assert_close(got, want, HALF_TOL, str((x_cl, y_cl, generic, tune)))
+                        G.assert_close(got, base, 1e-2, "vs plane-major " + str((x_cl, y_cl, generic, tune)))
+        finally:
+            hiplib.thhip_conv_set_generic_cl(0)
+            hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])

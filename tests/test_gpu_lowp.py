@@ -148,11 +148,15 @@ def test_conv_u8_channels_last_bit_exact(hiplib, oracle, i):
         for tune in ((0, 0, 0, 0), (64, 64, 3, 2), (128, 128, 1, 0), (64, 128, 2, 1), (128, 64, 1, 4)):
             hiplib.thhip_conv_set_tuning(*tune)
             for (x_cl, y_cl) in orders:
-                got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, x_cl=x_cl, y_cl=y_cl)
-                assert np.array_equal(got, want), (tune, x_cl, y_cl, int((got != want).sum()))
-                got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, act=1, thr=thr, val=thr, x_cl=x_cl, y_cl=y_cl)
-                assert np.array_equal(got, oracle.lowp_threshold(want, thr, thr)), (tune, x_cl, y_cl)
+                # Ci a multiple of the K-tile: the scalar tap walk, then the per-thread decode
+                for generic in ((0, 1) if x_cl == 1 and Ci % 64 == 0 else (0,)):
+                    hiplib.thhip_conv_set_generic_cl(generic)
+                    got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, x_cl=x_cl, y_cl=y_cl)
+                    assert np.array_equal(got, want), (tune, x_cl, y_cl, generic, int((got != want).sum()))
+                    got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, act=1, thr=thr, val=thr, x_cl=x_cl, y_cl=y_cl)
+                    assert np.array_equal(got, oracle.lowp_threshold(want, thr, thr)), (tune, x_cl, y_cl, generic)
     finally:
+        hiplib.thhip_conv_set_generic_cl(0)
         hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 

@@ -85,6 +85,7 @@ PROTOTYPES = {
     "thhip_conv2d_affine": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv_set_ktile": (None, [C.c_int]),
     "thhip_conv_set_xcd_parts": (None, [C.c_int]),
+    "thhip_conv_set_generic_cl": (None, [C.c_int]),
     "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_linear_batched_supported": (C.c_int, [C.c_int] * 4),
