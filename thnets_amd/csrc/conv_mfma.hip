@@ -580,10 +580,13 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 	read_frags(0, 0, af[0], bf[0]);
 	static_assert(KCH % 2 == 0, "fragment sets alternate by chunk parity");
 	/* tile kt is in stage st, tile kt+1 in st1, and tile kt+2 goes to st2 */
-	auto step = [&](int kt, auto st, auto st1, auto st2) {
+	auto step = [&](int kt, auto st, auto st1, auto st2, auto steady_) {
+		/* steady: tiles kt+2 and kt+2+PFD exist, no tests (and no branches for
+		 * the instruction scheduler to stop at) */
+		constexpr bool steady = decltype(steady_)::value;
 		/* tile kt+2 was requested a whole step ago: it has had the time to
 		 * arrive, so parking it in LDS does not stall the MFMAs */
-		if (kt + 2 < nkt)
+		if (steady || kt + 2 < nkt)
 			store_tile(st2);
 #pragma unroll
 		for (int r = 0; r + 1 < PFD; r++) {	/* the tiles in flight move up */
@@ -596,13 +599,13 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 				bmask[r][j] = bmask[r + 1][j];
 			}
 		}
-		if (kt + 2 + PFD < nkt)
+		if (steady || kt + 2 + PFD < nkt)
 			load_tile(kt + 2 + PFD, RL{});
 #pragma unroll
 		for (int c = 0; c < KCH; c++) {
 			if (c + 1 < KCH)
 				read_frags(st, c + 1, af[(c + 1) & 1], bf[(c + 1) & 1]);
-			else if (kt + 1 < nkt)
+			else if (steady || kt + 1 < nkt)
 				read_frags(st1, 0, af[0], bf[0]);
 #pragma unroll
 			for (int i = 0; i < TM; i++)
@@ -634,22 +637,27 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 		typedef std::integral_constant<int, 1> S1;
 		typedef std::integral_constant<int, 2> S2;
 		int kt = kt0;
-		for (; kt + 2 < nkt; kt += 3) {
-			step(kt, S0{}, S1{}, S2{});
-			step(kt + 1, S1{}, S2{}, S0{});
-			step(kt + 2, S2{}, S0{}, S1{});
+		for (; kt + 4 + PFD < nkt; kt += 3) {	/* steady state */
+			step(kt, S0{}, S1{}, S2{}, std::true_type{});
+			step(kt + 1, S1{}, S2{}, S0{}, std::true_type{});
+			step(kt + 2, S2{}, S0{}, S1{}, std::true_type{});
+		}
+		for (; kt + 2 < nkt; kt += 3) {		/* the last tiles drain */
+			step(kt, S0{}, S1{}, S2{}, std::false_type{});
+			step(kt + 1, S1{}, S2{}, S0{}, std::false_type{});
+			step(kt + 2, S2{}, S0{}, S1{}, std::false_type{});
 		}
 		if (kt < nkt) {
-			step(kt, S0{}, S1{}, S2{});
+			step(kt, S0{}, S1{}, S2{}, std::false_type{});
 			if (kt + 1 < nkt)
-				step(kt + 1, S1{}, S2{}, S0{});
+				step(kt + 1, S1{}, S2{}, S0{}, std::false_type{});
 		}
 	} else {
 		/* the element-wise gather is long: one copy, stages rotate at run time */
 		int st = 0;
 		for (int kt = kt0; kt < nkt; kt++) {
 			const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
-			step(kt, st, st1, st2);
+			step(kt, st, st1, st2, std::false_type{});
 			st = st1;
 		}
 	}
