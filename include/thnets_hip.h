@@ -255,7 +255,20 @@ void THMakeSpatial(THNETWORK *network, int size);
 /* thapi.c:692-728.  Only switches the module type tag (MM <-> VirtMM);
  * this library carries no direct-convolution path, mm_type 0 is refused. */
 int THUseSpatialConvolutionMM(THNETWORK *network, int mm_type);
-/* thapi.c:601-635 (engine networks only: frees device state). */
+/* thapi.c:244-333 for Torch7 model directories: reads <path>/model.net (an
+ * nn.Sequential saved with torch.save, binary mode, 8- or 4-byte longs) and,
+ * when present, <path>/stat.t7 ({mean = FloatTensor(3), std = FloatTensor(3)})
+ * into a host description (engine ENGINE_CPU) for THCreateHipNetwork /
+ * THCreateHipLowpNetwork.  Returns 0 with the reason in THLastError() when a
+ * file cannot be read; module types the engine does not run are fatal
+ * (thload.c:776).  PyTorch dumps and ONNX files are not read. */
+THNETWORK *THLoadNetwork(const char *path);
+/* A Float / Double tensor saved with torch.save, as a new contiguous host
+ * tensor (what thnets-test.c:166-178 does for `-i input.t7` with loadtorch +
+ * THFloatTensor_newFromObject, thload.c:408-426, 701-711).  0 on failure. */
+THFloatTensor *THLoadTensor(const char *path);
+/* thapi.c:601-635: engine networks (frees device state) and the host networks
+ * THLoadNetwork returns. */
 void THFreeNetwork(THNETWORK *network);
 /* thapi.c:637-640 */
 int THLastError(void);

@@ -170,3 +170,62 @@ def test_vgg16_full_size_properties(hiplib, oracle):
     want = oracle.run_layers(cfg["layers"][:5], cfg["input"][:1])
     G.assert_close(net.module_output(4), want, 2e-5, "first block")
     net.free()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small"])
+def test_loaded_model_directory_runs_like_the_layer_list(hiplib, oracle, tmp_path, name):
+    """THLoadNetwork -> THCreateHipNetwork -> THProcessFloat on a Torch7 model
+    directory gives, bit for bit, what the same weights give when the module array
+    is assembled by hand, in fp32, fp16 and uint8 form."""
+    from thnets_amd import t7
+    cfg = cases.small_networks()[name]
+    t7.save_model_dir(str(tmp_path), cfg["layers"], cfg["mean"], cfg["std"], longsize=4 if name == "tiny_cnn" else 8)
+    G.note("model directory %s" % name)
+    for kw in ({}, {"half": 1}) + (({"lowp_range": 16.0, "make_spatial": 8},) if name == "tiny_cnn" else ()):
+        a = api.HipNetwork(str(tmp_path), **kw)
+        b = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"], **kw)
+        got, want = a.process_float(cfg["input"]), b.process_float(cfg["input"])
+        a.free()
+        b.free()
+        assert got.shape == want.shape and np.array_equal(got, want), kw
+
+
+@pytest.mark.gpu
+def test_command_line_driver(hiplib, oracle, tmp_path):
+    """thnets-hip-test (the counterpart of thnets-test.c) on a model directory and
+    a .t7 input prints the values THProcessFloat returns; a PPM image goes through
+    THProcessImages."""
+    import subprocess
+    from thnets_amd import t7
+    cfg = cases.small_networks()["tiny_cnn"]
+    t7.save_model_dir(str(tmp_path), cfg["layers"], cfg["mean"], cfg["std"])
+    x = cfg["input"][0]
+    t7.save(str(tmp_path / "in.t7"), np.ascontiguousarray(x))
+    exe = os.path.join(os.path.dirname(api.LIB_PATH), "thnets-hip-test")
+    assert os.path.exists(exe), "build it with make -C thnets_amd/csrc"
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    want = net.process_float(np.stack([x, x]))
+    G.note("thnets-hip-test fp32 batch 2")
+    r = subprocess.run([exe, "-m", str(tmp_path), "-i", str(tmp_path / "in.t7"), "-p", "-b", "2", "-r", "2"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    vals = [float(l.split(":")[1]) for l in r.stdout.splitlines() if l.startswith("(")]
+    assert len(vals) == want.size and np.allclose(vals, want, rtol=0, atol=5e-7)
+    assert "1 run processing time:" in r.stdout
+    # an 8-bit image through THProcessImages
+    g = cases.rng(91)
+    img = g.integers(0, 256, (8, 8, 3), dtype=np.uint8)
+    with open(tmp_path / "in.ppm", "wb") as fp:
+        fp.write(b"P6\n# test image\n8 8\n255\n" + img.tobytes())
+    want = net.process_images([img])
+    net.free()
+    G.note("thnets-hip-test ppm")
+    r = subprocess.run([exe, "-m", str(tmp_path), "-i", str(tmp_path / "in.ppm"), "-p", "-L", "4"],
+                       capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    vals = [float(l.split(":")[1]) for l in r.stdout.splitlines() if l.startswith("(")]
+    assert len(vals) == 4 and np.allclose(vals, want[:4], rtol=0, atol=5e-7)
+    # a model directory that does not exist: the reference's message, exit code 0 (thnets-test.c:199)
+    r = subprocess.run([exe, "-m", str(tmp_path / "none"), "-i", "random"], capture_output=True, text=True, timeout=120)
+    assert "The network could not be loaded: -1" in r.stdout

@@ -49,6 +49,8 @@ PROTOTYPES = {
     "THMakeSpatial": (None, [vp, C.c_int]),
     "THUseSpatialConvolutionMM": (C.c_int, [vp, C.c_int]),
     "THFreeNetwork": (None, [vp]),
+    "THLoadNetwork": (vp, [C.c_char_p]),
+    "THLoadTensor": (vp, [C.c_char_p]),
     "THLastError": (C.c_int, []),
     "THCreateHipNetwork": (vp, [vp]),
     "THHipHalfFloat": (C.c_int, [C.c_int]),
@@ -202,28 +204,40 @@ def from_device_dtype(dev, shape, dtype):
 
 
 class HipNetwork:
-    """A network on the engine, made from a layer list (see netbuild)."""
+    """A network on the engine, made from a layer list (see netbuild) or from a
+    Torch7 model directory (``model.net`` + ``stat.t7``, read by ``THLoadNetwork``)."""
 
     def __init__(self, layers, mean=(0.0, 0.0, 0.0), std=(1.0, 1.0, 1.0), half=0, lowp_range=None,
                  make_spatial=None, fold_bn=True):
         self.lib = lib = load_library()
         lib.THInit()
-        self.host = HostNetwork(lib, abi.ABI, resolve_cpu=False).build(layers, mean, std)
+        loaded = None
+        if isinstance(layers, (str, bytes, os.PathLike)):
+            loaded = lib.THLoadNetwork(os.fsencode(layers))
+            if not loaded:
+                raise IOError("THLoadNetwork(%r) failed: error %d" % (layers, lib.THLastError()))
+            self.host = HostNetwork(lib, abi.ABI, resolve_cpu=False)      # only makes host tensors for upload()
+            source = loaded
+        else:
+            self.host = HostNetwork(lib, abi.ABI, resolve_cpu=False).build(layers, mean, std)
+            source = C.addressof(self.host.thnet)
         if make_spatial:
-            lib.THMakeSpatial(C.addressof(self.host.thnet), int(make_spatial))
+            lib.THMakeSpatial(source, int(make_spatial))
         self.half = half
         self.lowp = lowp_range is not None
         if self.lowp:
-            self.handle = lib.THCreateHipLowpNetwork(C.addressof(self.host.thnet), C.c_float(lowp_range))
+            self.handle = lib.THCreateHipLowpNetwork(source, C.c_float(lowp_range))
             self.dtype = abi.THHIP_U8
         else:
             if lib.THHipHalfFloat(half) != 0:
                 raise ValueError("THHipHalfFloat(%r) refused" % half)
             old_fold = lib.THHipFoldBatchNorm(1 if fold_bn else 0)
-            self.handle = lib.THCreateHipNetwork(C.addressof(self.host.thnet))
+            self.handle = lib.THCreateHipNetwork(source)
             lib.THHipFoldBatchNorm(old_fold)
             lib.THHipHalfFloat(0)
             self.dtype = (abi.THHIP_F32, abi.THHIP_F16, abi.THHIP_BF16)[half]
+        if loaded:
+            lib.THFreeNetwork(loaded)      # the engine copied what it needs (thnets-test.c:130-134)
         self.thnet = C.cast(self.handle, C.POINTER(abi.ABI.THNETWORK)).contents
         self._dev_in = None
 
@@ -305,8 +319,7 @@ class HipNetwork:
 
 class thnets:
     """Drop-in for the class in the reference's thnets.py, over the HIP engine.
-    ``LoadNetwork`` takes a layer list instead of a model directory (the .t7 / ONNX
-    loaders are outside this repository's scope)."""
+    ``LoadNetwork`` takes a Torch7 model directory, as there, or a layer list."""
 
     def __init__(self):
         self.net = None

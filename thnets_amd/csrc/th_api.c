@@ -13,9 +13,11 @@
 
 static int lasterror;
 
+/* thapi.c:637-640: the code of the last recoverable failure (loaders, and the
+ * calls this engine does not implement) */
 int THLastError(void)
 {
-	return lasterror;
+	return lasterror ? lasterror : thhip_load_error();
 }
 
 void THInit(void)
@@ -64,6 +66,10 @@ static int engine_of(THNETWORK *network)
 
 void THFreeNetwork(THNETWORK *network)
 {
+	if (network && network->net && network->net->engine == ENGINE_CPU && network->netobj) {
+		thhip_free_loaded_network(network);	/* made by THLoadNetwork */
+		return;
+	}
 	engine_of(network);
 	thhip_sync();
 	thhip_free_network(network->net);
@@ -327,12 +333,16 @@ void THMakeSpatial(THNETWORK *network, int size)
 	for (int i = 0; i < net->nelem; i++) {
 		struct module *m = &net->modules[i];
 		if (m->type == MT_View || m->type == MT_Reshape) {
+			if (network->netobj)		/* loaded network: the library owns the module */
+				THFloatTensor_free(m->output);
 			memmove(m, m + 1, sizeof(*m) * (net->nelem - i - 1));
 			net->nelem--;
 			i--;
 		} else if (m->type == MT_Linear) {
 			THFloatTensor *w = m->Linear.weight, *b = m->Linear.bias;
 			struct SpatialConvolution *c = &m->SpatialConvolution;
+			if (network->netobj)
+				THFloatTensor_free(m->Linear.addBuffer);	/* thapi.c:656; its slot becomes finput */
 			m->type = MT_SpatialConvolutionVirtMM;
 			memset(c, 0, sizeof(*c));
 			c->weight = w;

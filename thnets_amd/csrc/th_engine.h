@@ -48,5 +48,8 @@ struct network *THHip_ToHip(struct network *net, int lowp, float range);
 THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in);
 void thhip_free_network(struct network *net);
 void thhip_storage_release(THFloatStorage *s);
+/* th_load.c */
+int thhip_load_error(void);
+void thhip_free_loaded_network(THNETWORK *n);
 
 #endif
