@@ -72,6 +72,20 @@ struct SpatialConvolution {
 	int dlH, dlW;
 };
 
+/* thnets.h:132-138; weight is [nInputPlane][nOutputPlane][kH][kW] */
+struct SpatialFullConvolution {
+	THFloatTensor *bias, *weight;
+	int dW, dH, padW, padH, kW, kH, nInputPlane, nOutputPlane;
+	int adjW, adjH;
+	THFloatTensor *ones, *columns;
+};
+
+/* thnets.h:191-194: `pooling` names the SpatialMaxPooling whose indices are
+ * used, by the value of that module's `nnmodule` member */
+struct SpatialMaxUnpooling {
+	void *pooling;
+};
+
 struct SpatialMaxPooling {
 	int padW, padH, dW, dH, kW, kH, ceil_mode;
 	int iwidth, iheight;
@@ -178,6 +192,8 @@ struct module {
 	int inputs[MAXMODULEINPUTS];
 	union {
 		struct SpatialConvolution SpatialConvolution;
+		struct SpatialFullConvolution SpatialFullConvolution;
+		struct SpatialMaxUnpooling SpatialMaxUnpooling;
 		struct SpatialMaxPooling SpatialMaxPooling;
 		struct SpatialAveragePooling SpatialAveragePooling;
 		struct Linear Linear;
@@ -435,6 +451,38 @@ void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W, int oH, i
 	int kH, int kW, int dH, int dW, int padH, int padW, int dtype);
 void thhip_pool_outsize(int H, int W, int kH, int kW, int dH, int dW, int padH, int padW, int ceil_mode,
 	int *oH, int *oW);
+/* nn_SpatialMaxPooling_updateOutput including its `indices` output
+ * (SpatialMaxPooling.c:100-114), fp32 / fp16 / bf16: ind[i] = position of the
+ * first maximum inside the input plane (the reference stores position + 1 as a
+ * float), -1 for an empty window. */
+void thhip_maxpool_indices(const void *x, void *y, int *ind, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype);
+/* Replaces nn_SpatialMaxUnpooling_updateOutput (SpatialMaxUnpooling.c:43-120):
+ * x [B][C][oH][oW] and the indices of the pooling described by the geometry
+ * arguments (H x W in, oH x oW out) -> y [B][C][H][W], zero where no window's
+ * maximum sat; of several windows naming one element the last in row-major
+ * order gives the value, as in the reference's serial loop.  An index outside
+ * the plane (THError in the reference) matches nothing. */
+void thhip_maxunpool(const void *x, const int *ind, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype);
+
+/* Replaces nn_SpatialFullConvolution_updateOutput
+ * (SpatialFullConvolution.c:136-250) for fp32 / fp16 / bf16: x [B][Ci][H][W],
+ * w [Ci][Co][kH][kW] -> y [B][Co][oH][oW], oH = (H-1)*dH - 2*padH + kH + adjH.
+ * thhip_fullconv_pack_weight packs the host weights once (device pointer,
+ * thhip_free); thhip_fullconv2d multiplies (the MFMA convolution kernel as a
+ * 1x1 convolution with Co*kH*kW output planes, into `col`: device scratch of
+ * B*Co*kH*kW*H*W elements) and gathers (thhip_col2im, the reference's col2im
+ * :104-134 without scatter).  With a bias the result is beta * sum + bias[o]
+ * -- the reference passes beta = 11 to its bias GEMM (:231-237), so 11
+ * reproduces it and 1 is the textbook operator; without a bias the plain sum.
+ * act / thr / val: fused Threshold as in thhip_conv2d. */
+void *thhip_fullconv_pack_weight(const float *w, int Ci, int Co, int kH, int kW, int dtype);
+void thhip_fullconv2d(const void *x, const void *wp, const float *bias, float beta, void *col, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int adjH, int adjW,
+	int act, float thr, float val, int dtype);
+void thhip_col2im(const void *col, const float *bias, float beta, void *y, int B, int Co, int H, int W,
+	int kH, int kW, int dH, int dW, int padH, int padW, int adjH, int adjW, int act, float thr, float val, int dtype);
 
 /* Replaces nn_SpatialAveragePooling_updateOutput
  * (SpatialAveragePooling.c:71-207). */

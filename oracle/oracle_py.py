@@ -129,6 +129,49 @@ class Oracle:
         self.lib.orc_maxpool_f32(_p(x), _p(y), B, Cn, H, W, oH, oW, kH, kW, dH, dW, padH, padW)
         return y
 
+    def maxpool_indices(self, x, kH, kW, dH, dW, padH=0, padW=0, ceil_mode=0):
+        """(output, indices): indices are float, position of the maximum in the input plane + 1."""
+        x = np.ascontiguousarray(x, np.float32)
+        B, Cn, H, W = x.shape
+        oH, oW = self.pool_outsize(H, W, kH, kW, dH, dW, padH, padW, ceil_mode)
+        y = np.empty((B, Cn, oH, oW), np.float32)
+        ind = np.empty((B, Cn, oH, oW), np.float32)
+        self.lib.orc_maxpool_indices_f32(_p(x), _p(y), _p(ind), B, Cn, H, W, oH, oW, kH, kW, dH, dW, padH, padW)
+        return y, ind
+
+    def maxunpool(self, x, ind, oH, oW):
+        x = np.ascontiguousarray(x, np.float32)
+        ind = np.ascontiguousarray(ind, np.float32)
+        B, Cn, iH, iW = x.shape
+        y = np.empty((B, Cn, oH, oW), np.float32)
+        if self.lib.orc_maxunpool_f32(_p(x), _p(ind), _p(y), B, Cn, iH, iW, oH, oW):
+            raise ValueError("invalid max index")
+        return y
+
+    def fullconv2d(self, x, w, bias, d=(1, 1), pad=(0, 0), adj=(0, 0)):
+        """x [B,Ci,H,W], w [Ci,Co,kH,kW]; the reference's arithmetic (11 * result + bias when there is a bias)."""
+        x = np.ascontiguousarray(x, np.float32)
+        w = np.ascontiguousarray(w, np.float32)
+        B, Ci, H, W = x.shape
+        _, Co, kH, kW = w.shape
+        oH, oW = (H - 1) * d[0] - 2 * pad[0] + kH + adj[0], (W - 1) * d[1] - 2 * pad[1] + kW + adj[1]
+        y = np.empty((B, Co, oH, oW), np.float32)
+        b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+        self.lib.orc_fullconv2d_f32(_p(x), _p(w), _p(b) if b is not None else None, _p(y), B, Ci, H, W, Co, kH, kW,
+                                    d[0], d[1], pad[0], pad[1], adj[0], adj[1])
+        return y
+
+    def fullconv2d_f64(self, x, w, d=(1, 1), pad=(0, 0), adj=(0, 0)):
+        x = np.ascontiguousarray(x, np.float32)
+        w = np.ascontiguousarray(w, np.float32)
+        B, Ci, H, W = x.shape
+        _, Co, kH, kW = w.shape
+        oH, oW = (H - 1) * d[0] - 2 * pad[0] + kH + adj[0], (W - 1) * d[1] - 2 * pad[1] + kW + adj[1]
+        y = np.empty((B, Co, oH, oW), np.float64)
+        self.lib.orc_fullconv2d_f64(_p(x), _p(w), y.ctypes.data_as(C.c_void_p), B, Ci, H, W, Co, kH, kW,
+                                    d[0], d[1], pad[0], pad[1], adj[0], adj[1])
+        return y
+
     def avgpool(self, x, kH, kW, dH, dW, padH=0, padW=0, ceil_mode=0, count_include_pad=1):
         x = np.ascontiguousarray(x, np.float32)
         B, Cn, H, W = x.shape
@@ -193,8 +236,22 @@ class Oracle:
     def run_layers(self, layers, x, collect=None):
         """x: float32 array, 4-D [B,C,H,W] or as produced by earlier layers.  Returns
         the output; ``collect`` (a list) receives every top-level module output."""
-        for spec in layers:
-            x = self._run_one(spec, x)
+        kept = {}       # position of a maxpool -> (indices, input height, input width), for maxunpool
+        for pos, spec in enumerate(layers):
+            if spec["type"] == "maxpool":
+                h, w = x.shape[-2:]
+                x4 = x if x.ndim == 4 else x[None]
+                y, ind = self.maxpool_indices(x4, spec["kH"], spec["kW"], spec["dH"], spec["dW"], spec["padH"], spec["padW"],
+                                              spec.get("ceil_mode", 0))
+                kept[pos] = (ind, h, w)
+                x = y if x.ndim == 4 else y[0]
+            elif spec["type"] == "maxunpool":
+                ind, h, w = kept[spec["pooling"]]
+                x4 = x if x.ndim == 4 else x[None]
+                y = self.maxunpool(x4, ind, h, w)
+                x = y if x.ndim == 4 else y[0]
+            else:
+                x = self._run_one(spec, x)
             if collect is not None:
                 collect.append(x if not isinstance(x, list) else [v.copy() for v in x])
         return x
@@ -204,6 +261,11 @@ class Oracle:
         if k == "conv":
             return self.conv2d(x, spec["weight"], spec["bias"], (spec["dH"], spec["dW"]), (spec["padH"], spec["padW"]),
                                use_unfold=spec.get("mm") == "mm")
+        if k == "fullconv":
+            x4 = x if x.ndim == 4 else x[None]
+            y = self.fullconv2d(x4, spec["weight"], spec.get("bias"), (spec.get("dH", 1), spec.get("dW", 1)),
+                                (spec.get("padH", 0), spec.get("padW", 0)), (spec.get("adjH", 0), spec.get("adjW", 0)))
+            return y if x.ndim == 4 else y[0]
         if k == "linear":
             xs = np.squeeze(x)          # THFloatTensor_squeeze, Linear.c:86
             return self.linear(xs, spec["weight"], spec["bias"])

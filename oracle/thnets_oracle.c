@@ -12,6 +12,11 @@
  *   from the reference sources) on seeded inputs, committed golden vectors
  *   made with it, and closed forms (double precision direct convolution,
  *   delta kernels, 1x1 conv == Linear, brute force on tiny shapes).
+ *   full (transposed) convolution, max pooling indices, max unpooling: the
+ *   reference's compiled CPU library on seeded inputs, and closed forms
+ *   (double precision scatter form of the transposed convolution; it is the
+ *   adjoint of the convolution: <conv(x), y> == <x, fullconv(y)>; unpooling
+ *   of a pooling's own output restores the maxima in place).
  *   lowp quantize / dequantize / threshold / maxpool / softmax: the
  *   reference's lowp_*.c compiled -DLOWP (oracle/_ref, without gemm8.cc).
  *   lowp gemm (orc_lowp_gemm): PARITY UNPINNED against the reference -- the
@@ -391,6 +396,129 @@ void orc_maxpool_f32(const float *x, float *y, int B, int C, int H, int W, int o
 				op[(long)i * oW + j] = m;
 			}
 	}
+}
+
+/* The same with the float `indices` the reference keeps for unpooling
+ * (modules/SpatialMaxPooling.c:100-114): position of the first maximum inside
+ * the input plane, plus one; 0 when the window is empty. */
+void orc_maxpool_indices_f32(const float *x, float *y, float *ind, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW)
+{
+	long p;
+#pragma omp parallel for
+	for (p = 0; p < (long)B * C; p++) {
+		const float *ip = x + p * H * W;
+		float *op = y + p * oH * oW, *np = ind + p * oH * oW;
+		for (int i = 0; i < oH; i++)
+			for (int j = 0; j < oW; j++) {
+				long hs = (long)i * dH - padH, ws = (long)j * dW - padW;
+				long he = ORC_MIN(hs + kH, (long)H), we = ORC_MIN(ws + kW, (long)W);
+				hs = ORC_MAX(hs, 0L);
+				ws = ORC_MAX(ws, 0L);
+				float m = -INFINITY;
+				long at = -1;
+				for (long yy = hs; yy < he; yy++)
+					for (long xx = ws; xx < we; xx++) {
+						float v = ip[yy * W + xx];
+						if (v > m) {
+							m = v;
+							at = yy * W + xx;
+						}
+					}
+				op[(long)i * oW + j] = m;
+				np[(long)i * oW + j] = (float)(at + 1);
+			}
+	}
+}
+
+/* nn_SpatialMaxUnpooling_updateOutput, modules/SpatialMaxUnpooling.c:14-41,
+ * 92-119: the output plane (the pooling's input extent) is zeroed, then every
+ * input element is written at the position its index names, in row-major
+ * order, so of several elements with one index the last one stays.  Returns -1
+ * for an index outside the plane (the reference calls THError). */
+int orc_maxunpool_f32(const float *x, const float *ind, float *y, int B, int C, int iH, int iW, int oH, int oW)
+{
+	int bad = 0;
+	memset(y, 0, sizeof(float) * (size_t)B * C * oH * oW);
+	long p;
+#pragma omp parallel for
+	for (p = 0; p < (long)B * C; p++) {
+		const float *ip = x + p * iH * iW, *np = ind + p * iH * iW;
+		float *op = y + p * oH * oW;
+		for (long e = 0; e < (long)iH * iW; e++) {
+			long at = (long)np[e] - 1;
+			if (at < 0 || at >= (long)oH * oW)
+				bad = 1;
+			else
+				op[at] = ip[e];
+		}
+	}
+	return bad ? -1 : 0;
+}
+
+/* nn_SpatialFullConvolution_updateOutput, modules/SpatialFullConvolution.c:136-250:
+ * per image columns = W^T x (W is [Ci][Co*kH*kW]), col2im (:104-134) adds
+ * columns[(o*kH+kh)*kW+kw][iy*W+ix] into out[o][iy*dH-padH+kh][ix*dW-padW+kw],
+ * then the bias GEMM.  That GEMM is called with beta = 11 (:231-237), so with a
+ * bias the result is 11 * (transposed convolution) + bias; without one the
+ * transposed convolution itself.  oH = (H-1)*dH - 2*padH + kH + adjH. */
+void orc_fullconv2d_f32(const float *x, const float *w, const float *bias, float *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int adjH, int adjW)
+{
+	const int oH = (H - 1) * dH - 2 * padH + kH + adjH, oW = (W - 1) * dW - 2 * padW + kW + adjW;
+	const long M = (long)Co * kH * kW, N = (long)H * W;
+	float *col = malloc(sizeof(float) * M * N);
+	for (int b = 0; b < B; b++) {
+		const float *xb = x + (long)b * Ci * N;
+		float *yb = y + (long)b * Co * oH * oW;
+		long m;
+#pragma omp parallel for
+		for (m = 0; m < M; m++)
+			for (long n = 0; n < N; n++) {
+				float acc = 0;
+				for (int c = 0; c < Ci; c++)
+					acc += w[(long)c * M + m] * xb[(long)c * N + n];
+				col[m * N + n] = acc;
+			}
+		memset(yb, 0, sizeof(float) * (size_t)Co * oH * oW);
+		for (m = 0; m < M; m++) {
+			const int kw = (int)(m % kW), kh = (int)(m / kW % kH), o = (int)(m / kW / kH);
+			for (int iy = 0; iy < H; iy++)
+				for (int ix = 0; ix < W; ix++) {
+					const int oy = iy * dH - padH + kh, ox = ix * dW - padW + kw;
+					if (oy >= 0 && oy < oH && ox >= 0 && ox < oW)
+						yb[((long)o * oH + oy) * oW + ox] += col[m * N + (long)iy * W + ix];
+				}
+		}
+		if (bias)
+			for (int o = 0; o < Co; o++)
+				for (long e = 0; e < (long)oH * oW; e++)
+					yb[(long)o * oH * oW + e] = 11.0f * yb[(long)o * oH * oW + e] + bias[o];
+	}
+	free(col);
+}
+
+/* The transposed convolution in double precision, scatter form straight from
+ * the definition (no columns, no bias rule): for checks against the above. */
+void orc_fullconv2d_f64(const float *x, const float *w, double *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int adjH, int adjW)
+{
+	const int oH = (H - 1) * dH - 2 * padH + kH + adjH, oW = (W - 1) * dW - 2 * padW + kW + adjW;
+	memset(y, 0, sizeof(double) * (size_t)B * Co * oH * oW);
+	for (int b = 0; b < B; b++)
+		for (int c = 0; c < Ci; c++)
+			for (int iy = 0; iy < H; iy++)
+				for (int ix = 0; ix < W; ix++) {
+					const double v = x[(((long)b * Ci + c) * H + iy) * W + ix];
+					for (int o = 0; o < Co; o++)
+						for (int kh = 0; kh < kH; kh++)
+							for (int kw = 0; kw < kW; kw++) {
+								const int oy = iy * dH - padH + kh, ox = ix * dW - padW + kw;
+								if (oy >= 0 && oy < oH && ox >= 0 && ox < oW)
+									y[(((long)b * Co + o) * oH + oy) * oW + ox] +=
+										v * w[(((long)c * Co + o) * kH + kh) * kW + kw];
+							}
+				}
 }
 
 /* nn_SpatialAveragePooling_updateOutput, modules/SpatialAveragePooling.c:156-203:

@@ -111,7 +111,50 @@ def small_networks():
                    {"type": "softmax"}],
         "input": g.uniform(0, 1, (3, 3, 8, 8)).astype(np.float32),
         "mean": (0.4, 0.5, 0.6), "std": (0.2, 0.25, 0.3)}
+    g = rng(601)
+
+    def wgt(*shape):
+        fan = np.prod(shape[1:]) if len(shape) == 4 else shape[0]
+        return (g.standard_normal(shape, dtype=np.float32) * np.float32(np.sqrt(1.0 / fan))).astype(np.float32)
+
+    def fullconv(w, b, d=1, pad=0, adj=0):
+        return {"type": "fullconv", "weight": w, "bias": b, "dW": d, "dH": d, "padW": pad, "padH": pad, "adjW": adj, "adjH": adj}
+    # encoder / decoder: poolings whose indices steer SpatialMaxUnpooling, full convolutions
+    # with and without a bias (the reference scales by 11 when there is one), strides 1 and 2
+    nets["segnet_small"] = {
+        "name": "segnet_small",
+        "layers": [conv(wgt(8, 3, 3, 3), wgt(8) * np.float32(0.1), 1, 1), relu(), maxpool(2, 2),
+                   conv(wgt(16, 8, 3, 3), wgt(16) * np.float32(0.1), 1, 1), relu(), maxpool(3, 2, 1),
+                   fullconv(wgt(16, 16, 3, 3) * np.float32(0.1), wgt(16) * np.float32(0.1), 1, 1),
+                   {"type": "maxunpool", "pooling": 5},
+                   fullconv(wgt(16, 8, 3, 3) * np.float32(0.1), wgt(8) * np.float32(0.1), 1, 1), relu(),
+                   {"type": "maxunpool", "pooling": 2},
+                   fullconv(wgt(8, 4, 2, 2), None, 2, 0),
+                   fullconv(wgt(4, 3, 3, 3) * np.float32(0.1), wgt(3) * np.float32(0.1), 2, 1, 1)],
+        "input": g.uniform(0, 1, (2, 3, 16, 16)).astype(np.float32),
+        "mean": (0.4, 0.5, 0.6), "std": (0.2, 0.25, 0.3)}
     return nets
+
+
+# (B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, adjH, adjW, bias)
+FULLCONV_CASES = [
+    (2, 8, 5, 6, 4, 3, 3, 1, 1, 1, 1, 0, 0, True),
+    (1, 16, 7, 7, 12, 2, 2, 2, 2, 0, 0, 0, 0, False),
+    (3, 5, 4, 9, 7, 3, 3, 2, 2, 1, 1, 1, 1, True),
+    (2, 32, 8, 8, 16, 4, 4, 2, 2, 1, 1, 0, 0, True),
+    (1, 3, 6, 5, 2, 5, 3, 3, 2, 2, 0, 2, 1, False),
+    (2, 64, 12, 12, 3, 2, 2, 2, 2, 0, 0, 0, 0, True),
+]
+
+
+def fullconv_case(i):
+    B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW, aH, aW, has_bias = FULLCONV_CASES[i]
+    g = rng(800 + i)
+    x = g.standard_normal((B, Ci, H, W), dtype=np.float32)
+    w = g.standard_normal((Ci, Co, kH, kW), dtype=np.float32) * np.float32(np.sqrt(1.0 / (Ci * kH * kW)))
+    b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.5) if has_bias else None
+    spec = {"type": "fullconv", "weight": w, "bias": b, "dW": dW, "dH": dH, "padW": pW, "padH": pH, "adjW": aW, "adjH": aH}
+    return x, spec
 
 
 def sample_indices(n, count=4096, seed=7):

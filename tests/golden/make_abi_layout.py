@@ -37,6 +37,9 @@ int main(void)
 	S("SpatialConvolution", struct SpatialConvolution);
 	O("conv_dW", struct SpatialConvolution, dW);
 	O("conv_nOutputPlane", struct SpatialConvolution, nOutputPlane);
+	S("SpatialFullConvolution", struct SpatialFullConvolution);
+	O("fullconv_adjW", struct SpatialFullConvolution, adjW);
+	O("fullconv_ones", struct SpatialFullConvolution, ones);
 	S("SpatialMaxPooling", struct SpatialMaxPooling);
 	O("maxpool_indices", struct SpatialMaxPooling, indices);
 	S("SpatialBatchNormalization", struct SpatialBatchNormalization);

@@ -67,6 +67,17 @@ def main():
         layers = [{"type": "concattable", "branches": [[cases.conv(w, None)] for w in ws[:nb]]}, {"type": "caddtable"}]
         hn = ref.host_network({"layers": layers, "mean": (0, 0, 0), "std": (1, 1, 1)})
         out["caddtable%d" % nb] = ref.forward(hn, xt)
+    for i in range(len(cases.FULLCONV_CASES)):
+        x, spec = cases.fullconv_case(i)
+        out["fullconv%d" % i] = run_single(ref, spec, x)
+    # a pooling with overlapping windows, its indices, and the unpooling of a second tensor by them
+    g = cases.rng(701)
+    xp = g.standard_normal((2, 3, 9, 8), dtype=np.float32)
+    for j, (k, d, pad) in enumerate([(2, 2, 0), (3, 2, 1), (3, 1, 1)]):
+        layers = [cases.maxpool(k, d, pad), {"type": "threshold", "threshold": -0.2, "val": 7.0, "alpha": 0, "inplace": 0},
+                  {"type": "maxunpool", "pooling": 0}]
+        hn = ref.host_network({"layers": layers, "mean": (0, 0, 0), "std": (1, 1, 1)})
+        out["maxunpool%d" % j] = ref.forward(hn, xp)
     for name, cfg in cases.small_networks().items():
         hn = ref.host_network(cfg)
         out["net_" + name] = ref.process_float(hn, cfg["input"])

@@ -45,6 +45,7 @@ int main(void)
 		"\"sizeof_SpatialMaxPooling\": %zu, \"off_maxpool_indices\": %zu, \"off_bn_eps\": %zu,"
 		"\"sizeof_network\": %zu, \"sizeof_THNETWORK\": %zu, \"off_thnetwork_net\": %zu,"
 		"\"off_thnetwork_out\": %zu, \"off_thnetwork_mean\": %zu, \"off_thnetwork_std\": %zu,"
+		"\"sizeof_SpatialFullConvolution\": %zu, \"off_fullconv_adjW\": %zu, \"off_fullconv_ones\": %zu,"
 		"\"n_module_types\": %d, \"MT_Linear\": %d, \"MT_CAddTable\": %d, \"ENGINE_LOWP\": %d}\n",
 		sizeof(THFloatStorage), sizeof(THFloatTensor), sizeof(struct module),
 		offsetof(struct module, SpatialConvolution), offsetof(struct module, output), offsetof(struct module, net),
@@ -52,7 +53,9 @@ int main(void)
 		offsetof(struct SpatialConvolution, nOutputPlane), sizeof(struct SpatialMaxPooling),
 		offsetof(struct SpatialMaxPooling, indices), offsetof(struct SpatialBatchNormalization, eps),
 		sizeof(struct network), sizeof(THNETWORK), offsetof(THNETWORK, net), offsetof(THNETWORK, out),
-		offsetof(THNETWORK, mean), offsetof(THNETWORK, std), MT_Transpose + 1, MT_Linear, MT_CAddTable, ENGINE_LOWP);
+		offsetof(THNETWORK, mean), offsetof(THNETWORK, std), sizeof(struct SpatialFullConvolution),
+		offsetof(struct SpatialFullConvolution, adjW), offsetof(struct SpatialFullConvolution, ones),
+		MT_Transpose + 1, MT_Linear, MT_CAddTable, ENGINE_LOWP);
 	return 0;
 }
 '''

@@ -391,3 +391,74 @@ def test_events_and_profile_counters(hiplib):
     assert n.value == 1 and ms.value > 0
     B, Ci, H, W, Co, kH, kW = 1, 3, 19, 23, 5, 3, 3
     assert work.value == 2.0 * Co * Ci * kH * kW * (B * 19 * 23)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt,tol", [(G.F32, FP32_TOL), (G.F16, HALF_TOL), (G.BF16, HALF_TOL)])
+@pytest.mark.parametrize("i", range(len(cases.FULLCONV_CASES)))
+def test_fullconv_vs_oracle(hiplib, oracle, i, dt, tol):
+    """thhip_fullconv2d (MFMA product + gather col2im) against the restatement of
+    nn_SpatialFullConvolution_updateOutput, with the reference's bias factor (11), the
+    textbook one (1) and a fused threshold."""
+    from thnets_amd import api
+    x, spec = cases.fullconv_case(i)
+    w, b = spec["weight"], spec["bias"]
+    Ci, Co, kH, kW = w.shape
+    B, _, H, W = x.shape
+    d, pad, adj = (spec["dH"], spec["dW"]), (spec["padH"], spec["padW"]), (spec["adjH"], spec["adjW"])
+    xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
+    wr = api.from_device_dtype(api.to_device_dtype(hiplib, w, dt), w.shape, dt)
+    want11 = oracle.fullconv2d(xr, wr, b, d, pad, adj)
+    plain = oracle.fullconv2d(xr, wr, None, d, pad, adj)
+    G.note("fullconv case %d dtype %d" % (i, dt))
+    wp = hiplib.thhip_fullconv_pack_weight(np.ascontiguousarray(w).ctypes.data, Ci, Co, kH, kW, dt)
+    dx = api.to_device_dtype(hiplib, x, dt)
+    db = api.DeviceArray(hiplib, b) if b is not None else None
+    es = 4 if dt == G.F32 else 2
+    col = api.DeviceArray(hiplib, nbytes=B * Co * kH * kW * H * W * es)
+    dy = api.DeviceArray(hiplib, nbytes=want11.size * es)
+    for beta, act, want in ((11.0, 0, want11), (1.0, 0, plain + (b[None, :, None, None] if b is not None else 0)),
+                            (11.0, 1, np.where(want11 > 0.1, want11, -2.0))):
+        hiplib.thhip_fullconv2d(dx.ptr, wp, db.ptr if db else None, beta, col.ptr, dy.ptr, B, Ci, H, W, Co, kH, kW,
+                                d[0], d[1], pad[0], pad[1], adj[0], adj[1], act, 0.1, -2.0, dt)
+        hiplib.thhip_sync()
+        got = api.from_device_dtype(dy, want11.shape, dt)
+        if act and dt != G.F32:
+            # values next to the threshold may fall on either side after rounding
+            near = np.abs(want11 - 0.1) < tol * np.abs(want11).max()
+            got, want = np.where(near, 0, got), np.where(near, 0, want)
+        G.assert_close(got, want, tol, "beta %g act %d" % (beta, act))
+    hiplib.thhip_free(wp)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dt", [G.F32, G.F16, G.BF16])
+def test_maxpool_indices_and_unpool_vs_oracle(hiplib, oracle, dt):
+    """Pooling with indices and the gather form of SpatialMaxUnpooling: bit-exact,
+    including overlapping windows, where the last window in row-major order wins."""
+    from thnets_amd import api
+    g = cases.rng(870)
+    for (B, Cn, H, W, k, d, pad, ceil) in ((2, 3, 9, 8, 2, 2, 0, 0), (2, 5, 9, 8, 3, 2, 1, 0), (1, 4, 7, 7, 3, 1, 1, 0),
+                                           (3, 2, 10, 11, 3, 2, 0, 1), (1, 1, 5, 5, 5, 5, 2, 0)):
+        x = g.standard_normal((B, Cn, H, W), dtype=np.float32)
+        # ties: repeated values inside windows (first maximum wins)
+        x[:, :, ::3, ::2] = np.float32(0.75)
+        xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
+        pooled, ind = oracle.maxpool_indices(xr, k, k, d, d, pad, pad, ceil)
+        oH, oW = pooled.shape[2:]
+        G.note("maxpool_indices/unpool %s dtype %d" % ((B, Cn, H, W, k, d, pad, ceil), dt))
+        es = 4 if dt == G.F32 else 2
+        dx = api.to_device_dtype(hiplib, x, dt)
+        dy = api.DeviceArray(hiplib, nbytes=pooled.size * es)
+        di = api.DeviceArray(hiplib, nbytes=pooled.size * 4)
+        hiplib.thhip_maxpool_indices(dx.ptr, dy.ptr, di.ptr, B, Cn, H, W, oH, oW, k, k, d, d, pad, pad, dt)
+        hiplib.thhip_sync()
+        assert np.array_equal(api.from_device_dtype(dy, pooled.shape, dt), pooled)
+        assert np.array_equal(di.get(pooled.shape, np.int32) + 1, ind.astype(np.int32))
+        v = g.standard_normal(pooled.shape, dtype=np.float32)
+        vr = api.from_device_dtype(api.to_device_dtype(hiplib, v, dt), v.shape, dt)
+        dv = api.to_device_dtype(hiplib, v, dt)
+        du = api.DeviceArray(hiplib, nbytes=x.size * es)
+        hiplib.thhip_maxunpool(dv.ptr, di.ptr, du.ptr, B, Cn, H, W, oH, oW, k, k, d, d, pad, pad, dt)
+        hiplib.thhip_sync()
+        assert np.array_equal(api.from_device_dtype(du, x.shape, dt), oracle.maxunpool(vr, ind, H, W))

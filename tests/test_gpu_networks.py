@@ -34,7 +34,7 @@ def layerwise(net, oracle, cfg, tol, folded_bn=True):
             if i + 2 < len(layers) and layers[i + 2]["type"] == "threshold":
                 want = outs[i + 2]
         elif i + 1 < len(layers) and layers[i + 1]["type"] == "threshold" and (
-                layers[i]["type"] in ("conv", "linear", "caddtable") or layers[i + 1].get("inplace", 1) == 1):
+                layers[i]["type"] in ("conv", "linear", "caddtable", "fullconv") or layers[i + 1].get("inplace", 1) == 1):
             want = outs[i + 1]
         G.assert_close(net.module_output(i).ravel(), np.asarray(want).ravel(), tol, "module %d %s" % (i, layers[i]["type"]))
 
@@ -173,7 +173,7 @@ def test_vgg16_full_size_properties(hiplib, oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small"])
+@pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small", "segnet_small"])
 def test_loaded_model_directory_runs_like_the_layer_list(hiplib, oracle, tmp_path, name):
     """THLoadNetwork -> THCreateHipNetwork -> THProcessFloat on a Torch7 model
     directory gives, bit for bit, what the same weights give when the module array

@@ -59,6 +59,15 @@ def describe(pnet):
                 d[k] = getattr(p, k)
             if name == "MT_SpatialAveragePooling":
                 d["count_include_pad"] = m.SpatialAveragePooling.count_include_pad
+        elif name == "MT_SpatialFullConvolution":
+            c = m.SpatialFullConvolution
+            for k in ("dW", "dH", "padW", "padH", "adjW", "adjH", "kW", "kH", "nInputPlane", "nOutputPlane"):
+                d[k] = getattr(c, k)
+            d["weight"], d["bias"] = _tensor(c.weight), _tensor(c.bias)
+        elif name == "MT_SpatialMaxUnpooling":
+            # which module of this network it names (by that module's loader object)
+            d["pooling"] = [j for j in range(net.nelem) if net.modules[j].nnmodule and
+                            net.modules[j].nnmodule == m.SpatialMaxUnpooling.pooling]
         elif name == "MT_View":
             d["numElements"] = m.View.numElements
         elif name == "MT_SpatialBatchNormalization":
@@ -98,7 +107,7 @@ def built_description(lib, cfg):
     return describe(host.thnet.net), host
 
 
-@pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small"])
+@pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small", "segnet_small"])
 @pytest.mark.parametrize("variant", ["long8", "long4", "conv4d_boolceil"])
 def test_loaded_network_equals_hand_built(lib, tmp_path, name, variant):
     cfg = cases.small_networks()[name]
@@ -231,7 +240,7 @@ def test_python_reader_round_trip(tmp_path):
 
 # ---- the writer against the reference's own reader and CPU forward ----
 
-@pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small"])
+@pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small", "segnet_small"])
 def test_reference_reads_the_same_files(reference, tmp_path, name):
     """The files this repository writes load in the reference (THLoadNetwork,
     thapi.c:244-333) and its CPU forward on them equals its forward on the network

@@ -67,6 +67,14 @@ class Abi:
                 (n, C.c_int) for n in ("dW", "dH", "padW", "padH", "kW", "kH", "nInputPlane", "nOutputPlane",
                                        "refl_pad", "padW2", "padH2", "autopad", "dlH", "dlW")]
 
+        class SpatialFullConvolution(C.Structure):
+            _fields_ = [("bias", PT), ("weight", PT)] + [
+                (n, C.c_int) for n in ("dW", "dH", "padW", "padH", "kW", "kH", "nInputPlane", "nOutputPlane",
+                                       "adjW", "adjH")] + [("ones", PT), ("columns", PT)]
+
+        class SpatialMaxUnpooling(C.Structure):
+            _fields_ = [("pooling", C.c_void_p)]
+
         class SpatialMaxPooling(C.Structure):
             _fields_ = [(n, C.c_int) for n in ("padW", "padH", "dW", "dH", "kW", "kH", "ceil_mode",
                                                "iwidth", "iheight")] + [("indices", PT)] + [
@@ -104,6 +112,8 @@ class Abi:
         class ModuleUnion(C.Union):
             _fields_ = [
                 ("SpatialConvolution", SpatialConvolution),
+                ("SpatialFullConvolution", SpatialFullConvolution),
+                ("SpatialMaxUnpooling", SpatialMaxUnpooling),
                 ("SpatialMaxPooling", SpatialMaxPooling),
                 ("SpatialAveragePooling", SpatialAveragePooling),
                 ("Linear", Linear),
@@ -148,6 +158,8 @@ class Abi:
 
         self.SpatialConvolution = SpatialConvolution
         self.SpatialMaxPooling = SpatialMaxPooling
+        self.SpatialFullConvolution = SpatialFullConvolution
+        self.SpatialMaxUnpooling = SpatialMaxUnpooling
         self.SpatialAveragePooling = SpatialAveragePooling
         self.Linear = Linear
         self.Threshold = Threshold
@@ -180,6 +192,9 @@ class Abi:
             "sizeof_SpatialConvolution": C.sizeof(s),
             "off_conv_dW": s.dW.offset,
             "off_conv_nOutputPlane": s.nOutputPlane.offset,
+            "sizeof_SpatialFullConvolution": C.sizeof(self.SpatialFullConvolution),
+            "off_fullconv_adjW": self.SpatialFullConvolution.adjW.offset,
+            "off_fullconv_ones": self.SpatialFullConvolution.ones.offset,
             "sizeof_SpatialMaxPooling": C.sizeof(self.SpatialMaxPooling),
             "off_maxpool_indices": self.SpatialMaxPooling.indices.offset,
             "sizeof_SpatialBatchNormalization": C.sizeof(self.SpatialBatchNormalization),

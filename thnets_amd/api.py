@@ -86,6 +86,11 @@ PROTOTYPES = {
     "thhip_maxpool_cl": (None, [vp, vp] + [C.c_int] * 13),
     "thhip_conv2d_affine": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv_set_ktile": (None, [C.c_int]),
+    "thhip_maxpool_indices": (None, [vp, vp, vp] + [C.c_int] * 13),
+    "thhip_maxunpool": (None, [vp, vp, vp] + [C.c_int] * 13),
+    "thhip_fullconv_pack_weight": (vp, [vp] + [C.c_int] * 5),
+    "thhip_fullconv2d": (None, [vp, vp, vp, C.c_float, vp, vp] + [C.c_int] * 14 + [C.c_float, C.c_float, C.c_int]),
+    "thhip_col2im": (None, [vp, vp, C.c_float, vp] + [C.c_int] * 13 + [C.c_float, C.c_float, C.c_int]),
     "thhip_conv_set_xcd_parts": (None, [C.c_int]),
     "thhip_conv_set_generic_cl": (None, [C.c_int]),
     "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),

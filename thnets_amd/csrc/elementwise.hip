@@ -6,6 +6,7 @@
  * and writes its output once; lanes run along the innermost (W) dimension.
  */
 #include <float.h>
+#include <stdlib.h>
 #include <string.h>
 #include <math.h>
 #include "thhip_internal.h"
@@ -157,6 +158,202 @@ extern "C" void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W
 	case THHIP_U8: maxpool_kernel<THHIP_U8><<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, p); break;
 	default: THError("thhip_maxpool: unsupported dtype %d", dtype);
 	}
+}
+
+/* Max pooling that also records where each maximum was found, for
+ * SpatialMaxUnpooling: the reference keeps float `indices` (position in the
+ * input plane + 1, SpatialMaxPooling.c:100-114); here an int per output
+ * element, the position itself, -1 for an empty window.  First maximum wins. */
+template <int DT>
+__global__ void maxpool_indices_kernel(const void *x, void *y, int *ind, PoolParams p)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < p.total; i += step) {
+		const int ox = (int)(i % p.oW);
+		const long t = i / p.oW;
+		const int oy = (int)(t % p.oH);
+		const long plane = t / p.oH;
+		int hs = oy * p.dH - p.padH, ws = ox * p.dW - p.padW;
+		const int he = min(hs + p.kH, p.H), we = min(ws + p.kW, p.W);
+		hs = max(hs, 0);
+		ws = max(ws, 0);
+		const long base = plane * p.H * p.W;
+		float m = -INFINITY;	/* SpatialMaxPooling.c:100 */
+		int at = -1;
+		for (int yy = hs; yy < he; yy++)
+			for (int xx = ws; xx < we; xx++) {
+				const float v = ThhipElem<DT>::ld(x, base + (long)yy * p.W + xx);
+				if (v > m) {
+					m = v;
+					at = yy * p.W + xx;
+				}
+			}
+		ThhipElem<DT>::st(y, i, m);
+		ind[i] = at;
+	}
+}
+
+extern "C" void thhip_maxpool_indices(const void *x, void *y, int *ind, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype)
+{
+	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * C * oH * oW };
+	if (p.total <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, thhip_esize(dtype) * ((double)B * C * H * W + (double)p.total) + 4.0 * p.total);
+	THHIP_DISPATCH_FLOAT(dtype, (maxpool_indices_kernel<DT><<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, ind, p)));
+}
+
+/* nn_SpatialMaxUnpooling_updateOutput (SpatialMaxUnpooling.c:14-41, 92-119)
+ * as a gather, so that no two threads write one element: the reference zeroes
+ * the output plane and then writes every input element at its index in
+ * row-major order, the last writer staying.  An output element therefore holds
+ * the input of the last pooling window (row-major) whose maximum sat there;
+ * only the windows that contain the element can name it.  p describes the
+ * pooling: H x W its input (this output), oH x oW its output (this input). */
+template <int DT>
+__global__ void maxunpool_kernel(const void *x, const int *ind, void *y, PoolParams p)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < p.total; i += step) {
+		const int px = (int)(i % p.W);
+		const long t = i / p.W;
+		const int py = (int)(t % p.H);
+		const long plane = t / p.H;
+		const int at = py * p.W + px;
+		/* windows row r covers rows r*dH - padH .. r*dH - padH + kH - 1 */
+		const int r1 = min((py + p.padH) / p.dH, p.oH - 1), c1 = min((px + p.padW) / p.dW, p.oW - 1);
+		const int r0 = max(0, (py + p.padH - p.kH + p.dH) / p.dH), c0 = max(0, (px + p.padW - p.kW + p.dW) / p.dW);
+		const long base = plane * p.oH * p.oW;
+		float v = 0;
+		bool found = false;
+		for (int r = r1; r >= r0 && !found; r--)
+			for (int c = c1; c >= c0; c--)
+				if (ind[base + (long)r * p.oW + c] == at) {
+					v = ThhipElem<DT>::ld(x, base + (long)r * p.oW + c);
+					found = true;
+					break;
+				}
+		ThhipElem<DT>::st(y, i, v);
+	}
+}
+
+extern "C" void thhip_maxunpool(const void *x, const int *ind, void *y, int B, int C, int H, int W, int oH, int oW,
+	int kH, int kW, int dH, int dW, int padH, int padW, int dtype)
+{
+	PoolParams p = { C, H, W, oH, oW, kH, kW, dH, dW, padH, padW, (long)B * C * H * W };
+	if (p.total <= 0)
+		return;
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, thhip_esize(dtype) * ((double)B * C * oH * oW + (double)p.total) + 4.0 * B * C * oH * oW);
+	THHIP_DISPATCH_FLOAT(dtype, (maxunpool_kernel<DT><<<ew_grid(p.total), dim3(EW_THREADS), 0, thhip_stream()>>>(x, ind, y, p)));
+}
+
+/* col2im of nn_SpatialFullConvolution_updateOutput (SpatialFullConvolution.c:104-134)
+ * as a gather, with the bias step (:225-237) and an optional threshold fused:
+ * columns [B][Co*kH*kW][H*W] (the product of the transposed weights with the
+ * input planes) -> y [B][Co][oH][oW],
+ *   y = beta * sum_{kh,kw} columns[(o*kH+kh)*kW+kw][iy*W+ix] + bias[o],  oy = iy*dH - padH + kh, ox = ix*dW - padW + kw
+ * (no bias: the plain sum).  The taps are added in the reference's order. */
+struct Col2imParams {
+	int Co, H, W, oH, oW, kH, kW, dH, dW, padH, padW;
+	long total;
+	float beta;
+	int act;
+	float thr, val;
+};
+
+/* A thread makes the dW neighbouring outputs ox = xb*dW .. xb*dW + dW - 1 of
+ * one row: which taps (kh, kw) reach an output depends only on (oy + padH) mod
+ * dH and (ox + padW) mod dW, so all lanes of a wave (consecutive xb, one oy)
+ * walk the same taps, read consecutive column elements and together write one
+ * contiguous stretch of the output row. */
+template <int DT>
+__global__ void col2im_kernel(const void *col, const float *bias, void *y, Col2imParams p)
+{
+	const int kHW = p.kH * p.kW;
+	const long HW = (long)p.H * p.W;
+	const unsigned nxb = (p.oW + p.dW - 1) / p.dW;
+	const unsigned groups = (unsigned)p.total;	/* (b, o, oy, xb), fewer than 2^31 */
+	const unsigned step = gridDim.x * blockDim.x;
+	for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < groups; i += step) {
+		const unsigned xb = i % nxb;
+		unsigned t = i / nxb;
+		const int oy = (int)(t % (unsigned)p.oH);
+		t /= (unsigned)p.oH;		/* b * Co + o */
+		const int o = (int)(t % (unsigned)p.Co);
+		const long cbase = (long)t * kHW * HW;
+		const float bo = bias ? bias[o] : 0.0f;
+		/* tap kh = ry + n*dH reads row qy - n; the same along x */
+		const int qy = (oy + p.padH) / p.dH, ry = oy + p.padH - qy * p.dH;
+		for (int rx = 0; rx < p.dW; rx++) {
+			const int ox = (int)xb * p.dW + rx;
+			if (ox >= p.oW)
+				break;
+			const int cx = rx + p.padW;	/* the same for every lane */
+			const int qx = (int)xb + cx / p.dW, rxx = cx % p.dW;
+			float acc = 0;
+			for (int n = 0, kh = ry; kh < p.kH && n <= qy; n++, kh += p.dH) {
+				const int iy = qy - n;
+				if (iy >= p.H)
+					continue;
+				const long rbase = cbase + (long)kh * p.kW * HW + (long)iy * p.W;
+				for (int m = 0, kw = rxx; kw < p.kW && m <= qx; m++, kw += p.dW) {
+					const int ix = qx - m;
+					if (ix >= p.W)
+						continue;
+					acc += ThhipElem<DT>::ld(col, rbase + (long)kw * HW + ix);
+				}
+			}
+			float v = bias ? p.beta * acc + bo : acc;
+			if (p.act)
+				v = v > p.thr ? v : p.val;
+			ThhipElem<DT>::st(y, ((long)t * p.oH + oy) * p.oW + ox, v);
+		}
+	}
+}
+
+extern "C" void thhip_col2im(const void *col, const float *bias, float beta, void *y, int B, int Co, int H, int W,
+	int kH, int kW, int dH, int dW, int padH, int padW, int adjH, int adjW, int act, float thr, float val, int dtype)
+{
+	const int oH = (H - 1) * dH - 2 * padH + kH + adjH, oW = (W - 1) * dW - 2 * padW + kW + adjW;
+	if (oH < 1 || oW < 1 || dH < 1 || dW < 1)
+		THError("thhip_col2im: output %dx%d", oH, oW);
+	const long groups = (long)B * Co * oH * ((oW + dW - 1) / dW);
+	if (groups >= (1L << 31))
+		THError("thhip_col2im: %ld output groups (at most 2^31 - 1)", groups);
+	Col2imParams p = { Co, H, W, oH, oW, kH, kW, dH, dW, padH, padW, groups, beta, act, thr, val };
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, thhip_esize(dtype) * ((double)B * Co * kH * kW * H * W + (double)B * Co * oH * oW));
+	THHIP_DISPATCH_FLOAT(dtype, (col2im_kernel<DT><<<ew_grid(groups), dim3(EW_THREADS), 0, thhip_stream()>>>(col, bias, y, p)));
+}
+
+/* Weights of a full convolution, [Ci][Co][kH][kW] host floats, as the packed
+ * operand of the 1x1 convolution that makes the columns: row (o*kH+kh)*kW+kw
+ * holds the Ci factors of that output tap (the reference multiplies with the
+ * transposed weight matrix, SpatialFullConvolution.c:204-212). */
+extern "C" void *thhip_fullconv_pack_weight(const float *w, int Ci, int Co, int kH, int kW, int dtype)
+{
+	const long M = (long)Co * kH * kW;
+	float *wt = (float *)malloc(sizeof(float) * M * Ci);
+	if (!wt)
+		THError("thhip_fullconv_pack_weight: out of memory");
+	for (int c = 0; c < Ci; c++)
+		for (long m = 0; m < M; m++)
+			wt[m * Ci + c] = w[(long)c * M + m];
+	void *wp = thhip_conv_pack_weight(wt, (int)M, Ci, 1, dtype);
+	free(wt);
+	return wp;
+}
+
+/* nn_SpatialFullConvolution_updateOutput (SpatialFullConvolution.c:136-250):
+ * columns = 1x1 convolution with the packed transposed weights (the MFMA
+ * kernel; col is scratch for B*Co*kH*kW*H*W elements), then thhip_col2im. */
+extern "C" void thhip_fullconv2d(const void *x, const void *wp, const float *bias, float beta, void *col, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int adjH, int adjW,
+	int act, float thr, float val, int dtype)
+{
+	thhip_conv2d(x, wp, 0, col, B, Ci, H, W, Co * kH * kW, 1, 1, 1, 1, 0, 0, 0, 0, 0, dtype);
+	thhip_col2im(col, bias, beta, y, B, Co, H, W, kH, kW, dH, dW, padH, padW, adjH, adjW, act, thr, val, dtype);
 }
 
 /* The same pooling on channels-last codes [B][H][W][C], C % 4 == 0: a thread

@@ -254,12 +254,84 @@ static THFloatTensor *Hip_SpatialMaxPooling_updateOutput(struct module *m, THFlo
 		THError("SpatialMaxPooling: input %dx%d smaller than the window", p.H, p.W);
 	const void *x = thhip_tensor_ptr(in, hn->dtype);
 	void *y = planes_out(m, hn->dtype, &p, oH, oW);
-	if (hn->cur_cl)
+	struct hipmod *hm = hipmod_of(m);
+	if (hm->want_indices) {
+		/* a SpatialMaxUnpooling later in this network scatters by these
+		 * (SpatialMaxPooling.c:213-217 keeps them in every forward) */
+		const size_t need = sizeof(int) * (size_t)p.B * p.C * oH * oW;
+		if (hn->cur_cl)
+			THError("HIP engine: a pooling that keeps indices got channels-last input");
+		if (hm->pool_ind_cap < need) {
+			thhip_free(hm->pool_ind);
+			hm->pool_ind = thhip_malloc(need);
+			hm->pool_ind_cap = need;
+		}
+		thhip_maxpool_indices(x, y, hm->pool_ind, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH,
+			q->padW, hn->dtype);
+	} else if (hn->cur_cl)
 		thhip_maxpool_cl(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, hn->dtype);
 	else
 		thhip_maxpool(x, y, p.B, p.C, p.H, p.W, oH, oW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, hn->dtype);
 	if (oH * oW == 1)
 		hn->cur_cl = 0;		/* one pixel per plane: both orders coincide */
+	return m->output;
+}
+
+/* SpatialMaxUnpooling.c:43-120: the output has the extent the paired pooling
+ * saw at its last forward; its indices say where each value goes. */
+static THFloatTensor *Hip_SpatialMaxUnpooling_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	struct module *pm = &hn->pub.modules[hm->pool_index];
+	struct hipmod *ph = &hn->hm[hm->pool_index];
+	const struct SpatialMaxPooling *q = &pm->SpatialMaxPooling;
+	struct planes p = planes_of(in, "SpatialMaxUnpooling");
+	THFloatTensor *po = pm->output;
+	if (!ph->pool_ind || !po || po->nDimension != in->nDimension)
+		THError("Invalid input size w.r.t current indices size");	/* :73-74 */
+	for (int i = 0; i < in->nDimension; i++)
+		if (po->size[i] != in->size[i])
+			THError("Invalid input size w.r.t current indices size");
+	if (hn->cur_cl)
+		THError("HIP engine: SpatialMaxUnpooling got channels-last input");
+	void *y = planes_out(m, hn->dtype, &p, q->iheight, q->iwidth);
+	thhip_maxunpool(thhip_tensor_ptr(in, hn->dtype), ph->pool_ind, y, p.B, p.C, q->iheight, q->iwidth, p.H, p.W,
+		q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, hn->dtype);
+	return m->output;
+}
+
+/* SpatialFullConvolution.c:136-250.  With a bias the reference's bias GEMM
+ * scales the transposed convolution by its beta argument, 11 (:231-237). */
+#define FULLCONV_BIAS_BETA 11.0f
+
+static THFloatTensor *Hip_SpatialFullConvolution_updateOutput(struct module *m, THFloatTensor *in)
+{
+	struct hipnet *hn = hipnet_of(m);
+	struct hipmod *hm = hipmod_of(m);
+	const struct SpatialFullConvolution *c = &m->SpatialFullConvolution;
+	const int dt = hn->dtype;
+	struct planes p = planes_of(in, "SpatialFullConvolution");
+	if (p.C != c->nInputPlane)
+		THError("input channels and nInputPlane dont match");	/* :160-166 */
+	if (hn->cur_cl)
+		THError("HIP engine: SpatialFullConvolution got channels-last input");
+	const int oW = (p.W - 1) * c->dW - 2 * c->padW + c->kW + c->adjW;
+	const int oH = (p.H - 1) * c->dH - 2 * c->padH + c->kH + c->adjH;
+	if (oW < 1 || oH < 1)
+		THError("SpatialFullConvolution: output size %dx%d is too small", oH, oW);
+	const size_t need = (size_t)p.B * c->nOutputPlane * c->kH * c->kW * p.H * p.W * esize_of(dt);
+	if (hm->col_cap < need) {
+		thhip_free(hm->col);
+		hm->col = thhip_malloc(need);
+		hm->col_cap = need;
+	}
+	struct planes po = p;
+	po.C = c->nOutputPlane;
+	void *y = planes_out(m, dt, &po, oH, oW);
+	thhip_fullconv2d(thhip_tensor_ptr(in, dt), hm->wpacked, hm->bias, FULLCONV_BIAS_BETA, hm->col, y, p.B, p.C, p.H, p.W,
+		c->nOutputPlane, c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, c->adjH, c->adjW, hm->fused_act, hm->thr,
+		hm->val, dt);
 	return m->output;
 }
 
@@ -801,6 +873,46 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 		}
 		break;
 	}
+	case MT_SpatialFullConvolution: {
+		if (lowp)
+			THError("MT_SpatialFullConvolution not supported in Lowp");
+		struct SpatialFullConvolution *c = &sm->SpatialFullConvolution;
+		THFloatTensor *w = c->weight;
+		if (!w || w->nDimension != 4 || c->dW < 1 || c->dH < 1)
+			THError("SpatialFullConvolution needs a 4-D weight [nInputPlane][nOutputPlane][kH][kW] and positive strides");
+		/* the weight's own extents rule (SpatialFullConvolution.c:153-154) */
+		m->SpatialFullConvolution.nInputPlane = (int)w->size[0];
+		m->SpatialFullConvolution.nOutputPlane = (int)w->size[1];
+		m->SpatialFullConvolution.kH = (int)w->size[2];
+		m->SpatialFullConvolution.kW = (int)w->size[3];
+		if (!contiguous_host_floats(w, "full convolution weight", -1))
+			THError("SpatialFullConvolution without weights");
+		hm->wpacked = thhip_fullconv_pack_weight(THFloatTensor_data(w), (int)w->size[0], (int)w->size[1], (int)w->size[2],
+			(int)w->size[3], dtype);
+		hm->bias = upload_floats(c->bias, "full convolution bias", w->size[1]);
+		m->SpatialFullConvolution.weight = m->SpatialFullConvolution.bias = 0;
+		m->SpatialFullConvolution.ones = m->SpatialFullConvolution.columns = 0;
+		m->updateOutput = Hip_SpatialFullConvolution_updateOutput;
+		break;
+	}
+	case MT_SpatialMaxUnpooling: {
+		if (lowp)
+			THError("MT_SpatialMaxUnpooling not supported in Lowp");
+		/* SpatialMaxUnpooling.c:63-72: the pooling is looked up among the
+		 * modules of the same network by its loader object */
+		hm->pool_index = -1;
+		for (int j = 0; j < src->nelem; j++)
+			if (src->modules[j].type == MT_SpatialMaxPooling && sm->SpatialMaxUnpooling.pooling &&
+			    src->modules[j].nnmodule == sm->SpatialMaxUnpooling.pooling) {
+				hm->pool_index = j;
+				break;
+			}
+		if (hm->pool_index < 0)
+			THError("SpatialMaxUnpooling: its SpatialMaxPooling is not a module of the same network");
+		hn->hm[hm->pool_index].want_indices = 1;
+		m->updateOutput = Hip_SpatialMaxUnpooling_updateOutput;
+		break;
+	}
 	case MT_Threshold:
 		m->updateOutput = lowp ? HipLowp_Threshold_updateOutput : Hip_Threshold_updateOutput;
 		break;
@@ -901,7 +1013,7 @@ static void plan_channels_last(struct hipnet *hn, struct network *src)
 				hm->in_cl = 1;
 			}
 			prev = i;
-		} else if (m->type != MT_Threshold && m->type != MT_SpatialMaxPooling && m->type != MT_Dropout &&
+		} else if (m->type != MT_Threshold && !(m->type == MT_SpatialMaxPooling && !hm->want_indices) && m->type != MT_Dropout &&
 			m->type != MT_Identity && !(m->type == MT_SpatialBatchNormalization && hm->passthrough))
 			prev = -1;
 	}
@@ -1008,7 +1120,7 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 		struct module *t = &hn->pub.modules[ti];
 		if (!foldable_threshold(t))
 			continue;
-		if (is_conv_type(m->type)) {
+		if (is_conv_type(m->type) || (m->type == MT_SpatialFullConvolution && ti == i + 1)) {
 			hn->hm[i].fused_act = 1;
 			hn->hm[i].thr = t->Threshold.threshold;
 			hn->hm[i].val = t->Threshold.val;
@@ -1052,6 +1164,8 @@ void thhip_free_network(struct network *net)
 		thhip_free(hm->addend);
 		thhip_free(hm->wrow_u8);
 		thhip_free(hm->rowsum_u8);
+		thhip_free(hm->col);
+		thhip_free(hm->pool_ind);
 		for (int j = 0; j < 4; j++)
 			thhip_free(hm->bn[j]);
 	}

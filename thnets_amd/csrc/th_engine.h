@@ -24,6 +24,13 @@ struct hipmod {
 	unsigned char *wrow_u8;	/* row-major weight codes for one-position layers (device) */
 	int *rowsum_u8;		/* their re-centred row sums (device) */
 	unsigned char *wq_host;	/* weight codes on the host, only while the network is being built */
+	/* SpatialFullConvolution: columns scratch; SpatialMaxPooling feeding a SpatialMaxUnpooling: its indices */
+	void *col;
+	size_t col_cap;
+	int *pool_ind;
+	size_t pool_ind_cap;
+	int want_indices;	/* a SpatialMaxUnpooling of this network reads this pooling's indices */
+	int pool_index;		/* SpatialMaxUnpooling: position of its pooling in the network */
 	int in_cl, out_cl;	/* input / output codes are channels-last [B][H][W][C] in memory */
 	int x_layout;		/* how the convolution reads its input: thhip_conv_pack_weight_u8_layout */
 	float wm, wsub;		/* weight quantisation */

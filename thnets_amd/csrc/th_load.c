@@ -523,6 +523,14 @@ static void free_bn(struct module *m)
 	THFloatTensor_free(m->SpatialBatchNormalization.bias);
 }
 
+static void free_fullconv(struct module *m)
+{
+	THFloatTensor_free(m->SpatialFullConvolution.bias);
+	THFloatTensor_free(m->SpatialFullConvolution.weight);
+	THFloatTensor_free(m->SpatialFullConvolution.ones);
+	THFloatTensor_free(m->SpatialFullConvolution.columns);
+}
+
 static void free_host_network(struct network *net);
 
 static void free_container(struct module *m)
@@ -645,6 +653,34 @@ static void load_module(struct module *m, const struct t7value *o)
 		m->Sequential.net = network_of(o);
 		if (!m->Sequential.net)
 			THError("%s without a module list", cls);
+	} else if (!strcmp(cls, "nn.SpatialFullConvolution")) {
+		struct SpatialFullConvolution *c = &m->SpatialFullConvolution;
+		m->type = MT_SpatialFullConvolution;	/* modules/SpatialFullConvolution.c:12-35 */
+		m->nnfree = free_fullconv;
+		c->padW = (int)field_number(o, "padW");
+		c->padH = (int)field_number(o, "padH");
+		c->adjW = (int)field_number(o, "adjW");
+		c->adjH = (int)field_number(o, "adjH");
+		c->dW = (int)field_number(o, "dW");
+		c->dH = (int)field_number(o, "dH");
+		c->kW = (int)field_number(o, "kW");
+		c->kH = (int)field_number(o, "kH");
+		c->nInputPlane = (int)field_number(o, "nInputPlane");
+		c->nOutputPlane = (int)field_number(o, "nOutputPlane");
+		c->bias = field_tensor(o, "bias", cls);
+		c->weight = field_tensor(o, "weight", cls);
+		c->columns = THFloatTensor_new();
+		c->ones = THFloatTensor_new();
+		if (!c->weight->storage || c->weight->nDimension != 4)
+			THError("nn.SpatialFullConvolution: weight must be a 4-D tensor");
+	} else if (!strcmp(cls, "nn.SpatialMaxUnpooling")) {
+		/* modules/SpatialMaxUnpooling.c:4-12: the pooling module is named by its
+		 * loader object, which SpatialMaxPooling modules carry in `nnmodule` */
+		const struct t7value *pool = field(o, "pooling");
+		if (!pool || pool->kind != T7_OBJECT)
+			THError("nn.SpatialMaxUnpooling without its pooling module");
+		m->type = MT_SpatialMaxUnpooling;
+		m->SpatialMaxUnpooling.pooling = (void *)pool;
 	} else if (!strcmp(cls, "nn.CAddTable"))
 		m->type = MT_CAddTable;
 	else if (!strcmp(cls, "nn.CSubTable"))

@@ -21,6 +21,8 @@ A layer list is a list of dicts; ``type`` selects the module:
     dropout     p inplace v2
     sequential  layers=[...]
     concattable branches=[[...], [...]]
+    fullconv    weight [Ci,Co,kH,kW], bias [Co] | None, dW dH padW padH adjW adjH
+    maxunpool   pooling=<position of its maxpool in the same list>
     caddtable | csubtable
 """
 import ctypes as C
@@ -42,6 +44,8 @@ CPU_UPDATE = {
     "dropout": "nn_Dropout_updateOutput",
     "sequential": "nn_Sequential_updateOutput",
     "concattable": "nn_ConcatTable_updateOutput",
+    "fullconv": "nn_SpatialFullConvolution_updateOutput",
+    "maxunpool": "nn_SpatialMaxUnpooling_updateOutput",
     "caddtable": "nn_CAddTable_updateOutput",
     "csubtable": "nn_CAddTable_updateOutput",
 }
@@ -175,6 +179,24 @@ class HostNetwork:
                 # each branch is one module of the table's network; a list becomes a Sequential
                 branches = [b[0] if len(b) == 1 else {"type": "sequential", "layers": b} for b in spec["branches"]]
                 m.ConcatTable.net = self._network(branches)
+            elif kind == "fullconv":
+                w = np.asarray(spec["weight"], dtype=np.float32)
+                ci, co, kh, kw = w.shape
+                m.type = MT["MT_SpatialFullConvolution"]
+                c = m.SpatialFullConvolution
+                c.weight = self.tensor(w)
+                c.bias = self.tensor(spec.get("bias"))
+                c.ones = self._new_lib_tensor()
+                c.columns = self._new_lib_tensor()
+                c.dW, c.dH, c.padW, c.padH = spec.get("dW", 1), spec.get("dH", 1), spec.get("padW", 0), spec.get("padH", 0)
+                c.adjW, c.adjH = spec.get("adjW", 0), spec.get("adjH", 0)
+                c.kW, c.kH, c.nInputPlane, c.nOutputPlane = kw, kh, ci, co
+            elif kind == "maxunpool":
+                # names its pooling (a position in this list) by that module's nnmodule tag
+                m.type = MT["MT_SpatialMaxUnpooling"]
+                tag = 0x7000 + spec["pooling"]
+                mods[spec["pooling"]].nnmodule = tag
+                m.SpatialMaxUnpooling.pooling = tag
             elif kind == "caddtable":
                 m.type = MT["MT_CAddTable"]
             elif kind == "csubtable":

@@ -308,6 +308,12 @@ def module_of(spec, conv_as_4d=False, boolean_ceil=False):
     if kind == "concattable":
         branches = [b[0] if len(b) == 1 else {"type": "sequential", "layers": b} for b in spec["branches"]]
         return Obj("nn.ConcatTable", modules=[module_of(b, conv_as_4d, boolean_ceil) for b in branches])
+    if kind == "fullconv":
+        w = _f32(spec["weight"])
+        ci, co, kh, kw = w.shape
+        return Obj("nn.SpatialFullConvolution", padW=spec.get("padW", 0), padH=spec.get("padH", 0), dW=spec.get("dW", 1),
+                   dH=spec.get("dH", 1), adjW=spec.get("adjW", 0), adjH=spec.get("adjH", 0), kW=kw, kH=kh, nInputPlane=ci,
+                   nOutputPlane=co, weight=w, bias=None if spec.get("bias") is None else _f32(spec["bias"]))
     if kind == "caddtable":
         return Obj("nn.CAddTable", inplace=False)
     if kind == "csubtable":
@@ -316,7 +322,15 @@ def module_of(spec, conv_as_4d=False, boolean_ceil=False):
 
 
 def sequential_of(layers, conv_as_4d=False, boolean_ceil=False):
-    return Obj("nn.Sequential", modules=[module_of(s, conv_as_4d, boolean_ceil) for s in layers])
+    """A ``maxunpool`` layer names its pooling by position in the same list; in the
+    file it holds a reference to that very nn.SpatialMaxPooling object."""
+    mods = []
+    for s in layers:
+        if s["type"] == "maxunpool":
+            mods.append(Obj("nn.SpatialMaxUnpooling", pooling=mods[s["pooling"]]))
+        else:
+            mods.append(module_of(s, conv_as_4d, boolean_ceil))
+    return Obj("nn.Sequential", modules=mods)
 
 
 def save_model_dir(path, layers, mean=None, std=None, longsize=8, conv_as_4d=False, boolean_ceil=False):
