@@ -462,3 +462,17 @@ def test_maxpool_indices_and_unpool_vs_oracle(hiplib, oracle, dt):
         hiplib.thhip_maxunpool(dv.ptr, di.ptr, du.ptr, B, Cn, H, W, oH, oW, k, k, d, d, pad, pad, dt)
         hiplib.thhip_sync()
         assert np.array_equal(api.from_device_dtype(du, x.shape, dt), oracle.maxunpool(vr, ind, H, W))
+
+
+@pytest.mark.gpu
+def test_maxpool_2x2_vector_path(hiplib, oracle):
+    """2x2 / stride 2 pooling of fp32 planes with a width that is a multiple of four
+    takes 16-byte loads; widths and heights that do not qualify take the general
+    kernel.  Both bit-exact, -inf and large negative values included."""
+    g = cases.rng(880)
+    for (B, Cn, H, W) in ((2, 3, 8, 8), (1, 5, 6, 12), (3, 2, 224, 224), (2, 2, 7, 8), (2, 2, 8, 6), (1, 1, 2, 4)):
+        x = g.standard_normal((B, Cn, H, W), dtype=np.float32)
+        x[0, 0, :2, :4] = np.float32(-3e38)
+        oH, oW = oracle.pool_outsize(H, W, 2, 2, 2, 2, 0, 0, 0)
+        y = G.unary(hiplib, hiplib.thhip_maxpool, x, (B, Cn, oH, oW), G.F32, B, Cn, H, W, oH, oW, 2, 2, 2, 2, 0, 0, G.F32)
+        assert np.array_equal(y, oracle.maxpool(x, 2, 2, 2, 2)), (B, Cn, H, W)

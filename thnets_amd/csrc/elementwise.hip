@@ -142,6 +142,38 @@ __global__ void maxpool_kernel(const void *x, void *y, PoolParams p)
 	}
 }
 
+/* The common 2x2 / stride 2 / no padding pooling of fp32 planes whose width is a
+ * multiple of four: a thread reads four columns of two rows as two 16-byte
+ * vectors and writes two outputs.  Same comparisons in the same order as the
+ * general kernel. */
+__global__ void maxpool_f32_2x2_kernel(const floatx4 *x, float2 *y, int H4, int oH, int oW2, long total2)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total2; i += step) {
+		const int xq = (int)(i % oW2);
+		const long t = i / oW2;
+		const int oy = (int)(t % oH);
+		const long plane = t / oH;
+		const floatx4 *row = x + (plane * H4 * 2 + (long)oy * 2) * oW2 + xq;	/* W/4 == oW/2 vectors per row */
+		const floatx4 a = row[0], b = row[oW2];
+		float2 o;
+		float m = -FLT_MAX;
+		m = a[0] > m ? a[0] : m;
+		m = a[1] > m ? a[1] : m;
+		m = b[0] > m ? b[0] : m;
+		m = b[1] > m ? b[1] : m;
+		o.x = m;
+		m = -FLT_MAX;
+		m = a[2] > m ? a[2] : m;
+		m = a[3] > m ? a[3] : m;
+		m = b[2] > m ? b[2] : m;
+		m = b[3] > m ? b[3] : m;
+		o.y = m;
+		y[i] = o;
+	}
+}
+
 extern "C" void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
 	int kH, int kW, int dH, int dW, int padH, int padW, int dtype)
 {
@@ -150,6 +182,13 @@ extern "C" void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W
 		return;
 	const double esz = thhip_esize(dtype);
 	ThhipLaunchScope scope(THHIP_FAM_OTHER, esz * ((double)B * C * H * W + (double)p.total));
+	if (dtype == THHIP_F32 && kH == 2 && kW == 2 && dH == 2 && dW == 2 && padH == 0 && padW == 0 && W % 4 == 0 &&
+	    H % 2 == 0 && oH == H / 2 && oW == W / 2 && ((size_t)x & 15) == 0 && ((size_t)y & 7) == 0) {
+		const long total2 = p.total / 2;
+		maxpool_f32_2x2_kernel<<<ew_grid(total2), dim3(EW_THREADS), 0, thhip_stream()>>>((const floatx4 *)x, (float2 *)y,
+			H / 2, oH, oW / 2, total2);
+		return;
+	}
 	const dim3 grid = ew_grid(p.total);
 	switch (dtype) {
 	case THHIP_F32: maxpool_kernel<THHIP_F32><<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(x, y, p); break;
