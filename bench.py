@@ -120,8 +120,8 @@ def main():
     ap.add_argument("--no-int8", action="store_true", help="skip the uint8 AlexNet leg")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this engine runs on one GPU; --gpus %d is not supported (the path shards by batch, "
-              "see DESIGN.md)" % args.gpus, file=sys.stderr)
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported (images are independent, so "
+              "more GPUs would each take a slice of the batch with replicated weights)" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     lib = api.load_library()
