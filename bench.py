@@ -153,6 +153,14 @@ def main():
     extra = {"vgg16_conv_ms_per_step": round(conv_ms / args.steps, 4),
              "vgg16_batched_fc_ms_per_step": round(fam[1][0] / args.steps, 4),
              "vgg16_other_kernels_ms_per_step": round(fam[3][0] / args.steps, 4)}
+    # the HBM-bound kernels of the same step against the 8 TB/s peak: batched Linear (weights read once)
+    # and max pooling (input read + output written once)
+    if fam[1][0] > 0:
+        extra["vgg16_batched_fc_GB/s"] = round(fam[1][2] / (fam[1][0] * 1e-3) / 1e9, 1)
+        extra["vgg16_batched_fc_frac_of_hbm_peak"] = round(fam[1][2] / (fam[1][0] * 1e-3) / 8e12, 4)
+    if fam[3][0] > 0:
+        extra["vgg16_pooling_GB/s"] = round(fam[3][2] / (fam[3][0] * 1e-3) / 1e9, 1)
+        extra["vgg16_pooling_frac_of_hbm_peak"] = round(fam[3][2] / (fam[3][0] * 1e-3) / 8e12, 4)
     # the same step through the drop-in call: host normalisation + H2D + kernels + D2H
     net.process_float(cfg["input"])
     t0 = time.perf_counter()

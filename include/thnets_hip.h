@@ -439,6 +439,9 @@ void thhip_gemv(const void *x, const void *w, const float *bias, void *y,
 int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtype);
 void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
 	int B, int nIn, int nOut, int act, float thr, float val, int dtype);
+/* Tests and tuning: 16-row blocks a wavefront of thhip_linear_batched owns
+ * (1 or 4); 0 restores the choice by the layer's width. */
+void thhip_linear_batched_set_tuning(int row_blocks);
 
 /* Replaces nn_Threshold_updateOutput (Threshold.c:38-63), out of place or
  * in place (y == x).  alpha != 0 selects the LeakyReLU branch. */

@@ -178,7 +178,8 @@ def test_gemv_ragged_sizes(hiplib, oracle):
 def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
     from thnets_amd import api
     g = cases.rng(906)
-    shapes = [(4, 128, 64), (16, 512, 100), (2, 64, 17), (16, 4096, 1000), (32, 1028, 515), (17, 200, 33), (7, 25088, 48)]
+    shapes = [(4, 128, 64), (16, 512, 100), (2, 64, 17), (16, 4096, 1000), (32, 1028, 515), (17, 200, 33), (7, 25088, 48),
+              (16, 1024, 1100), (20, 516, 1030)]
     for (B, nIn, nOut) in shapes:
         assert hiplib.thhip_linear_batched_supported(B, nIn, nOut, G.F32)
         x = g.standard_normal((B, nIn), dtype=np.float32)
@@ -187,10 +188,13 @@ def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
         G.note("linear_batched %s" % ((B, nIn, nOut),))
         dx, dw, db = api.DeviceArray(hiplib, x), api.DeviceArray(hiplib, w), api.DeviceArray(hiplib, b)
         dy = api.DeviceArray(hiplib, nbytes=B * nOut * 4)
-        hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 0, 0.0, 0.0, G.F32)
-        hiplib.thhip_sync()
-        y = dy.get((B, nOut), np.float32)
-        G.assert_close(y, oracle.linear(x, w, b), FP32_TOL, str((B, nIn, nOut)))
+        for rb in (0, 1, 4):        # chosen by width, one and four row blocks per wavefront
+            hiplib.thhip_linear_batched_set_tuning(rb)
+            hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 0, 0.0, 0.0, G.F32)
+            hiplib.thhip_sync()
+            y = dy.get((B, nOut), np.float32)
+            G.assert_close(y, oracle.linear(x, w, b), FP32_TOL, str((B, nIn, nOut, rb)))
+        hiplib.thhip_linear_batched_set_tuning(0)
         hiplib.thhip_linear_batched(dx.ptr, dw.ptr, None, dy.ptr, B, nIn, nOut, 1, 0.0, 0.0, G.F32)
         hiplib.thhip_sync()
         G.assert_close(dy.get((B, nOut), np.float32), np.maximum(oracle.linear(x, w, None), 0), FP32_TOL)
@@ -287,12 +291,15 @@ def test_linear_batched_half_types(hiplib, oracle, dt):
         dx, dw = api.to_device_dtype(hiplib, x, dt), api.to_device_dtype(hiplib, w, dt)
         db = api.DeviceArray(hiplib, b)
         dy = api.DeviceArray(hiplib, nbytes=B * nOut * 2)
-        hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 1, 0.0, 0.0, dt)
-        hiplib.thhip_sync()
         xr = api.from_device_dtype(dx, x.shape, dt)
         wr = api.from_device_dtype(dw, w.shape, dt)
         want = np.maximum(oracle.linear(xr, wr, b), 0)
-        G.assert_close(api.from_device_dtype(dy, (B, nOut), dt), want, HALF_TOL, str((B, nIn, nOut)))
+        for rb in (1, 4):
+            hiplib.thhip_linear_batched_set_tuning(rb)
+            hiplib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy.ptr, B, nIn, nOut, 1, 0.0, 0.0, dt)
+            hiplib.thhip_sync()
+            G.assert_close(api.from_device_dtype(dy, (B, nOut), dt), want, HALF_TOL, str((B, nIn, nOut, rb)))
+        hiplib.thhip_linear_batched_set_tuning(0)
 
 
 def test_threshold_bit_exact(hiplib, oracle):

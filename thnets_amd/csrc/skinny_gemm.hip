@@ -16,6 +16,10 @@
  * product is free as long as both operands use the same one.  K is split over the four wavefronts of a workgroup (summed
  * through LDS) and over gridDim.y workgroups (partials in a scratch buffer,
  * summed by a second tiny kernel that also applies bias and Threshold).
+ * For wide layers a wavefront owns RB = 4 such blocks of 16 rows: the batch
+ * operand, which every wavefront has to fetch from L2 for its K slice and
+ * which is as large per step as a block's weights, is then read once for 64
+ * rows instead of once for 16.
  */
 #include <stdlib.h>
 #include "thhip_internal.h"
@@ -41,7 +45,7 @@ template <> __device__ __forceinline__ void skinny_mma<THHIP_BF16>(floatx4 &acc,
 	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
 }
 
-template <int DT, int NB>	/* NB 16-column groups: batch <= 16 * NB */
+template <int DT, int NB, int RB>	/* NB 16-column groups: batch <= 16 * NB; RB 16-row blocks per wavefront */
 __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const void *xv, const void *wv, float *part,
 	int B, int nIn, int nOut, int ksplit)
 {
@@ -52,55 +56,67 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const void *xv, cons
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int m = lane & 15, q = lane >> 4;
-	const int row0 = blockIdx.x * 16;
-	const int row = min(row0 + m, nOut - 1);
+	const int row0 = blockIdx.x * (16 * RB);
 	/* K-steps are dealt round-robin to (workgroup slice, wave) */
 	const int nsteps = (nIn + KSTEP - 1) / KSTEP;
 	const int stride = ksplit * 4;
-	const elem *wr = w + (size_t)row * nIn;
+	const elem *wr[RB];
+#pragma unroll
+	for (int rb = 0; rb < RB; rb++)
+		wr[rb] = w + (size_t)min(row0 + rb * 16 + m, nOut - 1) * nIn;
 	const elem *xr[NB];
 #pragma unroll
 	for (int g = 0; g < NB; g++)
 		xr[g] = x + (size_t)min(g * 16 + m, B - 1) * nIn;
 
-	floatx4 acc[NB];
+	floatx4 acc[RB][NB];
 #pragma unroll
-	for (int g = 0; g < NB; g++)
-		acc[g] = floatx4{ 0, 0, 0, 0 };
+	for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+		for (int g = 0; g < NB; g++)
+			acc[rb][g] = floatx4{ 0, 0, 0, 0 };
 
 	for (int st = blockIdx.y * 4 + wave; st < nsteps; st += stride) {
 		/* load j of the four lane quarters covers 64 adjacent bytes of a row */
 		const int kb = st * KSTEP + q * VEC;
-		floatx4 a[4], b[NB][4];
+		constexpr int NJ = SK_KBYTES / 64;
+		floatx4 a[RB][NJ], b[NB][NJ];
 #pragma unroll
-		for (int j = 0; j < 4; j++) {
+		for (int j = 0; j < NJ; j++) {
 			const int k = kb + j * (4 * VEC);
 			const bool ok = k < nIn;	/* nIn % VEC == 0: a vector is all in or all out */
-			a[j] = ok ? *(const floatx4 *)(wr + k) : floatx4{ 0, 0, 0, 0 };
+#pragma unroll
+			for (int rb = 0; rb < RB; rb++)
+				a[rb][j] = ok ? *(const floatx4 *)(wr[rb] + k) : floatx4{ 0, 0, 0, 0 };
 #pragma unroll
 			for (int g = 0; g < NB; g++)
 				b[g][j] = ok ? *(const floatx4 *)(xr[g] + k) : floatx4{ 0, 0, 0, 0 };
 		}
 #pragma unroll
-		for (int j = 0; j < 4; j++)
+		for (int j = 0; j < NJ; j++)
 #pragma unroll
-			for (int g = 0; g < NB; g++)
-				skinny_mma<DT>(acc[g], a[j], b[g][j]);
+			for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+				for (int g = 0; g < NB; g++)
+					skinny_mma<DT>(acc[rb][g], a[rb][j], b[g][j]);
 	}
 
 	/* D layout: lane holds column n = lane%16, rows 4*(lane/16) + r */
-	__shared__ float red[4][NB][16][17];
+	__shared__ float red[4][RB * NB][16][17];
 #pragma unroll
-	for (int g = 0; g < NB; g++)
+	for (int rb = 0; rb < RB; rb++)
 #pragma unroll
-		for (int r = 0; r < 4; r++)
-			red[wave][g][q * 4 + r][m] = acc[g][r];
+		for (int g = 0; g < NB; g++)
+#pragma unroll
+			for (int r = 0; r < 4; r++)
+				red[wave][rb * NB + g][q * 4 + r][m] = acc[rb][g][r];
 	__syncthreads();
-	for (int i = tid; i < NB * 256; i += SK_THREADS) {
-		const int g = i >> 8, rr = (i >> 4) & 15, n = i & 15;
-		const int o = row0 + rr, bcol = g * 16 + n;
+	for (int i = tid; i < RB * NB * 256; i += SK_THREADS) {
+		const int t = i >> 8, rr = (i >> 4) & 15, n = i & 15;
+		const int rb = t / NB, g = t - rb * NB;
+		const int o = row0 + rb * 16 + rr, bcol = g * 16 + n;
 		if (o < nOut && bcol < B) {
-			const float s = (red[0][g][rr][n] + red[1][g][rr][n]) + (red[2][g][rr][n] + red[3][g][rr][n]);
+			const float s = (red[0][t][rr][n] + red[1][t][rr][n]) + (red[2][t][rr][n] + red[3][t][rr][n]);
 			part[((size_t)blockIdx.y * B + bcol) * nOut + o] = s;
 		}
 	}
@@ -149,16 +165,20 @@ extern "C" int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtyp
 
 template <int DT>
 static void skinny_launch(const void *x, const void *wrow, const float *bias, void *y, float *part,
-	int B, int nIn, int nOut, int groups, int ksplit, int act, float thr, float val)
+	int B, int nIn, int nOut, int rb, int groups, int ksplit, int act, float thr, float val)
 {
 	{
 		/* algorithmic bytes: W once, X once, Y once */
 		ThhipLaunchScope scope(THHIP_FAM_GEMV, (double)thhip_esize(DT) * ((double)nOut * nIn + (double)B * nIn + (double)B * nOut));
 		dim3 grid(groups, ksplit);
-		if (B <= 16)
-			skinny_kernel<DT, 1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+		if (B <= 16 && rb == 4)
+			skinny_kernel<DT, 1, 4><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+		else if (B <= 16)
+			skinny_kernel<DT, 1, 1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+		else if (rb == 4)
+			skinny_kernel<DT, 2, 4><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
 		else
-			skinny_kernel<DT, 2><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+			skinny_kernel<DT, 2, 1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
 	}
 	{
 		ThhipLaunchScope scope(THHIP_FAM_OTHER, 4.0 * (ksplit + 1.0) * B * nOut);
@@ -169,12 +189,27 @@ static void skinny_launch(const void *x, const void *wrow, const float *bias, vo
 	}
 }
 
+/* Tests and tuning: force the 16-row blocks per wavefront (1 or 4); 0 = choose by the layer's width. */
+static int g_skinny_rb;
+extern "C" void thhip_linear_batched_set_tuning(int row_blocks)
+{
+	if (row_blocks != 0 && row_blocks != 1 && row_blocks != 4)
+		THError("thhip_linear_batched_set_tuning(%d): 0, 1 or 4", row_blocks);
+	g_skinny_rb = row_blocks;
+}
+
 extern "C" void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
 	int B, int nIn, int nOut, int act, float thr, float val, int dtype)
 {
 	if (!thhip_linear_batched_supported(B, nIn, nOut, dtype))
 		THError("thhip_linear_batched: unsupported shape B=%d nIn=%d nOut=%d dtype=%d", B, nIn, nOut, dtype);
-	const int groups = (nOut + 15) / 16;
+	/* four row blocks per wavefront for wide layers and batches that fill most of
+	 * the 16 MFMA columns (measured: 12 % on 25088 -> 4096 at batch 16; at batch 4
+	 * the unused columns re-read their rows from L1 and one block is faster) */
+	int rb = nOut >= 1024 && B > 8 ? 4 : 1;
+	if (g_skinny_rb)
+		rb = g_skinny_rb;
+	const int groups = (nOut + 16 * rb - 1) / (16 * rb);
 	const int kstep = SK_KBYTES / thhip_esize(dtype);
 	const int nsteps = (nIn + kstep - 1) / kstep;
 	/* aim at ~4096 wavefronts, at least two K-steps per wavefront */
@@ -186,7 +221,7 @@ extern "C" void thhip_linear_batched(const void *x, const void *wrow, const floa
 	if (ksplit > 64)
 		ksplit = 64;
 	float *part = skinny_scratch((size_t)ksplit * B * nOut * sizeof(float));
-	THHIP_DISPATCH_FLOAT(dtype, skinny_launch<DT>(x, wrow, bias, y, part, B, nIn, nOut, groups, ksplit, act, thr, val));
+	THHIP_DISPATCH_FLOAT(dtype, skinny_launch<DT>(x, wrow, bias, y, part, B, nIn, nOut, rb, groups, ksplit, act, thr, val));
 }
 
 /* ------------------------------------------------------------------ */
