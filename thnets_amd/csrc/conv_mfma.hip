@@ -1186,9 +1186,8 @@ static void conv_dispatch(ConvParams &p)
 	 * is 10-25 % faster for its operand reuse.
 	 *   half types: 128x128 (64x128 for <= 64 planes) from 200 such tiles up
 	 * for the operand reuse, 64x64 below.
-	 * Splitting K is available (thhip_conv_set_tuning) but measured slower
-	 * than unsplit 64x64 tiles on every layer shape tried, so it is never
-	 * chosen; so is a cap on the workgroups per CU. */
+	 * Splitting K measured slower than unsplit 64x64 tiles on every layer that
+	 * has tiles for all CUs, so only layers of a few tiles are split (below). */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	int bm = 64, bn = 64, splitk = 1, wgs = 0, kch = conv_kch(DT, p.x_cl != 0);
 	if (DT == THHIP_F16 || DT == THHIP_BF16) {
@@ -1205,6 +1204,22 @@ static void conv_dispatch(ConvParams &p)
 			bm = 128;
 		else if (p.Co > 64)
 			wgs = 4;
+	}
+	/* A layer of a few tiles (batch 1) leaves most CUs idle and every workgroup
+	 * alone with the whole K loop, which then sets the layer's time: there the
+	 * deterministic K split pays, one part per sixteen K-tiles up to eight parts
+	 * (AlexNet batch 1: conv3 42 -> 23 us, conv4 81 -> 27 us, conv5 55 -> 29 us;
+	 * more parts lose again to the serial sum of the last arriver). */
+	const long t64 = (long)((p.Co + 63) / 64) * ((p.N + 63) / 64);
+	if (bm == 64 && bn == 64 && t64 <= 64) {
+		const int nkt = p.KC / kch;
+		int parts = (nkt + 8) / 16;
+		if (parts > 256 / t64)
+			parts = (int)(256 / t64);
+		if (parts > 8)
+			parts = 8;
+		if (parts > 1)
+			splitk = parts;
 	}
 	if (g_force_bm)
 		bm = g_force_bm;
