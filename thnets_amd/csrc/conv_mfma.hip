@@ -1211,7 +1211,7 @@ static void conv_dispatch(ConvParams &p)
 	 * (AlexNet batch 1: conv3 42 -> 23 us, conv4 81 -> 27 us, conv5 55 -> 29 us;
 	 * more parts lose again to the serial sum of the last arriver). */
 	const long t64 = (long)((p.Co + 63) / 64) * ((p.N + 63) / 64);
-	if (bm == 64 && bn == 64 && t64 <= 64) {
+	if (bm == 64 && bn == 64 && t64 <= 128) {	/* 65..128 tiles: two parts at most */
 		const int nkt = p.KC / kch;
 		int parts = (nkt + 8) / 16;
 		if (parts > 256 / t64)
