@@ -162,10 +162,13 @@ def main():
         extra["vgg16_pooling_GB/s"] = round(fam[3][2] / (fam[3][0] * 1e-3) / 1e9, 1)
         extra["vgg16_pooling_frac_of_hbm_peak"] = round(fam[3][2] / (fam[3][0] * 1e-3) / 8e12, 4)
     # the same step through the drop-in call: host normalisation + H2D + kernels + D2H
+    # (the call normalises its argument in place: every call gets its own copy, made outside the timed region)
     net.process_float(cfg["input"])
+    copies = [np.array(cfg["input"], np.float32, copy=True, order="C") for _ in range(5)]
+    res, ow, oh = C.POINTER(C.c_float)(), C.c_int(), C.c_int()
     t0 = time.perf_counter()
-    for _ in range(5):
-        net.process_float(cfg["input"])
+    for x in copies:
+        lib.THProcessFloat(net.handle, x.ctypes.data, 16, 224, 224, 3, C.byref(res), C.byref(ow), C.byref(oh))
     extra["vgg16_THProcessFloat_images_per_sec_pcie_inclusive"] = round(16 * 5 / (time.perf_counter() - t0), 1)
     net.free()
 

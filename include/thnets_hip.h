@@ -510,6 +510,13 @@ void thhip_axpby2(const void *a, const void *b, void *y, long na, long nb, float
 /* fp32 host-layout conversions on the device. */
 void thhip_convert(const void *src, int src_dtype, void *dst, int dst_dtype, long n);
 
+/* The normalisation loop of THProcessFloat (thapi.c:389-403) on a device copy
+ * of the caller's [B][C][HW] fp32 data: planes 0..2 become (x - mean) / std,
+ * further planes pass through; dst takes the engine's float dtype.  Same bits
+ * as the host loop (fp32 subtraction, correctly rounded division). */
+void thhip_normalize(const float *src, void *dst, int B, int C, long HW, const float *mean3, const float *std3,
+	int dtype);
+
 /* Replaces rgb2float / bgr2float (thapi.c:20-46; CUDA analogue
  * cudnn_copy.cu:13-116): one interleaved 8-bit image (device copy, `stride`
  * bytes per row, cp planes) -> normalised planar dst in `dtype`. */

@@ -93,6 +93,7 @@ PROTOTYPES = {
     "thhip_col2im": (None, [vp, vp, C.c_float, vp] + [C.c_int] * 13 + [C.c_float, C.c_float, C.c_int]),
     "thhip_conv_set_xcd_parts": (None, [C.c_int]),
     "thhip_conv_set_generic_cl": (None, [C.c_int]),
+    "thhip_normalize": (None, [vp, vp, C.c_int, C.c_int, C.c_long, vp, vp, C.c_int]),
     "thhip_linear_batched_set_tuning": (None, [C.c_int]),
     "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),

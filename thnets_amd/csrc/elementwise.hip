@@ -851,6 +851,37 @@ extern "C" void thhip_convert(const void *src, int sd, void *dst, int dd, long n
 	THError("thhip_convert: unsupported conversion %d -> %d", sd, dd);
 }
 
+/* ---------------- (x - mean) / std on the first three planes (thapi.c:389-403) ---------------- */
+
+/* THProcessFloat's normalisation of a [B][C][HW] fp32 tensor, on the device
+ * copy: the same subtraction and correctly rounded division as the host loop,
+ * so both give the same bits.  src is fp32; dst may be any float dtype. */
+template <int DT>
+__global__ void normalize_kernel(const float *src, void *dst, int C, long HW, long total, floatx4 mean, floatx4 std)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total; i += step) {
+		const int c = (int)((i / HW) % C);
+		float v = src[i];
+		if (c < 3)
+			v = (v - mean[c]) / std[c];
+		ThhipElem<DT>::st(dst, i, v);
+	}
+}
+
+extern "C" void thhip_normalize(const float *src, void *dst, int B, int C, long HW, const float *mean3, const float *std3,
+	int dtype)
+{
+	const long total = (long)B * C * HW;
+	if (total <= 0)
+		return;
+	const floatx4 mean = { mean3[0], mean3[1], mean3[2], 0 }, std = { std3[0], std3[1], std3[2], 1 };
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, (4.0 + thhip_esize(dtype)) * total);
+	THHIP_DISPATCH_FLOAT(dtype, (normalize_kernel<DT><<<ew_grid(total, 4), dim3(EW_THREADS), 0, thhip_stream()>>>(src, dst, C, HW,
+		total, mean, std)));
+}
+
 /* ---------------- 8-bit image -> normalised planar float (thapi.c:20-46) ---------------- */
 
 template <int DT>

@@ -199,10 +199,34 @@ static THFloatTensor *run_codes(THNETWORK *network, THFloatTensor *q)
 /* Runs a device tensor of floats (engine dtype for ENGINE_HIP, fp32 for the
  * uint8 engine, which quantises it first) and leaves the float result in
  * network->out. */
-static THFloatTensor *run_float_input(THNETWORK *network, THFloatTensor *dev_in)
+/* The caller's buffer as THProcessFloat leaves it: planes 0..2 normalised in
+ * place (thapi.c:389-403).  mean/std hold three planes: further planes are left
+ * untouched here (the reference reads past the arrays for them). */
+struct host_input {
+	float *data;
+	int batchsize, nplanes;
+	long hw;
+	const float *mean, *std;
+};
+
+static void normalize_on_host(const struct host_input *h)
+{
+	for (int b = 0; b < h->batchsize; b++)
+		for (int c = 0; c < h->nplanes && c < 3; c++) {
+			float *p = h->data + ((long)b * h->nplanes + c) * h->hw;
+			const float mean = h->mean[c], std = h->std[c];
+			for (long i = 0; i < h->hw; i++)
+				p[i] = (p[i] - mean) / std;
+		}
+}
+
+/* Runs a device tensor in the engine's float dtype (fp32 for the
+ * uint8 engine, which quantises it first) and leaves the float result in
+ * network->out.  The kernels of the forward pass are queued without waiting;
+ * `host` (if any) is normalised while they run. */
+static THFloatTensor *run_float_input(THNETWORK *network, THFloatTensor *dev_in, const struct host_input *host)
 {
 	struct hipnet *hn = (struct hipnet *)network->net;
-	THFloatTensor *out;
 	if (network->net->engine == ENGINE_HIPLOWP) {
 		/* THLowpTensor_newFromFloatTensor on the whole batch (one min/max),
 		 * lowp_basic.c:15-35 */
@@ -210,10 +234,21 @@ static THFloatTensor *run_float_input(THNETWORK *network, THFloatTensor *dev_in)
 		THFloatTensor *q = device_tensor_like(dev_in, THHIP_U8);
 		thhip_quantize((const float *)thhip_tensor_ptr(dev_in, THHIP_F32), (unsigned char *)q->storage->data, cnt,
 			&hn->cur_mult, &hn->cur_sub);
-		run_codes(network, q);
+		THFloatTensor *out = thhip_forward(network->net, q);
+		THFloatTensor *f = device_tensor_like(out, THHIP_F32);
+		thhip_dequantize(thhip_tensor_ptr(out, THHIP_U8), f->storage->data, THFloatTensor_nElement(out),
+			hn->cur_mult, hn->cur_sub);
+		if (host)
+			normalize_on_host(host);
+		if (network->out)
+			THFloatTensor_free(network->out);
+		network->out = download_as_float(f, THHIP_F32);
+		THFloatTensor_free(f);
 		THFloatTensor_free(q);
 	} else {
-		out = thhip_forward(network->net, dev_in);
+		THFloatTensor *out = thhip_forward(network->net, dev_in);
+		if (host)
+			normalize_on_host(host);
 		if (network->out)
 			THFloatTensor_free(network->out);
 		network->out = download_as_float(out, hn->dtype);
@@ -228,16 +263,11 @@ int THProcessFloat(THNETWORK *network, float *data, int batchsize, int width, in
 	struct hipnet *hn = (struct hipnet *)network->net;
 	const long hw = (long)width * height;
 	/* The reference normalises the caller's buffer in place before any engine
-	 * sees it (thapi.c:389-403); callers observe that, so it stays on the host.
-	 * mean/std hold three planes: further planes are left untouched here (the
-	 * reference reads past the arrays for them). */
-	for (int b = 0; b < batchsize; b++)
-		for (int c = 0; c < nplanes && c < 3; c++) {
-			float *p = data + ((long)b * nplanes + c) * hw;
-			const float mean = network->mean[c], std = network->std[c];
-			for (long i = 0; i < hw; i++)
-				p[i] = (p[i] - mean) / std;
-		}
+	 * sees it (thapi.c:389-403), and callers observe that.  Here the raw data
+	 * goes to the device first (the copy has finished when the call returns),
+	 * a kernel applies the same arithmetic there, and the host loop over the
+	 * caller's buffer runs while the GPU works on the forward pass: same bits
+	 * on both sides, the host pass off the critical path. */
 	THFloatTensor t;
 	memset(&t, 0, sizeof(t));
 	THFloatStorage st = { data, 1, 0 };
@@ -245,8 +275,14 @@ int THProcessFloat(THNETWORK *network, float *data, int batchsize, int width, in
 	t.size[0] = batchsize; t.size[1] = nplanes; t.size[2] = height; t.size[3] = width;
 	t.stride[3] = 1; t.stride[2] = width; t.stride[1] = hw; t.stride[0] = hw * nplanes;
 	t.storage = &st;
-	THFloatTensor *dev = upload_as(&t, engine == ENGINE_HIPLOWP ? THHIP_F32 : hn->dtype);
-	THFloatTensor *out = run_float_input(network, dev);
+	const int dt = engine == ENGINE_HIPLOWP ? THHIP_F32 : hn->dtype;
+	THFloatTensor *raw = upload_as(&t, THHIP_F32);
+	THFloatTensor *dev = dt == THHIP_F32 ? raw : device_tensor_like(&t, dt);
+	thhip_normalize(raw->storage->data, dev->storage->data, batchsize, nplanes, hw, network->mean, network->std, dt);
+	const struct host_input host = { data, batchsize, nplanes, hw, network->mean, network->std };
+	THFloatTensor *out = run_float_input(network, dev, &host);
+	if (dev != raw)
+		THFloatTensor_free(raw);
 	THFloatTensor_free(dev);
 	return finish(network, out, result, outwidth, outheight);
 }
@@ -317,7 +353,7 @@ int THProcessImages(THNETWORK *network, unsigned char **images, int batchsize, i
 			t->stride[i] = st;
 		}
 	}
-	THFloatTensor *out = run_float_input(network, t);
+	THFloatTensor *out = run_float_input(network, t, 0);
 	THFloatTensor_free(t);
 	return finish(network, out, results, outwidth, outheight);
 }
