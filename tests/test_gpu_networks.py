@@ -89,6 +89,30 @@ def test_process_float_normalises_callers_buffer_in_place(hiplib, oracle):
     n = hiplib.THProcessFloat(net.handle, x.ctypes.data, B, W, H, Cn, C.byref(res), C.byref(ow), C.byref(oh))
     assert n == 30 and (ow.value, oh.value) == (1, 1)
     assert np.array_equal(x, oracle.normalize(cfg["input"], cfg["mean"], cfg["std"]))   # thapi.c:397-402
+    got = np.ctypeslib.as_array(res, shape=(n,)).copy()
+    net.free()
+    # the device applies the normalisation to its own copy of the raw data: same bits as the host
+    # pass, on every engine (odd sizes, planes beyond the third left alone)
+    g = cases.rng(95)
+    for (B, Cn, H, W) in ((3, 3, 7, 5), (2, 5, 6, 9), (1, 1, 4, 4)):
+        raw = g.uniform(-2, 3, (B, Cn, H, W)).astype(np.float32)
+        mean, std = np.float32([0.3, -0.2, 0.7]), np.float32([0.9, 1.7, 0.31])
+        want = raw.copy()
+        for c in range(min(Cn, 3)):
+            want[:, c] = (want[:, c] - mean[c]) / std[c]
+        for dt in (G.F32, G.F16, G.BF16):
+            G.note("thhip_normalize %s dtype %d" % ((B, Cn, H, W), dt))
+            d_in = api.DeviceArray(hiplib, raw)
+            d_out = api.DeviceArray(hiplib, nbytes=raw.size * (4 if dt == G.F32 else 2))
+            hiplib.thhip_normalize(d_in.ptr, d_out.ptr, B, Cn, H * W, mean.ctypes.data, std.ctypes.data, dt)
+            hiplib.thhip_sync()
+            ref = api.from_device_dtype(api.to_device_dtype(hiplib, want, dt), want.shape, dt)
+            assert np.array_equal(api.from_device_dtype(d_out, raw.shape, dt), ref), (B, Cn, H, W, dt)
+    # and the whole call equals a forward pass on host-normalised data
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    net.upload(oracle.normalize(cfg["input"], cfg["mean"], cfg["std"]))
+    net.forward()
+    assert np.array_equal(net.module_output(net.nelem - 1).ravel(), got)
     net.free()
 
 
