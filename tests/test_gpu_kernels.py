@@ -252,6 +252,45 @@ def test_conv_half_channels_last(hiplib, oracle, dt):
 
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
+def test_conv_half_wide_tile(hiplib, oracle, dt):
+    """The 256-position tiles whose operands go from global memory straight to LDS: K-tile
+    counts around every edge of their pipelines (prologue of up to four tiles, steady state in
+    rounds of three or four, drain), partial tiles along both axes, padding, strides, both
+    output orders."""
+    from thnets_amd import api
+    g = cases.rng(911)
+    shapes = [(2, 32, 12, 13, 300, 1, 1, 1, 1, 0, 0), (1, 64, 20, 17, 260, 1, 1, 1, 1, 0, 0), (1, 96, 9, 9, 40, 1, 1, 1, 1, 0, 0),
+              (2, 32, 10, 10, 72, 2, 2, 1, 1, 1, 1), (1, 160, 8, 8, 64, 1, 1, 1, 1, 0, 0), (1, 224, 6, 7, 36, 1, 1, 1, 1, 0, 0),
+              (1, 256, 5, 9, 132, 1, 1, 2, 1, 0, 0), (1, 32, 11, 11, 64, 3, 3, 1, 1, 1, 1), (1, 352, 7, 6, 68, 1, 1, 1, 1, 0, 0),
+              (1, 384, 6, 6, 260, 1, 1, 1, 1, 0, 0), (3, 64, 7, 7, 200, 5, 5, 2, 2, 2, 2), (2, 64, 16, 16, 512, 3, 3, 1, 1, 1, 1),
+              (1, 128, 9, 10, 72, 1, 1, 1, 1, 0, 0), (1, 192, 8, 8, 36, 1, 1, 1, 1, 0, 0), (2, 64, 9, 9, 40, 2, 2, 1, 1, 1, 0),
+              (1, 320, 7, 5, 260, 1, 1, 1, 1, 0, 0)]
+    try:
+        for (B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW) in shapes:
+            x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+            w = g.standard_normal((Co, Ci, kH, kW), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * kH * kW)))
+            b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+            xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
+            wr = api.from_device_dtype(api.to_device_dtype(hiplib, w, dt), w.shape, dt)
+            raw = oracle.conv2d(xr, wr, None, (dH, dW), (pH, pW))
+            want = np.maximum(raw * sc[None, :, None, None] + b[None, :, None, None], 0)
+            for y_cl in (1, 0):
+                G.note("wide tile %s y_cl %d dtype %d" % ((B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW), y_cl, dt))
+                hiplib.thhip_conv_set_tuning(128, 128, 0, 0)
+                narrow = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
+                # eight and four waves; for 256 rows K-tiles of 32 (four LDS stages) or, with the
+                # third argument 4 and Ci % 64 == 0, of 64 (two stages)
+                for (bm, kt64) in ((256, 0), (256, 4), (128, 0)):
+                    hiplib.thhip_conv_set_tuning(bm, 256, kt64, 0)
+                    got = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
+                    G.assert_close(got, want, HALF_TOL, str((Ci, Co, kH, y_cl, bm, kt64)))
+                    G.assert_close(got, narrow, 1e-2, "vs the 128x128 tile " + str((Ci, Co, kH, y_cl, bm, kt64)))
+    finally:
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+
+
+@pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_maxpool_and_relayout_half_channels_last(hiplib, oracle, dt):
     from thnets_amd import api
     g = cases.rng(909)

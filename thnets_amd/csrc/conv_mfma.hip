@@ -49,6 +49,7 @@ struct ConvParams {
 	int tiles_m, tiles_n;
 	int mparts;		/* the tile grid is cut mparts x (8 / mparts) over the XCDs */
 	unsigned x_bytes;
+	unsigned w_bytes;	/* packed weights (the wide kernel's buffer descriptor) */
 	/* split-K: S workgroups share an output tile, each over a K range */
 	int splitk;
 	int *ws;		/* [tile][S][BM*BN] partial accumulators (float or int bits) */
@@ -852,10 +853,326 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 }
 
 /* ------------------------------------------------------------------ */
+/* wide tile for the half types                                        */
+/* ------------------------------------------------------------------ */
+
+/* A 32x32x16 half MFMA retires in 32 cycles what the fp32 one needs 512 for,
+ * so a 128x128 tile asks the LDS and the path from L2 for about as many bytes
+ * per cycle as they can deliver.  This kernel halves both appetites: a 256x256
+ * tile, eight waves of 128x64 each, K-tiles of 32 values, and the operands go
+ * from global memory straight into LDS (buffer loads with the LDS bit: no
+ * staging registers, no ds_write), four stages deep.
+ *
+ * For channels-last input whose plane count is a multiple of the K-tile (the
+ * GM_CL_UNIFORM case).  A wave-wide 16-byte load puts lane l's data at
+ * base + 16 l, so what a lane fetches decides the LDS layout:
+ *   A: the packed weights already are [32-row block][chunk][h][32][16 B]; a
+ *      wave copies 1 KiB blocks unchanged.
+ *   B: a position's K-tile slice is 64 contiguous bytes (four vectors), so four
+ *      neighbouring lanes fetch one position and a wave sixteen positions.  Slot
+ *      4 pl + s of a sixteen-position group holds vector s ^ (pl / 4) of
+ *      position pl: the fragment reads (32 positions x 2 vectors) then hit every
+ *      bank equally (measured at the full ds_read_b128 rate; 4x slower unswizzled).
+ * Loads outside the image are sent out of the buffer's range and write zeros.
+ *
+ * The compiler does not track these LDS writes: the waits are explicit
+ * (s_waitcnt vmcnt counts whole tiles, four loads per wave each), and the
+ * barrier sits in the middle of a step, between the two chunks of a K-tile:
+ * before it a wave has seen its share of tile kt+1 land and has read the last
+ * fragments of tile kt, after it that stage is free for tile kt+4 and tile
+ * kt+1 is complete, so its first fragments are fetched under the second
+ * chunk's MFMAs. */
+#define WIDE_BN 256
+#define WIDE_LDS(p) ((__attribute__((address_space(3))) void *)(p))
+/* s_waitcnt immediate that waits for all but n vector-memory operations only */
+#define WIDE_VMCNT(n) (0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
+
+/* Waits until at most N vector-memory operations of the wave are outstanding
+ * (LGKM0: and no LDS / scalar ones).  The builtin wants a literal: a value that
+ * depends on a template parameter makes the host pass drop the kernel. */
+template <int N, bool LGKM0>
+__device__ __forceinline__ void wide_wait()
+{
+	static_assert(N >= 0 && N <= 24 && N % 2 == 0, "add the count below");
+#define WIDE_WAIT_CASE(n)                                                          \
+	if constexpr (N == n) {                                                    \
+		if constexpr (LGKM0)                                               \
+			__builtin_amdgcn_s_waitcnt(WIDE_VMCNT(n) & 0xf0ff);        \
+		else                                                               \
+			__builtin_amdgcn_s_waitcnt(WIDE_VMCNT(n));                 \
+	}
+	WIDE_WAIT_CASE(0) WIDE_WAIT_CASE(2) WIDE_WAIT_CASE(4) WIDE_WAIT_CASE(6) WIDE_WAIT_CASE(8)
+	WIDE_WAIT_CASE(10) WIDE_WAIT_CASE(12) WIDE_WAIT_CASE(14) WIDE_WAIT_CASE(16) WIDE_WAIT_CASE(18)
+	WIDE_WAIT_CASE(20) WIDE_WAIT_CASE(22) WIDE_WAIT_CASE(24)
+#undef WIDE_WAIT_CASE
+}
+
+template <int DT, bool CLO, int BM, int WGM, int WGN, int KCH, int NST>
+__global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
+{
+	/* The host pass only needs the launch stub; it gets no body, because it
+	 * silently drops the whole kernel when it meets the LDS-load builtin in a
+	 * generic lambda of this template (the launch then fails to link). */
+#if defined(__HIP_DEVICE_COMPILE__)
+	typedef ConvTraits<DT> TR;
+	typedef typename TR::elem elem;
+	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC;
+	static_assert(CHUNK == 16 && sizeof(elem) == 2, "a half type");
+	constexpr int BN = WIDE_BN, WAVES = WGM * WGN;
+	constexpr int MB = BM / 32, TM = BM / WGM / 32, TN = BN / WGN / 32;
+	constexpr int VPP = 2 * KCH;			/* 16-byte vectors of a position's K-tile slice */
+	constexpr int PPG = 64 / VPP;			/* positions one wave-wide load covers (a group) */
+	constexpr int FSH = KCH == 2 ? 2 : 1;		/* swizzle: vector index ^ (position >> FSH) */
+	constexpr int A_VECS = MB * KCH * 64, B_VECS = BN * VPP, STAGE_VECS = A_VECS + B_VECS;
+	constexpr int A_PW = MB * KCH / WAVES;		/* 1 KiB weight blocks per wave and K-tile */
+	constexpr int NPOS = BN / PPG / WAVES;		/* position groups per wave */
+	constexpr int LOADS = A_PW + NPOS;		/* per wave and K-tile */
+	static_assert(KCH == 2 || KCH == 4, "K-tiles of 32 or 64 values");
+	static_assert(MB * KCH % WAVES == 0 && BN / PPG % WAVES == 0 && NST >= 2 && NST <= 4, "tile shape");
+	static_assert(2 * BM * sizeof(int) <= NST * STAGE_VECS * sizeof(floatx4), "the epilogue's row constants fit");
+	__shared__ floatx4 lds[NST * STAGE_VECS];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wm = wave % WGM, wn = wave / WGM;
+
+	int tile_m, tile_n;
+	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
+		const int bid = blockIdx.x;
+		const int xcd = bid & 7;
+		const int local = bid >> 3;
+		const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
+		const int m0 = p.tiles_m * mp / p.mparts, m1 = p.tiles_m * (mp + 1) / p.mparts;
+		const int n0 = p.tiles_n * np / nparts, n1 = p.tiles_n * (np + 1) / nparts;
+		const int mw = m1 - m0;
+		if (local >= mw * (n1 - n0))
+			return;
+		tile_m = m0 + local % mw;
+		tile_n = n0 + local / mw;
+	}
+
+	/* ---- what this lane fetches: slot lane % VPP of position lane / VPP of a group ---- */
+	bool n_ok_[NPOS];
+	int iy0_[NPOS], ix0_[NPOS], xoff_[NPOS];
+#pragma unroll
+	for (int q = 0; q < NPOS; q++) {
+		const int n_tile = (wave + WAVES * q) * PPG + lane / VPP;
+		const int myvec = (lane % VPP) ^ ((n_tile >> FSH) & (VPP - 1));
+		const int n_glob = tile_n * BN + n_tile;
+		n_ok_[q] = n_glob < p.N;
+		const int nn = n_ok_[q] ? n_glob : 0;
+		const int b = nn / p.oHW, r = nn - b * p.oHW;
+		const int oy = r / p.oW, ox = r - oy * p.oW;
+		iy0_[q] = oy * p.dH - p.padH;
+		ix0_[q] = ox * p.dW - p.padW;
+		xoff_[q] = (((b * p.H + iy0_[q]) * p.W + ix0_[q]) * p.Ci + myvec * VEC) * (int)sizeof(elem);
+	}
+	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
+	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
+	/* this wave's weight blocks: wave + WAVES i counts (chunk, 32-row block), 1 KiB each */
+	unsigned a_off_[A_PW];
+	int a_lds_[A_PW];
+#pragma unroll
+	for (int i = 0; i < A_PW; i++) {
+		const int idx = wave + WAVES * i, mbi = idx % MB, kci = idx / MB;
+		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
+		a_lds_[i] = (kci * MB + mbi) * 64;
+	}
+	int t_cb = 0, t_kh = 0, t_kw = 0, t_kc = 0;
+
+	auto issue = [&](auto st_) {
+		constexpr int st = decltype(st_)::value;
+		floatx4 *la = lds + st * STAGE_VECS, *lb = la + A_VECS;
+#pragma unroll
+		for (int i = 0; i < A_PW; i++)
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(la + a_lds_[i]), 16, lane * 16,
+				a_off_[i] + (unsigned)t_kc * 1024u, 0, 0);
+		const int cl_off = ((t_kh * p.W + t_kw) * p.Ci + t_cb) * (int)sizeof(elem);
+#pragma unroll
+		for (int q = 0; q < NPOS; q++) {
+			const int iy = iy0_[q] + t_kh, ix = ix0_[q] + t_kw;
+			const bool ok = n_ok_[q] && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			const unsigned voff = ok ? (unsigned)(xoff_[q] + cl_off) : 0x80000000u;
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(lb + (wave + WAVES * q) * 64), 16, voff, 0, 0, 0);
+		}
+		t_kc += KCH;
+		t_cb += KCH * CHUNK;
+		if (t_cb == p.Ci) {
+			t_cb = 0;
+			if (++t_kw == p.kW) {
+				t_kw = 0;
+				++t_kh;
+			}
+		}
+	};
+
+	/* fragment addresses: A rows lane % 32 of a block, half lane / 32; B position
+	 * lane % 32 of a block, vector 2 chunk + lane / 32, through the swizzle */
+	const int b_pos = ((lane & 31) / PPG) * 64 + ((lane & 31) % PPG) * VPP;
+	const int b_f = ((lane & 31) >> FSH) & (VPP - 1);
+	floatx4 af[2][TM], bf[2][TN];
+	auto read_frags = [&](auto st_, int kci, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
+		constexpr int st = decltype(st_)::value;
+		const floatx4 *la = lds + st * STAGE_VECS, *lb = la + A_VECS;
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+			a[i] = la[(kci * MB + wm * TM + i) * 64 + lane];
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+			b[j] = lb[(wn * TN + j) * 32 * VPP + b_pos + ((kci * 2 + (lane >> 5)) ^ b_f)];
+	};
+
+	typename ConvAcc<DT>::T acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; i++)
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[i][j][r] = 0;
+	auto mma = [&](int set) {
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+				conv_mma<DT>(acc[i][j], af[set][i], bf[set][j]);
+	};
+
+	typedef std::integral_constant<int, 0> S0;
+	typedef std::integral_constant<int, 1> S1;
+	typedef std::integral_constant<int, NST >= 3 ? 2 : 0> S2;
+	typedef std::integral_constant<int, NST >= 4 ? 3 : 0> S3;
+	const int nkt = p.KC / KCH;
+	issue(S0{});
+	if (1 < nkt)
+		issue(S1{});
+	if constexpr (NST >= 3) {
+		if (2 < nkt)
+			issue(S2{});
+	}
+	if constexpr (NST >= 4) {
+		if (3 < nkt)
+			issue(S3{});
+	}
+	if (NST - 1 < nkt)
+		wide_wait<(NST - 1) * LOADS, false>();
+	else
+		wide_wait<0, false>();
+	__builtin_amdgcn_s_barrier();
+	read_frags(S0{}, 0, af[0], bf[0]);
+
+	/* tile kt is in stage st (its first fragments in set 0), tile kt+1 in st1 */
+	auto step = [&](int kt, auto st, auto st1, auto steady_) {
+		constexpr bool steady = decltype(steady_)::value;	/* tiles up to kt+NST exist */
+#pragma unroll
+		for (int c = 0; c + 1 < KCH; c++) {
+			read_frags(st, c + 1, af[(c + 1) & 1], bf[(c + 1) & 1]);
+			mma(c & 1);
+		}
+		/* this wave's loads of tile kt+1 are in LDS (younger tiles may still be
+		 * on their way) and the fragments just requested have arrived */
+		if (steady)
+			wide_wait<(NST - 2) * LOADS, true>();
+		else
+			wide_wait<0, true>();
+		__builtin_amdgcn_s_barrier();
+		if (steady || kt + NST < nkt)
+			issue(st);
+		if (steady || kt + 1 < nkt)
+			read_frags(st1, 0, af[0], bf[0]);
+		mma((KCH - 1) & 1);
+	};
+	/* NST steps: every stage index a constant */
+	auto round = [&](int kt, auto steady_) {
+		if constexpr (NST == 2) {
+			step(kt, S0{}, S1{}, steady_);
+			step(kt + 1, S1{}, S0{}, steady_);
+		} else if constexpr (NST == 3) {
+			step(kt, S0{}, S1{}, steady_);
+			step(kt + 1, S1{}, S2{}, steady_);
+			step(kt + 2, S2{}, S0{}, steady_);
+		} else {
+			step(kt, S0{}, S1{}, steady_);
+			step(kt + 1, S1{}, S2{}, steady_);
+			step(kt + 2, S2{}, S3{}, steady_);
+			step(kt + 3, S3{}, S0{}, steady_);
+		}
+	};
+	int kt = 0;
+	for (; kt + 2 * NST - 1 < nkt; kt += NST)
+		round(kt, std::true_type{});
+	for (; kt + NST - 1 < nkt; kt += NST)
+		round(kt, std::false_type{});
+	if (kt < nkt) {
+		step(kt, S0{}, S1{}, std::false_type{});
+		if constexpr (NST >= 3) {
+			if (kt + 1 < nkt)
+				step(kt + 1, S1{}, S2{}, std::false_type{});
+		}
+		if constexpr (NST >= 4) {
+			if (kt + 2 < nkt)
+				step(kt + 2, S2{}, S3{}, std::false_type{});
+		}
+	}
+
+	/* ---- epilogue: (folded batch norm factor,) bias, optional threshold, store ---- */
+	elem *y = (elem *)p.y;
+	int *lrow = (int *)lds;		/* [BM] bias bits, [BM..2BM) factor bits */
+	__syncthreads();		/* every wave is done with the tiles */
+	if (tid < BM) {
+		const int mc = min(tile_m * BM + tid, p.Co - 1);
+		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+		if (p.scale)
+			lrow[BM + tid] = __float_as_int(p.scale[mc]);
+	}
+	__syncthreads();
+	const bool has_scale = p.scale != 0;
+#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
+		if (n >= p.N)
+			continue;
+		const int b = n / p.oHW, rem = n - b * p.oHW;
+		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+			for (int g = 0; g < 4; g++) {
+				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+				const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
+				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+				floatx4 rowscale = { 1, 1, 1, 1 };
+				if (has_scale)
+					rowscale = *(const floatx4 *)(lrow + BM + ml);
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int r = 4 * g + e, m = m0 + 8 * g + e;
+					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
+					if (p.act)
+						v = v > p.thr ? v : p.val;
+					if constexpr (!CLO) {
+						if (m < p.Co)
+							y[ybase + (size_t)m * p.oHW] = (elem)v;
+					}
+					quad.v[e] = (elem)v;
+				}
+				if constexpr (CLO) {
+					if (m0 + 8 * g < p.Co)
+						*(Quad *)(y + (size_t)n * p.Co + m0 + 8 * g) = quad;
+				}
+			}
+		}
+	}
+#endif
+}
+
+/* ------------------------------------------------------------------ */
 /* host side                                                           */
 /* ------------------------------------------------------------------ */
 
-#define CONV_MPAD 128	/* packed rows are padded to the largest M tile */
+#define CONV_MPAD 256	/* packed rows are padded to the largest M tile */
 
 static inline int conv_chunk(int dtype) { return dtype == THHIP_F32 ? 8 : dtype == THHIP_U8 ? 32 : 16; }
 
@@ -1166,6 +1483,49 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 #undef CONV_GO
 }
 
+/* Whether the wide kernels can run this layer: a half type, channels-last input
+ * with whole K-tiles of 32 planes inside a tap, 32-bit byte offsets. */
+template <int DT>
+static bool conv_wide_ok(const ConvParams &p)
+{
+	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16)
+		return p.x_cl == 1 && p.Ci % 32 == 0 && p.x_bytes < 0x7fffffffu && !g_force_generic_cl &&
+			(!p.y_cl || p.Co % 4 == 0);
+	return false;
+}
+
+template <int DT, int BM, int WGM, int WGN, int KCH, int NST>
+static void conv_launch_wide(ConvParams &p)
+{
+	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
+		p.tiles_m = (p.Co + BM - 1) / BM;
+		p.tiles_n = (p.N + WIDE_BN - 1) / WIDE_BN;
+		p.splitk = 1;
+		if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
+			THError("thhip_conv2d: packed weights shorter than the tile grid");
+		const double wbytes = (double)p.Co * p.K * thhip_esize(DT);
+		p.mparts = 1;
+		while (p.mparts < 8 && p.mparts * 2 <= p.tiles_m && wbytes / p.mparts > 2.5e6)
+			p.mparts *= 2;
+		if (g_force_mparts)
+			p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
+		size_t maxcnt = 0;
+		for (int x = 0; x < 8; x++) {
+			const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
+			const size_t cnt = (size_t)(p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
+				(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
+			if (cnt > maxcnt)
+				maxcnt = cnt;
+		}
+		dim3 grid((unsigned)(8 * maxcnt));
+		if (p.y_cl)
+			conv_wide_kernel<DT, true, BM, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+		else
+			conv_wide_kernel<DT, false, BM, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+	} else
+		THError("thhip_conv2d: the 256-position tiles are for the half types");
+}
+
 template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
@@ -1191,7 +1551,19 @@ static void conv_dispatch(ConvParams &p)
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	int bm = 64, bn = 64, splitk = 1, wgs = 0, kch = conv_kch(DT, p.x_cl != 0);
 	if (DT == THHIP_F16 || DT == THHIP_BF16) {
-		if (p.Co <= 64)
+		/* tiles of 256 positions (operands straight to LDS) where whole tiles of
+		 * 256 planes fill most CUs for a turn: one such tile per CU multiplies
+		 * 1.3-1.4x faster than two 128x128 ones (measured with random data:
+		 * 256->256 @56^2 batch 16, 196 tiles, 97 -> 68 us; 512->512 @28^2 batch
+		 * 32, 133 vs 187 us); with 80..128 of them the 128-plane tile (two
+		 * workgroups per CU) wins by 6-15 %; with fewer, and for layers of 128
+		 * planes or less, the smaller tiles below do. */
+		const long t256 = (long)((p.Co + 255) / 256) * ((p.N + 255) / 256);
+		if (conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128)
+			bm = bn = 256;
+		else if (conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 >= 80)
+			bm = 128, bn = 256;
+		else if (p.Co <= 64)
 			bn = 128;
 		else if (t128 >= 200)
 			bm = bn = 128;
@@ -1231,6 +1603,19 @@ static void conv_dispatch(ConvParams &p)
 		wgs = g_force_wgs;
 	if (DT == THHIP_F32 && g_force_kch)
 		kch = g_force_kch;
+	if (bn == WIDE_BN) {
+		if (!conv_wide_ok<DT>(p))
+			THError("thhip_conv2d: the 256-position tiles need a half type and channels-last input with Ci %% 32 == 0");
+		/* K-tiles of 64 values in two stages measured the same as 32 in four
+		 * (the tuning hook's split-K argument, 4, selects them for the tests) */
+		if (bm == 256 && p.Ci % 64 == 0 && g_force_splitk == 4)
+			return conv_launch_wide<DT, 256, 2, 4, 4, 2>(p);
+		if (bm == 256)
+			return conv_launch_wide<DT, 256, 2, 4, 2, 4>(p);
+		if (bm == 128)
+			return conv_launch_wide<DT, 128, 1, 4, 2, 3>(p);
+		THError("thhip_conv2d: no %dx%d tile", bm, bn);
+	}
 #define CONV_TILES(KCH)                                                      \
 	do {                                                                 \
 		if (bm == 128 && bn == 128)                                  \
@@ -1367,6 +1752,7 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 		p.mhi_ci = (unsigned)(conv_magic(Ci) >> 32);
 		p.act = act; p.thr = thr; p.val = val;
 		p.x_bytes = (unsigned)(bn * in_img * esize);
+		p.w_bytes = (unsigned)conv_packed_bytes(Co, Ci, kH, kW, dtype, xl);
 		if (u8) {
 			p.rowsum = (const int *)((const char *)wpacked + conv_packed_bytes(Co, Ci, kH, kW, THHIP_U8, xl));
 			p.addend = u8->addend;
