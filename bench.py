@@ -184,6 +184,20 @@ def main():
         "workload": "VGG-16 shape, fp16 storage and MFMA, batch 16 (BASELINE configs[2], fp16 leg)"}
     nh.free()
 
+    # ---- the same at batch 64: enough whole 256 x 256 tiles for every layer of 256 planes and more ----
+    cfg64 = configs.vgg16(batch=64)
+    nh = api.HipNetwork(cfg64["layers"], cfg64["mean"], cfg64["std"], half=1)
+    nh.upload(cfg64["input"])
+    msh, famh = timed_forward(lib, nh, max(args.steps // 2, 5), args.warmup, (0, 1, 3), profiled=False)
+    hc_ms, hc_n, hc_fl = famh[0]
+    extra["vgg16_fp16_b64"] = {
+        "images_per_sec": round(64.0 / (msh * 1e-3), 1), "ms_per_step": round(msh, 4),
+        "conv_TFLOP/s": round(hc_fl / (hc_ms * 1e-3) / 1e12, 1) if hc_ms > 0 else None,
+        "frac_of_fp16_mfma_peak": round(hc_fl / (hc_ms * 1e-3) / 1e12 / 2500.0, 4) if hc_ms > 0 else None,
+        "workload": "VGG-16 shape, fp16 storage and MFMA, batch 64"}
+    nh.free()
+    del cfg64
+
     # ---- AlexNet-OWT fp32 batch 1 (GEMV-bound Linear layers) ----
     c2 = configs.alexnet_owt()
     n2 = api.HipNetwork(c2["layers"], c2["mean"], c2["std"])

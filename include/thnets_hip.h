@@ -434,8 +434,9 @@ void thhip_gemv(const void *x, const void *w, const float *bias, void *y,
  * (Linear.c:92-108: addmm with beta 0, then the rank-1 bias update through
  * addr / sger, thbasic.c:757-789): Y[b][o] = bias[o] + sum_k W[o][k] X[b][k],
  * X [B][nIn], W row-major [nOut][nIn], Y [B][nOut].  thhip_linear_batched_supported
- * says whether the shape is taken (fp32, B <= 32, nIn % 4 == 0); other shapes
- * run as a 1x1 convolution through thhip_conv2d. */
+ * says whether the shape is taken (B <= 128, run in slices of 32 that each read
+ * the weights; rows in 16-byte vectors: nIn % 4 == 0 for fp32, % 8 for the half
+ * types); other shapes run as a 1x1 convolution through thhip_conv2d. */
 int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtype);
 void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
 	int B, int nIn, int nOut, int act, float thr, float val, int dtype);

@@ -179,7 +179,7 @@ def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
     from thnets_amd import api
     g = cases.rng(906)
     shapes = [(4, 128, 64), (16, 512, 100), (2, 64, 17), (16, 4096, 1000), (32, 1028, 515), (17, 200, 33), (7, 25088, 48),
-              (16, 1024, 1100), (20, 516, 1030)]
+              (16, 1024, 1100), (20, 516, 1030), (64, 1024, 260), (45, 516, 1030), (128, 256, 48)]   # the last: slices of 32
     for (B, nIn, nOut) in shapes:
         assert hiplib.thhip_linear_batched_supported(B, nIn, nOut, G.F32)
         x = g.standard_normal((B, nIn), dtype=np.float32)
@@ -198,7 +198,7 @@ def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
         hiplib.thhip_linear_batched(dx.ptr, dw.ptr, None, dy.ptr, B, nIn, nOut, 1, 0.0, 0.0, G.F32)
         hiplib.thhip_sync()
         G.assert_close(dy.get((B, nOut), np.float32), np.maximum(oracle.linear(x, w, None), 0), FP32_TOL)
-    assert not hiplib.thhip_linear_batched_supported(33, 128, 64, G.F32)
+    assert not hiplib.thhip_linear_batched_supported(129, 128, 64, G.F32)
     assert not hiplib.thhip_linear_batched_supported(4, 130, 64, G.F32)
     assert hiplib.thhip_linear_batched_supported(4, 128, 64, G.F16)
     assert not hiplib.thhip_linear_batched_supported(4, 132, 64, G.F16)        # half rows come in 16-byte vectors
@@ -322,7 +322,7 @@ def test_linear_batched_half_types(hiplib, oracle, dt):
     the rounded operands at the half tolerance (2e-2 of the largest reference value)."""
     from thnets_amd import api
     g = cases.rng(907)
-    for (B, nIn, nOut) in [(4, 128, 64), (16, 4096, 1000), (32, 1032, 515), (17, 200, 33), (3, 25088, 40)]:
+    for (B, nIn, nOut) in [(4, 128, 64), (16, 4096, 1000), (32, 1032, 515), (17, 200, 33), (3, 25088, 40), (70, 1032, 260)]:
         x = g.standard_normal((B, nIn), dtype=np.float32)
         w = g.standard_normal((nOut, nIn), dtype=np.float32) * np.float32(np.sqrt(2.0 / nIn))
         b = g.standard_normal(nOut, dtype=np.float32)

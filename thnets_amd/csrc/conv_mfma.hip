@@ -882,7 +882,6 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
  * fragments of tile kt, after it that stage is free for tile kt+4 and tile
  * kt+1 is complete, so its first fragments are fetched under the second
  * chunk's MFMAs. */
-#define WIDE_BN 256
 #define WIDE_LDS(p) ((__attribute__((address_space(3))) void *)(p))
 /* s_waitcnt immediate that waits for all but n vector-memory operations only */
 #define WIDE_VMCNT(n) (0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
@@ -893,7 +892,7 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 template <int N, bool LGKM0>
 __device__ __forceinline__ void wide_wait()
 {
-	static_assert(N >= 0 && N <= 24 && N % 2 == 0, "add the count below");
+	static_assert(N >= 0 && N <= 24, "add the count below");
 #define WIDE_WAIT_CASE(n)                                                          \
 	if constexpr (N == n) {                                                    \
 		if constexpr (LGKM0)                                               \
@@ -901,13 +900,15 @@ __device__ __forceinline__ void wide_wait()
 		else                                                               \
 			__builtin_amdgcn_s_waitcnt(WIDE_VMCNT(n));                 \
 	}
-	WIDE_WAIT_CASE(0) WIDE_WAIT_CASE(2) WIDE_WAIT_CASE(4) WIDE_WAIT_CASE(6) WIDE_WAIT_CASE(8)
-	WIDE_WAIT_CASE(10) WIDE_WAIT_CASE(12) WIDE_WAIT_CASE(14) WIDE_WAIT_CASE(16) WIDE_WAIT_CASE(18)
-	WIDE_WAIT_CASE(20) WIDE_WAIT_CASE(22) WIDE_WAIT_CASE(24)
+	WIDE_WAIT_CASE(0) WIDE_WAIT_CASE(1) WIDE_WAIT_CASE(2) WIDE_WAIT_CASE(3) WIDE_WAIT_CASE(4)
+	WIDE_WAIT_CASE(5) WIDE_WAIT_CASE(6) WIDE_WAIT_CASE(7) WIDE_WAIT_CASE(8) WIDE_WAIT_CASE(9)
+	WIDE_WAIT_CASE(10) WIDE_WAIT_CASE(11) WIDE_WAIT_CASE(12) WIDE_WAIT_CASE(13) WIDE_WAIT_CASE(14)
+	WIDE_WAIT_CASE(15) WIDE_WAIT_CASE(16) WIDE_WAIT_CASE(17) WIDE_WAIT_CASE(18) WIDE_WAIT_CASE(19)
+	WIDE_WAIT_CASE(20) WIDE_WAIT_CASE(21) WIDE_WAIT_CASE(22) WIDE_WAIT_CASE(23) WIDE_WAIT_CASE(24)
 #undef WIDE_WAIT_CASE
 }
 
-template <int DT, bool CLO, int BM, int WGM, int WGN, int KCH, int NST>
+template <int DT, bool CLO, int BM, int BN, int WGM, int WGN, int KCH, int NST>
 __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 {
 	/* The host pass only needs the launch stub; it gets no body, because it
@@ -918,7 +919,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	typedef typename TR::elem elem;
 	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC;
 	static_assert(CHUNK == 16 && sizeof(elem) == 2, "a half type");
-	constexpr int BN = WIDE_BN, WAVES = WGM * WGN;
+	constexpr int WAVES = WGM * WGN;
 	constexpr int MB = BM / 32, TM = BM / WGM / 32, TN = BN / WGN / 32;
 	constexpr int VPP = 2 * KCH;			/* 16-byte vectors of a position's K-tile slice */
 	constexpr int PPG = 64 / VPP;			/* positions one wave-wide load covers (a group) */
@@ -1494,12 +1495,12 @@ static bool conv_wide_ok(const ConvParams &p)
 	return false;
 }
 
-template <int DT, int BM, int WGM, int WGN, int KCH, int NST>
+template <int DT, int BM, int BN, int WGM, int WGN, int KCH, int NST>
 static void conv_launch_wide(ConvParams &p)
 {
 	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
 		p.tiles_m = (p.Co + BM - 1) / BM;
-		p.tiles_n = (p.N + WIDE_BN - 1) / WIDE_BN;
+		p.tiles_n = (p.N + BN - 1) / BN;
 		p.splitk = 1;
 		if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
 			THError("thhip_conv2d: packed weights shorter than the tile grid");
@@ -1519,9 +1520,9 @@ static void conv_launch_wide(ConvParams &p)
 		}
 		dim3 grid((unsigned)(8 * maxcnt));
 		if (p.y_cl)
-			conv_wide_kernel<DT, true, BM, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+			conv_wide_kernel<DT, true, BM, BN, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
 		else
-			conv_wide_kernel<DT, false, BM, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+			conv_wide_kernel<DT, false, BM, BN, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
 	} else
 		THError("thhip_conv2d: the 256-position tiles are for the half types");
 }
@@ -1603,17 +1604,19 @@ static void conv_dispatch(ConvParams &p)
 		wgs = g_force_wgs;
 	if (DT == THHIP_F32 && g_force_kch)
 		kch = g_force_kch;
-	if (bn == WIDE_BN) {
+	if (bn >= 256) {
 		if (!conv_wide_ok<DT>(p))
 			THError("thhip_conv2d: the 256-position tiles need a half type and channels-last input with Ci %% 32 == 0");
 		/* K-tiles of 64 values in two stages measured the same as 32 in four
 		 * (the tuning hook's split-K argument, 4, selects them for the tests) */
-		if (bm == 256 && p.Ci % 64 == 0 && g_force_splitk == 4)
-			return conv_launch_wide<DT, 256, 2, 4, 4, 2>(p);
-		if (bm == 256)
-			return conv_launch_wide<DT, 256, 2, 4, 2, 4>(p);
-		if (bm == 128)
-			return conv_launch_wide<DT, 128, 1, 4, 2, 3>(p);
+		if (bm == 256 && bn == 256 && p.Ci % 64 == 0 && g_force_splitk == 4)
+			return conv_launch_wide<DT, 256, 256, 2, 4, 4, 2>(p);
+		if (bm == 256 && bn == 256)
+			return conv_launch_wide<DT, 256, 256, 2, 4, 2, 4>(p);
+		if (bm == 128 && bn == 256)
+			return conv_launch_wide<DT, 128, 256, 1, 4, 2, 3>(p);
+		if (bm == 128 && bn == 512)
+			return conv_launch_wide<DT, 128, 512, 2, 4, 2, 3>(p);
 		THError("thhip_conv2d: no %dx%d tile", bm, bn);
 	}
 #define CONV_TILES(KCH)                                                      \
