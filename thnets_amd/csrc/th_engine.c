@@ -174,8 +174,10 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 		THError("HIP engine: a convolution planned for %s input got the other memory order",
 			hm->in_cl ? "channels-last" : "plane-major");
 	hn->cur_cl = hm->out_cl && oH * oW > 1;
+	/* the row-major copy is made from plane-major packing; for a 1x1 kernel the
+	 * channels-last packing is the same (k is the plane in both) */
 	const int one_position = oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
-		!hm->x_layout;	/* the row-major copy is made from plane-major packing */
+		(!hm->x_layout || (hm->x_layout == 1 && c->kH == 1 && c->kW == 1));
 	if (one_position && !hm->scale && (s.B == 1 || thhip_linear_batched_supported(s.B, K, c->nOutputPlane, dt))) {
 		/* one output position per image: a matrix-vector (or skinny matrix)
 		 * product over the flattened input, bound by reading the weights once */
