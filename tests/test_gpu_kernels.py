@@ -291,6 +291,38 @@ def test_conv_half_wide_tile(hiplib, oracle, dt):
 
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
+def test_conv_half_patch_kernel(hiplib, oracle, dt):
+    """3x3 stride-1 convolutions of 64 planes whose taps come from an input patch in LDS:
+    images smaller and larger than the 8 x 32 tile, partial tiles on both axes, padding 0, 1
+    and 2, plane counts that leave a partial 64-row tile, both output orders."""
+    from thnets_amd import api
+    g = cases.rng(912)
+    shapes = [(2, 5, 7, 64, 1, 1), (1, 8, 32, 128, 1, 1), (3, 19, 45, 72, 1, 1), (1, 40, 33, 200, 0, 0), (2, 9, 70, 36, 2, 1),
+              (1, 16, 64, 260, 1, 0), (1, 3, 3, 64, 0, 0)]
+    try:
+        for (B, H, W, Co, pH, pW) in shapes:
+            Ci = 64
+            x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+            w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
+            b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+            xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
+            wr = api.from_device_dtype(api.to_device_dtype(hiplib, w, dt), w.shape, dt)
+            raw = oracle.conv2d(xr, wr, None, (1, 1), (pH, pW))
+            want = np.maximum(raw * sc[None, :, None, None] + b[None, :, None, None], 0)
+            for y_cl in (1, 0):
+                G.note("patch kernel %s y_cl %d dtype %d" % ((B, H, W, Co, pH, pW), y_cl, dt))
+                hiplib.thhip_conv_set_tuning(64, 64, 0, 0)
+                narrow = G.conv2d_layout(hiplib, x, w, b, (1, 1), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
+                hiplib.thhip_conv_set_tuning(64, 1, 0, 0)
+                got = G.conv2d_layout(hiplib, x, w, b, (1, 1), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
+                G.assert_close(got, want, HALF_TOL, str((B, H, W, Co, pH, pW, y_cl)))
+                G.assert_close(got, narrow, 1e-2, "vs the 64x64 tile " + str((B, H, W, Co, pH, pW, y_cl)))
+    finally:
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+
+
+@pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_maxpool_and_relayout_half_channels_last(hiplib, oracle, dt):
     from thnets_amd import api
     g = cases.rng(909)

@@ -1170,6 +1170,235 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 }
 
 /* ------------------------------------------------------------------ */
+/* 3x3, stride 1, 64 planes in: taps from an input patch held in LDS   */
+/* ------------------------------------------------------------------ */
+
+/* With 64 input planes a K-tile of the kernels above moves 64 bytes per
+ * position from L2 for 32 multiply-adds per output plane, nine times per
+ * pixel (once per tap), and the path from L2 to LDS, not the matrix core, sets
+ * their time.  Here a workgroup owns 8 rows x 32 columns of one image's output,
+ * copies the 10 x 34 pixel patch those positions read once (43.5 KiB, straight
+ * to LDS), and takes the B fragments of all nine taps from it: a fragment of
+ * tap (kh, kw) is the patch shifted by (kh, kw).  Only the weights stream
+ * (K-tiles of one tap x 32 planes, four stages, as in conv_wide_kernel).
+ *
+ * Patch layout: 1 KiB blocks of eight pixels x eight 16-byte vectors, pixel pp
+ * of the patch (row-major, 34 wide) in block pp / 8; inside a block vector v of
+ * pixel pp sits in slot 8 (pp % 8) + (v ^ ((pp / 2) % 8)).  A fragment read
+ * takes one vector index from 32 consecutive pixels; the swizzle spreads every
+ * run of sixteen over all banks wherever it starts.  Pixels outside the image
+ * are fetched out of the buffer's range and arrive as zeros.
+ *
+ * Four waves; wave w computes all BM planes of tile rows 2w and 2w+1. */
+#define PATCH_TW 32
+#define PATCH_TH 8
+#define PATCH_CI 64
+
+template <int DT, bool CLO, int BM>
+__global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
+	typedef ConvTraits<DT> TR;
+	typedef typename TR::elem elem;
+	static_assert(TR::CHUNK == 16 && sizeof(elem) == 2, "a half type");
+	constexpr int TW = PATCH_TW, TH = PATCH_TH, PW = TW + 2, PH = TH + 2, CI = PATCH_CI;
+	constexpr int NPIX = PW * PH, PBLOCKS = (NPIX + 7) / 8, P_PW = (PBLOCKS + 3) / 4;
+	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = 4, WAVES = 4;
+	constexpr int A_VECS = MB * KCH * 64, A_PW = MB * KCH / WAVES;
+	constexpr int NKT = 9 * CI / 32;	/* K-tiles: tap kt / 2, planes 32 (kt % 2) .. + 32 */
+	static_assert(CI == 64 && MB * KCH % WAVES == 0 && TH == 2 * WAVES, "shape");
+	__shared__ floatx4 patch[PBLOCKS * 64];
+	__shared__ floatx4 astage[NST * A_VECS];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+	/* consecutive tiles (plane block fastest, then along the row) share halo
+	 * pixels: each XCD takes one run of them */
+	const int tx_n = (p.oW + TW - 1) / TW, ty_n = (p.oH + TH - 1) / TH;
+	int tile_m, tx, ty, img;
+	{
+		const int total = p.tiles_m * p.tiles_n, per_xcd = (total + 7) / 8;
+		const int local = blockIdx.x >> 3;
+		const int t = (blockIdx.x & 7) * per_xcd + local;
+		if (local >= per_xcd || t >= total)
+			return;
+		tile_m = t % p.tiles_m;
+		const int sp = t / p.tiles_m;
+		tx = sp % tx_n;
+		ty = (sp / tx_n) % ty_n;
+		img = sp / (tx_n * ty_n);
+	}
+
+	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
+	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
+	/* ---- the patch: block wave + 4 i, this lane pixel lane / 8, slot lane % 8 ---- */
+#pragma unroll
+	for (int i = 0; i < P_PW; i++) {
+		const int blk = wave + WAVES * i;
+		if (blk < PBLOCKS) {
+			const int pp = blk * 8 + (lane >> 3);
+			const int v = (lane & 7) ^ ((pp >> 1) & 7);
+			const int pr = pp / PW, pc = pp - pr * PW;
+			const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
+			const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			const unsigned voff = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + v * 8) * (int)sizeof(elem)) : 0x80000000u;
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(patch + blk * 64), 16, voff, 0, 0, 0);
+		}
+	}
+	/* ---- the weights: block wave + 4 i counts (chunk, 32-row block) of a K-tile ---- */
+	unsigned a_off_[A_PW];
+	int a_lds_[A_PW];
+#pragma unroll
+	for (int i = 0; i < A_PW; i++) {
+		const int idx = wave + WAVES * i, mbi = idx % MB, kci = idx / MB;
+		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
+		a_lds_[i] = (kci * MB + mbi) * 64;
+	}
+	int t_kc = 0;
+	auto issue = [&](auto st_) {
+		constexpr int st = decltype(st_)::value;
+#pragma unroll
+		for (int i = 0; i < A_PW; i++)
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16, lane * 16,
+				a_off_[i] + (unsigned)t_kc * 1024u, 0, 0);
+		t_kc += KCH;
+	};
+
+	/* patch pixel of this lane's position at tap (0, 0), for its two tile rows */
+	int pbase_[TN];
+#pragma unroll
+	for (int j = 0; j < TN; j++)
+		pbase_[j] = (2 * wave + j) * PW + (lane & 31);
+	floatx4 af[2][TM], bf[2][TN];
+	auto read_frags = [&](auto st_, int kci, int kt, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
+		constexpr int st = decltype(st_)::value;
+		const floatx4 *la = astage + st * A_VECS;
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+			a[i] = la[(kci * MB + i) * 64 + lane];
+		const int tap = kt >> 1, kh = (tap * 11) >> 5, kw = tap - 3 * kh;	/* tap / 3 for tap < 9 */
+		const int toff = kh * PW + kw;
+		const int v = (kt & 1) * 4 + kci * 2 + (lane >> 5);
+#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			const int pp = pbase_[j] + toff;
+			b[j] = patch[pp * 8 + (v ^ ((pp >> 1) & 7))];
+		}
+	};
+
+	typename ConvAcc<DT>::T acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; i++)
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[i][j][r] = 0;
+	auto mma = [&](int set) {
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+				conv_mma<DT>(acc[i][j], af[set][i], bf[set][j]);
+	};
+
+	typedef std::integral_constant<int, 0> S0;
+	typedef std::integral_constant<int, 1> S1;
+	typedef std::integral_constant<int, 2> S2;
+	typedef std::integral_constant<int, 3> S3;
+	issue(S0{});
+	issue(S1{});
+	issue(S2{});
+	issue(S3{});
+	wide_wait<3 * A_PW, false>();	/* the patch and the first K-tile */
+	__builtin_amdgcn_s_barrier();
+	read_frags(S0{}, 0, 0, af[0], bf[0]);
+	auto step = [&](int kt, auto st, auto st1, auto steady_) {
+		constexpr bool steady = decltype(steady_)::value;
+		read_frags(st, 1, kt, af[1], bf[1]);
+		mma(0);
+		if (steady)
+			wide_wait<2 * A_PW, true>();
+		else
+			wide_wait<0, true>();
+		__builtin_amdgcn_s_barrier();
+		if (steady || kt + NST < NKT)
+			issue(st);
+		if (steady || kt + 1 < NKT)
+			read_frags(st1, 0, kt + 1, af[0], bf[0]);
+		mma(1);
+	};
+	static_assert(NKT == 18 && NST == 4, "the schedule below");
+	int kt = 0;
+	for (; kt + 7 < NKT; kt += 4) {		/* kt = 0, 4, 8 */
+		step(kt, S0{}, S1{}, std::true_type{});
+		step(kt + 1, S1{}, S2{}, std::true_type{});
+		step(kt + 2, S2{}, S3{}, std::true_type{});
+		step(kt + 3, S3{}, S0{}, std::true_type{});
+	}
+	step(12, S0{}, S1{}, std::false_type{});
+	step(13, S1{}, S2{}, std::false_type{});
+	step(14, S2{}, S3{}, std::false_type{});
+	step(15, S3{}, S0{}, std::false_type{});
+	step(16, S0{}, S1{}, std::false_type{});
+	step(17, S1{}, S2{}, std::false_type{});
+
+	/* ---- epilogue ---- */
+	elem *y = (elem *)p.y;
+	int *lrow = (int *)astage;
+	__syncthreads();
+	if (tid < BM) {
+		const int mc = min(tile_m * BM + tid, p.Co - 1);
+		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+		if (p.scale)
+			lrow[BM + tid] = __float_as_int(p.scale[mc]);
+	}
+	__syncthreads();
+	const bool has_scale = p.scale != 0;
+#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int oy = ty * TH + 2 * wave + j, ox = tx * TW + (lane & 31);
+		if (oy >= p.oH || ox >= p.oW)
+			continue;
+		const int rem = oy * p.oW + ox;
+		const size_t n = (size_t)img * p.oHW + rem;
+		const size_t ybase = (size_t)img * p.Co * p.oHW + rem;
+#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			const int m0 = tile_m * BM + i * 32 + 4 * (lane >> 5);
+#pragma unroll
+			for (int g = 0; g < 4; g++) {
+				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+				const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
+				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+				floatx4 rowscale = { 1, 1, 1, 1 };
+				if (has_scale)
+					rowscale = *(const floatx4 *)(lrow + BM + ml);
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int r = 4 * g + e, m = m0 + 8 * g + e;
+					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
+					if (p.act)
+						v = v > p.thr ? v : p.val;
+					if constexpr (!CLO) {
+						if (m < p.Co)
+							y[ybase + (size_t)m * p.oHW] = (elem)v;
+					}
+					quad.v[e] = (elem)v;
+				}
+				if constexpr (CLO) {
+					if (m0 + 8 * g < p.Co)
+						*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
+				}
+			}
+		}
+	}
+#endif
+}
+
+/* ------------------------------------------------------------------ */
 /* host side                                                           */
 /* ------------------------------------------------------------------ */
 
@@ -1527,6 +1756,35 @@ static void conv_launch_wide(ConvParams &p)
 		THError("thhip_conv2d: the 256-position tiles are for the half types");
 }
 
+/* Whether conv_patch_kernel can run this layer. */
+template <int DT>
+static bool conv_patch_ok(const ConvParams &p)
+{
+	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16)
+		return p.x_cl == 1 && p.Ci == PATCH_CI && p.kH == 3 && p.kW == 3 && p.dH == 1 && p.dW == 1 &&
+			p.x_bytes < 0x7fffffffu && !g_force_generic_cl && (!p.y_cl || p.Co % 4 == 0);
+	return false;
+}
+
+template <int DT, int BM>
+static void conv_launch_patch(ConvParams &p)
+{
+	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
+		p.tiles_m = (p.Co + BM - 1) / BM;
+		p.tiles_n = p.B * ((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH);
+		p.splitk = 1;
+		if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
+			THError("thhip_conv2d: packed weights shorter than the tile grid");
+		const long total = (long)p.tiles_m * p.tiles_n;
+		dim3 grid((unsigned)(8 * ((total + 7) / 8)));
+		if (p.y_cl)
+			conv_patch_kernel<DT, true, BM><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+		else
+			conv_patch_kernel<DT, false, BM><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+	} else
+		THError("thhip_conv2d: the patch kernel is for the half types");
+}
+
 template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
@@ -1560,7 +1818,14 @@ static void conv_dispatch(ConvParams &p)
 		 * workgroups per CU) wins by 6-15 %; with fewer, and for layers of 128
 		 * planes or less, the smaller tiles below do. */
 		const long t256 = (long)((p.Co + 255) / 256) * ((p.N + 255) / 256);
-		if (conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128)
+		/* 64 input planes, 3x3: the taps come from a patch in LDS (measured with
+		 * random data, batch 16 / 64: 64->64 @224^2 129 -> 101 / 560 -> 414 us,
+		 * 64->128 @112^2 55 -> 49 / 226 -> 209 us, 64->64 @56^2 12.9 -> 11.3 /
+		 * 36 -> 29 us; 128 rows per workgroup measured slower than 64) */
+		const long tpatch = (long)((p.Co + 63) / 64) * p.B * ((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH);
+		if (conv_patch_ok<DT>(p) && tpatch >= 128)
+			bm = 64, bn = 1;
+		else if (conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128)
 			bm = bn = 256;
 		else if (conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 >= 80)
 			bm = 128, bn = 256;
@@ -1604,6 +1869,11 @@ static void conv_dispatch(ConvParams &p)
 		wgs = g_force_wgs;
 	if (DT == THHIP_F32 && g_force_kch)
 		kch = g_force_kch;
+	if (bn == 1) {	/* (64, 1): the patch kernel */
+		if (!conv_patch_ok<DT>(p))
+			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64 planes, 3x3, stride 1");
+		return conv_launch_patch<DT, 64>(p);
+	}
 	if (bn >= 256) {
 		if (!conv_wide_ok<DT>(p))
 			THError("thhip_conv2d: the 256-position tiles need a half type and channels-last input with Ci %% 32 == 0");
