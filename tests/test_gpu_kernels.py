@@ -253,7 +253,7 @@ def test_conv_half_channels_last(hiplib, oracle, dt):
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_conv_half_wide_tile(hiplib, oracle, dt):
-    """The 256-position tiles whose operands go from global memory straight to LDS: K-tile
+    """The tiles whose operands go from global memory straight to LDS, every shape: K-tile
     counts around every edge of their pipelines (prologue of up to four tiles, steady state in
     rounds of three or four, drain), partial tiles along both axes, padding, strides, both
     output orders."""
@@ -279,29 +279,30 @@ def test_conv_half_wide_tile(hiplib, oracle, dt):
                 G.note("wide tile %s y_cl %d dtype %d" % ((B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW), y_cl, dt))
                 hiplib.thhip_conv_set_tuning(128, 128, 0, 0)
                 narrow = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
-                # eight and four waves; for 256 rows K-tiles of 32 (four LDS stages) or, with the
-                # third argument 4 and Ci % 64 == 0, of 64 (two stages)
-                for (bm, kt64) in ((256, 0), (256, 4), (128, 0)):
-                    hiplib.thhip_conv_set_tuning(bm, 256, kt64, 0)
+                # 256 positions: eight and four waves; for 256 rows K-tiles of 32 (four LDS stages) or,
+                # with the third argument 4 and Ci % 64 == 0, of 64 (two stages).  The smaller tiles
+                # (third argument 9: the kernel that loads straight into LDS): four waves, four stages.
+                for tune in ((256, 256, 0), (256, 256, 4), (128, 256, 0), (128, 128, 9), (128, 64, 9), (64, 128, 9), (64, 64, 9)):
+                    hiplib.thhip_conv_set_tuning(tune[0], tune[1], tune[2], 0)
                     got = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
-                    G.assert_close(got, want, HALF_TOL, str((Ci, Co, kH, y_cl, bm, kt64)))
-                    G.assert_close(got, narrow, 1e-2, "vs the 128x128 tile " + str((Ci, Co, kH, y_cl, bm, kt64)))
+                    G.assert_close(got, want, HALF_TOL, str((Ci, Co, kH, y_cl, tune)))
+                    G.assert_close(got, narrow, 1e-2, "vs the register-staged 128x128 tile " + str((Ci, Co, kH, y_cl, tune)))
     finally:
         hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_conv_half_patch_kernel(hiplib, oracle, dt):
-    """3x3 stride-1 convolutions of 64 planes whose taps come from an input patch in LDS:
+    """3x3 stride-1 convolutions of 64 or 128 planes whose taps come from an input patch in LDS:
     images smaller and larger than the 8 x 32 tile, partial tiles on both axes, padding 0, 1
     and 2, plane counts that leave a partial 64-row tile, both output orders."""
     from thnets_amd import api
     g = cases.rng(912)
-    shapes = [(2, 5, 7, 64, 1, 1), (1, 8, 32, 128, 1, 1), (3, 19, 45, 72, 1, 1), (1, 40, 33, 200, 0, 0), (2, 9, 70, 36, 2, 1),
-              (1, 16, 64, 260, 1, 0), (1, 3, 3, 64, 0, 0)]
+    shapes = [(2, 5, 7, 64, 1, 1, 64), (1, 8, 32, 128, 1, 1, 64), (3, 19, 45, 72, 1, 1, 64), (1, 40, 33, 200, 0, 0, 64),
+              (2, 9, 70, 36, 2, 1, 64), (1, 16, 64, 260, 1, 0, 64), (1, 3, 3, 64, 0, 0, 64),
+              (2, 11, 37, 72, 1, 1, 128), (1, 8, 32, 128, 0, 1, 128), (1, 21, 9, 40, 1, 1, 128)]   # 128 planes: two patches
     try:
-        for (B, H, W, Co, pH, pW) in shapes:
-            Ci = 64
+        for (B, H, W, Co, pH, pW, Ci) in shapes:
             x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
             w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
             b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
@@ -311,7 +312,7 @@ def test_conv_half_patch_kernel(hiplib, oracle, dt):
             raw = oracle.conv2d(xr, wr, None, (1, 1), (pH, pW))
             want = np.maximum(raw * sc[None, :, None, None] + b[None, :, None, None], 0)
             for y_cl in (1, 0):
-                G.note("patch kernel %s y_cl %d dtype %d" % ((B, H, W, Co, pH, pW), y_cl, dt))
+                G.note("patch kernel %s y_cl %d dtype %d" % ((B, Ci, H, W, Co, pH, pW), y_cl, dt))
                 hiplib.thhip_conv_set_tuning(64, 64, 0, 0)
                 narrow = G.conv2d_layout(hiplib, x, w, b, (1, 1), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
                 hiplib.thhip_conv_set_tuning(64, 1, 0, 0)

@@ -1170,7 +1170,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 }
 
 /* ------------------------------------------------------------------ */
-/* 3x3, stride 1, 64 planes in: taps from an input patch held in LDS   */
+/* 3x3, stride 1, 64 or 128 planes in: taps from an input patch in LDS */
 /* ------------------------------------------------------------------ */
 
 /* With 64 input planes a K-tile of the kernels above moves 64 bytes per
@@ -1181,6 +1181,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
  * to LDS), and takes the B fragments of all nine taps from it: a fragment of
  * tap (kh, kw) is the patch shifted by (kh, kw).  Only the weights stream
  * (K-tiles of one tap x 32 planes, four stages, as in conv_wide_kernel).
+ * 128 planes run as two blocks of 64: patch, nine taps, next patch, nine taps.
  *
  * Patch layout: 1 KiB blocks of eight pixels x eight 16-byte vectors, pixel pp
  * of the patch (row-major, 34 wide) in block pp / 8; inside a block vector v of
@@ -1192,21 +1193,20 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
  * Four waves; wave w computes all BM planes of tile rows 2w and 2w+1. */
 #define PATCH_TW 32
 #define PATCH_TH 8
-#define PATCH_CI 64
 
-template <int DT, bool CLO, int BM>
+template <int DT, bool CLO, int BM, int CI>
 __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
 	static_assert(TR::CHUNK == 16 && sizeof(elem) == 2, "a half type");
-	constexpr int TW = PATCH_TW, TH = PATCH_TH, PW = TW + 2, PH = TH + 2, CI = PATCH_CI;
+	constexpr int TW = PATCH_TW, TH = PATCH_TH, PW = TW + 2, PH = TH + 2, PCI = 64, NCB = CI / PCI;
 	constexpr int NPIX = PW * PH, PBLOCKS = (NPIX + 7) / 8, P_PW = (PBLOCKS + 3) / 4;
 	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = 4, WAVES = 4;
 	constexpr int A_VECS = MB * KCH * 64, A_PW = MB * KCH / WAVES;
-	constexpr int NKT = 9 * CI / 32;	/* K-tiles: tap kt / 2, planes 32 (kt % 2) .. + 32 */
-	static_assert(CI == 64 && MB * KCH % WAVES == 0 && TH == 2 * WAVES, "shape");
+	constexpr int NKT = 9 * PCI / 32;	/* K-tiles per block of 64 planes: tap kt / 2, planes 32 (kt % 2) .. + 32 */
+	static_assert(CI % PCI == 0 && MB * KCH % WAVES == 0 && TH == 2 * WAVES, "shape");
 	__shared__ floatx4 patch[PBLOCKS * 64];
 	__shared__ floatx4 astage[NST * A_VECS];
 
@@ -1233,20 +1233,23 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 
 	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
 	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
-	/* ---- the patch: block wave + 4 i, this lane pixel lane / 8, slot lane % 8 ---- */
+	/* ---- the patch of plane block cb: block wave + 4 i, this lane pixel lane / 8, slot lane % 8 ---- */
+	auto load_patch = [&](int cb) {
 #pragma unroll
-	for (int i = 0; i < P_PW; i++) {
-		const int blk = wave + WAVES * i;
-		if (blk < PBLOCKS) {
-			const int pp = blk * 8 + (lane >> 3);
-			const int v = (lane & 7) ^ ((pp >> 1) & 7);
-			const int pr = pp / PW, pc = pp - pr * PW;
-			const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
-			const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-			const unsigned voff = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + v * 8) * (int)sizeof(elem)) : 0x80000000u;
-			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(patch + blk * 64), 16, voff, 0, 0, 0);
+		for (int i = 0; i < P_PW; i++) {
+			const int blk = wave + WAVES * i;
+			if (blk < PBLOCKS) {
+				const int pp = blk * 8 + (lane >> 3);
+				const int v = (lane & 7) ^ ((pp >> 1) & 7);
+				const int pr = pp / PW, pc = pp - pr * PW;
+				const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
+				const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+				const unsigned voff = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + cb * PCI + v * 8) * (int)sizeof(elem))
+					: 0x80000000u;
+				__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(patch + blk * 64), 16, voff, 0, 0, 0);
+			}
 		}
-	}
+	};
 	/* ---- the weights: block wave + 4 i counts (chunk, 32-row block) of a K-tile ---- */
 	unsigned a_off_[A_PW];
 	int a_lds_[A_PW];
@@ -1256,14 +1259,16 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
 		a_lds_[i] = (kci * MB + mbi) * 64;
 	}
-	int t_kc = 0;
+	/* K-tile ikt of plane block t_cb: chunks (k = tap Ci + plane) / 16 */
+	int ikt = 0, t_cb = 0;
 	auto issue = [&](auto st_) {
 		constexpr int st = decltype(st_)::value;
+		const int kc = (ikt >> 1) * (CI / 16) + t_cb * (PCI / 16) + (ikt & 1) * KCH;
 #pragma unroll
 		for (int i = 0; i < A_PW; i++)
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16, lane * 16,
-				a_off_[i] + (unsigned)t_kc * 1024u, 0, 0);
-		t_kc += KCH;
+				a_off_[i] + (unsigned)kc * 1024u, 0, 0);
+		++ikt;
 	};
 
 	/* patch pixel of this lane's position at tap (0, 0), for its two tile rows */
@@ -1308,13 +1313,6 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	typedef std::integral_constant<int, 1> S1;
 	typedef std::integral_constant<int, 2> S2;
 	typedef std::integral_constant<int, 3> S3;
-	issue(S0{});
-	issue(S1{});
-	issue(S2{});
-	issue(S3{});
-	wide_wait<3 * A_PW, false>();	/* the patch and the first K-tile */
-	__builtin_amdgcn_s_barrier();
-	read_frags(S0{}, 0, 0, af[0], bf[0]);
 	auto step = [&](int kt, auto st, auto st1, auto steady_) {
 		constexpr bool steady = decltype(steady_)::value;
 		read_frags(st, 1, kt, af[1], bf[1]);
@@ -1331,19 +1329,34 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 		mma(1);
 	};
 	static_assert(NKT == 18 && NST == 4, "the schedule below");
-	int kt = 0;
-	for (; kt + 7 < NKT; kt += 4) {		/* kt = 0, 4, 8 */
-		step(kt, S0{}, S1{}, std::true_type{});
-		step(kt + 1, S1{}, S2{}, std::true_type{});
-		step(kt + 2, S2{}, S3{}, std::true_type{});
-		step(kt + 3, S3{}, S0{}, std::true_type{});
+	/* One block of 64 planes at a time: its patch, then its 18 K-tiles.  After the
+	 * last barrier of a block no wave reads LDS any more, so the next block's
+	 * loads may start at once. */
+	for (int cb = 0; cb < NCB; cb++) {
+		t_cb = cb;
+		ikt = 0;
+		load_patch(cb);
+		issue(S0{});
+		issue(S1{});
+		issue(S2{});
+		issue(S3{});
+		wide_wait<3 * A_PW, false>();	/* the patch and the first K-tile */
+		__builtin_amdgcn_s_barrier();
+		read_frags(S0{}, 0, 0, af[0], bf[0]);
+		int kt = 0;
+		for (; kt + 7 < NKT; kt += 4) {		/* kt = 0, 4, 8 */
+			step(kt, S0{}, S1{}, std::true_type{});
+			step(kt + 1, S1{}, S2{}, std::true_type{});
+			step(kt + 2, S2{}, S3{}, std::true_type{});
+			step(kt + 3, S3{}, S0{}, std::true_type{});
+		}
+		step(12, S0{}, S1{}, std::false_type{});
+		step(13, S1{}, S2{}, std::false_type{});
+		step(14, S2{}, S3{}, std::false_type{});
+		step(15, S3{}, S0{}, std::false_type{});
+		step(16, S0{}, S1{}, std::false_type{});
+		step(17, S1{}, S2{}, std::false_type{});
 	}
-	step(12, S0{}, S1{}, std::false_type{});
-	step(13, S1{}, S2{}, std::false_type{});
-	step(14, S2{}, S3{}, std::false_type{});
-	step(15, S3{}, S0{}, std::false_type{});
-	step(16, S0{}, S1{}, std::false_type{});
-	step(17, S1{}, S2{}, std::false_type{});
 
 	/* ---- epilogue ---- */
 	elem *y = (elem *)p.y;
@@ -1761,7 +1774,7 @@ template <int DT>
 static bool conv_patch_ok(const ConvParams &p)
 {
 	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16)
-		return p.x_cl == 1 && p.Ci == PATCH_CI && p.kH == 3 && p.kW == 3 && p.dH == 1 && p.dW == 1 &&
+		return p.x_cl == 1 && (p.Ci == 64 || p.Ci == 128) && p.kH == 3 && p.kW == 3 && p.dH == 1 && p.dW == 1 &&
 			p.x_bytes < 0x7fffffffu && !g_force_generic_cl && (!p.y_cl || p.Co % 4 == 0);
 	return false;
 }
@@ -1777,10 +1790,14 @@ static void conv_launch_patch(ConvParams &p)
 			THError("thhip_conv2d: packed weights shorter than the tile grid");
 		const long total = (long)p.tiles_m * p.tiles_n;
 		dim3 grid((unsigned)(8 * ((total + 7) / 8)));
-		if (p.y_cl)
-			conv_patch_kernel<DT, true, BM><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+		if (p.Ci == 64 && p.y_cl)
+			conv_patch_kernel<DT, true, BM, 64><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+		else if (p.Ci == 64)
+			conv_patch_kernel<DT, false, BM, 64><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+		else if (p.y_cl)
+			conv_patch_kernel<DT, true, BM, 128><<<grid, dim3(256), 0, thhip_stream()>>>(p);
 		else
-			conv_patch_kernel<DT, false, BM><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+			conv_patch_kernel<DT, false, BM, 128><<<grid, dim3(256), 0, thhip_stream()>>>(p);
 	} else
 		THError("thhip_conv2d: the patch kernel is for the half types");
 }
@@ -1808,7 +1825,9 @@ static void conv_dispatch(ConvParams &p)
 	 * Splitting K measured slower than unsplit 64x64 tiles on every layer that
 	 * has tiles for all CUs, so only layers of a few tiles are split (below). */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
+	const long t64 = (long)((p.Co + 63) / 64) * ((p.N + 63) / 64);
 	int bm = 64, bn = 64, splitk = 1, wgs = 0, kch = conv_kch(DT, p.x_cl != 0);
+	bool direct = false;	/* half types: operands loaded straight into LDS (conv_wide_kernel) */
 	if (DT == THHIP_F16 || DT == THHIP_BF16) {
 		/* tiles of 256 positions (operands straight to LDS) where whole tiles of
 		 * 256 planes fill most CUs for a turn: one such tile per CU multiplies
@@ -1818,18 +1837,36 @@ static void conv_dispatch(ConvParams &p)
 		 * workgroups per CU) wins by 6-15 %; with fewer, and for layers of 128
 		 * planes or less, the smaller tiles below do. */
 		const long t256 = (long)((p.Co + 255) / 256) * ((p.N + 255) / 256);
-		/* 64 input planes, 3x3: the taps come from a patch in LDS (measured with
-		 * random data, batch 16 / 64: 64->64 @224^2 129 -> 101 / 560 -> 414 us,
+		/* 64 or 128 input planes, 3x3: the taps come from a patch in LDS (measured
+		 * with random data, batch 16 / 64: 64->64 @224^2 129 -> 101 / 560 -> 414 us,
 		 * 64->128 @112^2 55 -> 49 / 226 -> 209 us, 64->64 @56^2 12.9 -> 11.3 /
-		 * 36 -> 29 us; 128 rows per workgroup measured slower than 64) */
+		 * 36 -> 29 us, 128->128 @112^2 90 -> 76 / 382 -> 361 us, 128->256 @56^2
+		 * 54 -> 42 / 183 -> 157 us (the 256x256 tile: 41 / 171 us); 128 rows per
+		 * workgroup measured slower than 64) */
 		const long tpatch = (long)((p.Co + 63) / 64) * p.B * ((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH);
-		if (conv_patch_ok<DT>(p) && tpatch >= 128)
+		const bool wide256 = conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128;
+		if (conv_patch_ok<DT>(p) && tpatch >= 128 && !(wide256 && p.Ci > 64))	/* (inside a network 128->256 is better off below) */
 			bm = 64, bn = 1;
-		else if (conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128)
-			bm = bn = 256;
-		else if (conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 >= 80)
-			bm = 128, bn = 256;
-		else if (p.Co <= 64)
+		else if (conv_wide_ok<DT>(p)) {
+			/* operands straight into LDS, the tile by how many there are (random
+			 * data; us for the register-staged kernel's best tile -> this one):
+			 * 256x256 from 129 whole tiles (256->256 @56^2 batch 16 97 -> 68);
+			 * below that 128x128 from 300 tiles of that size (512->512 @28^2 batch
+			 * 16 96 -> 73, where 128x256 takes 86), 128x64 from 150 (256->256
+			 * @14^2 batch 64 37 -> 25), else 64x64 (512->512 @14^2 batch 16 41 ->
+			 * 31, @7^2 48 -> 24, 192->384 @13^2 17 -> 13; also at batch 1, where
+			 * the other kernel splits K: 192->384 @13^2 22 -> 11, 512->512 @14^2
+			 * 31 -> 24); 64-row tiles when 128 rows would leave a partly empty tile */
+			direct = true;
+			if (wide256)
+				bm = bn = 256;
+			else if (p.Co % 128 == 0 && t128 >= 300)
+				bm = bn = 128;
+			else if (p.Co % 128 == 0 && t128 >= 150)
+				bm = 128;
+			else if (t128 >= 150)
+				bn = 128;
+		} else if (p.Co <= 64)
 			bn = 128;
 		else if (t128 >= 200)
 			bm = bn = 128;
@@ -1848,8 +1885,7 @@ static void conv_dispatch(ConvParams &p)
 	 * deterministic K split pays, one part per sixteen K-tiles up to eight parts
 	 * (AlexNet batch 1: conv3 42 -> 23 us, conv4 81 -> 27 us, conv5 55 -> 29 us;
 	 * more parts lose again to the serial sum of the last arriver). */
-	const long t64 = (long)((p.Co + 63) / 64) * ((p.N + 63) / 64);
-	if (bm == 64 && bn == 64 && t64 <= 128) {	/* 65..128 tiles: two parts at most */
+	if (!direct && bm == 64 && bn == 64 && t64 <= 128) {	/* 65..128 tiles: two parts at most */
 		const int nkt = p.KC / kch;
 		int parts = (nkt + 8) / 16;
 		if (parts > 256 / t64)
@@ -1859,11 +1895,13 @@ static void conv_dispatch(ConvParams &p)
 		if (parts > 1)
 			splitk = parts;
 	}
+	if (g_force_bm || g_force_bn)
+		direct = g_force_splitk == 9;
 	if (g_force_bm)
 		bm = g_force_bm;
 	if (g_force_bn)
 		bn = g_force_bn;
-	if (g_force_splitk)
+	if (g_force_splitk && g_force_splitk != 9)
 		splitk = g_force_splitk;
 	if (g_force_wgs)
 		wgs = g_force_wgs;
@@ -1871,12 +1909,14 @@ static void conv_dispatch(ConvParams &p)
 		kch = g_force_kch;
 	if (bn == 1) {	/* (64, 1): the patch kernel */
 		if (!conv_patch_ok<DT>(p))
-			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64 planes, 3x3, stride 1");
+			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64 or 128 planes, 3x3, stride 1");
 		return conv_launch_patch<DT, 64>(p);
 	}
-	if (bn >= 256) {
+	/* tiles whose operands are loaded straight into LDS (the tuning hook asks for
+	 * them with 9 as its split-K argument, or with a 256-position tile) */
+	if (direct || bn >= 256) {
 		if (!conv_wide_ok<DT>(p))
-			THError("thhip_conv2d: the 256-position tiles need a half type and channels-last input with Ci %% 32 == 0");
+			THError("thhip_conv2d: tiles loaded straight into LDS need a half type and channels-last input with Ci %% 32 == 0");
 		/* K-tiles of 64 values in two stages measured the same as 32 in four
 		 * (the tuning hook's split-K argument, 4, selects them for the tests) */
 		if (bm == 256 && bn == 256 && p.Ci % 64 == 0 && g_force_splitk == 4)
@@ -1885,8 +1925,14 @@ static void conv_dispatch(ConvParams &p)
 			return conv_launch_wide<DT, 256, 256, 2, 4, 2, 4>(p);
 		if (bm == 128 && bn == 256)
 			return conv_launch_wide<DT, 128, 256, 1, 4, 2, 3>(p);
-		if (bm == 128 && bn == 512)
-			return conv_launch_wide<DT, 128, 512, 2, 4, 2, 3>(p);
+		if (bm == 128 && bn == 128)
+			return conv_launch_wide<DT, 128, 128, 2, 2, 2, 4>(p);
+		if (bm == 128 && bn == 64)
+			return conv_launch_wide<DT, 128, 64, 2, 2, 2, 4>(p);
+		if (bm == 64 && bn == 128)
+			return conv_launch_wide<DT, 64, 128, 2, 2, 2, 4>(p);
+		if (bm == 64 && bn == 64)
+			return conv_launch_wide<DT, 64, 64, 2, 2, 2, 4>(p);
 		THError("thhip_conv2d: no %dx%d tile", bm, bn);
 	}
 #define CONV_TILES(KCH)                                                      \
