@@ -571,6 +571,17 @@ void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const i
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
 	int act, int thr, int val, int x_layout, int y_channels_last);
 
+/* The same when x is followed by x_tail_bytes (>= 64 to matter) bytes holding the
+ * code `zero`: channels-last layers with Ci % 64 == 0 then run on the kernel
+ * that loads its operands straight into LDS and fetches its padding from that
+ * tail (a load out of the buffer's range would give code 0 instead).  No
+ * counterpart in the reference: its im2col fills the padding itself
+ * (lowp_SpatialConvolution.c:90-134). */
+void thhip_conv2d_u8_layout_tail(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
+	int act, int thr, int val, int x_layout, int y_channels_last, int x_tail_bytes);
+
 /* Lowp_SpatialMaxPooling_updateOutput (lowp_SpatialMaxPooling.c:45-108) on
  * channels-last codes, C % 4 == 0. */
 void thhip_maxpool_u8_cl(const unsigned char *x, unsigned char *y, int B, int C, int H, int W, int oH, int oW,

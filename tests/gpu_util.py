@@ -78,10 +78,11 @@ def unary(lib, fn, x, out_shape, dtype, *args):
     return api.from_device_dtype(dy, out_shape, dtype)
 
 
-def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0, x_cl=0, y_cl=0):
+def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0, x_cl=0, y_cl=0, tail=0):
     """xq and the result are [B][C][H][W] arrays; x_cl = 1 / y_cl = 1 make the device
     copies channels-last ([B][H][W][C]), x_cl = 2 asks for the four-plane pixel path
-    (plane-major in memory); both call the layout entry point."""
+    (plane-major in memory); both call the layout entry point.  tail > 0 (with x_cl = 1):
+    the device copy is followed by that many bytes of the code `zero` and the call says so."""
     xq = np.ascontiguousarray(xq, np.uint8)
     wq = np.ascontiguousarray(wq, np.uint8)
     B, Ci, H, W = xq.shape
@@ -93,10 +94,19 @@ def conv2d_u8(lib, xq, wq, addend, d, pad, zero, prm, act=0, thr=0, val=0, x_cl=
         wp = lib.thhip_conv_pack_weight_u8_layout(wq.ctypes.data, Co, Ci, kH, kW, x_cl)
     else:
         wp = lib.thhip_conv_pack_weight_u8(wq.ctypes.data, Co, Ci, kH * kW)
-    dx = api.DeviceArray(lib, np.ascontiguousarray(xq.transpose(0, 2, 3, 1)) if x_cl == 1 else xq)
+    if tail:
+        assert x_cl == 1
+        dx = api.DeviceArray(lib, np.concatenate([np.ascontiguousarray(xq.transpose(0, 2, 3, 1)).ravel(),
+                                                  np.full(tail, zero, np.uint8)]))
+    else:
+        dx = api.DeviceArray(lib, np.ascontiguousarray(xq.transpose(0, 2, 3, 1)) if x_cl == 1 else xq)
     da = api.DeviceArray(lib, np.ascontiguousarray(addend, np.int32)) if addend is not None else None
     dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW)
-    if x_cl or y_cl:
+    if tail:
+        lib.thhip_conv2d_u8_layout_tail(dx.ptr, wp, da.ptr if da else None, dy.ptr, B, Ci, H, W, Co, kH, kW, d[0], d[1],
+                                        pad[0], pad[1], zero, prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"],
+                                        prm["c_shift"], act, thr, val, x_cl, y_cl, tail)
+    elif x_cl or y_cl:
         lib.thhip_conv2d_u8_layout(dx.ptr, wp, da.ptr if da else None, dy.ptr, B, Ci, H, W, Co, kH, kW, d[0], d[1],
                                    pad[0], pad[1], zero, prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"],
                                    prm["c_shift"], act, thr, val, x_cl, y_cl)

@@ -160,6 +160,49 @@ def test_conv_u8_channels_last_bit_exact(hiplib, oracle, i):
         hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
+DIRECT_CASES = [c for c in CL_CASES if c[1] % 64 == 0] + [
+    (2, 64, 20, 17, 260, 3, 3, 1, 1, 1, 1),      # several tiles along both axes, partial ones
+    (1, 128, 30, 30, 72, 1, 1, 1, 1, 0, 0),      # two K-tiles
+    (1, 64, 12, 12, 40, 1, 1, 1, 1, 0, 0),       # one K-tile
+    (3, 192, 13, 13, 384, 3, 3, 1, 1, 1, 1),     # an AlexNet layer: every border position reads the tail
+]
+
+
+@pytest.mark.parametrize("i", range(len(DIRECT_CASES)))
+def test_conv_u8_loaded_straight_into_lds_bit_exact(hiplib, oracle, i):
+    """Channels-last codes whose tensor is followed by a tail of the padding code: the kernel
+    that loads its operands straight into LDS (re-centring and column sums done on the
+    fragments, padding fetched from the tail) gives the codes of the restatement, on every
+    tile shape, with the bias add's tail rule and the fused threshold."""
+    B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW = DIRECT_CASES[i]
+    g = cases.rng(1500 + i)
+    x = g.uniform(-3, 3, (B, Ci, H, W)).astype(np.float32)
+    w = g.standard_normal((Co, Ci, kH, kW), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * kH * kW)))
+    b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.5)
+    d, p = (dH, dW), (pH, pW)
+    rngv = 16.0
+    om, osub = float(np.float32(255) / np.float32(rngv)), -rngv / 2
+    xq, im, isub = oracle.lowp_quantize(x)
+    wq, wm, wsub = oracle.lowp_quantize(w)
+    bq, bm, bsub = oracle.lowp_quantize(b)
+    want = oracle.lowp_conv2d(xq, im, isub, wq, wm, wsub, bq, bm, bsub, om, osub, d, p)
+    prm = oracle.lowp_mm_params(wm, wsub, im, isub, om, osub)
+    zero = int(np.round(np.float32(-isub) * np.float32(im)))
+    addend = np.array([oracle.lowp_bias_addend(int(c), bm, bsub, om) for c in bq], np.int32)
+    thr = oracle.lowp_scale_float(om, osub, 0.0)
+    try:
+        for tune in ((0, 0, 0, 0), (64, 64, 9, 0), (128, 64, 9, 0), (64, 128, 9, 0), (128, 128, 9, 0)):
+            hiplib.thhip_conv_set_tuning(*tune)
+            for y_cl in (1, 0):
+                for tail in (64, 200):
+                    got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, x_cl=1, y_cl=y_cl, tail=tail)
+                    assert np.array_equal(got, want), (tune, y_cl, tail, int((got != want).sum()))
+                got = G.conv2d_u8(hiplib, xq, wq, addend, d, p, zero, prm, act=1, thr=thr, val=thr, x_cl=1, y_cl=y_cl, tail=64)
+                assert np.array_equal(got, oracle.lowp_threshold(want, thr, thr)), (tune, y_cl)
+    finally:
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+
+
 def test_maxpool_and_relayout_channels_last(hiplib, oracle):
     g = cases.rng(1400)
     for (B, Cn, H, W, kH, kW, dH, dW, pH, pW, ceil) in ((2, 8, 13, 13, 3, 3, 2, 2, 0, 0, 0), (3, 64, 27, 27, 3, 3, 2, 2, 0, 0, 0),

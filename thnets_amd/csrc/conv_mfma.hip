@@ -50,6 +50,7 @@ struct ConvParams {
 	int mparts;		/* the tile grid is cut mparts x (8 / mparts) over the XCDs */
 	unsigned x_bytes;
 	unsigned w_bytes;	/* packed weights (the wide kernel's buffer descriptor) */
+	unsigned x_tail;	/* uint8: bytes of the padding code that follow x (0: none) */
 	/* split-K: S workgroups share an output tile, each over a K range */
 	int splitk;
 	int *ws;		/* [tile][S][BM*BN] partial accumulators (float or int bits) */
@@ -918,7 +919,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
 	constexpr int CHUNK = TR::CHUNK, VEC = TR::VEC;
-	static_assert(CHUNK == 16 && sizeof(elem) == 2, "a half type");
+	static_assert(CHUNK * sizeof(elem) == 32 && DT != THHIP_F32, "a half type or uint8 codes");
 	constexpr int WAVES = WGM * WGN;
 	constexpr int MB = BM / 32, TM = BM / WGM / 32, TN = BN / WGN / 32;
 	constexpr int VPP = 2 * KCH;			/* 16-byte vectors of a position's K-tile slice */
@@ -930,7 +931,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	constexpr int LOADS = A_PW + NPOS;		/* per wave and K-tile */
 	static_assert(KCH == 2 || KCH == 4, "K-tiles of 32 or 64 values");
 	static_assert(MB * KCH % WAVES == 0 && BN / PPG % WAVES == 0 && NST >= 2 && NST <= 4, "tile shape");
-	static_assert(2 * BM * sizeof(int) <= NST * STAGE_VECS * sizeof(floatx4), "the epilogue's row constants fit");
+	static_assert((2 * BM + BN) * sizeof(int) <= NST * STAGE_VECS * sizeof(floatx4), "the epilogue's row and column constants fit");
 	__shared__ floatx4 lds[NST * STAGE_VECS];
 
 	const int tid = threadIdx.x;
@@ -969,7 +970,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		ix0_[q] = ox * p.dW - p.padW;
 		xoff_[q] = (((b * p.H + iy0_[q]) * p.W + ix0_[q]) * p.Ci + myvec * VEC) * (int)sizeof(elem);
 	}
-	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
+	/* uint8: the tensor is followed by x_tail >= 64 bytes of the padding code, and
+	 * what lies outside the image is fetched from there (a load out of range would
+	 * give code 0, which is not the code of 0.0) */
+	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes + p.x_tail, 0x00020000);
+	const unsigned outside = DT == THHIP_U8 ? p.x_bytes + (unsigned)(lane & 3) * 16u : 0x80000000u;
 	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
 	/* this wave's weight blocks: wave + WAVES i counts (chunk, 32-row block), 1 KiB each */
 	unsigned a_off_[A_PW];
@@ -994,7 +999,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		for (int q = 0; q < NPOS; q++) {
 			const int iy = iy0_[q] + t_kh, ix = ix0_[q] + t_kw;
 			const bool ok = n_ok_[q] && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-			const unsigned voff = ok ? (unsigned)(xoff_[q] + cl_off) : 0x80000000u;
+			const unsigned voff = ok ? (unsigned)(xoff_[q] + cl_off) : outside;
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(lb + (wave + WAVES * q) * 64), 16, voff, 0, 0, 0);
 		}
 		t_kc += KCH;
@@ -1032,7 +1037,26 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 #pragma unroll
 			for (int r = 0; r < 16; r++)
 				acc[i][j][r] = 0;
+	int colsum[TN];		/* uint8, waves with wm == 0: this lane's share of the column sums of the re-centred codes */
+#pragma unroll
+	for (int j = 0; j < TN; j++)
+		colsum[j] = 0;
 	auto mma = [&](int set) {
+		if constexpr (DT == THHIP_U8) {
+			/* code - 128 as a signed byte, done on the fragments (they never
+			 * pass through registers on their way to LDS) */
+#pragma unroll
+			for (int j = 0; j < TN; j++) {
+				intx4 cw = __builtin_bit_cast(intx4, bf[set][j]);
+#pragma unroll
+				for (int d = 0; d < 4; d++) {
+					cw[d] ^= (int)0x80808080;
+					if (wm == 0)
+						colsum[j] = __builtin_amdgcn_sdot4(cw[d], 0x01010101, colsum[j], false);
+				}
+				bf[set][j] = __builtin_bit_cast(floatx4, cw);
+			}
+		}
 #pragma unroll
 		for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -1117,17 +1141,81 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		}
 	}
 
-	/* ---- epilogue: (folded batch norm factor,) bias, optional threshold, store ---- */
+	/* ---- epilogue ---- */
 	elem *y = (elem *)p.y;
-	int *lrow = (int *)lds;		/* [BM] bias bits, [BM..2BM) factor bits */
+	int *lrow = (int *)lds;		/* [BM] bias bits or uint8 row term, [BM..2BM) factor bits or uint8 addend */
+	int *cs = lrow + 2 * BM;	/* uint8: [BN] column sums */
 	__syncthreads();		/* every wave is done with the tiles */
 	if (tid < BM) {
 		const int mc = min(tile_m * BM + tid, p.Co - 1);
-		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
-		if (p.scale)
-			lrow[BM + tid] = __float_as_int(p.scale[mc]);
+		if constexpr (DT == THHIP_U8) {
+			lrow[tid] = p.offB * p.rowsum[mc] + p.K * p.offA * p.offB;
+			lrow[BM + tid] = p.addend ? p.addend[mc] : 0;
+		} else {
+			lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+			if (p.scale)
+				lrow[BM + tid] = __float_as_int(p.scale[mc]);
+		}
+	}
+	if constexpr (DT == THHIP_U8) {
+		for (int i = tid; i < BN; i += 64 * WAVES)
+			cs[i] = 0;
+		__syncthreads();
+		if (wm == 0) {	/* the two halves of a column's K values sit in lanes l and l + 32 */
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+				atomicAdd(&cs[(wn * TN + j) * 32 + (lane & 31)], colsum[j]);
+		}
 	}
 	__syncthreads();
+	if constexpr (DT == THHIP_U8) {
+		/* as in conv_mfma_kernel: sum (w+a_off)(x+b_off) expanded, gemmlowp's
+		 * output stage, lowpadd with its unclamped tail, threshold */
+		const int tail0 = (p.oHW / 8) * 8;
+		const bool has_add = p.addend != 0;
+#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			const int nl = (wn * TN + j) * 32 + (lane & 31);
+			const int n = tile_n * BN + nl;
+			if (n >= p.N)
+				continue;
+			const int b = n / p.oHW, rem = n - b * p.oHW;
+			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+			const int colterm = p.offA * cs[nl];
+			const bool tail = rem >= tail0;
+#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+				for (int g = 0; g < 4; g++) {
+					unsigned packed = 0;
+					const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
+					const intx4 rowterm = *(const intx4 *)(lrow + ml);
+					const intx4 rowadd = *(const intx4 *)(lrow + BM + ml);
+#pragma unroll
+					for (int e = 0; e < 4; e++) {
+						const int r = 4 * g + e, m = m0 + 8 * g + e;
+						const int a = acc[i][j][r] + rowterm[e] + colterm;
+						int q = conv_requant(a, p.c_off, p.c_mult, p.c_shift);
+						if (has_add) {
+							const int sum = q + rowadd[e];
+							q = sum > 255 ? 255 : (tail ? (sum & 255) : (sum < 0 ? 0 : sum));
+						}
+						if (p.act)
+							q = q > p.ithr ? q : p.ival;
+						if constexpr (CLO)
+							packed |= (unsigned)q << (8 * e);
+						else if (m < p.Co)
+							y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
+					}
+					if constexpr (CLO) {
+						if (m0 + 8 * g < p.Co)
+							*(unsigned *)(y + (size_t)n * p.Co + m0 + 8 * g) = packed;
+					}
+				}
+			}
+		}
+	} else {
 	const bool has_scale = p.scale != 0;
 #pragma unroll
 	for (int j = 0; j < TN; j++) {
@@ -1165,6 +1253,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 				}
 			}
 		}
+	}
 	}
 #endif
 }
@@ -1726,13 +1815,18 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 #undef CONV_GO
 }
 
-/* Whether the wide kernels can run this layer: a half type, channels-last input
- * with whole K-tiles of 32 planes inside a tap, 32-bit byte offsets. */
+/* Whether the kernel that loads straight into LDS can run this layer: a half
+ * type or uint8, channels-last input with whole K-tiles (32 halfs, 64 codes)
+ * inside a tap, 32-bit byte offsets; uint8 input followed by a K-tile slice of
+ * the padding code. */
 template <int DT>
 static bool conv_wide_ok(const ConvParams &p)
 {
 	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16)
 		return p.x_cl == 1 && p.Ci % 32 == 0 && p.x_bytes < 0x7fffffffu && !g_force_generic_cl &&
+			(!p.y_cl || p.Co % 4 == 0);
+	if constexpr (DT == THHIP_U8)
+		return p.x_cl == 1 && p.Ci % 64 == 0 && p.x_bytes < 0x7fffff00u && !g_force_generic_cl && p.x_tail >= 64 &&
 			(!p.y_cl || p.Co % 4 == 0);
 	return false;
 }
@@ -1740,7 +1834,7 @@ static bool conv_wide_ok(const ConvParams &p)
 template <int DT, int BM, int BN, int WGM, int WGN, int KCH, int NST>
 static void conv_launch_wide(ConvParams &p)
 {
-	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
+	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16 || (DT == THHIP_U8 && BM <= 128 && BN <= 128 && KCH == 2)) {
 		p.tiles_m = (p.Co + BM - 1) / BM;
 		p.tiles_n = (p.N + BN - 1) / BN;
 		p.splitk = 1;
@@ -1766,7 +1860,7 @@ static void conv_launch_wide(ConvParams &p)
 		else
 			conv_wide_kernel<DT, false, BM, BN, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
 	} else
-		THError("thhip_conv2d: the 256-position tiles are for the half types");
+		THError("thhip_conv2d: no such tile loaded straight into LDS for this type");
 }
 
 /* Whether conv_patch_kernel can run this layer. */
@@ -1871,7 +1965,15 @@ static void conv_dispatch(ConvParams &p)
 		else if (t128 >= 200)
 			bm = bn = 128;
 	} else if (DT == THHIP_U8) {
-		if (p.x_cl == 1 && t128 >= 512)
+		if (conv_wide_ok<DT>(p)) {	/* as for the half types */
+			direct = true;
+			if (p.Co % 128 == 0 && t128 >= 300)
+				bm = bn = 128;
+			else if (p.Co % 128 == 0 && t128 >= 150)
+				bm = 128;
+			else if (t128 >= 150)
+				bn = 128;
+		} else if (p.x_cl == 1 && t128 >= 512)
 			bm = bn = 128;
 	} else if (DT == THHIP_F32 && t128 >= 300) {
 		kch = 2;
@@ -1916,7 +2018,7 @@ static void conv_dispatch(ConvParams &p)
 	 * them with 9 as its split-K argument, or with a 256-position tile) */
 	if (direct || bn >= 256) {
 		if (!conv_wide_ok<DT>(p))
-			THError("thhip_conv2d: tiles loaded straight into LDS need a half type and channels-last input with Ci %% 32 == 0");
+			THError("thhip_conv2d: tiles loaded straight into LDS need channels-last input with whole K-tiles of planes (and, uint8, a tail of padding codes)");
 		/* K-tiles of 64 values in two stages measured the same as 32 in four
 		 * (the tuning hook's split-K argument, 4, selects them for the tests) */
 		if (bm == 256 && bn == 256 && p.Ci % 64 == 0 && g_force_splitk == 4)
@@ -1968,6 +2070,7 @@ struct ConvU8Args {
 	int zero, a_off, b_off, c_off, c_mult, c_shift, ithr, ival;
 	int x_cl;	/* 0 plane-major, 1 channels-last, 2 plane-major read through a four-plane pixel copy */
 	int y_cl;
+	int x_tail;	/* bytes of the padding code after x */
 };
 
 /* Codes [B][C][HW], C <= 4 -> [B][HW][4] with code 128 (0 once re-centred) in
@@ -2081,6 +2184,7 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 			p.c_off = u8->c_off; p.c_mult = u8->c_mult; p.c_shift = u8->c_shift;
 			p.ithr = u8->ithr; p.ival = u8->ival;
 			p.x_cl = xl; p.y_cl = u8->y_cl;
+			p.x_tail = b0 + bn == B ? (unsigned)u8->x_tail : 0;	/* (a batch slice that ends inside x has no tail) */
 			if (xl == 2) {
 				/* the kernel reads a [B][H][W][4] copy with slack on both sides */
 				const long pixels = (long)bn * H * W;
@@ -2185,16 +2289,27 @@ extern "C" void *thhip_conv_pack_weight_u8(const unsigned char *w, int Co, int C
 	return thhip_conv_pack_weight_u8_layout(w, Co, Ci, 1, kHW, 0);
 }
 
+extern "C" void thhip_conv2d_u8_layout_tail(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
+	int act, int thr, int val, int x_layout, int y_channels_last, int x_tail_bytes)
+{
+	if (c_shift < 0 || c_shift > 31)
+		THError("thhip_conv2d_u8: shift %d out of range", c_shift);
+	if (x_tail_bytes < 0)
+		THError("thhip_conv2d_u8: negative tail");
+	ConvU8Args u8 = { addend, zero & 255, a_off, b_off, c_off, c_mult, c_shift, thr, val,
+		x_layout, y_channels_last != 0, x_tail_bytes };
+	conv_run(x, wpacked, 0, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
+}
+
 extern "C" void thhip_conv2d_u8_layout(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift,
 	int act, int thr, int val, int x_layout, int y_channels_last)
 {
-	if (c_shift < 0 || c_shift > 31)
-		THError("thhip_conv2d_u8: shift %d out of range", c_shift);
-	ConvU8Args u8 = { addend, zero & 255, a_off, b_off, c_off, c_mult, c_shift, thr, val,
-		x_layout, y_channels_last != 0 };
-	conv_run(x, wpacked, 0, 0, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, 0, 0, THHIP_U8, &u8);
+	thhip_conv2d_u8_layout_tail(x, wpacked, addend, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW,
+		zero, a_off, b_off, c_off, c_mult, c_shift, act, thr, val, x_layout, y_channels_last, 0);
 }
 
 extern "C" void thhip_conv2d_u8(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,

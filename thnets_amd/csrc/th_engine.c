@@ -87,16 +87,25 @@ static void *out_resize(struct module *m, int dtype, int nd, const long *size)
 	for (int i = 0; i < nd; i++)
 		n *= size[i];
 	size_t bytes = (size_t)n * esize_of(dtype);
-	if (!o->storage || o->storage->mustfree != TH_MUSTFREE_HIP || hm->cap < bytes || !hm->owns_output) {
+	/* uint8 tensors are followed by a few codes of 0.0 as a convolution output
+	 * has it (range / 2 * 255 / range rounds to 128): the convolution kernel that
+	 * loads straight into LDS fetches its padding from there */
+	const size_t tail = dtype == THHIP_U8 ? TH_U8_TAIL : 0;
+	if (!o->storage || o->storage->mustfree != TH_MUSTFREE_HIP || hm->cap < bytes + tail || !hm->owns_output) {
 		THFloatStorage *s = malloc(sizeof(*s));
-		s->data = thhip_malloc(bytes);
+		s->data = thhip_malloc(bytes + tail);
 		s->nref = 1;
 		s->mustfree = TH_MUSTFREE_HIP;
 		if (o->storage)
 			thhip_storage_release(o->storage);
 		o->storage = s;
-		hm->cap = bytes;
+		hm->cap = bytes + tail;
 		hm->owns_output = 1;
+		hm->tail_at = (size_t)-1;
+	}
+	if (tail && hm->tail_at != bytes) {
+		thhip_memset((char *)o->storage->data + bytes, TH_U8_TAIL_CODE, tail);
+		hm->tail_at = bytes;
 	}
 	o->storageOffset = 0;
 	o->nDimension = nd;
@@ -579,9 +588,12 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 		thhip_linear_batched_u8(x, hm->wrow_u8, hm->rowsum_u8, hm->addend, y, s.B, K, c->nOutputPlane,
 			a_off, b_off, offset, mult, shift, hm->fused_act, thr, val);
 	else
-		thhip_conv2d_u8_layout(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+		/* a planned channels-last input is an output of this engine: it has the tail */
+		thhip_conv2d_u8_layout_tail(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
 			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
-			hm->fused_act, thr, val, x_cl, hm->out_cl);
+			hm->fused_act, thr, val, x_cl, hm->out_cl,
+			x_cl == 1 && zero == TH_U8_TAIL_CODE && in->storage && in->storage->mustfree == TH_MUSTFREE_HIP &&
+			in->storageOffset == 0 ? TH_U8_TAIL : 0);
 	hn->cur_cl = hm->out_cl;
 	hn->cur_mult = om;
 	hn->cur_sub = osub;

@@ -6,6 +6,10 @@
 
 /* Per-module state the engine keeps beside `struct module` (index-parallel to
  * network.modules), so that the public structure keeps the reference layout. */
+/* uint8 outputs: bytes of the code of 0.0 (128 for every convolution output) kept after the tensor */
+#define TH_U8_TAIL 64
+#define TH_U8_TAIL_CODE 128
+
 struct hipmod {
 	int fused_act;		/* the following Threshold is applied in this module's epilogue */
 	float thr, val;
@@ -13,6 +17,7 @@ struct hipmod {
 	int is_linear;		/* MT_Linear in the source network */
 	int owns_output;	/* output storage was allocated by this module */
 	size_t cap;		/* bytes allocated for the output */
+	size_t tail_at;		/* uint8: offset at which the padding-code tail was last written */
 	void *wpacked;		/* convolution weights in the kernel's packed layout (device) */
 	void *wrow;		/* the same weights row-major, made on first matrix-vector use (device) */
 	float *bias;		/* fp32 bias (device) */
