@@ -71,6 +71,31 @@ def test_conv_f32_ktile_depths_tap_major_and_split(hiplib, oracle):
             hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
+def test_conv_f32_loaded_straight_into_lds(hiplib, oracle):
+    """The fp32 kernel whose operands go from global memory straight to LDS (plane-major
+    tensors, planes in blocks of 32): K-tile counts 1..13 around the edges of its
+    three-stage pipeline, partial tiles on both axes, strides, padding, the folded
+    batch-norm factor and the fused threshold, every tile shape."""
+    from thnets_amd import api
+    g = cases.rng(913)
+    shapes = [(2, 32, 9, 10, 70, 1, 1, 0), (1, 64, 7, 7, 130, 1, 2, 0), (1, 96, 6, 5, 64, 1, 1, 0), (2, 32, 12, 11, 36, 2, 1, 1),
+              (1, 160, 5, 5, 40, 1, 1, 0), (1, 192, 6, 6, 72, 1, 1, 0), (1, 224, 4, 7, 33, 1, 1, 0), (2, 32, 23, 17, 300, 3, 1, 1),
+              (1, 96, 7, 7, 130, 3, 2, 1), (3, 64, 14, 14, 96, 3, 1, 1), (1, 416, 4, 4, 64, 1, 1, 0), (1, 64, 20, 20, 64, 5, 1, 2)]
+    try:
+        for (B, Ci, H, W, Co, k, dd, pp) in shapes:
+            x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+            w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+            b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            want = np.maximum(oracle.conv2d(x, w, b, (dd, dd), (pp, pp)), 0)
+            for tune in ((64, 64, 9, 0), (128, 64, 9, 0), (64, 128, 9, 0), (128, 128, 9, 0)):
+                G.note("fp32 straight to LDS %s tile %s" % ((B, Ci, H, W, Co, k, dd, pp), tune))
+                hiplib.thhip_conv_set_tuning(*tune)
+                got = G.conv2d(hiplib, x, w, b, (dd, dd), (pp, pp), act=1, thr=0.0, val=0.0)
+                G.assert_close(got, want, FP32_TOL, str((Ci, Co, k, tune)))
+    finally:
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+
+
 @pytest.mark.parametrize("dtype", [G.F16, G.BF16])
 @pytest.mark.parametrize("i", [0, 1, 3, 5, 10])
 def test_conv_half_vs_fp32_oracle(hiplib, oracle, i, dtype):

@@ -893,7 +893,7 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 template <int N, bool LGKM0>
 __device__ __forceinline__ void wide_wait()
 {
-	static_assert(N >= 0 && N <= 24, "add the count below");
+	static_assert(N >= 0 && N <= 48, "add the count below");
 #define WIDE_WAIT_CASE(n)                                                          \
 	if constexpr (N == n) {                                                    \
 		if constexpr (LGKM0)                                               \
@@ -901,11 +901,55 @@ __device__ __forceinline__ void wide_wait()
 		else                                                               \
 			__builtin_amdgcn_s_waitcnt(WIDE_VMCNT(n));                 \
 	}
-	WIDE_WAIT_CASE(0) WIDE_WAIT_CASE(1) WIDE_WAIT_CASE(2) WIDE_WAIT_CASE(3) WIDE_WAIT_CASE(4)
-	WIDE_WAIT_CASE(5) WIDE_WAIT_CASE(6) WIDE_WAIT_CASE(7) WIDE_WAIT_CASE(8) WIDE_WAIT_CASE(9)
-	WIDE_WAIT_CASE(10) WIDE_WAIT_CASE(11) WIDE_WAIT_CASE(12) WIDE_WAIT_CASE(13) WIDE_WAIT_CASE(14)
-	WIDE_WAIT_CASE(15) WIDE_WAIT_CASE(16) WIDE_WAIT_CASE(17) WIDE_WAIT_CASE(18) WIDE_WAIT_CASE(19)
-	WIDE_WAIT_CASE(20) WIDE_WAIT_CASE(21) WIDE_WAIT_CASE(22) WIDE_WAIT_CASE(23) WIDE_WAIT_CASE(24)
+	WIDE_WAIT_CASE(0)
+	WIDE_WAIT_CASE(1)
+	WIDE_WAIT_CASE(2)
+	WIDE_WAIT_CASE(3)
+	WIDE_WAIT_CASE(4)
+	WIDE_WAIT_CASE(5)
+	WIDE_WAIT_CASE(6)
+	WIDE_WAIT_CASE(7)
+	WIDE_WAIT_CASE(8)
+	WIDE_WAIT_CASE(9)
+	WIDE_WAIT_CASE(10)
+	WIDE_WAIT_CASE(11)
+	WIDE_WAIT_CASE(12)
+	WIDE_WAIT_CASE(13)
+	WIDE_WAIT_CASE(14)
+	WIDE_WAIT_CASE(15)
+	WIDE_WAIT_CASE(16)
+	WIDE_WAIT_CASE(17)
+	WIDE_WAIT_CASE(18)
+	WIDE_WAIT_CASE(19)
+	WIDE_WAIT_CASE(20)
+	WIDE_WAIT_CASE(21)
+	WIDE_WAIT_CASE(22)
+	WIDE_WAIT_CASE(23)
+	WIDE_WAIT_CASE(24)
+	WIDE_WAIT_CASE(25)
+	WIDE_WAIT_CASE(26)
+	WIDE_WAIT_CASE(27)
+	WIDE_WAIT_CASE(28)
+	WIDE_WAIT_CASE(29)
+	WIDE_WAIT_CASE(30)
+	WIDE_WAIT_CASE(31)
+	WIDE_WAIT_CASE(32)
+	WIDE_WAIT_CASE(33)
+	WIDE_WAIT_CASE(34)
+	WIDE_WAIT_CASE(35)
+	WIDE_WAIT_CASE(36)
+	WIDE_WAIT_CASE(37)
+	WIDE_WAIT_CASE(38)
+	WIDE_WAIT_CASE(39)
+	WIDE_WAIT_CASE(40)
+	WIDE_WAIT_CASE(41)
+	WIDE_WAIT_CASE(42)
+	WIDE_WAIT_CASE(43)
+	WIDE_WAIT_CASE(44)
+	WIDE_WAIT_CASE(45)
+	WIDE_WAIT_CASE(46)
+	WIDE_WAIT_CASE(47)
+	WIDE_WAIT_CASE(48)
 #undef WIDE_WAIT_CASE
 }
 
@@ -1501,6 +1545,259 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 }
 
 /* ------------------------------------------------------------------ */
+/* fp32, plane-major: operands straight into LDS                       */
+/* ------------------------------------------------------------------ */
+
+/* The pipeline of conv_wide_kernel for the fp32 path (plane-major tensors as
+ * the reference has them, tap-major K order: a K-tile is one filter tap x 32
+ * planes).  The packed weights are copied in 1 KiB blocks as there.  Of the
+ * input a wave-wide 4-byte load fetches one K value for 64 neighbouring
+ * positions (coalesced along the output row; what lies outside the image is
+ * pointed past the buffer's range and arrives as 0.0) and lands as one row of
+ * the stage's B tile, [k][position].  A 32x32x2 MFMA takes B[k][n] from lane
+ * (n, k): step s of a chunk reads rows 8 c + s (lanes 0..31) and 8 c + 4 + s
+ * (lanes 32..63); rows are BN + 8 floats apart, so the two halves use different
+ * banks.  Needs Ci % 32 == 0. */
+template <int BM, int BN, int NST>
+__global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
+	constexpr int KCH = 4, CHUNK = 8, KT = KCH * CHUNK, WAVES = 4, WGM = 2, WGN = 2;
+	constexpr int MB = BM / 32, TM = BM / WGM / 32, TN = BN / WGN / 32;
+	constexpr int BROW = BN + 8;				/* floats between B rows */
+	constexpr int A_VECS = MB * KCH * 64, B_VECS = KT * BROW / 4, STAGE_VECS = A_VECS + B_VECS;
+	constexpr int A_PW = MB * KCH / WAVES;			/* 1 KiB weight blocks per wave and K-tile */
+	constexpr int NPOS = BN / 64;				/* positions per lane */
+	constexpr int B_PW = KT / WAVES * NPOS;			/* 256-byte input rows per wave and K-tile */
+	constexpr int LOADS = A_PW + B_PW;
+	static_assert(MB * KCH % WAVES == 0 && BN % 64 == 0 && NST >= 3 && NST <= 4 && (NST - 1) * LOADS <= 48, "tile shape");
+	static_assert(2 * BM * sizeof(int) <= NST * STAGE_VECS * sizeof(floatx4), "the epilogue's row constants fit");
+	__shared__ floatx4 lds[NST * STAGE_VECS];
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wm = wave % WGM, wn = wave / WGM;
+
+	int tile_m, tile_n;
+	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
+		const int bid = blockIdx.x;
+		const int xcd = bid & 7;
+		const int local = bid >> 3;
+		const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
+		const int m0 = p.tiles_m * mp / p.mparts, m1 = p.tiles_m * (mp + 1) / p.mparts;
+		const int n0 = p.tiles_n * np / nparts, n1 = p.tiles_n * (np + 1) / nparts;
+		const int mw = m1 - m0;
+		if (local >= mw * (n1 - n0))
+			return;
+		tile_m = m0 + local % mw;
+		tile_n = n0 + local / mw;
+	}
+
+	/* ---- this lane's positions: lane + 64 q of the tile ---- */
+	bool n_ok_[NPOS];
+	int iy0_[NPOS], ix0_[NPOS], xoff_[NPOS];
+#pragma unroll
+	for (int q = 0; q < NPOS; q++) {
+		const int n_glob = tile_n * BN + q * 64 + lane;
+		n_ok_[q] = n_glob < p.N;
+		const int nn = n_ok_[q] ? n_glob : 0;
+		const int b = nn / p.oHW, r = nn - b * p.oHW;
+		const int oy = r / p.oW, ox = r - oy * p.oW;
+		iy0_[q] = oy * p.dH - p.padH;
+		ix0_[q] = ox * p.dW - p.padW;
+		xoff_[q] = b * p.Ci * p.HW + iy0_[q] * p.W + ix0_[q];
+	}
+	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
+	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
+	unsigned a_off_[A_PW];
+	int a_lds_[A_PW];
+#pragma unroll
+	for (int i = 0; i < A_PW; i++) {
+		const int idx = wave + WAVES * i, mbi = idx % MB, kci = idx / MB;
+		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
+		a_lds_[i] = (kci * MB + mbi) * 64;
+	}
+	/* K-tiles: plane block outer, tap inner */
+	int t_cb = 0, t_kh = 0, t_kw = 0, t_kc = 0;
+	const int plane_bytes = p.HW * (int)sizeof(float);
+
+	auto issue = [&](auto st_) {
+		constexpr int st = decltype(st_)::value;
+		floatx4 *la = lds + st * STAGE_VECS;
+		float *lb = (float *)(la + A_VECS);
+#pragma unroll
+		for (int i = 0; i < A_PW; i++)
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(la + a_lds_[i]), 16, lane * 16,
+				a_off_[i] + (unsigned)t_kc * 1024u, 0, 0);
+		const int tap_off = t_kh * p.W + t_kw;
+		const int plane0 = t_cb * KT;
+#pragma unroll
+		for (int q = 0; q < NPOS; q++) {
+			const int iy = iy0_[q] + t_kh, ix = ix0_[q] + t_kw;
+			const bool ok = n_ok_[q] && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			const unsigned voff = ok ? (unsigned)(xoff_[q] + tap_off) * (unsigned)sizeof(float) : 0x80000000u;
+#pragma unroll
+			for (int r = 0; r < KT / WAVES; r++) {
+				const int k = wave + WAVES * r;	/* row of the K-tile */
+				/* the scalar offset is not range checked: the planes exist */
+				__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(lb + k * BROW + q * 64), 4, voff,
+					(plane0 + k) * plane_bytes, 0, 0);
+			}
+		}
+		t_kc += KCH;
+		if (++t_kw == p.kW) {
+			t_kw = 0;
+			if (++t_kh == p.kH) {
+				t_kh = 0;
+				++t_cb;
+			}
+		}
+	};
+
+	floatx4 af[2][TM], bf[2][TN];
+	auto read_frags = [&](auto st_, int kci, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
+		constexpr int st = decltype(st_)::value;
+		const floatx4 *la = lds + st * STAGE_VECS;
+		const float *lb = (const float *)(la + A_VECS);
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+			a[i] = la[(kci * MB + wm * TM + i) * 64 + lane];
+		const float *row = lb + (kci * CHUNK + (lane >> 5) * 4) * BROW + (lane & 31);
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+#pragma unroll
+			for (int e = 0; e < 4; e++)
+				b[j][e] = row[e * BROW + (wn * TN + j) * 32];
+	};
+
+	floatx16 acc[TM][TN];
+#pragma unroll
+	for (int i = 0; i < TM; i++)
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[i][j][r] = 0;
+	auto mma = [&](int set) {
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+				conv_mma<THHIP_F32>(acc[i][j], af[set][i], bf[set][j]);
+	};
+
+	typedef std::integral_constant<int, 0> S0;
+	typedef std::integral_constant<int, 1> S1;
+	typedef std::integral_constant<int, 2> S2;
+	typedef std::integral_constant<int, NST >= 4 ? 3 : 0> S3;
+	const int nkt = p.KC / KCH;
+	issue(S0{});
+	if (1 < nkt)
+		issue(S1{});
+	if (2 < nkt)
+		issue(S2{});
+	if constexpr (NST >= 4) {
+		if (3 < nkt)
+			issue(S3{});
+	}
+	if (NST - 1 < nkt)
+		wide_wait<(NST - 1) * LOADS, false>();
+	else
+		wide_wait<0, false>();
+	__builtin_amdgcn_s_barrier();
+	read_frags(S0{}, 0, af[0], bf[0]);
+	/* as in conv_wide_kernel: one barrier per K-tile, before its last chunk */
+	auto step = [&](int kt, auto st, auto st1, auto steady_) {
+		constexpr bool steady = decltype(steady_)::value;
+#pragma unroll
+		for (int c = 0; c + 1 < KCH; c++) {
+			read_frags(st, c + 1, af[(c + 1) & 1], bf[(c + 1) & 1]);
+			mma(c & 1);
+		}
+		if (steady)
+			wide_wait<(NST - 2) * LOADS, true>();
+		else
+			wide_wait<0, true>();
+		__builtin_amdgcn_s_barrier();
+		if (steady || kt + NST < nkt)
+			issue(st);
+		if (steady || kt + 1 < nkt)
+			read_frags(st1, 0, af[0], bf[0]);
+		mma((KCH - 1) & 1);
+	};
+	auto round = [&](int kt, auto steady_) {
+		if constexpr (NST == 3) {
+			step(kt, S0{}, S1{}, steady_);
+			step(kt + 1, S1{}, S2{}, steady_);
+			step(kt + 2, S2{}, S0{}, steady_);
+		} else {
+			step(kt, S0{}, S1{}, steady_);
+			step(kt + 1, S1{}, S2{}, steady_);
+			step(kt + 2, S2{}, S3{}, steady_);
+			step(kt + 3, S3{}, S0{}, steady_);
+		}
+	};
+	int kt = 0;
+	for (; kt + 2 * NST - 1 < nkt; kt += NST)
+		round(kt, std::true_type{});
+	for (; kt + NST - 1 < nkt; kt += NST)
+		round(kt, std::false_type{});
+	if (kt < nkt) {
+		step(kt, S0{}, S1{}, std::false_type{});
+		if (kt + 1 < nkt)
+			step(kt + 1, S1{}, S2{}, std::false_type{});
+		if constexpr (NST >= 4) {
+			if (kt + 2 < nkt)
+				step(kt + 2, S2{}, S3{}, std::false_type{});
+		}
+	}
+
+	/* ---- epilogue: (folded batch norm factor,) bias, optional threshold, store (plane-major) ---- */
+	float *y = (float *)p.y;
+	int *lrow = (int *)lds;
+	__syncthreads();
+	if (tid < BM) {
+		const int mc = min(tile_m * BM + tid, p.Co - 1);
+		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+		if (p.scale)
+			lrow[BM + tid] = __float_as_int(p.scale[mc]);
+	}
+	__syncthreads();
+	const bool has_scale = p.scale != 0;
+#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
+		if (n >= p.N)
+			continue;
+		const int b = n / p.oHW, rem = n - b * p.oHW;
+		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+			for (int g = 0; g < 4; g++) {
+				const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
+				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+				floatx4 rowscale = { 1, 1, 1, 1 };
+				if (has_scale)
+					rowscale = *(const floatx4 *)(lrow + BM + ml);
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int r = 4 * g + e, m = m0 + 8 * g + e;
+					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
+					if (p.act)
+						v = v > p.thr ? v : p.val;
+					if (m < p.Co)
+						y[ybase + (size_t)m * p.oHW] = v;
+				}
+			}
+		}
+	}
+#endif
+}
+
+/* ------------------------------------------------------------------ */
 /* host side                                                           */
 /* ------------------------------------------------------------------ */
 
@@ -1863,6 +2160,38 @@ static void conv_launch_wide(ConvParams &p)
 		THError("thhip_conv2d: no such tile loaded straight into LDS for this type");
 }
 
+/* Whether conv_f32_direct_kernel can run this layer: plane-major fp32 on both
+ * sides, whole blocks of 32 planes, 32-bit byte offsets. */
+static bool conv_f32_direct_ok(const ConvParams &p)
+{
+	return !p.x_cl && !p.y_cl && p.Ci % 32 == 0 && p.x_bytes < 0x7fffffffu;
+}
+
+template <int BM, int BN, int NST>
+static void conv_launch_f32_direct(ConvParams &p)
+{
+	p.tiles_m = (p.Co + BM - 1) / BM;
+	p.tiles_n = (p.N + BN - 1) / BN;
+	p.splitk = 1;
+	if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
+		THError("thhip_conv2d: packed weights shorter than the tile grid");
+	const double wbytes = (double)p.Co * p.K * 4;
+	p.mparts = 1;
+	while (p.mparts < 8 && p.mparts * 2 <= p.tiles_m && wbytes / p.mparts > 2.5e6)
+		p.mparts *= 2;
+	if (g_force_mparts)
+		p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
+	size_t maxcnt = 0;
+	for (int x = 0; x < 8; x++) {
+		const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
+		const size_t cnt = (size_t)(p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
+			(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
+		if (cnt > maxcnt)
+			maxcnt = cnt;
+	}
+	conv_f32_direct_kernel<BM, BN, NST><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
+}
+
 /* Whether conv_patch_kernel can run this layer. */
 template <int DT>
 static bool conv_patch_ok(const ConvParams &p)
@@ -1975,6 +2304,11 @@ static void conv_dispatch(ConvParams &p)
 				bn = 128;
 		} else if (p.x_cl == 1 && t128 >= 512)
 			bm = bn = 128;
+	} else if (DT == THHIP_F32 && conv_f32_direct_ok(p) && t64 > 128 && !g_force_kch) {
+		/* planes in blocks of 32: operands straight into LDS, 64x64 tiles
+		 * (measured 2-7 % over the register-staged kernel on every VGG layer,
+		 * random data; larger tiles are slower) */
+		direct = true;
 	} else if (DT == THHIP_F32 && t128 >= 300) {
 		kch = 2;
 		if (p.Co > 64 && t128 >= 700)
@@ -2013,6 +2347,21 @@ static void conv_dispatch(ConvParams &p)
 		if (!conv_patch_ok<DT>(p))
 			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64 or 128 planes, 3x3, stride 1");
 		return conv_launch_patch<DT, 64>(p);
+	}
+	if constexpr (DT == THHIP_F32) {
+		if (direct) {
+			if (!conv_f32_direct_ok(p))
+				THError("thhip_conv2d: fp32 tiles loaded straight into LDS need plane-major tensors and Ci %% 32 == 0");
+			if (bm == 64 && bn == 64)
+				return conv_launch_f32_direct<64, 64, 3>(p);
+			if (bm == 128 && bn == 64)
+				return conv_launch_f32_direct<128, 64, 3>(p);
+			if (bm == 64 && bn == 128)
+				return conv_launch_f32_direct<64, 128, 3>(p);
+			if (bm == 128 && bn == 128)
+				return conv_launch_f32_direct<128, 128, 3>(p);
+			THError("thhip_conv2d: no %dx%d tile", bm, bn);
+		}
 	}
 	/* tiles whose operands are loaded straight into LDS (the tuning hook asks for
 	 * them with 9 as its split-K argument, or with a 256-position tile) */
