@@ -75,7 +75,7 @@ def test_conv_f32_loaded_straight_into_lds(hiplib, oracle):
     """The fp32 kernel whose operands go from global memory straight to LDS (plane-major
     tensors, planes in blocks of 32): K-tile counts 1..13 around the edges of its
     three-stage pipeline, partial tiles on both axes, strides, padding, the folded
-    batch-norm factor and the fused threshold, every tile shape."""
+    batch-norm factor and the fused threshold, both tile shapes and K-tile depths."""
     from thnets_amd import api
     g = cases.rng(913)
     shapes = [(2, 32, 9, 10, 70, 1, 1, 0), (1, 64, 7, 7, 130, 1, 2, 0), (1, 96, 6, 5, 64, 1, 1, 0), (2, 32, 12, 11, 36, 2, 1, 1),
@@ -87,7 +87,7 @@ def test_conv_f32_loaded_straight_into_lds(hiplib, oracle):
             w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
             b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
             want = np.maximum(oracle.conv2d(x, w, b, (dd, dd), (pp, pp)), 0)
-            for tune in ((64, 64, 9, 0), (128, 64, 9, 0), (64, 128, 9, 0), (128, 128, 9, 0)):
+            for tune in ((64, 64, 9, 0), (128, 64, 9, 0), (64, 64, 9, 2), (128, 64, 9, 2)):     # K-tiles of 32, of 16
                 G.note("fp32 straight to LDS %s tile %s" % ((B, Ci, H, W, Co, k, dd, pp), tune))
                 hiplib.thhip_conv_set_tuning(*tune)
                 got = G.conv2d(hiplib, x, w, b, (dd, dd), (pp, pp), act=1, thr=0.0, val=0.0)

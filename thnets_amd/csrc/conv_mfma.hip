@@ -1558,11 +1558,12 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
  * (n, k): step s of a chunk reads rows 8 c + s (lanes 0..31) and 8 c + 4 + s
  * (lanes 32..63); rows are BN + 8 floats apart, so the two halves use different
  * banks.  Needs Ci % 32 == 0. */
-template <int BM, int BN, int NST>
+template <int BM, int BN, int KCH, int NST>
 __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
-	constexpr int KCH = 4, CHUNK = 8, KT = KCH * CHUNK, WAVES = 4, WGM = 2, WGN = 2;
+	constexpr int CHUNK = 8, KT = KCH * CHUNK, SUB = 4 / KCH, WAVES = 4, WGM = 2, WGN = 2;
+	static_assert(KCH == 2 || KCH == 4, "the packed blocks of 32 planes are walked in one or two K-tiles");
 	constexpr int MB = BM / 32, TM = BM / WGM / 32, TN = BN / WGN / 32;
 	constexpr int BROW = BN + 8;				/* floats between B rows */
 	constexpr int A_VECS = MB * KCH * 64, B_VECS = KT * BROW / 4, STAGE_VECS = A_VECS + B_VECS;
@@ -1619,7 +1620,7 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		a_lds_[i] = (kci * MB + mbi) * 64;
 	}
 	/* K-tiles: plane block outer, tap inner */
-	int t_cb = 0, t_kh = 0, t_kw = 0, t_kc = 0;
+	int t_cb = 0, t_kh = 0, t_kw = 0, t_kc = 0, t_sub = 0;
 	const int plane_bytes = p.HW * (int)sizeof(float);
 
 	auto issue = [&](auto st_) {
@@ -1631,7 +1632,7 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(la + a_lds_[i]), 16, lane * 16,
 				a_off_[i] + (unsigned)t_kc * 1024u, 0, 0);
 		const int tap_off = t_kh * p.W + t_kw;
-		const int plane0 = t_cb * KT;
+		const int plane0 = (t_cb * SUB + t_sub) * KT;
 #pragma unroll
 		for (int q = 0; q < NPOS; q++) {
 			const int iy = iy0_[q] + t_kh, ix = ix0_[q] + t_kw;
@@ -1646,11 +1647,14 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 			}
 		}
 		t_kc += KCH;
-		if (++t_kw == p.kW) {
-			t_kw = 0;
-			if (++t_kh == p.kH) {
-				t_kh = 0;
-				++t_cb;
+		if (++t_sub == SUB) {	/* the next planes of the block first, then the next tap */
+			t_sub = 0;
+			if (++t_kw == p.kW) {
+				t_kw = 0;
+				if (++t_kh == p.kH) {
+					t_kh = 0;
+					++t_cb;
+				}
 			}
 		}
 	};
@@ -2167,7 +2171,7 @@ static bool conv_f32_direct_ok(const ConvParams &p)
 	return !p.x_cl && !p.y_cl && p.Ci % 32 == 0 && p.x_bytes < 0x7fffffffu;
 }
 
-template <int BM, int BN, int NST>
+template <int BM, int BN, int KCH, int NST>
 static void conv_launch_f32_direct(ConvParams &p)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
@@ -2189,7 +2193,7 @@ static void conv_launch_f32_direct(ConvParams &p)
 		if (cnt > maxcnt)
 			maxcnt = cnt;
 	}
-	conv_f32_direct_kernel<BM, BN, NST><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
+	conv_f32_direct_kernel<BM, BN, KCH, NST><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
 /* Whether conv_patch_kernel can run this layer. */
@@ -2307,8 +2311,15 @@ static void conv_dispatch(ConvParams &p)
 	} else if (DT == THHIP_F32 && conv_f32_direct_ok(p) && t64 > 128 && !g_force_kch) {
 		/* planes in blocks of 32: operands straight into LDS, 64x64 tiles
 		 * (measured 2-7 % over the register-staged kernel on every VGG layer,
-		 * random data; larger tiles are slower) */
+		 * random data; 64x128 and 128x128 tiles are slower).  Layers of many
+		 * tiles take K-tiles of 16 (1-3 %), and 128x64 tiles when that is one
+		 * tile of planes (128->128 @112^2 batch 16: 584 -> 569 us). */
 		direct = true;
+		if (t64 >= 2000) {
+			kch = 2;
+			if (p.Co == 128)
+				bm = 128;
+		}
 	} else if (DT == THHIP_F32 && t128 >= 300) {
 		kch = 2;
 		if (p.Co > 64 && t128 >= 700)
@@ -2352,14 +2363,16 @@ static void conv_dispatch(ConvParams &p)
 		if (direct) {
 			if (!conv_f32_direct_ok(p))
 				THError("thhip_conv2d: fp32 tiles loaded straight into LDS need plane-major tensors and Ci %% 32 == 0");
+			/* K-tiles of 16 or 32 values (the tuning hook's last argument, 2, asks for 16) */
+			const bool k16 = g_force_bm ? g_force_wgs == 2 : kch == 2;
+			if (bm == 64 && bn == 64 && k16)
+				return conv_launch_f32_direct<64, 64, 2, 3>(p);
 			if (bm == 64 && bn == 64)
-				return conv_launch_f32_direct<64, 64, 3>(p);
+				return conv_launch_f32_direct<64, 64, 4, 3>(p);
+			if (bm == 128 && bn == 64 && k16)
+				return conv_launch_f32_direct<128, 64, 2, 3>(p);
 			if (bm == 128 && bn == 64)
-				return conv_launch_f32_direct<128, 64, 3>(p);
-			if (bm == 64 && bn == 128)
-				return conv_launch_f32_direct<64, 128, 3>(p);
-			if (bm == 128 && bn == 128)
-				return conv_launch_f32_direct<128, 128, 3>(p);
+				return conv_launch_f32_direct<128, 64, 4, 3>(p);
 			THError("thhip_conv2d: no %dx%d tile", bm, bn);
 		}
 	}
