@@ -28,10 +28,10 @@ from thnets_amd import api, configs  # noqa: E402
 
 PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_TOPS_INT8_MFMA = 5030.0
-# Bytes moved past L2 per conv_mfma_kernel launch in the VGG-16 b16 step (average of the
-# 13), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled against a 256 MiB copy
-# (profiles/conv_mfma_vgg16_fp32_b16_counters.md); algorithmic bytes are 115.9e6.
-CONV_HBM_BYTES_PER_LAUNCH = 152.2e6
+# Bytes moved past L2 per convolution launch in the VGG-16 b16 step (average of the 13), from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled against a 256 MiB copy
+# (profiles/conv_f32_vgg16_fp32_b16_counters.md); algorithmic bytes are 115.9e6.
+CONV_HBM_BYTES_PER_LAUNCH = 152.8e6
 
 
 def profile_get(lib, fam):
@@ -147,7 +147,7 @@ def main():
     achieved = conv_flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4), "traffic": CONV_HBM_BYTES_PER_LAUNCH,
-                "kernel": "conv_mfma_kernel<fp32> (implicit-GEMM convolution, the 13 convolution launches of a step)",
+                "kernel": "conv_f32_direct_kernel (implicit-GEMM convolution, operands loaded straight into LDS; 12 of the 13 convolution launches of a step, the image layer on conv_mfma_kernel<fp32>)",
                 "launches_per_step": conv_n / args.steps, "avg_launch_ms": round(conv_ms / max(conv_n, 1), 5),
                 "flops_per_launch": conv_flops / max(conv_n, 1)}
     extra = {"vgg16_conv_ms_per_step": round(conv_ms / args.steps, 4),
