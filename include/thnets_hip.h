@@ -408,9 +408,19 @@ void thhip_conv2d_layout(const void *x, const void *wpacked, const float *scale,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, int x_layout, int y_channels_last);
 
-/* Tuning override for experiments: force the convolution's workgroup tile
- * (bm x bn in {64,128}), its split-K factor and the number of workgroups
- * allowed to share a CU; 0 leaves a choice automatic. */
+/* Tuning override for tests and experiments: force the convolution's workgroup
+ * tile (bm x bn in {64,128}), its split-K factor and the number of workgroups
+ * allowed to share a CU; 0 leaves a choice automatic.  A forced tile runs on
+ * the kernel that stages its operands through registers, except:
+ *   splitk == 9 asks for the kernels that load their operands straight into
+ *     LDS (no K split there): half types and uint8 with channels-last input,
+ *     tiles 64x64, 128x64, 64x128, 128x128; fp32 plane-major with Ci % 32 == 0,
+ *     tiles 64x64 and 128x64, wgs_per_cu == 2 selecting K-tiles of 16 values;
+ *   bn == 256 (half types): the 256x256 and 128x256 tiles of the same kernel
+ *     (splitk == 4 with bm == 256: K-tiles of 64 values in two stages);
+ *   (64, 1): the half-type kernel for 3x3 stride-1 layers of 64 or 128 planes
+ *     that keeps an input patch in LDS.
+ * A layer the forced kernel cannot take ends in THError. */
 void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);
 /* fp32 only: force K-tiles of 16 values (chunks = 2) or 32 (4); 0 restores the
  * per-layer choice.  Tests and tuning, like thhip_conv_set_tuning. */
