@@ -197,6 +197,30 @@ def test_vgg16_full_size_properties(hiplib, oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("half", [1, 2])
+def test_vgg16_full_size_half_engines(hiplib, oracle, half):
+    """Full-size VGG-16 on the half engines (the kernels that keep an input patch in LDS and
+    the tiles loaded straight into LDS all run at their real shapes): against the fp32
+    engine on the same input, image by image against the batch, and the first block
+    against the oracle."""
+    cfg = configs.vgg16(batch=3)
+    n32 = api.HipNetwork(cfg["layers"])
+    want = n32.process_float(cfg["input"]).reshape(3, -1)
+    n32.free()
+    net = api.HipNetwork(cfg["layers"], half=half)
+    tol = 3e-2 if half == 1 else 1.5e-1
+    y = net.process_float(cfg["input"]).reshape(3, -1)
+    G.assert_close(y, want, tol, "half engine vs fp32 engine")
+    y1 = net.process_float(cfg["input"][1:2]).ravel()
+    G.assert_close(y1, y[1], 1e-2 if half == 1 else 5e-2, "batch vs single image")     # (other tiles, other rounding order)
+    net.upload(cfg["input"][:1])
+    net.forward()
+    ref = oracle.run_layers(cfg["layers"][:5], cfg["input"][:1])
+    G.assert_close(net.module_output(4), ref, 2e-2 if half == 1 else 6e-2, "first block")
+    net.free()
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("name", ["tiny_cnn", "vgg16_small", "resnet18_small", "segnet_small"])
 def test_loaded_model_directory_runs_like_the_layer_list(hiplib, oracle, tmp_path, name):
     """THLoadNetwork -> THCreateHipNetwork -> THProcessFloat on a Torch7 model
