@@ -87,7 +87,8 @@ def test_conv_f32_loaded_straight_into_lds(hiplib, oracle):
             w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
             b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
             want = np.maximum(oracle.conv2d(x, w, b, (dd, dd), (pp, pp)), 0)
-            for tune in ((64, 64, 9, 0), (128, 64, 9, 0), (64, 64, 9, 2), (128, 64, 9, 2)):     # K-tiles of 32, of 16
+            # K-tiles of 32, of 16; then K split in 2, 3 and 7 parts (last argument / 10), more parts than K-tiles included
+            for tune in ((64, 64, 9, 0), (128, 64, 9, 0), (64, 64, 9, 2), (128, 64, 9, 2), (64, 64, 9, 20), (128, 64, 9, 32), (64, 64, 9, 70)):
                 G.note("fp32 straight to LDS %s tile %s" % ((B, Ci, H, W, Co, k, dd, pp), tune))
                 hiplib.thhip_conv_set_tuning(*tune)
                 got = G.conv2d(hiplib, x, w, b, (dd, dd), (pp, pp), act=1, thr=0.0, val=0.0)

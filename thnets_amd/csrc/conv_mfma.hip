@@ -1580,11 +1580,15 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wm = wave % WGM, wn = wave / WGM;
 
-	int tile_m, tile_n;
+	int tile_m, tile_n, split = 0;
 	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
 		const int bid = blockIdx.x;
 		const int xcd = bid & 7;
-		const int local = bid >> 3;
+		int local = bid >> 3;
+		if (p.splitk > 1) {	/* the parts of a tile are neighbours in the order */
+			split = local % p.splitk;
+			local /= p.splitk;
+		}
 		const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
 		const int m0 = p.tiles_m * mp / p.mparts, m1 = p.tiles_m * (mp + 1) / p.mparts;
 		const int n0 = p.tiles_n * np / nparts, n1 = p.tiles_n * (np + 1) / nparts;
@@ -1619,8 +1623,20 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
 		a_lds_[i] = (kci * MB + mbi) * 64;
 	}
-	/* K-tiles: plane block outer, tap inner */
-	int t_cb = 0, t_kh = 0, t_kw = 0, t_kc = 0, t_sub = 0;
+	/* K-tiles: plane block outer, tap inner; with a K split this workgroup walks
+	 * the K-tiles [kt0, kt0 + nkt) */
+	const int nkt_all = p.KC / KCH;
+	const int kt0 = p.splitk > 1 ? (int)((long)nkt_all * split / p.splitk) : 0;
+	const int nkt = (p.splitk > 1 ? (int)((long)nkt_all * (split + 1) / p.splitk) : nkt_all) - kt0;
+	int t_cb, t_kh, t_kw, t_kc = kt0 * KCH, t_sub;
+	{
+		const int blk = kt0 / SUB;
+		t_sub = kt0 - blk * SUB;
+		t_cb = blk / p.kHW;
+		const int tap = blk - t_cb * p.kHW;
+		t_kh = tap / p.kW;
+		t_kw = tap - t_kh * p.kW;
+	}
 	const int plane_bytes = p.HW * (int)sizeof(float);
 
 	auto issue = [&](auto st_) {
@@ -1695,7 +1711,6 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 	typedef std::integral_constant<int, 1> S1;
 	typedef std::integral_constant<int, 2> S2;
 	typedef std::integral_constant<int, NST >= 4 ? 3 : 0> S3;
-	const int nkt = p.KC / KCH;
 	issue(S0{});
 	if (1 < nkt)
 		issue(S1{});
@@ -1757,6 +1772,28 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		}
 	}
 
+	if (p.splitk > 1) {
+		/* this part's sums as they are, [part][plane][position]; a finishing kernel
+		 * adds the parts in a fixed order (the result does not depend on timing) */
+		float *part = (float *)p.ws + (size_t)split * p.Co * p.N;
+#pragma unroll
+		for (int j = 0; j < TN; j++) {
+			const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
+			if (n >= p.N)
+				continue;
+#pragma unroll
+			for (int i = 0; i < TM; i++) {
+				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					const int m = m0 + 8 * (r >> 2) + (r & 3);
+					if (m < p.Co)
+						part[(size_t)m * p.N + n] = acc[i][j][r];
+				}
+			}
+		}
+		return;
+	}
 	/* ---- epilogue: (folded batch norm factor,) bias, optional threshold, store (plane-major) ---- */
 	float *y = (float *)p.y;
 	int *lrow = (int *)lds;
@@ -1799,6 +1836,27 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		}
 	}
 #endif
+}
+
+/* Sums the parts of a K split, [part][plane][position] fp32, in their order and
+ * finishes as the convolution epilogue does; plane-major output. */
+__global__ void conv_f32_splitk_finish_kernel(const float *ws, const float *bias, const float *scale, float *y,
+	int parts, int Co, int N, int oHW, int act, float thr, float val)
+{
+	const long total = (long)Co * N;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total; i += step) {
+		const int m = (int)(i / N), n = (int)(i - (long)m * N);
+		float v = 0;
+		for (int s = 0; s < parts; s++)
+			v += ws[(size_t)s * total + i];
+		v = scale ? v * scale[m] + (bias ? bias[m] : 0.0f) : v + (bias ? bias[m] : 0.0f);
+		if (act)
+			v = v > thr ? v : val;
+		const int b = n / oHW, rem = n - b * oHW;
+		y[((size_t)b * Co + m) * oHW + rem] = v;
+	}
 }
 
 /* ------------------------------------------------------------------ */
@@ -2172,11 +2230,24 @@ static bool conv_f32_direct_ok(const ConvParams &p)
 }
 
 template <int BM, int BN, int KCH, int NST>
-static void conv_launch_f32_direct(ConvParams &p)
+static void conv_launch_f32_direct(ConvParams &p, int splitk)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
 	p.tiles_n = (p.N + BN - 1) / BN;
-	p.splitk = 1;
+	const int nkt = p.KC / KCH;
+	if (splitk > nkt)
+		splitk = nkt;
+	p.splitk = splitk < 1 ? 1 : splitk;
+	if (p.splitk > 1) {
+		const size_t need = (size_t)p.splitk * p.Co * p.N * sizeof(float);
+		if (need > g_ws_bytes) {
+			hipcheck(hipStreamSynchronize(thhip_stream()));
+			thhip_free(g_ws);
+			g_ws = (int *)thhip_malloc(need);
+			g_ws_bytes = need;
+		}
+		p.ws = g_ws;
+	}
 	if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
 		THError("thhip_conv2d: packed weights shorter than the tile grid");
 	const double wbytes = (double)p.Co * p.K * 4;
@@ -2193,7 +2264,14 @@ static void conv_launch_f32_direct(ConvParams &p)
 		if (cnt > maxcnt)
 			maxcnt = cnt;
 	}
-	conv_f32_direct_kernel<BM, BN, KCH, NST><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
+	conv_f32_direct_kernel<BM, BN, KCH, NST><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
+	if (p.splitk > 1) {
+		long blocks = ((long)p.Co * p.N + 255) / 256;
+		if (blocks > 4096)
+			blocks = 4096;
+		conv_f32_splitk_finish_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
+			(float *)p.y, p.splitk, p.Co, p.N, p.oHW, p.act, p.thr, p.val);
+	}
 }
 
 /* Whether conv_patch_kernel can run this layer. */
@@ -2308,7 +2386,7 @@ static void conv_dispatch(ConvParams &p)
 				bn = 128;
 		} else if (p.x_cl == 1 && t128 >= 512)
 			bm = bn = 128;
-	} else if (DT == THHIP_F32 && conv_f32_direct_ok(p) && t64 > 128 && !g_force_kch) {
+	} else if (DT == THHIP_F32 && conv_f32_direct_ok(p) && !g_force_kch) {
 		/* planes in blocks of 32: operands straight into LDS, 64x64 tiles
 		 * (measured 2-7 % over the register-staged kernel on every VGG layer,
 		 * random data; 64x128 and 128x128 tiles are slower).  Layers of many
@@ -2319,6 +2397,22 @@ static void conv_dispatch(ConvParams &p)
 			kch = 2;
 			if (p.Co == 128)
 				bm = 128;
+		} else if (t64 <= 512) {
+			/* Few tiles of a long K (a 32x32 MFMA tile over K = 4608 is most of a
+			 * SIMD's fair share of a 392-tile layer): split K, about 1024
+			 * workgroups, at least eight K-tiles each; the parts go to scratch and
+			 * a small kernel adds them in order.  Measured: 512->512 @14^2 batch 16
+			 * 181 -> 161 us (3 parts), @7^2 batch 32 108 -> 96 us; AlexNet batch 1,
+			 * against the other kernel's in-kernel split: conv2 32 -> 15, conv3
+			 * 25 -> 14, conv4 27 -> 16, conv5 31 -> 15 us. */
+			const int nkt = p.KC / kch;
+			int parts = (int)((1024 + t64 - 1) / t64);
+			if (parts > nkt / 8)
+				parts = nkt / 8;
+			if (parts > 16)
+				parts = 16;
+			if (parts > 1)
+				splitk = parts;
 		}
 	} else if (DT == THHIP_F32 && t128 >= 300) {
 		kch = 2;
@@ -2364,15 +2458,17 @@ static void conv_dispatch(ConvParams &p)
 			if (!conv_f32_direct_ok(p))
 				THError("thhip_conv2d: fp32 tiles loaded straight into LDS need plane-major tensors and Ci %% 32 == 0");
 			/* K-tiles of 16 or 32 values (the tuning hook's last argument, 2, asks for 16) */
-			const bool k16 = g_force_bm ? g_force_wgs == 2 : kch == 2;
+			const bool k16 = g_force_bm ? g_force_wgs % 10 == 2 : kch == 2;
+			/* (forced tuning: the last argument / 10 is the K split) */
+			const int dsplit = g_force_bm ? g_force_wgs / 10 : splitk;
 			if (bm == 64 && bn == 64 && k16)
-				return conv_launch_f32_direct<64, 64, 2, 3>(p);
+				return conv_launch_f32_direct<64, 64, 2, 3>(p, dsplit);
 			if (bm == 64 && bn == 64)
-				return conv_launch_f32_direct<64, 64, 4, 3>(p);
+				return conv_launch_f32_direct<64, 64, 4, 3>(p, dsplit);
 			if (bm == 128 && bn == 64 && k16)
-				return conv_launch_f32_direct<128, 64, 2, 3>(p);
+				return conv_launch_f32_direct<128, 64, 2, 3>(p, dsplit);
 			if (bm == 128 && bn == 64)
-				return conv_launch_f32_direct<128, 64, 4, 3>(p);
+				return conv_launch_f32_direct<128, 64, 4, 3>(p, dsplit);
 			THError("thhip_conv2d: no %dx%d tile", bm, bn);
 		}
 	}
