@@ -408,6 +408,20 @@ void thhip_conv2d_layout(const void *x, const void *wpacked, const float *scale,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, int x_layout, int y_channels_last);
 
+/* thhip_conv2d_layout followed by a 2x2 / stride 2 max pooling without padding
+ * (floor mode) in one kernel: y is [B][Co][oH/2][oW/2] (or channels-last), the
+ * Threshold applied before the pooling as the modules run.  Replaces the module
+ * sequence SpatialConvolutionMM -> Threshold -> SpatialMaxPooling
+ * (modules/SpatialMaxPooling.c:6-98 after SpatialConvolutionMM.c:111-225) for the
+ * layers thhip_conv2d_pool2_supported accepts: half types, channels-last input
+ * of 64 or 128 planes, 3x3, stride 1, enough tiles for the kernel that keeps an
+ * input patch in LDS. */
+int thhip_conv2d_pool2_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int dtype, int x_layout, int y_channels_last);
+void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype, int x_layout, int y_channels_last);
+
 /* Tuning override for tests and experiments: force the convolution's workgroup
  * tile (bm x bn in {64,128}), its split-K factor and the number of workgroups
  * allowed to share a CU; 0 leaves a choice automatic.  A forced tile runs on

@@ -50,6 +50,7 @@ struct ConvParams {
 	int mparts;		/* the tile grid is cut mparts x (8 / mparts) over the XCDs */
 	unsigned x_bytes;
 	unsigned w_bytes;	/* packed weights (the wide kernel's buffer descriptor) */
+	int pool;		/* half types, conv_patch_kernel: the 2x2 / stride 2 max pooling that follows is done in the epilogue */
 	unsigned x_tail;	/* uint8: bytes of the padding code that follow x (0: none) */
 	/* split-K: S workgroups share an output tile, each over a K range */
 	int splitk;
@@ -1327,7 +1328,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 #define PATCH_TW 32
 #define PATCH_TH 8
 
-template <int DT, bool CLO, int BM, int CI>
+template <int DT, bool CLO, int BM, int CI, bool POOL>
 __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
@@ -1503,6 +1504,52 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	}
 	__syncthreads();
 	const bool has_scale = p.scale != 0;
+	if constexpr (POOL) {
+		/* The 2x2 / stride 2 max pooling that follows, here: the two rows of a
+		 * window are this wave's two tile rows (the same accumulator index), its
+		 * two columns neighbouring lanes.  Threshold first, as the modules run. */
+		const int pH = p.oH / 2, pW = p.oW / 2;
+		const int py = ty * (TH / 2) + wave, px = tx * (TW / 2) + ((lane & 31) >> 1);
+		const bool store = !(lane & 1) && py < pH && px < pW;
+		const size_t n = ((size_t)img * pH + py) * pW + px;
+		const size_t ybase = (size_t)img * p.Co * pH * pW + (size_t)py * pW + px;
+#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			const int m0 = tile_m * BM + i * 32 + 4 * (lane >> 5);
+#pragma unroll
+			for (int g = 0; g < 4; g++) {
+				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+				const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
+				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+				floatx4 rowscale = { 1, 1, 1, 1 };
+				if (has_scale)
+					rowscale = *(const floatx4 *)(lrow + BM + ml);
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int r = 4 * g + e, m = m0 + 8 * g + e;
+					float v0 = has_scale ? acc[i][0][r] * rowscale[e] + rowbias[e] : acc[i][0][r] + rowbias[e];
+					float v1 = has_scale ? acc[i][1][r] * rowscale[e] + rowbias[e] : acc[i][1][r] + rowbias[e];
+					if (p.act) {
+						v0 = v0 > p.thr ? v0 : p.val;
+						v1 = v1 > p.thr ? v1 : p.val;
+					}
+					/* the pooling compares the stored (rounded) values */
+					float v = fmaxf((float)(elem)v0, (float)(elem)v1);
+					v = fmaxf(v, __shfl_xor(v, 1));
+					if constexpr (!CLO) {
+						if (store && m < p.Co)
+							y[ybase + (size_t)m * pH * pW] = (elem)v;
+					}
+					quad.v[e] = (elem)v;
+				}
+				if constexpr (CLO) {
+					if (store && m0 + 8 * g < p.Co)
+						*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
+				}
+			}
+		}
+		return;
+	}
 #pragma unroll
 	for (int j = 0; j < TN; j++) {
 		const int oy = ty * TH + 2 * wave + j, ox = tx * TW + (lane & 31);
@@ -2295,14 +2342,22 @@ static void conv_launch_patch(ConvParams &p)
 			THError("thhip_conv2d: packed weights shorter than the tile grid");
 		const long total = (long)p.tiles_m * p.tiles_n;
 		dim3 grid((unsigned)(8 * ((total + 7) / 8)));
+#define CONV_PATCH_GO(CLO, CI)                                                                               \
+	do {                                                                                                \
+		if (p.pool)                                                                                 \
+			conv_patch_kernel<DT, CLO, BM, CI, true><<<grid, dim3(256), 0, thhip_stream()>>>(p);  \
+		else                                                                                        \
+			conv_patch_kernel<DT, CLO, BM, CI, false><<<grid, dim3(256), 0, thhip_stream()>>>(p); \
+	} while (0)
 		if (p.Ci == 64 && p.y_cl)
-			conv_patch_kernel<DT, true, BM, 64><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+			CONV_PATCH_GO(true, 64);
 		else if (p.Ci == 64)
-			conv_patch_kernel<DT, false, BM, 64><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+			CONV_PATCH_GO(false, 64);
 		else if (p.y_cl)
-			conv_patch_kernel<DT, true, BM, 128><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+			CONV_PATCH_GO(true, 128);
 		else
-			conv_patch_kernel<DT, false, BM, 128><<<grid, dim3(256), 0, thhip_stream()>>>(p);
+			CONV_PATCH_GO(false, 128);
+#undef CONV_PATCH_GO
 	} else
 		THError("thhip_conv2d: the patch kernel is for the half types");
 }
@@ -2448,6 +2503,8 @@ static void conv_dispatch(ConvParams &p)
 		wgs = g_force_wgs;
 	if (DT == THHIP_F32 && g_force_kch)
 		kch = g_force_kch;
+	if (p.pool)
+		bm = 64, bn = 1;	/* only the patch kernel pools */
 	if (bn == 1) {	/* (64, 1): the patch kernel */
 		if (!conv_patch_ok<DT>(p))
 			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64 or 128 planes, 3x3, stride 1");
@@ -2584,7 +2641,7 @@ static unsigned char *conv_pixels4_scratch(size_t bytes)
 
 static void conv_run(const void *x, const void *wpacked, const float *scale, const float *bias, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
-	int act, float thr, float val, int dtype, const ConvU8Args *u8, int f_x_layout = 0, int f_y_cl = 0)
+	int act, float thr, float val, int dtype, const ConvU8Args *u8, int f_x_layout = 0, int f_y_cl = 0, int f_pool2 = 0)
 {
 	if (B < 1 || Ci < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
 		THError("thhip_conv2d: bad geometry");
@@ -2600,7 +2657,7 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 	/* 32-bit offsets inside the kernel: run the batch in slices whose input
 	 * and output stay below 2^31 bytes. */
 	const int xl = u8 ? u8->x_cl : f_x_layout;
-	const long in_img = (long)Ci * H * W, out_img = (long)Co * oH * oW;
+	const long in_img = (long)Ci * H * W, out_img = f_pool2 ? (long)Co * (oH / 2) * (oW / 2) : (long)Co * oH * oW;
 	const long in_eff = xl == 2 ? 4L * H * W : in_img;	/* bytes the kernel addresses per image */
 	long bmax = ((1L << 31) - 64) / (esize * (in_eff > out_img ? in_eff : out_img));
 	if (bmax < 1)
@@ -2677,6 +2734,7 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 		} else {
 			p.x_cl = xl;
 			p.y_cl = f_y_cl;
+			p.pool = f_pool2;
 			ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N);
 			THHIP_DISPATCH_FLOAT(dtype, conv_dispatch<DT>(p));
 		}
@@ -2702,6 +2760,44 @@ extern "C" void thhip_conv2d_layout(const void *x, const void *wpacked, const fl
 		THError("thhip_conv2d: unsupported dtype %d", dtype);
 	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0,
 		x_layout, y_channels_last != 0);
+}
+
+/* Whether thhip_conv2d_layout_pool2 takes this layer (and is the kernel the
+ * layer would run on anyway): half type, channels-last input of 64 or 128
+ * planes, 3x3, stride 1, enough tiles. */
+extern "C" int thhip_conv2d_pool2_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int dtype, int x_layout, int y_channels_last)
+{
+	if (dtype != THHIP_F16 && dtype != THHIP_BF16)
+		return 0;
+	if (x_layout != 1 || (Ci != 64 && Ci != 128) || kH != 3 || kW != 3 || dH != 1 || dW != 1 || padH < 0 || padW < 0)
+		return 0;
+	if (y_channels_last && Co % 4)
+		return 0;
+	const int oW = W + 2 * padW - 2, oH = H + 2 * padH - 2;
+	if (oW < 2 || oH < 2)
+		return 0;
+	if ((double)B * Ci * H * W * 2 >= 2147483000.0 || (double)B * Co * oH * oW * 2 >= 2147483000.0)
+		return 0;	/* (the batch would be cut into slices) */
+	const long tpatch = (long)((Co + 63) / 64) * B * ((oW + PATCH_TW - 1) / PATCH_TW) * ((oH + PATCH_TH - 1) / PATCH_TH);
+	const long t256 = (long)((Co + 255) / 256) * (((long)B * oH * oW + 255) / 256);
+	const bool wide256 = Ci % 32 == 0 && Co % 256 == 0 && t256 > 128;
+	return tpatch >= 128 && !(wide256 && Ci > 64) && !g_force_generic_cl && !g_force_bm && !g_force_bn;
+}
+
+/* thhip_conv2d_layout followed by a 2x2 / stride 2 max pooling without padding
+ * (floor mode), in one kernel: y is [B][Co][oH/2][oW/2] (or channels-last).  For
+ * layers thhip_conv2d_pool2_supported accepts.  Replaces the module sequence
+ * SpatialConvolutionMM -> Threshold -> SpatialMaxPooling
+ * (modules/SpatialMaxPooling.c:6-98) for those layers. */
+extern "C" void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype, int x_layout, int y_channels_last)
+{
+	if (!thhip_conv2d_pool2_supported(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, dtype, x_layout, y_channels_last))
+		THError("thhip_conv2d_layout_pool2: layer not supported (see thhip_conv2d_pool2_supported)");
+	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0,
+		x_layout, y_channels_last != 0, 1);
 }
 
 extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,

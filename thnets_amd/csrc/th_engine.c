@@ -175,13 +175,25 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 		THError("Given input size: (%dx%dx%d). Calculated output size: (%dx%dx%d). Output size is too small",
 			c->nInputPlane, s.H, s.W, c->nOutputPlane, oH, oW);
 	const void *x = thhip_tensor_ptr(in, dt);
-	void *y = conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
 	const int K = c->nInputPlane * c->kH * c->kW;
 	/* the weights were packed for the planned memory order of the input; with
 	 * one pixel per plane both orders coincide */
 	if (s.H * s.W > 1 && hn->cur_cl != hm->in_cl)
 		THError("HIP engine: a convolution planned for %s input got the other memory order",
 			hm->in_cl ? "channels-last" : "plane-major");
+	/* conv -> (Threshold) -> 2x2 max pooling in one kernel, where the kernel that
+	 * would run this layer can do it */
+	if (hm->pool_next && thhip_conv2d_pool2_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW,
+			c->dH, c->dW, c->padH, c->padW, dt, hm->x_layout, hm->out_cl)) {
+		void *yp = conv_out(m, dt, &s, c->nOutputPlane, oH / 2, oW / 2);
+		hn->cur_cl = hm->out_cl && (oH / 2) * (oW / 2) > 1;
+		thhip_conv2d_layout_pool2(x, hm->wpacked, hm->scale, hm->bias, yp, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, hm->fused_act, hm->thr, hm->val, dt, hm->x_layout,
+			hm->out_cl);
+		hn->hm[hm->pool_next].pooled_by_producer = 1;
+		return m->output;
+	}
+	void *y = conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
 	hn->cur_cl = hm->out_cl && oH * oW > 1;
 	/* the row-major copy is made from plane-major packing; for a 1x1 kernel the
 	 * channels-last packing is the same (k is the plane in both) */
@@ -256,6 +268,11 @@ static THFloatTensor *Hip_SpatialMaxPooling_updateOutput(struct module *m, THFlo
 {
 	struct hipnet *hn = hipnet_of(m);
 	struct SpatialMaxPooling *q = &m->SpatialMaxPooling;
+	if (hipmod_of(m)->pooled_by_producer) {	/* done in the convolution's epilogue */
+		hipmod_of(m)->pooled_by_producer = 0;
+		out_alias(m, in);
+		return m->output;
+	}
 	struct planes p = planes_of(in, "SpatialMaxPooling");
 	int oH, oW;
 	q->iwidth = p.W;
@@ -1148,6 +1165,21 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 		}
 	}
 	plan_channels_last(hn, net);
+	/* half engines: a 2x2 / stride 2 max pooling right after a convolution (and its
+	 * folded Threshold) between channels-last tensors may be done by the
+	 * convolution's epilogue; whether it is, is decided per forward by the layer's shape */
+	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIP && dtype != THHIP_F32; i++) {
+		if (!is_conv_type(hn->pub.modules[i].type) || hn->hm[i].is_linear || !hn->hm[i].in_cl)
+			continue;
+		int j = i + 1;
+		while (j < net->nelem && hn->hm[j].passthrough)
+			j++;
+		if (j >= net->nelem || hn->pub.modules[j].type != MT_SpatialMaxPooling || hn->hm[j].want_indices)
+			continue;
+		const struct SpatialMaxPooling *q = &hn->pub.modules[j].SpatialMaxPooling;
+		if (q->kW == 2 && q->kH == 2 && q->dW == 2 && q->dH == 2 && q->padW == 0 && q->padH == 0 && !q->ceil_mode)
+			hn->hm[i].pool_next = j;
+	}
 	return &hn->pub;
 }
 

@@ -14,6 +14,8 @@ struct hipmod {
 	int fused_act;		/* the following Threshold is applied in this module's epilogue */
 	float thr, val;
 	int passthrough;	/* a Threshold whose work was folded into its producer */
+	int pool_next;		/* convolution: index of a 2x2 / stride 2 max pooling its epilogue may do (0: none) */
+	int pooled_by_producer;	/* max pooling: the convolution before it did the pooling in this forward */
 	int is_linear;		/* MT_Linear in the source network */
 	int owns_output;	/* output storage was allocated by this module */
 	size_t cap;		/* bytes allocated for the output */
