@@ -237,7 +237,10 @@ class Oracle:
         """x: float32 array, 4-D [B,C,H,W] or as produced by earlier layers.  Returns
         the output; ``collect`` (a list) receives every top-level module output."""
         kept = {}       # position of a maxpool -> (indices, input height, input width), for maxunpool
+        outs = []       # every output, for layers that name their inputs (thapi.c:173-193)
         for pos, spec in enumerate(layers):
+            if spec.get("inputs"):
+                x = outs[spec["inputs"][0]] if len(spec["inputs"]) == 1 else [outs[j] for j in spec["inputs"]]
             if spec["type"] == "maxpool":
                 h, w = x.shape[-2:]
                 x4 = x if x.ndim == 4 else x[None]
@@ -252,6 +255,7 @@ class Oracle:
                 x = y if x.ndim == 4 else y[0]
             else:
                 x = self._run_one(spec, x)
+            outs.append(x)
             if collect is not None:
                 collect.append(x if not isinstance(x, list) else [v.copy() for v in x])
         return x

@@ -8,7 +8,7 @@ import pytest
 
 import cases
 import gpu_util as G
-from thnets_amd import api, configs
+from thnets_amd import api, netbuild, configs
 
 pytestmark = pytest.mark.gpu
 
@@ -193,6 +193,48 @@ def test_vgg16_full_size_properties(hiplib, oracle):
     net.forward()
     want = oracle.run_layers(cfg["layers"][:5], cfg["input"][:1])
     G.assert_close(net.module_output(4), want, 2e-5, "first block")
+    net.free()
+
+
+@pytest.mark.gpu
+def test_graph_form_networks(hiplib, oracle):
+    """Modules that name their inputs (ninputs / inputs[], thapi.c:173-193): the residual
+    network as a flat graph gives bit for bit what its ConcatTable / CAddTable form gives,
+    with the batch norms folded and not; a module is folded into its producer only when it
+    is the producer's sole consumer."""
+    cfg = cases.small_networks()["resnet18_small"]
+    graph = configs.to_graph(cfg["layers"])
+    assert any(len(s["inputs"]) == 2 for s in graph) and all(s["type"] != "concattable" for s in graph)
+    want = oracle.run_layers(cfg["layers"], oracle.normalize(cfg["input"], cfg["mean"], cfg["std"]))
+    for fold in (1, 0):
+        hiplib.THHipFoldBatchNorm(fold)
+        try:
+            nt = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+            ng = api.HipNetwork(graph, cfg["mean"], cfg["std"])
+            yt, yg = nt.process_float(cfg["input"]), ng.process_float(cfg["input"])
+            assert np.array_equal(yt, yg), "graph form differs from table form (fold %d)" % fold
+            G.assert_close(yg, want.ravel(), 1e-3, "graph form vs oracle")
+            nt.free()
+            ng.free()
+        finally:
+            hiplib.THHipFoldBatchNorm(1)
+    # half engine: a graph stays plane-major
+    ng = api.HipNetwork(graph, cfg["mean"], cfg["std"], half=1)
+    G.assert_close(ng.process_float(cfg["input"]), want.ravel(), 4e-2, "graph form, fp16")
+    ng.free()
+    # a convolution read by two modules: its Threshold must not be folded into it
+    g = cases.rng(1700)
+    w0 = g.standard_normal((8, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+    w1 = g.standard_normal((8, 8, 3, 3), dtype=np.float32) * np.float32(0.2)
+    b = lambda: g.standard_normal(8, dtype=np.float32) * np.float32(0.1)
+    layers = [dict(netbuild.conv(w0, b(), 1, 1), inputs=[]),
+              dict(netbuild.relu(inplace=0), inputs=[0]),
+              dict(netbuild.conv(w1, b(), 1, 1), inputs=[0]),       # reads the convolution's raw output
+              {"type": "caddtable", "inputs": [1, 2]},
+              dict(netbuild.relu(), inputs=[3])]
+    x = g.uniform(-1, 1, (2, 3, 9, 7)).astype(np.float32)
+    net = api.HipNetwork(layers)
+    G.assert_close(net.process_float(x.copy()), oracle.run_layers(layers, x).ravel(), 1e-4, "two consumers")
     net.free()
 
 

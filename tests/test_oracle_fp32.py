@@ -289,3 +289,19 @@ def test_rgb2float_closed_form(oracle):
         want = (src.transpose(2, 0, 1).astype(np.float32) * np.float32(0.003921568) -
                 np.asarray(mean, np.float32)[:, None, None]) * (np.float32(1) / np.asarray(std, np.float32))[:, None, None]
         assert np.array_equal(y, want.astype(np.float32))
+
+
+def test_graph_form_equals_table_form(oracle):
+    """Layers that name their inputs (the reference's executor for graph formats,
+    thapi.c:173-193): laying a ConcatTable / CAddTable network out as a flat graph changes
+    nothing, bit for bit, and every named input must come earlier in the list."""
+    from thnets_amd import configs, netbuild
+    cfg = cases.small_networks()["resnet18_small"]
+    x = oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])
+    graph = configs.to_graph(cfg["layers"])
+    assert np.array_equal(oracle.run_layers(graph, x), oracle.run_layers(cfg["layers"], x))
+    # an identity branch disappears: such an add reads the main branch and, earlier in the list, the block input
+    adds = [s for s in graph if s["type"] == "caddtable"]
+    assert adds and all(len(s["inputs"]) == 2 for s in adds) and any(s["inputs"][0] > s["inputs"][1] for s in adds)
+    for i, s in enumerate(graph):
+        assert all(0 <= j < i for j in s["inputs"])

@@ -139,6 +139,32 @@ def resnet18(seed=4, batch=32, scale=1.0, side=224):
             "mean": (0, 0, 0), "std": (1, 1, 1)}
 
 
+def to_graph(layers):
+    """The same network as a flat list whose layers name their inputs ("inputs": positions
+    in the list), the form the reference's graph loaders produce and its executor routes by
+    (thapi.c:173-193): ConcatTable branches are laid out one after the other, an identity
+    branch disappears (the table add reads the block's input directly), the table add names
+    the branch ends."""
+    out, prev, ends = [], None, None
+    for spec in layers:
+        if spec["type"] == "concattable":
+            ends = []
+            for branch in spec["branches"]:
+                p = prev
+                if not (len(branch) == 1 and branch[0]["type"] == "dropout"):
+                    for s in branch:
+                        out.append(dict(s, inputs=[p] if p is not None else []))
+                        p = len(out) - 1
+                ends.append(p)
+            continue
+        if spec["type"] in ("caddtable", "csubtable"):
+            out.append(dict(spec, inputs=list(ends)))
+        else:
+            out.append(dict(spec, inputs=[prev] if prev is not None else []))
+        prev = len(out) - 1
+    return out
+
+
 def alexnet_lowp(seed=2, batch=64):
     """Configuration 5: the AlexNet-OWT weights in THMakeSpatial form, to be run
     through the uint8 engine with range 32.  No SoftMax: bit-exactness is asserted on

@@ -737,7 +737,32 @@ static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
 			thhip_sync();
 			t = seconds_now();
 		}
-		in = m->updateOutput(m, in);
+		/* A module that names its inputs (the loaders of graph formats fill
+		 * ninputs / inputs[]: thapi.c:173-193) takes them from the modules it
+		 * names, which come earlier in the list; several inputs are handed over
+		 * as a table, the way ConcatTable does it.  Without named inputs the
+		 * network is sequential. */
+		if (m->ninputs == 1 && m->type != MT_JoinTable) {
+			if (m->inputs[0] < 0 || m->inputs[0] >= i)
+				THError("module %d names input %d, which has not run yet", i + 1, m->inputs[0] + 1);
+			in = m->updateOutput(m, net->modules[m->inputs[0]].output);
+		} else if (m->ninputs >= 1) {
+			struct module srcs[MAXMODULEINPUTS], table;
+			struct network subnet;
+			if (m->ninputs > MAXMODULEINPUTS)
+				THError("module %d: too many inputs", i + 1);
+			for (int j = 0; j < m->ninputs; j++) {
+				if (m->inputs[j] < 0 || m->inputs[j] >= i)
+					THError("module %d names input %d, which has not run yet", i + 1, m->inputs[j] + 1);
+				srcs[j].output = net->modules[m->inputs[j]].output;
+			}
+			subnet.nelem = m->ninputs;
+			subnet.modules = srcs;
+			subnet.engine = net->engine;
+			table.ConcatTable.net = &subnet;
+			in = m->updateOutput(m, (THFloatTensor *)&table);
+		} else
+			in = m->updateOutput(m, in);
 		if (th_profile) {
 			thhip_sync();
 			t = seconds_now() - t;
@@ -1034,7 +1059,9 @@ static void plan_channels_last(struct hipnet *hn, struct network *src)
 	int prev = -1;
 	if (!lowp && hn->dtype == THHIP_F32)
 		return;		/* fp32 gathers element-wise at full speed; it stays plane-major */
-	for (int i = 0; i < hn->pub.nelem; i++) {
+	/* (a graph keeps every tensor plane-major: the chains below assume that a
+	 * module reads what the module before it wrote) */
+	for (int i = 0; i < hn->pub.nelem && !hn->dag; i++) {
 		struct module *m = &hn->pub.modules[i];
 		struct hipmod *hm = &hn->hm[i];
 		if (is_conv_type(m->type)) {
@@ -1111,12 +1138,29 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 	hn->range = range;
 	for (int i = 0; i < net->nelem; i++)
 		convert_module(hn, net, i, engine, dtype, range);
+	/* Modules that name their inputs make the list a graph: a module may then be
+	 * folded into its producer only if it is that producer's sole consumer. */
+	int dag = 0;
+	int *consumers = calloc(net->nelem ? net->nelem : 1, sizeof(int));
+	for (int i = 0; i < net->nelem; i++) {
+		if (net->modules[i].ninputs > 0)
+			dag = 1;
+		for (int j = 0; j < net->modules[i].ninputs && j < MAXMODULEINPUTS; j++)
+			if (net->modules[i].inputs[j] >= 0 && net->modules[i].inputs[j] < net->nelem)
+				consumers[net->modules[i].inputs[j]]++;
+	}
+	hn->dag = dag;
+#define FEEDS_ONLY(a, b) (!dag ? (b) == (a) + 1 : (net->modules[b].ninputs == 1 && net->modules[b].inputs[0] == (a) && consumers[a] == 1))
+	if (dag && engine == ENGINE_HIPLOWP)
+		for (int i = 1; i < net->nelem; i++)
+			if (net->modules[i].ninputs > 1 || (net->modules[i].ninputs == 1 && net->modules[i].inputs[0] != i - 1))
+				THError("the uint8 engine runs sequential networks only (module %d names other inputs)", i + 1);
 	/* fold a SpatialBatchNormalization into the convolution that feeds it:
 	 * ((sum + cb - mean) * invstd) * w + b  =  sum * s + ((cb - mean) * s + b),  s = invstd * w
 	 * (SpatialBatchNormalization.c:57-116; the reference's loader-side folding is absorb_bn, onnx.cc:529-557) */
 	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIP && g_fold_bn; i++) {
 		struct module *m = &hn->pub.modules[i], *sb = &net->modules[i + 1];
-		if (!is_conv_type(m->type) || hn->hm[i].is_linear || sb->type != MT_SpatialBatchNormalization)
+		if (!is_conv_type(m->type) || hn->hm[i].is_linear || sb->type != MT_SpatialBatchNormalization || !FEEDS_ONLY(i, i + 1))
 			continue;
 		struct SpatialBatchNormalization *bn = &sb->SpatialBatchNormalization;
 		const int Co = m->SpatialConvolution.nOutputPlane;
@@ -1146,8 +1190,13 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 	for (int i = 0; i + 1 < net->nelem; i++) {
 		struct module *m = &hn->pub.modules[i];
 		int ti = i + 1;
-		if (hn->hm[ti].passthrough && hn->pub.modules[ti].type == MT_SpatialBatchNormalization && ti + 1 < net->nelem)
+		if (!FEEDS_ONLY(i, i + 1))
+			continue;
+		if (hn->hm[ti].passthrough && hn->pub.modules[ti].type == MT_SpatialBatchNormalization && ti + 1 < net->nelem) {
 			ti++;	/* conv -> (folded BN) -> Threshold */
+			if (!FEEDS_ONLY(i + 1, i + 2))
+				continue;
+		}
 		struct module *t = &hn->pub.modules[ti];
 		if (!foldable_threshold(t))
 			continue;
@@ -1164,6 +1213,8 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			hn->hm[i + 1].passthrough = 1;
 		}
 	}
+#undef FEEDS_ONLY
+	free(consumers);
 	plan_channels_last(hn, net);
 	/* half engines: a 2x2 / stride 2 max pooling right after a convolution (and its
 	 * folded Threshold) between channels-last tensors may be done by the

@@ -52,6 +52,7 @@ struct hipnet {
 	float range;
 	float cur_mult, cur_sub;	/* uint8 engine: quantisation of the tensor in flight */
 	int cur_cl;		/* uint8 engine: the tensor in flight is channels-last in memory */
+	int dag;		/* modules name their inputs (ninputs / inputs[]): the list is a graph */
 };
 
 struct hipnet *hipnet_of(struct module *m);

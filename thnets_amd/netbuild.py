@@ -121,6 +121,14 @@ class HostNetwork:
             m.updateOutput = self._fn(kind)
             m.output = self._new_lib_tensor()
             m.net = pnet
+            # graph form (thapi.c:173-193): "inputs" lists the positions, in this list, of the
+            # modules whose outputs this one reads
+            inputs = spec.get("inputs", [])
+            m.ninputs = len(inputs)
+            for j, src in enumerate(inputs):
+                if not 0 <= src < i:
+                    raise ValueError("layer %d names input %d, which does not come before it" % (i, src))
+                m.inputs[j] = src
             if kind == "conv":
                 w = np.asarray(spec["weight"], dtype=np.float32)
                 co, ci, kh, kw = w.shape
