@@ -439,6 +439,13 @@ void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);
 /* fp32 only: force K-tiles of 16 values (chunks = 2) or 32 (4); 0 restores the
  * per-layer choice.  Tests and tuning, like thhip_conv_set_tuning. */
 void thhip_conv_set_ktile(int chunks);
+/* fp32 tiles loaded straight into LDS, layers without a K split of their own:
+ * the tiles an XCD cannot spread evenly over its CUs (its tile count modulo the
+ * workgroups it holds at once) are dispatched last and cut along K into up to
+ * `parts` parts of at least eight K-tiles, summed in their order by a small
+ * kernel (results do not depend on timing).  Default 8; 1 = never cut.  Tests
+ * and tuning. */
+void thhip_conv_set_tail_parts(int parts);
 /* Force how the tile grid is cut over the eight XCDs: the M tiles into
  * mparts (1, 2, 4, 8) groups, the N tiles into 8 / mparts ranges; 0 restores
  * the choice by weight size.  Tests and tuning. */

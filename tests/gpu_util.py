@@ -33,8 +33,9 @@ def conv2d(lib, x, w, bias, d=(1, 1), pad=(0, 0), act=0, thr=0.0, val=0.0, dtype
 
 
 def conv2d_layout(lib, x, w, bias, d=(1, 1), pad=(0, 0), act=0, thr=0.0, val=0.0, dtype=F16, x_cl=0, y_cl=0, scale=None):
-    """Half-type convolution with the device tensors channels-last on either side;
-    x and the result are [B][C][H][W] arrays."""
+    """Convolution with the device tensors channels-last on either side (half types) and
+    an optional per-plane factor applied before the bias; x and the result are
+    [B][C][H][W] arrays."""
     x = np.ascontiguousarray(x, np.float32)
     w = np.ascontiguousarray(w, np.float32)
     B, Ci, H, W = x.shape
@@ -45,7 +46,7 @@ def conv2d_layout(lib, x, w, bias, d=(1, 1), pad=(0, 0), act=0, thr=0.0, val=0.0
     dx = api.to_device_dtype(lib, np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if x_cl else x, dtype)
     db = api.DeviceArray(lib, np.ascontiguousarray(bias, np.float32)) if bias is not None else None
     ds = api.DeviceArray(lib, np.ascontiguousarray(scale, np.float32)) if scale is not None else None
-    dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW * 2)
+    dy = api.DeviceArray(lib, nbytes=B * Co * oH * oW * (4 if dtype == F32 else 2))
     lib.thhip_conv2d_layout(dx.ptr, wp, ds.ptr if ds else None, db.ptr if db else None, dy.ptr, B, Ci, H, W, Co, kH, kW,
                             d[0], d[1], pad[0], pad[1], act, thr, val, dtype, x_cl, y_cl)
     lib.thhip_sync()

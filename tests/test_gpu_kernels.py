@@ -97,6 +97,34 @@ def test_conv_f32_loaded_straight_into_lds(hiplib, oracle):
         hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
+def test_conv_f32_last_tiles_cut_along_k(hiplib, oracle):
+    """fp32 tiles loaded straight into LDS: the tiles an XCD cannot spread evenly over its
+    CUs are cut along K and summed in order by a second kernel.  Layers where every tile
+    is cut (few tiles), where only the last ones are (784 tiles: 98 per XCD), with
+    partial tiles on both axes, the folded batch-norm factor and the threshold; every
+    limit on the parts, 1 = never cut; the same call twice gives the same bits."""
+    g = cases.rng(917)
+    shapes = [(4, 64, 112, 112, 64, 3, 1, 1), (1, 64, 20, 20, 64, 5, 1, 2), (2, 96, 30, 30, 70, 3, 1, 1),
+              (5, 128, 28, 28, 128, 3, 1, 1), (3, 256, 27, 27, 100, 3, 2, 1)]
+    try:
+        for (B, Ci, H, W, Co, k, dd, pp) in shapes:
+            x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+            w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+            b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+            plain = oracle.conv2d(x, w, None, (dd, dd), (pp, pp))
+            want = np.maximum(plain * sc[None, :, None, None] + b[None, :, None, None], 0)
+            for parts in (1, 2, 8, 64):
+                G.note("fp32 last tiles cut along K %s parts %d" % ((B, Ci, H, W, Co, k, dd, pp), parts))
+                hiplib.thhip_conv_set_tail_parts(parts)
+                got = G.conv2d_layout(hiplib, x, w, b, (dd, dd), (pp, pp), act=1, dtype=G.F32, scale=sc)
+                G.assert_close(got, want, FP32_TOL, str((Ci, Co, k, parts)))
+                again = G.conv2d_layout(hiplib, x, w, b, (dd, dd), (pp, pp), act=1, dtype=G.F32, scale=sc)
+                assert np.array_equal(got, again), "cut tiles: results depend on timing"
+    finally:
+        hiplib.thhip_conv_set_tail_parts(8)
+
+
 @pytest.mark.parametrize("dtype", [G.F16, G.BF16])
 @pytest.mark.parametrize("i", [0, 1, 3, 5, 10])
 def test_conv_half_vs_fp32_oracle(hiplib, oracle, i, dtype):

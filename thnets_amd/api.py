@@ -86,6 +86,7 @@ PROTOTYPES = {
     "thhip_maxpool_cl": (None, [vp, vp] + [C.c_int] * 13),
     "thhip_conv2d_affine": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv_set_ktile": (None, [C.c_int]),
+    "thhip_conv_set_tail_parts": (None, [C.c_int]),
     "thhip_maxpool_indices": (None, [vp, vp, vp] + [C.c_int] * 13),
     "thhip_maxunpool": (None, [vp, vp, vp] + [C.c_int] * 13),
     "thhip_fullconv_pack_weight": (vp, [vp] + [C.c_int] * 5),

@@ -56,6 +56,10 @@ struct ConvParams {
 	int splitk;
 	int *ws;		/* [tile][S][BM*BN] partial accumulators (float or int bits) */
 	unsigned *cnt;		/* [tile] arrival counters, zero between launches */
+	/* conv_f32_direct_kernel: K split of the last tiles of every XCD only (0 slots: none) */
+	int tail_slots;		/* workgroups an XCD holds at once */
+	int tail_max;		/* most parts per tile */
+	int tail_cap;		/* scratch blocks reserved per XCD: [xcd][tail_cap][parts][BM*BN] */
 	/* uint8 path only */
 	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
 	const int *addend;	/* per-plane bias addend, or NULL */
@@ -1595,6 +1599,88 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 /* fp32, plane-major: operands straight into LDS                       */
 /* ------------------------------------------------------------------ */
 
+/* XCD x's rectangle of the tile grid (mparts x 8/mparts rectangles): first tile
+ * row, rows, first tile column, and the number of tiles. */
+__device__ inline void conv_xcd_rect(const ConvParams &p, int xcd, int &m0, int &mw, int &n0, int &cnt)
+{
+	const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
+	m0 = p.tiles_m * mp / p.mparts;
+	const int m1 = p.tiles_m * (mp + 1) / p.mparts;
+	n0 = p.tiles_n * np / nparts;
+	const int n1 = p.tiles_n * (np + 1) / nparts;
+	mw = m1 - m0;
+	cnt = mw * (n1 - n0);
+}
+
+/* The tiles an XCD cannot spread evenly: of its cnt tiles the last cnt % slots
+ * would run a few to a CU (or alone) while the other CUs idle.  Those are cut
+ * along K into as many parts as fill the slots once, at most smax; *full is
+ * the number of tiles that stay whole.  Returns the parts (1: no cut). */
+__host__ __device__ inline int conv_tail_parts(int cnt, int slots, int smax, int *full)
+{
+	*full = cnt;
+	if (slots <= 0)
+		return 1;
+	const int f = cnt / slots * slots, rem = cnt - f;
+	if (!rem)
+		return 1;
+	int s = slots / rem;
+	if (s > smax)
+		s = smax;
+	if (s < 2)
+		return 1;
+	*full = f;
+	return s;
+}
+
+/* Epilogue of the fp32 tiles whose accumulators are laid out as in
+ * conv_f32_direct_kernel (2 x 2 waves): (folded batch norm factor,) bias,
+ * optional threshold, plane-major store.  lrow: 2 * BM ints of LDS no wave
+ * still reads. */
+template <int BM, int BN, int TM, int TN>
+__device__ inline void conv_f32_direct_store(const ConvParams &p, floatx16 (&acc)[TM][TN], int tile_m, int tile_n, int *lrow)
+{
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave % 2, wn = wave / 2;
+	float *y = (float *)p.y;
+	if (tid < BM) {
+		const int mc = min(tile_m * BM + tid, p.Co - 1);
+		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+		if (p.scale)
+			lrow[BM + tid] = __float_as_int(p.scale[mc]);
+	}
+	__syncthreads();
+	const bool has_scale = p.scale != 0;
+#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
+		if (n >= p.N)
+			continue;
+		const int b = n / p.oHW, rem = n - b * p.oHW;
+		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+			for (int g = 0; g < 4; g++) {
+				const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
+				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+				floatx4 rowscale = { 1, 1, 1, 1 };
+				if (has_scale)
+					rowscale = *(const floatx4 *)(lrow + BM + ml);
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int r = 4 * g + e, m = m0 + 8 * g + e;
+					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
+					if (p.act)
+						v = v > p.thr ? v : p.val;
+					if (m < p.Co)
+						y[ybase + (size_t)m * p.oHW] = v;
+				}
+			}
+		}
+	}
+}
+
 /* The pipeline of conv_wide_kernel for the fp32 path (plane-major tensors as
  * the reference has them, tap-major K order: a K-tile is one filter tap x 32
  * planes).  The packed weights are copied in 1 KiB blocks as there.  Of the
@@ -1627,7 +1713,8 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wm = wave % WGM, wn = wave / WGM;
 
-	int tile_m, tile_n, split = 0;
+	int tile_m, tile_n, split = 0, nsplit = p.splitk > 1 ? p.splitk : 1;
+	long tail_blk = -1;
 	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
 		const int bid = blockIdx.x;
 		const int xcd = bid & 7;
@@ -1636,11 +1723,20 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 			split = local % p.splitk;
 			local /= p.splitk;
 		}
-		const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
-		const int m0 = p.tiles_m * mp / p.mparts, m1 = p.tiles_m * (mp + 1) / p.mparts;
-		const int n0 = p.tiles_n * np / nparts, n1 = p.tiles_n * (np + 1) / nparts;
-		const int mw = m1 - m0;
-		if (local >= mw * (n1 - n0))
+		int m0, mw, n0, cnt;
+		conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
+		if (p.tail_slots) {	/* the XCD's last tiles, dispatched last, in parts along K */
+			int full;
+			const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, &full);
+			if (s > 1 && local >= full) {
+				const int t = (local - full) / s;
+				split = (local - full) - t * s;
+				nsplit = s;
+				local = full + t;
+				tail_blk = ((long)xcd * p.tail_cap + t) * s + split;
+			}
+		}
+		if (local >= cnt)
 			return;
 		tile_m = m0 + local % mw;
 		tile_n = n0 + local / mw;
@@ -1673,8 +1769,8 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 	/* K-tiles: plane block outer, tap inner; with a K split this workgroup walks
 	 * the K-tiles [kt0, kt0 + nkt) */
 	const int nkt_all = p.KC / KCH;
-	const int kt0 = p.splitk > 1 ? (int)((long)nkt_all * split / p.splitk) : 0;
-	const int nkt = (p.splitk > 1 ? (int)((long)nkt_all * (split + 1) / p.splitk) : nkt_all) - kt0;
+	const int kt0 = nsplit > 1 ? (int)((long)nkt_all * split / nsplit) : 0;
+	const int nkt = (nsplit > 1 ? (int)((long)nkt_all * (split + 1) / nsplit) : nkt_all) - kt0;
 	int t_cb, t_kh, t_kw, t_kc = kt0 * KCH, t_sub;
 	{
 		const int blk = kt0 / SUB;
@@ -1819,6 +1915,20 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		}
 	}
 
+	if (tail_blk >= 0) {
+		/* a part of one of the XCD's last tiles: the accumulators as they lie in
+		 * the registers, [register][thread]; conv_f32_tail_finish_kernel adds the
+		 * parts in their order */
+		float *part = (float *)p.ws + tail_blk * (BM * BN);
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					part[((i * TN + j) * 16 + r) * 256 + tid] = acc[i][j][r];
+		return;
+	}
 	if (p.splitk > 1) {
 		/* this part's sums as they are, [part][plane][position]; a finishing kernel
 		 * adds the parts in a fixed order (the result does not depend on timing) */
@@ -1841,48 +1951,47 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		}
 		return;
 	}
-	/* ---- epilogue: (folded batch norm factor,) bias, optional threshold, store (plane-major) ---- */
-	float *y = (float *)p.y;
-	int *lrow = (int *)lds;
 	__syncthreads();
-	if (tid < BM) {
-		const int mc = min(tile_m * BM + tid, p.Co - 1);
-		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
-		if (p.scale)
-			lrow[BM + tid] = __float_as_int(p.scale[mc]);
-	}
-	__syncthreads();
-	const bool has_scale = p.scale != 0;
-#pragma unroll
-	for (int j = 0; j < TN; j++) {
-		const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
-		if (n >= p.N)
-			continue;
-		const int b = n / p.oHW, rem = n - b * p.oHW;
-		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
-#pragma unroll
-		for (int i = 0; i < TM; i++) {
-			const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
-#pragma unroll
-			for (int g = 0; g < 4; g++) {
-				const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
-				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
-				floatx4 rowscale = { 1, 1, 1, 1 };
-				if (has_scale)
-					rowscale = *(const floatx4 *)(lrow + BM + ml);
-#pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int r = 4 * g + e, m = m0 + 8 * g + e;
-					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
-					if (p.act)
-						v = v > p.thr ? v : p.val;
-					if (m < p.Co)
-						y[ybase + (size_t)m * p.oHW] = v;
-				}
-			}
-		}
-	}
+	conv_f32_direct_store<BM, BN, TM, TN>(p, acc, tile_m, tile_n, (int *)lds);
 #endif
+}
+
+/* Adds the K parts of the tiles conv_f32_direct_kernel cut (one workgroup per
+ * such tile, [xcd][tile][part][register][thread] in scratch) in their order
+ * and finishes them as that kernel's epilogue does. */
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void conv_f32_tail_finish_kernel(ConvParams p)
+{
+	constexpr int TM = BM / 64, TN = BN / 64;
+	__shared__ int lrow[2 * BM];
+	const int tid = threadIdx.x, xcd = blockIdx.x & 7, t = blockIdx.x >> 3;
+	int m0, mw, n0, cnt, full;
+	conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
+	const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, &full);
+	if (s < 2 || t >= cnt - full)
+		return;
+	const int local = full + t;
+	const float *part = (const float *)p.ws + ((long)xcd * p.tail_cap + t) * s * (BM * BN);
+	floatx16 acc[TM][TN];
+	/* part by part, so that the loads of one part are all in flight together */
+#pragma unroll
+	for (int i = 0; i < TM; i++)
+#pragma unroll
+		for (int j = 0; j < TN; j++)
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[i][j][r] = part[((i * TN + j) * 16 + r) * 256 + tid];
+	for (int q = 1; q < s; q++) {
+		part += BM * BN;
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					acc[i][j][r] += part[((i * TN + j) * 16 + r) * 256 + tid];
+	}
+	conv_f32_direct_store<BM, BN, TM, TN>(p, acc, m0 + local % mw, n0 + local / mw, lrow);
 }
 
 /* Sums the parts of a K split, [part][plane][position] fp32, in their order and
@@ -2059,6 +2168,16 @@ extern "C" void thhip_conv_set_xcd_parts(int mparts)
 	if (mparts != 0 && mparts != 1 && mparts != 2 && mparts != 4 && mparts != 8)
 		THError("thhip_conv_set_xcd_parts(%d): 0, 1, 2, 4 or 8", mparts);
 	g_force_mparts = mparts;
+}
+
+/* fp32 tiles loaded straight into LDS: the most K parts for the tiles an XCD
+ * cannot spread evenly over its CUs (1: never cut them). */
+static int g_tail_parts = 8;
+extern "C" void thhip_conv_set_tail_parts(int parts)
+{
+	if (parts < 1 || parts > 64)
+		THError("thhip_conv_set_tail_parts(%d): 1 .. 64", parts);
+	g_tail_parts = parts;
 }
 
 /* fp32 only: force K-tiles of 16 (chunks = 2) or 32 (4); 0 = choose automatically. */
@@ -2276,6 +2395,18 @@ static bool conv_f32_direct_ok(const ConvParams &p)
 	return !p.x_cl && !p.y_cl && p.Ci % 32 == 0 && p.x_bytes < 0x7fffffffu;
 }
 
+/* Points p.ws at scratch of at least that many bytes. */
+static void conv_f32_scratch(ConvParams &p, size_t need)
+{
+	if (need > g_ws_bytes) {
+		hipcheck(hipStreamSynchronize(thhip_stream()));
+		thhip_free(g_ws);
+		g_ws = (int *)thhip_malloc(need);
+		g_ws_bytes = need;
+	}
+	p.ws = g_ws;
+}
+
 template <int BM, int BN, int KCH, int NST>
 static void conv_launch_f32_direct(ConvParams &p, int splitk)
 {
@@ -2285,16 +2416,8 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 	if (splitk > nkt)
 		splitk = nkt;
 	p.splitk = splitk < 1 ? 1 : splitk;
-	if (p.splitk > 1) {
-		const size_t need = (size_t)p.splitk * p.Co * p.N * sizeof(float);
-		if (need > g_ws_bytes) {
-			hipcheck(hipStreamSynchronize(thhip_stream()));
-			thhip_free(g_ws);
-			g_ws = (int *)thhip_malloc(need);
-			g_ws_bytes = need;
-		}
-		p.ws = g_ws;
-	}
+	if (p.splitk > 1)
+		conv_f32_scratch(p, (size_t)p.splitk * p.Co * p.N * sizeof(float));
 	if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
 		THError("thhip_conv2d: packed weights shorter than the tile grid");
 	const double wbytes = (double)p.Co * p.K * 4;
@@ -2311,6 +2434,46 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 		if (cnt > maxcnt)
 			maxcnt = cnt;
 	}
+	/* Without a K split of the whole layer: the tiles an XCD cannot spread evenly
+	 * over its CUs are cut along K (conv_tail_parts), at least eight K-tiles a part. */
+	p.tail_slots = p.tail_max = p.tail_cap = 0;
+	if (p.splitk == 1 && g_tail_parts != 1) {
+		static int resident, cus;
+		if (!resident) {
+			int dev;
+			hipcheck(hipGetDevice(&dev));
+			hipcheck(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+			hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_direct_kernel<BM, BN, KCH, NST>, 256, 0));
+			if (resident < 1)
+				resident = 1;
+		}
+		p.tail_slots = cus / 8 * resident;
+		p.tail_max = nkt / 8 < g_tail_parts ? nkt / 8 : g_tail_parts;
+		if (p.tail_max < 2)
+			p.tail_slots = 0;
+	}
+	int smax = 1;
+	if (p.tail_slots) {
+		maxcnt = 0;
+		for (int x = 0; x < 8; x++) {
+			const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
+			const int cnt = (p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
+				(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
+			int full;
+			const int sx = conv_tail_parts(cnt, p.tail_slots, p.tail_max, &full);
+			if (sx > 1 && cnt - full > p.tail_cap)
+				p.tail_cap = cnt - full;
+			if (sx > smax)
+				smax = sx;
+			const size_t wgs = (size_t)full + (size_t)(cnt - full) * sx;
+			if (wgs > maxcnt)
+				maxcnt = wgs;
+		}
+		if (!p.tail_cap)
+			p.tail_slots = 0;
+		else
+			conv_f32_scratch(p, (size_t)8 * p.tail_cap * smax * BM * BN * sizeof(float));
+	}
 	conv_f32_direct_kernel<BM, BN, KCH, NST><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
 	if (p.splitk > 1) {
 		long blocks = ((long)p.Co * p.N + 255) / 256;
@@ -2319,6 +2482,8 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 		conv_f32_splitk_finish_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
 			(float *)p.y, p.splitk, p.Co, p.N, p.oHW, p.act, p.thr, p.val);
 	}
+	if (p.tail_slots)
+		conv_f32_tail_finish_kernel<BM, BN><<<dim3((unsigned)(8 * p.tail_cap)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
 /* Whether conv_patch_kernel can run this layer. */
