@@ -31,7 +31,7 @@ PEAK_TOPS_INT8_MFMA = 5030.0
 # Bytes moved past L2 per convolution launch in the VGG-16 b16 step (average of the 13), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled against a 256 MiB copy
 # (profiles/conv_f32_vgg16_fp32_b16_counters.md); algorithmic bytes are 115.9e6.
-CONV_HBM_BYTES_PER_LAUNCH = 165.8e6
+CONV_HBM_BYTES_PER_LAUNCH = 175.0e6
 
 
 def profile_get(lib, fam):
@@ -147,7 +147,7 @@ def main():
     achieved = conv_flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4), "traffic": CONV_HBM_BYTES_PER_LAUNCH,
-                "kernel": "conv_f32_direct_kernel (implicit-GEMM convolution, operands loaded straight into LDS; 12 of the 13 convolutions of a step, the three 14x14 layers with their K split and its finishing kernel; the image layer on conv_mfma_kernel<fp32>)",
+                "kernel": "conv_f32_direct_kernel (implicit-GEMM convolution, operands loaded straight into LDS; 12 of the 13 convolutions of a step, with the kernels that sum the K parts of the three 14x14 layers and of the last tiles of eight others; the image layer on conv_mfma_kernel<fp32>)",
                 "launches_per_step": conv_n / args.steps, "avg_launch_ms": round(conv_ms / max(conv_n, 1), 5),
                 "flops_per_launch": conv_flops / max(conv_n, 1)}
     extra = {"vgg16_conv_ms_per_step": round(conv_ms / args.steps, 4),
