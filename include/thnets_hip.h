@@ -361,7 +361,10 @@ void thhip_sync(void);
 void thhip_event_record(int slot);
 float thhip_event_ms(int slot_start, int slot_stop);
 /* Per-kernel-family accumulated time (ms) and launch count measured with
- * events around every launch while profiling is on (family ids below). */
+ * events around every launch while profiling is on (family ids below).
+ * thhip_profile_enable: 0 off, 1 every family, otherwise the sum of
+ * 2 << family over the families to time (an event pair costs a few
+ * microseconds of stream time per launch). */
 enum thhip_family { THHIP_FAM_CONV = 0, THHIP_FAM_GEMV = 1, THHIP_FAM_CONV_I8 = 2, THHIP_FAM_OTHER = 3, THHIP_FAM_COUNT = 4 };
 void thhip_profile_enable(int on);
 void thhip_profile_reset(void);

@@ -156,7 +156,8 @@ static void prof_drain(void)
 
 int thhip_prof_begin(int family)
 {
-	if (!g_prof_on)
+	/* 1: every family; otherwise the sum of 2 << family over the families wanted */
+	if (!g_prof_on || (g_prof_on != 1 && !(g_prof_on & (2 << family))))
 		return -1;
 	if (g_recs.size() >= 4096)
 		prof_drain();
