@@ -430,7 +430,7 @@ void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, const float *
  * allowed to share a CU; 0 leaves a choice automatic.  A forced tile runs on
  * the kernel that stages its operands through registers, except:
  *   splitk == 9 asks for the kernels that load their operands straight into
- *     LDS (no K split there): half types and uint8 with channels-last input,
+ *     LDS (no K split of the whole layer there): half types and uint8 with channels-last input,
  *     tiles 64x64, 128x64, 64x128, 128x128; fp32 plane-major with Ci % 32 == 0,
  *     tiles 64x64 and 128x64, wgs_per_cu == 2 selecting K-tiles of 16 values;
  *   bn == 256 (half types): the 256x256 and 128x256 tiles of the same kernel
@@ -442,9 +442,10 @@ void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);
 /* fp32 only: force K-tiles of 16 values (chunks = 2) or 32 (4); 0 restores the
  * per-layer choice.  Tests and tuning, like thhip_conv_set_tuning. */
 void thhip_conv_set_ktile(int chunks);
-/* fp32 tiles loaded straight into LDS, layers without a K split of their own:
- * the tiles an XCD cannot spread evenly over its CUs (its tile count modulo the
- * workgroups it holds at once) are dispatched last and cut along K into up to
+/* fp32 and half-type tiles loaded straight into LDS, layers without a K split
+ * of their own: the tiles an XCD cannot spread evenly over its CUs (its tile
+ * count modulo the workgroups it holds at once; half types: only after at
+ * least one whole round) are dispatched last and cut along K into up to
  * `parts` parts of at least eight K-tiles, summed in their order by a small
  * kernel (results do not depend on timing).  Default 8; 1 = never cut.  Tests
  * and tuning. */

@@ -126,6 +126,40 @@ def test_conv_f32_last_tiles_cut_along_k(hiplib, oracle):
 
 
 @pytest.mark.parametrize("dtype", [G.F16, G.BF16])
+def test_conv_half_last_tiles_cut_along_k(hiplib, oracle, dtype):
+    """Half-type tiles loaded straight into LDS (channels-last input): the tiles an XCD
+    cannot spread evenly over its CUs are cut along K, as on the fp32 path, where at least
+    one whole round of tiles precedes them.  518 tiles of 128x128 (64 or 65 per XCD, two
+    resident per CU: one tile cut on some XCDs, none on others; 100 of 128 planes), 265
+    tiles of 256x256 (33 per XCD, one per CU), a layer of few tiles (never cut); both
+    output orders, the factor and the threshold, every limit on the parts (1 = never
+    cut), same bits twice."""
+    g = cases.rng(919)
+    shapes = [(8, 64, 91, 91, 100, 3, 1, 1, (128, 128, 9, 0)), (8, 128, 92, 92, 256, 3, 1, 1, (256, 256, 0, 0)),
+              (3, 96, 27, 27, 100, 3, 2, 1, (64, 128, 9, 0))]
+    try:
+        for (B, Ci, H, W, Co, k, dd, pp, tune) in shapes:
+            x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+            w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+            b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+            plain = oracle.conv2d(x, w, None, (dd, dd), (pp, pp))
+            want = np.maximum(plain * sc[None, :, None, None] + b[None, :, None, None], 0)
+            hiplib.thhip_conv_set_tuning(*tune)
+            for y_cl in (1, 0):
+                for parts in (1, 2, 8):
+                    G.note("half last tiles cut along K %s parts %d y_cl %d" % ((B, Ci, H, W, Co, k, dd, pp, tune), parts, y_cl))
+                    hiplib.thhip_conv_set_tail_parts(parts)
+                    got = G.conv2d_layout(hiplib, x, w, b, (dd, dd), (pp, pp), act=1, dtype=dtype, x_cl=1, y_cl=y_cl, scale=sc)
+                    G.assert_close(got, want, HALF_TOL, str((Ci, Co, k, parts, y_cl)))
+                    again = G.conv2d_layout(hiplib, x, w, b, (dd, dd), (pp, pp), act=1, dtype=dtype, x_cl=1, y_cl=y_cl, scale=sc)
+                    assert np.array_equal(got, again), "cut tiles: results depend on timing"
+    finally:
+        hiplib.thhip_conv_set_tail_parts(8)
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+
+
+@pytest.mark.parametrize("dtype", [G.F16, G.BF16])
 @pytest.mark.parametrize("i", [0, 1, 3, 5, 10])
 def test_conv_half_vs_fp32_oracle(hiplib, oracle, i, dtype):
     x, s = cases.conv_case(i)

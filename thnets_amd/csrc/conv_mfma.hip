@@ -59,7 +59,9 @@ struct ConvParams {
 	/* conv_f32_direct_kernel: K split of the last tiles of every XCD only (0 slots: none) */
 	int tail_slots;		/* workgroups an XCD holds at once */
 	int tail_max;		/* most parts per tile */
-	int tail_cap;		/* scratch blocks reserved per XCD: [xcd][tail_cap][parts][BM*BN] */
+	int tail_cap;		/* scratch blocks (parts of BM*BN sums) reserved per XCD: [xcd][tile][part] */
+	int tail_tiles;		/* most cut tiles of an XCD */
+	int tail_round;		/* 1: an XCD with less than one whole round of tiles is left uncut */
 	/* uint8 path only */
 	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
 	const int *addend;	/* per-plane bias addend, or NULL */
@@ -958,6 +960,102 @@ __device__ __forceinline__ void wide_wait()
 #undef WIDE_WAIT_CASE
 }
 
+/* XCD x's rectangle of the tile grid (mparts x 8/mparts rectangles): first tile
+ * row, rows, first tile column, and the number of tiles. */
+__device__ inline void conv_xcd_rect(const ConvParams &p, int xcd, int &m0, int &mw, int &n0, int &cnt)
+{
+	const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
+	m0 = p.tiles_m * mp / p.mparts;
+	const int m1 = p.tiles_m * (mp + 1) / p.mparts;
+	n0 = p.tiles_n * np / nparts;
+	const int n1 = p.tiles_n * (np + 1) / nparts;
+	mw = m1 - m0;
+	cnt = mw * (n1 - n0);
+}
+
+/* The tiles an XCD cannot spread evenly: of its cnt tiles the last cnt % slots
+ * would run a few to a CU (or alone) while the other CUs idle.  Those are cut
+ * along K into as many parts as fill the slots once, at most smax; *full is
+ * the number of tiles that stay whole.  need_round: cut only where at least
+ * one whole round precedes.  Returns the parts (1: no cut). */
+__host__ __device__ inline int conv_tail_parts(int cnt, int slots, int smax, int need_round, int *full)
+{
+	*full = cnt;
+	if (slots <= 0)
+		return 1;
+	const int f = cnt / slots * slots, rem = cnt - f;
+	/* after more than four rounds the workgroups of an XCD have drifted apart
+	 * and its CUs run dry at different times anyway (64->64 @224^2 batch 16,
+	 * eight rounds: 473 us uncut, 479 + 6 us cut) */
+	if (!rem || f > 4 * slots || (need_round && !f))
+		return 1;
+	int s = slots / rem;
+	if (s > smax)
+		s = smax;
+	if (s < 2)
+		return 1;
+	*full = f;
+	return s;
+}
+
+/* Epilogue of the half-type tiles of conv_wide_kernel (WGM x WGN waves, each
+ * TMF x TNF accumulators of 32x32, of which acc holds the TM x TN from
+ * (i0, j0) on): (folded batch norm factor,) bias, optional threshold, store in
+ * either memory order.  lrow: 2 * BM ints of LDS no wave still reads. */
+template <int DT, bool CLO, int BM, int BN, int WGM, int WGN, int TMF, int TNF, int TM, int TN>
+__device__ __forceinline__ void conv_wide_store_half(const ConvParams &p, floatx16 (&acc)[TM][TN], int tile_m, int tile_n, int *lrow,
+	int i0 = 0, int j0 = 0)
+{
+	typedef typename ConvTraits<DT>::elem elem;
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave % WGM, wn = wave / WGM;
+	elem *y = (elem *)p.y;
+	if (tid < BM) {
+		const int mc = min(tile_m * BM + tid, p.Co - 1);
+		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+		if (p.scale)
+			lrow[BM + tid] = __float_as_int(p.scale[mc]);
+	}
+	__syncthreads();
+	const bool has_scale = p.scale != 0;
+#pragma unroll
+	for (int j = 0; j < TN; j++) {
+		const int n = tile_n * BN + (wn * TNF + j0 + j) * 32 + (lane & 31);
+		if (n >= p.N)
+			continue;
+		const int b = n / p.oHW, rem = n - b * p.oHW;
+		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+#pragma unroll
+		for (int i = 0; i < TM; i++) {
+			const int m0 = tile_m * BM + (wm * TMF + i0 + i) * 32 + 4 * (lane >> 5);
+#pragma unroll
+			for (int g = 0; g < 4; g++) {
+				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+				const int ml = (wm * TMF + i0 + i) * 32 + 4 * (lane >> 5) + 8 * g;
+				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+				floatx4 rowscale = { 1, 1, 1, 1 };
+				if (has_scale)
+					rowscale = *(const floatx4 *)(lrow + BM + ml);
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int r = 4 * g + e, m = m0 + 8 * g + e;
+					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
+					if (p.act)
+						v = v > p.thr ? v : p.val;
+					if constexpr (!CLO) {
+						if (m < p.Co)
+							y[ybase + (size_t)m * p.oHW] = (elem)v;
+					}
+					quad.v[e] = (elem)v;
+				}
+				if constexpr (CLO) {
+					if (m0 + 8 * g < p.Co)
+						*(Quad *)(y + (size_t)n * p.Co + m0 + 8 * g) = quad;
+				}
+			}
+		}
+	}
+}
+
 template <int DT, bool CLO, int BM, int BN, int WGM, int WGN, int KCH, int NST>
 __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 {
@@ -988,16 +1086,26 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wm = wave % WGM, wn = wave / WGM;
 
-	int tile_m, tile_n;
+	int tile_m, tile_n, split = 0, nsplit = 1;
+	long tail_blk = -1;
 	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
 		const int bid = blockIdx.x;
 		const int xcd = bid & 7;
-		const int local = bid >> 3;
-		const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
-		const int m0 = p.tiles_m * mp / p.mparts, m1 = p.tiles_m * (mp + 1) / p.mparts;
-		const int n0 = p.tiles_n * np / nparts, n1 = p.tiles_n * (np + 1) / nparts;
-		const int mw = m1 - m0;
-		if (local >= mw * (n1 - n0))
+		int local = bid >> 3;
+		int m0, mw, n0, cnt;
+		conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
+		if (DT != THHIP_U8 && p.tail_slots) {	/* the XCD's last tiles, dispatched last, in parts along K */
+			int full;
+			const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, p.tail_round, &full);
+			if (s > 1 && local >= full) {
+				const int t = (local - full) / s;
+				split = (local - full) - t * s;
+				nsplit = s;
+				local = full + t;
+				tail_blk = (long)xcd * p.tail_cap + t * s + split;
+			}
+		}
+		if (local >= cnt)
 			return;
 		tile_m = m0 + local % mw;
 		tile_n = n0 + local / mw;
@@ -1034,7 +1142,17 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
 		a_lds_[i] = (kci * MB + mbi) * 64;
 	}
-	int t_cb = 0, t_kh = 0, t_kw = 0, t_kc = 0;
+	/* K-tiles: tap outer, planes inner; a part of a cut tile walks [kt0, kt0 + nkt) */
+	const int nkt_all = p.KC / KCH;
+	const int kt0 = nsplit > 1 ? (int)((long)nkt_all * split / nsplit) : 0;
+	const int nkt = (nsplit > 1 ? (int)((long)nkt_all * (split + 1) / nsplit) : nkt_all) - kt0;
+	int t_cb, t_kh, t_kw, t_kc = kt0 * KCH;
+	{
+		const int per_tap = p.Ci / (KCH * CHUNK), tap = kt0 / per_tap;
+		t_cb = (kt0 - tap * per_tap) * (KCH * CHUNK);
+		t_kh = tap / p.kW;
+		t_kw = tap - t_kh * p.kW;
+	}
 
 	auto issue = [&](auto st_) {
 		constexpr int st = decltype(st_)::value;
@@ -1117,7 +1235,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	typedef std::integral_constant<int, 1> S1;
 	typedef std::integral_constant<int, NST >= 3 ? 2 : 0> S2;
 	typedef std::integral_constant<int, NST >= 4 ? 3 : 0> S3;
-	const int nkt = p.KC / KCH;
 	issue(S0{});
 	if (1 < nkt)
 		issue(S1{});
@@ -1191,20 +1308,32 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	}
 
 	/* ---- epilogue ---- */
+	if constexpr (DT != THHIP_U8) {
+		if (tail_blk >= 0) {
+			/* a part of one of the XCD's last tiles: the accumulators as they lie in
+			 * the registers, [register][thread]; conv_wide_tail_finish_kernel adds
+			 * the parts in their order */
+			float *part = (float *)p.ws + tail_blk * (BM * BN);
+#pragma unroll
+			for (int i = 0; i < TM; i++)
+#pragma unroll
+				for (int j = 0; j < TN; j++)
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						part[((i * TN + j) * 16 + r) * (64 * WAVES) + tid] = acc[i][j][r];
+			return;
+		}
+		__syncthreads();		/* every wave is done with the tiles */
+		conv_wide_store_half<DT, CLO, BM, BN, WGM, WGN, TM, TN, TM, TN>(p, acc, tile_m, tile_n, (int *)lds);
+	} else {
 	elem *y = (elem *)p.y;
 	int *lrow = (int *)lds;		/* [BM] bias bits or uint8 row term, [BM..2BM) factor bits or uint8 addend */
 	int *cs = lrow + 2 * BM;	/* uint8: [BN] column sums */
 	__syncthreads();		/* every wave is done with the tiles */
 	if (tid < BM) {
 		const int mc = min(tile_m * BM + tid, p.Co - 1);
-		if constexpr (DT == THHIP_U8) {
-			lrow[tid] = p.offB * p.rowsum[mc] + p.K * p.offA * p.offB;
-			lrow[BM + tid] = p.addend ? p.addend[mc] : 0;
-		} else {
-			lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
-			if (p.scale)
-				lrow[BM + tid] = __float_as_int(p.scale[mc]);
-		}
+		lrow[tid] = p.offB * p.rowsum[mc] + p.K * p.offA * p.offB;
+		lrow[BM + tid] = p.addend ? p.addend[mc] : 0;
 	}
 	if constexpr (DT == THHIP_U8) {
 		for (int i = tid; i < BN; i += 64 * WAVES)
@@ -1264,47 +1393,41 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 				}
 			}
 		}
-	} else {
-	const bool has_scale = p.scale != 0;
-#pragma unroll
-	for (int j = 0; j < TN; j++) {
-		const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
-		if (n >= p.N)
-			continue;
-		const int b = n / p.oHW, rem = n - b * p.oHW;
-		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
-#pragma unroll
-		for (int i = 0; i < TM; i++) {
-			const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
-#pragma unroll
-			for (int g = 0; g < 4; g++) {
-				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
-				const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
-				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
-				floatx4 rowscale = { 1, 1, 1, 1 };
-				if (has_scale)
-					rowscale = *(const floatx4 *)(lrow + BM + ml);
-#pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int r = 4 * g + e, m = m0 + 8 * g + e;
-					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
-					if (p.act)
-						v = v > p.thr ? v : p.val;
-					if constexpr (!CLO) {
-						if (m < p.Co)
-							y[ybase + (size_t)m * p.oHW] = (elem)v;
-					}
-					quad.v[e] = (elem)v;
-				}
-				if constexpr (CLO) {
-					if (m0 + 8 * g < p.Co)
-						*(Quad *)(y + (size_t)n * p.Co + m0 + 8 * g) = quad;
-				}
-			}
-		}
 	}
 	}
 #endif
+}
+
+/* Adds the K parts of the tiles conv_wide_kernel cut
+ * ([xcd][tile][part][register][thread] in scratch) in their order and finishes
+ * them as that kernel's epilogue does.  One workgroup per cut tile and
+ * accumulator (i, j) of a wave, so that a thread waits for as many loads in
+ * turn as there are parts, not TM * TN times that. */
+template <int DT, bool CLO, int BM, int BN, int WGM, int WGN>
+__global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_tail_finish_kernel(ConvParams p)
+{
+	constexpr int TM = BM / WGM / 32, TN = BN / WGN / 32, THREADS = 64 * WGM * WGN;
+	__shared__ int lrow[2 * BM];
+	const int tid = threadIdx.x, xcd = blockIdx.x & 7;
+	const int t = (blockIdx.x >> 3) / (TM * TN), ij = (blockIdx.x >> 3) % (TM * TN);
+	int m0, mw, n0, cnt, full;
+	conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
+	const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, p.tail_round, &full);
+	if (s < 2 || t >= cnt - full)
+		return;
+	const int local = full + t;
+	const float *part = (const float *)p.ws + ((long)xcd * p.tail_cap + t * s) * (BM * BN) + (ij * 16) * THREADS + tid;
+	floatx16 acc[1][1];
+#pragma unroll
+	for (int r = 0; r < 16; r++)
+		acc[0][0][r] = part[r * THREADS];
+	for (int q = 1; q < s; q++) {
+		part += BM * BN;
+#pragma unroll
+		for (int r = 0; r < 16; r++)
+			acc[0][0][r] += part[r * THREADS];
+	}
+	conv_wide_store_half<DT, CLO, BM, BN, WGM, WGN, TM, TN, 1, 1>(p, acc, m0 + local % mw, n0 + local / mw, lrow, ij / TN, ij % TN);
 }
 
 /* ------------------------------------------------------------------ */
@@ -1599,49 +1722,12 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 /* fp32, plane-major: operands straight into LDS                       */
 /* ------------------------------------------------------------------ */
 
-/* XCD x's rectangle of the tile grid (mparts x 8/mparts rectangles): first tile
- * row, rows, first tile column, and the number of tiles. */
-__device__ inline void conv_xcd_rect(const ConvParams &p, int xcd, int &m0, int &mw, int &n0, int &cnt)
-{
-	const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
-	m0 = p.tiles_m * mp / p.mparts;
-	const int m1 = p.tiles_m * (mp + 1) / p.mparts;
-	n0 = p.tiles_n * np / nparts;
-	const int n1 = p.tiles_n * (np + 1) / nparts;
-	mw = m1 - m0;
-	cnt = mw * (n1 - n0);
-}
-
-/* The tiles an XCD cannot spread evenly: of its cnt tiles the last cnt % slots
- * would run a few to a CU (or alone) while the other CUs idle.  Those are cut
- * along K into as many parts as fill the slots once, at most smax; *full is
- * the number of tiles that stay whole.  Returns the parts (1: no cut). */
-__host__ __device__ inline int conv_tail_parts(int cnt, int slots, int smax, int *full)
-{
-	*full = cnt;
-	if (slots <= 0)
-		return 1;
-	const int f = cnt / slots * slots, rem = cnt - f;
-	/* after more than four rounds the workgroups of an XCD have drifted apart
-	 * and its CUs run dry at different times anyway (64->64 @224^2 batch 16,
-	 * eight rounds: 473 us uncut, 479 + 6 us cut) */
-	if (!rem || f > 4 * slots)
-		return 1;
-	int s = slots / rem;
-	if (s > smax)
-		s = smax;
-	if (s < 2)
-		return 1;
-	*full = f;
-	return s;
-}
-
 /* Epilogue of the fp32 tiles whose accumulators are laid out as in
  * conv_f32_direct_kernel (2 x 2 waves): (folded batch norm factor,) bias,
  * optional threshold, plane-major store.  lrow: 2 * BM ints of LDS no wave
  * still reads. */
 template <int BM, int BN, int TM, int TN>
-__device__ inline void conv_f32_direct_store(const ConvParams &p, floatx16 (&acc)[TM][TN], int tile_m, int tile_n, int *lrow)
+__device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, floatx16 (&acc)[TM][TN], int tile_m, int tile_n, int *lrow)
 {
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave % 2, wn = wave / 2;
 	float *y = (float *)p.y;
@@ -1730,13 +1816,13 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
 		if (p.tail_slots) {	/* the XCD's last tiles, dispatched last, in parts along K */
 			int full;
-			const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, &full);
+			const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, p.tail_round, &full);
 			if (s > 1 && local >= full) {
 				const int t = (local - full) / s;
 				split = (local - full) - t * s;
 				nsplit = s;
 				local = full + t;
-				tail_blk = ((long)xcd * p.tail_cap + t) * s + split;
+				tail_blk = (long)xcd * p.tail_cap + t * s + split;
 			}
 		}
 		if (local >= cnt)
@@ -1970,11 +2056,11 @@ __global__ __launch_bounds__(256) void conv_f32_tail_finish_kernel(ConvParams p)
 	const int tid = threadIdx.x, xcd = blockIdx.x & 7, t = blockIdx.x >> 3;
 	int m0, mw, n0, cnt, full;
 	conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
-	const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, &full);
+	const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, p.tail_round, &full);
 	if (s < 2 || t >= cnt - full)
 		return;
 	const int local = full + t;
-	const float *part = (const float *)p.ws + ((long)xcd * p.tail_cap + t) * s * (BM * BN);
+	const float *part = (const float *)p.ws + ((long)xcd * p.tail_cap + t * s) * (BM * BN);
 	floatx16 acc[TM][TN];
 	/* part by part, so that the loads of one part are all in flight together */
 #pragma unroll
@@ -2173,8 +2259,8 @@ extern "C" void thhip_conv_set_xcd_parts(int mparts)
 	g_force_mparts = mparts;
 }
 
-/* fp32 tiles loaded straight into LDS: the most K parts for the tiles an XCD
- * cannot spread evenly over its CUs (1: never cut them). */
+/* fp32 and half-type tiles loaded straight into LDS: the most K parts for the
+ * tiles an XCD cannot spread evenly over its CUs (1: never cut them). */
 static int g_tail_parts = 8;
 extern "C" void thhip_conv_set_tail_parts(int parts)
 {
@@ -2343,6 +2429,62 @@ static void conv_launch(ConvParams &p, int splitk, int wgs)
 #undef CONV_GO
 }
 
+/* Points p.ws at scratch of at least that many bytes. */
+static void conv_f32_scratch(ConvParams &p, size_t need)
+{
+	if (need > g_ws_bytes) {
+		hipcheck(hipStreamSynchronize(thhip_stream()));
+		thhip_free(g_ws);
+		g_ws = (int *)thhip_malloc(need);
+		g_ws_bytes = need;
+	}
+	p.ws = g_ws;
+}
+
+/* Plans the cut of every XCD's last tiles (conv_tail_parts) for a kernel that
+ * holds `resident` workgroups per CU and walks nkt K-tiles per tile: sets
+ * p.tail_*, points p.ws at scratch for the parts and returns the largest
+ * number of workgroups an XCD needs (its whole tiles plus the parts). */
+static size_t conv_tail_plan(ConvParams &p, int resident, int nkt, size_t tile_floats, int need_round)
+{
+	static int cus;
+	if (!cus) {
+		int dev;
+		hipcheck(hipGetDevice(&dev));
+		hipcheck(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+	}
+	p.tail_slots = p.tail_max = p.tail_cap = p.tail_tiles = 0;
+	p.tail_round = need_round;
+	if (p.splitk == 1 && g_tail_parts != 1) {
+		p.tail_slots = cus / 8 * (resident < 1 ? 1 : resident);
+		p.tail_max = nkt / 8 < g_tail_parts ? nkt / 8 : g_tail_parts;	/* at least eight K-tiles a part */
+		if (p.tail_max < 2)
+			p.tail_slots = 0;
+	}
+	size_t maxwgs = 0;
+	for (int x = 0; x < 8; x++) {
+		const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
+		const int cnt = (p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
+			(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
+		int full;
+		const int sx = conv_tail_parts(cnt, p.tail_slots, p.tail_max, p.tail_round, &full);
+		if (sx > 1) {
+			if ((cnt - full) * sx > p.tail_cap)
+				p.tail_cap = (cnt - full) * sx;
+			if (cnt - full > p.tail_tiles)
+				p.tail_tiles = cnt - full;
+		}
+		const size_t wgs = (size_t)full + (size_t)(cnt - full) * sx;
+		if (wgs > maxwgs)
+			maxwgs = wgs;
+	}
+	if (!p.tail_cap)
+		p.tail_slots = 0;
+	else
+		conv_f32_scratch(p, (size_t)8 * p.tail_cap * tile_floats * sizeof(float));
+	return maxwgs;
+}
+
 /* Whether the kernel that loads straight into LDS can run this layer: a half
  * type or uint8, channels-last input with whole K-tiles (32 halfs, 64 codes)
  * inside a tap, 32-bit byte offsets; uint8 input followed by a K-tile slice of
@@ -2374,19 +2516,39 @@ static void conv_launch_wide(ConvParams &p)
 			p.mparts *= 2;
 		if (g_force_mparts)
 			p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
-		size_t maxcnt = 0;
-		for (int x = 0; x < 8; x++) {
-			const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
-			const size_t cnt = (size_t)(p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
-				(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
-			if (cnt > maxcnt)
-				maxcnt = cnt;
+		/* half types: the tiles an XCD cannot spread evenly over its CUs are cut
+		 * along K, as in conv_launch_f32_direct (uint8 tiles stay whole: their
+		 * column sums run over all of K) */
+		int resident = 0;
+		if constexpr (DT != THHIP_U8) {
+			static int res_cl, res_pm;
+			int &res = p.y_cl ? res_cl : res_pm;
+			if (!res) {
+				if (p.y_cl)
+					hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&res, conv_wide_kernel<DT, true, BM, BN, WGM, WGN, KCH, NST>, 64 * WGM * WGN, 0));
+				else
+					hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&res, conv_wide_kernel<DT, false, BM, BN, WGM, WGN, KCH, NST>, 64 * WGM * WGN, 0));
+				if (res < 1)
+					res = 1;
+			}
+			resident = res;
 		}
+		/* few tiles all cut measured slower here (512->512 @14^2 batch 16, fp16: 31 -> 36 us) */
+		const size_t maxcnt = conv_tail_plan(p, resident, DT == THHIP_U8 ? 0 : p.KC / KCH, (size_t)BM * BN, 1);
 		dim3 grid((unsigned)(8 * maxcnt));
 		if (p.y_cl)
 			conv_wide_kernel<DT, true, BM, BN, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
 		else
 			conv_wide_kernel<DT, false, BM, BN, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+		if constexpr (DT != THHIP_U8) {
+			if (p.tail_slots) {
+				dim3 fgrid((unsigned)(8 * p.tail_tiles * (BM / WGM / 32) * (BN / WGN / 32)));
+				if (p.y_cl)
+					conv_wide_tail_finish_kernel<DT, true, BM, BN, WGM, WGN><<<fgrid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+				else
+					conv_wide_tail_finish_kernel<DT, false, BM, BN, WGM, WGN><<<fgrid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+			}
+		}
 	} else
 		THError("thhip_conv2d: no such tile loaded straight into LDS for this type");
 }
@@ -2396,18 +2558,6 @@ static void conv_launch_wide(ConvParams &p)
 static bool conv_f32_direct_ok(const ConvParams &p)
 {
 	return !p.x_cl && !p.y_cl && p.Ci % 32 == 0 && p.x_bytes < 0x7fffffffu;
-}
-
-/* Points p.ws at scratch of at least that many bytes. */
-static void conv_f32_scratch(ConvParams &p, size_t need)
-{
-	if (need > g_ws_bytes) {
-		hipcheck(hipStreamSynchronize(thhip_stream()));
-		thhip_free(g_ws);
-		g_ws = (int *)thhip_malloc(need);
-		g_ws_bytes = need;
-	}
-	p.ws = g_ws;
 }
 
 template <int BM, int BN, int KCH, int NST>
@@ -2429,54 +2579,15 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 		p.mparts *= 2;
 	if (g_force_mparts)
 		p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
-	size_t maxcnt = 0;
-	for (int x = 0; x < 8; x++) {
-		const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
-		const size_t cnt = (size_t)(p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
-			(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
-		if (cnt > maxcnt)
-			maxcnt = cnt;
-	}
 	/* Without a K split of the whole layer: the tiles an XCD cannot spread evenly
-	 * over its CUs are cut along K (conv_tail_parts), at least eight K-tiles a part. */
-	p.tail_slots = p.tail_max = p.tail_cap = 0;
-	if (p.splitk == 1 && g_tail_parts != 1) {
-		static int resident, cus;
-		if (!resident) {
-			int dev;
-			hipcheck(hipGetDevice(&dev));
-			hipcheck(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
-			hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_direct_kernel<BM, BN, KCH, NST>, 256, 0));
-			if (resident < 1)
-				resident = 1;
-		}
-		p.tail_slots = cus / 8 * resident;
-		p.tail_max = nkt / 8 < g_tail_parts ? nkt / 8 : g_tail_parts;
-		if (p.tail_max < 2)
-			p.tail_slots = 0;
+	 * over its CUs are cut along K (conv_tail_parts). */
+	static int resident;
+	if (!resident) {
+		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_direct_kernel<BM, BN, KCH, NST>, 256, 0));
+		if (resident < 1)
+			resident = 1;
 	}
-	int smax = 1;
-	if (p.tail_slots) {
-		maxcnt = 0;
-		for (int x = 0; x < 8; x++) {
-			const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
-			const int cnt = (p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
-				(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
-			int full;
-			const int sx = conv_tail_parts(cnt, p.tail_slots, p.tail_max, &full);
-			if (sx > 1 && cnt - full > p.tail_cap)
-				p.tail_cap = cnt - full;
-			if (sx > smax)
-				smax = sx;
-			const size_t wgs = (size_t)full + (size_t)(cnt - full) * sx;
-			if (wgs > maxcnt)
-				maxcnt = wgs;
-		}
-		if (!p.tail_cap)
-			p.tail_slots = 0;
-		else
-			conv_f32_scratch(p, (size_t)8 * p.tail_cap * smax * BM * BN * sizeof(float));
-	}
+	const size_t maxcnt = conv_tail_plan(p, resident, nkt, (size_t)BM * BN, 0);
 	conv_f32_direct_kernel<BM, BN, KCH, NST><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
 	if (p.splitk > 1) {
 		long blocks = ((long)p.Co * p.N + 255) / 256;
@@ -2486,7 +2597,7 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 			(float *)p.y, p.splitk, p.Co, p.N, p.oHW, p.act, p.thr, p.val);
 	}
 	if (p.tail_slots)
-		conv_f32_tail_finish_kernel<BM, BN><<<dim3((unsigned)(8 * p.tail_cap)), dim3(256), 0, thhip_stream()>>>(p);
+		conv_f32_tail_finish_kernel<BM, BN><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
 /* Whether conv_patch_kernel can run this layer. */
