@@ -447,8 +447,8 @@ void thhip_conv_set_ktile(int chunks);
  * count modulo the workgroups it holds at once; half types: only after at
  * least one whole round) are dispatched last and cut along K into up to
  * `parts` parts of at least eight K-tiles, summed in their order by a small
- * kernel (results do not depend on timing).  Default 8; 1 = never cut.  Tests
- * and tuning. */
+ * kernel (results do not depend on timing).  Default 8, which is also the most
+ * that is used; 1 = never cut.  Tests and tuning. */
 void thhip_conv_set_tail_parts(int parts);
 /* Force how the tile grid is cut over the eight XCDs: the M tiles into
  * mparts (1, 2, 4, 8) groups, the N tiles into 8 / mparts ranges; 0 restores

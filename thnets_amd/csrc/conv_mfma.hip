@@ -1417,16 +1417,23 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_tail_finish_kernel(C
 		return;
 	const int local = full + t;
 	const float *part = (const float *)p.ws + ((long)xcd * p.tail_cap + t * s) * (BM * BN) + (ij * 16) * THREADS + tid;
-	floatx16 acc[1][1];
+	/* all parts requested at once (at most eight: conv_tail_plan), added in their order */
+	floatx16 acc[1][1], in[8];
 #pragma unroll
-	for (int r = 0; r < 16; r++)
-		acc[0][0][r] = part[r * THREADS];
-	for (int q = 1; q < s; q++) {
-		part += BM * BN;
+	for (int q = 0; q < 8; q++)
+		if (q < s) {
 #pragma unroll
-		for (int r = 0; r < 16; r++)
-			acc[0][0][r] += part[r * THREADS];
-	}
+			for (int r = 0; r < 16; r++)
+				in[q][r] = part[(long)q * (BM * BN) + r * THREADS];
+		}
+	acc[0][0] = in[0];
+#pragma unroll
+	for (int q = 1; q < 8; q++)
+		if (q < s) {
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[0][0][r] += in[q][r];
+		}
 	conv_wide_store_half<DT, CLO, BM, BN, WGM, WGN, TM, TN, 1, 1>(p, acc, m0 + local % mw, n0 + local / mw, lrow, ij / TN, ij % TN);
 }
 
@@ -2062,24 +2069,29 @@ __global__ __launch_bounds__(256) void conv_f32_tail_finish_kernel(ConvParams p)
 	const int local = full + t;
 	const float *part = (const float *)p.ws + ((long)xcd * p.tail_cap + t * s) * (BM * BN);
 	floatx16 acc[TM][TN];
-	/* part by part, so that the loads of one part are all in flight together */
+	/* accumulator by accumulator: all parts requested at once (at most eight:
+	 * conv_tail_plan), added in their order */
 #pragma unroll
 	for (int i = 0; i < TM; i++)
 #pragma unroll
-		for (int j = 0; j < TN; j++)
+		for (int j = 0; j < TN; j++) {
+			floatx16 in[8];
 #pragma unroll
-			for (int r = 0; r < 16; r++)
-				acc[i][j][r] = part[((i * TN + j) * 16 + r) * 256 + tid];
-	for (int q = 1; q < s; q++) {
-		part += BM * BN;
+			for (int q = 0; q < 8; q++)
+				if (q < s) {
 #pragma unroll
-		for (int i = 0; i < TM; i++)
+					for (int r = 0; r < 16; r++)
+						in[q][r] = part[(long)q * (BM * BN) + ((i * TN + j) * 16 + r) * 256 + tid];
+				}
+			acc[i][j] = in[0];
 #pragma unroll
-			for (int j = 0; j < TN; j++)
+			for (int q = 1; q < 8; q++)
+				if (q < s) {
 #pragma unroll
-				for (int r = 0; r < 16; r++)
-					acc[i][j][r] += part[((i * TN + j) * 16 + r) * 256 + tid];
-	}
+					for (int r = 0; r < 16; r++)
+						acc[i][j][r] += in[q][r];
+				}
+		}
 	conv_f32_direct_store<BM, BN, TM, TN>(p, acc, m0 + local % mw, n0 + local / mw, lrow);
 }
 
@@ -2458,6 +2470,8 @@ static size_t conv_tail_plan(ConvParams &p, int resident, int nkt, size_t tile_f
 	if (p.splitk == 1 && g_tail_parts != 1) {
 		p.tail_slots = cus / 8 * (resident < 1 ? 1 : resident);
 		p.tail_max = nkt / 8 < g_tail_parts ? nkt / 8 : g_tail_parts;	/* at least eight K-tiles a part */
+		if (p.tail_max > 8)
+			p.tail_max = 8;	/* the finishing kernels hold eight parts in registers */
 		if (p.tail_max < 2)
 			p.tail_slots = 0;
 	}
