@@ -31,7 +31,7 @@ PEAK_TOPS_INT8_MFMA = 5030.0
 # Bytes moved past L2 per convolution launch in the VGG-16 b16 step (average of the 13), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled against a 256 MiB copy
 # (profiles/conv_f32_vgg16_fp32_b16_counters.md); algorithmic bytes are 115.9e6.
-CONV_HBM_BYTES_PER_LAUNCH = 175.6e6
+CONV_HBM_BYTES_PER_LAUNCH = 175.0e6
 
 
 def profile_get(lib, fam):
