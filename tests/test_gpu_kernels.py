@@ -104,10 +104,12 @@ def test_conv_f32_last_tiles_cut_along_k(hiplib, oracle):
     partial tiles on both axes, the folded batch-norm factor and the threshold; every
     limit on the parts, 1 = never cut; the same call twice gives the same bits."""
     g = cases.rng(917)
-    shapes = [(4, 64, 112, 112, 64, 3, 1, 1), (1, 64, 20, 20, 64, 5, 1, 2), (2, 96, 30, 30, 70, 3, 1, 1),
-              (5, 128, 28, 28, 128, 3, 1, 1), (3, 256, 27, 27, 100, 3, 2, 1)]
+    # last entry: the M tiles cut into that many groups over the XCDs (0: by weight size)
+    shapes = [(4, 64, 112, 112, 64, 3, 1, 1, 0), (1, 64, 20, 20, 64, 5, 1, 2, 0), (2, 96, 30, 30, 70, 3, 1, 1, 0),
+              (5, 128, 28, 28, 128, 3, 1, 1, 0), (3, 256, 27, 27, 100, 3, 2, 1, 0), (4, 64, 112, 112, 128, 3, 1, 1, 2)]
     try:
-        for (B, Ci, H, W, Co, k, dd, pp) in shapes:
+        for (B, Ci, H, W, Co, k, dd, pp, mparts) in shapes:
+            hiplib.thhip_conv_set_xcd_parts(mparts)
             x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
             w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
             b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
@@ -123,6 +125,7 @@ def test_conv_f32_last_tiles_cut_along_k(hiplib, oracle):
                 assert np.array_equal(got, again), "cut tiles: results depend on timing"
     finally:
         hiplib.thhip_conv_set_tail_parts(8)
+        hiplib.thhip_conv_set_xcd_parts(0)
 
 
 @pytest.mark.parametrize("dtype", [G.F16, G.BF16])
@@ -135,10 +138,12 @@ def test_conv_half_last_tiles_cut_along_k(hiplib, oracle, dtype):
     output orders, the factor and the threshold, every limit on the parts (1 = never
     cut), same bits twice."""
     g = cases.rng(919)
-    shapes = [(8, 64, 91, 91, 100, 3, 1, 1, (128, 128, 9, 0)), (8, 128, 92, 92, 256, 3, 1, 1, (256, 256, 0, 0)),
-              (3, 96, 27, 27, 100, 3, 2, 1, (64, 128, 9, 0))]
+    # last entry: the M tiles cut into that many groups over the XCDs (0: by weight size)
+    shapes = [(8, 64, 91, 91, 100, 3, 1, 1, (128, 128, 9, 0), 0), (8, 128, 92, 92, 256, 3, 1, 1, (256, 256, 0, 0), 0),
+              (3, 96, 27, 27, 100, 3, 2, 1, (64, 128, 9, 0), 0), (8, 64, 91, 91, 256, 3, 1, 1, (128, 128, 9, 0), 2)]
     try:
-        for (B, Ci, H, W, Co, k, dd, pp, tune) in shapes:
+        for (B, Ci, H, W, Co, k, dd, pp, tune, mparts) in shapes:
+            hiplib.thhip_conv_set_xcd_parts(mparts)
             x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
             w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
             b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
@@ -157,6 +162,7 @@ def test_conv_half_last_tiles_cut_along_k(hiplib, oracle, dtype):
     finally:
         hiplib.thhip_conv_set_tail_parts(8)
         hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+        hiplib.thhip_conv_set_xcd_parts(0)
 
 
 @pytest.mark.parametrize("dtype", [G.F16, G.BF16])
