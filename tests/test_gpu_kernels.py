@@ -527,6 +527,27 @@ def test_threshold_bit_exact(hiplib, oracle):
                           GOLD["threshold0"])
 
 
+def test_maxpool_f32_vector_paths_bit_exact(hiplib, oracle):
+    """The fp32 pooling kernels that make several outputs per thread (2x2 / stride 2, and
+    3x3 / stride 2 / padding 1 on planes whose width is a multiple of eight), against the
+    oracle bit for bit: odd and even heights, signed zeros (the first maximum wins), the
+    most negative float, windows that reach outside the plane."""
+    g = cases.rng(930)
+    for (B, Cn, H, W, k, d, pad) in [(2, 3, 16, 16, 3, 2, 1), (1, 5, 15, 24, 3, 2, 1), (2, 2, 8, 8, 3, 2, 1), (1, 2, 7, 40, 3, 2, 1),
+                                     (2, 3, 12, 16, 2, 2, 0), (1, 1, 2, 8, 3, 2, 1)]:
+        x = g.standard_normal((B, Cn, H, W), dtype=np.float32)
+        flat = x.ravel()
+        flat[g.integers(0, flat.size, flat.size // 5)] = 0.0
+        flat[g.integers(0, flat.size, flat.size // 5)] = -0.0
+        flat[g.integers(0, flat.size, flat.size // 7)] = -np.finfo(np.float32).max
+        x[:, :, 0, :] = -np.abs(x[:, :, 0, :])      # a border row whose maxima are zeros of either sign
+        want = oracle.maxpool(x, k, k, d, d, pad, pad, 0)
+        oH, oW = want.shape[2:]
+        G.note("maxpool fp32 vector path %s" % ((B, Cn, H, W, k, d, pad),))
+        y = G.unary(hiplib, hiplib.thhip_maxpool, x, (B, Cn, oH, oW), G.F32, B, Cn, H, W, oH, oW, k, k, d, d, pad, pad, G.F32)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32)), (B, Cn, H, W, k, d, pad)
+
+
 @pytest.mark.parametrize("i", range(len(cases.POOL_CASES)))
 def test_pooling_bit_exact(hiplib, oracle, i):
     x = cases.pool_case(i)

@@ -174,6 +174,46 @@ __global__ void maxpool_f32_2x2_kernel(const floatx4 *x, float2 *y, int H4, int 
 	}
 }
 
+/* The 3x3 / stride 2 / padding 1 pooling of fp32 planes whose width is a
+ * multiple of eight (ResNet's stem): a thread makes four neighbouring outputs
+ * of a row from the nine columns they read, fetched per input row as one
+ * scalar and two 16-byte vectors.  Same comparisons in the same order as the
+ * general kernel (what lies outside the plane is never the maximum). */
+__global__ void maxpool_f32_3x3s2p1_kernel(const float *x, floatx4 *y, int H, int W, int oH, int oW4, long total4)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total4; i += step) {
+		const int xq = (int)(i % oW4);
+		const long t = i / oW4;
+		const int oy = (int)(t % oH);
+		const long plane = t / oH;
+		const float *px = x + plane * H * W + 8 * xq;
+		floatx4 m = { -FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX };
+#pragma unroll
+		for (int r = 0; r < 3; r++) {
+			const int yy = 2 * oy - 1 + r;
+			if (yy < 0 || yy >= H)
+				continue;
+			const float *row = px + (long)yy * W;
+			float v[9];
+			v[0] = xq ? row[-1] : -FLT_MAX;
+			const floatx4 a = *(const floatx4 *)row, b = *(const floatx4 *)(row + 4);
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				v[1 + e] = a[e];
+				v[5 + e] = b[e];
+			}
+#pragma unroll
+			for (int o = 0; o < 4; o++)
+#pragma unroll
+				for (int c = 0; c < 3; c++)
+					m[o] = v[2 * o + c] > m[o] ? v[2 * o + c] : m[o];
+		}
+		y[i] = m;
+	}
+}
+
 extern "C" void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
 	int kH, int kW, int dH, int dW, int padH, int padW, int dtype)
 {
@@ -187,6 +227,13 @@ extern "C" void thhip_maxpool(const void *x, void *y, int B, int C, int H, int W
 		const long total2 = p.total / 2;
 		maxpool_f32_2x2_kernel<<<ew_grid(total2), dim3(EW_THREADS), 0, thhip_stream()>>>((const floatx4 *)x, (float2 *)y,
 			H / 2, oH, oW / 2, total2);
+		return;
+	}
+	if (dtype == THHIP_F32 && kH == 3 && kW == 3 && dH == 2 && dW == 2 && padH == 1 && padW == 1 && W % 8 == 0 &&
+	    oW == W / 2 && oH == (H - 1) / 2 + 1 && ((size_t)x & 15) == 0 && ((size_t)y & 15) == 0) {
+		const long total4 = p.total / 4;
+		maxpool_f32_3x3s2p1_kernel<<<ew_grid(total4), dim3(EW_THREADS), 0, thhip_stream()>>>((const float *)x, (floatx4 *)y,
+			H, W, oH, oW / 4, total4);
 		return;
 	}
 	const dim3 grid = ew_grid(p.total);
