@@ -9,11 +9,14 @@
  * the batch-1 matrix-vector kernel, but every weight is used B times, which is
  * exactly one 16x16x4 fp32 MFMA per 16 rows x 16 batch columns x 4 k.  A
  * wavefront owns 16 output rows and a slice of K: per step lane (m = lane%16,
- * q = lane/16) issues four 16-byte loads of row m (k = k0 + 16j + 4q + s, so
- * the four quarters of a load cover 64 adjacent bytes), the matching lane of
- * the B operand reads the same k of batch row n = lane%16 (X is small and
- * stays in L2), and 16 MFMAs contract them; the order of k inside a dot
- * product is free as long as both operands use the same one.  K is split over the four wavefronts of a workgroup (summed
+ * q = lane/16) holds four 16-byte vectors of row m (k = k0 + 16j + 4q + s),
+ * the matching lane of the B operand the same k of batch row n = lane%16 (X
+ * is small and stays in L2), and 16 MFMAs contract them; the order of k
+ * inside a dot product is free as long as both operands use the same one.
+ * The vectors are loaded by other lanes than the ones that use them, so that
+ * neighbouring lanes read neighbouring addresses (64 or 128 adjacent bytes of
+ * a row instead of 16), and moved with lane permutes: 25088 -> 4096 at batch
+ * 16, fp32, 107 -> 83 us.  K is split over the four wavefronts of a workgroup (summed
  * through LDS) and over gridDim.y workgroups (partials in a scratch buffer,
  * summed by a second tiny kernel that also applies bias and Threshold).
  * For wide layers a wavefront owns RB = 4 such blocks of 16 rows: the batch
@@ -45,6 +48,16 @@ template <> __device__ __forceinline__ void skinny_mma<THHIP_BF16>(floatx4 &acc,
 	acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
 }
 
+/* The vector held by the lane whose byte index (lane * 4) is given. */
+__device__ __forceinline__ floatx4 skinny_permute(const floatx4 &v, int src_lane4)
+{
+	floatx4 r;
+#pragma unroll
+	for (int e = 0; e < 4; e++)
+		r[e] = __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane4, __float_as_int(v[e])));
+	return r;
+}
+
 template <int DT, int NB, int RB>	/* NB 16-column groups: batch <= 16 * NB; RB 16-row blocks per wavefront */
 __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const void *xv, const void *wv, float *part,
 	int B, int nIn, int nOut, int ksplit)
@@ -56,18 +69,34 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const void *xv, cons
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int m = lane & 15, q = lane >> 4;
+	/* The MFMA wants row m = lane % 16 in lane q * 16 + m, so neighbouring lanes
+	 * would load from rows a whole row length apart, 64 separate 16-byte requests
+	 * per instruction.  Instead neighbouring lanes load neighbouring vectors and a
+	 * lane permute brings every vector to the lane that feeds it to the matrix
+	 * core.  Batch operand: lane 4 m' + q' loads for (row m', quarter q'), 64
+	 * adjacent bytes per four lanes.  Weights (four row blocks per wavefront): load i of a step takes rows
+	 * 8 (i % 2) + lane / 8 and vector 8 (i / 2) + lane % 8 of the step's sixteen,
+	 * whole 128-byte lines per eight lanes; the vector for (m, q) of MFMA group j
+	 * then sits in load 2 (j / 2) + m / 8, lane 8 (m % 8) + 4 (j % 2) + q. */
+	constexpr bool WIDE_W = RB == 4;
+	const int lm = lane >> 2, lq = lane & 3;
+	const int src_lane4 = (m * 4 + q) * 4;	/* byte index of the lane that loaded for (m, q) */
+	const int wsrc4[2] = { ((m & 7) * 8 + q) * 4, ((m & 7) * 8 + 4 + q) * 4 };
+	const bool upper = m >= 8;
 	const int row0 = blockIdx.x * (16 * RB);
 	/* K-steps are dealt round-robin to (workgroup slice, wave) */
 	const int nsteps = (nIn + KSTEP - 1) / KSTEP;
 	const int stride = ksplit * 4;
-	const elem *wr[RB];
+	const elem *wr[RB][2];
 #pragma unroll
 	for (int rb = 0; rb < RB; rb++)
-		wr[rb] = w + (size_t)min(row0 + rb * 16 + m, nOut - 1) * nIn;
+#pragma unroll
+		for (int h = 0; h < 2; h++)
+			wr[rb][h] = w + (size_t)min(row0 + rb * 16 + (WIDE_W ? h * 8 + (lane >> 3) : lm), nOut - 1) * nIn;
 	const elem *xr[NB];
 #pragma unroll
 	for (int g = 0; g < NB; g++)
-		xr[g] = x + (size_t)min(g * 16 + m, B - 1) * nIn;
+		xr[g] = x + (size_t)min(g * 16 + lm, B - 1) * nIn;
 
 	floatx4 acc[RB][NB];
 #pragma unroll
@@ -78,19 +107,42 @@ __global__ __launch_bounds__(SK_THREADS) void skinny_kernel(const void *xv, cons
 
 	for (int st = blockIdx.y * 4 + wave; st < nsteps; st += stride) {
 		/* load j of the four lane quarters covers 64 adjacent bytes of a row */
-		const int kb = st * KSTEP + q * VEC;
+		const int kb = st * KSTEP + lq * VEC;
 		constexpr int NJ = SK_KBYTES / 64;
-		floatx4 a[RB][NJ], b[NB][NJ];
+		static_assert(NJ == 4, "the weight loads pair up: two rows halves x two vector halves");
+		floatx4 a[RB][NJ], raw[RB][NJ], b[NB][NJ];
 #pragma unroll
 		for (int j = 0; j < NJ; j++) {
 			const int k = kb + j * (4 * VEC);
 			const bool ok = k < nIn;	/* nIn % VEC == 0: a vector is all in or all out */
+			/* whole lines per eight lanes with four row blocks per wavefront; with one
+			 * the second permute costs more than it saves (9216 -> 4096 at batch 4:
+			 * 27 against 31 us) and the weights are loaded like the batch operand */
+			const int kw = WIDE_W ? st * KSTEP + ((j >> 1) * 8 + (lane & 7)) * VEC : k;
+			const bool okw = kw < nIn;
 #pragma unroll
 			for (int rb = 0; rb < RB; rb++)
-				a[rb][j] = ok ? *(const floatx4 *)(wr[rb] + k) : floatx4{ 0, 0, 0, 0 };
+				raw[rb][j] = okw ? *(const floatx4 *)(wr[rb][WIDE_W ? j & 1 : 0] + kw) : floatx4{ 0, 0, 0, 0 };
 #pragma unroll
 			for (int g = 0; g < NB; g++)
 				b[g][j] = ok ? *(const floatx4 *)(xr[g] + k) : floatx4{ 0, 0, 0, 0 };
+		}
+#pragma unroll
+		for (int j = 0; j < NJ; j++) {
+#pragma unroll
+			for (int rb = 0; rb < RB; rb++) {
+				if constexpr (WIDE_W) {
+					const floatx4 lo = skinny_permute(raw[rb][2 * (j >> 1)], wsrc4[j & 1]);
+					const floatx4 hi = skinny_permute(raw[rb][2 * (j >> 1) + 1], wsrc4[j & 1]);
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						a[rb][j][e] = upper ? hi[e] : lo[e];
+				} else
+					a[rb][j] = skinny_permute(raw[rb][j], src_lane4);
+			}
+#pragma unroll
+			for (int g = 0; g < NB; g++)
+				b[g][j] = skinny_permute(b[g][j], src_lane4);
 		}
 #pragma unroll
 		for (int j = 0; j < NJ; j++)
