@@ -168,6 +168,52 @@ __device__ __forceinline__ int conv_requant(int acc, int c_off, int c_mult, int 
 	return t < 0 ? 0 : t > 255 ? 255 : t;
 }
 
+/* Channels-last stores of a 32x32 accumulator.  Lane l holds, for position
+ * l % 32, the four planes 4 (l / 32) + 8 g + e of group g = 0..3: stored as it
+ * lies, an instruction writes 64 separate pieces of four values.
+ * v_permlane32_swap(x, y) exchanges x of lanes 32..63 with y of lanes 0..31, so
+ * after it the low lane owns both halves of x's group and the high lane both
+ * halves of y's: every lane then writes 16 bytes, in half (uint8: a quarter)
+ * as many instructions, and lanes l and l + 32 write neighbouring pieces.
+ * Every lane of the wave must take part (no divergence around the calls). */
+__device__ __forceinline__ void conv_swap32(unsigned &x, unsigned &y)
+{
+	const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+	x = r[0];
+	y = r[1];
+}
+
+/* Half types: lo[g], hi[g] = planes 0..1 and 2..3 of group g as packed pairs.
+ * yn points at the position's plane 0 of this accumulator's 32 planes; planes
+ * from `left` on do not exist (left % 8 == 0, rows 16-byte aligned). */
+__device__ __forceinline__ void conv_store_cl_half(unsigned short *yn, int left, bool valid, unsigned (&lo)[4], unsigned (&hi)[4], int lane)
+{
+#pragma unroll
+	for (int h = 0; h < 2; h++) {
+		conv_swap32(lo[2 * h], lo[2 * h + 1]);
+		conv_swap32(hi[2 * h], hi[2 * h + 1]);
+		const int m = 16 * h + 8 * (lane >> 5);
+		if (valid && m < left) {
+			uintx4 v = { lo[2 * h], hi[2 * h], lo[2 * h + 1], hi[2 * h + 1] };
+			*(uintx4 *)(yn + m) = v;
+		}
+	}
+}
+
+/* uint8: w[g] = the four codes of group g; left % 16 == 0. */
+__device__ __forceinline__ void conv_store_cl_u8(unsigned char *yn, int left, bool valid, unsigned (&w)[4], int lane)
+{
+	conv_swap32(w[0], w[1]);
+	conv_swap32(w[2], w[3]);
+	conv_swap32(w[0], w[2]);
+	conv_swap32(w[1], w[3]);
+	const int m = 16 * (lane >> 5);
+	if (valid && m < left) {
+		uintx4 v = { w[0], w[1], w[2], w[3] };
+		*(uintx4 *)(yn + m) = v;
+	}
+}
+
 /* Scalar (wave-uniform) decode of k -> offset of tap (c,kh,kw) in the image. */
 struct KTap { int koff, kh, kw; };
 
@@ -773,11 +819,13 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 		 *   sum w'x' + (128+b_off) rowsum + (128+a_off) colsum + K (128+a_off)(128+b_off) */
 		const int tail0 = (p.oHW / 8) * 8;	/* lowpadd's unclamped tail starts here */
 		const bool has_add = p.addend != 0;
+		const bool cl16 = CLO && p.Co % 16 == 0 && ((size_t)p.y & 15) == 0;	/* whole 16-byte stores (conv_store_cl_u8) */
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
 			const int nl = (wn * TN + j) * 32 + (lane & 31);
 			const int n = tile_n * BN + nl;
-			if (n >= p.N)
+			const bool valid = n < p.N;
+			if (!cl16 && !valid)
 				continue;
 			const int b = n / p.oHW, rem = n - b * p.oHW;
 			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
@@ -786,6 +834,7 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 #pragma unroll
 			for (int i = 0; i < TM; i++) {
 				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+				unsigned word[4];
 #pragma unroll
 				for (int g = 0; g < 4; g++) {
 					unsigned packed = 0;
@@ -810,9 +859,16 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 							y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
 					}
 					if constexpr (CLO) {
+						word[g] = packed;
 						/* Co % 4 == 0: the four planes are one aligned word */
-						if (m0 + 8 * g < p.Co)
+						if (!cl16 && m0 + 8 * g < p.Co)
 							*(unsigned *)(y + (size_t)n * p.Co + m0 + 8 * g) = packed;
+					}
+				}
+				if constexpr (CLO) {
+					if (cl16) {
+						const int mt = tile_m * BM + (wm * TM + i) * 32;
+						conv_store_cl_u8(y + (size_t)n * p.Co + mt, p.Co - mt, valid, word, lane);
 					}
 				}
 			}
@@ -820,16 +876,20 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 	} else {
 		/* (folded batch norm factor,) bias, optional threshold, store */
 		const bool has_scale = p.scale != 0;
+		/* half types, channels-last: whole 16-byte stores (conv_store_cl_half) */
+		const bool cl16 = CLO && sizeof(elem) == 2 && p.Co % 8 == 0 && ((size_t)p.y & 15) == 0;
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
 			const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
-			if (n >= p.N)
+			const bool valid = n < p.N;
+			if (!cl16 && !valid)
 				continue;
 			const int b = n / p.oHW, rem = n - b * p.oHW;
 			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
 #pragma unroll
 			for (int i = 0; i < TM; i++) {
 				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+				unsigned lo[4], hi[4];
 #pragma unroll
 				for (int g = 0; g < 4; g++) {
 					struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
@@ -851,8 +911,20 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 						quad.v[e] = (elem)v;
 					}
 					if constexpr (CLO) {
-						if (m0 + 8 * g < p.Co)
+						if constexpr (sizeof(elem) == 2) {
+							unsigned pair[2];
+							__builtin_memcpy(pair, &quad, 8);
+							lo[g] = pair[0];
+							hi[g] = pair[1];
+						}
+						if (!cl16 && m0 + 8 * g < p.Co)
 							*(Quad *)(y + (size_t)n * p.Co + m0 + 8 * g) = quad;
+					}
+				}
+				if constexpr (CLO && sizeof(elem) == 2) {
+					if (cl16) {
+						const int mt = tile_m * BM + (wm * TM + i) * 32;
+						conv_store_cl_half((unsigned short *)y + (size_t)n * p.Co + mt, p.Co - mt, valid, lo, hi, lane);
 					}
 				}
 			}
@@ -1017,16 +1089,20 @@ __device__ __forceinline__ void conv_wide_store_half(const ConvParams &p, floatx
 	}
 	__syncthreads();
 	const bool has_scale = p.scale != 0;
+	/* channels-last: whole 16-byte stores (conv_store_cl_half) */
+	const bool cl16 = CLO && p.Co % 8 == 0 && ((size_t)p.y & 15) == 0;
 #pragma unroll
 	for (int j = 0; j < TN; j++) {
 		const int n = tile_n * BN + (wn * TNF + j0 + j) * 32 + (lane & 31);
-		if (n >= p.N)
+		const bool valid = n < p.N;
+		if (!cl16 && !valid)
 			continue;
 		const int b = n / p.oHW, rem = n - b * p.oHW;
 		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
 #pragma unroll
 		for (int i = 0; i < TM; i++) {
 			const int m0 = tile_m * BM + (wm * TMF + i0 + i) * 32 + 4 * (lane >> 5);
+			unsigned lo[4], hi[4];
 #pragma unroll
 			for (int g = 0; g < 4; g++) {
 				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
@@ -1048,8 +1124,18 @@ __device__ __forceinline__ void conv_wide_store_half(const ConvParams &p, floatx
 					quad.v[e] = (elem)v;
 				}
 				if constexpr (CLO) {
-					if (m0 + 8 * g < p.Co)
+					unsigned pair[2];
+					__builtin_memcpy(pair, &quad, 8);
+					lo[g] = pair[0];
+					hi[g] = pair[1];
+					if (!cl16 && m0 + 8 * g < p.Co)
 						*(Quad *)(y + (size_t)n * p.Co + m0 + 8 * g) = quad;
+				}
+			}
+			if constexpr (CLO) {
+				if (cl16) {
+					const int mt = tile_m * BM + (wm * TMF + i0 + i) * 32;
+					conv_store_cl_half((unsigned short *)y + (size_t)n * p.Co + mt, p.Co - mt, valid, lo, hi, lane);
 				}
 			}
 		}
@@ -1351,11 +1437,13 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		 * output stage, lowpadd with its unclamped tail, threshold */
 		const int tail0 = (p.oHW / 8) * 8;
 		const bool has_add = p.addend != 0;
+		const bool cl16 = CLO && p.Co % 16 == 0 && ((size_t)p.y & 15) == 0;	/* whole 16-byte stores (conv_store_cl_u8) */
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
 			const int nl = (wn * TN + j) * 32 + (lane & 31);
 			const int n = tile_n * BN + nl;
-			if (n >= p.N)
+			const bool valid = n < p.N;
+			if (!cl16 && !valid)
 				continue;
 			const int b = n / p.oHW, rem = n - b * p.oHW;
 			const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
@@ -1364,6 +1452,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 #pragma unroll
 			for (int i = 0; i < TM; i++) {
 				const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+				unsigned word[4];
 #pragma unroll
 				for (int g = 0; g < 4; g++) {
 					unsigned packed = 0;
@@ -1387,8 +1476,15 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 							y[ybase + (size_t)m * p.oHW] = (unsigned char)q;
 					}
 					if constexpr (CLO) {
-						if (m0 + 8 * g < p.Co)
+						word[g] = packed;
+						if (!cl16 && m0 + 8 * g < p.Co)
 							*(unsigned *)(y + (size_t)n * p.Co + m0 + 8 * g) = packed;
+					}
+				}
+				if constexpr (CLO) {
+					if (cl16) {
+						const int mt = tile_m * BM + (wm * TM + i) * 32;
+						conv_store_cl_u8(y + (size_t)n * p.Co + mt, p.Co - mt, valid, word, lane);
 					}
 				}
 			}
