@@ -114,6 +114,7 @@ CL_CASES = [
     (5, 64, 6, 6, 132, 6, 6, 1, 1, 0, 0),
     (2, 16, 10, 10, 8, 3, 3, 1, 1, 1, 1),       # K = 144 ends inside a K-tile
     (2, 48, 5, 6, 40, 2, 3, 1, 1, 0, 1),
+    (2, 64, 9, 7, 80, 3, 3, 1, 1, 1, 1),         # 16-byte channels-last stores; the last accumulator has 16 of 32 planes
     (2, 3, 21, 19, 64, 7, 7, 2, 2, 3, 3),       # plane-major in only (generic K order), channels-last out
     (3, 3, 35, 35, 64, 11, 11, 4, 4, 2, 2),     # the image layer: also through the four-plane pixel copy
     (2, 1, 9, 12, 12, 3, 3, 1, 1, 1, 1),
