@@ -162,3 +162,21 @@ def sample_indices(n, count=4096, seed=7):
     if n <= count:
         return np.arange(n)
     return np.sort(rng(seed).choice(n, count, replace=False))
+
+
+def tensor_summary(y):
+    """What the full-size golden files keep of one module output: shape, a strided sample,
+    sum, sum of squares and max|.| of the whole tensor, and the sum of every (image, plane)
+    slice (every element is in one of them) -- float64 accumulation, stored as float32."""
+    a = np.ascontiguousarray(y, np.float32)
+    flat = a.ravel()
+    d = flat.astype(np.float64)
+    out = {"shape": np.array(a.shape, np.int64), "sample": flat[sample_indices(flat.size)],
+           "sum": np.array(d.sum()), "sumsq": np.array((d * d).sum()), "absmax": np.array(np.abs(flat).max())}
+    if a.ndim == 4:
+        out["psum"] = d.reshape(a.shape[0] * a.shape[1], -1).sum(axis=1).astype(np.float32)
+    elif a.ndim == 2:
+        out["psum"] = d.reshape(a.shape).sum(axis=1).astype(np.float32)
+    else:
+        out["psum"] = np.array([d.sum()], np.float32)
+    return out
