@@ -479,6 +479,25 @@ void thhip_linear_batched(const void *x, const void *wrow, const float *bias, vo
  * (1 or 4); 0 restores the choice by the layer's width. */
 void thhip_linear_batched_set_tuning(int row_blocks);
 
+/* thhip_linear_batched for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same arguments, same kernels and the same bits
+ * as thhip_linear_batched; the partial sums of the K slices go to a fixed array of
+ * thhip_linear_batched_noalloc_limit() bytes (8 MiB) that every GPU the library
+ * runs on holds until the process ends, instead of a buffer that grows on demand.
+ * The call allocates and frees nothing on the device or through the runtime.
+ * Returns 0, or (with a message on stderr, nothing launched) -1 for a shape
+ * thhip_linear_batched_supported refuses, -2 when a slice of 32 batch rows needs
+ * more than the array holds (K slices x rows x nOut x 4 bytes; e.g. 25088 -> 4096
+ * at batch 16 needs 2 MiB), -3 when the array's address cannot be resolved.
+ * thhip_linear_batched_noalloc_init() resolves the address for the current device
+ * ahead of the first call (THInit calls it).  Calls that overlap on one GPU share
+ * the array and race; calls on the library's stream, one after the other, do not. */
+int thhip_linear_batched_noalloc(const void *x, const void *wrow, const float *bias, void *y,
+	int B, int nIn, int nOut, int act, float thr, float val, int dtype);
+int thhip_linear_batched_noalloc_init(void);
+size_t thhip_linear_batched_noalloc_limit(void);
+
 /* Replaces nn_Threshold_updateOutput (Threshold.c:38-63), out of place or
  * in place (y == x).  alpha != 0 selects the LeakyReLU branch. */
 void thhip_threshold(const void *x, void *y, long n, float thr, float val, float alpha, int inplace, int dtype);

@@ -100,6 +100,9 @@ PROTOTYPES = {
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_linear_batched_supported": (C.c_int, [C.c_int] * 4),
     "thhip_linear_batched": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
+    "thhip_linear_batched_noalloc": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
+    "thhip_linear_batched_noalloc_init": (C.c_int, []),
+    "thhip_linear_batched_noalloc_limit": (C.c_size_t, []),
     "thhip_threshold": (None, [vp, vp, C.c_long, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]),
     "thhip_maxpool": (None, [vp, vp] + [C.c_int] * 13),
     "thhip_pool_outsize": (None, [C.c_int] * 9 + [c_ip, c_ip]),

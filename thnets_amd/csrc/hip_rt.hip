@@ -157,7 +157,8 @@ static void prof_drain(void)
 int thhip_prof_begin(int family)
 {
 	/* 1: every family; otherwise the sum of 2 << family over the families wanted */
-	if (!g_prof_on || (g_prof_on != 1 && !(g_prof_on & (2 << family))))
+	/* a negative family: a launch that must not be bracketed (no events made) */
+	if (family < 0 || !g_prof_on || (g_prof_on != 1 && !(g_prof_on & (2 << family))))
 		return -1;
 	if (g_recs.size() >= 4096)
 		prof_drain();

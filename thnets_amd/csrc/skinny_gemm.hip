@@ -24,6 +24,7 @@
  * which is as large per step as a block's weights, is then read once for 64
  * rows instead of once for 16.
  */
+#include <stdio.h>
 #include <stdlib.h>
 #include "thhip_internal.h"
 
@@ -221,13 +222,13 @@ extern "C" int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtyp
 	return B >= 1 && B <= SK_MAX_BATCH && nIn % vec == 0 && nIn >= vec && nOut >= 1;
 }
 
-template <int DT>
+template <int DT, bool SCOPED>
 static void skinny_launch(const void *x, const void *wrow, const float *bias, void *y, float *part,
 	int B, int nIn, int nOut, int rb, int groups, int ksplit, int act, float thr, float val)
 {
 	{
 		/* algorithmic bytes: W once, X once, Y once */
-		ThhipLaunchScope scope(THHIP_FAM_GEMV, (double)thhip_esize(DT) * ((double)nOut * nIn + (double)B * nIn + (double)B * nOut));
+		ThhipLaunchScope scope(SCOPED ? THHIP_FAM_GEMV : -1, (double)thhip_esize(DT) * ((double)nOut * nIn + (double)B * nIn + (double)B * nOut));
 		dim3 grid(groups, ksplit);
 		if (B <= 16 && rb == 4)
 			skinny_kernel<DT, 1, 4><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
@@ -239,7 +240,7 @@ static void skinny_launch(const void *x, const void *wrow, const float *bias, vo
 			skinny_kernel<DT, 2, 1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
 	}
 	{
-		ThhipLaunchScope scope(THHIP_FAM_OTHER, 4.0 * (ksplit + 1.0) * B * nOut);
+		ThhipLaunchScope scope(SCOPED ? THHIP_FAM_OTHER : -1, 4.0 * (ksplit + 1.0) * B * nOut);
 		long total = (long)B * nOut;
 		long blocks = (total + 255) / 256;
 		skinny_finish_kernel<DT><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(part, bias, y, B, nOut,
@@ -256,6 +257,34 @@ extern "C" void thhip_linear_batched_set_tuning(int row_blocks)
 	g_skinny_rb = row_blocks;
 }
 
+/* Row blocks per wavefront, row groups and K split of one launch (B <= 32). */
+struct skinny_plan { int rb, groups, ksplit; };
+static struct skinny_plan skinny_choose(int B, int nIn, int nOut, int dtype)
+{
+	struct skinny_plan p;
+	/* four row blocks per wavefront for wide layers and batches that fill most of
+	 * the 16 MFMA columns (measured: 12 % on 25088 -> 4096 at batch 16; at batch 4
+	 * the unused columns re-read their rows from L1 and one block is faster) */
+	p.rb = nOut >= 1024 && B > 8 ? 4 : 1;
+	if (g_skinny_rb)
+		p.rb = g_skinny_rb;
+	p.groups = (nOut + 16 * p.rb - 1) / (16 * p.rb);
+	const int kstep = SK_KBYTES / thhip_esize(dtype);
+	const int nsteps = (nIn + kstep - 1) / kstep;
+	/* aim at ~4096 wavefronts, ~2048 with four row blocks each (two per SIMD:
+	 * 25088 -> 4096 at batch 16 runs 4 % (fp32) and 8 % (fp16) faster than with
+	 * four, and 16-27 % faster than with eight or sixteen), at least two K-steps
+	 * per wavefront */
+	p.ksplit = ((p.rb == 4 ? 512 : 1024) + p.groups - 1) / p.groups;
+	if (p.ksplit > nsteps / 8)
+		p.ksplit = nsteps / 8;
+	if (p.ksplit < 1)
+		p.ksplit = 1;
+	if (p.ksplit > 64)
+		p.ksplit = 64;
+	return p;
+}
+
 extern "C" void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
 	int B, int nIn, int nOut, int act, float thr, float val, int dtype)
 {
@@ -268,28 +297,88 @@ extern "C" void thhip_linear_batched(const void *x, const void *wrow, const floa
 				B - b0 < 32 ? B - b0 : 32, nIn, nOut, act, thr, val, dtype);
 		return;
 	}
-	/* four row blocks per wavefront for wide layers and batches that fill most of
-	 * the 16 MFMA columns (measured: 12 % on 25088 -> 4096 at batch 16; at batch 4
-	 * the unused columns re-read their rows from L1 and one block is faster) */
-	int rb = nOut >= 1024 && B > 8 ? 4 : 1;
-	if (g_skinny_rb)
-		rb = g_skinny_rb;
-	const int groups = (nOut + 16 * rb - 1) / (16 * rb);
-	const int kstep = SK_KBYTES / thhip_esize(dtype);
-	const int nsteps = (nIn + kstep - 1) / kstep;
-	/* aim at ~4096 wavefronts, ~2048 with four row blocks each (two per SIMD:
-	 * 25088 -> 4096 at batch 16 runs 4 % (fp32) and 8 % (fp16) faster than with
-	 * four, and 16-27 % faster than with eight or sixteen), at least two K-steps
-	 * per wavefront */
-	int ksplit = ((rb == 4 ? 512 : 1024) + groups - 1) / groups;
-	if (ksplit > nsteps / 8)
-		ksplit = nsteps / 8;
-	if (ksplit < 1)
-		ksplit = 1;
-	if (ksplit > 64)
-		ksplit = 64;
-	float *part = skinny_scratch((size_t)ksplit * B * nOut * sizeof(float));
-	THHIP_DISPATCH_FLOAT(dtype, skinny_launch<DT>(x, wrow, bias, y, part, B, nIn, nOut, rb, groups, ksplit, act, thr, val));
+	const struct skinny_plan p = skinny_choose(B, nIn, nOut, dtype);
+	float *part = skinny_scratch((size_t)p.ksplit * B * nOut * sizeof(float));
+	THHIP_DISPATCH_FLOAT(dtype, (skinny_launch<DT, true>(x, wrow, bias, y, part, B, nIn, nOut, p.rb, p.groups, p.ksplit, act, thr, val)));
+}
+
+/*
+ * The same product for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid it): the partial sums
+ * of the K slices go to a fixed array in device memory instead of a buffer that
+ * grows on demand.  Every GPU the library runs on holds its own copy of the
+ * array at its own address until the process ends; the address is looked up
+ * once per device (at THInit for the current device, else at the first call)
+ * and only that pointer is ever handed to a kernel.  The kernels write every
+ * partial sum they later read, so nothing has to be cleared between calls, but
+ * two calls that overlap on one GPU (other streams, other threads) race on the
+ * array.
+ */
+#define SK_STATIC_BYTES (8u << 20)
+#define SK_STATIC_MAXDEV 16
+static __device__ __align__(256) float scratch[SK_STATIC_BYTES / sizeof(float)];
+static float *g_static_part[SK_STATIC_MAXDEV];
+
+static float *skinny_static_part(void)
+{
+	int dev = -1;
+	thhip_stream();		/* first use: selects the device and makes the stream */
+	if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= SK_STATIC_MAXDEV)
+		return 0;
+	if (!g_static_part[dev]) {
+		float *p = 0;
+		const hipError_t rc = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+		if (rc != hipSuccess || !p) {
+			fprintf(stderr, "thhip_linear_batched_noalloc: hipGetSymbolAddress failed on device %d: %s\n", dev,
+				hipGetErrorString(rc));
+			return 0;
+		}
+		g_static_part[dev] = p;
+	}
+	return g_static_part[dev];
+}
+
+extern "C" int thhip_linear_batched_noalloc_init(void)
+{
+	return skinny_static_part() ? 0 : -1;
+}
+
+extern "C" size_t thhip_linear_batched_noalloc_limit(void)
+{
+	return SK_STATIC_BYTES;
+}
+
+extern "C" int thhip_linear_batched_noalloc(const void *x, const void *wrow, const float *bias, void *y,
+	int B, int nIn, int nOut, int act, float thr, float val, int dtype)
+{
+	if (!thhip_linear_batched_supported(B, nIn, nOut, dtype)) {
+		fprintf(stderr, "thhip_linear_batched_noalloc: unsupported shape B=%d nIn=%d nOut=%d dtype=%d\n", B, nIn, nOut, dtype);
+		return -1;
+	}
+	/* every slice of 32 batch rows must fit: check before anything is launched */
+	for (int b0 = 0; b0 < B; b0 += 32) {
+		const int bs = B - b0 < 32 ? B - b0 : 32;
+		const struct skinny_plan p = skinny_choose(bs, nIn, nOut, dtype);
+		const size_t need = (size_t)p.ksplit * bs * nOut * sizeof(float);
+		if (need > SK_STATIC_BYTES) {
+			fprintf(stderr, "thhip_linear_batched_noalloc: B=%d nIn=%d nOut=%d needs %zu bytes of partial sums "
+				"(%d K slices x %d rows x %d outputs), the fixed array holds %u; use thhip_linear_batched\n",
+				B, nIn, nOut, need, p.ksplit, bs, nOut, (unsigned)SK_STATIC_BYTES);
+			return -2;
+		}
+	}
+	float *part = skinny_static_part();
+	if (!part)
+		return -3;
+	const size_t esize = thhip_esize(dtype);
+	for (int b0 = 0; b0 < B; b0 += 32) {
+		const int bs = B - b0 < 32 ? B - b0 : 32;
+		const struct skinny_plan p = skinny_choose(bs, nIn, nOut, dtype);
+		const void *xs = (const char *)x + (size_t)b0 * nIn * esize;
+		void *ys = (char *)y + (size_t)b0 * nOut * esize;
+		THHIP_DISPATCH_FLOAT(dtype, (skinny_launch<DT, false>(xs, wrow, bias, ys, part, bs, nIn, nOut, p.rb, p.groups, p.ksplit, act, thr, val)));
+	}
+	return 0;
 }
 
 /* ------------------------------------------------------------------ */

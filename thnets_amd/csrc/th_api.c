@@ -26,6 +26,9 @@ void THInit(void)
 	 * no GPU is visible */
 	if (thhip_device_count() < 1)
 		THError("thnets HIP engine: no AMD GPU visible; this library has no CPU fallback");
+	/* the fixed partial-sum array of thhip_linear_batched_noalloc: look its address up now */
+	if (thhip_linear_batched_noalloc_init())
+		THError("thnets HIP engine: the fixed device array of thhip_linear_batched_noalloc could not be resolved");
 }
 
 static THNETWORK *create_engine_network(THNETWORK *net, int lowp, float range)
