@@ -33,6 +33,24 @@ extern "C" {
 /* 1. thnets ABI                                                       */
 /* ------------------------------------------------------------------ */
 
+#ifdef THNETS_IN_TREE
+/* Built inside the thnets tree (its Makefile's HIP=1 option): structures, module
+ * types, tensor helpers and the high level prototypes come from the tree's own
+ * thnets.h, so the engine sees exactly the layout every other translation unit of
+ * libthnets sees (all of them must agree on -DLOWP / -DOPENCL, thnets.h:117-119,
+ * 300-303).  The tree appends ENGINE_HIP, ENGINE_HIPLOWP to the enum at thnets.h:401
+ * and defines THNETS_HAS_ENGINE_HIP; against an unpatched header the two values are
+ * declared here. */
+#include "thnets.h"
+#ifndef THNETS_HAS_ENGINE_HIP
+enum { ENGINE_HIP = ENGINE_LOWP + 1, ENGINE_HIPLOWP = ENGINE_LOWP + 2 };
+#endif
+#ifndef MAXMODULEINPUTS
+#define MAXMODULEINPUTS 16	/* int inputs[16], thnets.h:310 */
+#endif
+extern int th_debug, th_profile, th_minmax;
+extern double th_convtot, th_convflops;
+#else
 /* thnets.h:16-22 */
 enum therror {
 	ERR_OPENFILE = -1,
@@ -43,13 +61,15 @@ enum therror {
 };
 
 /* thnets.h:104-108.  mustfree: 0 borrowed, 1 free(), 2 cudaFree (unused
- * here), 3 OpenCL (unused here), 4 = device memory owned by this engine. */
+ * here), 3 OpenCL (unused here), 4..7 = device memory owned by this engine,
+ * holding elements of type (mustfree - 4) of enum thhip_dtype: a device tensor
+ * says what it holds, so a tensor made for one network type is refused by
+ * another instead of being read with the wrong element size. */
 typedef struct THFloatStorage {
 	float *data;
 	int nref, mustfree;
 } THFloatStorage;
 
-#define TH_MUSTFREE_HIP 4
 
 /* thnets.h:110-120 (default build: no sub/mult members). */
 typedef struct THFloatTensor {
@@ -292,6 +312,13 @@ int THLastError(void);
 extern int th_debug, th_profile, th_minmax;
 extern double th_convtot, th_convflops;
 
+#endif /* THNETS_IN_TREE */
+
+#define TH_MUSTFREE_HIP 4
+#define TH_MUSTFREE_HIP_OF(dtype) (TH_MUSTFREE_HIP + (dtype))
+#define TH_IS_HIP_STORAGE(mustfree) ((mustfree) >= TH_MUSTFREE_HIP && (mustfree) <= TH_MUSTFREE_HIP + 3)
+#define TH_HIP_STORAGE_DTYPE(mustfree) ((mustfree) - TH_MUSTFREE_HIP)
+
 /* New: the MI355X engine.  Same shape as THCreateCudaNetwork
  * (thapi.c:730-742): returns a new THNETWORK whose modules own device
  * copies of every weight; the source network may be freed afterwards.
@@ -497,6 +524,12 @@ int thhip_linear_batched_noalloc(const void *x, const void *wrow, const float *b
 	int B, int nIn, int nOut, int act, float thr, float val, int dtype);
 int thhip_linear_batched_noalloc_init(void);
 size_t thhip_linear_batched_noalloc_limit(void);
+
+/* Replaces FindMinMax (thapi.c:141-154), which the executor prints after every
+ * module when th_minmax is set (thapi.c:197-202): smallest and largest of n
+ * elements of the given type on the device (codes as numbers for uint8),
+ * +inf / -inf for n = 0, NaNs skipped as the reference's comparisons skip them. */
+void thhip_minmax(const void *x, long n, int dtype, float *min_out, float *max_out);
 
 /* Replaces nn_Threshold_updateOutput (Threshold.c:38-63), out of place or
  * in place (y == x).  alpha != 0 selects the LeakyReLU branch. */

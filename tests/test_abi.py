@@ -84,6 +84,26 @@ def test_golden_layout_is_current_when_reference_is_mounted(tmp_path):
     assert mod.probe(ref, ["-DLOWP"]) == GOLDEN["lowp"]
 
 
+@pytest.mark.parametrize("flags", [[], ["-DLOWP"]])
+def test_engine_compiles_against_the_reference_header(tmp_path, flags):
+    """With -DTHNETS_IN_TREE the engine's host code takes every structure, module type and
+    tensor helper from the reference's own thnets.h (the way its objects are linked into
+    libthnets with the Makefile's HIP=1 option) instead of this repository's mirror: it must
+    compile, warning-free, against the unmodified header, in the default and the -DLOWP
+    layout; so must a kernel file's host side."""
+    ref = "/root/reference"
+    if not os.path.exists(os.path.join(ref, "thnets.h")):
+        pytest.skip("reference tree not mounted")
+    csrc = os.path.join(ROOT, "thnets_amd", "csrc")
+    r = subprocess.run(["gcc", "-std=gnu11", "-Wall", "-Werror", "-Wno-unused-function", "-c", "-DTHNETS_IN_TREE"] + flags +
+                       ["-I", ref, os.path.join(csrc, "th_engine.c"), "-o", str(tmp_path / "th_engine.o")],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    # the object refers to the reference's tensor helpers and to the kernel launchers only
+    syms = subprocess.check_output(["nm", "-u", str(tmp_path / "th_engine.o")]).decode()
+    assert "THFloatTensor_set" in syms and "thhip_conv2d_layout" in syms
+
+
 def declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)

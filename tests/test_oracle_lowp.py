@@ -142,6 +142,66 @@ def test_mm_params_hand_computed(oracle):
     assert oracle.lowp_bias_addend(0, 2.0, -60.0, 7.96875) == round(-60.0 * 7.96875)
 
 
+def test_mm_params_more_hand_cases(oracle):
+    """lowp_basic.c:309-320 with three different multipliers, so that swapping any two of them,
+    another logarithm or another rounding shows.  Every expected value is worked out by hand
+    below from the reference's expressions:
+        scaling = wm * im / om (float);  shift = roundf(log(scaling) / log(2)) + 10, where the
+        double quotient is converted to float before roundf rounds it half away from zero;
+        c_mult = roundf(2^shift / scaling);  c_off = roundf(-osub * wm * im);
+        a_off = roundf(wsub * wm);  b_off = roundf(isub * im)."""
+    # scaling = 100 * 4 / 20 = 20 (500 with im and om swapped, 0.8 with wm and om swapped);
+    # log2 20 = 4.32 -> 4, shift 14; 16384 / 20 = 819.2 -> 819; c_off = 3 * 100 * 4 = 1200;
+    # a_off = roundf(-37) = -37; b_off = roundf(-5.2) = -5
+    assert oracle.lowp_mm_params(100.0, -0.37, 4.0, -1.3, 20.0, -3.0) == dict(
+        a_off=-37, b_off=-5, c_off=1200, c_mult=819, c_shift=14)
+    # either side of log2 = 4.5 (2^4.5 = 22.627): scaling = 45.2 * 2 / 4 = 22.6, log2 = 4.4983 -> 4,
+    # shift 14, 16384 / 22.6 = 724.96 -> 725;  45.4 * 2 / 4 = 22.7, log2 = 4.5046 -> 5, shift 15,
+    # 32768 / 22.7 = 1443.5 -> 1444.  A positive osub gives a negative c_off: -2.5 * 90.4 = -226,
+    # -2.5 * 90.8 = -227.  a_off = roundf(-11.3) = -11 (-11.35 -> -11), b_off = roundf(1.0) = 1
+    assert oracle.lowp_mm_params(45.2, -0.25, 2.0, 0.5, 4.0, 2.5) == dict(
+        a_off=-11, b_off=1, c_off=-226, c_mult=725, c_shift=14)
+    assert oracle.lowp_mm_params(45.4, -0.25, 2.0, 0.5, 4.0, 2.5) == dict(
+        a_off=-11, b_off=1, c_off=-227, c_mult=1444, c_shift=15)
+    # scaling = 0x1.6a09dcp+8 = 362.03851318359375, five float steps below 2^8.5: log(s)/log(2) =
+    # 8.49999936726 in double, 8.49999904633 as a float, below one half -> 8, shift 18,
+    # 2^18 / 362.0385 = 724.08 -> 724.  With logf(s) / logf(2) the quotient is 8.5f -> 9 -> shift 19.
+    s = float.fromhex("0x1.6a09dcp+8")
+    assert oracle.lowp_mm_params(2 * s, -1.0, 2.0, -3.0, 4.0, -8.0) == dict(
+        a_off=-724, b_off=-6, c_off=11585, c_mult=724, c_shift=18)     # 8 * 4 s = 11585.23 -> 11585
+    # scaling = 0x1.6a09e6p+7 = 181.0193328857422, the float just below 2^7.5: the double quotient
+    # 7.4999999753 becomes 7.5f on its way into roundf -> 8 (half away from zero), shift 18,
+    # 2^18 / 181.01933 = 1448.15 -> 1448.  round() on the double, or logf (7.4999995f), gives 7.
+    s = float.fromhex("0x1.6a09e6p+7")
+    assert oracle.lowp_mm_params(2 * s, -1.0, 2.0, -3.0, 4.0, -8.0) == dict(
+        a_off=-362, b_off=-6, c_off=5793, c_mult=1448, c_shift=18)     # 8 * 4 s = 5792.62 -> 5793
+    # a wide output range: om = 255 / 128, osub = -64; wm * im = 3187.5 * 63.75 = 203203.125 (exact in
+    # float), scaling = 203203.125 * 128 / 255 = 102000, log2 = 16.638 -> 17, shift 27,
+    # 2^27 / 102000 = 1315.86 -> 1316; c_off = 64 * 203203.125 = 13005000; a_off = roundf(-127.5) = -128,
+    # b_off = roundf(-127.5) = -128 (both half away from zero)
+    assert oracle.lowp_mm_params(3187.5, -0.04, 63.75, -2.0, 1.9921875, -64.0) == dict(
+        a_off=-128, b_off=-128, c_off=13005000, c_mult=1316, c_shift=27)
+    # positive half-way offsets round up, not to even: a_off = roundf(25.5) = 26, b_off = roundf(2.5) = 3;
+    # scaling = 51 * 5 / 7.96875 = 32 exactly, log2 = 5, shift 15, c_mult = 1024, c_off = 16 * 255 = 4080
+    assert oracle.lowp_mm_params(51.0, 0.5, 5.0, 0.5, 7.96875, -16.0) == dict(
+        a_off=26, b_off=3, c_off=4080, c_mult=1024, c_shift=15)
+
+
+def test_bias_addend_rounds_each_term_half_away_from_zero(oracle):
+    """lowp_SpatialConvolution.c:111-120: addend = roundf(code * (om / bm)) + roundf(bsub * om), two
+    separate roundings, each half away from zero."""
+    # om / bm = 8 / 16 = 0.5: 5 * 0.5 = 2.5 -> 3 (to even: 2); bsub * om = -1.25 -> -1; 3 - 1 = 2
+    # (rounding the sum 1.25 once would give 1)
+    assert oracle.lowp_bias_addend(5, 16.0, -0.15625, 8.0) == 2
+    # 7 * 0.5 = 3.5 -> 4; 0.3125 * 8 = 2.5 -> 3 (to even: 2); 4 + 3 = 7 (the sum 6.0 rounded once: 6)
+    assert oracle.lowp_bias_addend(7, 16.0, 0.3125, 8.0) == 7
+    # 1 * 0.5 = 0.5 -> 1 (truncation: 0); -0.3125 * 8 = -2.5 -> -3 (to even or truncated: -2); 1 - 3 = -2
+    assert oracle.lowp_bias_addend(1, 16.0, -0.3125, 8.0) == -2
+    # a large factor: om / bm = 7.96875 / 3 = 2.65625 exactly; 200 * 2.65625 = 531.25 -> 531;
+    # -1.7 * 7.96875 = -13.546875 -> -14; 531 - 14 = 517
+    assert oracle.lowp_bias_addend(200, 3.0, -1.7, 7.96875) == 517
+
+
 def test_lowpadd_tail_is_not_clamped_below(oracle):
     x = np.array([0, 1, 2, 3, 250, 251, 252, 253, 5, 200, 0], np.uint8)   # 8 + 3
     y = oracle.lowp_add(x, -3)

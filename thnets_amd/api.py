@@ -103,6 +103,7 @@ PROTOTYPES = {
     "thhip_linear_batched_noalloc": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_linear_batched_noalloc_init": (C.c_int, []),
     "thhip_linear_batched_noalloc_limit": (C.c_size_t, []),
+    "thhip_minmax": (None, [vp, C.c_long, C.c_int, c_fp, c_fp]),
     "thhip_threshold": (None, [vp, vp, C.c_long, C.c_float, C.c_float, C.c_float, C.c_int, C.c_int]),
     "thhip_maxpool": (None, [vp, vp] + [C.c_int] * 13),
     "thhip_pool_outsize": (None, [C.c_int] * 9 + [c_ip, c_ip]),

@@ -1000,6 +1000,14 @@ extern "C" void thhip_rgb2code(unsigned char *dst, const unsigned char *src, int
 {
 	int sub[3];
 	float mult[3], mn = 1e30, mx = -1e30, tmult;
+	/* the kernel reads three bytes of every pixel: the source must hold
+	 * stride * (height - 1) + 3 * width bytes, which a copy of `height` rows of
+	 * `stride` bytes only does for stride >= 3 * width.  (The reference's loader
+	 * reads past its host image for narrower rows; a device read out of bounds
+	 * can fault.) */
+	if (stride < 3 * width)
+		THError("thhip_rgb2code: row stride %d is less than 3 * width %d: the uint8 image loader takes three-plane "
+			"images only (lowp_basic.c:82-131)", stride, width);
 	for (int i = 0; i < 3; i++) {
 		if (-mean[i] / std[i] < mn)
 			mn = -mean[i] / std[i];
@@ -1019,6 +1027,72 @@ extern "C" void thhip_rgb2code(unsigned char *dst, const unsigned char *src, int
 	}
 	*mult_out = tmult;
 	*sub_out = mn;
+}
+
+/* ---------------- smallest and largest element (FindMinMax, thapi.c:141-154) ---------------- */
+
+template <int DT>
+__global__ void minmax_any_kernel(const void *x, long n, float *part)
+{
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	float mn = INFINITY, mx = -INFINITY;	/* THInf / -THInf; comparisons skip NaN like the reference's */
+	for (; i < n; i += step) {
+		float v;
+		if constexpr (DT == THHIP_U8)
+			v = (float)((const unsigned char *)x)[i];
+		else
+			v = ThhipElem<DT>::ld(x, i);
+		mn = v < mn ? v : mn;
+		mx = v > mx ? v : mx;
+	}
+	for (int off = 32; off > 0; off >>= 1) {
+		const float a = __shfl_xor(mn, off, 64), b = __shfl_xor(mx, off, 64);
+		mn = a < mn ? a : mn;
+		mx = b > mx ? b : mx;
+	}
+	__shared__ float smn[4], smx[4];
+	if ((threadIdx.x & 63) == 0) {
+		smn[threadIdx.x >> 6] = mn;
+		smx[threadIdx.x >> 6] = mx;
+	}
+	__syncthreads();
+	if (threadIdx.x == 0) {
+		for (int w = 1; w < 4; w++) {
+			mn = smn[w] < mn ? smn[w] : mn;
+			mx = smx[w] > mx ? smx[w] : mx;
+		}
+		part[2 * blockIdx.x] = mn;
+		part[2 * blockIdx.x + 1] = mx;
+	}
+}
+
+extern "C" void thhip_minmax(const void *x, long n, int dtype, float *min_out, float *max_out)
+{
+	float mn = INFINITY, mx = -INFINITY;
+	if (n > 0) {
+		long blocks = (n + 1023) / 1024;
+		if (blocks > 1024)
+			blocks = 1024;
+		float *d = (float *)thhip_malloc(sizeof(float) * 2 * blocks);
+		float *h = (float *)malloc(sizeof(float) * 2 * blocks);
+		{
+			ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)thhip_esize(dtype) * n);
+			if (dtype == THHIP_U8)
+				minmax_any_kernel<THHIP_U8><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(x, n, d);
+			else
+				THHIP_DISPATCH_FLOAT(dtype, (minmax_any_kernel<DT><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>(x, n, d)));
+		}
+		thhip_memcpy_d2h(h, d, sizeof(float) * 2 * blocks);
+		for (long b = 0; b < blocks; b++) {
+			mn = h[2 * b] < mn ? h[2 * b] : mn;
+			mx = h[2 * b + 1] > mx ? h[2 * b + 1] : mx;
+		}
+		free(h);
+		thhip_free(d);
+	}
+	*min_out = mn;
+	*max_out = mx;
 }
 
 /* ---------------- uint8 quantise / de-quantise (lowp/lowp_basic.c:5-58) ---------------- */

@@ -97,7 +97,7 @@ static THFloatTensor *device_tensor_like(THFloatTensor *t, int dtype)
 		}
 		n->storage = malloc(sizeof(*n->storage));
 		n->storage->nref = 1;
-		n->storage->mustfree = TH_MUSTFREE_HIP;
+		n->storage->mustfree = TH_MUSTFREE_HIP_OF(dtype);
 		n->storage->data = thhip_malloc((size_t)THFloatTensor_nElement(t) * (dtype == THHIP_F32 ? 4 : dtype == THHIP_U8 ? 1 : 2));
 	}
 	return n;
@@ -300,11 +300,17 @@ int THProcessImages(THNETWORK *network, unsigned char **images, int batchsize, i
 		cp = 1;	/* thapi.c:458-459 */
 	if (engine == ENGINE_HIPLOWP) {
 		/* thapi.c:485-487, 551-558: Lowp_LoadImages (always three planes, always
-		 * 4-D), forward, de-quantise */
+		 * 4-D), forward, de-quantise.  It reads three bytes per pixel whatever the
+		 * stride: with stride < 3 * width (what the float engines take as one
+		 * plane, thapi.c:458-459) the reference reads past the image; here that
+		 * would be a device read past the staging copy, so it is refused. */
+		if (cp != 3)
+			THError("THProcessImages: the uint8 engine takes three-plane images only (stride %d < 3 * width %d)",
+				stride, width);
 		THFloatTensor *q = THFloatTensor_new();
 		q->storage = malloc(sizeof(*q->storage));
 		q->storage->nref = 1;
-		q->storage->mustfree = TH_MUSTFREE_HIP;
+		q->storage->mustfree = TH_MUSTFREE_HIP_OF(THHIP_U8);
 		q->storage->data = thhip_malloc((size_t)batchsize * 3 * width * height);
 		unsigned char *staging = thhip_malloc((size_t)stride * height);
 		for (int i = 0; i < batchsize; i++) {
@@ -330,7 +336,7 @@ int THProcessImages(THNETWORK *network, unsigned char **images, int batchsize, i
 	THFloatTensor *t = THFloatTensor_new();
 	t->storage = malloc(sizeof(*t->storage));
 	t->storage->nref = 1;
-	t->storage->mustfree = TH_MUSTFREE_HIP;
+	t->storage->mustfree = TH_MUSTFREE_HIP_OF(dt);
 	t->storage->data = thhip_malloc((size_t)batchsize * cp * width * height * esz);
 	unsigned char *staging = thhip_malloc((size_t)stride * height);
 	for (int i = 0; i < batchsize; i++) {

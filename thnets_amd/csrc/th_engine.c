@@ -68,12 +68,21 @@ struct hipmod *hipmod_of(struct module *m)
 	return &hn->hm[m - hn->pub.modules];
 }
 
+static const char *thhip_dtype_name(int dtype)
+{
+	return dtype == THHIP_F32 ? "fp32" : dtype == THHIP_F16 ? "fp16" : dtype == THHIP_BF16 ? "bf16" : "uint8";
+}
+
 void *thhip_tensor_ptr(THFloatTensor *t, int dtype)
 {
 	if (!t || !t->storage || !t->storage->data)
 		THError("HIP engine: tensor without storage");
-	if (t->storage->mustfree != TH_MUSTFREE_HIP)
+	if (!TH_IS_HIP_STORAGE(t->storage->mustfree))
 		THError("HIP engine: module input is not a device tensor (create it with THHipTensor_newFromFloatTensor)");
+	if (TH_HIP_STORAGE_DTYPE(t->storage->mustfree) != dtype)
+		THError("HIP engine: device tensor holds %s elements, %s expected (it was made under another THHipHalfFloat "
+			"setting or for another network type)", thhip_dtype_name(TH_HIP_STORAGE_DTYPE(t->storage->mustfree)),
+			thhip_dtype_name(dtype));
 	return (char *)t->storage->data + t->storageOffset * esize_of(dtype);
 }
 
@@ -91,11 +100,11 @@ static void *out_resize(struct module *m, int dtype, int nd, const long *size)
 	 * has it (range / 2 * 255 / range rounds to 128): the convolution kernel that
 	 * loads straight into LDS fetches its padding from there */
 	const size_t tail = dtype == THHIP_U8 ? TH_U8_TAIL : 0;
-	if (!o->storage || o->storage->mustfree != TH_MUSTFREE_HIP || hm->cap < bytes + tail || !hm->owns_output) {
+	if (!o->storage || !TH_IS_HIP_STORAGE(o->storage->mustfree) || hm->cap < bytes + tail || !hm->owns_output) {
 		THFloatStorage *s = malloc(sizeof(*s));
 		s->data = thhip_malloc(bytes + tail);
 		s->nref = 1;
-		s->mustfree = TH_MUSTFREE_HIP;
+		s->mustfree = TH_MUSTFREE_HIP_OF(dtype);
 		if (o->storage)
 			thhip_storage_release(o->storage);
 		o->storage = s;
@@ -107,6 +116,7 @@ static void *out_resize(struct module *m, int dtype, int nd, const long *size)
 		thhip_memset((char *)o->storage->data + bytes, TH_U8_TAIL_CODE, tail);
 		hm->tail_at = bytes;
 	}
+	o->storage->mustfree = TH_MUSTFREE_HIP_OF(dtype);
 	o->storageOffset = 0;
 	o->nDimension = nd;
 	for (int i = nd - 1; i >= 0; i--) {
@@ -609,7 +619,7 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 		thhip_conv2d_u8_layout_tail(x, hm->wpacked, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
 			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
 			hm->fused_act, thr, val, x_cl, hm->out_cl,
-			x_cl == 1 && zero == TH_U8_TAIL_CODE && in->storage && in->storage->mustfree == TH_MUSTFREE_HIP &&
+			x_cl == 1 && zero == TH_U8_TAIL_CODE && in->storage && TH_IS_HIP_STORAGE(in->storage->mustfree) &&
 			in->storageOffset == 0 ? TH_U8_TAIL : 0);
 	hn->cur_cl = hm->out_cl;
 	hn->cur_mult = om;
@@ -727,10 +737,13 @@ static int is_conv_type(int type)
 /* forward(), thapi.c:158-235, without the per-layer frees; with th_profile
  * the stream is drained around each module the way the OpenCL engine calls
  * clFinish (thapi.c:213-216), so the printed seconds are kernel time. */
+static int g_run_depth;	/* 1 while the top-level module list runs, more inside containers */
+
 static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
 {
 	double t = 0;
 	((struct hipnet *)net)->cur_cl = 0;	/* inputs arrive in the reference's plane-major order */
+	g_run_depth++;
 	for (int i = 0; i < net->nelem; i++) {
 		struct module *m = &net->modules[i];
 		if (th_profile) {
@@ -763,6 +776,19 @@ static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
 			in = m->updateOutput(m, (THFloatTensor *)&table);
 		} else
 			in = m->updateOutput(m, in);
+		/* thapi.c:197-202: the executor (not the containers) prints every module
+		 * output's range.  The uint8 engine prints the range of the values its
+		 * codes stand for (the reference reads the code bytes as floats there). */
+		if (th_minmax && g_run_depth == 1 && m->type != MT_ConcatTable && in && in->storage) {
+			struct hipnet *hn = (struct hipnet *)net;
+			float mn, mx;
+			thhip_minmax(thhip_tensor_ptr(in, hn->dtype), THFloatTensor_nElement(in), hn->dtype, &mn, &mx);
+			if (hn->dtype == THHIP_U8 && hn->cur_mult != 0) {
+				mn = mn * (1 / hn->cur_mult) + hn->cur_sub;	/* lowp_basic.c:52-55 */
+				mx = mx * (1 / hn->cur_mult) + hn->cur_sub;
+			}
+			printf("Layer %d output: min=%f, max=%f\n", i + 1, mn, mx);
+		}
 		if (th_profile) {
 			thhip_sync();
 			t = seconds_now() - t;
@@ -779,6 +805,7 @@ static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
 			printf("%d) %d %d %ld %ld %ld %ld\n", i + 1, m->type, in->nDimension, in->size[0], in->size[1],
 				in->size[2], in->size[3]);
 	}
+	g_run_depth--;
 	return in;
 }
 
@@ -803,7 +830,7 @@ static THFloatTensor *contiguous_host_floats(THFloatTensor *t, const char *what,
 {
 	if (!t || !t->storage || !t->storage->data)
 		return 0;
-	if (t->storage->mustfree == TH_MUSTFREE_HIP)
+	if (TH_IS_HIP_STORAGE(t->storage->mustfree))
 		THError("%s already lives on the device: pass the host network to THCreateHipNetwork", what);
 	long stride = 1;
 	for (int i = t->nDimension - 1; i >= 0; i--) {
@@ -1004,6 +1031,7 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 		    !contiguous_host_floats(bn->running_var, "running_var", -1))
 			THError("SpatialBatchNormalization needs running_mean and running_var");
 		const long C = THFloatTensor_nElement(bn->running_mean);
+		contiguous_host_floats(bn->running_var, "running_var", C);	/* one variance per mean */
 		float *invstd = malloc(sizeof(float) * C);
 		const float *var = THFloatTensor_data(bn->running_var);
 		for (long f = 0; f < C; f++)
@@ -1164,8 +1192,8 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			continue;
 		struct SpatialBatchNormalization *bn = &sb->SpatialBatchNormalization;
 		const int Co = m->SpatialConvolution.nOutputPlane;
-		if (THFloatTensor_nElement(bn->running_mean) != Co)
-			continue;	/* the mismatch is reported when the network runs */
+		if (THFloatTensor_nElement(bn->running_mean) != Co || THFloatTensor_nElement(bn->running_var) != Co)
+			continue;	/* the mismatch is reported by the module's own conversion or when the network runs */
 		const float *mean = THFloatTensor_data(bn->running_mean), *var = THFloatTensor_data(bn->running_var);
 		const float *w = contiguous_host_floats(bn->weight, "batchnorm weight", Co) ? THFloatTensor_data(bn->weight) : 0;
 		const float *b = contiguous_host_floats(bn->bias, "batchnorm bias", Co) ? THFloatTensor_data(bn->bias) : 0;

@@ -277,10 +277,13 @@ static void rd_tensor(struct t7doc *d, struct t7value *v, int scalar, int depth)
 			t7_fail(d, ERR_CORRUPTED);
 			return;
 		}
+		long span;
 		if (v->size[i] == 0)
 			empty = 1;
-		else
-			last += (v->size[i] - 1) * v->stride[i];
+		else if (__builtin_mul_overflow(v->size[i] - 1, v->stride[i], &span) || __builtin_add_overflow(last, span, &last)) {
+			t7_fail(d, ERR_CORRUPTED);	/* sizes and strides straight from the file: the sum must not wrap */
+			return;
+		}
 	}
 	if (!empty && (v->offset < 0 || last >= st->nelem)) {
 		t7_fail(d, ERR_CORRUPTED);
@@ -561,7 +564,10 @@ static void load_conv(struct module *m, const struct t7value *o)
 	THFloatTensor *w = c->weight;
 	if (!w->storage || (w->nDimension != 2 && w->nDimension != 4))
 		THError("%s: weight must be a 2-D or 4-D tensor", o->string);
-	if (w->nDimension == 4) {	/* [Co][Ci][kH][kW] is read as [Co][Ci*kH*kW] */
+	if (w->nDimension == 4) {	/* [Co][Ci][kH][kW] is read as [Co][Ci*kH*kW]: only when it lies that way */
+		if (w->stride[3] != 1 || w->stride[2] != w->size[3] || w->stride[1] != w->size[2] * w->size[3] ||
+		    w->stride[0] != w->size[1] * w->size[2] * w->size[3])
+			THError("%s: 4-D weight is not contiguous", o->string);
 		w->size[1] *= w->size[2] * w->size[3];
 		w->stride[1] = 1;
 		w->nDimension = 2;

@@ -53,7 +53,7 @@ void thhip_storage_release(THFloatStorage *s)
 {
 	if (__sync_sub_and_fetch(&s->nref, 1) > 0)
 		return;
-	if (s->mustfree == TH_MUSTFREE_HIP)
+	if (TH_IS_HIP_STORAGE(s->mustfree))
 		thhip_free(s->data);
 	else if (s->mustfree)
 		free(s->data);
@@ -116,7 +116,7 @@ void THFloatTensor_resize(THFloatTensor *t, long *size, int nDimension)
 	}
 	if (!t->storage)
 		t->storage = THFloatStorage_new(stride);
-	else if (t->storage->mustfree == TH_MUSTFREE_HIP)
+	else if (TH_IS_HIP_STORAGE(t->storage->mustfree))
 		THError("Resizing of device tensors is done by the engine, not by THFloatTensor_resize");
 	else
 		t->storage->data = realloc(t->storage->data, sizeof(float) * (size_t)stride);

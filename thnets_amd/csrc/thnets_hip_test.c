@@ -111,11 +111,12 @@ int main(int argc, char **argv)
 			break;
 		case 'p': print = 1; break;
 		case 'P': th_profile = 1; break;
+		case 'M': th_minmax = 1; break;
 		}
 	}
 	if (!modelsdir || !inputfile || alg < 8 || alg > 11 || runs < 1) {
 		fprintf(stderr, "Syntax: thnets-hip-test -m <models directory> -i <input.t7 | image.ppm | random>\n");
-		fprintf(stderr, "             [-r <number of runs>] [-p(rint results)] [-P(rofile)]\n");
+		fprintf(stderr, "             [-r <number of runs>] [-p(rint results)] [-P(rofile)] [-M(inmax of every layer)]\n");
 		fprintf(stderr, "             [-a <alg=8:HIP fp32 (default), 9:HIP fp16, 10:HIP bf16, 11:HIP 8bit>]\n");
 		fprintf(stderr, "             [-R <range of the 8 bit activations, default 4>]\n");
 		fprintf(stderr, "             [-b <nbatch>] [-d <debuglevel=0 (default),1 or 2>]\n");
