@@ -373,7 +373,7 @@ def _device_codes(hiplib, net, q):
     by the library)."""
     from thnets_amd import abi
     dev = api.DeviceArray(hiplib, np.ascontiguousarray(q, np.uint8))
-    st = abi.THFloatStorage(dev.ptr, 2, 4)
+    st = abi.THFloatStorage(dev.ptr, 2, abi.TH_MUSTFREE_HIP + abi.THHIP_U8)
     t = abi.ABI.THFloatTensor()
     t.nDimension = q.ndim
     stride = 1

@@ -35,6 +35,8 @@ ENGINE_CPU, ENGINE_CUDA, ENGINE_OPENCL, ENGINE_OPENCLINIT, ENGINE_LOWP, ENGINE_H
 
 # enum thhip_dtype
 THHIP_F32, THHIP_F16, THHIP_BF16, THHIP_U8 = range(4)
+# THFloatStorage.mustfree of device memory owned by the engine: 4 + the element type it holds
+TH_MUSTFREE_HIP = 4
 
 
 class THFloatStorage(C.Structure):
