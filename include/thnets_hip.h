@@ -687,16 +687,16 @@ void thhip_maxpool_cl(const void *x, void *y, int B, int C, int H, int W, int oH
 
 /* The same arithmetic as thhip_conv2d_u8 for layers with one output position
  * per image (Linear, or a window covering its whole input): x [B][K] codes,
- * wrow from thhip_linear_pack_weight_u8 (row-major [nOut][K] host codes ->
- * device copy re-centred to signed bytes), rowsum from thhip_u8_rowsums,
- * y [B][nOut].  Replaces the same reference lines; B <= 64, K % 16 == 0.
- * thhip_linear_batched_u8_set_tuning forces the K split and the 32-row groups
- * per wavefront (tests, tuning); zeros restore the heuristic. */
+ * wfrag from thhip_linear_pack_weight_u8 (row-major [nOut][K] host codes ->
+ * device copy re-centred to signed bytes, in the order the kernel streams them:
+ * 16-row blocks x 64-code K-steps, one matrix-core fragment after the other),
+ * rowsum from thhip_u8_rowsums, y [B][nOut].  Replaces the same reference
+ * lines; B <= 64, K % 16 == 0.  One kernel: a workgroup owns 16 rows and all of
+ * K, sums its wavefronts' tiles through LDS and requantises. */
 int thhip_linear_batched_u8_supported(int B, int K, int nOut);
 unsigned char *thhip_linear_pack_weight_u8(const unsigned char *w_host, int nOut, int K);
 int *thhip_u8_rowsums(const unsigned char *w_host, int nOut, int K);
-void thhip_linear_batched_u8_set_tuning(int ksplit, int rg);
-void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wrow, const int *rowsum,
+void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wfrag, const int *rowsum,
 	const int *addend, unsigned char *y, int B, int K, int nOut,
 	int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val);
 

@@ -250,29 +250,26 @@ def _linear_u8(hiplib, xq, wq, addend, prm, act=0, thr=0, val=0):
 def test_linear_batched_u8_bit_exact(hiplib, oracle):
     """One-position layers through the matrix kernel: against the GEMM + bias add of the
     restatement (a plane of one element is all tail: no lower clamp), ragged rows,
-    batches and K tails, every (K split, row group) variant, with wrapping parameters."""
+    batches (one, two and four groups of sixteen columns) and K tails (K % 64 of 16, 48;
+    fewer K-steps than wavefronts), with wrapping parameters."""
     g = cases.rng(1200)
     prms = (dict(a_off=-117, b_off=-128, c_off=32513, c_mult=1028, c_shift=18),
             dict(a_off=-255, b_off=3, c_off=-12345, c_mult=511, c_shift=14),
             dict(a_off=0, b_off=0, c_off=0, c_mult=9000, c_shift=20))
-    shapes = ((1, 16, 1), (2, 144, 37), (33, 1024, 100), (64, 2064, 70), (17, 4096, 130), (64, 9216, 64))
-    try:
-        for ci, (B, K, nOut) in enumerate(shapes):
-            xq = g.integers(0, 256, (B, K), dtype=np.uint8)
-            wq = g.integers(0, 256, (nOut, K), dtype=np.uint8)
-            addend = g.integers(-40, 41, nOut).astype(np.int32)
-            prm = prms[ci % len(prms)]
-            plain = oracle.lowp_gemm(wq, np.ascontiguousarray(xq.T), **prm).T        # [B][nOut]
-            biased = np.stack([[oracle.lowp_add(plain[b, o:o + 1], int(addend[o]))[0] for o in range(nOut)]
-                               for b in range(B)]).astype(np.uint8)
-            for (ks, rg) in ((0, 0), (1, 1), (3, 2), (64, 1)):
-                hiplib.thhip_linear_batched_u8_set_tuning(ks, rg)
-                assert np.array_equal(_linear_u8(hiplib, xq, wq, None, prm), plain), (B, K, nOut, ks, rg)
-                assert np.array_equal(_linear_u8(hiplib, xq, wq, addend, prm), biased), (B, K, nOut, ks, rg)
-                got = _linear_u8(hiplib, xq, wq, addend, prm, act=1, thr=100, val=97)
-                assert np.array_equal(got, oracle.lowp_threshold(biased, 100, 97)), (B, K, nOut, ks, rg)
-    finally:
-        hiplib.thhip_linear_batched_u8_set_tuning(0, 0)
+    shapes = ((1, 16, 1), (2, 144, 37), (33, 1024, 100), (64, 2064, 70), (17, 4096, 130), (64, 9216, 64),
+              (16, 1088, 16), (32, 64, 33), (48, 4144, 17), (5, 6400, 1000))
+    for ci, (B, K, nOut) in enumerate(shapes):
+        xq = g.integers(0, 256, (B, K), dtype=np.uint8)
+        wq = g.integers(0, 256, (nOut, K), dtype=np.uint8)
+        addend = g.integers(-40, 41, nOut).astype(np.int32)
+        prm = prms[ci % len(prms)]
+        plain = oracle.lowp_gemm(wq, np.ascontiguousarray(xq.T), **prm).T        # [B][nOut]
+        biased = np.stack([[oracle.lowp_add(plain[b, o:o + 1], int(addend[o]))[0] for o in range(nOut)]
+                           for b in range(B)]).astype(np.uint8)
+        assert np.array_equal(_linear_u8(hiplib, xq, wq, None, prm), plain), (B, K, nOut)
+        assert np.array_equal(_linear_u8(hiplib, xq, wq, addend, prm), biased), (B, K, nOut)
+        got = _linear_u8(hiplib, xq, wq, addend, prm, act=1, thr=100, val=97)
+        assert np.array_equal(got, oracle.lowp_threshold(biased, 100, 97)), (B, K, nOut)
     assert not hiplib.thhip_linear_batched_u8_supported(65, 1024, 10)
     assert not hiplib.thhip_linear_batched_u8_supported(4, 1000, 10)
 

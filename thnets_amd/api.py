@@ -127,7 +127,6 @@ PROTOTYPES = {
     "thhip_linear_batched_u8_supported": (C.c_int, [C.c_int] * 3),
     "thhip_u8_rowsums": (vp, [vp, C.c_int, C.c_int]),
     "thhip_linear_pack_weight_u8": (vp, [vp, C.c_int, C.c_int]),
-    "thhip_linear_batched_u8_set_tuning": (None, [C.c_int, C.c_int]),
     "thhip_linear_batched_u8": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 3 + [C.c_int] * 5 + [C.c_int] * 3),
     "thhip_rgb2code": (None, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, c_fp, c_fp]),
     "thhip_threshold_u8": (None, [vp, vp, C.c_long, C.c_int, C.c_int, C.c_int]),

@@ -387,230 +387,237 @@ extern "C" int thhip_linear_batched_noalloc(const void *x, const void *wrow, con
 
 /*
  * One output position per image in the uint8 engine (Linear layers, or a
- * convolution whose window covers its whole input): C[b][o] over K codes.
- * Both operands are K-contiguous in memory -- weights row-major [nOut][K],
- * activations [B][K] -- and v_mfma_i32_32x32x32_i8 wants 16 consecutive k per
- * lane (lane = row or column lane%32, k half lane/32), so operands go from
- * global memory to the matrix core through registers only.  A K-step is 128
- * codes, four MFMAs of 32: for MFMA j lane (m, h) reads the 16 bytes
- * k0 + 32j + 16h .. +15 of its row, so the two halves of a load are adjacent
- * in memory.  Weights are stored re-centred (code - 128, done
- * once at pack time), activations are re-centred on the fly (x ^ 0x80).
+ * convolution whose window covers its whole input): C[b][o] over K codes,
+ * batch <= 64.  The layer is bound by reading its weights once from HBM, so
+ * the weights are stored in the order the matrix core wants them and the whole
+ * layer is one kernel:
  *
- * The four wavefronts of a workgroup own the same RG*32 rows and every fourth
- * K-step of the workgroup's slice; their int32 tiles are summed through LDS
- * and written as one partial per (K slice, row, batch column).  A finishing
- * kernel sums the slices, applies the expanded offset terms, gemmlowp's output
- * stage, the saturating bias add (a plane of one element is all "tail": no
- * lower clamp, lowp_SpatialConvolution.c:86-87) and the threshold.  Integer
- * sums are exact, so the split changes nothing in the result.
+ * - v_mfma_i32_16x16x64_i8 takes, of a 16-row block, 16 consecutive k per lane
+ *   (lane = row lane % 16, k quarter lane / 16).  The pack step stores every
+ *   (16-row block, 64-code K-step) as the 1 KiB a wavefront loads for it, lane
+ *   by lane, re-centred to signed bytes (code - 128), K-steps of a block one
+ *   after the other: a load instruction reads 1 KiB contiguous, no permutes.
+ *   Rows and K are padded with re-centred zeros, which add nothing.
+ * - A workgroup of sixteen wavefronts owns one 16-row block and all of K, which
+ *   it walks in chunks of sixteen K-steps (1024 codes), wavefront w taking step
+ *   w of every chunk: the workgroup reads 16 KiB of contiguous weights per
+ *   chunk, each wavefront keeps the weights of the next three chunks on their
+ *   way.
+ * - The activations [B][K] of a chunk are needed by every wavefront's fragment
+ *   in a layout that is bad to fetch (16 rows x 64 bytes per load), so the
+ *   workgroup fetches them together, whole 1 KiB runs of a row per load, four
+ *   chunks ahead into registers, and passes them on through LDS (two buffers,
+ *   one barrier per chunk).  A 16-byte piece (row b, k piece p) goes to slot
+ *   b % 16 ^ p % 16 of its 256-byte line [step p / 4][group b / 16][quarter
+ *   p % 4], which keeps both the writes (one row, 64 pieces per wavefront) and
+ *   the fragment reads (16 rows of one piece per quarter) free of bank
+ *   conflicts.  Rows past B repeat the last one, pieces past K hold code 128
+ *   (0 once re-centred: x ^ 0x80); the column sums are taken with v_dot4.
+ * - The sixteen partial tiles are summed through LDS (integer sums: exact in
+ *   any order) and the same workgroup applies the expanded offset terms,
+ *   gemmlowp's output stage in wrapping int32, the saturating bias add (a plane
+ *   of one element is all "tail": no lower clamp,
+ *   lowp_SpatialConvolution.c:86-87) and the threshold, and writes y [B][nOut].
+ *   No partial sums in global memory, no second launch.
  */
-#define SKU_KSTEP 128
-#define SKU_BPAD 64	/* batch columns per partial row */
+#define LU_THREADS 1024
+#define LU_WAVES 16
+#define LU_KSTEP 64
+#define LU_ROWS 16
+#define LU_CHUNK (LU_WAVES * LU_KSTEP)	/* codes per chunk */
+#define LU_AHEAD 4			/* chunks of activations in flight (in registers); weights: one fewer */
 
-template <int RG, int NB>	/* RG 32-row groups per wavefront; NB 32-column groups: batch <= 32 * NB */
-__global__ __launch_bounds__(SK_THREADS) void skinny_u8_kernel(const unsigned char *x, const unsigned char *w,
-	int *part, int *cspart, int B, int K, int nOut, int ksplit)
-{
-	const int tid = threadIdx.x, lane = tid & 63;
-	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int m = lane & 31, h = lane >> 5;
-	const int row0 = blockIdx.x * (32 * RG);
-	const int nsteps = (K + SKU_KSTEP - 1) / SKU_KSTEP;
-	const int stride = ksplit * 4;
-	const bool want_cs = blockIdx.x == 0;
-	const unsigned char *wr[RG], *xr[NB];
-#pragma unroll
-	for (int rg = 0; rg < RG; rg++)
-		wr[rg] = w + (size_t)min(row0 + rg * 32 + m, nOut - 1) * K + h * 16;
-#pragma unroll
-	for (int g = 0; g < NB; g++)
-		xr[g] = x + (size_t)min(g * 32 + m, B - 1) * K + h * 16;
-	intx16 acc[RG][NB];
-	int cs[NB];
-#pragma unroll
-	for (int g = 0; g < NB; g++) {
-		cs[g] = 0;
-#pragma unroll
-		for (int rg = 0; rg < RG; rg++)
-#pragma unroll
-			for (int r = 0; r < 16; r++)
-				acc[rg][g][r] = 0;
-	}
-	const intx4 zero_a = { 0, 0, 0, 0 };
-	const intx4 zero_b = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
-	intx4 a[RG][4], b[NB][4], an[RG][4], bn[NB][4];
-
-	/* K % 16 == 0: a 16-byte piece is all inside the row or all outside */
-#define SKU_LOAD(A_, B_, ST_)                                                                  \
-	do {                                                                                   \
-		const int kk_ = (ST_) * SKU_KSTEP;                                             \
-		_Pragma("unroll") for (int j = 0; j < 4; j++) {                                \
-			const bool ok_ = kk_ + j * 32 + h * 16 < K;                            \
-			_Pragma("unroll") for (int rg = 0; rg < RG; rg++)                      \
-				A_[rg][j] = ok_ ? *(const intx4 *)(wr[rg] + kk_ + j * 32) : zero_a; \
-			_Pragma("unroll") for (int g = 0; g < NB; g++)                         \
-				B_[g][j] = ok_ ? *(const intx4 *)(xr[g] + kk_ + j * 32) : zero_b;  \
-		}                                                                              \
-	} while (0)
-
-	int st = blockIdx.y * 4 + wave;
-	if (st < nsteps)
-		SKU_LOAD(a, b, st);
-	for (; st < nsteps; st += stride) {
-		const int sn = st + stride;
-		if (sn < nsteps)
-			SKU_LOAD(an, bn, sn);
-#pragma unroll
-		for (int j = 0; j < 4; j++) {
-#pragma unroll
-			for (int g = 0; g < NB; g++) {
-#pragma unroll
-				for (int d = 0; d < 4; d++)
-					b[g][j][d] ^= (int)0x80808080;
-				if (want_cs) {
-#pragma unroll
-					for (int d = 0; d < 4; d++)
-						cs[g] = __builtin_amdgcn_sdot4(b[g][j][d], 0x01010101, cs[g], false);
-				}
-#pragma unroll
-				for (int rg = 0; rg < RG; rg++)
-					acc[rg][g] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[rg][j], b[g][j], acc[rg][g], 0, 0, 0);
-			}
-		}
-		if (sn < nsteps) {
-#pragma unroll
-			for (int j = 0; j < 4; j++) {
-#pragma unroll
-				for (int rg = 0; rg < RG; rg++)
-					a[rg][j] = an[rg][j];
-#pragma unroll
-				for (int g = 0; g < NB; g++)
-					b[g][j] = bn[g][j];
-			}
-		}
-	}
-#undef SKU_LOAD
-
-	/* D layout: lane holds column n = lane%32, rows 8*(r/4) + 4*(lane/32) + r%4 */
-	__shared__ int red[4][16][65];
-	__shared__ int csred[4][NB][64];
-#pragma unroll
-	for (int rg = 0; rg < RG; rg++)
-#pragma unroll
-		for (int g = 0; g < NB; g++) {
-			if (rg + g)
-				__syncthreads();
-#pragma unroll
-			for (int r = 0; r < 16; r++)
-				red[wave][r][lane] = acc[rg][g][r];
-			__syncthreads();
-#pragma unroll
-			for (int i = 0; i < 4; i++) {
-				const int idx = tid + i * SK_THREADS;
-				const int n = idx & 31, o = idx >> 5;
-				const int r = 4 * (o >> 3) + (o & 3), ln = n + 32 * ((o >> 2) & 1);
-				const int s = (red[0][r][ln] + red[1][r][ln]) + (red[2][r][ln] + red[3][r][ln]);
-				const int bcol = g * 32 + n, orow = row0 + rg * 32 + o;
-				if (orow < nOut && bcol < B)
-					part[((size_t)blockIdx.y * nOut + orow) * SKU_BPAD + bcol] = s;
-			}
-		}
-	if (want_cs) {
-#pragma unroll
-		for (int g = 0; g < NB; g++)
-			csred[wave][g][lane] = cs[g];
-		__syncthreads();
-		if (tid < 32 * NB) {
-			const int g = tid >> 5, n = tid & 31;
-			int s = 0;
-#pragma unroll
-			for (int wv = 0; wv < 4; wv++)
-				s += csred[wv][g][n] + csred[wv][g][n + 32];
-			cspart[blockIdx.y * SKU_BPAD + tid] = s;
-		}
-	}
-}
-
-/* One workgroup per 32 output rows x 16 batch columns: sums the K slices,
- * requantises and transposes [row][batch] partials into y [B][nOut] through LDS. */
-__global__ __launch_bounds__(256) void skinny_u8_finish_kernel(const int *part, const int *cspart, const int *rowsum,
-	const int *addend, unsigned char *y, int B, int K, int nOut, int ksplit, int offA, int offB,
+template <int NCG>	/* groups of 16 batch columns: batch <= 16 * NCG */
+__global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned char *x, const unsigned char *wfrag,
+	const int *rowsum, const int *addend, unsigned char *y, int B, int K, int nOut, int nsteps, int offA, int offB,
 	int c_off, int c_mult, int c_shift, int act, int thr, int val)
 {
-	__shared__ int t[32][17];
-	__shared__ int csum[16];
-	const int tid = threadIdx.x, o0 = blockIdx.x * 32, b0 = blockIdx.y * 16;
-	if (tid < 16) {
-		int s = 0;
-		for (int p = 0; p < ksplit; p++)
-			s += cspart[p * SKU_BPAD + b0 + tid];
-		csum[tid] = s;
-	}
-	{
-		const int bl = tid & 15, oo = tid >> 4;
+	extern __shared__ __align__(16) unsigned char lds[];	/* two buffers of NCG * 16 KiB */
+	constexpr int XBUF = NCG * 16 * LU_CHUNK;
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int m = lane & 15, q = lane >> 4;
+	const int nchunks = (nsteps + LU_WAVES - 1) / LU_WAVES;
+	/* uniform bases plus 32-bit lane offsets: the addresses stay on the scalar unit */
+	const unsigned char *wp = wfrag + ((size_t)blockIdx.x * nsteps) * 1024;
+	const unsigned woff = lane * 16;
+	/* staging: this thread moves piece `lane` of rows wave, wave + 16, ... of a chunk */
+	unsigned xsrc[NCG], xdst[NCG];
 #pragma unroll
-		for (int i = 0; i < 2; i++) {
-			const int ol = oo + 16 * i, o = o0 + ol;
-			int s = 0;
-			if (o < nOut && b0 + bl < B)
-				for (int p = 0; p < ksplit; p++)
-					s += part[((size_t)p * nOut + o) * SKU_BPAD + b0 + bl];
-			t[ol][bl] = s;
+	for (int g = 0; g < NCG; g++) {
+		xsrc[g] = (unsigned)min(g * 16 + wave, B - 1) * (unsigned)K + lane * 16;
+		xdst[g] = (((lane >> 2) * NCG + g) * 4 + (lane & 3)) * 256 + ((wave ^ lane) & 15) * 16;
+	}
+	/* fragments: step `wave` of the chunk, group g, quarter q, row m */
+	const unsigned fsrc = ((wave * NCG) * 4 + q) * 256 + ((m ^ (wave * 4 + q)) & 15) * 16;
+	intx4 acc[NCG];
+	int cs[NCG];
+#pragma unroll
+	for (int g = 0; g < NCG; g++) {
+		acc[g] = intx4{ 0, 0, 0, 0 };
+		cs[g] = 0;
+	}
+	intx4 a[LU_AHEAD], xr[LU_AHEAD][NCG];
+	const intx4 zero_b = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
+
+	/* Requests past the end repeat the last valid address (a hit, and never used), so
+	 * the loop body has no divergent branches. */
+#define LU_LOAD_A(SLOT_, C_) (a[SLOT_] = *(const intx4 *)(wp + (size_t)min((C_) * LU_WAVES + wave, nsteps - 1) * 1024 + woff))
+#define LU_LOAD_X(SLOT_, C_)                                                                       \
+	do {                                                                                       \
+		const int k_ = min((C_), nchunks - 1) * LU_CHUNK;                                  \
+		const bool ok_ = k_ + lane * 16 < K;	/* K % 16 == 0: a piece is all in or all out */ \
+		_Pragma("unroll") for (int g = 0; g < NCG; g++)                                    \
+			xr[SLOT_][g] = *(const intx4 *)(x + (ok_ ? k_ + xsrc[g] : 0u));            \
+	} while (0)
+	/* Staging re-centres the codes (x ^ 0x80) and takes their column sums, so that a
+	 * fragment read is followed by its MFMA and nothing else.  Pieces past K are
+	 * replaced here, not when they are requested (touching a register that a load is
+	 * still filling would wait for the load), and only the last chunk has any. */
+#define LU_STAGE(SLOT_, BUF_, C_)                                                                  \
+	do {                                                                                       \
+		if ((C_) < nchunks) {                                                              \
+			const bool tail_ = (C_) == nchunks - 1;                                    \
+			const bool ok_ = (C_) * LU_CHUNK + lane * 16 < K;                          \
+			_Pragma("unroll") for (int g = 0; g < NCG; g++) {                          \
+				intx4 v_ = xr[SLOT_][g];                                           \
+				if (tail_)                                                         \
+					v_ = ok_ ? v_ : zero_b;                                    \
+				_Pragma("unroll") for (int d = 0; d < 4; d++) {                    \
+					v_[d] ^= (int)0x80808080;                                  \
+					cs[g] = __builtin_amdgcn_sdot4(v_[d], 0x01010101, cs[g], false); \
+				}                                                                  \
+				*(intx4 *)(lds + (BUF_) * XBUF + xdst[g]) = v_;                    \
+			}                                                                          \
+		}                                                                                  \
+	} while (0)
+#define LU_MMA(SLOT_, C_)                                                                          \
+	do {                                                                                       \
+		if ((C_) * LU_WAVES + wave < nsteps) {                                             \
+			intx4 bb_[NCG];                                                            \
+			_Pragma("unroll") for (int g = 0; g < NCG; g++)                            \
+				bb_[g] = *(const intx4 *)(lds + ((C_) & 1) * XBUF + fsrc + g * 1024); \
+			_Pragma("unroll") for (int g = 0; g < NCG; g++)                            \
+				acc[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[SLOT_], bb_[g], acc[g], 0, 0, 0); \
+		}                                                                                  \
+	} while (0)
+
+	/* Loads complete in the order they were issued, so waiting for one waits for all
+	 * older ones: the activations of a chunk are requested four chunks before they
+	 * are staged, the weights three chunks before they are used, and each request
+	 * is issued after everything that is needed before it. */
+#pragma unroll
+	for (int i = 0; i < LU_AHEAD; i++)
+		LU_LOAD_X(i, i);
+#pragma unroll
+	for (int i = 0; i < LU_AHEAD - 1; i++)
+		LU_LOAD_A(i, i);
+	LU_STAGE(0, 0, 0);
+	LU_LOAD_X(0, LU_AHEAD);
+	__syncthreads();
+	for (int c = 0; c < nchunks; c += LU_AHEAD) {
+#pragma unroll
+		for (int i = 0; i < LU_AHEAD; i++) {
+			/* chunk c + i: its activations are in LDS buffer (c + i) % 2, those of the
+			 * following chunks in registers */
+			LU_LOAD_A((i + LU_AHEAD - 1) % LU_AHEAD, c + i + LU_AHEAD - 1);
+			LU_MMA(i, c + i);
+			LU_STAGE((i + 1) % LU_AHEAD, (c + i + 1) & 1, c + i + 1);
+			LU_LOAD_X((i + 1) % LU_AHEAD, c + i + 1 + LU_AHEAD);
+			__syncthreads();
 		}
+	}
+#undef LU_LOAD_A
+#undef LU_LOAD_X
+#undef LU_STAGE
+#undef LU_MMA
+
+	/* D layout: lane holds column n = lane % 16 of its group, rows 4 * (lane / 16) + r.
+	 * Waves 8..15 hand their tiles to waves 0..7, those put the pair sums into LDS,
+	 * and every thread finishes one (row, column).  (The loop's last barrier has
+	 * passed: the activation buffers are free.) */
+	int (*red)[NCG * 4][64] = (int (*)[NCG * 4][64])lds;				/* [8] */
+	int *colsum = (int *)(lds + 8 * NCG * 4 * 64 * sizeof(int));			/* [16 * NCG] */
+	/* a staging thread summed its pieces of rows wave, wave + 16, ...: the lanes of a
+	 * wavefront hold the 64 parts of one column sum */
+#pragma unroll
+	for (int g = 0; g < NCG; g++) {
+		int v = cs[g];
+#pragma unroll
+		for (int off = 32; off > 0; off >>= 1)
+			v += __shfl_xor(v, off, 64);
+		if (lane == 0)
+			colsum[g * 16 + wave] = v;
+	}
+	if (wave >= 8) {
+#pragma unroll
+		for (int g = 0; g < NCG; g++)
+#pragma unroll
+			for (int r = 0; r < 4; r++)
+				red[wave - 8][g * 4 + r][lane] = acc[g][r];
 	}
 	__syncthreads();
-	const int ol = tid & 31, o = o0 + ol, bb = tid >> 5;
-	if (o >= nOut)
-		return;
-	const int rs = offB * rowsum[o] + K * offA * offB;
-	const int add = addend ? addend[o] : 0;
+	if (wave < 8) {
 #pragma unroll
-	for (int i = 0; i < 2; i++) {
-		const int bl = bb + 8 * i, b = b0 + bl;
-		if (b >= B)
-			break;
-		const int a = t[ol][bl] + rs + offA * csum[bl];
-		unsigned u = ((unsigned)a + (unsigned)c_off) * (unsigned)c_mult;
-		u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
-		int q = (int)u >> c_shift;
-		q = q < 0 ? 0 : q > 255 ? 255 : q;
-		if (addend) {
-			const int sum = q + add;
-			q = sum > 255 ? 255 : (sum & 255);
-		}
-		if (act)
-			q = q > thr ? q : val;
-		y[(size_t)b * nOut + o] = (unsigned char)q;
+		for (int g = 0; g < NCG; g++)
+#pragma unroll
+			for (int r = 0; r < 4; r++)
+				acc[g][r] += red[wave][g * 4 + r][lane];
 	}
+	__syncthreads();
+	if (wave < 8) {
+#pragma unroll
+		for (int g = 0; g < NCG; g++)
+#pragma unroll
+			for (int r = 0; r < 4; r++)
+				red[wave][g * 4 + r][lane] = acc[g][r];
+	}
+	__syncthreads();
+	/* thread -> (row rr, batch column bcol): neighbouring threads write neighbouring bytes of y */
+	const int rr = tid & 15, bcol = tid >> 4;
+	const int o = blockIdx.x * LU_ROWS + rr;
+	if (bcol >= 16 * NCG || bcol >= B || o >= nOut)
+		return;
+	const int g = bcol >> 4, n = bcol & 15;
+	const int src = (rr >> 2) * 16 + n, reg = g * 4 + (rr & 3);
+	int sum = 0, csum = 0;
+#pragma unroll
+	for (int wv = 0; wv < 8; wv++)
+		sum += red[wv][reg][src];
+	csum = colsum[bcol];
+	const int t = sum + offB * rowsum[o] + K * offA * offB + offA * csum;
+	unsigned u = ((unsigned)t + (unsigned)c_off) * (unsigned)c_mult;
+	u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
+	int code = (int)u >> c_shift;
+	code = code < 0 ? 0 : code > 255 ? 255 : code;
+	if (addend) {
+		const int sa = code + addend[o];
+		code = sa > 255 ? 255 : (sa & 255);
+	}
+	if (act)
+		code = code > thr ? code : val;
+	y[(size_t)bcol * nOut + o] = (unsigned char)code;
 }
-
-static int *g_u8_scratch;
-static size_t g_u8_scratch_words;
-static int g_u8_ksplit, g_u8_rg;
 
 extern "C" int thhip_linear_batched_u8_supported(int B, int K, int nOut)
 {
 	return B >= 1 && B <= 64 && K % 16 == 0 && K >= 16 && nOut >= 1;
 }
 
-/* Test and tuning hook: force the K split (1..64) and the row groups per
- * wavefront (1 or 2) of thhip_linear_batched_u8; 0 restores the heuristic. */
-extern "C" void thhip_linear_batched_u8_set_tuning(int ksplit, int rg)
-{
-	if (ksplit < 0 || ksplit > 64 || rg < 0 || rg > 2)
-		THError("thhip_linear_batched_u8_set_tuning(%d, %d): out of range", ksplit, rg);
-	g_u8_ksplit = ksplit;
-	g_u8_rg = rg;
-}
-
-/* Device copy of row-major weight codes [nOut][K], re-centred to signed bytes. */
+/* Device copy of row-major weight codes [nOut][K] in the order linear_u8_kernel
+ * streams them: [16-row block][K-step of 64][lane][16 bytes], lane = row % 16 +
+ * 16 * (k quarter), re-centred to signed bytes; rows and K padded with zeros. */
 extern "C" unsigned char *thhip_linear_pack_weight_u8(const unsigned char *w_host, int nOut, int K)
 {
-	const size_t n = (size_t)nOut * K;
-	unsigned char *h = (unsigned char *)malloc(n);
-	for (size_t i = 0; i < n; i++)
-		h[i] = w_host[i] ^ 0x80;
+	const int nblocks = (nOut + LU_ROWS - 1) / LU_ROWS, nsteps = (K + LU_KSTEP - 1) / LU_KSTEP;
+	const size_t n = (size_t)nblocks * nsteps * 1024;
+	unsigned char *h = (unsigned char *)calloc(n, 1);
+	for (int o = 0; o < nOut; o++) {
+		const unsigned char *src = w_host + (size_t)o * K;
+		unsigned char *blk = h + ((size_t)(o / LU_ROWS) * nsteps) * 1024 + (o % LU_ROWS) * 16;
+		for (int k = 0; k < K; k++)
+			blk[(size_t)(k / LU_KSTEP) * 1024 + ((k % LU_KSTEP) / 16) * 256 + (k % 16)] = src[k] ^ 0x80;
+	}
 	unsigned char *d = (unsigned char *)thhip_malloc(n);
 	thhip_memcpy_h2d(d, h, n);
 	free(h);
@@ -633,14 +640,7 @@ extern "C" int *thhip_u8_rowsums(const unsigned char *w_host, int nOut, int K)
 	return d;
 }
 
-template <int RG, int NB>
-static void skinny_u8_launch(dim3 grid, const unsigned char *x, const unsigned char *wrow, int *part, int *cspart,
-	int B, int K, int nOut, int ksplit)
-{
-	skinny_u8_kernel<RG, NB><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, cspart, B, K, nOut, ksplit);
-}
-
-extern "C" void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wrow, const int *rowsum,
+extern "C" void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wfrag, const int *rowsum,
 	const int *addend, unsigned char *y, int B, int K, int nOut,
 	int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val)
 {
@@ -648,44 +648,26 @@ extern "C" void thhip_linear_batched_u8(const unsigned char *x, const unsigned c
 		THError("thhip_linear_batched_u8: unsupported shape B=%d K=%d nOut=%d", B, K, nOut);
 	if (c_shift < 0 || c_shift > 31)
 		THError("thhip_linear_batched_u8: shift %d out of range", c_shift);
-	const int rg = g_u8_rg ? g_u8_rg : nOut >= 2048 ? 2 : 1;
-	const int groups = (nOut + 32 * rg - 1) / (32 * rg);
-	const int nsteps = (K + SKU_KSTEP - 1) / SKU_KSTEP;
-	/* aim at ~1024 wavefronts with at least two K-steps each */
-	int ksplit = (256 + groups - 1) / groups;
-	if (ksplit > nsteps / 8)
-		ksplit = nsteps / 8;
-	if (g_u8_ksplit)
-		ksplit = g_u8_ksplit;
-	if (ksplit < 1)
-		ksplit = 1;
-	if (ksplit > 64)
-		ksplit = 64;
-	const size_t words = (size_t)ksplit * SKU_BPAD * ((size_t)nOut + 1);
-	if (words > g_u8_scratch_words) {
-		if (g_u8_scratch) {
-			hipcheck(hipStreamSynchronize(thhip_stream()));
-			thhip_free(g_u8_scratch);
-		}
-		g_u8_scratch_words = words < (1u << 20) ? (1u << 20) : words;
-		g_u8_scratch = (int *)thhip_malloc(g_u8_scratch_words * sizeof(int));
-	}
-	int *cspart = g_u8_scratch, *part = g_u8_scratch + (size_t)ksplit * SKU_BPAD;
-	{
-		ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * nOut * (double)K * B);
-		dim3 grid(groups, ksplit);
-		if (rg == 1 && B <= 32)
-			skinny_u8_launch<1, 1>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
-		else if (rg == 1)
-			skinny_u8_launch<1, 2>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
-		else if (B <= 32)
-			skinny_u8_launch<2, 1>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
-		else
-			skinny_u8_launch<2, 2>(grid, x, wrow, part, cspart, B, K, nOut, ksplit);
-	}
-	{
-		ThhipLaunchScope scope(THHIP_FAM_OTHER, (4.0 * ksplit + 1.0) * B * nOut);
-		skinny_u8_finish_kernel<<<dim3((nOut + 31) / 32, (B + 15) / 16), dim3(256), 0, thhip_stream()>>>(part, cspart, rowsum, addend, y,
-			B, K, nOut, ksplit, 128 + a_off, 128 + b_off, c_off, c_mult, c_shift, act, thr, val);
-	}
+	const int nblocks = (nOut + LU_ROWS - 1) / LU_ROWS, nsteps = (K + LU_KSTEP - 1) / LU_KSTEP;
+	/* algorithmic work for the profiler: 2 nOut K B operations */
+	ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * nOut * (double)K * B);
+	const dim3 grid(nblocks), block(LU_THREADS);
+	/* two activation buffers of NCG * 16 KiB: more than the 64 KiB a kernel gets without asking */
+	static bool lds_ok[3];
+#define LU_GO(NCG_, I_) do { \
+		const int bytes_ = 2 * NCG_ * 16 * LU_CHUNK; \
+		if (!lds_ok[I_]) { \
+			hipcheck(hipFuncSetAttribute((const void *)linear_u8_kernel<NCG_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes_)); \
+			lds_ok[I_] = true; \
+		} \
+		linear_u8_kernel<NCG_><<<grid, block, bytes_, thhip_stream()>>>(x, wfrag, rowsum, addend, y, B, K, nOut, \
+			nsteps, 128 + a_off, 128 + b_off, c_off, c_mult, c_shift, act, thr, val); \
+	} while (0)
+	if (B <= 16)
+		LU_GO(1, 0);
+	else if (B <= 32)
+		LU_GO(2, 1);
+	else
+		LU_GO(4, 2);
+#undef LU_GO
 }
