@@ -685,6 +685,22 @@ void thhip_relayout(const void *x, void *y, int B, int C, int HW, int to_channel
 void thhip_maxpool_cl(const void *x, void *y, int B, int C, int H, int W, int oH, int oW,
 	int kH, int kW, int dH, int dW, int padH, int padW, int dtype);
 
+/* thhip_conv2d_u8 for an image layer (at most four planes, plane-major x
+ * [B][Ci][H][W], W % 4 == 0, horizontal stride 4, Co % 64 == 0, wpacked from
+ * thhip_conv_pack_weight_u8_layout(..., 2)) followed by the uint8 Threshold and a
+ * 3x3 / stride 2 max pooling without padding (floor mode), in one kernel: replaces
+ * Lowp_SpatialConvolution_updateOutput -> Lowp_Threshold_updateOutput ->
+ * Lowp_SpatialMaxPooling_updateOutput (lowp_SpatialConvolution.c:124-187,
+ * lowp_Threshold.c:3-28, lowp_SpatialMaxPooling.c:45-108) for AlexNet's stem.  y is
+ * channels-last [B][pH][pW][Co], pH = (oH - 3) / 2 + 1; the convolution output is
+ * never written.  thhip_conv2d_u8_image_pool_supported says whether the shapes
+ * (convolution, then the pooling's kH kW dH dW padH padW ceil_mode) are taken. */
+int thhip_conv2d_u8_image_pool_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int pkH, int pkW, int pdH, int pdW, int ppadH, int ppadW, int ceil_mode);
+void thhip_conv2d_u8_image_pool(const unsigned char *x, const void *wpacked, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val);
+
 /* The same arithmetic as thhip_conv2d_u8 for layers with one output position
  * per image (Linear, or a window covering its whole input): x [B][K] codes,
  * wfrag from thhip_linear_pack_weight_u8 (row-major [nOut][K] host codes ->

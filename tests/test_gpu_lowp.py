@@ -228,6 +228,66 @@ def test_maxpool_and_relayout_channels_last(hiplib, oracle):
         assert np.array_equal(dy.get((B, oH, oW, Cn), np.uint8).transpose(0, 3, 1, 2), want)
 
 
+def test_image_layer_with_pooling_bit_exact(hiplib, oracle):
+    """thhip_conv2d_u8_image_pool (image layer + Threshold + 3x3 / stride 2 max pooling in one
+    kernel) against the restatement's convolution, threshold and pooling run one after the
+    other: AlexNet's stem shape, one to four planes, kernel rows of 11, 7, 4 and 5 taps (whole
+    and partial groups of four pixels), other vertical strides, images wide and high enough
+    for several workgroups per image (and ragged last ones), 64 and 128 output planes,
+    parameters that wrap, and the unclamped last positions of a plane."""
+    g = cases.rng(1900)
+    prms = (dict(a_off=-117, b_off=-128, c_off=32513, c_mult=1028, c_shift=18),
+            dict(a_off=-255, b_off=3, c_off=-12345, c_mult=511, c_shift=14),
+            dict(a_off=-100, b_off=-90, c_off=5000, c_mult=700, c_shift=17))
+    #        B  Ci  H    W   Co   kH  kW dH padH padW
+    shapes = ((2, 3, 224, 224, 64, 11, 11, 4, 2, 2),
+              (3, 3, 35, 36, 64, 11, 11, 4, 2, 2),
+              (1, 1, 47, 52, 64, 7, 7, 4, 3, 3),
+              (2, 4, 31, 480, 128, 3, 4, 2, 0, 1),
+              (1, 2, 300, 40, 64, 5, 5, 3, 1, 0),
+              (2, 3, 27, 28, 64, 11, 9, 4, 0, 5))
+    for ci, (B, Ci, H, W, Co, kH, kW, dH, pH, pW) in enumerate(shapes):
+        xq = g.integers(0, 256, (B, Ci, H, W), dtype=np.uint8)
+        wq = g.integers(0, 256, (Co, Ci, kH, kW), dtype=np.uint8)
+        addend = g.integers(-60, 61, Co).astype(np.int32)
+        prm = prms[ci % len(prms)]
+        zero = 128 if ci % 2 == 0 else 77
+        oH, oW = (H + 2 * pH - kH) // dH + 1, (W + 2 * pW - kW) // 4 + 1
+        assert hiplib.thhip_conv2d_u8_image_pool_supported(B, Ci, H, W, Co, kH, kW, dH, 4, pH, pW, 3, 3, 2, 2, 0, 0, 0)
+        # the restatement, step by step: im2col with the padding code, GEMM, bias add (with its tail), threshold, pooling
+        conv = np.empty((B, Co, oH, oW), np.uint8)
+        for b in range(B):
+            col = oracle.lowp_unfold(xq[b], (kH, kW), (dH, 4), (pH, pW), zero)
+            plain = oracle.lowp_gemm(wq.reshape(Co, -1), col, **prm)
+            for o in range(Co):
+                conv[b, o] = oracle.lowp_add(plain[o], int(addend[o])).reshape(oH, oW)
+        thr = oracle.lowp_threshold(conv, 100, 97)
+        want = oracle.lowp_maxpool(thr, 3, 3, 2, 2)
+        ph, pw = want.shape[2:]
+        G.note("conv2d_u8_image_pool x%s w%s dH%d pad(%d,%d) prm%s zero%d" % (xq.shape, wq.shape, dH, pH, pW, prm, zero))
+        wp = hiplib.thhip_conv_pack_weight_u8_layout(wq.ctypes.data, Co, Ci, kH, kW, 2)
+        dx, da = api.DeviceArray(hiplib, xq), api.DeviceArray(hiplib, addend)
+        dy = api.DeviceArray(hiplib, nbytes=B * ph * pw * Co)
+        hiplib.thhip_conv2d_u8_image_pool(dx.ptr, wp, da.ptr, dy.ptr, B, Ci, H, W, Co, kH, kW, dH, 4, pH, pW, zero,
+                                          prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"], prm["c_shift"], 1, 100, 97)
+        hiplib.thhip_sync()
+        got = dy.get((B, ph, pw, Co), np.uint8).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, want), (ci, int((got != want).sum()))
+        # without a bias addend and without a threshold
+        want2 = oracle.lowp_maxpool(np.stack([oracle.lowp_gemm(wq.reshape(Co, -1), oracle.lowp_unfold(
+            xq[b], (kH, kW), (dH, 4), (pH, pW), zero), **prm).reshape(Co, oH, oW) for b in range(B)]), 3, 3, 2, 2)
+        hiplib.thhip_conv2d_u8_image_pool(dx.ptr, wp, None, dy.ptr, B, Ci, H, W, Co, kH, kW, dH, 4, pH, pW, zero,
+                                          prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"], prm["c_shift"], 0, 0, 0)
+        hiplib.thhip_sync()
+        assert np.array_equal(dy.get((B, ph, pw, Co), np.uint8).transpose(0, 3, 1, 2), want2), ci
+        hiplib.thhip_free(wp)
+    # shapes the kernel leaves to the general path
+    assert not hiplib.thhip_conv2d_u8_image_pool_supported(1, 3, 224, 224, 64, 11, 11, 4, 2, 2, 2, 3, 3, 2, 2, 0, 0, 0)   # stride 2
+    assert not hiplib.thhip_conv2d_u8_image_pool_supported(1, 3, 224, 224, 64, 11, 11, 4, 4, 2, 2, 2, 2, 2, 2, 0, 0, 0)   # 2x2 pooling
+    assert not hiplib.thhip_conv2d_u8_image_pool_supported(1, 3, 224, 224, 48, 11, 11, 4, 4, 2, 2, 3, 3, 2, 2, 0, 0, 0)   # 48 planes
+    assert not hiplib.thhip_conv2d_u8_image_pool_supported(1, 5, 224, 224, 64, 11, 11, 4, 4, 2, 2, 3, 3, 2, 2, 0, 0, 0)   # 5 planes
+
+
 def _linear_u8(hiplib, xq, wq, addend, prm, act=0, thr=0, val=0):
     B, K = xq.shape
     nOut = wq.shape[0]
@@ -408,13 +468,22 @@ def test_alexnet_lowp_full_size_bit_exact_and_batch_property(hiplib, oracle):
     hiplib.THHipNetwork_setInputQuant(net.handle, im, isub)
     hiplib.THForward(net.handle, C.addressof(t2))
     layers = cfg["layers"]
+    fused_pool = False
     for i, (qo, mo, so) in enumerate(outs):
         want = qo
         if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold":
             want = outs[i + 1][0]
         got = net.module_output(i).astype(np.uint8)
+        if got.shape != want.shape:
+            # the image layer ran with its Threshold and max pooling in one kernel: its buffer
+            # (and the Threshold's view of it) holds the pooled codes
+            j = next(k for k in range(i + 1, len(layers)) if layers[k]["type"] == "maxpool")
+            assert layers[i]["type"] in ("conv", "threshold") and j <= i + 2, (i, got.shape, want.shape)
+            want = outs[j][0]
+            fused_pool = True
         assert np.array_equal(got, want), "module %d (%s): %d codes differ" % (i, layers[i]["type"], (got != want).sum())
         assert net.module_quant(i) == (np.float32(mo), np.float32(so))
+    assert fused_pool, "the image layer of AlexNet should take the fused convolution + pooling kernel"
     # the logits carry information (not saturated everywhere)
     assert len(np.unique(q)) > 20
     net.free()

@@ -122,6 +122,8 @@ PROTOTYPES = {
     "thhip_conv2d_pool2_supported": (C.c_int, [C.c_int] * 14),
     "thhip_conv2d_layout_pool2": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d_u8_layout_tail": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3 + [C.c_int] * 3),
+    "thhip_conv2d_u8_image_pool_supported": (C.c_int, [C.c_int] * 18),
+    "thhip_conv2d_u8_image_pool": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3),
     "thhip_maxpool_u8_cl": (None, [vp, vp] + [C.c_int] * 12),
     "thhip_relayout_u8": (None, [vp, vp] + [C.c_int] * 4),
     "thhip_linear_batched_u8_supported": (C.c_int, [C.c_int] * 3),

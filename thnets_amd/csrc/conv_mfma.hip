@@ -2291,6 +2291,18 @@ static size_t conv_packed_bytes(int Co, int Ci, int kH, int kW, int dtype, int x
 	return mpad / 32 * conv_kc(Ci, kH, kW, dtype, xl) * 1024;
 }
 
+/* For the kernels in other files that read weights packed by thhip_conv_pack_weight_u8_layout:
+ * K chunks of 32 codes per row block, and the bytes of packed codes (the per-row sums follow). */
+int thhip_conv_u8_packed_chunks(int Ci, int kH, int kW, int x_layout)
+{
+	return conv_kc(Ci, kH, kW, THHIP_U8, x_layout);
+}
+
+size_t thhip_conv_u8_packed_code_bytes(int Co, int Ci, int kH, int kW, int x_layout)
+{
+	return conv_packed_bytes(Co, Ci, kH, kW, THHIP_U8, x_layout);
+}
+
 /* (for plane-major input the packed size depends on kH * kW only) */
 extern "C" size_t thhip_conv_packed_bytes(int Co, int Ci, int kHW, int dtype)
 {

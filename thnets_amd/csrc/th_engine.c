@@ -602,7 +602,6 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 		val = lowp_scale_float(om, osub, hm->val);
 	}
 	const void *x = thhip_tensor_ptr(in, THHIP_U8);
-	void *y = conv_out(m, THHIP_U8, &s, c->nOutputPlane, oH, oW);
 	const int K = c->nInputPlane * c->kH * c->kW;
 	/* the weights were packed for the planned memory order of the input; with
 	 * one pixel per plane both orders coincide */
@@ -610,6 +609,24 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 		THError("uint8 engine: a convolution planned for %s input got the other memory order",
 			hm->in_cl ? "channels-last" : "plane-major");
 	const int x_cl = hm->x_layout;
+	/* image layer -> (Threshold) -> 3x3 / stride 2 max pooling in one kernel, where that kernel takes the shape */
+	if (hm->pool_next && x_cl == 2 && hm->out_cl && s.outnd >= 3) {
+		const struct SpatialMaxPooling *q = &hn->pub.modules[hm->pool_next].SpatialMaxPooling;
+		if (thhip_conv2d_u8_image_pool_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW,
+				c->padH, c->padW, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, q->ceil_mode)) {
+			const int pH = (oH - 3) / 2 + 1, pW = (oW - 3) / 2 + 1;
+			void *yp = conv_out(m, THHIP_U8, &s, c->nOutputPlane, pH, pW);
+			thhip_conv2d_u8_image_pool(x, hm->wpacked, hm->addend, yp, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+				c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
+				hm->fused_act, thr, val);
+			hn->hm[hm->pool_next].pooled_by_producer = 1;
+			hn->cur_cl = pH * pW > 1;
+			hn->cur_mult = om;
+			hn->cur_sub = osub;
+			return m->output;
+		}
+	}
+	void *y = conv_out(m, THHIP_U8, &s, c->nOutputPlane, oH, oW);
 	if (hm->wrow_u8 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
 	    thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
 		thhip_linear_batched_u8(x, hm->wrow_u8, hm->rowsum_u8, hm->addend, y, s.B, K, c->nOutputPlane,
@@ -657,6 +674,13 @@ static THFloatTensor *HipLowp_SpatialMaxPooling_updateOutput(struct module *m, T
 	struct hipnet *hn = hipnet_of(m);
 	struct hipmod *hm = hipmod_of(m);
 	struct SpatialMaxPooling *q = &m->SpatialMaxPooling;
+	if (hm->pooled_by_producer) {	/* done by the convolution before it */
+		hm->pooled_by_producer = 0;
+		out_alias(m, in);
+		hm->q_mult = hn->cur_mult;
+		hm->q_sub = hn->cur_sub;
+		return m->output;
+	}
 	struct planes p = planes_of(in, "SpatialMaxPooling");
 	int oH, oW;
 	thhip_pool_outsize(p.H, p.W, q->kH, q->kW, q->dH, q->dW, q->padH, q->padW, q->ceil_mode, &oH, &oW);
@@ -1257,6 +1281,22 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			continue;
 		const struct SpatialMaxPooling *q = &hn->pub.modules[j].SpatialMaxPooling;
 		if (q->kW == 2 && q->kH == 2 && q->dW == 2 && q->dH == 2 && q->padW == 0 && q->padH == 0 && !q->ceil_mode)
+			hn->hm[i].pool_next = j;
+	}
+	/* uint8 engine: the image layer (at most four planes, plane-major) followed by its
+	 * folded Threshold and a 3x3 / stride 2 max pooling may run as one kernel; whether it
+	 * does is decided per forward by the layer's shape */
+	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIPLOWP; i++) {
+		if (!is_conv_type(hn->pub.modules[i].type) || hn->hm[i].in_cl || !hn->hm[i].out_cl ||
+		    hn->pub.modules[i].SpatialConvolution.nInputPlane > 4)
+			continue;
+		int j = i + 1;
+		while (j < net->nelem && hn->hm[j].passthrough)
+			j++;
+		if (j >= net->nelem || hn->pub.modules[j].type != MT_SpatialMaxPooling)
+			continue;
+		const struct SpatialMaxPooling *q = &hn->pub.modules[j].SpatialMaxPooling;
+		if (q->kW == 3 && q->kH == 3 && q->dW == 2 && q->dH == 2 && q->padW == 0 && q->padH == 0 && !q->ceil_mode)
 			hn->hm[i].pool_next = j;
 	}
 	return &hn->pub;

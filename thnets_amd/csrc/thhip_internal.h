@@ -17,6 +17,10 @@ hipStream_t thhip_stream(void);
 int thhip_prof_begin(int family);
 void thhip_prof_end(int token, double work);
 
+/* conv_mfma.hip: layout of the weights thhip_conv_pack_weight_u8_layout makes */
+int thhip_conv_u8_packed_chunks(int Ci, int kH, int kW, int x_layout);
+size_t thhip_conv_u8_packed_code_bytes(int Co, int Ci, int kH, int kW, int x_layout);
+
 struct ThhipLaunchScope {
 	int token;
 	double work;
