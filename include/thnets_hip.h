@@ -701,6 +701,22 @@ void thhip_conv2d_u8_image_pool(const unsigned char *x, const void *wpacked, con
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val);
 
+/* thhip_conv2d_u8 for stride-1 layers on small channels-last images (x [B][H][W][Ci],
+ * Ci % 64 == 0, Co % 64 == 0, at least four taps, output rows of at most 64 positions when
+ * pooling and 192 otherwise), by a kernel that copies the input patch of a band of output
+ * rows into LDS once per block of 64 planes and takes every tap's operand from there, so
+ * that only the weights stream; optionally (pool = 1) with the 3x3 / stride 2 max pooling
+ * without padding (floor mode) that follows.  Replaces the same reference lines as
+ * thhip_conv2d_u8_image_pool.  wpatch comes from thhip_conv_pack_weight_u8_patch (host codes
+ * [Co][Ci][kH][kW]; K order: block of 64 planes, tap, plane).  y is channels-last,
+ * [B][oH][oW][Co] or the pooled [B][(oH - 3) / 2 + 1][(oW - 3) / 2 + 1][Co]. */
+int thhip_conv2d_u8_patch_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int pool);
+void *thhip_conv_pack_weight_u8_patch(const unsigned char *w, int Co, int Ci, int kH, int kW);
+void thhip_conv2d_u8_patch(const unsigned char *x, const void *wpatch, const int *addend, unsigned char *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int zero, int a_off, int b_off, int c_off, int c_mult, int c_shift, int act, int thr, int val, int pool);
+
 /* The same arithmetic as thhip_conv2d_u8 for layers with one output position
  * per image (Linear, or a window covering its whole input): x [B][K] codes,
  * wfrag from thhip_linear_pack_weight_u8 (row-major [nOut][K] host codes ->

@@ -288,6 +288,61 @@ def test_image_layer_with_pooling_bit_exact(hiplib, oracle):
     assert not hiplib.thhip_conv2d_u8_image_pool_supported(1, 5, 224, 224, 64, 11, 11, 4, 4, 2, 2, 3, 3, 2, 2, 0, 0, 0)   # 5 planes
 
 
+def test_conv_u8_patch_bit_exact(hiplib, oracle):
+    """thhip_conv2d_u8_patch (input patch kept in LDS, optional 3x3 / stride 2 pooling) against
+    the restatement step by step: AlexNet's conv2-5 shapes, several bands per image with and
+    without pooling, kernels of 2x3, 3x3 and 5x5 taps, one to six blocks of 64 input planes
+    (the patch of the next block is fetched while the current one is multiplied), padding codes
+    other than 128, wrapping parameters, and the unclamped last positions of a plane."""
+    g = cases.rng(2000)
+    prms = (dict(a_off=-117, b_off=-128, c_off=32513, c_mult=1028, c_shift=18),
+            dict(a_off=-255, b_off=3, c_off=-12345, c_mult=511, c_shift=14),
+            dict(a_off=-100, b_off=-90, c_off=5000, c_mult=700, c_shift=19))
+    #        B  Ci   H   W   Co  kH kW padH padW pool
+    shapes = ((2, 192, 13, 13, 384, 3, 3, 1, 1, 0),
+              (2, 64, 27, 27, 192, 5, 5, 2, 2, 1),
+              (3, 256, 13, 13, 256, 3, 3, 1, 1, 1),
+              (2, 64, 27, 27, 64, 5, 5, 2, 2, 0),
+              (1, 128, 9, 20, 64, 2, 3, 0, 1, 0),
+              (2, 384, 13, 13, 128, 3, 3, 1, 1, 0),
+              (1, 64, 40, 60, 64, 3, 3, 1, 1, 1),
+              (1, 64, 7, 100, 128, 3, 3, 0, 0, 0))
+    for ci, (B, Ci, H, W, Co, kH, kW, pH, pW, pool) in enumerate(shapes):
+        xq = g.integers(0, 256, (B, Ci, H, W), dtype=np.uint8)
+        wq = g.integers(0, 256, (Co, Ci, kH, kW), dtype=np.uint8)
+        addend = g.integers(-60, 61, Co).astype(np.int32)
+        prm = prms[ci % len(prms)]
+        zero = 128 if ci % 2 == 0 else 77
+        oH, oW = H + 2 * pH - kH + 1, W + 2 * pW - kW + 1
+        assert hiplib.thhip_conv2d_u8_patch_supported(B, Ci, H, W, Co, kH, kW, 1, 1, pH, pW, pool), ci
+        conv = np.empty((B, Co, oH, oW), np.uint8)
+        for b in range(B):
+            col = oracle.lowp_unfold(xq[b], (kH, kW), (1, 1), (pH, pW), zero)
+            plain = oracle.lowp_gemm(wq.reshape(Co, -1), col, **prm)
+            for o in range(Co):
+                conv[b, o] = oracle.lowp_add(plain[o], int(addend[o])).reshape(oH, oW)
+        want = oracle.lowp_threshold(conv, 100, 97)
+        if pool:
+            want = oracle.lowp_maxpool(want, 3, 3, 2, 2)
+        yh, yw = want.shape[2:]
+        G.note("conv2d_u8_patch x%s w%s pad(%d,%d) pool%d prm%s zero%d" % (xq.shape, wq.shape, pH, pW, pool, prm, zero))
+        wp = hiplib.thhip_conv_pack_weight_u8_patch(wq.ctypes.data, Co, Ci, kH, kW)
+        dx = api.DeviceArray(hiplib, np.ascontiguousarray(xq.transpose(0, 2, 3, 1)))
+        da = api.DeviceArray(hiplib, addend)
+        dy = api.DeviceArray(hiplib, nbytes=B * yh * yw * Co)
+        hiplib.thhip_memset(dy.ptr, 0x5a, B * yh * yw * Co)
+        hiplib.thhip_conv2d_u8_patch(dx.ptr, wp, da.ptr, dy.ptr, B, Ci, H, W, Co, kH, kW, 1, 1, pH, pW, zero,
+                                     prm["a_off"], prm["b_off"], prm["c_off"], prm["c_mult"], prm["c_shift"], 1, 100, 97, pool)
+        hiplib.thhip_sync()
+        got = dy.get((B, yh, yw, Co), np.uint8).transpose(0, 3, 1, 2)
+        assert np.array_equal(got, want), (ci, int((got != want).sum()))
+        hiplib.thhip_free(wp)
+    assert not hiplib.thhip_conv2d_u8_patch_supported(1, 64, 13, 13, 64, 3, 3, 2, 2, 1, 1, 0)    # stride 2
+    assert not hiplib.thhip_conv2d_u8_patch_supported(1, 96, 13, 13, 64, 3, 3, 1, 1, 1, 1, 0)    # 96 planes
+    assert not hiplib.thhip_conv2d_u8_patch_supported(1, 64, 13, 13, 64, 1, 1, 1, 1, 0, 0, 0)    # one tap
+    assert not hiplib.thhip_conv2d_u8_patch_supported(1, 64, 13, 300, 64, 3, 3, 1, 1, 1, 1, 0)   # rows of 300 positions
+
+
 def _linear_u8(hiplib, xq, wq, addend, prm, act=0, thr=0, val=0):
     B, K = xq.shape
     nOut = wq.shape[0]

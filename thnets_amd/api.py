@@ -124,6 +124,9 @@ PROTOTYPES = {
     "thhip_conv2d_u8_layout_tail": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3 + [C.c_int] * 3),
     "thhip_conv2d_u8_image_pool_supported": (C.c_int, [C.c_int] * 18),
     "thhip_conv2d_u8_image_pool": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3),
+    "thhip_conv2d_u8_patch_supported": (C.c_int, [C.c_int] * 12),
+    "thhip_conv_pack_weight_u8_patch": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),
+    "thhip_conv2d_u8_patch": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3 + [C.c_int]),
     "thhip_maxpool_u8_cl": (None, [vp, vp] + [C.c_int] * 12),
     "thhip_relayout_u8": (None, [vp, vp] + [C.c_int] * 4),
     "thhip_linear_batched_u8_supported": (C.c_int, [C.c_int] * 3),

@@ -29,6 +29,7 @@ struct hipmod {
 	/* uint8 engine */
 	int *addend;		/* per-plane bias addend (device) */
 	unsigned char *wrow_u8;	/* row-major weight codes for one-position layers (device) */
+	void *wpatch_u8;	/* the weights packed for the kernel that keeps the input patch in LDS (device), or NULL */
 	int *rowsum_u8;		/* their re-centred row sums (device) */
 	unsigned char *wq_host;	/* weight codes on the host, only while the network is being built */
 	/* SpatialFullConvolution: columns scratch; SpatialMaxPooling feeding a SpatialMaxUnpooling: its indices */
