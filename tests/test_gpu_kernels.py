@@ -345,6 +345,44 @@ def test_conv_half_channels_last(hiplib, oracle, dt):
             hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
+@pytest.mark.parametrize("dt", [G.F32, G.F16, G.BF16])
+def test_conv_image_layer_from_lds_patch(hiplib, oracle, dt):
+    """The 3 -> 64 n planes, 3x3, stride 1, padding 1 image layer that runs from an input
+    patch in LDS: ragged widths and heights (part tiles, part bands), one to four rows per
+    workgroup (batch x height decides), 64 / 128 / 192 planes, with and without the folded
+    batch-norm factor and Threshold, channels-last output for the half types; against the
+    fp32 restatement on the rounded operands and against the generic kernel (a forced tile)."""
+    from thnets_amd import api
+    g = cases.rng(4100 + dt)
+    tol = FP32_TOL if dt == G.F32 else HALF_TOL
+    shapes = [(1, 7, 5, 64), (2, 33, 70, 64), (1, 224, 224, 64), (3, 40, 31, 128), (40, 13, 32, 64), (300, 3, 9, 64),
+              (2, 1, 1, 192), (1, 600, 97, 64)]
+    for (B, H, W, Co) in shapes:
+        x = g.uniform(-1, 1, (B, 3, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
+        wr = api.from_device_dtype(api.to_device_dtype(hiplib, w, dt), w.shape, dt)
+        raw = oracle.conv2d(xr, wr, None, (1, 1), (1, 1))
+        for (scale, act) in ((None, 0), (sc, 1)):
+            want = raw * (scale[None, :, None, None] if scale is not None else 1) + b[None, :, None, None]
+            if act:
+                want = np.where(want > 0.05, want, np.float32(-0.5))
+            kw = dict(act=act, thr=0.05, val=-0.5, dtype=dt, scale=scale)
+            got = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), **kw)
+            G.assert_close(got, want, tol, "stem " + str((B, H, W, Co, act)))
+            try:
+                hiplib.thhip_conv_set_tuning(64, 64, 1, 0)
+                generic = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), **kw)
+            finally:
+                hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+            G.assert_close(got, generic, 2e-6 if dt == G.F32 else 1e-2, "stem vs generic " + str((B, H, W, Co, act)))
+            if dt != G.F32:
+                cl = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), y_cl=1, **kw)
+                assert np.array_equal(cl, got), "channels-last output " + str((B, H, W, Co, act))
+
+
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_conv_half_wide_tile(hiplib, oracle, dt):
     """The tiles whose operands go from global memory straight to LDS, every shape: K-tile

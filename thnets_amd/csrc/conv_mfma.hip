@@ -3137,7 +3137,12 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 			p.y_cl = f_y_cl;
 			p.pool = f_pool2;
 			ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N);
-			THHIP_DISPATCH_FLOAT(dtype, conv_dispatch<DT>(p));
+			/* a 3x3 image layer: whole rows from a patch in LDS (conv_stem.hip), unless a test forces a tile */
+			if (!f_pool2 && xl == 0 && !g_force_bm &&
+			    thhip_conv_stem_ok(bn, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, dtype, f_y_cl))
+				thhip_conv_stem(p.x, wpacked, p.KC, scale, bias, p.y, bn, H, W, Co, act, thr, val, dtype, f_y_cl);
+			else
+				THHIP_DISPATCH_FLOAT(dtype, conv_dispatch<DT>(p));
 		}
 	}
 }

@@ -21,6 +21,13 @@ void thhip_prof_end(int token, double work);
 int thhip_conv_u8_packed_chunks(int Ci, int kH, int kW, int x_layout);
 size_t thhip_conv_u8_packed_code_bytes(int Co, int Ci, int kH, int kW, int x_layout);
 
+/* conv_stem.hip: 3 -> 64 n planes, 3x3, stride 1, padding 1 on plane-major input, read from
+ * weights packed by thhip_conv_pack_weight_layout (KC chunks per 32-row block) */
+bool thhip_conv_stem_ok(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int dtype, int y_cl);
+void thhip_conv_stem(const void *x, const void *wpacked, int KC, const float *scale, const float *bias, void *y,
+	int B, int H, int W, int Co, int act, float thr, float val, int dtype, int y_cl);
+
 struct ThhipLaunchScope {
 	int token;
 	double work;
