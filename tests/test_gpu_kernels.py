@@ -345,6 +345,53 @@ def test_conv_half_channels_last(hiplib, oracle, dt):
             hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
+def test_conv_f32_with_pooling_in_the_epilogue(hiplib, oracle):
+    """fp32 convolution -> (factor, bias, Threshold) -> 2x2 / stride 2 max pooling in one
+    kernel: against the pooling kernel on the plain convolution's output (the same comparisons;
+    the sums differ in their last bits only where one of the two runs cut a tile along K, since
+    the positions are tiled in another order) and against the restatement.
+    Odd output sizes (the pooling drops the last row / column), strides, 64- and 128-plane
+    tiles, tiles cut along K, both K-tile depths."""
+    from thnets_amd import api
+    g = cases.rng(5200)
+    shapes = [(20, 32, 47, 45, 64, 3, 3, 1, 1, 1, 1), (12, 64, 64, 96, 128, 3, 3, 1, 1, 1, 1), (32, 32, 71, 70, 96, 5, 5, 2, 2, 2, 2),
+              (32, 64, 36, 36, 64, 3, 3, 1, 1, 1, 1), (1, 32, 130, 129, 128, 1, 1, 1, 1, 0, 0), (16, 96, 30, 30, 192, 3, 3, 1, 1, 1, 1)]
+    for (B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW) in shapes:
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, kH, kW), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * kH * kW)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        oH, oW = (H + 2 * pH - kH) // dH + 1, (W + 2 * pW - kW) // dW + 1
+        args = (B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW, G.F32, 0, 0)
+        assert hiplib.thhip_conv2d_pool2_supported(*args), args
+        wp = hiplib.thhip_conv_pack_weight_layout(w.ctypes.data, Co, Ci, kH, kW, G.F32, 0)
+        dx, db, ds = api.DeviceArray(hiplib, x), api.DeviceArray(hiplib, b), api.DeviceArray(hiplib, sc)
+        dy = api.DeviceArray(hiplib, nbytes=B * Co * oH * oW * 4)
+        dp = api.DeviceArray(hiplib, nbytes=B * Co * (oH // 2) * (oW // 2) * 4)
+        dq = api.DeviceArray(hiplib, nbytes=B * Co * (oH // 2) * (oW // 2) * 4)
+        for (scale, act) in ((None, 0), (ds, 1)):
+            G.note("conv+pool fp32 %s act %d" % (args, act))
+            sp = scale.ptr if scale else None
+            hiplib.thhip_conv2d_layout(dx.ptr, wp, sp, db.ptr, dy.ptr, B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW, act, 0.05, 0.05, G.F32, 0, 0)
+            hiplib.thhip_maxpool(dy.ptr, dp.ptr, B, Co, oH, oW, oH // 2, oW // 2, 2, 2, 2, 2, 0, 0, G.F32)
+            hiplib.thhip_conv2d_layout_pool2(dx.ptr, wp, sp, db.ptr, dq.ptr, B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW, act, 0.05, 0.05,
+                                             G.F32, 0, 0)
+            hiplib.thhip_sync()
+            plain = dp.get((B, Co, oH // 2, oW // 2), np.float32)
+            fused = dq.get((B, Co, oH // 2, oW // 2), np.float32)
+            G.assert_close(fused, plain, 4e-6, "conv+pool vs conv, pool " + str(args))
+            raw = oracle.conv2d(x, w, None, (dH, dW), (pH, pW))
+            want = raw * (sc[None, :, None, None] if scale else 1) + b[None, :, None, None]
+            if act:
+                want = np.where(want > 0.05, want, np.float32(0.05))      # (continuous: a sum next to the threshold moves the result little)
+            want = want[:, :, :oH // 2 * 2, :oW // 2 * 2].reshape(B, Co, oH // 2, 2, oW // 2, 2).max(axis=(3, 5))
+            G.assert_close(fused, want, FP32_TOL, "conv+pool " + str(args))
+        hiplib.thhip_free(wp)
+    # layers the K split takes, and forced tiles, are not pooled in the epilogue
+    assert not hiplib.thhip_conv2d_pool2_supported(16, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1, G.F32, 0, 0)
+    assert not hiplib.thhip_conv2d_pool2_supported(16, 3, 224, 224, 64, 3, 3, 1, 1, 1, 1, G.F32, 0, 0)
+
+
 @pytest.mark.parametrize("dt", [G.F32, G.F16, G.BF16])
 def test_conv_image_layer_from_lds_patch(hiplib, oracle, dt):
     """The 3 -> 64 n planes, 3x3, stride 1, padding 1 image layer that runs from an input

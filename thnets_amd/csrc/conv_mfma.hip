@@ -25,6 +25,7 @@
  * are stored [chunk][32-row block][h][32][16 B]: every ds_read_b128 /
  * ds_write_b128 of a wave touches 1 KiB contiguous, i.e. no bank conflicts.
  */
+#include <float.h>
 #include <stdlib.h>
 #include <string.h>
 #include <type_traits>
@@ -50,7 +51,9 @@ struct ConvParams {
 	int mparts;		/* the tile grid is cut mparts x (8 / mparts) over the XCDs */
 	unsigned x_bytes;
 	unsigned w_bytes;	/* packed weights (the wide kernel's buffer descriptor) */
-	int pool;		/* half types, conv_patch_kernel: the 2x2 / stride 2 max pooling that follows is done in the epilogue */
+	int pool;		/* the 2x2 / stride 2 max pooling that follows is done in the epilogue (conv_patch_kernel, conv_f32_direct_kernel) */
+	int pW, pHW, npool;	/* pooled width, plane size and positions in all; conv_f32_direct_kernel then walks the
+				 * positions in blocks of 64 = sixteen windows (conv_pool_member), N = 64 ceil(npool / 16) */
 	unsigned x_tail;	/* uint8: bytes of the padding code that follow x (0: none) */
 	/* split-K: S workgroups share an output tile, each over a K range */
 	int splitk;
@@ -1829,6 +1832,30 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
  * conv_f32_direct_kernel (2 x 2 waves): (folded batch norm factor,) bias,
  * optional threshold, plane-major store.  lrow: 2 * BM ints of LDS no wave
  * still reads. */
+/* conv_f32_direct_kernel with the 2x2 / stride 2 pooling in its epilogue: member t of a block of
+ * 64 positions.  The block is sixteen neighbouring pooling windows; t = 32 half + 16 dy + 2 w + dx
+ * is column dx of row dy of window 8 half + w.  Sixteen neighbouring lanes thus gather sixteen
+ * neighbouring pixels of a row (whole 64-byte runs, as without the pooling), a 32-position MFMA
+ * tile holds eight whole windows, the other column of a window is the next lane and the other
+ * row is lane ^ 16. */
+__device__ __forceinline__ void conv_pool_member(int n, int &pp, int &dy, int &dx)
+{
+	pp = (n >> 6) * 16 + ((n >> 5) & 1) * 8 + ((n >> 1) & 7);
+	dy = (n >> 4) & 1;
+	dx = n & 1;
+}
+
+/* v of lane + 1 (for even lanes), v of lane ^ 16 */
+__device__ __forceinline__ float conv_lane_next(float v)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xF5, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float conv_lane_xor16(float v)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+}
+
 template <int BM, int BN, int TM, int TN>
 __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, floatx16 (&acc)[TM][TN], int tile_m, int tile_n, int *lrow)
 {
@@ -1842,13 +1869,22 @@ __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, float
 	}
 	__syncthreads();
 	const bool has_scale = p.scale != 0;
+	/* With the pooling the first lane of a window (conv_pool_member) takes the maximum, with
+	 * SpatialMaxPooling.c:51-66's comparisons in their order, and stores it. */
+	const int oHW = p.pool ? p.pHW : p.oHW;
 #pragma unroll
 	for (int j = 0; j < TN; j++) {
 		const int n = tile_n * BN + (wn * TN + j) * 32 + (lane & 31);
-		if (n >= p.N)
+		int pos = n;
+		bool valid = n < p.N;
+		if (p.pool) {
+			int dy, dx;
+			conv_pool_member(n, pos, dy, dx);
+			valid = pos < p.npool && !dy && !dx;
+		} else if (!valid)
 			continue;
-		const int b = n / p.oHW, rem = n - b * p.oHW;
-		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+		const int b = pos / oHW, rem = pos - b * oHW;
+		const size_t ybase = (size_t)b * p.Co * oHW + rem;
 #pragma unroll
 		for (int i = 0; i < TM; i++) {
 			const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
@@ -1865,8 +1901,18 @@ __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, float
 					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
 					if (p.act)
 						v = v > p.thr ? v : p.val;
-					if (m < p.Co)
-						y[ybase + (size_t)m * p.oHW] = v;
+					if (p.pool) {
+						const float v01 = conv_lane_next(v);
+						const float v10 = conv_lane_xor16(v), v11 = conv_lane_xor16(v01);
+						float mx = -FLT_MAX;
+						mx = v > mx ? v : mx;
+						mx = v01 > mx ? v01 : mx;
+						mx = v10 > mx ? v10 : mx;
+						mx = v11 > mx ? v11 : mx;
+						v = mx;
+					}
+					if (valid && m < p.Co)
+						y[ybase + (size_t)m * oHW] = v;
 				}
 			}
 		}
@@ -1942,8 +1988,22 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		const int n_glob = tile_n * BN + q * 64 + lane;
 		n_ok_[q] = n_glob < p.N;
 		const int nn = n_ok_[q] ? n_glob : 0;
-		const int b = nn / p.oHW, r = nn - b * p.oHW;
-		const int oy = r / p.oW, ox = r - oy * p.oW;
+		int b, oy, ox;
+		if (p.pool) {
+			int pp, dy, dx;
+			conv_pool_member(n_glob, pp, dy, dx);
+			n_ok_[q] = pp < p.npool;
+			pp = n_ok_[q] ? pp : 0;
+			b = pp / p.pHW;
+			const int r = pp - b * p.pHW, py = r / p.pW;
+			oy = 2 * py + dy;
+			ox = 2 * (r - py * p.pW) + dx;
+		} else {
+			b = nn / p.oHW;
+			const int r = nn - b * p.oHW;
+			oy = r / p.oW;
+			ox = r - oy * p.oW;
+		}
 		iy0_[q] = oy * p.dH - p.padH;
 		ix0_[q] = ox * p.dW - p.padW;
 		xoff_[q] = b * p.Ci * p.HW + iy0_[q] * p.W + ix0_[q];
@@ -2785,6 +2845,8 @@ static void conv_dispatch(ConvParams &p)
 	 * for the operand reuse, 64x64 below.
 	 * Splitting K measured slower than unsplit 64x64 tiles on every layer that
 	 * has tiles for all CUs, so only layers of a few tiles are split (below). */
+	if (p.pool && DT == THHIP_F32)
+		p.N = 64 * ((p.npool + 15) / 16);	/* whole pooling windows only: a last odd row or column is not computed */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	const long t64 = (long)((p.Co + 63) / 64) * ((p.N + 63) / 64);
 	int bm = 64, bn = 64, splitk = 1, wgs = 0, kch = conv_kch(DT, p.x_cl != 0);
@@ -2904,8 +2966,10 @@ static void conv_dispatch(ConvParams &p)
 		wgs = g_force_wgs;
 	if (DT == THHIP_F32 && g_force_kch)
 		kch = g_force_kch;
-	if (p.pool)
-		bm = 64, bn = 1;	/* only the patch kernel pools */
+	if (p.pool && DT != THHIP_F32)
+		bm = 64, bn = 1;	/* of the half-type kernels only the patch kernel pools */
+	if (p.pool && DT == THHIP_F32 && (!direct || splitk != 1))
+		THError("thhip_conv2d: fp32 pooling in the epilogue needs the tiles loaded straight into LDS, without a K split");
 	if (bn == 1) {	/* (64, 1): the patch kernel */
 		if (!conv_patch_ok<DT>(p))
 			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64 or 128 planes, 3x3, stride 1");
@@ -3080,6 +3144,9 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 		p.KC = conv_kc(Ci, kH, kW, dtype, xl);
 		p.N = bn * oH * oW;
 		p.oHW = oH * oW;
+		p.pW = oW / 2;
+		p.pHW = (oH / 2) * (oW / 2);
+		p.npool = bn * p.pHW;
 		p.HW = H * W;
 		p.kHW = kH * kW;
 		p.magic_khw = (unsigned)conv_magic(kH * kW);
@@ -3170,10 +3237,23 @@ extern "C" void thhip_conv2d_layout(const void *x, const void *wpacked, const fl
 
 /* Whether thhip_conv2d_layout_pool2 takes this layer (and is the kernel the
  * layer would run on anyway): half type, channels-last input of 64 or 128
- * planes, 3x3, stride 1, enough tiles. */
+ * planes, 3x3, stride 1, enough tiles; or fp32, plane-major, planes in blocks
+ * of 32 and enough tiles that K is not split. */
 extern "C" int thhip_conv2d_pool2_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
 	int padH, int padW, int dtype, int x_layout, int y_channels_last)
 {
+	if (dtype == THHIP_F32) {
+		/* conv_f32_direct_kernel without a K split (conv_dispatch's choice for more than 512 tiles of 64 x 64) */
+		if (x_layout || y_channels_last || Ci % 32 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
+			return 0;
+		const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
+		if (oW < 2 || oH < 2)
+			return 0;
+		if ((double)B * Ci * H * W * 4 >= 2147483000.0 || (double)B * Co * oH * oW * 4 >= 2147483000.0)
+			return 0;	/* (the batch would be cut into slices) */
+		const long t64 = (long)((Co + 63) / 64) * (((long)B * (oH / 2) * (oW / 2) + 15) / 16);
+		return t64 > 512 && !g_force_kch && !g_force_bm && !g_force_bn && !g_force_splitk;
+	}
 	if (dtype != THHIP_F16 && dtype != THHIP_BF16)
 		return 0;
 	if (x_layout != 1 || (Ci != 64 && Ci != 128) || kH != 3 || kW != 3 || dH != 1 || dW != 1 || padH < 0 || padW < 0)

@@ -1289,11 +1289,12 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 #undef FEEDS_ONLY
 	free(consumers);
 	plan_channels_last(hn, net);
-	/* half engines: a 2x2 / stride 2 max pooling right after a convolution (and its
-	 * folded Threshold) between channels-last tensors may be done by the
+	/* a 2x2 / stride 2 max pooling right after a convolution (and its folded
+	 * Threshold; half engines: between channels-last tensors) may be done by the
 	 * convolution's epilogue; whether it is, is decided per forward by the layer's shape */
-	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIP && dtype != THHIP_F32; i++) {
-		if (!is_conv_type(hn->pub.modules[i].type) || hn->hm[i].is_linear || !hn->hm[i].in_cl)
+	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIP; i++) {
+		/* (fp32: plane-major tensors, the kernel that loads its tiles straight into LDS) */
+		if (!is_conv_type(hn->pub.modules[i].type) || hn->hm[i].is_linear || (dtype != THHIP_F32 && !hn->hm[i].in_cl))
 			continue;
 		int j = i + 1;
 		while (j < net->nelem && hn->hm[j].passthrough)
