@@ -4,12 +4,15 @@
 
 One "step" is one THForward of the VGG-16-shape network (fp32, batch 16, 3x224x224,
 synthetic seeded input and weights) with the input already resident in HBM; the
-value is whole-job images/second.  The same run also times the uint8 AlexNet-OWT
-batch-64 network (reported under "extra"), measures the convolution kernel family
-with HIP events around every launch inside the timed region (-> "roofline"), and
-times the CPU baseline on the host cores (-> "cpu_baseline": the reference's own
-CPU library when oracle/_ref holds a build of it, else this repository's C
-restatement).  Prints one JSON line.
+value is whole-job images/second.  The same run also measures the convolution kernel
+family with HIP events around every launch inside the timed region (-> "roofline"),
+times the same network through THProcessFloat call by call as the reference's CLI does
+(-> "process_float": best and mean of at least 20 calls after 2 warm-ups, host
+transfers included), times the uint8 AlexNet-OWT batch-64 network (-> "roofline_int8"
+and "extra"), the fp16 VGG-16, AlexNet-OWT batch 1 and ResNet-18 networks (-> "extra"),
+what the matrix cores sustain from registers alone (-> "extra"), and the CPU baseline
+on the host cores (-> "cpu_baseline": the reference's own CPU library when oracle/_ref
+holds a build of it, else this repository's C restatement).  Prints one JSON line.
 """
 import argparse
 import ctypes as C
@@ -28,10 +31,20 @@ from thnets_amd import api, configs  # noqa: E402
 
 PEAK_TFLOPS_FP32_MFMA = 157.3
 PEAK_TOPS_INT8_MFMA = 5030.0
-# Bytes moved past L2 per convolution launch in the VGG-16 b16 step (average of the 13), from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled against a 256 MiB copy
-# (profiles/conv_f32_vgg16_fp32_b16_counters.md); algorithmic bytes are 115.9e6.
-CONV_HBM_BYTES_PER_LAUNCH = 175.0e6
+
+
+def counter_traffic(profile, key):
+    """HBM bytes per launch as the counter summary under profiles/ states them: the line
+    `<key> = <bytes>` of that file (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this program,
+    scaled against a plain copy of known size), or None when the summary is not there."""
+    try:
+        with open(os.path.join(ROOT, "profiles", profile)) as f:
+            for line in f:
+                if line.strip().startswith(key + " ="):
+                    return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def profile_get(lib, fam):
@@ -155,8 +168,12 @@ def main():
     value = 16.0 / (ms * 1e-3)
     achieved = conv_flops / (conv_ms * 1e-3) / 1e12 if conv_ms > 0 else 0.0
     roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
-                "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4), "traffic": CONV_HBM_BYTES_PER_LAUNCH,
-                "kernel": "conv_f32_direct_kernel (implicit-GEMM convolution, operands loaded straight into LDS; 12 of the 13 convolutions of a step, with the kernels that sum the K parts of the three 14x14 layers and of the last tiles of eight others; the image layer on conv_mfma_kernel<fp32>)",
+                "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4),
+                "traffic": counter_traffic("conv_f32_vgg16_fp32_b16_counters.md", "conv_hbm_bytes_per_launch"),
+                "kernel": "conv_f32_direct_kernel (implicit-GEMM convolution, operands loaded straight into LDS; 12 of the 13 "
+                          "convolutions of a step, four of them with the 2x2 max pooling that follows in their epilogue, with the "
+                          "kernels that sum the K parts of the three 14x14 layers and of the last tiles of eight others; the image "
+                          "layer on conv_stem_kernel<fp32>)",
                 "launches_per_step": conv_n / args.steps, "avg_launch_ms": round(conv_ms / max(conv_n, 1), 5),
                 "flops_per_launch": conv_flops / max(conv_n, 1)}
     extra = {"vgg16_conv_ms_per_step": round(conv_ms / args.steps, 4),
@@ -170,15 +187,23 @@ def main():
     if fam[3][0] > 0:
         extra["vgg16_pooling_GB/s"] = round(fam[3][2] / (fam[3][0] * 1e-3) / 1e9, 1)
         extra["vgg16_pooling_frac_of_hbm_peak"] = round(fam[3][2] / (fam[3][0] * 1e-3) / 8e12, 4)
-    # the same step through the drop-in call: host normalisation + H2D + kernels + D2H
-    # (the call normalises its argument in place: every call gets its own copy, made outside the timed region)
-    net.process_float(cfg["input"])
-    copies = [np.array(cfg["input"], np.float32, copy=True, order="C") for _ in range(5)]
+    # the same step through the drop-in call, timed the way the reference's CLI times it (thnets-test.c:161-200:
+    # a loop of THProcessFloat calls; its first GPU run is dropped): host normalisation + H2D + kernels + D2H,
+    # 2 warm-up calls, then every call on its own (the call normalises its argument in place: each gets a
+    # fresh copy, made outside the timed region)
+    calls = max(args.steps, 20)
     res, ow, oh = C.POINTER(C.c_float)(), C.c_int(), C.c_int()
-    t0 = time.perf_counter()
-    for x in copies:
+    times = []
+    for i in range(calls + 2):
+        x = np.array(cfg["input"], np.float32, copy=True, order="C")
+        t0 = time.perf_counter()
         lib.THProcessFloat(net.handle, x.ctypes.data, 16, 224, 224, 3, C.byref(res), C.byref(ow), C.byref(oh))
-    extra["vgg16_THProcessFloat_images_per_sec_pcie_inclusive"] = round(16 * 5 / (time.perf_counter() - t0), 1)
+        if i >= 2:
+            times.append(time.perf_counter() - t0)
+    process_float = {"images_per_sec_best": round(16.0 / min(times), 1),
+                     "images_per_sec_mean": round(16.0 * len(times) / sum(times), 1), "calls": len(times), "warmup": 2,
+                     "what": "B / wall time of one THProcessFloat call of the same network (normalisation on the host, "
+                             "H2D of the input, all kernels, D2H of the result): PCIe-inclusive, never `value`"}
     net.free()
 
     # ---- VGG-16 fp16 batch 16 (THHipHalfFloat(1): fp16 storage and MFMA, fp32 accumulation) ----
@@ -239,6 +264,7 @@ def main():
     n4.free()
 
     # ---- uint8 AlexNet-OWT batch 64 ----
+    roofline_int8 = None
     if not args.no_int8:
         c5 = configs.alexnet_lowp(batch=64)
         x5 = c5["input"].copy()
@@ -253,7 +279,32 @@ def main():
             "images_per_sec": round(64.0 / (ms5 * 1e-3), 1), "ms_per_step": round(ms5, 4),
             "conv_i8_TOP/s": round(i8_tops, 2), "frac_of_int8_mfma_peak": round(i8_tops / PEAK_TOPS_INT8_MFMA, 4),
             "dtype": "u8 x u8 -> i32", "workload": "AlexNet-OWT THMakeSpatial form, range 32 (BASELINE configs[4])"}
+        # the uint8 convolution family (the eight layers of a step, fc6-8 as one-position convolutions) like `roofline`:
+        # ops = 2 M K N B per launch over the time of the launches (events around each, in a second pass of K steps)
+        roofline_int8 = {
+            "bound": "mfma", "achieved": round(i8_tops, 3), "peak": PEAK_TOPS_INT8_MFMA, "unit": "TOP/s",
+            "frac": round(i8_tops / PEAK_TOPS_INT8_MFMA, 4),
+            "traffic": counter_traffic("conv_u8_alexnet_owt_b64_counters.md", "conv_hbm_bytes_per_launch"),
+            "kernel": "conv_u8_image_pool_kernel, conv_u8_patch_kernel<pool>, conv_wide_kernel<uint8>, linear_u8_kernel "
+                      "(uint8 AlexNet-OWT batch 64: eight launches per step)",
+            "launches_per_step": i8_n / max(args.steps, 20), "avg_launch_ms": round(i8_ms / max(i8_n, 1), 5),
+            "ops_per_launch": i8_ops / max(i8_n, 1),
+            "cpu_baseline": None,
+            "cpu_baseline_note": "no CPU baseline of the reference's LOWP path can exist for this workload: its GEMM is "
+                                 "gemmlowp, which the reference does not carry (lowp/gemm8.cc includes it from a directory "
+                                 "the user must fetch), and its uint8 forward holds one image (batch 64 is 64 engine "
+                                 "constructions); parity is against this repository's restatement, image by image"}
         n5.free()
+
+    # ---- what the matrix cores sustain from registers alone on this device (no memory traffic), for scale ----
+    extra["mfma_register_loop"] = {
+        "fp32_32x32x2_TFLOP/s_by_waves_per_simd": {str(w): round(lib.thhip_probe_mfma(0, w, 30.0) / 1e12, 1) for w in (1, 2, 3, 4)},
+        "fp16_32x32x16_TFLOP/s": round(lib.thhip_probe_mfma(1, 2, 600.0) / 1e12, 1),
+        "int8_32x32x32_TOP/s": round(lib.thhip_probe_mfma(3, 2, 600.0) / 1e12, 1),
+        "what": "MFMAs on four accumulators per wavefront with operands (random values) in registers and nothing else; "
+                "fp32 for about 30 ms per occupancy, fp16 and int8 with two wavefronts per SIMD for about 600 ms (their "
+                "rate climbs over the first few hundred ms of such a loop and falls with the operands' bit activity: all "
+                "zeros run at 2480 / 4960); the published peaks are 157.3 / 2500 / 5030"}
 
     cpu = None
     if not args.no_cpu:
@@ -266,7 +317,8 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "VGG-16 shape, fp32, batch 16, 3x224x224, THForward with the input resident in HBM "
                                "(BASELINE configs[2])", "batch": 16},
-        "roofline": roofline, "cpu_baseline": cpu, "extra": extra,
+        "roofline": roofline, "cpu_baseline": cpu, "process_float": process_float, "roofline_int8": roofline_int8,
+        "extra": extra,
     }
     print(json.dumps(line))
 

@@ -396,6 +396,13 @@ enum thhip_family { THHIP_FAM_CONV = 0, THHIP_FAM_GEMV = 1, THHIP_FAM_CONV_I8 = 
 void thhip_profile_enable(int on);
 void thhip_profile_reset(void);
 void thhip_profile_get(int family, double *ms, long *launches, double *work);
+/* What the matrix cores sustain from registers alone on this device: a loop of
+ * MFMAs (fp32 32x32x2, fp16 32x32x16 or int8 32x32x32; dtype THHIP_F32 /
+ * THHIP_F16 / THHIP_U8) on four accumulators per wavefront, `waves_per_simd`
+ * (1..8) wavefronts resident per SIMD, run for about `ms` milliseconds; returns
+ * operations per second (two per multiply-add).  A measurement aid (the
+ * reference has none: its thnets-test.c:214-235 prints GFLOP/s of whole layers). */
+double thhip_probe_mfma(int dtype, int waves_per_simd, double ms);
 
 /* Weight packing for the implicit-GEMM convolution: row-major
  * [Co][Ci][kHW = kH*kW] (SpatialConvolutionMM.c:141-144) -> the K-chunked,

@@ -76,6 +76,7 @@ PROTOTYPES = {
     "thhip_profile_enable": (None, [C.c_int]),
     "thhip_profile_reset": (None, []),
     "thhip_profile_get": (None, [C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_long), C.POINTER(C.c_double)]),
+    "thhip_probe_mfma": (C.c_double, [C.c_int, C.c_int, C.c_double]),
     "thhip_conv_pack_weight": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv_packed_bytes": (C.c_size_t, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv_unpack_rows": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int]),

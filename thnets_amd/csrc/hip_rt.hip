@@ -204,3 +204,135 @@ extern "C" void thhip_profile_get(int family, double *ms, long *launches, double
 	*launches = g_fam_n[family];
 	*work = g_fam_work[family];
 }
+
+/* ---- what the matrix cores sustain from registers alone ----
+ * A loop of MFMAs on four independent accumulators, operands in registers (random values), no
+ * memory traffic: the rate a convolution kernel could reach if everything else were free.
+ * `waves_per_simd` workgroups of four wavefronts per CU (1..8) are resident for the whole run.
+ * Measured on one MI355X: fp32 32x32x2 reaches 154 TFLOP/s with one or two wavefronts per SIMD
+ * but 117 with three and 87-101 with four and more; fp16 32x32x16 1.64-1.71 PFLOP/s and int8
+ * 32x32x32 3.5-3.7 POP/s with random operands once the loop has run for half a second (1.2
+ * PFLOP/s over its first 40 ms), 2.48 PFLOP/s and 4.96 POP/s with all-zero operands: the
+ * half and 8-bit rates are set by the power the operands' bit activity draws. */
+template <int DT>
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float *out, const float *in, int iters)
+{
+	float s = 0;
+	if constexpr (DT == THHIP_F32) {
+		floatx16 acc[4];
+		for (int i = 0; i < 4; i++)
+			for (int r = 0; r < 16; r++)
+				acc[i][r] = 0;
+		float a[8], b[8];
+		for (int u = 0; u < 8; u++) {
+			a[u] = in[(threadIdx.x * 8 + u) & 4095];
+			b[u] = in[(threadIdx.x * 8 + u + 1777) & 4095];
+		}
+		for (int it = 0; it < iters; it++) {
+#pragma unroll
+			for (int u = 0; u < 8; u++)
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+					acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u], b[u], acc[i], 0, 0, 0);
+		}
+		for (int i = 0; i < 4; i++)
+			for (int r = 0; r < 16; r++)
+				s += acc[i][r];
+	} else if constexpr (DT == THHIP_F16) {
+		floatx16 acc[4];
+		for (int i = 0; i < 4; i++)
+			for (int r = 0; r < 16; r++)
+				acc[i][r] = 0;
+		halfx8 a[8], b[8];
+		for (int u = 0; u < 8; u++)
+			for (int e = 0; e < 8; e++) {
+				a[u][e] = (_Float16)in[(threadIdx.x * 8 + u + 3 * e) & 4095];
+				b[u][e] = (_Float16)in[(threadIdx.x * 8 + u + 1777 + 5 * e) & 4095];
+			}
+		for (int it = 0; it < iters; it++) {
+#pragma unroll
+			for (int u = 0; u < 8; u++)
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+					acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[u], b[u], acc[i], 0, 0, 0);
+		}
+		for (int i = 0; i < 4; i++)
+			for (int r = 0; r < 16; r++)
+				s += acc[i][r];
+	} else {
+		intx16 acc[4];
+		for (int i = 0; i < 4; i++)
+			for (int r = 0; r < 16; r++)
+				acc[i][r] = 0;
+		intx4 a[8], b[8];
+		for (int u = 0; u < 8; u++)
+			for (int e = 0; e < 4; e++) {
+				a[u][e] = (int)(in[(threadIdx.x * 8 + u + 3 * e) & 4095] * 2e9f);
+				b[u][e] = (int)(in[(threadIdx.x * 8 + u + 1777 + 5 * e) & 4095] * 2e9f);
+			}
+		for (int it = 0; it < iters; it++) {
+#pragma unroll
+			for (int u = 0; u < 8; u++)
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+					acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[u], b[u], acc[i], 0, 0, 0);
+		}
+		for (int i = 0; i < 4; i++)
+			for (int r = 0; r < 16; r++)
+				s += (float)acc[i][r];
+	}
+	out[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+/* Runs the loop above for about `ms` milliseconds and returns the rate in operations per
+ * second (2 per multiply-add); dtype THHIP_F32, THHIP_F16 or THHIP_U8 (signed 8-bit operands). */
+extern "C" double thhip_probe_mfma(int dtype, int waves_per_simd, double ms)
+{
+	if (waves_per_simd < 1 || waves_per_simd > 8 || ms <= 0 || (dtype != THHIP_F32 && dtype != THHIP_F16 && dtype != THHIP_U8))
+		THError("thhip_probe_mfma(%d, %d, %g): dtype fp32 / fp16 / uint8, 1 to 8 wavefronts per SIMD", dtype, waves_per_simd, ms);
+	thhip_init_once();
+	int dev, cus;
+	hipcheck(hipGetDevice(&dev));
+	hipcheck(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+	const int blocks = cus * waves_per_simd;
+	float host[4096];
+	unsigned long long st = 88172645463325252ull;
+	for (int i = 0; i < 4096; i++) {	/* xorshift64: uniform in [-1, 1) */
+		st ^= st << 13;
+		st ^= st >> 7;
+		st ^= st << 17;
+		host[i] = (float)((double)(st >> 11) / 9007199254740992.0 * 2.0 - 1.0);
+	}
+	float *in = (float *)thhip_malloc(sizeof(host)), *out = (float *)thhip_malloc((size_t)blocks * 256 * sizeof(float));
+	thhip_memcpy_h2d(in, host, sizeof(host));
+	const double per_mfma = dtype == THHIP_F32 ? 4096.0 : dtype == THHIP_F16 ? 32768.0 : 65536.0;
+	hipEvent_t e0, e1;
+	hipcheck(hipEventCreate(&e0));
+	hipcheck(hipEventCreate(&e1));
+	double rate = 0;
+	int iters = 64;
+	for (int pass = 0; pass < 2; pass++) {	/* a short run sizes the long one */
+		hipcheck(hipEventRecord(e0, g_stream));
+		if (dtype == THHIP_F32)
+			mfma_probe_kernel<THHIP_F32><<<dim3(blocks), dim3(256), 0, g_stream>>>(out, in, iters);
+		else if (dtype == THHIP_F16)
+			mfma_probe_kernel<THHIP_F16><<<dim3(blocks), dim3(256), 0, g_stream>>>(out, in, iters);
+		else
+			mfma_probe_kernel<THHIP_U8><<<dim3(blocks), dim3(256), 0, g_stream>>>(out, in, iters);
+		hipcheck(hipGetLastError());
+		hipcheck(hipEventRecord(e1, g_stream));
+		hipcheck(hipEventSynchronize(e1));
+		float t;
+		hipcheck(hipEventElapsedTime(&t, e0, e1));
+		rate = (double)blocks * 4 * iters * 32 * per_mfma / (t * 1e-3);
+		if (pass == 0) {
+			const double want = ms / (t > 1e-3 ? t : 1e-3) * iters;
+			iters = want > 5e7 ? 50000000 : want < 64 ? 64 : (int)want;
+		}
+	}
+	hipcheck(hipEventDestroy(e0));
+	hipcheck(hipEventDestroy(e1));
+	thhip_free(in);
+	thhip_free(out);
+	return rate;
+}
