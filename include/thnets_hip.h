@@ -463,6 +463,22 @@ void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, const float *
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, int x_layout, int y_channels_last);
 
+/* thhip_conv2d_affine followed by the two-input table add of a residual block and
+ * the Threshold(0, 0) after it, in the convolution's epilogue.  With v = the
+ * convolution's result (after factor, bias and its own Threshold) and r = res (a
+ * device tensor of y's shape): y = v + c r (mode 1) or r + c v (mode 2), then
+ * max(y, 0) if res_act.  Replaces SpatialConvolutionMM -> CAddTable -> Threshold
+ * (modules/CAddTable.c:59-70; c = -1 is the reference's two-input CAddTable, which
+ * subtracts) for the layers thhip_conv2d_residual_supported accepts (fp32,
+ * plane-major tensors, input planes in blocks of 32); bit for bit the values of
+ * thhip_conv2d_affine followed by thhip_axpby2. */
+int thhip_conv2d_residual_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int dtype);
+void thhip_conv2d_residual(const void *x, const void *wpacked, const float *scale, const float *shift,
+	const void *res, int mode, float c, int res_act, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype);
+
 /* Tuning override for tests and experiments: force the convolution's workgroup
  * tile (bm x bn in {64,128}), its split-K factor and the number of workgroups
  * allowed to share a CU; 0 leaves a choice automatic.  A forced tile runs on

@@ -345,6 +345,51 @@ def test_conv_half_channels_last(hiplib, oracle, dt):
             hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
+def test_conv_f32_with_table_add_in_the_epilogue(hiplib, oracle):
+    """fp32 convolution -> (factor, bias) -> two-input table add -> Threshold(0, 0) in one kernel:
+    bit for bit the convolution followed by thhip_axpby2 (the same sums in the same order, one
+    rounding per operation), both operand orders, layers that split K (the finishing kernel adds),
+    layers with tiles cut along K, 1x1 strided projections; and against the restatement with the
+    reference's a - b."""
+    from thnets_amd import api
+    g = cases.rng(5300)
+    shapes = [(4, 64, 56, 56, 64, 3, 3, 1, 1, 1, 1), (8, 32, 30, 30, 96, 3, 3, 1, 1, 1, 1), (4, 256, 14, 14, 256, 3, 3, 1, 1, 1, 1),
+              (6, 64, 56, 56, 128, 1, 1, 2, 2, 0, 0), (2, 512, 7, 7, 512, 3, 3, 1, 1, 1, 1), (32, 128, 28, 28, 128, 3, 3, 1, 1, 1, 1)]
+    for (B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW) in shapes:
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, kH, kW), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * kH * kW)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        oH, oW = (H + 2 * pH - kH) // dH + 1, (W + 2 * pW - kW) // dW + 1
+        r = g.standard_normal((B, Co, oH, oW), dtype=np.float32)
+        args = (B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW)
+        assert hiplib.thhip_conv2d_residual_supported(*args, G.F32), args
+        wp = hiplib.thhip_conv_pack_weight_layout(w.ctypes.data, Co, Ci, kH, kW, G.F32, 0)
+        dx, db, ds, dr = (api.DeviceArray(hiplib, a) for a in (x, b, sc, r))
+        n = B * Co * oH * oW
+        dy, dz, dq = (api.DeviceArray(hiplib, nbytes=n * 4) for _ in range(3))
+        raw = oracle.conv2d(x, w, None, (dH, dW), (pH, pW)) * sc[None, :, None, None] + b[None, :, None, None]
+        for mode in (1, 2):
+            for act in (0, 1):
+                G.note("conv + table add fp32 %s mode %d act %d" % (args, mode, act))
+                hiplib.thhip_conv2d_layout(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, *args, 0, 0.0, 0.0, G.F32, 0, 0)
+                if mode == 1:
+                    hiplib.thhip_axpby2(dy.ptr, dr.ptr, dz.ptr, n, n, -1.0, act, G.F32)
+                else:
+                    hiplib.thhip_axpby2(dr.ptr, dy.ptr, dz.ptr, n, n, -1.0, act, G.F32)
+                hiplib.thhip_conv2d_residual(dx.ptr, wp, ds.ptr, db.ptr, dr.ptr, mode, -1.0, act, dq.ptr, *args, 0, 0.0, 0.0, G.F32)
+                hiplib.thhip_sync()
+                plain, fused = dz.get((B, Co, oH, oW), np.float32), dq.get((B, Co, oH, oW), np.float32)
+                assert np.array_equal(plain, fused), (args, mode, act, np.abs(plain - fused).max())
+                want = raw - r if mode == 1 else r - raw
+                if act:
+                    want = np.maximum(want, 0)
+                G.assert_close(fused, want, FP32_TOL, "conv + table add " + str(args))
+        hiplib.thhip_free(wp)
+    assert not hiplib.thhip_conv2d_residual_supported(2, 3, 32, 32, 64, 3, 3, 1, 1, 1, 1, G.F32)
+    assert not hiplib.thhip_conv2d_residual_supported(2, 64, 32, 32, 64, 3, 3, 1, 1, 1, 1, G.F16)
+
+
 def test_conv_f32_with_pooling_in_the_epilogue(hiplib, oracle):
     """fp32 convolution -> (factor, bias, Threshold) -> 2x2 / stride 2 max pooling in one
     kernel: against the pooling kernel on the plain convolution's output (the same comparisons;

@@ -121,6 +121,9 @@ PROTOTYPES = {
     "thhip_conv_pack_weight_u8_layout": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d_u8_layout": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3 + [C.c_int] * 2),
     "thhip_conv2d_pool2_supported": (C.c_int, [C.c_int] * 14),
+    "thhip_conv2d_residual_supported": (C.c_int, [C.c_int] * 12),
+    "thhip_conv2d_residual": (None, [vp, vp, vp, vp, vp, C.c_int, C.c_float, C.c_int, vp] + [C.c_int] * 11 +
+                              [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv2d_layout_pool2": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d_u8_layout_tail": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3 + [C.c_int] * 3),
     "thhip_conv2d_u8_image_pool_supported": (C.c_int, [C.c_int] * 18),

@@ -52,6 +52,12 @@ struct ConvParams {
 	unsigned x_bytes;
 	unsigned w_bytes;	/* packed weights (the wide kernel's buffer descriptor) */
 	int pool;		/* the 2x2 / stride 2 max pooling that follows is done in the epilogue (conv_patch_kernel, conv_f32_direct_kernel) */
+	/* conv_f32_direct_kernel: a second tensor of the output's shape combined with the result after the
+	 * (factor,) bias and Threshold: res_mode 1: v + res_c * res, 2: res + res_c * v; then ReLU if res_act
+	 * (the table add of a residual block and the Threshold after it, modules/CAddTable.c:59-70) */
+	const float *res;
+	int res_mode, res_act;
+	float res_c;
 	int pW, pHW, npool;	/* pooled width, plane size and positions in all; conv_f32_direct_kernel then walks the
 				 * positions in blocks of 64 = sixteen windows (conv_pool_member), N = 64 ceil(npool / 16) */
 	unsigned x_tail;	/* uint8: bytes of the padding code that follow x (0: none) */
@@ -1888,6 +1894,15 @@ __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, float
 #pragma unroll
 		for (int i = 0; i < TM; i++) {
 			const int m0 = tile_m * BM + (wm * TM + i) * 32 + 4 * (lane >> 5);
+			/* the other tensor's sixteen values of this accumulator, all requested before the first is used */
+			float other[16];
+			if (p.res_mode) {
+#pragma unroll
+				for (int r = 0; r < 16; r++) {
+					const int m = m0 + 8 * (r >> 2) + (r & 3);
+					other[r] = valid && m < p.Co ? p.res[ybase + (size_t)m * oHW] : 0.0f;
+				}
+			}
 #pragma unroll
 			for (int g = 0; g < 4; g++) {
 				const int ml = (wm * TM + i) * 32 + 4 * (lane >> 5) + 8 * g;
@@ -1911,8 +1926,14 @@ __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, float
 						mx = v11 > mx ? v11 : mx;
 						v = mx;
 					}
-					if (valid && m < p.Co)
+					if (valid && m < p.Co) {
+						if (p.res_mode) {
+							v = p.res_mode == 1 ? v + p.res_c * other[r] : other[r] + p.res_c * v;
+							if (p.res_act)
+								v = v > 0.0f ? v : 0.0f;
+						}
 						y[ybase + (size_t)m * oHW] = v;
+					}
 				}
 			}
 		}
@@ -2254,7 +2275,7 @@ __global__ __launch_bounds__(256) void conv_f32_tail_finish_kernel(ConvParams p)
 /* Sums the parts of a K split, [part][plane][position] fp32, in their order and
  * finishes as the convolution epilogue does; plane-major output. */
 __global__ void conv_f32_splitk_finish_kernel(const float *ws, const float *bias, const float *scale, float *y,
-	int parts, int Co, int N, int oHW, int act, float thr, float val)
+	int parts, int Co, int N, int oHW, int act, float thr, float val, const float *res, int res_mode, float res_c, int res_act)
 {
 	const long total = (long)Co * N;
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -2268,7 +2289,14 @@ __global__ void conv_f32_splitk_finish_kernel(const float *ws, const float *bias
 		if (act)
 			v = v > thr ? v : val;
 		const int b = n / oHW, rem = n - b * oHW;
-		y[((size_t)b * Co + m) * oHW + rem] = v;
+		const size_t at = ((size_t)b * Co + m) * oHW + rem;
+		if (res_mode) {
+			const float r = res[at];
+			v = res_mode == 1 ? v + res_c * r : r + res_c * v;
+			if (res_act)
+				v = v > 0.0f ? v : 0.0f;
+		}
+		y[at] = v;
 	}
 }
 
@@ -2776,7 +2804,7 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 		if (blocks > 4096)
 			blocks = 4096;
 		conv_f32_splitk_finish_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
-			(float *)p.y, p.splitk, p.Co, p.N, p.oHW, p.act, p.thr, p.val);
+			(float *)p.y, p.splitk, p.Co, p.N, p.oHW, p.act, p.thr, p.val, p.res, p.res_mode, p.res_c, p.res_act);
 	}
 	if (p.tail_slots)
 		conv_f32_tail_finish_kernel<BM, BN><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
@@ -2968,6 +2996,8 @@ static void conv_dispatch(ConvParams &p)
 		kch = g_force_kch;
 	if (p.pool && DT != THHIP_F32)
 		bm = 64, bn = 1;	/* of the half-type kernels only the patch kernel pools */
+	if (p.res_mode && (DT != THHIP_F32 || !direct || p.pool))
+		THError("thhip_conv2d: a second tensor is combined only by the fp32 tiles loaded straight into LDS, without pooling");
 	if (p.pool && DT == THHIP_F32 && (!direct || splitk != 1))
 		THError("thhip_conv2d: fp32 pooling in the epilogue needs the tiles loaded straight into LDS, without a K split");
 	if (bn == 1) {	/* (64, 1): the patch kernel */
@@ -3104,9 +3134,16 @@ static unsigned char *conv_pixels4_scratch(size_t bytes)
 	return g_c4;
 }
 
+struct ConvResidual {
+	const float *res;
+	int mode, act;
+	float c;
+};
+
 static void conv_run(const void *x, const void *wpacked, const float *scale, const float *bias, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
-	int act, float thr, float val, int dtype, const ConvU8Args *u8, int f_x_layout = 0, int f_y_cl = 0, int f_pool2 = 0)
+	int act, float thr, float val, int dtype, const ConvU8Args *u8, int f_x_layout = 0, int f_y_cl = 0, int f_pool2 = 0,
+	const ConvResidual *f_res = 0)
 {
 	if (B < 1 || Ci < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
 		THError("thhip_conv2d: bad geometry");
@@ -3203,9 +3240,15 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 			p.x_cl = xl;
 			p.y_cl = f_y_cl;
 			p.pool = f_pool2;
+			if (f_res) {
+				p.res = f_res->res + (size_t)b0 * out_img;
+				p.res_mode = f_res->mode;
+				p.res_c = f_res->c;
+				p.res_act = f_res->act;
+			}
 			ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N);
 			/* a 3x3 image layer: whole rows from a patch in LDS (conv_stem.hip), unless a test forces a tile */
-			if (!f_pool2 && xl == 0 && !g_force_bm &&
+			if (!f_pool2 && !f_res && xl == 0 && !g_force_bm &&
 			    thhip_conv_stem_ok(bn, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, dtype, f_y_cl))
 				thhip_conv_stem(p.x, wpacked, p.KC, scale, bias, p.y, bn, H, W, Co, act, thr, val, dtype, f_y_cl);
 			else
@@ -3284,6 +3327,39 @@ extern "C" void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, co
 		THError("thhip_conv2d_layout_pool2: layer not supported (see thhip_conv2d_pool2_supported)");
 	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0,
 		x_layout, y_channels_last != 0, 1);
+}
+
+/* Whether thhip_conv2d_residual takes this layer: fp32, plane-major tensors, planes in blocks of 32 (the
+ * kernel that loads its tiles straight into LDS), the batch in one slice. */
+extern "C" int thhip_conv2d_residual_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int dtype)
+{
+	if (dtype != THHIP_F32 || Ci % 32 || B < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
+		return 0;
+	const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
+	if (oW < 1 || oH < 1)
+		return 0;
+	if ((double)B * Ci * H * W * 4 >= 2147483000.0 || (double)B * Co * oH * oW * 4 >= 2147483000.0)
+		return 0;
+	return !g_force_kch && !g_force_bm && !g_force_bn && !g_force_splitk;
+}
+
+/* thhip_conv2d_affine followed by the two-input table add of a residual block and the Threshold(0, 0)
+ * after it, in the convolution's epilogue: with v = the convolution's result (after factor, bias and its
+ * own Threshold) and r = res (a tensor of y's shape), y = v + c r (mode 1) or r + c v (mode 2), then
+ * max(y, 0) if res_act.  Replaces SpatialConvolutionMM -> CAddTable -> Threshold
+ * (modules/CAddTable.c:59-70 with the coefficient its caller gives: -1 for the reference's two-input
+ * CAddTable) for the layers thhip_conv2d_residual_supported accepts; the same values, bit for bit, as
+ * thhip_conv2d_affine followed by thhip_axpby2. */
+extern "C" void thhip_conv2d_residual(const void *x, const void *wpacked, const float *scale, const float *shift,
+	const void *res, int mode, float c, int res_act, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int act, float thr, float val, int dtype)
+{
+	if (!thhip_conv2d_residual_supported(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, dtype) || (mode != 1 && mode != 2) || !res)
+		THError("thhip_conv2d_residual: layer not supported (see thhip_conv2d_residual_supported), or mode %d not 1 or 2", mode);
+	const ConvResidual r = { (const float *)res, mode, res_act, c };
+	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0, 0, 0, 0, &r);
 }
 
 extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,

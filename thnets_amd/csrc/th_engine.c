@@ -205,6 +205,21 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 	}
 	void *y = conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
 	hn->cur_cl = hm->out_cl && oH * oW > 1;
+	/* the last convolution of a residual block: the table add and its Threshold in the epilogue */
+	if (hm->res_mode && hm->res_ptr) {
+		const void *res = hm->res_ptr;
+		const long res_n = hm->res_n;
+		hm->res_ptr = 0;
+		if (res != y && res_n == (long)s.B * c->nOutputPlane * oH * oW && s.outnd >= 3 &&
+		    thhip_conv2d_residual_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW,
+				c->padH, c->padW, dt)) {
+			thhip_conv2d_residual(x, hm->wpacked, hm->scale, hm->bias, res, hm->res_mode, hm->res_c, hm->res_act, y,
+				s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW, c->padH, c->padW,
+				hm->fused_act, hm->thr, hm->val, dt);
+			hm->res_add->added_by_producer = hm->res_mode;	/* mode 1: branch 0 holds the sum, mode 2: branch 1 */
+			return m->output;
+		}
+	}
 	/* the row-major copy is made from plane-major packing; for a 1x1 kernel the
 	 * channels-last packing is the same (k is the plane in both) */
 	const int one_position = oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
@@ -519,8 +534,20 @@ static THFloatTensor *Hip_Sequential_updateOutput(struct module *m, THFloatTenso
 static THFloatTensor *Hip_ConcatTable_updateOutput(struct module *m, THFloatTensor *in)
 {
 	struct network *net = m->ConcatTable.net;
-	for (int i = 0; i < net->nelem; i++)
+	struct hipmod *hm = hipmod_of(m);
+	struct hipmod *target = hm->res_target;
+	for (int i = 0; i < net->nelem; i++) {
+		if (target && i == (hm->res_from_input ? 0 : 1)) {
+			/* what the planned convolution combines its result with: the table's input (identity
+			 * branch), or what branch 0 has just made */
+			THFloatTensor *other = hm->res_from_input ? in : net->modules[0].output;
+			target->res_ptr = thhip_tensor_ptr(other, hipnet_of(m)->dtype);
+			target->res_n = THFloatTensor_nElement(other);
+		}
 		net->modules[i].updateOutput(&net->modules[i], in);
+	}
+	if (target)
+		target->res_ptr = 0;	/* (a convolution that did not run, or refused, leaves the add to the table add) */
 	return (THFloatTensor *)m;
 }
 
@@ -545,6 +572,11 @@ static THFloatTensor *Hip_CAddTable_updateOutput(struct module *m, THFloatTensor
 	}
 	THFloatTensor *a = mods[0].output;
 	const long na = THFloatTensor_nElement(a);
+	if (hm->added_by_producer) {	/* done, with the Threshold folded into this module, by a convolution's epilogue */
+		out_alias(m, mods[hm->added_by_producer - 1].output);
+		hm->added_by_producer = 0;
+		return m->output;
+	}
 	void *y = out_resize(m, dt, a->nDimension, a->size);
 	if (nelem == 2) {
 		THFloatTensor *b = mods[1].output;
@@ -1194,6 +1226,31 @@ static void plan_channels_last(struct hipnet *hn, struct network *src)
 	}
 }
 
+/* The convolution whose result is a ConcatTable branch's output: the branch itself, or the last
+ * module of a Sequential before its folded batch norms, if that is a convolution with no
+ * Threshold and no pooling of its own in its epilogue.  NULL otherwise. */
+static struct module *branch_last_conv(struct module *b)
+{
+	if (b->type == MT_Sequential && b->Sequential.net) {
+		struct network *sn = b->Sequential.net;
+		struct hipnet *shn = (struct hipnet *)sn;
+		int i = sn->nelem - 1;
+		if (shn->dag)
+			return 0;
+		while (i >= 0 && shn->hm[i].passthrough && sn->modules[i].type == MT_SpatialBatchNormalization)
+			i--;
+		if (i < 0)
+			return 0;
+		b = &sn->modules[i];
+	}
+	if (!is_conv_type(b->type))
+		return 0;
+	struct hipmod *hm = hipmod_of(b);
+	if (hm->is_linear || hm->fused_act || hm->pool_next || hm->passthrough)
+		return 0;
+	return b;
+}
+
 static int foldable_threshold(struct module *t)
 {
 	return t->type == MT_Threshold && t->Threshold.alpha == 0;
@@ -1320,6 +1377,29 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 		const struct SpatialMaxPooling *q = &hn->pub.modules[j].SpatialMaxPooling;
 		if (q->kW == 3 && q->kH == 3 && q->dW == 2 && q->dH == 2 && q->padW == 0 && q->padH == 0 && !q->ceil_mode)
 			hn->hm[i].pool_next = j;
+	}
+	/* fp32 residual blocks in table form, ConcatTable{main, shortcut} -> CAddTable (-> Threshold(0, 0)):
+	 * the add (and the Threshold folded into it) may be done by the epilogue of the convolution that
+	 * runs last in the table: the main branch's last one when the shortcut is the identity, else the
+	 * shortcut's (branch 0 has run by then).  Whether it is, is decided per forward by the layer's
+	 * shape; the table add then passes that convolution's tensor on. */
+	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIP && dtype == THHIP_F32 && !hn->dag; i++) {
+		struct module *ct = &hn->pub.modules[i], *add = &hn->pub.modules[i + 1];
+		if (ct->type != MT_ConcatTable || !ct->ConcatTable.net || ct->ConcatTable.net->nelem != 2 ||
+		    (add->type != MT_CAddTable && add->type != MT_CSubTable))
+			continue;
+		struct module *b0 = &ct->ConcatTable.net->modules[0], *b1 = &ct->ConcatTable.net->modules[1];
+		const int identity = b1->type == MT_Dropout || b1->type == MT_Identity;
+		struct module *conv = branch_last_conv(identity ? b0 : b1);
+		if (!conv)
+			continue;
+		struct hipmod *chm = hipmod_of(conv);
+		chm->res_mode = identity ? 1 : 2;
+		chm->res_c = add->type == MT_CSubTable ? 1.0f : -1.0f;	/* the arithmetic as shipped: CAddTable.c:59-70 */
+		chm->res_act = hn->hm[i + 1].fused_act;
+		chm->res_add = &hn->hm[i + 1];
+		hn->hm[i].res_target = chm;
+		hn->hm[i].res_from_input = identity;
 	}
 	for (int i = 0; i < net->nelem; i++)
 		if (hn->hm[i].wpatch_u8 && !hn->hm[i].pool_next) {	/* packed for a fusion that is not there */

@@ -16,6 +16,17 @@ struct hipmod {
 	int passthrough;	/* a Threshold whose work was folded into its producer */
 	int pool_next;		/* convolution: index of a 2x2 / stride 2 max pooling its epilogue may do (0: none) */
 	int pooled_by_producer;	/* max pooling: the convolution before it did the pooling in this forward */
+	/* fp32 residual blocks: the table add (and the Threshold folded into it) done by the epilogue of the
+	 * last convolution that runs in the ConcatTable before it */
+	int res_mode;		/* convolution: 1: result + res_c * other branch, 2: other branch + res_c * result; 0: none */
+	float res_c;
+	int res_act;
+	struct hipmod *res_add;	/* convolution: the table add's state, told when the epilogue did its work */
+	const void *res_ptr;	/* convolution: the other branch's values for this forward (set by the ConcatTable) */
+	long res_n;
+	struct hipmod *res_target;	/* ConcatTable: the convolution planned to do the add, or NULL */
+	int res_from_input;	/* ConcatTable: the other branch is the identity (the table's input), else branch 0's output */
+	int added_by_producer;	/* table add: 1 + the branch whose convolution did the add in this forward */
 	int is_linear;		/* MT_Linear in the source network */
 	int owns_output;	/* output storage was allocated by this module */
 	size_t cap;		/* bytes allocated for the output */
