@@ -503,10 +503,9 @@ def test_conv_half_wide_tile(hiplib, oracle, dt):
                 G.note("wide tile %s y_cl %d dtype %d" % ((B, Ci, H, W, Co, kH, kW, dH, dW, pH, pW), y_cl, dt))
                 hiplib.thhip_conv_set_tuning(128, 128, 0, 0)
                 narrow = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
-                # 256 positions: eight and four waves; for 256 rows K-tiles of 32 (four LDS stages) or,
-                # with the third argument 4 and Ci % 64 == 0, of 64 (two stages).  The smaller tiles
+                # 256 positions: eight and four waves, K-tiles of 32 in four LDS stages.  The smaller tiles
                 # (third argument 9: the kernel that loads straight into LDS): four waves, four stages.
-                for tune in ((256, 256, 0), (256, 256, 4), (128, 256, 0), (128, 128, 9), (128, 64, 9), (64, 128, 9), (64, 64, 9)):
+                for tune in ((256, 256, 0), (128, 256, 0), (128, 128, 9), (128, 64, 9), (64, 128, 9), (64, 64, 9)):
                     hiplib.thhip_conv_set_tuning(tune[0], tune[1], tune[2], 0)
                     got = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
                     G.assert_close(got, want, HALF_TOL, str((Ci, Co, kH, y_cl, tune)))

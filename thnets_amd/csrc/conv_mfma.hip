@@ -58,6 +58,7 @@ struct ConvParams {
 	const float *res;
 	int res_mode, res_act;
 	float res_c;
+	int cl_shift;		/* channels-last input in whole K-tiles of planes: log2 of the K-tile (K runs block, tap, plane); else 0 */
 	int pW, pHW, npool;	/* pooled width, plane size and positions in all; conv_f32_direct_kernel then walks the
 				 * positions in blocks of 64 = sixteen windows (conv_pool_member), N = 64 ceil(npool / 16) */
 	unsigned x_tail;	/* uint8: bytes of the padding code that follow x (0: none) */
@@ -411,8 +412,17 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 			cl_off = ((t_kh * p.W + t_kw) * p.Ci + t_cb) * (int)sizeof(elem);	/* scalar; t_cb counts planes */
 		} else if constexpr (CLI) {
 			const int kv = (kt * VPP + pv) * VEC;
-			const unsigned tap = (unsigned)kv * p.mhi_ci + __umulhi((unsigned)kv, p.magic_ci);
-			const int c = kv - tap * p.Ci;
+			unsigned tap;
+			int c;
+			if (p.cl_shift) {	/* K runs (block of planes, tap, plane of the block) */
+				const unsigned kb = (unsigned)kv >> p.cl_shift;
+				const unsigned blk = kb * p.mhi_khw + __umulhi(kb, p.magic_khw);
+				tap = kb - blk * p.kHW;
+				c = (int)(blk << p.cl_shift) + (kv & ((1 << p.cl_shift) - 1));
+			} else {
+				tap = (unsigned)kv * p.mhi_ci + __umulhi((unsigned)kv, p.magic_ci);
+				c = kv - tap * p.Ci;
+			}
 			const unsigned kh = tap * p.mhi_kw + __umulhi(tap, p.magic_kw);
 			cl_kh = (int)kh;
 			cl_kw = (int)(tap - kh * p.kW);
@@ -520,13 +530,12 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 			breg[set][j] = packed;
 		}
 		if constexpr (CLU) {
-			/* next block of planes of the tap, then the next tap */
-			t_cb += KCH * CHUNK;
-			if (t_cb == p.Ci) {
-				t_cb = 0;
-				if (++t_kw == p.kW) {
-					t_kw = 0;
-					++t_kh;
+			/* next tap of the block of planes, then the next block */
+			if (++t_kw == p.kW) {
+				t_kw = 0;
+				if (++t_kh == p.kH) {
+					t_kh = 0;
+					t_cb += KCH * CHUNK;
 				}
 			}
 		}
@@ -594,8 +603,8 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
 	const int kt0 = p.splitk > 1 ? (int)((long)nkt_all * split / p.splitk) : 0;
 	const int nkt = p.splitk > 1 ? (int)((long)nkt_all * (split + 1) / p.splitk) : nkt_all;
 	if constexpr (CLU) {
-		const int k0 = kt0 * KCH * CHUNK, tap = k0 / p.Ci;
-		t_cb = k0 - tap * p.Ci;
+		const int blk = kt0 / p.kHW, tap = kt0 - blk * p.kHW;
+		t_cb = blk * (KCH * CHUNK);
 		t_kh = tap / p.kW;
 		t_kw = tap - t_kh * p.kW;
 	}
@@ -1237,14 +1246,14 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
 		a_lds_[i] = (kci * MB + mbi) * 64;
 	}
-	/* K-tiles: tap outer, planes inner; a part of a cut tile walks [kt0, kt0 + nkt) */
+	/* K-tiles: block of planes outer, tap inner; a part of a cut tile walks [kt0, kt0 + nkt) */
 	const int nkt_all = p.KC / KCH;
 	const int kt0 = nsplit > 1 ? (int)((long)nkt_all * split / nsplit) : 0;
 	const int nkt = (nsplit > 1 ? (int)((long)nkt_all * (split + 1) / nsplit) : nkt_all) - kt0;
 	int t_cb, t_kh, t_kw, t_kc = kt0 * KCH;
 	{
-		const int per_tap = p.Ci / (KCH * CHUNK), tap = kt0 / per_tap;
-		t_cb = (kt0 - tap * per_tap) * (KCH * CHUNK);
+		const int blk = kt0 / p.kHW, tap = kt0 - blk * p.kHW;
+		t_cb = blk * (KCH * CHUNK);
 		t_kh = tap / p.kW;
 		t_kw = tap - t_kh * p.kW;
 	}
@@ -1265,12 +1274,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(lb + (wave + WAVES * q) * 64), 16, voff, 0, 0, 0);
 		}
 		t_kc += KCH;
-		t_cb += KCH * CHUNK;
-		if (t_cb == p.Ci) {
-			t_cb = 0;
-			if (++t_kw == p.kW) {
-				t_kw = 0;
-				++t_kh;
+		if (++t_kw == p.kW) {
+			t_kw = 0;
+			if (++t_kh == p.kH) {
+				t_kh = 0;
+				t_cb += KCH * CHUNK;
 			}
 		}
 	};
@@ -1632,11 +1640,12 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
 		a_lds_[i] = (kci * MB + mbi) * 64;
 	}
-	/* K-tile ikt of plane block t_cb: chunks (k = tap Ci + plane) / 16 */
+	/* K-tile ikt of the patch's 64 planes: tap ikt / 2 of its 32-plane block ikt % 2; K runs
+	 * (block of 32 planes, tap, plane), in chunks of 16 */
 	int ikt = 0, t_cb = 0;
 	auto issue = [&](auto st_) {
 		constexpr int st = decltype(st_)::value;
-		const int kc = (ikt >> 1) * (CI / 16) + t_cb * (PCI / 16) + (ikt & 1) * KCH;
+		const int kc = ((t_cb * (PCI / 32) + (ikt & 1)) * 9 + (ikt >> 1)) * KCH;
 #pragma unroll
 		for (int i = 0; i < A_PW; i++)
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16, lane * 16,
@@ -2311,7 +2320,7 @@ static inline int conv_chunk(int dtype) { return dtype == THHIP_F32 ? 8 : dtype 
 /* Order of (plane c, tap) along the packed K axis; follows how the input is
  * read (xl: 0 plane-major, 1 channels-last, 2 plane-major read through a
  * four-plane pixel copy), so weights are packed for one of them. */
-enum { KORD_PLANE_TAP, KORD_TAP_MAJOR, KORD_CHANNELS_LAST, KORD_PIXELS4 };
+enum { KORD_PLANE_TAP, KORD_TAP_MAJOR, KORD_CHANNELS_LAST, KORD_PIXELS4, KORD_CL_BLOCKED };
 
 /* Tap-major K order needs whole blocks of KCH*chunk input planes. */
 static inline bool conv_tap_major(int Ci, int dtype) { return Ci % (conv_kch(dtype, false) * conv_chunk(dtype)) == 0; }
@@ -2321,7 +2330,10 @@ static inline int conv_korder(int Ci, int dtype, int xl)
 	if (xl == 1) {
 		if (Ci % (conv_chunk(dtype) / 2))
 			THError("thhip_conv2d: channels-last input needs Ci %% %d == 0 (Ci = %d)", conv_chunk(dtype) / 2, Ci);
-		return KORD_CHANNELS_LAST;
+		/* whole K-tiles of planes: K runs (block of planes, tap, plane of the block), so that the taps
+		 * of a block, which read the same pixels shifted, follow one another while those pixels are
+		 * still in the caches; other plane counts: (tap, plane) */
+		return Ci % (conv_kch(dtype, true) * conv_chunk(dtype)) == 0 ? KORD_CL_BLOCKED : KORD_CHANNELS_LAST;
 	}
 	if (xl == 2) {
 		if (dtype != THHIP_U8 || Ci > 4)
@@ -2353,6 +2365,10 @@ static inline long conv_kpos(int c, int kh, int kw, int Ci, int kH, int kW, int 
 	switch (conv_korder(Ci, dtype, xl)) {
 	case KORD_CHANNELS_LAST:
 		return (long)tap * Ci + c;
+	case KORD_CL_BLOCKED: {
+		const int cb = conv_kch(dtype, true) * conv_chunk(dtype);
+		return ((long)(c / cb) * kHW + tap) * cb + c % cb;
+	}
 	case KORD_PIXELS4:
 		return (((long)kh * ((kW + 3) / 4) + kw / 4) * 4 + kw % 4) * 4 + c;
 	case KORD_TAP_MAJOR: {
@@ -3029,10 +3045,6 @@ static void conv_dispatch(ConvParams &p)
 	if (direct || bn >= 256) {
 		if (!conv_wide_ok<DT>(p))
 			THError("thhip_conv2d: tiles loaded straight into LDS need channels-last input with whole K-tiles of planes (and, uint8, a tail of padding codes)");
-		/* K-tiles of 64 values in two stages measured the same as 32 in four
-		 * (the tuning hook's split-K argument, 4, selects them for the tests) */
-		if (bm == 256 && bn == 256 && p.Ci % 64 == 0 && g_force_splitk == 4)
-			return conv_launch_wide<DT, 256, 256, 2, 4, 4, 2>(p);
 		if (bm == 256 && bn == 256)
 			return conv_launch_wide<DT, 256, 256, 2, 4, 2, 4>(p);
 		if (bm == 128 && bn == 256)
@@ -3181,6 +3193,9 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 		p.KC = conv_kc(Ci, kH, kW, dtype, xl);
 		p.N = bn * oH * oW;
 		p.oHW = oH * oW;
+		if (xl == 1 && conv_korder(Ci, dtype, xl) == KORD_CL_BLOCKED)
+			for (int cb = conv_kch(dtype, true) * conv_chunk(dtype); (1 << p.cl_shift) < cb; )
+				p.cl_shift++;
 		p.pW = oW / 2;
 		p.pHW = (oH / 2) * (oW / 2);
 		p.npool = bn * p.pHW;
