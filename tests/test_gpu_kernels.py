@@ -505,8 +505,10 @@ def test_conv_half_wide_tile(hiplib, oracle, dt):
                 narrow = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
                 # 256 positions: eight and four waves, K-tiles of 32 in four LDS stages.  The smaller tiles
                 # (third argument 9: the kernel that loads straight into LDS): four waves, four stages.
-                for tune in ((256, 256, 0), (128, 256, 0), (128, 128, 9), (128, 64, 9), (64, 128, 9), (64, 64, 9)):
-                    hiplib.thhip_conv_set_tuning(tune[0], tune[1], tune[2], 0)
+                # (fourth argument, 64 x 64 tiles: one K group, or two that share the tile and split its K-tiles)
+                for tune in ((256, 256, 0, 0), (128, 256, 0, 0), (128, 128, 9, 0), (128, 64, 9, 0), (64, 128, 9, 0), (64, 64, 9, 1),
+                             (64, 64, 9, 2)):
+                    hiplib.thhip_conv_set_tuning(*tune)
                     got = G.conv2d_layout(hiplib, x, w, b, (dH, dW), (pH, pW), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
                     G.assert_close(got, want, HALF_TOL, str((Ci, Co, kH, y_cl, tune)))
                     G.assert_close(got, narrow, 1e-2, "vs the register-staged 128x128 tile " + str((Ci, Co, kH, y_cl, tune)))

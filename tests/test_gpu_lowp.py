@@ -192,7 +192,8 @@ def test_conv_u8_loaded_straight_into_lds_bit_exact(hiplib, oracle, i):
     addend = np.array([oracle.lowp_bias_addend(int(c), bm, bsub, om) for c in bq], np.int32)
     thr = oracle.lowp_scale_float(om, osub, 0.0)
     try:
-        for tune in ((0, 0, 0, 0), (64, 64, 9, 0), (128, 64, 9, 0), (64, 128, 9, 0), (128, 128, 9, 0)):
+        # (64 x 64 tiles, fourth argument: one K group, or two that share the tile and split its K-tiles)
+        for tune in ((0, 0, 0, 0), (64, 64, 9, 1), (64, 64, 9, 2), (128, 64, 9, 0), (64, 128, 9, 0), (128, 128, 9, 0)):
             hiplib.thhip_conv_set_tuning(*tune)
             for y_cl in (1, 0):
                 for tail in (64, 200):

@@ -1160,8 +1160,8 @@ __device__ __forceinline__ void conv_wide_store_half(const ConvParams &p, floatx
 	}
 }
 
-template <int DT, bool CLO, int BM, int BN, int WGM, int WGN, int KCH, int NST>
-__global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
+template <int DT, bool CLO, int BM, int BN, int WGM, int WGN, int KCH, int NST, int KG = 1>
+__global__ __launch_bounds__(64 * WGM * WGN * KG) void conv_wide_kernel(ConvParams p)
 {
 	/* The host pass only needs the launch stub; it gets no body, because it
 	 * silently drops the whole kernel when it meets the LDS-load builtin in a
@@ -1183,12 +1183,22 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	static_assert(KCH == 2 || KCH == 4, "K-tiles of 32 or 64 values");
 	static_assert(MB * KCH % WAVES == 0 && BN / PPG % WAVES == 0 && NST >= 2 && NST <= 4, "tile shape");
 	static_assert((2 * BM + BN) * sizeof(int) <= NST * STAGE_VECS * sizeof(floatx4), "the epilogue's row and column constants fit");
-	__shared__ floatx4 lds[NST * STAGE_VECS];
+	/* KG = 2: two groups of WGM x WGN waves share the tile, each with its own LDS stages and its own half of
+	 * the K-tiles; their sums are added through LDS at the end (a K split inside the workgroup: no partial
+	 * sums in global memory, no second launch, the same order of additions every time).  For layers of few
+	 * tiles and a long K, where a CU holds one or two workgroups and little overlaps a K step's latency. */
+	static_assert(KG == 1 || KG == 2, "one or two K groups");
+	static_assert(KG == 1 || TM * TN * 16 * 64 * WAVES * sizeof(int) + TN * 64 * WAVES * sizeof(int) <= NST * STAGE_VECS * sizeof(floatx4),
+		"the exchange of the groups' sums fits one group's stages");
+	__shared__ floatx4 lds_all[KG * NST * STAGE_VECS];
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
-	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wave_all = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int kg = KG > 1 ? wave_all / WAVES : 0;
+	const int wave = KG > 1 ? wave_all - kg * WAVES : wave_all;	/* within the group */
 	const int wm = wave % WGM, wn = wave / WGM;
+	floatx4 *const lds = lds_all + kg * (NST * STAGE_VECS);
 
 	int tile_m, tile_n, split = 0, nsplit = 1;
 	long tail_blk = -1;
@@ -1248,8 +1258,16 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	}
 	/* K-tiles: block of planes outer, tap inner; a part of a cut tile walks [kt0, kt0 + nkt) */
 	const int nkt_all = p.KC / KCH;
-	const int kt0 = nsplit > 1 ? (int)((long)nkt_all * split / nsplit) : 0;
-	const int nkt = (nsplit > 1 ? (int)((long)nkt_all * (split + 1) / nsplit) : nkt_all) - kt0;
+	int kt0 = nsplit > 1 ? (int)((long)nkt_all * split / nsplit) : 0;
+	int nkt = (nsplit > 1 ? (int)((long)nkt_all * (split + 1) / nsplit) : nkt_all) - kt0;
+	int nkt_live = nkt;	/* K-tiles that exist; the groups walk the same number of steps (the barriers are the workgroup's) */
+	if constexpr (KG > 1) {
+		const int per = (nkt + KG - 1) / KG;
+		nkt_live = min(per, nkt - kg * per);
+		kt0 += kg * per;
+		nkt = per;
+	}
+	int issued = 0;
 	int t_cb, t_kh, t_kw, t_kc = kt0 * KCH;
 	{
 		const int blk = kt0 / p.kHW, tap = kt0 - blk * p.kHW;
@@ -1261,15 +1279,19 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 	auto issue = [&](auto st_) {
 		constexpr int st = decltype(st_)::value;
 		floatx4 *la = lds + st * STAGE_VECS, *lb = la + A_VECS;
+		/* (KG > 1) a step past this group's last K-tile loads zeros: weights out of the buffer's range,
+		 * positions as outside the image */
+		const bool live = KG == 1 || issued < nkt_live;
+		++issued;
 #pragma unroll
 		for (int i = 0; i < A_PW; i++)
-			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(la + a_lds_[i]), 16, lane * 16,
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(la + a_lds_[i]), 16, live ? lane * 16 : 0x80000000u,
 				a_off_[i] + (unsigned)t_kc * 1024u, 0, 0);
 		const int cl_off = ((t_kh * p.W + t_kw) * p.Ci + t_cb) * (int)sizeof(elem);
 #pragma unroll
 		for (int q = 0; q < NPOS; q++) {
 			const int iy = iy0_[q] + t_kh, ix = ix0_[q] + t_kw;
-			const bool ok = n_ok_[q] && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			const bool ok = live && n_ok_[q] && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
 			const unsigned voff = ok ? (unsigned)(xoff_[q] + cl_off) : outside;
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(lb + (wave + WAVES * q) * 64), 16, voff, 0, 0, 0);
 		}
@@ -1311,7 +1333,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 #pragma unroll
 	for (int j = 0; j < TN; j++)
 		colsum[j] = 0;
-	auto mma = [&](int set) {
+	auto mma = [&](int set, int kt) {
+		/* (KG > 1) a step past the group's last K-tile has read padding codes, which are not zero once
+		 * re-centred unless the padding code is 128: they meet zero weights, but stay out of the column sums */
+		const bool sums = wm == 0 && (KG == 1 || kt < nkt_live);
 		if constexpr (DT == THHIP_U8) {
 			/* code - 128 as a signed byte, done on the fragments (they never
 			 * pass through registers on their way to LDS) */
@@ -1321,7 +1346,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 #pragma unroll
 				for (int d = 0; d < 4; d++) {
 					cw[d] ^= (int)0x80808080;
-					if (wm == 0)
+					if (sums)
 						colsum[j] = __builtin_amdgcn_sdot4(cw[d], 0x01010101, colsum[j], false);
 				}
 				bf[set][j] = __builtin_bit_cast(floatx4, cw);
@@ -1362,7 +1387,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 #pragma unroll
 		for (int c = 0; c + 1 < KCH; c++) {
 			read_frags(st, c + 1, af[(c + 1) & 1], bf[(c + 1) & 1]);
-			mma(c & 1);
+			mma(c & 1, kt);
 		}
 		/* this wave's loads of tile kt+1 are in LDS (younger tiles may still be
 		 * on their way) and the fragments just requested have arrived */
@@ -1375,7 +1400,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 			issue(st);
 		if (steady || kt + 1 < nkt)
 			read_frags(st1, 0, af[0], bf[0]);
-		mma((KCH - 1) & 1);
+		mma((KCH - 1) & 1, kt);
 	};
 	/* NST steps: every stage index a constant */
 	auto round = [&](int kt, auto steady_) {
@@ -1410,6 +1435,43 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		}
 	}
 
+	/* ---- the second K group hands its sums (and its share of the column sums) to the first and is done ---- */
+	if constexpr (KG > 1) {
+		typedef typename std::conditional<DT == THHIP_U8, int, float>::type accel;
+		accel *xch = (accel *)lds_all;			/* [wave][accumulator register][lane] */
+		int *xcs = (int *)(xch + TM * TN * 16 * 64 * WAVES);	/* [wave][tile column][lane] */
+		__syncthreads();		/* every wave is done with the tiles */
+		if (kg == 1) {
+#pragma unroll
+			for (int i = 0; i < TM; i++)
+#pragma unroll
+				for (int j = 0; j < TN; j++)
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						xch[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
+			if constexpr (DT == THHIP_U8) {
+#pragma unroll
+				for (int j = 0; j < TN; j++)
+					xcs[(wave * TN + j) * 64 + lane] = colsum[j];
+			}
+		}
+		__syncthreads();
+		if (kg == 1)
+			return;		/* (a wavefront that has ended no longer counts at the workgroup's barriers) */
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					acc[i][j][r] += xch[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane];
+		if constexpr (DT == THHIP_U8) {
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+				colsum[j] += xcs[(wave * TN + j) * 64 + lane];
+		}
+	}
+	int *const lds_epi = (int *)lds_all;
 	/* ---- epilogue ---- */
 	if constexpr (DT != THHIP_U8) {
 		if (tail_blk >= 0) {
@@ -1427,10 +1489,10 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 			return;
 		}
 		__syncthreads();		/* every wave is done with the tiles */
-		conv_wide_store_half<DT, CLO, BM, BN, WGM, WGN, TM, TN, TM, TN>(p, acc, tile_m, tile_n, (int *)lds);
+		conv_wide_store_half<DT, CLO, BM, BN, WGM, WGN, TM, TN, TM, TN>(p, acc, tile_m, tile_n, lds_epi);
 	} else {
 	elem *y = (elem *)p.y;
-	int *lrow = (int *)lds;		/* [BM] bias bits or uint8 row term, [BM..2BM) factor bits or uint8 addend */
+	int *lrow = lds_epi;		/* [BM] bias bits or uint8 row term, [BM..2BM) factor bits or uint8 addend */
 	int *cs = lrow + 2 * BM;	/* uint8: [BN] column sums */
 	__syncthreads();		/* every wave is done with the tiles */
 	if (tid < BM) {
@@ -1439,7 +1501,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_kernel(ConvParams p)
 		lrow[BM + tid] = p.addend ? p.addend[mc] : 0;
 	}
 	if constexpr (DT == THHIP_U8) {
-		for (int i = tid; i < BN; i += 64 * WAVES)
+		for (int i = tid; i < BN; i += 64 * WAVES)	/* (the first K group's threads: the second has left) */
 			cs[i] = 0;
 		__syncthreads();
 		if (wm == 0) {	/* the two halves of a column's K values sit in lanes l and l + 32 */
@@ -2727,7 +2789,7 @@ static bool conv_wide_ok(const ConvParams &p)
 	return false;
 }
 
-template <int DT, int BM, int BN, int WGM, int WGN, int KCH, int NST>
+template <int DT, int BM, int BN, int WGM, int WGN, int KCH, int NST, int KG = 1>
 static void conv_launch_wide(ConvParams &p)
 {
 	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16 || (DT == THHIP_U8 && BM <= 128 && BN <= 128 && KCH == 2)) {
@@ -2746,7 +2808,7 @@ static void conv_launch_wide(ConvParams &p)
 		 * along K, as in conv_launch_f32_direct (uint8 tiles stay whole: their
 		 * column sums run over all of K) */
 		int resident = 0;
-		if constexpr (DT != THHIP_U8) {
+		if constexpr (DT != THHIP_U8 && KG == 1) {
 			static int res_cl, res_pm;
 			int &res = p.y_cl ? res_cl : res_pm;
 			if (!res) {
@@ -2760,12 +2822,13 @@ static void conv_launch_wide(ConvParams &p)
 			resident = res;
 		}
 		/* few tiles all cut measured slower here (512->512 @14^2 batch 16, fp16: 31 -> 36 us) */
-		const size_t maxcnt = conv_tail_plan(p, resident, DT == THHIP_U8 ? 0 : p.KC / KCH, (size_t)BM * BN, 1);
+		/* (tiles shared by two K groups stay whole, like the uint8 ones) */
+		const size_t maxcnt = conv_tail_plan(p, resident, DT == THHIP_U8 || KG > 1 ? 0 : p.KC / KCH, (size_t)BM * BN, 1);
 		dim3 grid((unsigned)(8 * maxcnt));
 		if (p.y_cl)
-			conv_wide_kernel<DT, true, BM, BN, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+			conv_wide_kernel<DT, true, BM, BN, WGM, WGN, KCH, NST, KG><<<grid, dim3(64 * WGM * WGN * KG), 0, thhip_stream()>>>(p);
 		else
-			conv_wide_kernel<DT, false, BM, BN, WGM, WGN, KCH, NST><<<grid, dim3(64 * WGM * WGN), 0, thhip_stream()>>>(p);
+			conv_wide_kernel<DT, false, BM, BN, WGM, WGN, KCH, NST, KG><<<grid, dim3(64 * WGM * WGN * KG), 0, thhip_stream()>>>(p);
 		if constexpr (DT != THHIP_U8) {
 			if (p.tail_slots) {
 				dim3 fgrid((unsigned)(8 * p.tail_tiles * (BM / WGM / 32) * (BN / WGN / 32)));
@@ -3055,8 +3118,16 @@ static void conv_dispatch(ConvParams &p)
 			return conv_launch_wide<DT, 128, 64, 2, 2, 2, 4>(p);
 		if (bm == 64 && bn == 128)
 			return conv_launch_wide<DT, 64, 128, 2, 2, 2, 4>(p);
-		if (bm == 64 && bn == 64)
+		if (bm == 64 && bn == 64) {
+			/* Few tiles and a long K: one or two workgroups per CU with little to overlap a K step's
+			 * latency with.  Two K groups per workgroup then walk half the K-tiles each: 512 -> 512 @14^2
+			 * batch 16, fp16, 33 -> 31 us; ResNet-18 fp16 batch 32 0.679 -> 0.662 ms (the tuning hook's
+			 * last argument forces one group, 1, or two, 2). */
+			const bool two = g_force_wgs ? g_force_wgs == 2 : t64 <= 512 && p.KC / 2 >= 32;
+			if (two)
+				return conv_launch_wide<DT, 64, 64, 2, 2, 2, 4, 2>(p);
 			return conv_launch_wide<DT, 64, 64, 2, 2, 2, 4>(p);
+		}
 		THError("thhip_conv2d: no %dx%d tile", bm, bn);
 	}
 #define CONV_TILES(KCH)                                                      \
