@@ -451,8 +451,9 @@ void thhip_conv2d_layout(const void *x, const void *wpacked, const float *scale,
  * sequence SpatialConvolutionMM -> Threshold -> SpatialMaxPooling
  * (modules/SpatialMaxPooling.c:6-98 after SpatialConvolutionMM.c:111-225) for the
  * layers thhip_conv2d_pool2_supported accepts: half types, channels-last input
- * of 64 or 128 planes, 3x3, stride 1, enough tiles for the kernel that keeps an
- * input patch in LDS; fp32, plane-major tensors, planes in blocks of 32, any
+ * with planes in blocks of 32 (the kernel that keeps an input patch in LDS for
+ * 3x3 / stride 1 layers of 64 or 128 planes with enough tiles, else the tiles
+ * loaded straight into LDS); fp32, plane-major tensors, planes in blocks of 32, any
  * kernel size and stride, more than 512 tiles of 64 planes x 64 positions (the
  * layers that run without a K split): the kernel then walks the positions window
  * by window, the four of a window in neighbouring lanes, and a last odd row or

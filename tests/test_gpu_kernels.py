@@ -551,35 +551,42 @@ def test_conv_half_patch_kernel(hiplib, oracle, dt):
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_conv_half_patch_kernel_with_pooling(hiplib, oracle, dt):
     """Convolution, threshold and the 2x2 / stride 2 max pooling that follows in one kernel:
-    the same values as the convolution entry point followed by the pooling entry point
-    (bit for bit: the pooling compares the rounded outputs), and the oracle's within the half
-    tolerance; odd output sizes (the last row / column is dropped), both output orders,
-    64 and 128 planes, the folded batch-norm factor with negative entries."""
+    the same values as the convolution entry point followed by the pooling (bit for bit on
+    the kernel that keeps an input patch in LDS: the pooling compares the rounded outputs; on
+    the tiles loaded straight into LDS up to the last bit of a sum, where one of the two runs
+    cut a tile along K), and the oracle's within the half tolerance; odd output sizes (the
+    last row / column is dropped), both output orders, the folded batch-norm factor with
+    negative entries; 64 and 128 planes (patch kernel), and 256 x 256, 128 x 128 and 64 x 64
+    tiles with one and two K groups, 1x1 and strided layers (tiles loaded straight into LDS)."""
     import ctypes as C
     from thnets_amd import api
     g = cases.rng(914)
-    for (B, Ci, H, W, Co, pad) in ((8, 64, 33, 47, 72, 1), (16, 128, 40, 64, 72, 1), (40, 64, 17, 19, 132, 0), (4, 64, 40, 64, 200, 1)):
+    shapes = [(8, 64, 33, 47, 72, 3, 1, 1, True), (16, 128, 40, 64, 72, 3, 1, 1, True), (40, 64, 17, 19, 132, 3, 1, 0, True),
+              (4, 64, 40, 64, 200, 3, 1, 1, True),
+              (16, 256, 56, 56, 256, 3, 1, 1, False), (16, 512, 28, 28, 512, 3, 1, 1, False), (4, 512, 14, 14, 512, 3, 1, 1, False),
+              (3, 32, 21, 23, 40, 1, 1, 0, False), (2, 96, 30, 31, 264, 5, 2, 2, False), (1, 64, 8, 8, 64, 3, 1, 1, False)]
+    for (B, Ci, H, W, Co, k, d, pad, exact) in shapes:
         x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
-        w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
+        w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
         b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
         sc = (g.uniform(0.5, 1.5, Co) * g.choice([-1.0, 1.0], Co)).astype(np.float32)
-        oH, oW = H + 2 * pad - 2, W + 2 * pad - 2
+        oH, oW = (H + 2 * pad - k) // d + 1, (W + 2 * pad - k) // d + 1
         pH, pW = oH // 2, oW // 2
         xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
         wr = api.from_device_dtype(api.to_device_dtype(hiplib, w, dt), w.shape, dt)
-        raw = oracle.conv2d(xr, wr, None, (1, 1), (pad, pad))
+        raw = oracle.conv2d(xr, wr, None, (d, d), (pad, pad))
         act = np.maximum(raw * sc[None, :, None, None] + b[None, :, None, None], 0)
         want = act[:, :, :2 * pH, :2 * pW].reshape(B, Co, pH, 2, pW, 2).max(axis=(3, 5))
         for y_cl in (1, 0):
-            G.note("conv + pool %s y_cl %d dtype %d" % ((B, Ci, H, W, Co, pad), y_cl, dt))
-            assert hiplib.thhip_conv2d_pool2_supported(B, Ci, H, W, Co, 3, 3, 1, 1, pad, pad, dt, 1, y_cl)
-            unpooled = G.conv2d_layout(hiplib, x, w, b, (1, 1), (pad, pad), act=1, dtype=dt, x_cl=1, y_cl=0, scale=sc)
+            G.note("conv + pool %s y_cl %d dtype %d" % ((B, Ci, H, W, Co, k, d, pad), y_cl, dt))
+            assert hiplib.thhip_conv2d_pool2_supported(B, Ci, H, W, Co, k, k, d, d, pad, pad, dt, 1, y_cl)
+            unpooled = G.conv2d_layout(hiplib, x, w, b, (d, d), (pad, pad), act=1, dtype=dt, x_cl=1, y_cl=0, scale=sc)
             ref = unpooled[:, :, :2 * pH, :2 * pW].reshape(B, Co, pH, 2, pW, 2).max(axis=(3, 5))
             dx = api.to_device_dtype(hiplib, np.ascontiguousarray(x.transpose(0, 2, 3, 1)), dt)
-            wp = hiplib.thhip_conv_pack_weight_layout(np.ascontiguousarray(w).ctypes.data, Co, Ci, 3, 3, dt, 1)
+            wp = hiplib.thhip_conv_pack_weight_layout(np.ascontiguousarray(w).ctypes.data, Co, Ci, k, k, dt, 1)
             db, ds = api.DeviceArray(hiplib, b), api.DeviceArray(hiplib, sc)
             dy = api.DeviceArray(hiplib, nbytes=B * Co * pH * pW * 2)
-            hiplib.thhip_conv2d_layout_pool2(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, B, Ci, H, W, Co, 3, 3, 1, 1, pad, pad,
+            hiplib.thhip_conv2d_layout_pool2(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, B, Ci, H, W, Co, k, k, d, d, pad, pad,
                                              1, 0.0, 0.0, dt, 1, y_cl)
             hiplib.thhip_sync()
             if y_cl:
@@ -587,12 +594,16 @@ def test_conv_half_patch_kernel_with_pooling(hiplib, oracle, dt):
             else:
                 got = api.from_device_dtype(dy, (B, Co, pH, pW), dt)
             hiplib.thhip_free(wp)
-            assert np.array_equal(got, ref), (B, Ci, H, W, Co, pad, y_cl, int((got != ref).sum()))
-            G.assert_close(got, want, HALF_TOL, str((B, Ci, H, W, Co, pad, y_cl)))
-    # layers the fused kernel does not take
-    assert not hiplib.thhip_conv2d_pool2_supported(1, 64, 8, 8, 64, 3, 3, 1, 1, 1, 1, dt, 1, 1)          # too few tiles
-    assert not hiplib.thhip_conv2d_pool2_supported(8, 32, 33, 47, 72, 3, 3, 1, 1, 1, 1, dt, 1, 1)        # 32 planes
-    assert not hiplib.thhip_conv2d_pool2_supported(8, 64, 33, 47, 72, 3, 3, 2, 2, 1, 1, dt, 1, 1)        # stride 2
+            if exact:
+                assert np.array_equal(got, ref), (B, Ci, H, W, Co, pad, y_cl, int((got != ref).sum()))
+            else:
+                G.assert_close(got, ref, 1e-2, "vs convolution, pooling " + str((B, Ci, H, W, Co, k, d, pad, y_cl)))
+                assert (got != ref).mean() < 1e-3, (B, Ci, H, W, Co, k, d, pad, y_cl, float((got != ref).mean()))
+            G.assert_close(got, want, HALF_TOL, str((B, Ci, H, W, Co, k, d, pad, y_cl)))
+    # layers the fused kernels do not take
+    assert not hiplib.thhip_conv2d_pool2_supported(8, 24, 33, 47, 72, 3, 3, 1, 1, 1, 1, dt, 1, 1)        # planes not in blocks of 32
+    assert not hiplib.thhip_conv2d_pool2_supported(8, 64, 33, 47, 72, 3, 3, 1, 1, 1, 1, dt, 0, 1)        # plane-major input
+    assert not hiplib.thhip_conv2d_pool2_supported(8, 64, 3, 47, 72, 3, 3, 1, 1, 0, 0, dt, 1, 1)         # one output row
     assert not hiplib.thhip_conv2d_pool2_supported(8, 64, 33, 47, 72, 3, 3, 1, 1, 1, 1, G.F32, 1, 1)
 
 

@@ -36,7 +36,15 @@ def layerwise(net, oracle, cfg, tol, folded_bn=True):
         elif i + 1 < len(layers) and layers[i + 1]["type"] == "threshold" and (
                 layers[i]["type"] in ("conv", "linear", "caddtable", "fullconv") or layers[i + 1].get("inplace", 1) == 1):
             want = outs[i + 1]
-        G.assert_close(net.module_output(i).ravel(), np.asarray(want).ravel(), tol, "module %d %s" % (i, layers[i]["type"]))
+        got = net.module_output(i)
+        if layers[i]["type"] in ("conv", "bn", "threshold") and got.size != np.asarray(want).size:
+            # a 2x2 pooling done in the convolution's epilogue: the buffer holds the pooled tensor
+            j = i + 1
+            while j < len(layers) and layers[j]["type"] in ("bn", "threshold"):
+                j += 1
+            assert j < len(layers) and layers[j]["type"] == "maxpool", (i, got.shape, np.asarray(want).shape)
+            want = outs[j]
+        G.assert_close(got.ravel(), np.asarray(want).ravel(), tol, "module %d %s" % (i, layers[i]["type"]))
 
 
 @pytest.mark.parametrize("name", sorted(cases.small_networks().keys()))

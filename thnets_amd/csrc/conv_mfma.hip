@@ -1088,6 +1088,30 @@ __host__ __device__ inline int conv_tail_parts(int cnt, int slots, int smax, int
 	return s;
 }
 
+/* conv_f32_direct_kernel and conv_wide_kernel with the 2x2 / stride 2 pooling in their epilogue: member t of a
+ * block of 64 positions.  The block is sixteen neighbouring pooling windows; t = 32 half + 16 dy + 2 w + dx
+ * is column dx of row dy of window 8 half + w.  Sixteen neighbouring lanes thus gather sixteen
+ * neighbouring pixels of a row (whole 64-byte runs, as without the pooling), a 32-position MFMA
+ * tile holds eight whole windows, the other column of a window is the next lane and the other
+ * row is lane ^ 16. */
+__device__ __forceinline__ void conv_pool_member(int n, int &pp, int &dy, int &dx)
+{
+	pp = (n >> 6) * 16 + ((n >> 5) & 1) * 8 + ((n >> 1) & 7);
+	dy = (n >> 4) & 1;
+	dx = n & 1;
+}
+
+/* v of lane + 1 (for even lanes), v of lane ^ 16 */
+__device__ __forceinline__ float conv_lane_next(float v)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xF5, 0xf, 0xf, true));
+}
+
+__device__ __forceinline__ float conv_lane_xor16(float v)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
+}
+
 /* Epilogue of the half-type tiles of conv_wide_kernel (WGM x WGN waves, each
  * TMF x TNF accumulators of 32x32, of which acc holds the TM x TN from
  * (i0, j0) on): (folded batch norm factor,) bias, optional threshold, store in
@@ -1109,14 +1133,23 @@ __device__ __forceinline__ void conv_wide_store_half(const ConvParams &p, floatx
 	const bool has_scale = p.scale != 0;
 	/* channels-last: whole 16-byte stores (conv_store_cl_half) */
 	const bool cl16 = CLO && p.Co % 8 == 0 && ((size_t)p.y & 15) == 0;
+	/* With the pooling (p.pool: positions counted in blocks of sixteen windows, conv_pool_member) the first
+	 * lane of a window takes the maximum of the four stored (rounded) values, with SpatialMaxPooling.c:51-66's
+	 * comparisons in their order, and stores it; every lane runs the loop (the lanes of a window exchange). */
+	const int oHW = p.pool ? p.pHW : p.oHW;
 #pragma unroll
 	for (int j = 0; j < TN; j++) {
-		const int n = tile_n * BN + (wn * TNF + j0 + j) * 32 + (lane & 31);
-		const bool valid = n < p.N;
-		if (!cl16 && !valid)
+		int n = tile_n * BN + (wn * TNF + j0 + j) * 32 + (lane & 31);
+		bool valid = n < p.N;
+		if (p.pool) {
+			int pp, dy, dx;
+			conv_pool_member(n, pp, dy, dx);
+			valid = pp < p.npool && !dy && !dx;
+			n = pp;
+		} else if (!cl16 && !valid)
 			continue;
-		const int b = n / p.oHW, rem = n - b * p.oHW;
-		const size_t ybase = (size_t)b * p.Co * p.oHW + rem;
+		const int b = n / oHW, rem = n - b * oHW;
+		const size_t ybase = (size_t)b * p.Co * oHW + rem;
 #pragma unroll
 		for (int i = 0; i < TM; i++) {
 			const int m0 = tile_m * BM + (wm * TMF + i0 + i) * 32 + 4 * (lane >> 5);
@@ -1135,9 +1168,19 @@ __device__ __forceinline__ void conv_wide_store_half(const ConvParams &p, floatx
 					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
 					if (p.act)
 						v = v > p.thr ? v : p.val;
+					if (p.pool) {
+						const float v00 = (float)(elem)v, v01 = conv_lane_next(v00);
+						const float v10 = conv_lane_xor16(v00), v11 = conv_lane_xor16(v01);
+						float mx = -FLT_MAX;
+						mx = v00 > mx ? v00 : mx;
+						mx = v01 > mx ? v01 : mx;
+						mx = v10 > mx ? v10 : mx;
+						mx = v11 > mx ? v11 : mx;
+						v = mx;
+					}
 					if constexpr (!CLO) {
-						if (m < p.Co)
-							y[ybase + (size_t)m * p.oHW] = (elem)v;
+						if (valid && m < p.Co)
+							y[ybase + (size_t)m * oHW] = (elem)v;
 					}
 					quad.v[e] = (elem)v;
 				}
@@ -1146,7 +1189,7 @@ __device__ __forceinline__ void conv_wide_store_half(const ConvParams &p, floatx
 					__builtin_memcpy(pair, &quad, 8);
 					lo[g] = pair[0];
 					hi[g] = pair[1];
-					if (!cl16 && m0 + 8 * g < p.Co)
+					if (!cl16 && valid && m0 + 8 * g < p.Co)
 						*(Quad *)(y + (size_t)n * p.Co + m0 + 8 * g) = quad;
 				}
 			}
@@ -1235,8 +1278,22 @@ __global__ __launch_bounds__(64 * WGM * WGN * KG) void conv_wide_kernel(ConvPara
 		const int n_glob = tile_n * BN + n_tile;
 		n_ok_[q] = n_glob < p.N;
 		const int nn = n_ok_[q] ? n_glob : 0;
-		const int b = nn / p.oHW, r = nn - b * p.oHW;
-		const int oy = r / p.oW, ox = r - oy * p.oW;
+		int b, oy, ox;
+		if (p.pool) {	/* positions in blocks of sixteen pooling windows */
+			int pp, dy, dx;
+			conv_pool_member(n_glob, pp, dy, dx);
+			n_ok_[q] = pp < p.npool;
+			pp = n_ok_[q] ? pp : 0;
+			b = pp / p.pHW;
+			const int r = pp - b * p.pHW, py = r / p.pW;
+			oy = 2 * py + dy;
+			ox = 2 * (r - py * p.pW) + dx;
+		} else {
+			b = nn / p.oHW;
+			const int r = nn - b * p.oHW;
+			oy = r / p.oW;
+			ox = r - oy * p.oW;
+		}
 		iy0_[q] = oy * p.dH - p.padH;
 		ix0_[q] = ox * p.dW - p.padW;
 		xoff_[q] = (((b * p.H + iy0_[q]) * p.W + ix0_[q]) * p.Ci + myvec * VEC) * (int)sizeof(elem);
@@ -1909,30 +1966,6 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
  * conv_f32_direct_kernel (2 x 2 waves): (folded batch norm factor,) bias,
  * optional threshold, plane-major store.  lrow: 2 * BM ints of LDS no wave
  * still reads. */
-/* conv_f32_direct_kernel with the 2x2 / stride 2 pooling in its epilogue: member t of a block of
- * 64 positions.  The block is sixteen neighbouring pooling windows; t = 32 half + 16 dy + 2 w + dx
- * is column dx of row dy of window 8 half + w.  Sixteen neighbouring lanes thus gather sixteen
- * neighbouring pixels of a row (whole 64-byte runs, as without the pooling), a 32-position MFMA
- * tile holds eight whole windows, the other column of a window is the next lane and the other
- * row is lane ^ 16. */
-__device__ __forceinline__ void conv_pool_member(int n, int &pp, int &dy, int &dx)
-{
-	pp = (n >> 6) * 16 + ((n >> 5) & 1) * 8 + ((n >> 1) & 7);
-	dy = (n >> 4) & 1;
-	dx = n & 1;
-}
-
-/* v of lane + 1 (for even lanes), v of lane ^ 16 */
-__device__ __forceinline__ float conv_lane_next(float v)
-{
-	return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xF5, 0xf, 0xf, true));
-}
-
-__device__ __forceinline__ float conv_lane_xor16(float v)
-{
-	return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x401F));
-}
-
 template <int BM, int BN, int TM, int TN>
 __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, floatx16 (&acc)[TM][TN], int tile_m, int tile_n, int *lrow)
 {
@@ -2930,6 +2963,21 @@ static void conv_launch_patch(ConvParams &p)
 		THError("thhip_conv2d: the patch kernel is for the half types");
 }
 
+/* Half types, convolution followed by a 2x2 pooling: whether the kernel that keeps an input patch in LDS is
+ * the one that runs (and pools) the layer; the rule conv_dispatch applies to the layer without the pooling. */
+template <int DT>
+static bool conv_pool_uses_patch(const ConvParams &p)
+{
+	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
+		const long n = (long)p.B * p.oH * p.oW;
+		const long t256 = (long)((p.Co + 255) / 256) * ((n + 255) / 256);
+		const long tpatch = (long)((p.Co + 63) / 64) * p.B * ((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH);
+		const bool wide256 = conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128;
+		return conv_patch_ok<DT>(p) && tpatch >= 128 && !(wide256 && p.Ci > 64);
+	}
+	return false;
+}
+
 template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
@@ -2952,7 +3000,12 @@ static void conv_dispatch(ConvParams &p)
 	 * for the operand reuse, 64x64 below.
 	 * Splitting K measured slower than unsplit 64x64 tiles on every layer that
 	 * has tiles for all CUs, so only layers of a few tiles are split (below). */
-	if (p.pool && DT == THHIP_F32)
+	/* pooling in the epilogue: the half types' patch kernel where that kernel would run the layer, else the
+	 * kernels that load their tiles straight into LDS, which then count positions in blocks of sixteen windows */
+	bool pool_patch = false;
+	if (p.pool && DT != THHIP_F32)
+		pool_patch = conv_pool_uses_patch<DT>(p);
+	if (p.pool && !pool_patch)
 		p.N = 64 * ((p.npool + 15) / 16);	/* whole pooling windows only: a last odd row or column is not computed */
 	const long t128 = (long)((p.Co + 127) / 128) * ((p.N + 127) / 128);
 	const long t64 = (long)((p.Co + 63) / 64) * ((p.N + 63) / 64);
@@ -3073,8 +3126,10 @@ static void conv_dispatch(ConvParams &p)
 		wgs = g_force_wgs;
 	if (DT == THHIP_F32 && g_force_kch)
 		kch = g_force_kch;
-	if (p.pool && DT != THHIP_F32)
-		bm = 64, bn = 1;	/* of the half-type kernels only the patch kernel pools */
+	if (pool_patch)
+		bm = 64, bn = 1;
+	if (p.pool && !pool_patch && DT != THHIP_F32 && (!direct || bn == 1))
+		THError("thhip_conv2d: half-type pooling in the epilogue needs the patch kernel or the tiles loaded straight into LDS");
 	if (p.res_mode && (DT != THHIP_F32 || !direct || p.pool))
 		THError("thhip_conv2d: a second tensor is combined only by the fp32 tiles loaded straight into LDS, without pooling");
 	if (p.pool && DT == THHIP_F32 && (!direct || splitk != 1))
@@ -3365,9 +3420,9 @@ extern "C" void thhip_conv2d_layout(const void *x, const void *wpacked, const fl
 }
 
 /* Whether thhip_conv2d_layout_pool2 takes this layer (and is the kernel the
- * layer would run on anyway): half type, channels-last input of 64 or 128
- * planes, 3x3, stride 1, enough tiles; or fp32, plane-major, planes in blocks
- * of 32 and enough tiles that K is not split. */
+ * layer would run on anyway): half type, channels-last input in blocks of 32
+ * planes; or fp32, plane-major, planes in blocks of 32 and enough tiles that K
+ * is not split. */
 extern "C" int thhip_conv2d_pool2_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
 	int padH, int padW, int dtype, int x_layout, int y_channels_last)
 {
@@ -3385,19 +3440,18 @@ extern "C" int thhip_conv2d_pool2_supported(int B, int Ci, int H, int W, int Co,
 	}
 	if (dtype != THHIP_F16 && dtype != THHIP_BF16)
 		return 0;
-	if (x_layout != 1 || (Ci != 64 && Ci != 128) || kH != 3 || kW != 3 || dH != 1 || dW != 1 || padH < 0 || padW < 0)
+	/* half types: channels-last input in whole K-tiles of planes (the patch kernel for 3x3 layers of 64 or 128
+	 * planes with enough tiles, else the tiles loaded straight into LDS: conv_dispatch decides) */
+	if (x_layout != 1 || Ci % 32 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
 		return 0;
 	if (y_channels_last && Co % 4)
 		return 0;
-	const int oW = W + 2 * padW - 2, oH = H + 2 * padH - 2;
+	const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
 	if (oW < 2 || oH < 2)
 		return 0;
 	if ((double)B * Ci * H * W * 2 >= 2147483000.0 || (double)B * Co * oH * oW * 2 >= 2147483000.0)
 		return 0;	/* (the batch would be cut into slices) */
-	const long tpatch = (long)((Co + 63) / 64) * B * ((oW + PATCH_TW - 1) / PATCH_TW) * ((oH + PATCH_TH - 1) / PATCH_TH);
-	const long t256 = (long)((Co + 255) / 256) * (((long)B * oH * oW + 255) / 256);
-	const bool wide256 = Ci % 32 == 0 && Co % 256 == 0 && t256 > 128;
-	return tpatch >= 128 && !(wide256 && Ci > 64) && !g_force_generic_cl && !g_force_bm && !g_force_bn;
+	return !g_force_generic_cl && !g_force_bm && !g_force_bn;
 }
 
 /* thhip_conv2d_layout followed by a 2x2 / stride 2 max pooling without padding
