@@ -335,6 +335,13 @@ int THHipHalfFloat(int enable);
  * nn_SpatialBatchNormalization_updateOutput.  Applies to engines created
  * afterwards; returns the previous setting. */
 int THHipFoldBatchNorm(int enable);
+/* 0 (default): CAddTable / CSubTable compute what the reference's shipped modules
+ * compute (modules/CAddTable.c:59-84: with two inputs CAddTable gives a - b and
+ * CSubTable a + b; with more, 2a + b + c + ... and 0 - b - c - ...).  1: what the
+ * modules' names say (the sum of all inputs; the first minus the others), for
+ * networks trained against Torch's modules.  Applies to engines created
+ * afterwards; returns the previous setting. */
+int THHipTableArithmetic(int as_named);
 /* New: the uint8 engine on the GPU, counterpart of THCreateLowpNetwork
  * (thapi.c:784-796, lowp_basic.c:133-212): activations quantised to
  * [-range/2, range/2) in 255 steps, int8 MFMA GEMM with gemmlowp offsets

@@ -205,6 +205,45 @@ def test_vgg16_full_size_properties(hiplib, oracle):
 
 
 @pytest.mark.gpu
+def test_table_arithmetic_as_named(hiplib, oracle):
+    """THHipTableArithmetic(1): CAddTable adds and CSubTable subtracts (the modules' documented
+    meaning), in the table add's own kernel, in the epilogue of a block's last convolution (identity
+    and projection shortcuts, fp32 planes in blocks of 32) and with three inputs; the default stays
+    the shipped arithmetic (CAddTable.c:59-84), which the other tests pin."""
+    g = cases.rng(7100)
+    def cv(ci, co, k, pad):
+        w = g.standard_normal((co, ci, k, k), dtype=np.float32) * np.float32(np.sqrt(1.0 / (ci * k * k)))
+        return configs.conv(w, g.standard_normal(co, dtype=np.float32) * np.float32(0.1), 1, pad)
+    ident = [{"type": "dropout", "p": 0.0, "inplace": 1, "v2": 1}]
+    stem = [cv(3, 32, 3, 1), configs.relu()]
+    main1, main2, short2 = [cv(32, 32, 3, 1), configs.relu(), cv(32, 32, 3, 1)], [cv(32, 64, 3, 1)], [cv(32, 64, 1, 0)]
+    three = [[cv(64, 8, 3, 1)], [cv(64, 8, 1, 0)], [cv(64, 8, 3, 1)]]
+    x = g.uniform(-1, 1, (2, 3, 12, 12)).astype(np.float32)
+    run = lambda layers, t: oracle.run_layers(layers, t)
+    for kind in ("caddtable", "csubtable"):
+        sign = np.float32(1 if kind == "caddtable" else -1)
+        layers = stem + [{"type": "concattable", "branches": [main1, ident]}, {"type": kind}, configs.relu(),
+                         {"type": "concattable", "branches": [main2, short2]}, {"type": kind}, configs.relu(),
+                         {"type": "concattable", "branches": three}, {"type": kind}]
+        t = run(stem, x)
+        t = np.maximum(run(main1, t) + sign * t, 0)
+        t = np.maximum(run(main2, t) + sign * run(short2, t), 0)
+        want = run(three[0], t) + sign * run(three[1], t) + sign * run(three[2], t)
+        old = hiplib.THHipTableArithmetic(1)
+        try:
+            assert old == 0
+            net = api.HipNetwork(layers)
+        finally:
+            hiplib.THHipTableArithmetic(0)
+        got = net.process_float(x)
+        G.assert_close(got, want.ravel(), NET_TOL, "tables as named, " + kind)
+        net.free()
+        shipped = api.HipNetwork(layers)      # the default again: what the reference's modules compute
+        G.assert_close(shipped.process_float(x), run(layers, x).ravel(), NET_TOL, "tables as shipped, " + kind)
+        shipped.free()
+
+
+@pytest.mark.gpu
 def test_graph_form_networks(hiplib, oracle):
     """Modules that name their inputs (ninputs / inputs[], thapi.c:173-193): the residual
     network as a flat graph gives bit for bit what its ConcatTable / CAddTable form gives,

@@ -55,6 +55,7 @@ PROTOTYPES = {
     "THCreateHipNetwork": (vp, [vp]),
     "THHipHalfFloat": (C.c_int, [C.c_int]),
     "THHipFoldBatchNorm": (C.c_int, [C.c_int]),
+    "THHipTableArithmetic": (C.c_int, [C.c_int]),
     "THCreateHipLowpNetwork": (vp, [vp, C.c_float]),
     "THHipTensor_newFromFloatTensor": (vp, [vp]),
     "THFloatTensor_newFromHipTensor": (vp, [vp]),

@@ -47,6 +47,20 @@ int THHipFoldBatchNorm(int enable)
 	return old;
 }
 
+static int g_table_math;
+
+/* 0 (default): CAddTable / CSubTable compute what the reference's shipped modules compute
+ * (two inputs: a - b for CAddTable and a + b for CSubTable; more: 2a + b + c + ..., 0 - b - c - ...
+ * CAddTable.c:59-84).  1: what the modules' names say (the sum of all inputs; the first minus the
+ * others), for networks trained against Torch's modules.  Read at engine creation; returns the
+ * previous setting. */
+int THHipTableArithmetic(int as_named)
+{
+	const int old = g_table_math;
+	g_table_math = as_named != 0;
+	return old;
+}
+
 int thhip_engine_dtype(void)
 {
 	return g_halfmode == 1 ? THHIP_F16 : g_halfmode == 2 ? THHIP_BF16 : THHIP_F32;
@@ -578,7 +592,13 @@ static THFloatTensor *Hip_CAddTable_updateOutput(struct module *m, THFloatTensor
 		return m->output;
 	}
 	void *y = out_resize(m, dt, a->nDimension, a->size);
-	if (nelem == 2) {
+	if (hm->table_named) {	/* THHipTableArithmetic(1): the first input plus (minus) every other one */
+		if (nelem == 1)
+			thhip_memcpy_d2d(y, thhip_tensor_ptr(a, dt), (size_t)na * esize_of(dt));
+		for (int i = 1; i < nelem; i++)
+			thhip_axpby2(i == 1 ? thhip_tensor_ptr(a, dt) : y, thhip_tensor_ptr(mods[i].output, dt), y, na,
+				THFloatTensor_nElement(mods[i].output), sub ? -1.0f : 1.0f, (i == nelem - 1) ? hm->fused_act : 0, dt);
+	} else if (nelem == 2) {
 		THFloatTensor *b = mods[1].output;
 		thhip_axpby2(thhip_tensor_ptr(a, dt), thhip_tensor_ptr(b, dt), y, na, THFloatTensor_nElement(b),
 			sub ? 1.0f : -1.0f, hm->fused_act, dt);
@@ -1138,6 +1158,7 @@ static void convert_module(struct hipnet *hn, struct network *src, int i, int en
 		if (lowp)
 			THError("MT_CAddTable not supported in lowp");
 		m->updateOutput = Hip_CAddTable_updateOutput;
+		hm->table_named = g_table_math;
 		break;
 	default:
 		THError("module type %d is not supported by the HIP engine", sm->type);
@@ -1395,7 +1416,8 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			continue;
 		struct hipmod *chm = hipmod_of(conv);
 		chm->res_mode = identity ? 1 : 2;
-		chm->res_c = add->type == MT_CSubTable ? 1.0f : -1.0f;	/* the arithmetic as shipped: CAddTable.c:59-70 */
+		/* the arithmetic as shipped (CAddTable.c:59-70: the two-input CAddTable subtracts), or as named */
+		chm->res_c = (add->type == MT_CSubTable) != (hn->hm[i + 1].table_named != 0) ? 1.0f : -1.0f;
 		chm->res_act = hn->hm[i + 1].fused_act;
 		chm->res_add = &hn->hm[i + 1];
 		hn->hm[i].res_target = chm;
