@@ -2172,7 +2172,8 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 #pragma unroll
 		for (int q = 0; q < NPOS; q++) {
 			const int iy = iy0_[q] + t_kh, ix = ix0_[q] + t_kw;
-			const bool ok = n_ok_[q] && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			/* (no branches in a K step: the compiler may then spread its loads between the MFMAs) */
+			const bool ok = (int)n_ok_[q] & (int)((unsigned)iy < (unsigned)p.H) & (int)((unsigned)ix < (unsigned)p.W);
 			const unsigned voff = ok ? (unsigned)(xoff_[q] + tap_off) * (unsigned)sizeof(float) : 0x80000000u;
 #pragma unroll
 			for (int r = 0; r < KT / WAVES; r++) {
@@ -2183,16 +2184,14 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 			}
 		}
 		t_kc += KCH;
-		if (++t_sub == SUB) {	/* the next planes of the block first, then the next tap */
-			t_sub = 0;
-			if (++t_kw == p.kW) {
-				t_kw = 0;
-				if (++t_kh == p.kH) {
-					t_kh = 0;
-					++t_cb;
-				}
-			}
-		}
+		/* the next planes of the block first, then the next tap */
+		const int sub1 = t_sub + 1, wrap_s = sub1 == SUB;
+		t_sub = __builtin_amdgcn_readfirstlane(wrap_s ? 0 : sub1);
+		const int kw1 = t_kw + wrap_s, wrap_w = kw1 == p.kW;
+		t_kw = __builtin_amdgcn_readfirstlane(wrap_w ? 0 : kw1);
+		const int kh1 = t_kh + wrap_w, wrap_h = kh1 == p.kH;
+		t_kh = __builtin_amdgcn_readfirstlane(wrap_h ? 0 : kh1);
+		t_cb = __builtin_amdgcn_readfirstlane(t_cb + wrap_h);
 	};
 
 	floatx4 af[2][TM], bf[2][TN];
