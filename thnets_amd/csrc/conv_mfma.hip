@@ -2251,6 +2251,9 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 #pragma unroll
 		for (int c = 0; c + 1 < KCH; c++) {
 			read_frags(st, c + 1, af[(c + 1) & 1], bf[(c + 1) & 1]);
+			/* the next chunk's fragments are asked for before this chunk's MFMAs (left alone, the
+			 * compiler puts the reads right before their first use) */
+			__builtin_amdgcn_sched_barrier(0);
 			mma(c & 1);
 		}
 		if (steady)
@@ -2258,10 +2261,11 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		else
 			wide_wait<0, true>();
 		__builtin_amdgcn_s_barrier();
-		if (steady || kt + NST < nkt)
-			issue(st);
 		if (steady || kt + 1 < nkt)
 			read_frags(st1, 0, af[0], bf[0]);
+		__builtin_amdgcn_sched_barrier(0);	/* (as above; the loads below mix with the MFMAs) */
+		if (steady || kt + NST < nkt)
+			issue(st);
 		mma((KCH - 1) & 1);
 	};
 	auto round = [&](int kt, auto steady_) {
