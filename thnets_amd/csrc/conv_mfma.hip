@@ -1348,18 +1348,17 @@ __global__ __launch_bounds__(64 * WGM * WGN * KG) void conv_wide_kernel(ConvPara
 #pragma unroll
 		for (int q = 0; q < NPOS; q++) {
 			const int iy = iy0_[q] + t_kh, ix = ix0_[q] + t_kw;
-			const bool ok = live && n_ok_[q] && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			/* (no branches in a K step: the compiler may then spread its loads between the MFMAs) */
+			const bool ok = (int)live & (int)n_ok_[q] & (int)((unsigned)iy < (unsigned)p.H) & (int)((unsigned)ix < (unsigned)p.W);
 			const unsigned voff = ok ? (unsigned)(xoff_[q] + cl_off) : outside;
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(lb + (wave + WAVES * q) * 64), 16, voff, 0, 0, 0);
 		}
 		t_kc += KCH;
-		if (++t_kw == p.kW) {
-			t_kw = 0;
-			if (++t_kh == p.kH) {
-				t_kh = 0;
-				t_cb += KCH * CHUNK;
-			}
-		}
+		const int kw1 = t_kw + 1, wrap_w = kw1 == p.kW;
+		t_kw = __builtin_amdgcn_readfirstlane(wrap_w ? 0 : kw1);
+		const int kh1 = t_kh + wrap_w, wrap_h = kh1 == p.kH;
+		t_kh = __builtin_amdgcn_readfirstlane(wrap_h ? 0 : kh1);
+		t_cb = __builtin_amdgcn_readfirstlane(t_cb + (wrap_h ? KCH * CHUNK : 0));
 	};
 
 	/* fragment addresses: A rows lane % 32 of a block, half lane / 32; B position
@@ -1444,6 +1443,9 @@ __global__ __launch_bounds__(64 * WGM * WGN * KG) void conv_wide_kernel(ConvPara
 #pragma unroll
 		for (int c = 0; c + 1 < KCH; c++) {
 			read_frags(st, c + 1, af[(c + 1) & 1], bf[(c + 1) & 1]);
+			/* the next chunk's fragments are asked for before this chunk's MFMAs (left alone, the
+			 * compiler puts the reads right before their first use) */
+			__builtin_amdgcn_sched_barrier(0);
 			mma(c & 1, kt);
 		}
 		/* this wave's loads of tile kt+1 are in LDS (younger tiles may still be
@@ -1453,10 +1455,11 @@ __global__ __launch_bounds__(64 * WGM * WGN * KG) void conv_wide_kernel(ConvPara
 		else
 			wide_wait<0, true>();
 		__builtin_amdgcn_s_barrier();
-		if (steady || kt + NST < nkt)
-			issue(st);
 		if (steady || kt + 1 < nkt)
 			read_frags(st1, 0, af[0], bf[0]);
+		__builtin_amdgcn_sched_barrier(0);	/* (as above; the loads below mix with the MFMAs) */
+		if (steady || kt + NST < nkt)
+			issue(st);
 		mma((KCH - 1) & 1, kt);
 	};
 	/* NST steps: every stage index a constant */
