@@ -24,9 +24,14 @@ static void thhip_init_once(void)
 	g_init = 1;
 }
 
+/* (counts how often the stream was handed out: the profiler uses it to see that nothing was put on
+ * the stream between two of its launches) */
+static unsigned long g_stream_uses;
+
 hipStream_t thhip_stream(void)
 {
 	thhip_init_once();
+	++g_stream_uses;
 	return g_stream;
 }
 
@@ -118,12 +123,18 @@ extern "C" float thhip_event_ms(int a, int b)
 }
 
 /* ---- per-launch profiler ---- */
-struct ProfRec { int family; hipEvent_t start, stop; double work; };
+struct ProfRec { int family; hipEvent_t start, stop; double work; bool shared_start; };
 static std::vector<ProfRec> g_recs;
 static std::vector<hipEvent_t> g_evpool;
 static int g_prof_on;
 static double g_fam_ms[THHIP_FAM_COUNT], g_fam_work[THHIP_FAM_COUNT];
 static long g_fam_n[THHIP_FAM_COUNT];
+
+/* A launch that follows another profiled launch with nothing put on the stream between them starts
+ * at that launch's stop event: one event per launch instead of two (an event costs a few
+ * microseconds of stream time, which shows on networks of short kernels). */
+static hipEvent_t g_last_stop;
+static unsigned long g_last_stop_uses;	/* g_stream_uses right after that event was recorded; 0: none */
 
 static hipEvent_t prof_event(void)
 {
@@ -148,10 +159,12 @@ static void prof_drain(void)
 		g_fam_ms[g_recs[i].family] += ms;
 		g_fam_work[g_recs[i].family] += g_recs[i].work;
 		g_fam_n[g_recs[i].family]++;
-		g_evpool.push_back(g_recs[i].start);
+		if (!g_recs[i].shared_start)
+			g_evpool.push_back(g_recs[i].start);
 		g_evpool.push_back(g_recs[i].stop);
 	}
 	g_recs.clear();
+	g_last_stop_uses = 0;
 }
 
 int thhip_prof_begin(int family)
@@ -164,10 +177,15 @@ int thhip_prof_begin(int family)
 		prof_drain();
 	ProfRec r;
 	r.family = family;
-	r.start = prof_event();
+	r.shared_start = g_last_stop_uses && g_last_stop_uses == g_stream_uses;
+	if (r.shared_start)
+		r.start = g_last_stop;
+	else {
+		r.start = prof_event();
+		hipcheck(hipEventRecord(r.start, thhip_stream()));
+	}
 	r.stop = prof_event();
 	r.work = 0;
-	hipcheck(hipEventRecord(r.start, thhip_stream()));
 	g_recs.push_back(r);
 	return (int)g_recs.size() - 1;
 }
@@ -178,6 +196,8 @@ void thhip_prof_end(int token, double work)
 		return;
 	g_recs[token].work = work;
 	hipcheck(hipEventRecord(g_recs[token].stop, thhip_stream()));
+	g_last_stop = g_recs[token].stop;
+	g_last_stop_uses = g_stream_uses;
 }
 
 extern "C" void thhip_profile_enable(int on)
