@@ -390,6 +390,72 @@ def test_conv_f32_with_table_add_in_the_epilogue(hiplib, oracle):
     assert not hiplib.thhip_conv2d_residual_supported(2, 64, 32, 32, 64, 3, 3, 1, 1, 1, 1, G.F16)
 
 
+def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
+    """The fp32 kernel for 3x3 / stride 1 / padding 1 layers whose output is whole 16 x 4 or 8 x 8
+    patches (every tap read from one patch of the input in LDS): forced on small layers of both
+    patch shapes, one to six half blocks of input planes, 64 to 192 output planes, with and without
+    the folded batch-norm factor and Threshold; and as the dispatcher picks it (2048 tiles), alone,
+    with the 2x2 pooling and with a table add in its epilogue, each bit for bit the separate
+    kernel on the plain result.  Against the restatement."""
+    from thnets_amd import api
+    g = cases.rng(5400)
+    small = [(2, 32, 16, 16, 64), (1, 64, 24, 24, 128), (3, 32, 8, 32, 64), (2, 96, 40, 24, 192), (1, 32, 4, 16, 64), (1, 32, 8, 8, 64)]
+    for (B, Ci, H, W, Co) in small:
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        raw = oracle.conv2d(x, w, None, (1, 1), (1, 1))
+        for (scale, act) in ((None, 0), (sc, 1)):
+            want = raw * (scale[None, :, None, None] if scale is not None else 1) + b[None, :, None, None]
+            if act:
+                want = np.where(want > 0.05, want, np.float32(-0.5))
+            G.note("fp32 patch kernel, forced, %s act %d" % ((B, Ci, H, W, Co), act))
+            try:
+                hiplib.thhip_conv_set_tuning(64, 1, 0, 0)
+                got = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), act=act, thr=0.05, val=-0.5, dtype=G.F32, scale=scale)
+            finally:
+                hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+            G.assert_close(got, want, FP32_TOL, "fp32 patch kernel " + str((B, Ci, H, W, Co, act)))
+    # as dispatched: 2048 tiles of 64 planes x 64 pixels
+    for (B, Ci, H, W, Co) in ((32, 32, 64, 64, 64), (24, 64, 56, 56, 128)):
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        r = g.standard_normal((B, Co, H, W), dtype=np.float32)
+        args = (B, Ci, H, W, Co, 3, 3, 1, 1, 1, 1)
+        assert hiplib.thhip_conv2d_pool2_supported(*args, G.F32, 0, 0) and hiplib.thhip_conv2d_residual_supported(*args, G.F32)
+        wp = hiplib.thhip_conv_pack_weight_layout(w.ctypes.data, Co, Ci, 3, 3, G.F32, 0)
+        dx, db, ds, dr = (api.DeviceArray(hiplib, a) for a in (x, b, sc, r))
+        n = B * Co * H * W
+        dy, dz, dq = (api.DeviceArray(hiplib, nbytes=n * 4) for _ in range(3))
+        dp, dpq = (api.DeviceArray(hiplib, nbytes=n) for _ in range(2))
+        G.note("fp32 patch kernel, dispatched, %s" % (args,))
+        hiplib.thhip_conv2d_layout(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, *args, 1, 0.05, 0.05, G.F32, 0, 0)
+        hiplib.thhip_maxpool(dy.ptr, dp.ptr, B, Co, H, W, H // 2, W // 2, 2, 2, 2, 2, 0, 0, G.F32)
+        hiplib.thhip_conv2d_layout_pool2(dx.ptr, wp, ds.ptr, db.ptr, dpq.ptr, *args, 1, 0.05, 0.05, G.F32, 0, 0)
+        hiplib.thhip_sync()
+        got = dy.get((B, Co, H, W), np.float32)
+        raw = oracle.conv2d(x, w, None, (1, 1), (1, 1)) * sc[None, :, None, None] + b[None, :, None, None]
+        G.assert_close(got, np.where(raw > 0.05, raw, np.float32(0.05)), FP32_TOL, "fp32 patch kernel, dispatched " + str(args))
+        plain, fused = dp.get((B, Co, H // 2, W // 2), np.float32), dpq.get((B, Co, H // 2, W // 2), np.float32)
+        assert np.array_equal(plain, fused), (args, np.abs(plain - fused).max())
+        assert np.array_equal(plain, got.reshape(B, Co, H // 2, 2, W // 2, 2).max(axis=(3, 5)))
+        for mode in (1, 2):
+            hiplib.thhip_conv2d_layout(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, *args, 0, 0.0, 0.0, G.F32, 0, 0)
+            if mode == 1:
+                hiplib.thhip_axpby2(dy.ptr, dr.ptr, dz.ptr, n, n, -1.0, 1, G.F32)
+            else:
+                hiplib.thhip_axpby2(dr.ptr, dy.ptr, dz.ptr, n, n, -1.0, 1, G.F32)
+            hiplib.thhip_conv2d_residual(dx.ptr, wp, ds.ptr, db.ptr, dr.ptr, mode, -1.0, 1, dq.ptr, *args, 0, 0.0, 0.0, G.F32)
+            hiplib.thhip_sync()
+            plain, fused = dz.get((B, Co, H, W), np.float32), dq.get((B, Co, H, W), np.float32)
+            assert np.array_equal(plain, fused), (args, mode, np.abs(plain - fused).max())
+            G.assert_close(fused, np.maximum(raw - r if mode == 1 else r - raw, 0), FP32_TOL, "fp32 patch kernel + table add " + str(args))
+        hiplib.thhip_free(wp)
+
+
 def test_conv_f32_with_pooling_in_the_epilogue(hiplib, oracle):
     """fp32 convolution -> (factor, bias, Threshold) -> 2x2 / stride 2 max pooling in one
     kernel: against the pooling kernel on the plain convolution's output (the same comparisons;

@@ -2339,6 +2339,249 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 #endif
 }
 
+/* ------------------------------------------------------------------ */
+/* fp32, plane-major, 3x3 / stride 1 / padding 1: taps from a patch in LDS */
+/* ------------------------------------------------------------------ */
+
+/* v of lane ^ 8 */
+__device__ __forceinline__ float conv_lane_xor8(float v)
+{
+	return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x201F));
+}
+
+/* Epilogue of conv_f32_patch_kernel: position n = wn 32 + lane % 32 of the tile is pixel (n / TW, n % TW)
+ * of the TW-wide patch of outputs at (y0, x0) of image b.  (Folded batch norm factor,) bias, threshold,
+ * the 2x2 / stride 2 max pooling that follows (a window's other column is the next lane, its other row
+ * lane ^ TW; SpatialMaxPooling.c:51-66's comparisons in their order), the second tensor of a table
+ * add, plane-major store.  lrow: 128 ints of LDS no wave still reads. */
+template <int TW>
+__device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx16 &acc, int tile_m, int b, int y0, int x0, int *lrow)
+{
+	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave % 2, wn = wave / 2;
+	float *y = (float *)p.y;
+	if (tid < 64) {
+		const int mc = min(tile_m * 64 + tid, p.Co - 1);
+		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
+		if (p.scale)
+			lrow[64 + tid] = __float_as_int(p.scale[mc]);
+	}
+	__syncthreads();
+	const bool has_scale = p.scale != 0;
+	const int n = wn * 32 + (lane & 31), py = n / TW, px = n % TW;
+	const int oHW = p.pool ? p.pHW : p.oHW;
+	const bool valid = !p.pool || (!(py & 1) && !(px & 1));
+	const size_t ybase = (size_t)b * p.Co * oHW +
+		(p.pool ? ((y0 + py) >> 1) * p.pW + ((x0 + px) >> 1) : (y0 + py) * p.oW + x0 + px);
+	const int m0 = tile_m * 64 + wm * 32 + 4 * (lane >> 5);
+	/* the other tensor's sixteen values, all requested before the first is used */
+	float other[16];
+	if (p.res_mode) {
+#pragma unroll
+		for (int r = 0; r < 16; r++) {
+			const int m = m0 + 8 * (r >> 2) + (r & 3);
+			other[r] = valid && m < p.Co ? p.res[ybase + (size_t)m * oHW] : 0.0f;
+		}
+	}
+#pragma unroll
+	for (int g = 0; g < 4; g++) {
+		const int ml = wm * 32 + 4 * (lane >> 5) + 8 * g;
+		const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+		floatx4 rowscale = { 1, 1, 1, 1 };
+		if (has_scale)
+			rowscale = *(const floatx4 *)(lrow + 64 + ml);
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			const int r = 4 * g + e, m = m0 + 8 * g + e;
+			float v = has_scale ? acc[r] * rowscale[e] + rowbias[e] : acc[r] + rowbias[e];
+			if (p.act)
+				v = v > p.thr ? v : p.val;
+			if (p.pool) {
+				const float v01 = conv_lane_next(v);
+				const float v10 = TW == 16 ? conv_lane_xor16(v) : conv_lane_xor8(v);
+				const float v11 = TW == 16 ? conv_lane_xor16(v01) : conv_lane_xor8(v01);
+				float mx = -FLT_MAX;
+				mx = v > mx ? v : mx;
+				mx = v01 > mx ? v01 : mx;
+				mx = v10 > mx ? v10 : mx;
+				mx = v11 > mx ? v11 : mx;
+				v = mx;
+			}
+			if (valid && m < p.Co) {
+				if (p.res_mode) {
+					v = p.res_mode == 1 ? v + p.res_c * other[r] : other[r] + p.res_c * v;
+					if (p.res_act)
+						v = v > 0.0f ? v : 0.0f;
+				}
+				y[ybase + (size_t)m * oHW] = v;
+			}
+		}
+	}
+}
+
+/* 3x3 / stride 1 / padding 1 layers whose output splits into whole TW x TH patches of 64 pixels: a
+ * workgroup computes 64 planes of one patch.  Where conv_f32_direct_kernel fetches every tap's 64
+ * pixels of a plane with a load of its own (nine loads a plane, 0.5 wave-wide loads per MFMA: measured,
+ * they cost 5-8 % of that kernel's time even when they all hit the cache), this kernel loads the
+ * (TH + 2) x (TW + 2) input pixels under the patch once per plane (two loads, what lies outside the
+ * image pointed past the buffer's range and so 0.0) and every tap reads them from LDS at its own
+ * offset; no tap arithmetic and no bounds tests remain in the K loop.  The packed weights' K order
+ * (block of 32 planes, tap, plane) is walked as (half block of 16 planes, tap): sixteen planes'
+ * patches are one buffer (two buffers, the next half block's loads spread over this one's taps),
+ * the weights' 1 KiB blocks go through a ring of three K-tiles as in conv_f32_direct_kernel.  The
+ * nine taps of a half block are straight-line code: every LDS offset and wait count a constant. */
+template <int TW, int TH>
+__global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
+	constexpr int MB = 2, KCH = 2, NST = 3, BLK = 16;
+	static_assert(TW * TH == 64 && (TW == 16 || TW == 8), "64 pixels, rows of 16 or 8");
+	constexpr int PWD = TW + 2, PEL = (TH + 2) * PWD;	/* the patch of one plane: row length, elements */
+	static_assert(PEL <= 128, "two wave-wide loads a plane");
+	constexpr int PSTRIDE = 132;	/* floats between the planes of a buffer: room for two loads of 64, four planes = 16 banks */
+	constexpr int A_VECS = MB * KCH * 64, B_FLOATS = BLK * PSTRIDE;
+	/* (one array, every stage and buffer at a constant offset, as in the kernels above: with separate
+	 * arrays, or a buffer index computed at run time, the compiler waits for all outstanding loads
+	 * before every LDS read) */
+	__shared__ floatx4 lds[NST * A_VECS + 2 * B_FLOATS / 4];
+	floatx4 *const lds_a = lds;
+	float *const lds_b0 = (float *)(lds + NST * A_VECS), *const lds_b1 = lds_b0 + B_FLOATS;
+
+	const int tid = threadIdx.x;
+	const int lane = tid & 63;
+	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+	const int wm = wave % 2, wn = wave / 2;
+	int tile_m, tile_n;
+	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
+		const int bid = blockIdx.x, xcd = bid & 7, local = bid >> 3;
+		int m0, mw, n0, cnt;
+		conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
+		if (local >= cnt)
+			return;
+		tile_m = m0 + local % mw;
+		tile_n = n0 + local / mw;
+	}
+	/* tile_n counts patches: image, patch row, patch column */
+	const int TX = p.oW / TW, TXY = TX * (p.oH / TH);
+	const int b = tile_n / TXY, trem = tile_n - b * TXY, ty = trem / TX;
+	const int y0 = ty * TH, x0 = (trem - ty * TX) * TW;
+
+	/* ---- what this lane fetches of every plane: patch elements lane and 64 + lane ---- */
+	unsigned voff_[2];
+#pragma unroll
+	for (int j = 0; j < 2; j++) {
+		const int e = 64 * j + lane, r = e / PWD, c = e - r * PWD;
+		const int iy = y0 - 1 + r, ix = x0 - 1 + c;
+		const bool ok = e < PEL && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+		voff_[j] = ok ? (unsigned)(((b * p.Ci * p.H + iy) * p.W + ix) * (int)sizeof(float)) : 0x80000000u;
+	}
+	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
+	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
+	const int plane_bytes = p.HW * (int)sizeof(float);
+	const int NB = p.Ci / BLK;	/* half blocks */
+	/* this wave's weight block of a K-tile: 32-row block wave % 2, chunk wave / 2 */
+	const unsigned a_base = (unsigned)(tile_m * MB + wave % MB) * (unsigned)p.KC * 1024u;
+	const int a_kci = wave / MB, a_lds = (a_kci * MB + wave % MB) * 64;
+
+	/* the weights of K-tile (half block hb, tap): chunks ((hb / 2) 9 + tap) 4 + (hb % 2) 2 + {0, 1};
+	 * past the last half block nothing is fetched (zeros arrive, nobody reads them) */
+	auto issue_a = [&](auto st_, int hb, int tap) {
+		constexpr int st = decltype(st_)::value;
+		const unsigned kc = (unsigned)(((hb >> 1) * 9 + tap) * 4 + (hb & 1) * 2 + a_kci);
+		__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(lds_a + st * A_VECS + a_lds), 16,
+			hb < NB ? lane * 16 : 0x80000000u, a_base + kc * 1024u, 0, 0);
+	};
+	/* load t (0..7) of this wave's share of half block hb's patches into buffer buf: plane wave + 4 (t / 2),
+	 * elements 64 (t % 2).. */
+	auto issue_b = [&](int t, int hb, auto buf_) {
+		constexpr int buf = decltype(buf_)::value;
+		const int plane = wave + 4 * (t >> 1), j = t & 1;
+		float *dst = (buf ? lds_b1 : lds_b0) + plane * PSTRIDE + 64 * j;
+		/* the scalar offset is not range checked: the planes exist (hb < NB) */
+		__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(dst), 4,
+			hb < NB ? voff_[j] : 0x80000000u, hb < NB ? (hb * BLK + plane) * plane_bytes : 0, 0, 0);
+	};
+
+	/* fragments: A rows lane % 32 of block wm, half lane / 32; B pixel n of the patch, planes
+	 * 8 chunk + 4 (lane / 32) + step of the half block, at the tap's offset */
+	const int n = wn * 32 + (lane & 31);
+	const int bfrag = (lane >> 5) * 4 * PSTRIDE + (n / TW) * PWD + n % TW;
+	auto read_frags = [&](auto st_, auto buf_, auto tap_, int c, floatx4 &a, floatx4 &bq) {
+		constexpr int st = decltype(st_)::value, tap = decltype(tap_)::value, buf = decltype(buf_)::value;
+		a = lds_a[st * A_VECS + (c * MB + wm) * 64 + lane];
+		const float *src = (buf ? lds_b1 : lds_b0) + bfrag + (tap / 3) * PWD + tap % 3 + c * 8 * PSTRIDE;
+#pragma unroll
+		for (int e = 0; e < 4; e++)
+			bq[e] = src[e * PSTRIDE];
+	};
+
+	floatx16 acc;
+#pragma unroll
+	for (int r = 0; r < 16; r++)
+		acc[r] = 0;
+	floatx4 af[2], bf[2];
+
+	typedef std::integral_constant<int, 0> C0;
+	typedef std::integral_constant<int, 1> C1;
+	typedef std::integral_constant<int, 2> C2;
+#pragma unroll
+	for (int t = 0; t < 8; t++)
+		issue_b(t, 0, C0{});
+	issue_a(C0{}, 0, 0);
+	issue_a(C1{}, 0, 1);
+	issue_a(C2{}, 0, 2);
+	wide_wait<2, false>();	/* the patches and the first K-tile's weights */
+	__builtin_amdgcn_s_barrier();
+	read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
+
+	/* K-tile (hb, tap): its weights in stage tap % 3, the next K-tile's in the next stage.  Loads are issued
+	 * patch first, weights second; the weights of the next K-tile were issued two steps ago, so at most the
+	 * last step's loads may still be on their way: its weights and, unless that step was a half block's
+	 * last, a patch load.  A half block's last step waits for the patch loads of the next as well. */
+	auto step = [&](int hb, auto buf_, auto tap_) {
+		constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
+		typedef std::integral_constant<int, tap % 3> ST;
+		typedef std::integral_constant<int, (tap + 1) % 3> ST1;
+		typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
+		typedef std::integral_constant<int, buf ^ 1> OTHER;
+		typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
+		read_frags(ST{}, buf_, tap_, 1, af[1], bf[1]);
+		/* (the fragments are asked for before the MFMAs that follow in the source; left alone, the
+		 * compiler puts the reads right before their first use) */
+		__builtin_amdgcn_sched_barrier(0);
+		conv_mma<THHIP_F32>(acc, af[0], bf[0]);
+		wide_wait<(tap >= 1 && tap <= 7) ? 2 : 1, true>();
+		__builtin_amdgcn_s_barrier();
+		read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[0], bf[0]);
+		__builtin_amdgcn_sched_barrier(0);
+		if constexpr (tap < 8)
+			issue_b(tap, hb + 1, OTHER{});
+		if constexpr (tap + 3 < 9)
+			issue_a(ST{}, hb, tap + 3);
+		else
+			issue_a(ST{}, hb + 1, tap + 3 - 9);
+		conv_mma<THHIP_F32>(acc, af[1], bf[1]);
+	};
+	auto half_block = [&](int hb, auto buf_) {
+		step(hb, buf_, std::integral_constant<int, 0>{});
+		step(hb, buf_, std::integral_constant<int, 1>{});
+		step(hb, buf_, std::integral_constant<int, 2>{});
+		step(hb, buf_, std::integral_constant<int, 3>{});
+		step(hb, buf_, std::integral_constant<int, 4>{});
+		step(hb, buf_, std::integral_constant<int, 5>{});
+		step(hb, buf_, std::integral_constant<int, 6>{});
+		step(hb, buf_, std::integral_constant<int, 7>{});
+		step(hb, buf_, std::integral_constant<int, 8>{});
+	};
+	for (int hb = 0; hb < NB; hb += 2) {	/* (Ci % 32 == 0: an even number of half blocks) */
+		half_block(hb, C0{});
+		half_block(hb + 1, C1{});
+	}
+	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the epilogue reuses it) */
+	__syncthreads();
+	conv_f32_patch_store<TW>(p, acc, tile_m, b, y0, x0, (int *)lds_a);
+#endif
+}
+
 /* Adds the K parts of the tiles conv_f32_direct_kernel cut (one workgroup per
  * such tile, [xcd][tile][part][register][thread] in scratch) in their order
  * and finishes them as that kernel's epilogue does. */
@@ -2928,6 +3171,40 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 		conv_f32_tail_finish_kernel<BM, BN><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
+/* Whether conv_f32_patch_kernel can run this layer, and with which patch: plane-major fp32 on both
+ * sides, 3x3 / stride 1 / padding 1, whole blocks of 32 input and 64 output planes, an output of whole
+ * 16 x 4 or 8 x 8 patches.  Returns the patch width (16, 8) or 0. */
+static int conv_f32_patch_width(const ConvParams &p)
+{
+	if (p.x_cl || p.y_cl || p.kH != 3 || p.kW != 3 || p.dH != 1 || p.dW != 1 || p.padH != 1 || p.padW != 1)
+		return 0;
+	if (p.Ci % 32 || p.Co % 64 || p.x_bytes >= 0x7fffffffu)
+		return 0;
+	if (p.oW % 16 == 0 && p.oH % 4 == 0)
+		return 16;
+	if (p.oW % 8 == 0 && p.oH % 8 == 0)
+		return 8;
+	return 0;
+}
+
+template <int TW, int TH>
+static void conv_launch_f32_patch(ConvParams &p)
+{
+	p.tiles_m = p.Co / 64;
+	p.tiles_n = p.B * (p.oH / TH) * (p.oW / TW);
+	p.splitk = 1;
+	if ((size_t)p.tiles_m * 2 * p.KC * 1024 > p.w_bytes || p.KC != p.Ci / 8 * 9)
+		THError("thhip_conv2d: packed weights do not fit the patch kernel's tile grid");
+	const double wbytes = (double)p.Co * p.K * 4;
+	p.mparts = 1;
+	while (p.mparts < 8 && p.mparts * 2 <= p.tiles_m && wbytes / p.mparts > 2.5e6)
+		p.mparts *= 2;
+	if (g_force_mparts)
+		p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
+	const size_t maxcnt = conv_tail_plan(p, 0, 0, 0, 0);	/* (no tiles are cut: the layers this kernel takes have thousands) */
+	conv_f32_patch_kernel<TW, TH><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
+}
+
 /* Whether conv_patch_kernel can run this layer. */
 template <int DT>
 static bool conv_patch_ok(const ConvParams &p)
@@ -3070,6 +3347,9 @@ static void conv_dispatch(ConvParams &p)
 				bn = 128;
 		} else if (p.x_cl == 1 && t128 >= 512)
 			bm = bn = 128;
+	} else if (DT == THHIP_F32 && conv_f32_patch_width(p) && t64 >= 2000 && !g_force_kch && !g_force_bm && !g_force_bn) {
+		/* 3x3 layers of many whole patches: the taps from a patch in LDS (conv_f32_patch_kernel) */
+		bn = 1;
 	} else if (DT == THHIP_F32 && conv_f32_direct_ok(p) && !g_force_kch) {
 		/* planes in blocks of 32: operands straight into LDS, 64x64 tiles
 		 * (measured 2-7 % over the register-staged kernel on every VGG layer,
@@ -3136,6 +3416,17 @@ static void conv_dispatch(ConvParams &p)
 		bm = 64, bn = 1;
 	if (p.pool && !pool_patch && DT != THHIP_F32 && (!direct || bn == 1))
 		THError("thhip_conv2d: half-type pooling in the epilogue needs the patch kernel or the tiles loaded straight into LDS");
+	if constexpr (DT == THHIP_F32) {
+		if (bn == 1) {	/* (64, 1): the fp32 patch kernel */
+			const int tw = conv_f32_patch_width(p);
+			if (!tw)
+				THError("thhip_conv2d: the fp32 patch kernel needs plane-major tensors, 3x3 / stride 1 / padding 1, "
+					"Ci %% 32 == 0, Co %% 64 == 0 and an output of whole 16x4 or 8x8 patches");
+			if (tw == 16)
+				return conv_launch_f32_patch<16, 4>(p);
+			return conv_launch_f32_patch<8, 8>(p);
+		}
+	}
 	if (p.res_mode && (DT != THHIP_F32 || !direct || p.pool))
 		THError("thhip_conv2d: a second tensor is combined only by the fp32 tiles loaded straight into LDS, without pooling");
 	if (p.pool && DT == THHIP_F32 && (!direct || splitk != 1))
