@@ -391,15 +391,17 @@ def test_conv_f32_with_table_add_in_the_epilogue(hiplib, oracle):
 
 
 def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
-    """The fp32 kernel for 3x3 / stride 1 / padding 1 layers whose output is whole 16 x 4 or 8 x 8
-    patches (every tap read from one patch of the input in LDS): forced on small layers of both
-    patch shapes, one to six half blocks of input planes, 64 to 192 output planes, with and without
-    the folded batch-norm factor and Threshold; and as the dispatcher picks it (2048 tiles), alone,
-    with the 2x2 pooling and with a table add in its epilogue, each bit for bit the separate
-    kernel on the plain result.  Against the restatement."""
+    """The fp32 kernel for 3x3 / stride 1 / padding 1 layers whose output is whole 16x4, 8x8 or 4x4
+    patches (every tap read from one patch of the input in LDS): forced on small layers of all
+    three patch shapes (a last tile of fewer than four 4x4 patches among them), two to six half
+    blocks of input planes, 64 to 192 output planes, with and without the folded batch-norm factor
+    and Threshold; and as the dispatcher picks it (2000 tiles and more; the last tiles of an XCD
+    cut along K), alone, with the 2x2 pooling and with a table add in its epilogue, each bit for
+    bit the separate kernel on the plain result.  Against the restatement."""
     from thnets_amd import api
     g = cases.rng(5400)
-    small = [(2, 32, 16, 16, 64), (1, 64, 24, 24, 128), (3, 32, 8, 32, 64), (2, 96, 40, 24, 192), (1, 32, 4, 16, 64), (1, 32, 8, 8, 64)]
+    small = [(2, 32, 16, 16, 64), (1, 64, 24, 24, 128), (3, 32, 8, 32, 64), (2, 96, 40, 24, 192), (1, 32, 4, 16, 64), (1, 32, 8, 8, 64),
+             (2, 32, 12, 12, 64), (1, 64, 28, 28, 128), (3, 32, 4, 4, 64)]
     for (B, Ci, H, W, Co) in small:
         x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
         w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
@@ -418,7 +420,7 @@ def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
                 hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
             G.assert_close(got, want, FP32_TOL, "fp32 patch kernel " + str((B, Ci, H, W, Co, act)))
     # as dispatched: 2048 tiles of 64 planes x 64 pixels
-    for (B, Ci, H, W, Co) in ((32, 32, 64, 64, 64), (24, 64, 56, 56, 128)):
+    for (B, Ci, H, W, Co) in ((32, 32, 64, 64, 64), (24, 64, 56, 56, 128), (44, 64, 28, 28, 256), (140, 32, 24, 40, 64)):
         x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
         w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
         b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)

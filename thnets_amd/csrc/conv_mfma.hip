@@ -2343,20 +2343,49 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 /* fp32, plane-major, 3x3 / stride 1 / padding 1: taps from a patch in LDS */
 /* ------------------------------------------------------------------ */
 
-/* v of lane ^ 8 */
+/* A tile of conv_f32_patch_kernel: 64 output pixels as NP patches of SW x SH (16x4, 8x8: one patch;
+ * 4x4: four neighbouring patches in the order image, patch row, patch column). */
+template <int SW, int SH>
+struct ConvPatchGeo {
+	static_assert((SW == 16 && SH == 4) || (SW == 8 && SH == 8) || (SW == 4 && SH == 4), "16x4, 8x8 or four 4x4 patches");
+	static constexpr int NPOS = SW * SH, NP = 64 / NPOS;
+	static constexpr int PWD = SW + 2, PEL_S = (SH + 2) * PWD;	/* the input under one patch: row length, elements */
+	static constexpr int PEL = NP * PEL_S, NL = (PEL + 63) / 64;	/* elements and wave-wide loads per plane */
+	static constexpr int PSTRIDE = 64 * NL + 4;	/* floats between the planes of a buffer (four planes = 16 banks) */
+};
+
+/* patch sp of the layer: image and first output pixel; false past the last patch */
+template <int SW, int SH>
+__device__ __forceinline__ bool conv_patch_origin(const ConvParams &p, int sp, int &b, int &y0, int &x0)
+{
+	const int SX = p.oW / SW, SXY = SX * (p.oH / SH);
+	b = sp / SXY;
+	const int rem = sp - b * SXY, sy = rem / SX;
+	y0 = sy * SH;
+	x0 = (rem - sy * SX) * SW;
+	return b < p.B;
+}
+
+/* v of lane ^ 8, v of lane ^ 4 */
 __device__ __forceinline__ float conv_lane_xor8(float v)
 {
 	return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x201F));
 }
 
-/* Epilogue of conv_f32_patch_kernel: position n = wn 32 + lane % 32 of the tile is pixel (n / TW, n % TW)
- * of the TW-wide patch of outputs at (y0, x0) of image b.  (Folded batch norm factor,) bias, threshold,
- * the 2x2 / stride 2 max pooling that follows (a window's other column is the next lane, its other row
- * lane ^ TW; SpatialMaxPooling.c:51-66's comparisons in their order), the second tensor of a table
- * add, plane-major store.  lrow: 128 ints of LDS no wave still reads. */
-template <int TW>
-__device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx16 &acc, int tile_m, int b, int y0, int x0, int *lrow)
+__device__ __forceinline__ float conv_lane_xor4(float v)
 {
+	return __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), 0x101F));
+}
+
+/* Epilogue of conv_f32_patch_kernel: position n = wn 32 + lane % 32 of tile tile_n is pixel
+ * ((n % NPOS) / SW, n % SW) of patch tile_n NP + n / NPOS.  (Folded batch norm factor,) bias, threshold,
+ * the 2x2 / stride 2 max pooling that follows (a window's other column is the next lane, its other row
+ * lane ^ SW; SpatialMaxPooling.c:51-66's comparisons in their order), the second tensor of a table
+ * add, plane-major store.  lrow: 128 ints of LDS no wave still reads. */
+template <int SW, int SH>
+__device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx16 &acc, int tile_m, int tile_n, int *lrow)
+{
+	typedef ConvPatchGeo<SW, SH> GEO;
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave % 2, wn = wave / 2;
 	float *y = (float *)p.y;
 	if (tid < 64) {
@@ -2367,9 +2396,13 @@ __device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx
 	}
 	__syncthreads();
 	const bool has_scale = p.scale != 0;
-	const int n = wn * 32 + (lane & 31), py = n / TW, px = n % TW;
+	const int n = wn * 32 + (lane & 31), ln = n % GEO::NPOS, py = ln / SW, px = ln % SW;
+	int b, y0, x0;
+	bool valid = conv_patch_origin<SW, SH>(p, tile_n * GEO::NP + n / GEO::NPOS, b, y0, x0);
+	b = valid ? b : 0;
 	const int oHW = p.pool ? p.pHW : p.oHW;
-	const bool valid = !p.pool || (!(py & 1) && !(px & 1));
+	if (p.pool)
+		valid = valid && !(py & 1) && !(px & 1);
 	const size_t ybase = (size_t)b * p.Co * oHW +
 		(p.pool ? ((y0 + py) >> 1) * p.pW + ((x0 + px) >> 1) : (y0 + py) * p.oW + x0 + px);
 	const int m0 = tile_m * 64 + wm * 32 + 4 * (lane >> 5);
@@ -2397,8 +2430,8 @@ __device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx
 				v = v > p.thr ? v : p.val;
 			if (p.pool) {
 				const float v01 = conv_lane_next(v);
-				const float v10 = TW == 16 ? conv_lane_xor16(v) : conv_lane_xor8(v);
-				const float v11 = TW == 16 ? conv_lane_xor16(v01) : conv_lane_xor8(v01);
+				const float v10 = SW == 16 ? conv_lane_xor16(v) : SW == 8 ? conv_lane_xor8(v) : conv_lane_xor4(v);
+				const float v11 = SW == 16 ? conv_lane_xor16(v01) : SW == 8 ? conv_lane_xor8(v01) : conv_lane_xor4(v01);
 				float mx = -FLT_MAX;
 				mx = v > mx ? v : mx;
 				mx = v01 > mx ? v01 : mx;
@@ -2418,26 +2451,29 @@ __device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx
 	}
 }
 
-/* 3x3 / stride 1 / padding 1 layers whose output splits into whole TW x TH patches of 64 pixels: a
- * workgroup computes 64 planes of one patch.  Where conv_f32_direct_kernel fetches every tap's 64
- * pixels of a plane with a load of its own (nine loads a plane, 0.5 wave-wide loads per MFMA: measured,
- * they cost 5-8 % of that kernel's time even when they all hit the cache), this kernel loads the
- * (TH + 2) x (TW + 2) input pixels under the patch once per plane (two loads, what lies outside the
- * image pointed past the buffer's range and so 0.0) and every tap reads them from LDS at its own
- * offset; no tap arithmetic and no bounds tests remain in the K loop.  The packed weights' K order
- * (block of 32 planes, tap, plane) is walked as (half block of 16 planes, tap): sixteen planes'
- * patches are one buffer (two buffers, the next half block's loads spread over this one's taps),
- * the weights' 1 KiB blocks go through a ring of three K-tiles as in conv_f32_direct_kernel.  The
- * nine taps of a half block are straight-line code: every LDS offset and wait count a constant. */
-template <int TW, int TH>
+/* 3x3 / stride 1 / padding 1 layers whose output splits into whole 16x4, 8x8 or 4x4 patches: a
+ * workgroup computes 64 planes of 64 pixels (one patch, or four of 4x4).  Where
+ * conv_f32_direct_kernel fetches every tap's 64 pixels of a plane with a load of its own (nine loads
+ * a plane, 0.5 wave-wide loads per MFMA: measured, they cost 5-8 % of that kernel's time even when
+ * they all hit the cache), this kernel loads the (SH + 2) x (SW + 2) input pixels under each patch
+ * once per plane (two or three loads, what lies outside the image pointed past the buffer's range
+ * and so 0.0) and every tap reads them from LDS at its own offset; no tap arithmetic and no bounds
+ * tests remain in the K loop.  The packed weights' K order (block of 32 planes, tap, plane) is
+ * walked as (half block of 16 planes, tap): sixteen planes' patches are one buffer (two buffers, the
+ * next half block's loads spread over this one's taps), the weights' 1 KiB blocks go through a ring
+ * of three K-tiles as in conv_f32_direct_kernel.  The nine taps of a half block are straight-line
+ * code: every LDS offset and wait count a constant.  The last tiles of an XCD are cut along K as
+ * there (conv_tail_parts; a part is whole blocks of 32 planes), summed by
+ * conv_f32_patch_tail_finish_kernel. */
+template <int SW, int SH>
 __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
+	typedef ConvPatchGeo<SW, SH> GEO;
 	constexpr int MB = 2, KCH = 2, NST = 3, BLK = 16;
-	static_assert(TW * TH == 64 && (TW == 16 || TW == 8), "64 pixels, rows of 16 or 8");
-	constexpr int PWD = TW + 2, PEL = (TH + 2) * PWD;	/* the patch of one plane: row length, elements */
-	static_assert(PEL <= 128, "two wave-wide loads a plane");
-	constexpr int PSTRIDE = 132;	/* floats between the planes of a buffer: room for two loads of 64, four planes = 16 banks */
+	constexpr int PWD = GEO::PWD, PSTRIDE = GEO::PSTRIDE, NL = GEO::NL;
+	constexpr int BL = 4 * NL;	/* patch loads per wave and half block: planes wave + 4 i, NL loads each */
+	static_assert(BL <= 8 || BL == 12, "the patch loads are spread over the first taps of a half block");
 	constexpr int A_VECS = MB * KCH * 64, B_FLOATS = BLK * PSTRIDE;
 	/* (one array, every stage and buffer at a constant offset, as in the kernels above: with separate
 	 * arrays, or a buffer index computed at run time, the compiler waits for all outstanding loads
@@ -2450,34 +2486,47 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 	const int lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int wm = wave % 2, wn = wave / 2;
-	int tile_m, tile_n;
-	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
-		const int bid = blockIdx.x, xcd = bid & 7, local = bid >> 3;
+	int tile_m, tile_n, split = 0, nsplit = 1;
+	long tail_blk = -1;
+	{	/* every XCD gets a rectangle of the tile grid, its last tiles in parts along K, as in conv_f32_direct_kernel */
+		const int bid = blockIdx.x, xcd = bid & 7;
+		int local = bid >> 3;
 		int m0, mw, n0, cnt;
 		conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
+		if (p.tail_slots) {
+			int full;
+			const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, p.tail_round, &full);
+			if (s > 1 && local >= full) {
+				const int t = (local - full) / s;
+				split = (local - full) - t * s;
+				nsplit = s;
+				local = full + t;
+				tail_blk = (long)xcd * p.tail_cap + t * s + split;
+			}
+		}
 		if (local >= cnt)
 			return;
 		tile_m = m0 + local % mw;
 		tile_n = n0 + local / mw;
 	}
-	/* tile_n counts patches: image, patch row, patch column */
-	const int TX = p.oW / TW, TXY = TX * (p.oH / TH);
-	const int b = tile_n / TXY, trem = tile_n - b * TXY, ty = trem / TX;
-	const int y0 = ty * TH, x0 = (trem - ty * TX) * TW;
+	/* this workgroup's half blocks [hb0, hb1): whole blocks of 32 planes */
+	const int blocks32 = p.Ci / 32;
+	const int hb0 = 2 * (int)((long)blocks32 * split / nsplit), hb1 = 2 * (int)((long)blocks32 * (split + 1) / nsplit);
 
-	/* ---- what this lane fetches of every plane: patch elements lane and 64 + lane ---- */
-	unsigned voff_[2];
+	/* ---- what this lane fetches of every plane: elements lane + 64 j of the tile's patches ---- */
+	unsigned voff_[NL];
 #pragma unroll
-	for (int j = 0; j < 2; j++) {
-		const int e = 64 * j + lane, r = e / PWD, c = e - r * PWD;
+	for (int j = 0; j < NL; j++) {
+		const int e = 64 * j + lane, q = e / GEO::PEL_S, le = e - q * GEO::PEL_S, r = le / PWD, c = le - r * PWD;
+		int b, y0, x0;
+		bool ok = conv_patch_origin<SW, SH>(p, tile_n * GEO::NP + q, b, y0, x0) && e < GEO::PEL;
 		const int iy = y0 - 1 + r, ix = x0 - 1 + c;
-		const bool ok = e < PEL && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+		ok = ok && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
 		voff_[j] = ok ? (unsigned)(((b * p.Ci * p.H + iy) * p.W + ix) * (int)sizeof(float)) : 0x80000000u;
 	}
 	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
 	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
 	const int plane_bytes = p.HW * (int)sizeof(float);
-	const int NB = p.Ci / BLK;	/* half blocks */
 	/* this wave's weight block of a K-tile: 32-row block wave % 2, chunk wave / 2 */
 	const unsigned a_base = (unsigned)(tile_m * MB + wave % MB) * (unsigned)p.KC * 1024u;
 	const int a_kci = wave / MB, a_lds = (a_kci * MB + wave % MB) * 64;
@@ -2488,23 +2537,24 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 		constexpr int st = decltype(st_)::value;
 		const unsigned kc = (unsigned)(((hb >> 1) * 9 + tap) * 4 + (hb & 1) * 2 + a_kci);
 		__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(lds_a + st * A_VECS + a_lds), 16,
-			hb < NB ? lane * 16 : 0x80000000u, a_base + kc * 1024u, 0, 0);
+			hb < hb1 ? lane * 16 : 0x80000000u, a_base + kc * 1024u, 0, 0);
 	};
-	/* load t (0..7) of this wave's share of half block hb's patches into buffer buf: plane wave + 4 (t / 2),
-	 * elements 64 (t % 2).. */
-	auto issue_b = [&](int t, int hb, auto buf_) {
-		constexpr int buf = decltype(buf_)::value;
-		const int plane = wave + 4 * (t >> 1), j = t & 1;
+	/* load t (0 .. BL-1) of this wave's share of half block hb's patches into buffer buf: plane
+	 * wave + 4 (t / NL), elements 64 (t % NL).. */
+	auto issue_b = [&](auto t_, int hb, auto buf_) {
+		constexpr int buf = decltype(buf_)::value, t = decltype(t_)::value;
+		const int plane = wave + 4 * (t / NL);
+		constexpr int j = t % NL;
 		float *dst = (buf ? lds_b1 : lds_b0) + plane * PSTRIDE + 64 * j;
-		/* the scalar offset is not range checked: the planes exist (hb < NB) */
+		/* the scalar offset is not range checked: the planes exist (hb < hb1) */
 		__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(dst), 4,
-			hb < NB ? voff_[j] : 0x80000000u, hb < NB ? (hb * BLK + plane) * plane_bytes : 0, 0, 0);
+			hb < hb1 ? voff_[j] : 0x80000000u, hb < hb1 ? (hb * BLK + plane) * plane_bytes : 0, 0, 0);
 	};
 
-	/* fragments: A rows lane % 32 of block wm, half lane / 32; B pixel n of the patch, planes
+	/* fragments: A rows lane % 32 of block wm, half lane / 32; B pixel n of the tile, planes
 	 * 8 chunk + 4 (lane / 32) + step of the half block, at the tap's offset */
-	const int n = wn * 32 + (lane & 31);
-	const int bfrag = (lane >> 5) * 4 * PSTRIDE + (n / TW) * PWD + n % TW;
+	const int n = wn * 32 + (lane & 31), ln = n % GEO::NPOS;
+	const int bfrag = (lane >> 5) * 4 * PSTRIDE + (n / GEO::NPOS) * GEO::PEL_S + (ln / SW) * PWD + ln % SW;
 	auto read_frags = [&](auto st_, auto buf_, auto tap_, int c, floatx4 &a, floatx4 &bq) {
 		constexpr int st = decltype(st_)::value, tap = decltype(tap_)::value, buf = decltype(buf_)::value;
 		a = lds_a[st * A_VECS + (c * MB + wm) * 64 + lane];
@@ -2523,20 +2573,32 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 	typedef std::integral_constant<int, 0> C0;
 	typedef std::integral_constant<int, 1> C1;
 	typedef std::integral_constant<int, 2> C2;
-#pragma unroll
-	for (int t = 0; t < 8; t++)
-		issue_b(t, 0, C0{});
-	issue_a(C0{}, 0, 0);
-	issue_a(C1{}, 0, 1);
-	issue_a(C2{}, 0, 2);
+	/* Patch loads of the next half block: BL of them over the nine steps of this one, step `tap` issues
+	 * numbers [PB(tap), PB(tap + 1)): one a step (BL = 8: none in the last) or two in each of the
+	 * first four steps and one after (BL = 12: none in the last). */
+#define CONV_PATCH_PB(tap) (BL == 8 ? ((tap) < 8 ? (tap) : 8) : ((tap) < 4 ? 2 * (tap) : (tap) < 8 ? 4 + (tap) : 12))
+	{
+		auto all_b = [&](auto self, auto t_) {
+			constexpr int t = decltype(t_)::value;
+			if constexpr (t < BL) {
+				issue_b(t_, hb0, C0{});
+				self(self, std::integral_constant<int, t + 1>{});
+			}
+		};
+		all_b(all_b, C0{});
+	}
+	issue_a(C0{}, hb0, 0);
+	issue_a(C1{}, hb0, 1);
+	issue_a(C2{}, hb0, 2);
 	wide_wait<2, false>();	/* the patches and the first K-tile's weights */
 	__builtin_amdgcn_s_barrier();
 	read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
 
-	/* K-tile (hb, tap): its weights in stage tap % 3, the next K-tile's in the next stage.  Loads are issued
-	 * patch first, weights second; the weights of the next K-tile were issued two steps ago, so at most the
-	 * last step's loads may still be on their way: its weights and, unless that step was a half block's
-	 * last, a patch load.  A half block's last step waits for the patch loads of the next as well. */
+	/* K-tile (hb, tap): its weights in stage tap % 3, the next K-tile's in the next stage.  A step issues its
+	 * patch loads first, its weights last; the weights of the next K-tile were issued two steps ago, so what
+	 * may still be on its way is the last step's loads.  A half block's last step waits for the patch loads
+	 * of the next as well (none are issued in that step, the last before it are older than that step's
+	 * weights). */
 	auto step = [&](int hb, auto buf_, auto tap_) {
 		constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
 		typedef std::integral_constant<int, tap % 3> ST;
@@ -2544,23 +2606,28 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 		typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
 		typedef std::integral_constant<int, buf ^ 1> OTHER;
 		typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
+		constexpr int prev = (tap + 8) % 9;	/* the step before */
+		constexpr int last_loads = 1 + CONV_PATCH_PB(prev + 1) - CONV_PATCH_PB(prev);
 		read_frags(ST{}, buf_, tap_, 1, af[1], bf[1]);
 		/* (the fragments are asked for before the MFMAs that follow in the source; left alone, the
 		 * compiler puts the reads right before their first use) */
 		__builtin_amdgcn_sched_barrier(0);
 		conv_mma<THHIP_F32>(acc, af[0], bf[0]);
-		wide_wait<(tap >= 1 && tap <= 7) ? 2 : 1, true>();
+		wide_wait<tap == 8 ? 1 : last_loads, true>();
 		__builtin_amdgcn_s_barrier();
 		read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[0], bf[0]);
 		__builtin_amdgcn_sched_barrier(0);
-		if constexpr (tap < 8)
-			issue_b(tap, hb + 1, OTHER{});
+		if constexpr (CONV_PATCH_PB(tap + 1) - CONV_PATCH_PB(tap) >= 1)
+			issue_b(std::integral_constant<int, CONV_PATCH_PB(tap)>{}, hb + 1, OTHER{});
+		if constexpr (CONV_PATCH_PB(tap + 1) - CONV_PATCH_PB(tap) >= 2)
+			issue_b(std::integral_constant<int, CONV_PATCH_PB(tap) + 1>{}, hb + 1, OTHER{});
 		if constexpr (tap + 3 < 9)
 			issue_a(ST{}, hb, tap + 3);
 		else
 			issue_a(ST{}, hb + 1, tap + 3 - 9);
 		conv_mma<THHIP_F32>(acc, af[1], bf[1]);
 	};
+#undef CONV_PATCH_PB
 	auto half_block = [&](int hb, auto buf_) {
 		step(hb, buf_, std::integral_constant<int, 0>{});
 		step(hb, buf_, std::integral_constant<int, 1>{});
@@ -2572,14 +2639,57 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 		step(hb, buf_, std::integral_constant<int, 7>{});
 		step(hb, buf_, std::integral_constant<int, 8>{});
 	};
-	for (int hb = 0; hb < NB; hb += 2) {	/* (Ci % 32 == 0: an even number of half blocks) */
+	for (int hb = hb0; hb < hb1; hb += 2) {	/* (whole blocks of 32 planes: an even number of half blocks) */
 		half_block(hb, C0{});
 		half_block(hb + 1, C1{});
 	}
-	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the epilogue reuses it) */
+	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the workgroup ends or the epilogue reuses it) */
+	if (tail_blk >= 0) {
+		/* a part of one of the XCD's last tiles: the accumulator as it lies in the registers,
+		 * [register][thread]; conv_f32_patch_tail_finish_kernel adds the parts in their order */
+		float *part = (float *)p.ws + tail_blk * (64 * 64);
+#pragma unroll
+		for (int r = 0; r < 16; r++)
+			part[r * 256 + tid] = acc[r];
+		return;
+	}
 	__syncthreads();
-	conv_f32_patch_store<TW>(p, acc, tile_m, b, y0, x0, (int *)lds_a);
+	conv_f32_patch_store<SW, SH>(p, acc, tile_m, tile_n, (int *)lds_a);
 #endif
+}
+
+/* Adds the K parts of the tiles conv_f32_patch_kernel cut (one workgroup per such tile,
+ * [xcd][tile][part][register][thread] in scratch) in their order and finishes them as that kernel's
+ * epilogue does. */
+template <int SW, int SH>
+__global__ __launch_bounds__(256) void conv_f32_patch_tail_finish_kernel(ConvParams p)
+{
+	__shared__ int lrow[128];
+	const int tid = threadIdx.x, xcd = blockIdx.x & 7, t = blockIdx.x >> 3;
+	int m0, mw, n0, cnt, full;
+	conv_xcd_rect(p, xcd, m0, mw, n0, cnt);
+	const int s = conv_tail_parts(cnt, p.tail_slots, p.tail_max, p.tail_round, &full);
+	if (s < 2 || t >= cnt - full)
+		return;
+	const int local = full + t;
+	const float *part = (const float *)p.ws + ((long)xcd * p.tail_cap + t * s) * (64 * 64);
+	floatx16 in[8];		/* all parts requested at once (at most eight: conv_tail_plan), added in their order */
+#pragma unroll
+	for (int q = 0; q < 8; q++)
+		if (q < s) {
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				in[q][r] = part[(long)q * (64 * 64) + r * 256 + tid];
+		}
+	floatx16 acc = in[0];
+#pragma unroll
+	for (int q = 1; q < 8; q++)
+		if (q < s) {
+#pragma unroll
+			for (int r = 0; r < 16; r++)
+				acc[r] += in[q][r];
+		}
+	conv_f32_patch_store<SW, SH>(p, acc, m0 + local % mw, n0 + local / mw, lrow);
 }
 
 /* Adds the K parts of the tiles conv_f32_direct_kernel cut (one workgroup per
@@ -3171,9 +3281,9 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 		conv_f32_tail_finish_kernel<BM, BN><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
-/* Whether conv_f32_patch_kernel can run this layer, and with which patch: plane-major fp32 on both
+/* Whether conv_f32_patch_kernel can run this layer, and with which patches: plane-major fp32 on both
  * sides, 3x3 / stride 1 / padding 1, whole blocks of 32 input and 64 output planes, an output of whole
- * 16 x 4 or 8 x 8 patches.  Returns the patch width (16, 8) or 0. */
+ * 16x4, 8x8 or 4x4 patches.  Returns the patch width (16, 8, 4) or 0. */
 static int conv_f32_patch_width(const ConvParams &p)
 {
 	if (p.x_cl || p.y_cl || p.kH != 3 || p.kW != 3 || p.dH != 1 || p.dW != 1 || p.padH != 1 || p.padW != 1)
@@ -3184,14 +3294,17 @@ static int conv_f32_patch_width(const ConvParams &p)
 		return 16;
 	if (p.oW % 8 == 0 && p.oH % 8 == 0)
 		return 8;
+	if (p.oW % 4 == 0 && p.oH % 4 == 0)
+		return 4;
 	return 0;
 }
 
-template <int TW, int TH>
+template <int SW, int SH>
 static void conv_launch_f32_patch(ConvParams &p)
 {
+	typedef ConvPatchGeo<SW, SH> GEO;
 	p.tiles_m = p.Co / 64;
-	p.tiles_n = p.B * (p.oH / TH) * (p.oW / TW);
+	p.tiles_n = (int)(((long)p.B * (p.oH / SH) * (p.oW / SW) + GEO::NP - 1) / GEO::NP);
 	p.splitk = 1;
 	if ((size_t)p.tiles_m * 2 * p.KC * 1024 > p.w_bytes || p.KC != p.Ci / 8 * 9)
 		THError("thhip_conv2d: packed weights do not fit the patch kernel's tile grid");
@@ -3201,8 +3314,18 @@ static void conv_launch_f32_patch(ConvParams &p)
 		p.mparts *= 2;
 	if (g_force_mparts)
 		p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
-	const size_t maxcnt = conv_tail_plan(p, 0, 0, 0, 0);	/* (no tiles are cut: the layers this kernel takes have thousands) */
-	conv_f32_patch_kernel<TW, TH><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
+	/* the tiles an XCD cannot spread evenly over its CUs are cut along K into parts of whole blocks of
+	 * 32 planes (conv_tail_parts; `8 blocks` K-tiles so that conv_tail_plan allows at most one part a block) */
+	static int resident;
+	if (!resident) {
+		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_patch_kernel<SW, SH>, 256, 0));
+		if (resident < 1)
+			resident = 1;
+	}
+	const size_t maxcnt = conv_tail_plan(p, resident, p.Ci / 32 * 8, 64 * 64, 0);
+	conv_f32_patch_kernel<SW, SH><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
+	if (p.tail_slots)
+		conv_f32_patch_tail_finish_kernel<SW, SH><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
 /* Whether conv_patch_kernel can run this layer. */
@@ -3261,6 +3384,11 @@ static bool conv_pool_uses_patch(const ConvParams &p)
 	return false;
 }
 
+/* conv_f32_patch_kernel takes layers of at least this many 64 x 64 tiles: with fewer (VGG-16's 28^2
+ * layers at batch 16: 1568; ResNet-18's 56^2 and 28^2 layers at batch 32) it measured the same as
+ * conv_f32_direct_kernel or a little slower (445 -> 452 us), five resident workgroups per CU spreading
+ * one and a half rounds of tiles worse than three */
+#define CONV_F32_PATCH_MIN 2000
 template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
@@ -3347,7 +3475,7 @@ static void conv_dispatch(ConvParams &p)
 				bn = 128;
 		} else if (p.x_cl == 1 && t128 >= 512)
 			bm = bn = 128;
-	} else if (DT == THHIP_F32 && conv_f32_patch_width(p) && t64 >= 2000 && !g_force_kch && !g_force_bm && !g_force_bn) {
+	} else if (DT == THHIP_F32 && conv_f32_patch_width(p) && t64 >= CONV_F32_PATCH_MIN && !g_force_kch && !g_force_bm && !g_force_bn) {
 		/* 3x3 layers of many whole patches: the taps from a patch in LDS (conv_f32_patch_kernel) */
 		bn = 1;
 	} else if (DT == THHIP_F32 && conv_f32_direct_ok(p) && !g_force_kch) {
@@ -3421,10 +3549,12 @@ static void conv_dispatch(ConvParams &p)
 			const int tw = conv_f32_patch_width(p);
 			if (!tw)
 				THError("thhip_conv2d: the fp32 patch kernel needs plane-major tensors, 3x3 / stride 1 / padding 1, "
-					"Ci %% 32 == 0, Co %% 64 == 0 and an output of whole 16x4 or 8x8 patches");
+					"Ci %% 32 == 0, Co %% 64 == 0 and an output of whole 16x4, 8x8 or 4x4 patches");
 			if (tw == 16)
 				return conv_launch_f32_patch<16, 4>(p);
-			return conv_launch_f32_patch<8, 8>(p);
+			if (tw == 8)
+				return conv_launch_f32_patch<8, 8>(p);
+			return conv_launch_f32_patch<4, 4>(p);
 		}
 	}
 	if (p.res_mode && (DT != THHIP_F32 || !direct || p.pool))
