@@ -395,7 +395,7 @@ def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
     patches (every tap read from one patch of the input in LDS): forced on small layers of all
     three patch shapes (a last tile of fewer than four 4x4 patches among them), two to six half
     blocks of input planes, 64 to 192 output planes, with and without the folded batch-norm factor
-    and Threshold; and as the dispatcher picks it (2000 tiles and more; the last tiles of an XCD
+    and Threshold; and as the dispatcher picks it (more than 512 tiles; the last tiles of an XCD
     cut along K), alone, with the 2x2 pooling and with a table add in its epilogue, each bit for
     bit the separate kernel on the plain result.  Against the restatement."""
     from thnets_amd import api

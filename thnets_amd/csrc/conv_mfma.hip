@@ -3316,14 +3316,56 @@ static void conv_launch_f32_patch(ConvParams &p)
 		p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
 	/* the tiles an XCD cannot spread evenly over its CUs are cut along K into parts of whole blocks of
 	 * 32 planes (conv_tail_parts; `8 blocks` K-tiles so that conv_tail_plan allows at most one part a block) */
-	static int resident;
+	static int resident, static_lds, cus;
 	if (!resident) {
 		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_patch_kernel<SW, SH>, 256, 0));
 		if (resident < 1)
 			resident = 1;
+		hipFuncAttributes attr;
+		hipcheck(hipFuncGetAttributes(&attr, (const void *)conv_f32_patch_kernel<SW, SH>));
+		static_lds = (int)attr.sharedSizeBytes;
+		int dev;
+		hipcheck(hipGetDevice(&dev));
+		hipcheck(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
 	}
-	const size_t maxcnt = conv_tail_plan(p, resident, p.Ci / 32 * 8, 64 * 64, 0);
-	conv_f32_patch_kernel<SW, SH><<<dim3((unsigned)(8 * maxcnt)), dim3(256), 0, thhip_stream()>>>(p);
+	/* How many workgroups a CU should hold: with few rounds of tiles, the number that leaves the smallest
+	 * part of a round empty after the cut (VGG-16's 28^2 layers at batch 16, 196 tiles an XCD: four a CU
+	 * leave a second round half empty with nothing to cut, three make two rounds and four tiles cut in
+	 * eight).  Rounds an XCD needs: whole rounds, plus 1 / parts for the cut tiles or 1 if they cannot be cut. */
+	int use = resident;
+	{
+		const int smax = p.Ci / 32 < g_tail_parts ? p.Ci / 32 : g_tail_parts;
+		double best = 0;
+		for (int r = resident; r >= 3 && r >= resident - 2; r--) {
+			double worst = 1.0;
+			for (int x = 0; x < 8; x++) {
+				const int mp = x % p.mparts, np = x / p.mparts, nparts = 8 / p.mparts;
+				const int cnt = (p.tiles_m * (mp + 1) / p.mparts - p.tiles_m * mp / p.mparts) *
+					(p.tiles_n * (np + 1) / nparts - p.tiles_n * np / nparts);
+				if (!cnt)
+					continue;
+				int full;
+				const int slots = cus / 8 * r;
+				const int sx = g_tail_parts != 1 ? conv_tail_parts(cnt, slots, smax > 8 ? 8 : smax, 0, &full) : (full = cnt, 1);
+				const double rounds = sx > 1 ? (double)full / slots + 1.0 / sx : (double)((cnt + slots - 1) / slots);
+				const double eff = (double)cnt / slots / rounds;
+				if (eff < worst)
+					worst = eff;
+			}
+			if (worst > best + 0.02) {	/* (fewer residents only for a clear gain) */
+				best = worst;
+				use = r;
+			}
+		}
+	}
+	int dyn = 0;
+	if (use < resident) {	/* LDS nobody uses, so that no more than `use` workgroups fit a CU */
+		dyn = CONV_LDS_PER_CU / (use + 1) + 512 - static_lds;
+		if (dyn < 0)
+			dyn = 0;
+	}
+	const size_t maxcnt = conv_tail_plan(p, use, p.Ci / 32 * 8, 64 * 64, 0);
+	conv_f32_patch_kernel<SW, SH><<<dim3((unsigned)(8 * maxcnt)), dim3(256), dyn, thhip_stream()>>>(p);
 	if (p.tail_slots)
 		conv_f32_patch_tail_finish_kernel<SW, SH><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
@@ -3384,11 +3426,9 @@ static bool conv_pool_uses_patch(const ConvParams &p)
 	return false;
 }
 
-/* conv_f32_patch_kernel takes layers of at least this many 64 x 64 tiles: with fewer (VGG-16's 28^2
- * layers at batch 16: 1568; ResNet-18's 56^2 and 28^2 layers at batch 32) it measured the same as
- * conv_f32_direct_kernel or a little slower (445 -> 452 us), five resident workgroups per CU spreading
- * one and a half rounds of tiles worse than three */
-#define CONV_F32_PATCH_MIN 2000
+/* conv_f32_patch_kernel takes layers of at least this many 64 x 64 tiles (below, conv_dispatch splits K
+ * of the whole layer) */
+#define CONV_F32_PATCH_MIN 513
 template <int DT>
 static void conv_dispatch(ConvParams &p)
 {
