@@ -176,10 +176,11 @@ def main():
     roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_TFLOPS_FP32_MFMA, "unit": "TFLOP/s",
                 "frac": round(achieved / PEAK_TFLOPS_FP32_MFMA, 4),
                 "traffic": counter_traffic("conv_f32_vgg16_fp32_b16_counters.md", "conv_hbm_bytes_per_launch"),
-                "kernel": "conv_f32_direct_kernel (implicit-GEMM convolution, operands loaded straight into LDS; 12 of the 13 "
-                          "convolutions of a step, four of them with the 2x2 max pooling that follows in their epilogue, with the "
-                          "kernels that sum the K parts of the three 14x14 layers and of the last tiles of eight others; the image "
-                          "layer on conv_stem_kernel<fp32>)",
+                "kernel": "conv_f32_patch_kernel (implicit-GEMM convolution, every tap of a 3x3 layer read from one input patch "
+                          "per plane in LDS: nine of the 13 convolutions of a step, four of them with the 2x2 max pooling that "
+                          "follows in their epilogue, six with the kernel that sums the K parts of their last tiles) and "
+                          "conv_f32_direct_kernel (operands loaded straight into LDS: the three 14x14 layers, K split in three, with "
+                          "the kernel that sums the parts); the image layer on conv_stem_kernel<fp32>",
                 "launches_per_step": conv_n / args.steps, "avg_launch_ms": round(conv_ms / max(conv_n, 1), 5),
                 "flops_per_launch": conv_flops / max(conv_n, 1)}
     extra = {"vgg16_conv_ms_per_step": round(conv_ms / args.steps, 4),
