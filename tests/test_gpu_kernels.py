@@ -390,6 +390,37 @@ def test_conv_f32_with_table_add_in_the_epilogue(hiplib, oracle):
     assert not hiplib.thhip_conv2d_residual_supported(2, 64, 32, 32, 64, 3, 3, 1, 1, 1, 1, G.F16)
 
 
+def test_conv_f32_rows_with_their_own_taps(hiplib, oracle):
+    """fp32 plane-major layers whose planes are not whole blocks of 32 on the kernel that loads
+    straight into LDS with a (plane, tap) of its own per K row: many tiles at stride 1 (7x7 on
+    three planes, 5x5 on twenty), few tiles with strides and a K split (11x11 / stride 4 on
+    three planes, 3x3 / stride 2 on 48), K values past the last plane in the last K-tile.
+    Against the restatement and against the register-staged kernel (a forced tile)."""
+    g = cases.rng(5500)
+    shapes = [(40, 3, 64, 64, 64, 7, 1, 3), (8, 20, 40, 40, 64, 5, 1, 2), (2, 3, 227, 227, 64, 11, 4, 2), (2, 48, 30, 30, 96, 3, 2, 1),
+              (3, 33, 17, 19, 70, 1, 1, 0), (1, 5, 9, 9, 64, 3, 1, 1)]
+    for (B, Ci, H, W, Co, k, d, pad) in shapes:
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        raw = oracle.conv2d(x, w, None, (d, d), (pad, pad))
+        for (scale, act) in ((None, 0), (sc, 1)):
+            want = raw * (scale[None, :, None, None] if scale is not None else 1) + b[None, :, None, None]
+            if act:
+                want = np.where(want > 0.05, want, np.float32(0.05))      # (continuous: a sum next to the threshold moves the result little)
+            kw = dict(act=act, thr=0.05, val=0.05, dtype=G.F32, scale=scale)
+            G.note("fp32 rows kernel %s act %d" % ((B, Ci, H, W, Co, k, d, pad), act))
+            got = G.conv2d_layout(hiplib, x, w, b, (d, d), (pad, pad), **kw)
+            G.assert_close(got, want, FP32_TOL, "fp32 rows kernel " + str((B, Ci, H, W, Co, k, d, pad, act)))
+            try:
+                hiplib.thhip_conv_set_tuning(64, 64, 1, 0)
+                staged = G.conv2d_layout(hiplib, x, w, b, (d, d), (pad, pad), **kw)
+            finally:
+                hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+            G.assert_close(got, staged, FP32_TOL, "fp32 rows kernel against the register-staged one " + str((B, Ci, H, W, Co, k, d, pad)))
+
+
 def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
     """The fp32 kernel for 3x3 / stride 1 / padding 1 layers whose output is whole 16x4, 8x8 or 4x4
     patches (every tap read from one patch of the input in LDS): forced on small layers of all
@@ -411,11 +442,11 @@ def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
         for (scale, act) in ((None, 0), (sc, 1)):
             want = raw * (scale[None, :, None, None] if scale is not None else 1) + b[None, :, None, None]
             if act:
-                want = np.where(want > 0.05, want, np.float32(-0.5))
+                want = np.where(want > 0.05, want, np.float32(0.05))      # (continuous: a sum next to the threshold moves the result little)
             G.note("fp32 patch kernel, forced, %s act %d" % ((B, Ci, H, W, Co), act))
             try:
                 hiplib.thhip_conv_set_tuning(64, 1, 0, 0)
-                got = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), act=act, thr=0.05, val=-0.5, dtype=G.F32, scale=scale)
+                got = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), act=act, thr=0.05, val=0.05, dtype=G.F32, scale=scale)
             finally:
                 hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
             G.assert_close(got, want, FP32_TOL, "fp32 patch kernel " + str((B, Ci, H, W, Co, act)))

@@ -2057,7 +2057,7 @@ __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, float
  * (n, k): step s of a chunk reads rows 8 c + s (lanes 0..31) and 8 c + 4 + s
  * (lanes 32..63); rows are BN + 8 floats apart, so the two halves use different
  * banks.  Needs Ci % 32 == 0. */
-template <int BM, int BN, int KCH, int NST>
+template <int BM, int BN, int KCH, int NST, bool ROWS = false>
 __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
@@ -2161,6 +2161,26 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		t_kw = tap - t_kh * p.kW;
 	}
 	const int plane_bytes = p.HW * (int)sizeof(float);
+	/* ROWS (any number of planes, K order (plane, tap)): every row of a K-tile is a (plane, tap) of its own.
+	 * This wave's rows wave + 4 r of the K-tile: plane, kernel row and column, walked on the scalar unit
+	 * KT values at a time (KT = d_c kH kW + d_kh kW + d_kw). */
+	constexpr int RPW = KT / WAVES;
+	int r_c[RPW], r_kh[RPW], r_kw[RPW];
+	int d_c = 0, d_kh = 0, d_kw = 0;
+	if constexpr (ROWS) {
+#pragma unroll
+		for (int r = 0; r < RPW; r++) {
+			const int k = kt0 * KT + wave + WAVES * r;
+			r_c[r] = k / p.kHW;
+			const int tap = k - r_c[r] * p.kHW;
+			r_kh[r] = tap / p.kW;
+			r_kw[r] = tap - r_kh[r] * p.kW;
+		}
+		d_c = KT / p.kHW;
+		const int tap = KT - d_c * p.kHW;
+		d_kh = tap / p.kW;
+		d_kw = tap - d_kh * p.kW;
+	}
 
 	auto issue = [&](auto st_) {
 		constexpr int st = decltype(st_)::value;
@@ -2170,6 +2190,30 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 		for (int i = 0; i < A_PW; i++)
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(la + a_lds_[i]), 16, lane * 16,
 				a_off_[i] + (unsigned)t_kc * 1024u, 0, 0);
+		if constexpr (ROWS) {
+#pragma unroll
+			for (int r = 0; r < RPW; r++) {
+				const int k = wave + WAVES * r;	/* row of the K-tile */
+				const int tap_off = r_kh[r] * p.W + r_kw[r];
+				const bool row_ok = r_c[r] < p.Ci;	/* (rows past K: zero weights, no plane) */
+#pragma unroll
+				for (int q = 0; q < NPOS; q++) {
+					const int iy = iy0_[q] + r_kh[r], ix = ix0_[q] + r_kw[r];
+					const bool ok = (int)n_ok_[q] & (int)row_ok & (int)((unsigned)iy < (unsigned)p.H) & (int)((unsigned)ix < (unsigned)p.W);
+					const unsigned voff = ok ? (unsigned)(xoff_[q] + tap_off) * (unsigned)sizeof(float) : 0x80000000u;
+					__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(lb + k * BROW + q * 64), 4, voff,
+						row_ok ? r_c[r] * plane_bytes : 0, 0, 0);
+				}
+				/* KT values on: column, row and plane with their carries */
+				const int kw1 = r_kw[r] + d_kw, cw = kw1 >= p.kW;
+				r_kw[r] = __builtin_amdgcn_readfirstlane(cw ? kw1 - p.kW : kw1);
+				const int kh1 = r_kh[r] + d_kh + cw, ch = kh1 >= p.kH;
+				r_kh[r] = __builtin_amdgcn_readfirstlane(ch ? kh1 - p.kH : kh1);
+				r_c[r] = __builtin_amdgcn_readfirstlane(r_c[r] + d_c + ch);
+			}
+			t_kc += KCH;
+			return;
+		}
 		const int tap_off = t_kh * p.W + t_kw;
 		const int plane0 = (t_cb * SUB + t_sub) * KT;
 #pragma unroll
@@ -3241,7 +3285,14 @@ static bool conv_f32_direct_ok(const ConvParams &p)
 	return !p.x_cl && !p.y_cl && p.Ci % 32 == 0 && p.x_bytes < 0x7fffffffu;
 }
 
-template <int BM, int BN, int KCH, int NST>
+/* The same kernel with a (plane, tap) of its own for every row of a K-tile: plane-major fp32 layers of any
+ * other number of planes (K order (plane, tap)). */
+static bool conv_f32_rows_ok(const ConvParams &p)
+{
+	return !p.x_cl && !p.y_cl && p.Ci % 32 != 0 && p.x_bytes < 0x7fffffffu && p.kHW <= 4096;
+}
+
+template <int BM, int BN, int KCH, int NST, bool ROWS = false>
 static void conv_launch_f32_direct(ConvParams &p, int splitk)
 {
 	p.tiles_m = (p.Co + BM - 1) / BM;
@@ -3264,12 +3315,12 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 	 * over its CUs are cut along K (conv_tail_parts). */
 	static int resident;
 	if (!resident) {
-		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_direct_kernel<BM, BN, KCH, NST>, 256, 0));
+		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_direct_kernel<BM, BN, KCH, NST, ROWS>, 256, 0));
 		if (resident < 1)
 			resident = 1;
 	}
 	const size_t maxcnt = conv_tail_plan(p, resident, nkt, (size_t)BM * BN, 0);
-	conv_f32_direct_kernel<BM, BN, KCH, NST><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
+	conv_f32_direct_kernel<BM, BN, KCH, NST, ROWS><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
 	if (p.splitk > 1) {
 		long blocks = ((long)p.Co * p.N + 255) / 256;
 		if (blocks > 4096)
@@ -3462,6 +3513,7 @@ static void conv_dispatch(ConvParams &p)
 	const long t64 = (long)((p.Co + 63) / 64) * ((p.N + 63) / 64);
 	int bm = 64, bn = 64, splitk = 1, wgs = 0, kch = conv_kch(DT, p.x_cl != 0);
 	bool direct = false;	/* half types: operands loaded straight into LDS (conv_wide_kernel) */
+	bool rows = false;	/* fp32: conv_f32_direct_kernel with a (plane, tap) per K row */
 	if (DT == THHIP_F16 || DT == THHIP_BF16) {
 		/* tiles of 256 positions (operands straight to LDS) where whole tiles of
 		 * 256 planes fill most CUs for a turn: one such tile per CU multiplies
@@ -3546,6 +3598,24 @@ static void conv_dispatch(ConvParams &p)
 			if (parts > 1)
 				splitk = parts;
 		}
+	} else if (DT == THHIP_F32 && conv_f32_rows_ok(p) && (p.dW == 1 || t64 <= 512) && !g_force_kch && !g_force_bm && !g_force_bn) {
+		/* any other number of planes (image layers with larger kernels): the same kernel with a tap of
+		 * its own per K row, K-tiles of 16.  Not for strided layers of many tiles: a wave-wide load
+		 * then spans twice the cache lines, and ResNet-18's 7x7 / stride 2 image layer at batch 32 took
+		 * 117 us against the register-staged kernel's 108 (AlexNet's 11x11 / stride 4 one at batch 1,
+		 * a few tiles with a K split: 17 -> 11 us). */
+		direct = rows = true;
+		kch = 2;
+		if (t64 <= 512) {
+			const int nkt = p.KC / kch;
+			int parts = (int)((1024 + t64 - 1) / t64);
+			if (parts > nkt / 8)
+				parts = nkt / 8;
+			if (parts > 16)
+				parts = 16;
+			if (parts > 1)
+				splitk = parts;
+		}
 	} else if (DT == THHIP_F32 && t128 >= 300) {
 		kch = 2;
 		if (p.Co > 64 && t128 >= 700)
@@ -3607,6 +3677,8 @@ static void conv_dispatch(ConvParams &p)
 		return conv_launch_patch<DT, 64>(p);
 	}
 	if constexpr (DT == THHIP_F32) {
+		if (direct && rows)
+			return conv_launch_f32_direct<64, 64, 2, 3, true>(p, splitk);
 		if (direct) {
 			if (!conv_f32_direct_ok(p))
 				THError("thhip_conv2d: fp32 tiles loaded straight into LDS need plane-major tensors and Ci %% 32 == 0");
