@@ -450,6 +450,23 @@ def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
             finally:
                 hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
             G.assert_close(got, want, FP32_TOL, "fp32 patch kernel " + str((B, Ci, H, W, Co, act)))
+    # seeded random shapes (all three patch shapes, last tiles of one to three 4x4 patches): against the kernel
+    # that fetches every tap with a load of its own (another order of the sums)
+    for it in range(16):
+        B, Ci, Co = int(g.integers(1, 6)), int(g.choice([32, 64, 96, 160])), int(g.choice([64, 128, 192]))
+        H, W = 4 * int(g.integers(1, 13)), 4 * int(g.integers(1, 13))
+        x = g.standard_normal((B, Ci, H, W), dtype=np.float32)
+        w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(0.05)
+        b = g.standard_normal(Co, dtype=np.float32)
+        outs = []
+        for tune in ((64, 1, 0, 0), (64, 64, 9, 2)):
+            G.note("fp32 patch kernel, random shape %s tile %s" % ((B, Ci, H, W, Co), tune))
+            try:
+                hiplib.thhip_conv_set_tuning(*tune)
+                outs.append(G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), act=1, thr=0.0, val=0.0, dtype=G.F32))
+            finally:
+                hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+        G.assert_close(outs[0], outs[1], FP32_TOL, "fp32 patch kernel against the other " + str((B, Ci, H, W, Co)))
     # as dispatched: 2048 tiles of 64 planes x 64 pixels
     for (B, Ci, H, W, Co) in ((32, 32, 64, 64, 64), (24, 64, 56, 56, 128), (44, 64, 28, 28, 256), (140, 32, 24, 40, 64)):
         x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
