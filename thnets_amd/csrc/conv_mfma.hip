@@ -1680,18 +1680,22 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_tail_finish_kernel(C
  * position from L2 for 32 multiply-adds per output plane, nine times per
  * pixel (once per tap), and the path from L2 to LDS, not the matrix core, sets
  * their time.  Here a workgroup owns 8 rows x 32 columns of one image's output,
- * copies the 10 x 34 pixel patch those positions read once (43.5 KiB, straight
- * to LDS), and takes the B fragments of all nine taps from it: a fragment of
- * tap (kh, kw) is the patch shifted by (kh, kw).  Only the weights stream
- * (K-tiles of one tap x 32 planes, four stages, as in conv_wide_kernel).
- * 128 planes run as two blocks of 64: patch, nine taps, next patch, nine taps.
+ * copies the 10 x 34 pixel patch those positions read once per block of 32
+ * planes (21 KiB, straight to LDS), and takes the B fragments of all nine taps
+ * from it: a fragment of tap (kh, kw) is the patch shifted by (kh, kw).  The
+ * pipeline is conv_f32_patch_kernel's: two patch buffers, the next block's six
+ * loads per wavefront spread over the nine taps of this one, the weights
+ * (K-tiles of one tap x 32 planes) through a ring of three stages, the nine
+ * steps of a block straight-line code with constant wait counts.  (An earlier
+ * form held one patch of 64 planes, 43.5 KiB, and drained the pipeline between
+ * blocks: VGG-16 fp16 batch 16 0.735 -> 0.713 ms, batch 64 2.33 -> 2.26 ms.)
  *
- * Patch layout: 1 KiB blocks of eight pixels x eight 16-byte vectors, pixel pp
- * of the patch (row-major, 34 wide) in block pp / 8; inside a block vector v of
- * pixel pp sits in slot 8 (pp % 8) + (v ^ ((pp / 2) % 8)).  A fragment read
- * takes one vector index from 32 consecutive pixels; the swizzle spreads every
- * run of sixteen over all banks wherever it starts.  Pixels outside the image
- * are fetched out of the buffer's range and arrive as zeros.
+ * Patch layout: 1 KiB blocks of sixteen pixels x four 16-byte vectors, pixel pp
+ * of the patch (row-major, 34 wide) in block pp / 16; vector v of pixel pp sits
+ * in slot 4 pp + (v ^ ((pp / 2) % 4)).  A fragment read takes one vector index
+ * from 32 consecutive pixels; the swizzle spreads every run of eight over all
+ * banks wherever it starts.  Pixels outside the image are fetched out of the
+ * buffer's range and arrive as zeros.
  *
  * Four waves; wave w computes all BM planes of tile rows 2w and 2w+1. */
 #define PATCH_TW 32
@@ -1704,14 +1708,17 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	typedef ConvTraits<DT> TR;
 	typedef typename TR::elem elem;
 	static_assert(TR::CHUNK == 16 && sizeof(elem) == 2, "a half type");
-	constexpr int TW = PATCH_TW, TH = PATCH_TH, PW = TW + 2, PH = TH + 2, PCI = 64, NCB = CI / PCI;
-	constexpr int NPIX = PW * PH, PBLOCKS = (NPIX + 7) / 8, P_PW = (PBLOCKS + 3) / 4;
-	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = 4, WAVES = 4;
+	constexpr int TW = PATCH_TW, TH = PATCH_TH, PW = TW + 2, PH = TH + 2, PCI = 32, NB = CI / PCI;
+	constexpr int NPIX = PW * PH, WAVES = 4;
+	constexpr int BL = ((NPIX + 15) / 16 + WAVES - 1) / WAVES;	/* patch loads (sixteen pixels x four vectors) per wave and block */
+	constexpr int B_VECS = BL * WAVES * 64;				/* a buffer: every load's 1 KiB, the unused ones' too */
+	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = 3;
 	constexpr int A_VECS = MB * KCH * 64, A_PW = MB * KCH / WAVES;
-	constexpr int NKT = 9 * PCI / 32;	/* K-tiles per block of 64 planes: tap kt / 2, planes 32 (kt % 2) .. + 32 */
-	static_assert(CI % PCI == 0 && MB * KCH % WAVES == 0 && TH == 2 * WAVES, "shape");
-	__shared__ floatx4 patch[PBLOCKS * 64];
-	__shared__ floatx4 astage[NST * A_VECS];
+	static_assert(CI % (2 * PCI) == 0 && A_PW == 1 && TH == 2 * WAVES && BL <= 8, "shape");
+	/* (one array, every stage and buffer at a constant offset: conv_f32_patch_kernel says why) */
+	__shared__ floatx4 lds[NST * A_VECS + 2 * B_VECS];
+	floatx4 *const astage = lds;
+	floatx4 *const patch0 = lds + NST * A_VECS, *const patch1 = patch0 + B_VECS;
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -1736,43 +1743,34 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 
 	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
 	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
-	/* ---- the patch of plane block cb: block wave + 4 i, this lane pixel lane / 8, slot lane % 8 ---- */
-	auto load_patch = [&](int cb) {
+	/* ---- what this lane fetches of every block of 32 planes: load t of the wave covers pixels
+	 * 16 (wave + 4 t) .. + 15 of the patch, this lane pixel lane / 4 of them, vector lane % 4
+	 * through the swizzle ---- */
+	unsigned voff_[BL];
 #pragma unroll
-		for (int i = 0; i < P_PW; i++) {
-			const int blk = wave + WAVES * i;
-			if (blk < PBLOCKS) {
-				const int pp = blk * 8 + (lane >> 3);
-				const int v = (lane & 7) ^ ((pp >> 1) & 7);
-				const int pr = pp / PW, pc = pp - pr * PW;
-				const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
-				const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-				const unsigned voff = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + cb * PCI + v * 8) * (int)sizeof(elem))
-					: 0x80000000u;
-				__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS(patch + blk * 64), 16, voff, 0, 0, 0);
-			}
-		}
-	};
-	/* ---- the weights: block wave + 4 i counts (chunk, 32-row block) of a K-tile ---- */
-	unsigned a_off_[A_PW];
-	int a_lds_[A_PW];
-#pragma unroll
-	for (int i = 0; i < A_PW; i++) {
-		const int idx = wave + WAVES * i, mbi = idx % MB, kci = idx / MB;
-		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
-		a_lds_[i] = (kci * MB + mbi) * 64;
+	for (int t = 0; t < BL; t++) {
+		const int pp = (wave + WAVES * t) * 16 + (lane >> 2);
+		const int v = (lane & 3) ^ ((pp >> 1) & 3);
+		const int pr = pp / PW, pc = pp - pr * PW;
+		const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
+		const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+		voff_[t] = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + v * 8) * (int)sizeof(elem)) : 0x80000000u;
 	}
-	/* K-tile ikt of the patch's 64 planes: tap ikt / 2 of its 32-plane block ikt % 2; K runs
-	 * (block of 32 planes, tap, plane), in chunks of 16 */
-	int ikt = 0, t_cb = 0;
-	auto issue = [&](auto st_) {
+	/* this wave's weight block of a K-tile: 32-row block wave % MB, chunk wave / MB */
+	const unsigned a_base = (unsigned)(tile_m * MB + wave % MB) * (unsigned)p.KC * 1024u;
+	const int a_kci = wave / MB, a_lds = (a_kci * MB + wave % MB) * 64;
+
+	/* the weights of K-tile (block hb of 32 planes, tap): K runs (block, tap, plane) in chunks of 16 */
+	auto issue_a = [&](auto st_, int hb, int tap) {
 		constexpr int st = decltype(st_)::value;
-		const int kc = ((t_cb * (PCI / 32) + (ikt & 1)) * 9 + (ikt >> 1)) * KCH;
-#pragma unroll
-		for (int i = 0; i < A_PW; i++)
-			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16, lane * 16,
-				a_off_[i] + (unsigned)kc * 1024u, 0, 0);
-		++ikt;
+		const unsigned kc = (unsigned)((hb * 9 + tap) * KCH + a_kci);
+		__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds), 16,
+			hb < NB ? lane * 16 : 0x80000000u, a_base + kc * 1024u, 0, 0);
+	};
+	auto issue_b = [&](auto t_, int hb, auto buf_) {
+		constexpr int buf = decltype(buf_)::value, t = decltype(t_)::value;
+		__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS((buf ? patch1 : patch0) + (wave + WAVES * t) * 64), 16,
+			hb < NB ? voff_[t] : 0x80000000u, hb < NB ? hb * PCI * (int)sizeof(elem) : 0, 0, 0);
 	};
 
 	/* patch pixel of this lane's position at tap (0, 0), for its two tile rows */
@@ -1781,19 +1779,17 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	for (int j = 0; j < TN; j++)
 		pbase_[j] = (2 * wave + j) * PW + (lane & 31);
 	floatx4 af[2][TM], bf[2][TN];
-	auto read_frags = [&](auto st_, int kci, int kt, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
-		constexpr int st = decltype(st_)::value;
+	auto read_frags = [&](auto st_, auto buf_, auto tap_, int c, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
+		constexpr int st = decltype(st_)::value, buf = decltype(buf_)::value, tap = decltype(tap_)::value;
 		const floatx4 *la = astage + st * A_VECS;
 #pragma unroll
 		for (int i = 0; i < TM; i++)
-			a[i] = la[(kci * MB + i) * 64 + lane];
-		const int tap = kt >> 1, kh = (tap * 11) >> 5, kw = tap - 3 * kh;	/* tap / 3 for tap < 9 */
-		const int toff = kh * PW + kw;
-		const int v = (kt & 1) * 4 + kci * 2 + (lane >> 5);
+			a[i] = la[(c * MB + i) * 64 + lane];
+		const int v = c * 2 + (lane >> 5);
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
-			const int pp = pbase_[j] + toff;
-			b[j] = patch[pp * 8 + (v ^ ((pp >> 1) & 7))];
+			const int pp = pbase_[j] + (tap / 3) * PW + tap % 3;
+			b[j] = (buf ? patch1 : patch0)[pp * 4 + (v ^ ((pp >> 1) & 3))];
 		}
 	};
 
@@ -1813,54 +1809,74 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 				conv_mma<DT>(acc[i][j], af[set][i], bf[set][j]);
 	};
 
-	typedef std::integral_constant<int, 0> S0;
-	typedef std::integral_constant<int, 1> S1;
-	typedef std::integral_constant<int, 2> S2;
-	typedef std::integral_constant<int, 3> S3;
-	auto step = [&](int kt, auto st, auto st1, auto steady_) {
-		constexpr bool steady = decltype(steady_)::value;
-		read_frags(st, 1, kt, af[1], bf[1]);
+	typedef std::integral_constant<int, 0> C0;
+	typedef std::integral_constant<int, 1> C1;
+	typedef std::integral_constant<int, 2> C2;
+	/* patch loads of the next block: BL of them over the nine steps of this one, step `tap` issues
+	 * numbers [PB(tap), PB(tap + 1)), none in the last */
+#define CONV_PATCH_PB(tap) ((BL * ((tap) < 8 ? (tap) : 8) + 7) / 8)
+	{
+		auto all_b = [&](auto self, auto t_) {
+			constexpr int t = decltype(t_)::value;
+			if constexpr (t < BL) {
+				issue_b(t_, 0, C0{});
+				self(self, std::integral_constant<int, t + 1>{});
+			}
+		};
+		all_b(all_b, C0{});
+	}
+	issue_a(C0{}, 0, 0);
+	issue_a(C1{}, 0, 1);
+	issue_a(C2{}, 0, 2);
+	wide_wait<2, false>();	/* the patch and the first K-tile's weights */
+	__builtin_amdgcn_s_barrier();
+	read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
+	/* The pipeline of conv_f32_patch_kernel: K-tile (hb, tap) has its weights in stage tap % 3; a step issues
+	 * its patch loads first and its weights last, so at most the last step's loads may be outstanding when
+	 * the next K-tile's weights are waited for, and a block's last step waits for the next patch as well. */
+	auto step = [&](int hb, auto buf_, auto tap_) {
+		constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
+		typedef std::integral_constant<int, tap % 3> ST;
+		typedef std::integral_constant<int, (tap + 1) % 3> ST1;
+		typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
+		typedef std::integral_constant<int, buf ^ 1> OTHER;
+		typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
+		constexpr int prev = (tap + 8) % 9;
+		constexpr int last_loads = 1 + CONV_PATCH_PB(prev + 1) - CONV_PATCH_PB(prev);
+		read_frags(ST{}, buf_, tap_, 1, af[1], bf[1]);
+		__builtin_amdgcn_sched_barrier(0);	/* (the fragments are asked for before the MFMAs that follow in the source) */
 		mma(0);
-		if (steady)
-			wide_wait<2 * A_PW, true>();
-		else
-			wide_wait<0, true>();
+		wide_wait<tap == 8 ? 1 : last_loads, true>();
 		__builtin_amdgcn_s_barrier();
-		if (steady || kt + NST < NKT)
-			issue(st);
-		if (steady || kt + 1 < NKT)
-			read_frags(st1, 0, kt + 1, af[0], bf[0]);
+		read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[0], bf[0]);
+		__builtin_amdgcn_sched_barrier(0);
+		if constexpr (CONV_PATCH_PB(tap + 1) - CONV_PATCH_PB(tap) >= 1)
+			issue_b(std::integral_constant<int, CONV_PATCH_PB(tap)>{}, hb + 1, OTHER{});
+		if constexpr (CONV_PATCH_PB(tap + 1) - CONV_PATCH_PB(tap) >= 2)
+			issue_b(std::integral_constant<int, CONV_PATCH_PB(tap) + 1>{}, hb + 1, OTHER{});
+		if constexpr (tap + 3 < 9)
+			issue_a(ST{}, hb, tap + 3);
+		else
+			issue_a(ST{}, hb + 1, tap + 3 - 9);
 		mma(1);
 	};
-	static_assert(NKT == 18 && NST == 4, "the schedule below");
-	/* One block of 64 planes at a time: its patch, then its 18 K-tiles.  After the
-	 * last barrier of a block no wave reads LDS any more, so the next block's
-	 * loads may start at once. */
-	for (int cb = 0; cb < NCB; cb++) {
-		t_cb = cb;
-		ikt = 0;
-		load_patch(cb);
-		issue(S0{});
-		issue(S1{});
-		issue(S2{});
-		issue(S3{});
-		wide_wait<3 * A_PW, false>();	/* the patch and the first K-tile */
-		__builtin_amdgcn_s_barrier();
-		read_frags(S0{}, 0, 0, af[0], bf[0]);
-		int kt = 0;
-		for (; kt + 7 < NKT; kt += 4) {		/* kt = 0, 4, 8 */
-			step(kt, S0{}, S1{}, std::true_type{});
-			step(kt + 1, S1{}, S2{}, std::true_type{});
-			step(kt + 2, S2{}, S3{}, std::true_type{});
-			step(kt + 3, S3{}, S0{}, std::true_type{});
-		}
-		step(12, S0{}, S1{}, std::false_type{});
-		step(13, S1{}, S2{}, std::false_type{});
-		step(14, S2{}, S3{}, std::false_type{});
-		step(15, S3{}, S0{}, std::false_type{});
-		step(16, S0{}, S1{}, std::false_type{});
-		step(17, S1{}, S2{}, std::false_type{});
+#undef CONV_PATCH_PB
+	auto block = [&](int hb, auto buf_) {
+		step(hb, buf_, std::integral_constant<int, 0>{});
+		step(hb, buf_, std::integral_constant<int, 1>{});
+		step(hb, buf_, std::integral_constant<int, 2>{});
+		step(hb, buf_, std::integral_constant<int, 3>{});
+		step(hb, buf_, std::integral_constant<int, 4>{});
+		step(hb, buf_, std::integral_constant<int, 5>{});
+		step(hb, buf_, std::integral_constant<int, 6>{});
+		step(hb, buf_, std::integral_constant<int, 7>{});
+		step(hb, buf_, std::integral_constant<int, 8>{});
+	};
+	for (int hb = 0; hb < NB; hb += 2) {
+		block(hb, C0{});
+		block(hb + 1, C1{});
 	}
+	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the epilogue reuses it) */
 
 	/* ---- epilogue ---- */
 	elem *y = (elem *)p.y;
