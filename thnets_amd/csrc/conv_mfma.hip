@@ -1714,7 +1714,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	constexpr int B_VECS = BL * WAVES * 64;				/* a buffer: every load's 1 KiB, the unused ones' too */
 	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = 3;
 	constexpr int A_VECS = MB * KCH * 64, A_PW = MB * KCH / WAVES;
-	static_assert(CI % (2 * PCI) == 0 && A_PW == 1 && TH == 2 * WAVES && BL <= 8, "shape");
+	static_assert(CI % (2 * PCI) == 0 && MB * KCH % WAVES == 0 && TH == 2 * WAVES && BL <= 8, "shape");
 	/* (one array, every stage and buffer at a constant offset: conv_f32_patch_kernel says why) */
 	__shared__ floatx4 lds[NST * A_VECS + 2 * B_VECS];
 	floatx4 *const astage = lds;
@@ -1756,16 +1756,24 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 		const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
 		voff_[t] = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + v * 8) * (int)sizeof(elem)) : 0x80000000u;
 	}
-	/* this wave's weight block of a K-tile: 32-row block wave % MB, chunk wave / MB */
-	const unsigned a_base = (unsigned)(tile_m * MB + wave % MB) * (unsigned)p.KC * 1024u;
-	const int a_kci = wave / MB, a_lds = (a_kci * MB + wave % MB) * 64;
+	/* this wave's weight blocks of a K-tile: wave + 4 i counts (chunk, 32-row block) */
+	unsigned a_off_[A_PW];
+	int a_lds_[A_PW];
+#pragma unroll
+	for (int i = 0; i < A_PW; i++) {
+		const int idx = wave + WAVES * i, mbi = idx % MB, kci = idx / MB;
+		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
+		a_lds_[i] = (kci * MB + mbi) * 64;
+	}
 
 	/* the weights of K-tile (block hb of 32 planes, tap): K runs (block, tap, plane) in chunks of 16 */
 	auto issue_a = [&](auto st_, int hb, int tap) {
 		constexpr int st = decltype(st_)::value;
-		const unsigned kc = (unsigned)((hb * 9 + tap) * KCH + a_kci);
-		__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds), 16,
-			hb < NB ? lane * 16 : 0x80000000u, a_base + kc * 1024u, 0, 0);
+		const unsigned kc = (unsigned)((hb * 9 + tap) * KCH);
+#pragma unroll
+		for (int i = 0; i < A_PW; i++)
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16,
+				hb < NB ? lane * 16 : 0x80000000u, a_off_[i] + kc * 1024u, 0, 0);
 	};
 	auto issue_b = [&](auto t_, int hb, auto buf_) {
 		constexpr int buf = decltype(buf_)::value, t = decltype(t_)::value;
@@ -1828,7 +1836,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	issue_a(C0{}, 0, 0);
 	issue_a(C1{}, 0, 1);
 	issue_a(C2{}, 0, 2);
-	wide_wait<2, false>();	/* the patch and the first K-tile's weights */
+	wide_wait<2 * A_PW, false>();	/* the patch and the first K-tile's weights */
 	__builtin_amdgcn_s_barrier();
 	read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
 	/* The pipeline of conv_f32_patch_kernel: K-tile (hb, tap) has its weights in stage tap % 3; a step issues
@@ -1842,11 +1850,11 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 		typedef std::integral_constant<int, buf ^ 1> OTHER;
 		typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
 		constexpr int prev = (tap + 8) % 9;
-		constexpr int last_loads = 1 + CONV_PATCH_PB(prev + 1) - CONV_PATCH_PB(prev);
+		constexpr int last_loads = A_PW + CONV_PATCH_PB(prev + 1) - CONV_PATCH_PB(prev);
 		read_frags(ST{}, buf_, tap_, 1, af[1], bf[1]);
 		__builtin_amdgcn_sched_barrier(0);	/* (the fragments are asked for before the MFMAs that follow in the source) */
 		mma(0);
-		wide_wait<tap == 8 ? 1 : last_loads, true>();
+		wide_wait<tap == 8 ? A_PW : last_loads, true>();
 		__builtin_amdgcn_s_barrier();
 		read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[0], bf[0]);
 		__builtin_amdgcn_sched_barrier(0);
@@ -3442,7 +3450,7 @@ template <int DT>
 static bool conv_patch_ok(const ConvParams &p)
 {
 	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16)
-		return p.x_cl == 1 && (p.Ci == 64 || p.Ci == 128) && p.kH == 3 && p.kW == 3 && p.dH == 1 && p.dW == 1 &&
+		return p.x_cl == 1 && (p.Ci == 64 || p.Ci == 128 || p.Ci == 256 || p.Ci == 512) && p.kH == 3 && p.kW == 3 && p.dH == 1 && p.dW == 1 &&
 			p.x_bytes < 0x7fffffffu && !g_force_generic_cl && (!p.y_cl || p.Co % 4 == 0);
 	return false;
 }
@@ -3469,6 +3477,14 @@ static void conv_launch_patch(ConvParams &p)
 			CONV_PATCH_GO(true, 64);
 		else if (p.Ci == 64)
 			CONV_PATCH_GO(false, 64);
+		else if (p.Ci == 256 && p.y_cl)
+			CONV_PATCH_GO(true, 256);
+		else if (p.Ci == 256)
+			CONV_PATCH_GO(false, 256);
+		else if (p.Ci == 512 && p.y_cl)
+			CONV_PATCH_GO(true, 512);
+		else if (p.Ci == 512)
+			CONV_PATCH_GO(false, 512);
 		else if (p.y_cl)
 			CONV_PATCH_GO(true, 128);
 		else
@@ -3484,11 +3500,11 @@ template <int DT>
 static bool conv_pool_uses_patch(const ConvParams &p)
 {
 	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
-		const long n = (long)p.B * p.oH * p.oW;
-		const long t256 = (long)((p.Co + 255) / 256) * ((n + 255) / 256);
 		const long tpatch = (long)((p.Co + 63) / 64) * p.B * ((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH);
-		const bool wide256 = conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128;
-		return conv_patch_ok<DT>(p) && tpatch >= 128 && !(wide256 && p.Ci > 64);
+		/* 256 and 512 planes: where the 32 x 8 tiles waste at most three tenths of their pixels (56^2: an
+		 * eighth; 28^2: 31 %, left to the tiles loaded straight into LDS) */
+		const bool fits = (long)((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH) * 256 * 10 <= (long)p.oH * p.oW * 13;
+		return conv_patch_ok<DT>(p) && tpatch >= 128 && (fits || p.Ci <= 128);
 	}
 	return false;
 }
@@ -3544,10 +3560,13 @@ static void conv_dispatch(ConvParams &p)
 		 * 64->128 @112^2 55 -> 49 / 226 -> 209 us, 64->64 @56^2 12.9 -> 11.3 /
 		 * 36 -> 29 us, 128->128 @112^2 90 -> 76 / 382 -> 361 us, 128->256 @56^2
 		 * 54 -> 42 / 183 -> 157 us (the 256x256 tile: 41 / 171 us); 128 rows per
-		 * workgroup measured slower than 64) */
-		const long tpatch = (long)((p.Co + 63) / 64) * p.B * ((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH);
+		 * workgroup measured slower than 64).  With its patches in two buffers the
+		 * same kernel also takes 256 and 512 input planes where its 32 x 8 tiles fit
+		 * the output (VGG-16's 56^2 layers; with them and 128->256 @56^2, which the
+		 * 256x256 tile used to take: fp16 batch 16 0.691 -> 0.676 ms, batch 64
+		 * 2.18 -> 2.14 ms in one session). */
 		const bool wide256 = conv_wide_ok<DT>(p) && p.Co % 256 == 0 && t256 > 128;
-		if (conv_patch_ok<DT>(p) && tpatch >= 128 && !(wide256 && p.Ci > 64))	/* (inside a network 128->256 is better off below) */
+		if (conv_pool_uses_patch<DT>(p))	/* (the rule is there: the fused pooling asks the same question) */
 			bm = 64, bn = 1;
 		else if (conv_wide_ok<DT>(p)) {
 			/* operands straight into LDS, the tile by how many there are (random
@@ -3689,7 +3708,10 @@ static void conv_dispatch(ConvParams &p)
 		THError("thhip_conv2d: fp32 pooling in the epilogue needs the tiles loaded straight into LDS, without a K split");
 	if (bn == 1) {	/* (64, 1): the patch kernel */
 		if (!conv_patch_ok<DT>(p))
-			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64 or 128 planes, 3x3, stride 1");
+			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64, 128, 256 or 512 planes, 3x3, stride 1");
+		/* (the tuning hook's last argument 2: 128 planes per workgroup) */
+		if (g_force_wgs == 2 && p.Co % 128 == 0)
+			return conv_launch_patch<DT, 128>(p);
 		return conv_launch_patch<DT, 64>(p);
 	}
 	if constexpr (DT == THHIP_F32) {
