@@ -459,7 +459,7 @@ void thhip_conv2d_layout(const void *x, const void *wpacked, const float *scale,
  * (modules/SpatialMaxPooling.c:6-98 after SpatialConvolutionMM.c:111-225) for the
  * layers thhip_conv2d_pool2_supported accepts: half types, channels-last input
  * with planes in blocks of 32 (the kernel that keeps an input patch in LDS for
- * 3x3 / stride 1 layers of 64 or 128 planes with enough tiles, else the tiles
+ * 3x3 / stride 1 layers of 64, 128, 256 or 512 planes with enough tiles, else the tiles
  * loaded straight into LDS); fp32, plane-major tensors, planes in blocks of 32, any
  * kernel size and stride, more than 512 tiles of 64 planes x 64 positions (the
  * layers that run without a K split): the kernel then walks the positions window
@@ -497,7 +497,7 @@ void thhip_conv2d_residual(const void *x, const void *wpacked, const float *scal
  *     tiles 64x64 and 128x64, wgs_per_cu == 2 selecting K-tiles of 16 values;
  *   bn == 256 (half types): the 256x256 and 128x256 tiles of the same kernel
  *     (splitk == 4 with bm == 256: K-tiles of 64 values in two stages);
- *   (64, 1): the half-type kernel for 3x3 stride-1 layers of 64 or 128 planes
+ *   (64, 1): the half-type kernel for 3x3 stride-1 layers of 64, 128, 256 or 512 planes
  *     that keeps an input patch in LDS.
  * A layer the forced kernel cannot take ends in THError. */
 void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);

@@ -634,14 +634,15 @@ def test_conv_half_wide_tile(hiplib, oracle, dt):
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_conv_half_patch_kernel(hiplib, oracle, dt):
-    """3x3 stride-1 convolutions of 64 or 128 planes whose taps come from an input patch in LDS:
+    """3x3 stride-1 convolutions of 64 to 512 planes whose taps come from an input patch in LDS:
     images smaller and larger than the 8 x 32 tile, partial tiles on both axes, padding 0, 1
     and 2, plane counts that leave a partial 64-row tile, both output orders."""
     from thnets_amd import api
     g = cases.rng(912)
     shapes = [(2, 5, 7, 64, 1, 1, 64), (1, 8, 32, 128, 1, 1, 64), (3, 19, 45, 72, 1, 1, 64), (1, 40, 33, 200, 0, 0, 64),
               (2, 9, 70, 36, 2, 1, 64), (1, 16, 64, 260, 1, 0, 64), (1, 3, 3, 64, 0, 0, 64),
-              (2, 11, 37, 72, 1, 1, 128), (1, 8, 32, 128, 0, 1, 128), (1, 21, 9, 40, 1, 1, 128)]   # 128 planes: two patches
+              (2, 11, 37, 72, 1, 1, 128), (1, 8, 32, 128, 0, 1, 128), (1, 21, 9, 40, 1, 1, 128),   # 128 planes: four blocks of 32
+              (1, 13, 40, 72, 1, 1, 256), (2, 8, 33, 64, 1, 1, 512)]                                 # eight and sixteen blocks
     try:
         for (B, H, W, Co, pH, pW, Ci) in shapes:
             x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)

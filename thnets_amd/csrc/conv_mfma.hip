@@ -1673,7 +1673,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_tail_finish_kernel(C
 }
 
 /* ------------------------------------------------------------------ */
-/* 3x3, stride 1, 64 or 128 planes in: taps from an input patch in LDS */
+/* 3x3, stride 1, 64 to 512 planes in: taps from an input patch in LDS */
 /* ------------------------------------------------------------------ */
 
 /* With 64 input planes a K-tile of the kernels above moves 64 bytes per
