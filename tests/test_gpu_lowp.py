@@ -367,13 +367,16 @@ def test_linear_batched_u8_bit_exact(hiplib, oracle):
     """One-position layers through the matrix kernel: against the GEMM + bias add of the
     restatement (a plane of one element is all tail: no lower clamp), ragged rows,
     batches (one, two and four groups of sixteen columns) and K tails (K % 64 of 16, 48;
-    fewer K-steps than wavefronts), with wrapping parameters."""
+    fewer K-steps than wavefronts), layers wide enough for two row blocks per workgroup, with
+    wrapping parameters."""
     g = cases.rng(1200)
     prms = (dict(a_off=-117, b_off=-128, c_off=32513, c_mult=1028, c_shift=18),
             dict(a_off=-255, b_off=3, c_off=-12345, c_mult=511, c_shift=14),
             dict(a_off=0, b_off=0, c_off=0, c_mult=9000, c_shift=20))
     shapes = ((1, 16, 1), (2, 144, 37), (33, 1024, 100), (64, 2064, 70), (17, 4096, 130), (64, 9216, 64),
-              (16, 1088, 16), (32, 64, 33), (48, 4144, 17), (5, 6400, 1000))
+              (16, 1088, 16), (32, 64, 33), (48, 4144, 17), (5, 6400, 1000),
+              # wide layers, two blocks of sixteen rows per workgroup: whole, a ragged last block, an odd number of blocks
+              (64, 1024, 4096), (20, 320, 4090), (33, 128, 4104))
     for ci, (B, K, nOut) in enumerate(shapes):
         xq = g.integers(0, 256, (B, K), dtype=np.uint8)
         wq = g.integers(0, 256, (nOut, K), dtype=np.uint8)

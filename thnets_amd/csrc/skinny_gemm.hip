@@ -398,7 +398,7 @@ extern "C" int thhip_linear_batched_noalloc(const void *x, const void *wrow, con
  *   by lane, re-centred to signed bytes (code - 128), K-steps of a block one
  *   after the other: a load instruction reads 1 KiB contiguous, no permutes.
  *   Rows and K are padded with re-centred zeros, which add nothing.
- * - A workgroup of sixteen wavefronts owns one 16-row block and all of K, which
+ * - A workgroup of sixteen wavefronts owns one 16-row block (or two, see below) and all of K, which
  *   it walks in chunks of sixteen K-steps (1024 codes), wavefront w taking step
  *   w of every chunk: the workgroup reads 16 KiB of contiguous weights per
  *   chunk, each wavefront keeps the weights of the next three chunks on their
@@ -419,6 +419,15 @@ extern "C" int thhip_linear_batched_noalloc(const void *x, const void *wrow, con
  *   of one element is all "tail": no lower clamp,
  *   lowp_SpatialConvolution.c:86-87) and the threshold, and writes y [B][nOut].
  *   No partial sums in global memory, no second launch.
+ * - What a wide layer at batch 64 waits for is the path from L2 to the CUs: every workgroup fetches the
+ *   activations of all its batch columns, four times the bytes of a row block's weights.  So a workgroup
+ *   takes RB row blocks and NCG groups of sixteen columns, gridDim.y slices of the batch: two row blocks x
+ *   32 columns for layers of 256 row blocks and more (a fifth fewer bytes than 16 rows x 64 columns for
+ *   as many outputs; two row blocks x 64 columns do not fit the 128 registers a thread of 1024 has), and
+ *   one row block x 16 columns for layers of fewer row blocks than CUs, which then spread over four
+ *   times the CUs.  AlexNet-OWT batch 64: 9216 -> 4096 18.1 -> 14.4 us, 4096 -> 4096 12.2 -> 9.4 us,
+ *   4096 -> 1000 10.5 -> 5.8 us.  (Walking the chunks from a different one on in every workgroup, so that
+ *   they do not ask for the same activations at the same time, was slower.)
  */
 #define LU_THREADS 1024
 #define LU_WAVES 16
@@ -427,19 +436,27 @@ extern "C" int thhip_linear_batched_noalloc(const void *x, const void *wrow, con
 #define LU_CHUNK (LU_WAVES * LU_KSTEP)	/* codes per chunk */
 #define LU_AHEAD 4			/* chunks of activations in flight (in registers); weights: one fewer */
 
-template <int NCG>	/* groups of 16 batch columns: batch <= 16 * NCG */
+template <int NCG, int RB>	/* groups of 16 batch columns: batch <= 16 * NCG; 16-row blocks per workgroup */
 __global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned char *x, const unsigned char *wfrag,
 	const int *rowsum, const int *addend, unsigned char *y, int B, int K, int nOut, int nsteps, int offA, int offB,
 	int c_off, int c_mult, int c_shift, int act, int thr, int val)
 {
 	extern __shared__ __align__(16) unsigned char lds[];	/* two buffers of NCG * 16 KiB */
+	/* (gridDim.y slices of 16 NCG batch columns) */
+	x += (size_t)blockIdx.y * (16 * NCG) * K;
+	y += (size_t)blockIdx.y * (16 * NCG) * nOut;
+	B = min(B - (int)blockIdx.y * (16 * NCG), 16 * NCG);
 	constexpr int XBUF = NCG * 16 * LU_CHUNK;
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int m = lane & 15, q = lane >> 4;
 	const int nchunks = (nsteps + LU_WAVES - 1) / LU_WAVES;
 	/* uniform bases plus 32-bit lane offsets: the addresses stay on the scalar unit */
-	const unsigned char *wp = wfrag + ((size_t)blockIdx.x * nsteps) * 1024;
+	const int nblocks = (nOut + LU_ROWS - 1) / LU_ROWS;
+	const unsigned char *wp[RB];	/* (a block past the last one reads the last one again: never stored) */
+#pragma unroll
+	for (int rb = 0; rb < RB; rb++)
+		wp[rb] = wfrag + ((size_t)min((int)blockIdx.x * RB + rb, nblocks - 1) * nsteps) * 1024;
 	const unsigned woff = lane * 16;
 	/* staging: this thread moves piece `lane` of rows wave, wave + 16, ... of a chunk */
 	unsigned xsrc[NCG], xdst[NCG];
@@ -450,19 +467,26 @@ __global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned ch
 	}
 	/* fragments: step `wave` of the chunk, group g, quarter q, row m */
 	const unsigned fsrc = ((wave * NCG) * 4 + q) * 256 + ((m ^ (wave * 4 + q)) & 15) * 16;
-	intx4 acc[NCG];
+	intx4 acc[RB][NCG];
 	int cs[NCG];
 #pragma unroll
 	for (int g = 0; g < NCG; g++) {
-		acc[g] = intx4{ 0, 0, 0, 0 };
+#pragma unroll
+		for (int rb = 0; rb < RB; rb++)
+			acc[rb][g] = intx4{ 0, 0, 0, 0 };
 		cs[g] = 0;
 	}
-	intx4 a[LU_AHEAD], xr[LU_AHEAD][NCG];
+	intx4 a[LU_AHEAD][RB], xr[LU_AHEAD][NCG];
 	const intx4 zero_b = { (int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080 };
 
 	/* Requests past the end repeat the last valid address (a hit, and never used), so
 	 * the loop body has no divergent branches. */
-#define LU_LOAD_A(SLOT_, C_) (a[SLOT_] = *(const intx4 *)(wp + (size_t)min((C_) * LU_WAVES + wave, nsteps - 1) * 1024 + woff))
+#define LU_LOAD_A(SLOT_, C_)                                                                       \
+	do {                                                                                       \
+		const size_t o_ = (size_t)min((C_) * LU_WAVES + wave, nsteps - 1) * 1024 + woff;   \
+		_Pragma("unroll") for (int rb = 0; rb < RB; rb++)                                  \
+			a[SLOT_][rb] = *(const intx4 *)(wp[rb] + o_);                              \
+	} while (0)
 #define LU_LOAD_X(SLOT_, C_)                                                                       \
 	do {                                                                                       \
 		const int k_ = min((C_), nchunks - 1) * LU_CHUNK;                                  \
@@ -497,8 +521,9 @@ __global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned ch
 			intx4 bb_[NCG];                                                            \
 			_Pragma("unroll") for (int g = 0; g < NCG; g++)                            \
 				bb_[g] = *(const intx4 *)(lds + ((C_) & 1) * XBUF + fsrc + g * 1024); \
+			_Pragma("unroll") for (int rb = 0; rb < RB; rb++)                          \
 			_Pragma("unroll") for (int g = 0; g < NCG; g++)                            \
-				acc[g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[SLOT_], bb_[g], acc[g], 0, 0, 0); \
+				acc[rb][g] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[SLOT_][rb], bb_[g], acc[rb][g], 0, 0, 0); \
 		}                                                                                  \
 	} while (0)
 
@@ -549,54 +574,59 @@ __global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned ch
 		if (lane == 0)
 			colsum[g * 16 + wave] = v;
 	}
-	if (wave >= 8) {
-#pragma unroll
-		for (int g = 0; g < NCG; g++)
-#pragma unroll
-			for (int r = 0; r < 4; r++)
-				red[wave - 8][g * 4 + r][lane] = acc[g][r];
-	}
-	__syncthreads();
-	if (wave < 8) {
-#pragma unroll
-		for (int g = 0; g < NCG; g++)
-#pragma unroll
-			for (int r = 0; r < 4; r++)
-				acc[g][r] += red[wave][g * 4 + r][lane];
-	}
-	__syncthreads();
-	if (wave < 8) {
-#pragma unroll
-		for (int g = 0; g < NCG; g++)
-#pragma unroll
-			for (int r = 0; r < 4; r++)
-				red[wave][g * 4 + r][lane] = acc[g][r];
-	}
-	__syncthreads();
 	/* thread -> (row rr, batch column bcol): neighbouring threads write neighbouring bytes of y */
 	const int rr = tid & 15, bcol = tid >> 4;
-	const int o = blockIdx.x * LU_ROWS + rr;
-	if (bcol >= 16 * NCG || bcol >= B || o >= nOut)
-		return;
-	const int g = bcol >> 4, n = bcol & 15;
+	const int g = (bcol >> 4) % NCG, n = bcol & 15;	/* (bcol < 16 NCG is checked before use) */
 	const int src = (rr >> 2) * 16 + n, reg = g * 4 + (rr & 3);
-	int sum = 0, csum = 0;
 #pragma unroll
-	for (int wv = 0; wv < 8; wv++)
-		sum += red[wv][reg][src];
-	csum = colsum[bcol];
-	const int t = sum + offB * rowsum[o] + K * offA * offB + offA * csum;
-	unsigned u = ((unsigned)t + (unsigned)c_off) * (unsigned)c_mult;
-	u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
-	int code = (int)u >> c_shift;
-	code = code < 0 ? 0 : code > 255 ? 255 : code;
-	if (addend) {
-		const int sa = code + addend[o];
-		code = sa > 255 ? 255 : (sa & 255);
+	for (int rb = 0; rb < RB; rb++) {
+		if (rb)
+			__syncthreads();	/* the previous block's sums have been read */
+		if (wave >= 8) {
+#pragma unroll
+			for (int gg = 0; gg < NCG; gg++)
+#pragma unroll
+				for (int r = 0; r < 4; r++)
+					red[wave - 8][gg * 4 + r][lane] = acc[rb][gg][r];
+		}
+		__syncthreads();
+		if (wave < 8) {
+#pragma unroll
+			for (int gg = 0; gg < NCG; gg++)
+#pragma unroll
+				for (int r = 0; r < 4; r++)
+					acc[rb][gg][r] += red[wave][gg * 4 + r][lane];
+		}
+		__syncthreads();
+		if (wave < 8) {
+#pragma unroll
+			for (int gg = 0; gg < NCG; gg++)
+#pragma unroll
+				for (int r = 0; r < 4; r++)
+					red[wave][gg * 4 + r][lane] = acc[rb][gg][r];
+		}
+		__syncthreads();
+		const int o = ((int)blockIdx.x * RB + rb) * LU_ROWS + rr;
+		if (bcol >= 16 * NCG || bcol >= B || o >= nOut)
+			continue;
+		int sum = 0;
+#pragma unroll
+		for (int wv = 0; wv < 8; wv++)
+			sum += red[wv][reg][src];
+		const int csum = colsum[bcol];
+		const int t = sum + offB * rowsum[o] + K * offA * offB + offA * csum;
+		unsigned u = ((unsigned)t + (unsigned)c_off) * (unsigned)c_mult;
+		u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
+		int code = (int)u >> c_shift;
+		code = code < 0 ? 0 : code > 255 ? 255 : code;
+		if (addend) {
+			const int sa = code + addend[o];
+			code = sa > 255 ? 255 : (sa & 255);
+		}
+		if (act)
+			code = code > thr ? code : val;
+		y[(size_t)bcol * nOut + o] = (unsigned char)code;
 	}
-	if (act)
-		code = code > thr ? code : val;
-	y[(size_t)bcol * nOut + o] = (unsigned char)code;
 }
 
 extern "C" int thhip_linear_batched_u8_supported(int B, int K, int nOut)
@@ -651,23 +681,38 @@ extern "C" void thhip_linear_batched_u8(const unsigned char *x, const unsigned c
 	const int nblocks = (nOut + LU_ROWS - 1) / LU_ROWS, nsteps = (K + LU_KSTEP - 1) / LU_KSTEP;
 	/* algorithmic work for the profiler: 2 nOut K B operations */
 	ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * nOut * (double)K * B);
-	const dim3 grid(nblocks), block(LU_THREADS);
+	/* Every workgroup fetches the activations of all its batch columns, at batch 64 four times the bytes
+	 * of a row block's weights, and the path from L2 to the CUs is what a wide layer waits for: there a
+	 * workgroup takes two row blocks and 32 columns (a fifth fewer bytes for as many outputs; two row
+	 * blocks and all 64 columns would not fit the 128 registers a thread of 1024 has). */
+	const bool square = nblocks >= 256 && B > 32;
+	const int rb = square ? 2 : 1;
+	/* a narrow layer (fewer row blocks than CUs): slices of 16 or 32 batch columns to more workgroups,
+	 * each of which then waits for a quarter or half of the activations only */
+	int ncg = square ? 2 : B <= 16 ? 1 : B <= 32 ? 2 : 4;
+	if (!square && ncg > 1 && nblocks * ((B + 15) / 16) <= 256)
+		ncg = 1;
+	else if (!square && ncg > 2 && nblocks * ((B + 31) / 32) <= 256)
+		ncg = 2;
+	const dim3 grid((nblocks + rb - 1) / rb, (B + 16 * ncg - 1) / (16 * ncg)), block(LU_THREADS);
 	/* two activation buffers of NCG * 16 KiB: more than the 64 KiB a kernel gets without asking */
-	static bool lds_ok[3];
-#define LU_GO(NCG_, I_) do { \
+	static bool lds_ok[4];
+#define LU_GO(NCG_, RB_, I_) do { \
 		const int bytes_ = 2 * NCG_ * 16 * LU_CHUNK; \
 		if (!lds_ok[I_]) { \
-			hipcheck(hipFuncSetAttribute((const void *)linear_u8_kernel<NCG_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes_)); \
+			hipcheck(hipFuncSetAttribute((const void *)linear_u8_kernel<NCG_, RB_>, hipFuncAttributeMaxDynamicSharedMemorySize, bytes_)); \
 			lds_ok[I_] = true; \
 		} \
-		linear_u8_kernel<NCG_><<<grid, block, bytes_, thhip_stream()>>>(x, wfrag, rowsum, addend, y, B, K, nOut, \
+		linear_u8_kernel<NCG_, RB_><<<grid, block, bytes_, thhip_stream()>>>(x, wfrag, rowsum, addend, y, B, K, nOut, \
 			nsteps, 128 + a_off, 128 + b_off, c_off, c_mult, c_shift, act, thr, val); \
 	} while (0)
-	if (B <= 16)
-		LU_GO(1, 0);
-	else if (B <= 32)
-		LU_GO(2, 1);
+	if (square)
+		LU_GO(2, 2, 3);
+	else if (ncg == 1)
+		LU_GO(1, 1, 0);
+	else if (ncg == 2)
+		LU_GO(2, 1, 1);
 	else
-		LU_GO(4, 2);
+		LU_GO(4, 1, 2);
 #undef LU_GO
 }
