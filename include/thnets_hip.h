@@ -531,7 +531,7 @@ void thhip_gemv(const void *x, const void *w, const float *bias, void *y,
  * (Linear.c:92-108: addmm with beta 0, then the rank-1 bias update through
  * addr / sger, thbasic.c:757-789): Y[b][o] = bias[o] + sum_k W[o][k] X[b][k],
  * X [B][nIn], W row-major [nOut][nIn], Y [B][nOut].  thhip_linear_batched_supported
- * says whether the shape is taken (B <= 128, run in slices of 32 that each read
+ * says whether the shape is taken (B <= 128, run in slices of 64 that each read
  * the weights; rows in 16-byte vectors: nIn % 4 == 0 for fp32, % 8 for the half
  * types); other shapes run as a 1x1 convolution through thhip_conv2d. */
 int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtype);
@@ -549,7 +549,7 @@ void thhip_linear_batched_set_tuning(int row_blocks);
  * runs on holds until the process ends, instead of a buffer that grows on demand.
  * The call allocates and frees nothing on the device or through the runtime.
  * Returns 0, or (with a message on stderr, nothing launched) -1 for a shape
- * thhip_linear_batched_supported refuses, -2 when a slice of 32 batch rows needs
+ * thhip_linear_batched_supported refuses, -2 when a slice of 64 batch rows needs
  * more than the array holds (K slices x rows x nOut x 4 bytes; e.g. 25088 -> 4096
  * at batch 16 needs 2 MiB), -3 when the array's address cannot be resolved.
  * thhip_linear_batched_noalloc_init() resolves the address for the current device

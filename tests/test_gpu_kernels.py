@@ -273,7 +273,7 @@ def test_linear_batched_vs_oracle_and_golden(hiplib, oracle):
     from thnets_amd import api
     g = cases.rng(906)
     shapes = [(4, 128, 64), (16, 512, 100), (2, 64, 17), (16, 4096, 1000), (32, 1028, 515), (17, 200, 33), (7, 25088, 48),
-              (16, 1024, 1100), (20, 516, 1030), (64, 1024, 260), (45, 516, 1030), (128, 256, 48)]   # the last: slices of 32
+              (16, 1024, 1100), (20, 516, 1030), (64, 1024, 260), (45, 516, 1030), (128, 256, 48)]   # the last: slices of 64 (of 32 with the row blocks forced)
     for (B, nIn, nOut) in shapes:
         assert hiplib.thhip_linear_batched_supported(B, nIn, nOut, G.F32)
         x = g.standard_normal((B, nIn), dtype=np.float32)

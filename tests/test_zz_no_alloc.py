@@ -47,8 +47,9 @@ def test_noalloc_linear_two_calls_second_smaller(hiplib, oracle):
     # ... then a small ragged one that reuses the front of the same array
     both(hiplib, oracle, 5, 516, 70, 0, G.F32, 2101, 2e-5)
     both(hiplib, oracle, 3, 1024, 33, 1, G.F32, 2102, 2e-5)
-    # two slices of 32 and 8 rows, and the half types
+    # 40 rows (four column groups), 100 rows (two slices), and the half types
     both(hiplib, oracle, 40, 4096, 1000, 0, G.F32, 2103, 2e-5)
+    both(hiplib, oracle, 100, 1024, 1100, 1, G.F32, 2106, 2e-5)
     both(hiplib, oracle, 16, 4096, 4096, 0, G.F16, 2104, 2e-2)   # (no threshold: a rounded value may fall on its other side)
     both(hiplib, oracle, 7, 2048, 100, 0, G.BF16, 2105, 6e-2)
 

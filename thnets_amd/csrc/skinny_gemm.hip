@@ -1,5 +1,5 @@
 /*
- * Linear on a small batch (2..32 rows): Y[b][o] = bias[o] + sum_k W[o][k] X[b][k].
+ * Linear on a small batch (2..64 rows a launch): Y[b][o] = bias[o] + sum_k W[o][k] X[b][k].
  *
  * Replaces the matrix branch of nn_Linear_updateOutput (modules/Linear.c:92-108:
  * addmm with beta = 0, then the rank-1 bias update through addr / sger,
@@ -22,7 +22,9 @@
  * For wide layers a wavefront owns RB = 4 such blocks of 16 rows: the batch
  * operand, which every wavefront has to fetch from L2 for its K slice and
  * which is as large per step as a block's weights, is then read once for 64
- * rows instead of once for 16.
+ * rows instead of once for 16.  A launch takes up to 64 batch rows: four groups of
+ * sixteen columns, beside which two row blocks per wavefront are what the registers
+ * hold.
  */
 #include <stdio.h>
 #include <stdlib.h>
@@ -208,10 +210,10 @@ static float *skinny_scratch(size_t bytes)
 	return g_scratch;
 }
 
-/* A launch takes 32 batch columns; larger batches run in slices of 32, each
- * reading the weights again: up to four slices that still beats the tiled
- * GEMM on the layers this is for (25088 -> 4096 fp16 at batch 64: 283 us as a
- * convolution of one position, two slices of 60 us here). */
+/* A launch takes 64 batch columns (four groups of sixteen beside two row blocks per wavefront:
+ * what the registers hold); larger batches run in slices of 64, each reading the weights again,
+ * which still beats the tiled GEMM on the layers this is for (25088 -> 4096 fp16 at batch 64:
+ * 283 us as a convolution of one position, two slices of 32 of 50 + 39 us, one launch here). */
 #define SK_MAX_BATCH 128
 
 extern "C" int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtype)
@@ -230,7 +232,11 @@ static void skinny_launch(const void *x, const void *wrow, const float *bias, vo
 		/* algorithmic bytes: W once, X once, Y once */
 		ThhipLaunchScope scope(SCOPED ? THHIP_FAM_GEMV : -1, (double)thhip_esize(DT) * ((double)nOut * nIn + (double)B * nIn + (double)B * nOut));
 		dim3 grid(groups, ksplit);
-		if (B <= 16 && rb == 4)
+		if (B > 32 && rb == 2)
+			skinny_kernel<DT, 4, 2><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+		else if (B > 32)
+			skinny_kernel<DT, 4, 1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
+		else if (B <= 16 && rb == 4)
 			skinny_kernel<DT, 1, 4><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
 		else if (B <= 16)
 			skinny_kernel<DT, 1, 1><<<grid, dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, ksplit);
@@ -257,7 +263,10 @@ extern "C" void thhip_linear_batched_set_tuning(int row_blocks)
 	g_skinny_rb = row_blocks;
 }
 
-/* Row blocks per wavefront, row groups and K split of one launch (B <= 32). */
+/* Batch rows one launch takes: 64, or 32 when the row blocks per wavefront are forced. */
+static inline int skinny_slice(void);
+
+/* Row blocks per wavefront, row groups and K split of one launch (B <= 64). */
 struct skinny_plan { int rb, groups, ksplit; };
 static struct skinny_plan skinny_choose(int B, int nIn, int nOut, int dtype)
 {
@@ -268,6 +277,8 @@ static struct skinny_plan skinny_choose(int B, int nIn, int nOut, int dtype)
 	p.rb = nOut >= 1024 && B > 8 ? 4 : 1;
 	if (g_skinny_rb)
 		p.rb = g_skinny_rb;
+	else if (B > 32 && p.rb == 4)
+		p.rb = 2;	/* 33..64 batch rows: four column groups, and the registers of two row blocks beside them */
 	p.groups = (nOut + 16 * p.rb - 1) / (16 * p.rb);
 	const int kstep = SK_KBYTES / thhip_esize(dtype);
 	const int nsteps = (nIn + kstep - 1) / kstep;
@@ -275,7 +286,7 @@ static struct skinny_plan skinny_choose(int B, int nIn, int nOut, int dtype)
 	 * 25088 -> 4096 at batch 16 runs 4 % (fp32) and 8 % (fp16) faster than with
 	 * four, and 16-27 % faster than with eight or sixteen), at least two K-steps
 	 * per wavefront */
-	p.ksplit = ((p.rb == 4 ? 512 : 1024) + p.groups - 1) / p.groups;
+	p.ksplit = ((p.rb == 4 ? 512 : p.rb == 2 ? 768 : 1024) + p.groups - 1) / p.groups;
 	if (p.ksplit > nsteps / 8)
 		p.ksplit = nsteps / 8;
 	if (p.ksplit < 1)
@@ -285,16 +296,19 @@ static struct skinny_plan skinny_choose(int B, int nIn, int nOut, int dtype)
 	return p;
 }
 
+static inline int skinny_slice(void) { return g_skinny_rb ? 32 : 64; }
+
 extern "C" void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
 	int B, int nIn, int nOut, int act, float thr, float val, int dtype)
 {
 	if (!thhip_linear_batched_supported(B, nIn, nOut, dtype))
 		THError("thhip_linear_batched: unsupported shape B=%d nIn=%d nOut=%d dtype=%d", B, nIn, nOut, dtype);
-	if (B > 32) {
+	const int slice = skinny_slice();
+	if (B > slice) {
 		const size_t esize = thhip_esize(dtype);
-		for (int b0 = 0; b0 < B; b0 += 32)
+		for (int b0 = 0; b0 < B; b0 += slice)
 			thhip_linear_batched((const char *)x + (size_t)b0 * nIn * esize, wrow, bias, (char *)y + (size_t)b0 * nOut * esize,
-				B - b0 < 32 ? B - b0 : 32, nIn, nOut, act, thr, val, dtype);
+				B - b0 < slice ? B - b0 : slice, nIn, nOut, act, thr, val, dtype);
 		return;
 	}
 	const struct skinny_plan p = skinny_choose(B, nIn, nOut, dtype);
@@ -355,9 +369,10 @@ extern "C" int thhip_linear_batched_noalloc(const void *x, const void *wrow, con
 		fprintf(stderr, "thhip_linear_batched_noalloc: unsupported shape B=%d nIn=%d nOut=%d dtype=%d\n", B, nIn, nOut, dtype);
 		return -1;
 	}
-	/* every slice of 32 batch rows must fit: check before anything is launched */
-	for (int b0 = 0; b0 < B; b0 += 32) {
-		const int bs = B - b0 < 32 ? B - b0 : 32;
+	/* every slice of batch rows must fit: check before anything is launched */
+	const int slice = skinny_slice();
+	for (int b0 = 0; b0 < B; b0 += slice) {
+		const int bs = B - b0 < slice ? B - b0 : slice;
 		const struct skinny_plan p = skinny_choose(bs, nIn, nOut, dtype);
 		const size_t need = (size_t)p.ksplit * bs * nOut * sizeof(float);
 		if (need > SK_STATIC_BYTES) {
@@ -371,8 +386,8 @@ extern "C" int thhip_linear_batched_noalloc(const void *x, const void *wrow, con
 	if (!part)
 		return -3;
 	const size_t esize = thhip_esize(dtype);
-	for (int b0 = 0; b0 < B; b0 += 32) {
-		const int bs = B - b0 < 32 ? B - b0 : 32;
+	for (int b0 = 0; b0 < B; b0 += slice) {
+		const int bs = B - b0 < slice ? B - b0 : slice;
 		const struct skinny_plan p = skinny_choose(bs, nIn, nOut, dtype);
 		const void *xs = (const char *)x + (size_t)b0 * nIn * esize;
 		void *ys = (char *)y + (size_t)b0 * nOut * esize;
