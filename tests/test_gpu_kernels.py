@@ -842,6 +842,19 @@ def test_softmax(hiplib, oracle, i):
     G.assert_close(y, GOLD["softmax%d" % i], 1e-5)
 
 
+def test_softmax_long_vectors(hiplib, oracle):
+    """A few long vectors take a workgroup of sixteen wavefronts each: lengths below and above what the
+    threads keep in registers (four values each), a strided one, against the restatement."""
+    g = cases.rng(440)
+    for sh in ((1, 1000), (2, 4096), (3, 5000), (2, 600, 3, 2), (1, 513)):
+        x = (g.standard_normal(sh, dtype=np.float32) * np.float32(4.0)).astype(np.float32)
+        nframe, dim, stride = _softmax_dims(sh)
+        G.note("softmax %s" % (sh,))
+        y = G.unary(hiplib, hiplib.thhip_softmax, x, sh, G.F32, nframe, dim, stride, G.F32)
+        G.assert_close(y, oracle.softmax(x), 1e-5, str(sh))
+        assert np.allclose(y.sum(axis=1), 1.0, atol=1e-4)
+
+
 def test_batchnorm_and_table_add(hiplib, oracle):
     from thnets_amd import api
     x, s = cases.bn_case()

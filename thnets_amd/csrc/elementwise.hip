@@ -699,27 +699,59 @@ __device__ __forceinline__ double exp_minus_approx(double x)
 	return 0;
 }
 
-/* modules/SoftMax.c:24-90: one wavefront per (frame, position). */
-template <int DT>
-__global__ __launch_bounds__(64) void softmax_kernel(const void *x, void *y, long dim, long stride)
+/* modules/SoftMax.c:24-90: one workgroup of T threads per (frame, position): a wavefront where there
+ * are many positions, sixteen for a few long vectors (a classifier's 1000 values at batch 1 took 11 us
+ * with one wavefront, the double-precision exponential twice per value; a thread's first four values are
+ * kept). */
+template <int DT, int T>
+__global__ __launch_bounds__(T) void softmax_kernel(const void *x, void *y, long dim, long stride)
 {
+	constexpr int KEEP = 4, WAVES = T / 64;
+	__shared__ float red[2][WAVES > 1 ? WAVES : 1];
 	const long t = blockIdx.x;
 	const long base = (t / stride) * dim * stride + t % stride;
-	const int lane = threadIdx.x;
+	const int tid = threadIdx.x;
 	float m = -FLT_MAX;
-	for (long d = lane; d < dim; d += 64)
+	for (long d = tid; d < dim; d += T)
 		m = fmaxf(m, ThhipElem<DT>::ld(x, base + d * stride));
 	for (int off = 32; off > 0; off >>= 1)
 		m = fmaxf(m, __shfl_xor(m, off, 64));
-	float sum = 0;
-	for (long d = lane; d < dim; d += 64) {
-		const float z = (float)exp_minus_approx((double)(m - ThhipElem<DT>::ld(x, base + d * stride)));
-		sum += z;
+	if constexpr (WAVES > 1) {
+		if ((tid & 63) == 0)
+			red[0][tid >> 6] = m;
+		__syncthreads();
+#pragma unroll
+		for (int w = 0; w < WAVES; w++)
+			m = fmaxf(m, red[0][w]);
 	}
+	float sum = 0, zk[KEEP];
+#pragma unroll
+	for (int i = 0; i < KEEP; i++) {
+		const long d = tid + (long)i * T;
+		zk[i] = d < dim ? (float)exp_minus_approx((double)(m - ThhipElem<DT>::ld(x, base + d * stride))) : 0.0f;
+		sum += zk[i];
+	}
+	for (long d = tid + (long)KEEP * T; d < dim; d += T)
+		sum += (float)exp_minus_approx((double)(m - ThhipElem<DT>::ld(x, base + d * stride)));
 	for (int off = 32; off > 0; off >>= 1)
 		sum += __shfl_xor(sum, off, 64);
+	if constexpr (WAVES > 1) {
+		if ((tid & 63) == 0)
+			red[1][tid >> 6] = sum;
+		__syncthreads();
+		sum = 0;
+#pragma unroll
+		for (int w = 0; w < WAVES; w++)
+			sum += red[1][w];
+	}
 	const float inv = 1 / sum;
-	for (long d = lane; d < dim; d += 64) {
+#pragma unroll
+	for (int i = 0; i < KEEP; i++) {
+		const long d = tid + (long)i * T;
+		if (d < dim)
+			ThhipElem<DT>::st(y, base + d * stride, zk[i] * inv);
+	}
+	for (long d = tid + (long)KEEP * T; d < dim; d += T) {
 		const float z = (float)exp_minus_approx((double)(m - ThhipElem<DT>::ld(x, base + d * stride)));
 		ThhipElem<DT>::st(y, base + d * stride, z * inv);
 	}
@@ -733,8 +765,12 @@ extern "C" void thhip_softmax(const void *x, void *y, long nframe, long dim, lon
 	if (npos > 0x7fffffffL)
 		THError("thhip_softmax: too many positions");
 	ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * npos * dim * thhip_esize(dtype));
-	THHIP_DISPATCH_FLOAT(dtype, (softmax_kernel<DT><<<dim3((unsigned)npos), dim3(64), 0, thhip_stream()>>>(
-		x, y, dim, stride)));
+	if (dim >= 512 && npos <= 2048)
+		THHIP_DISPATCH_FLOAT(dtype, (softmax_kernel<DT, 1024><<<dim3((unsigned)npos), dim3(1024), 0, thhip_stream()>>>(
+			x, y, dim, stride)));
+	else
+		THHIP_DISPATCH_FLOAT(dtype, (softmax_kernel<DT, 64><<<dim3((unsigned)npos), dim3(64), 0, thhip_stream()>>>(
+			x, y, dim, stride)));
 }
 
 /* lowp/lowp_SoftMax.c:3-89.  The exponent argument keeps the tensor offset,
