@@ -823,6 +823,18 @@ def test_pooling_bit_exact(hiplib, oracle, i):
     assert np.array_equal(yq, oracle.lowp_maxpool(q, kH, kW, dH, dW, pH, pW, ceil))
 
 
+def test_avgpool_whole_plane(hiplib, oracle):
+    """A window that is the whole plane (the pooling before a classifier) has a kernel of its own,
+    sixteen lanes per plane: against the restatement, plane sizes below, at and above sixteen."""
+    g = cases.rng(230)
+    for (B, Cn, H, W) in ((3, 70, 7, 7), (2, 33, 5, 4), (1, 5, 13, 13), (2, 9, 4, 4), (2, 3, 3, 3)):
+        x = g.standard_normal((B, Cn, H, W), dtype=np.float32)
+        G.note("avgpool whole plane %s" % ((B, Cn, H, W),))
+        for cip in (0, 1):
+            y = G.unary(hiplib, hiplib.thhip_avgpool, x, (B, Cn, 1, 1), G.F32, B, Cn, H, W, 1, 1, H, W, 1, 1, 0, 0, cip, G.F32)
+            G.assert_close(y, oracle.avgpool(x, H, W, 1, 1, 0, 0, 0, cip), 1e-6, str((B, Cn, H, W)))
+
+
 def _softmax_dims(sh):
     if len(sh) == 1:
         return 1, sh[0], 1
