@@ -471,6 +471,22 @@ void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, const float *
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, int x_layout, int y_channels_last);
 
+/* thhip_conv2d_affine followed by a max pooling of any window, stride, padding and
+ * rounding (modules/SpatialMaxPooling.c:6-98; the module sequence SpatialConvolutionMM
+ * -> Threshold -> SpatialMaxPooling), y = [B][Co][pH][pW] from thhip_pool_outsize of the
+ * convolution's output.  For the layers thhip_conv2d_poolk_supported accepts: fp32,
+ * plane-major, at most 512 tiles of 64 planes x 64 positions (a batch of one or a few
+ * images), i.e. the layers whose K is split over workgroups and whose parts a second
+ * kernel adds: that kernel takes the maximum of every window too, and the pooling's own
+ * launch is saved.  The same values, bit for bit, as thhip_conv2d_affine followed by
+ * thhip_maxpool. */
+int thhip_conv2d_poolk_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int pkH, int pkW, int pdH, int pdW, int ppH, int ppW, int ceil_mode, int dtype);
+void thhip_conv2d_poolk(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int pkH, int pkW, int pdH, int pdW, int ppH, int ppW, int ceil_mode,
+	int act, float thr, float val, int dtype);
+
 /* thhip_conv2d_affine followed by the two-input table add of a residual block and
  * the Threshold(0, 0) after it, in the convolution's epilogue.  With v = the
  * convolution's result (after factor, bias and its own Threshold) and r = res (a

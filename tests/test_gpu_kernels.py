@@ -128,6 +128,49 @@ def test_conv_f32_last_tiles_cut_along_k(hiplib, oracle):
         hiplib.thhip_conv_set_xcd_parts(0)
 
 
+def test_conv_f32_k_split_with_a_pooling_of_any_window(hiplib, oracle):
+    """fp32 layers of a few tiles split K and a second kernel adds the parts; that kernel also takes a max
+    pooling that follows (any window, stride, padding, rounding): the same bits as the convolution entry
+    point followed by the pooling one, the oracle's values, on AlexNet's batch-1 layers (planes in blocks of
+    32 or not), with the folded factor, with and without the threshold; layers it does not take."""
+    from thnets_amd import api
+    g = cases.rng(931)
+    # (B, Ci, H, W, Co, k, d, pad), (pool kH, kW, dH, dW, padH, padW, ceil)
+    shapes = [((1, 3, 224, 224, 64, 11, 4, 2), (3, 3, 2, 2, 0, 0, 0)), ((1, 64, 27, 27, 192, 5, 1, 2), (3, 3, 2, 2, 0, 0, 0)),
+              ((1, 256, 13, 13, 256, 3, 1, 1), (3, 3, 2, 2, 0, 0, 0)), ((2, 96, 20, 21, 70, 3, 1, 1), (2, 2, 2, 2, 0, 0, 1)),
+              ((3, 40, 17, 15, 33, 3, 1, 0), (3, 2, 2, 1, 1, 1, 1)), ((1, 128, 9, 9, 100, 3, 1, 1), (9, 9, 1, 1, 0, 0, 0))]
+    for (B, Ci, H, W, Co, k, d, pad), (pkH, pkW, pdH, pdW, ppH, ppW, ceil) in shapes:
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        sc = (g.uniform(0.5, 1.5, Co) * g.choice([-1.0, 1.0], Co)).astype(np.float32)
+        oH, oW = (H + 2 * pad - k) // d + 1, (W + 2 * pad - k) // d + 1
+        pH, pW = oracle.pool_outsize(oH, oW, pkH, pkW, pdH, pdW, ppH, ppW, ceil)
+        raw = oracle.conv2d(x, w, None, (d, d), (pad, pad)) * sc[None, :, None, None] + b[None, :, None, None]
+        for act in (1, 0):
+            G.note("conv + pooling of any window %s %s act %d" % ((B, Ci, H, W, Co, k, d, pad), (pkH, pkW, pdH, pdW, ppH, ppW, ceil), act))
+            assert hiplib.thhip_conv2d_poolk_supported(B, Ci, H, W, Co, k, k, d, d, pad, pad, pkH, pkW, pdH, pdW, ppH, ppW, ceil, G.F32)
+            unpooled = G.conv2d_layout(hiplib, x, w, b, (d, d), (pad, pad), act=act, dtype=G.F32, scale=sc)
+            ref = G.unary(hiplib, hiplib.thhip_maxpool, unpooled, (B, Co, pH, pW), G.F32, B, Co, oH, oW, pH, pW, pkH, pkW, pdH, pdW,
+                          ppH, ppW, G.F32)
+            dx = api.DeviceArray(hiplib, x)
+            wp = hiplib.thhip_conv_pack_weight_layout(np.ascontiguousarray(w).ctypes.data, Co, Ci, k, k, G.F32, 0)
+            db, ds = api.DeviceArray(hiplib, b), api.DeviceArray(hiplib, sc)
+            dy = api.DeviceArray(hiplib, nbytes=B * Co * pH * pW * 4)
+            hiplib.thhip_conv2d_poolk(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, B, Ci, H, W, Co, k, k, d, d, pad, pad,
+                                      pkH, pkW, pdH, pdW, ppH, ppW, ceil, act, 0.0, 0.0, G.F32)
+            hiplib.thhip_sync()
+            got = dy.get((B, Co, pH, pW), np.float32)
+            hiplib.thhip_free(wp)
+            assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), ((B, Ci, H, W, Co, k), int((got != ref).sum()))
+            want = oracle.maxpool(np.maximum(raw, 0) if act else raw, pkH, pkW, pdH, pdW, ppH, ppW, ceil)
+            G.assert_close(got, want, FP32_TOL, str((B, Ci, H, W, Co, k, d, pad)))
+    # layers of many tiles run without a K split, the half types have their own fused poolings
+    assert not hiplib.thhip_conv2d_poolk_supported(16, 64, 112, 112, 64, 3, 3, 1, 1, 1, 1, 3, 3, 2, 2, 0, 0, 0, G.F32)
+    assert not hiplib.thhip_conv2d_poolk_supported(1, 64, 27, 27, 192, 5, 5, 1, 1, 2, 2, 3, 3, 2, 2, 0, 0, 0, G.F16)
+    assert not hiplib.thhip_conv2d_poolk_supported(1, 64, 27, 27, 192, 5, 5, 1, 1, 2, 2, 3, 3, 2, 2, 2, 2, 0, G.F32)   # padding over half the window
+
+
 @pytest.mark.parametrize("dtype", [G.F16, G.BF16])
 def test_conv_half_last_tiles_cut_along_k(hiplib, oracle, dtype):
     """Half-type tiles loaded straight into LDS (channels-last input): the tiles an XCD

@@ -122,6 +122,8 @@ PROTOTYPES = {
     "thhip_conv_pack_weight_u8_layout": (vp, [vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_conv2d_u8_layout": (None, [vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int] * 6 + [C.c_int] * 3 + [C.c_int] * 2),
     "thhip_conv2d_pool2_supported": (C.c_int, [C.c_int] * 14),
+    "thhip_conv2d_poolk_supported": (C.c_int, [C.c_int] * 19),
+    "thhip_conv2d_poolk": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 18 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv2d_residual_supported": (C.c_int, [C.c_int] * 12),
     "thhip_conv2d_residual": (None, [vp, vp, vp, vp, vp, C.c_int, C.c_float, C.c_int, vp] + [C.c_int] * 11 +
                               [C.c_int, C.c_float, C.c_float, C.c_int]),

@@ -72,6 +72,9 @@ struct ConvParams {
 	int tail_cap;		/* scratch blocks (parts of BM*BN sums) reserved per XCD: [xcd][tile][part] */
 	int tail_tiles;		/* most cut tiles of an XCD */
 	int tail_round;		/* 1: an XCD with less than one whole round of tiles is left uncut */
+	/* conv_f32_direct_kernel with a K split of the whole layer: a max pooling that follows, taken by the kernel
+	 * that adds the parts (pk_kH 0: none); pk_oH x pk_oW is the pooled plane */
+	int pk_kH, pk_kW, pk_dH, pk_dW, pk_padH, pk_padW, pk_oH, pk_oW;
 	/* uint8 path only */
 	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
 	const int *addend;	/* per-plane bias addend, or NULL */
@@ -2816,7 +2819,8 @@ __global__ void conv_f32_splitk_finish_kernel(const float *ws, const float *bias
 		float v = 0;
 		for (int s = 0; s < parts; s++)
 			v += ws[(size_t)s * total + i];
-		v = scale ? v * scale[m] + (bias ? bias[m] : 0.0f) : v + (bias ? bias[m] : 0.0f);
+		/* (the factor and the bias in one rounding, said here so that it does not hang on how the compiler contracts) */
+		v = scale ? __builtin_fmaf(v, scale[m], bias ? bias[m] : 0.0f) : v + (bias ? bias[m] : 0.0f);
 		if (act)
 			v = v > thr ? v : val;
 		const int b = n / oHW, rem = n - b * oHW;
@@ -2829,6 +2833,62 @@ __global__ void conv_f32_splitk_finish_kernel(const float *ws, const float *bias
 		}
 		y[at] = v;
 	}
+}
+
+/* The same followed by a max pooling (any window, SpatialMaxPooling.c:6-98): sixteen lanes per pooled
+ * value, a lane per value of the window (lane, lane + 16, ... for larger windows).  A lane adds the
+ * parts of its values and finishes them as above; the maximum is then taken over the sixteen lanes as
+ * the reference's scan would: the first of equal values wins (+0 and -0), values that are not greater
+ * than -FLT_MAX (NaNs) never do.  y is the pooled tensor, plane-major.  For the layers of a few tiles
+ * that split K (a batch of one or a few images), where the pooling's own launch costs as much as its
+ * work. */
+__global__ __launch_bounds__(256) void conv_f32_splitk_finish_pool_kernel(const float *ws, const float *bias, const float *scale, float *y,
+	int parts, int B, int Co, int N, int oH, int oW, int act, float thr, float val,
+	int kH, int kW, int dH, int dW, int padH, int padW, int pH, int pW)
+{
+	const long total = (long)B * Co * pH * pW, part = (long)Co * N;
+	const long i = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
+	const int l = threadIdx.x & 15;
+	float mx = -FLT_MAX;
+	int me = 0x7fffffff;	/* the window element mx came from */
+	if (i < total) {
+		const int px = (int)(i % pW);
+		long t = i / pW;
+		const int py = (int)(t % pH);
+		t /= pH;
+		const int m = (int)(t % Co), b = (int)(t / Co);
+		const int hs = py * dH - padH, wst = px * dW - padW;
+		const float sc = scale ? scale[m] : 1.0f, bi = bias ? bias[m] : 0.0f;
+		const float *src = ws + (long)m * N + (long)b * oH * oW;
+		for (int e = l; e < kH * kW; e += 16) {
+			const int yy = hs + e / kW, xx = wst + e % kW;
+			if (yy < 0 || yy >= oH || xx < 0 || xx >= oW)
+				continue;
+			const float *at = src + yy * oW + xx;
+			float v = 0;
+#pragma unroll 4
+			for (int q = 0; q < parts; q++)
+				v += at[q * part];
+			v = scale ? __builtin_fmaf(v, sc, bi) : v + bi;	/* (one rounding, as in conv_f32_splitk_finish_kernel) */
+			if (act)
+				v = v > thr ? v : val;
+			if (v > mx) {
+				mx = v;
+				me = e;
+			}
+		}
+	}
+#pragma unroll
+	for (int off = 8; off > 0; off >>= 1) {
+		const float ov = __shfl_xor(mx, off, 64);
+		const int oe = __shfl_xor(me, off, 64);
+		if (ov > mx || (ov == mx && oe < me)) {
+			mx = ov;
+			me = oe;
+		}
+	}
+	if (i < total && l == 0)
+		y[i] = mx;
 }
 
 /* ------------------------------------------------------------------ */
@@ -3325,6 +3385,8 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 	if (splitk > nkt)
 		splitk = nkt;
 	p.splitk = splitk < 1 ? 1 : splitk;
+	if (p.pk_kH && p.splitk < 2)
+		THError("thhip_conv2d: a pooling after the convolution is taken by the kernel that adds the parts of a K split only");
 	if (p.splitk > 1)
 		conv_f32_scratch(p, (size_t)p.splitk * p.Co * p.N * sizeof(float));
 	if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
@@ -3345,7 +3407,14 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 	}
 	const size_t maxcnt = conv_tail_plan(p, resident, nkt, (size_t)BM * BN, 0);
 	conv_f32_direct_kernel<BM, BN, KCH, NST, ROWS><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
-	if (p.splitk > 1) {
+	if (p.pk_kH) {
+		const long blocks = ((long)p.B * p.Co * p.pk_oH * p.pk_oW + 15) / 16;
+		if (blocks > 0x7fffffffL)
+			THError("thhip_conv2d: pooled output too large");
+		conv_f32_splitk_finish_pool_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
+			(float *)p.y, p.splitk, p.B, p.Co, p.N, p.oH, p.oW, p.act, p.thr, p.val,
+			p.pk_kH, p.pk_kW, p.pk_dH, p.pk_dW, p.pk_padH, p.pk_padW, p.pk_oH, p.pk_oW);
+	} else if (p.splitk > 1) {
 		long blocks = ((long)p.Co * p.N + 255) / 256;
 		if (blocks > 4096)
 			blocks = 4096;
@@ -3688,6 +3757,9 @@ static void conv_dispatch(ConvParams &p)
 		kch = g_force_kch;
 	if (pool_patch)
 		bm = 64, bn = 1;
+	if (p.pk_kH && !(DT == THHIP_F32 && direct && bn != 1 && splitk > 1 && !g_force_bm))
+		THError("thhip_conv2d: a pooling after the convolution is taken by the kernel that adds the parts of a K split only "
+			"(see thhip_conv2d_poolk_supported)");
 	if (p.pool && !pool_patch && DT != THHIP_F32 && (!direct || bn == 1))
 		THError("thhip_conv2d: half-type pooling in the epilogue needs the patch kernel or the tiles loaded straight into LDS");
 	if constexpr (DT == THHIP_F32) {
@@ -3850,6 +3922,9 @@ static unsigned char *conv_pixels4_scratch(size_t bytes)
 	return g_c4;
 }
 
+/* A max pooling that follows the convolution, for conv_run: window, stride, padding, pooled plane. */
+struct ConvPoolK { int kH, kW, dH, dW, padH, padW, oH, oW; };
+
 struct ConvResidual {
 	const float *res;
 	int mode, act;
@@ -3859,7 +3934,7 @@ struct ConvResidual {
 static void conv_run(const void *x, const void *wpacked, const float *scale, const float *bias, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, const ConvU8Args *u8, int f_x_layout = 0, int f_y_cl = 0, int f_pool2 = 0,
-	const ConvResidual *f_res = 0)
+	const ConvResidual *f_res = 0, const ConvPoolK *f_pk = 0)
 {
 	if (B < 1 || Ci < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
 		THError("thhip_conv2d: bad geometry");
@@ -3875,7 +3950,8 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 	/* 32-bit offsets inside the kernel: run the batch in slices whose input
 	 * and output stay below 2^31 bytes. */
 	const int xl = u8 ? u8->x_cl : f_x_layout;
-	const long in_img = (long)Ci * H * W, out_img = f_pool2 ? (long)Co * (oH / 2) * (oW / 2) : (long)Co * oH * oW;
+	const long in_img = (long)Ci * H * W;
+	const long out_img = f_pk ? (long)Co * f_pk->oH * f_pk->oW : f_pool2 ? (long)Co * (oH / 2) * (oW / 2) : (long)Co * oH * oW;
 	const long in_eff = xl == 2 ? 4L * H * W : in_img;	/* bytes the kernel addresses per image */
 	long bmax = ((1L << 31) - 64) / (esize * (in_eff > out_img ? in_eff : out_img));
 	if (bmax < 1)
@@ -3959,6 +4035,12 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 			p.x_cl = xl;
 			p.y_cl = f_y_cl;
 			p.pool = f_pool2;
+			if (f_pk) {
+				if (bn != B)
+					THError("thhip_conv2d: a pooling after the convolution needs the batch in one slice");
+				p.pk_kH = f_pk->kH; p.pk_kW = f_pk->kW; p.pk_dH = f_pk->dH; p.pk_dW = f_pk->dW;
+				p.pk_padH = f_pk->padH; p.pk_padW = f_pk->padW; p.pk_oH = f_pk->oH; p.pk_oW = f_pk->oW;
+			}
 			if (f_res) {
 				p.res = f_res->res + (size_t)b0 * out_img;
 				p.res_mode = f_res->mode;
@@ -3967,7 +4049,7 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 			}
 			ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N);
 			/* a 3x3 image layer: whole rows from a patch in LDS (conv_stem.hip), unless a test forces a tile */
-			if (!f_pool2 && !f_res && xl == 0 && !g_force_bm &&
+			if (!f_pool2 && !f_res && !f_pk && xl == 0 && !g_force_bm &&
 			    thhip_conv_stem_ok(bn, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, dtype, f_y_cl))
 				thhip_conv_stem(p.x, wpacked, p.KC, scale, bias, p.y, bn, H, W, Co, act, thr, val, dtype, f_y_cl);
 			else
@@ -4078,6 +4160,70 @@ extern "C" void thhip_conv2d_residual(const void *x, const void *wpacked, const 
 		THError("thhip_conv2d_residual: layer not supported (see thhip_conv2d_residual_supported), or mode %d not 1 or 2", mode);
 	const ConvResidual r = { (const float *)res, mode, res_act, c };
 	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0, 0, 0, 0, &r);
+}
+
+/* Parts of the K split conv_dispatch gives an fp32 plane-major layer that runs on conv_f32_direct_kernel
+ * and has its parts added by a second kernel (its rule, restated: at most 512 tiles of 64 x 64, about
+ * 1024 workgroups, at least eight K-tiles a part); 0: another kernel, or no split. */
+static int conv_f32_split_parts(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW)
+{
+	if (B < 1 || Ci < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
+		return 0;
+	if (g_force_kch || g_force_bm || g_force_bn || g_force_splitk)
+		return 0;
+	const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
+	if (oW < 1 || oH < 1)
+		return 0;
+	if ((double)B * Ci * H * W * 4 >= 2147483000.0 || (double)B * Co * oH * oW * 4 >= 2147483000.0)
+		return 0;	/* (the batch would be cut into slices) */
+	const long N = (long)B * oH * oW, t64 = (long)((Co + 63) / 64) * ((N + 63) / 64);
+	if (t64 > 512)
+		return 0;
+	int kch;
+	if (Ci % 32 == 0)
+		kch = CONV_KCH_F32;
+	else if (kH * kW <= 4096)
+		kch = 2;	/* a (plane, tap) per K row */
+	else
+		return 0;
+	const int nkt = conv_kc(Ci, kH, kW, THHIP_F32, 0) / kch;
+	int parts = (int)((1024 + t64 - 1) / t64);
+	if (parts > nkt / 8)
+		parts = nkt / 8;
+	if (parts > 16)
+		parts = 16;
+	return parts > 1 ? parts : 0;
+}
+
+extern "C" int thhip_conv2d_poolk_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int pkH, int pkW, int pdH, int pdW, int ppH, int ppW, int ceil_mode, int dtype)
+{
+	if (dtype != THHIP_F32 || pkH < 1 || pkW < 1 || pdH < 1 || pdW < 1 || ppH < 0 || ppW < 0 || 2 * ppH > pkH || 2 * ppW > pkW)
+		return 0;
+	if (conv_f32_split_parts(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW) < 2)
+		return 0;
+	const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
+	int pH, pW;
+	thhip_pool_outsize(oH, oW, pkH, pkW, pdH, pdW, ppH, ppW, ceil_mode, &pH, &pW);
+	return pH >= 1 && pW >= 1;
+}
+
+/* thhip_conv2d_affine followed by a max pooling of any window (SpatialMaxPooling.c:6-98), for the layers
+ * thhip_conv2d_poolk_supported accepts: fp32 layers of a few tiles, whose K is split and whose parts a
+ * second kernel adds -- that kernel then takes the maximum of every window as well, and the pooling's
+ * own launch is saved.  y is [B][Co][pH][pW].  Replaces SpatialConvolutionMM -> Threshold ->
+ * SpatialMaxPooling; the same values, bit for bit, as the convolution followed by thhip_maxpool. */
+extern "C" void thhip_conv2d_poolk(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
+	int pkH, int pkW, int pdH, int pdW, int ppH, int ppW, int ceil_mode,
+	int act, float thr, float val, int dtype)
+{
+	if (!thhip_conv2d_poolk_supported(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, pkH, pkW, pdH, pdW, ppH, ppW, ceil_mode, dtype))
+		THError("thhip_conv2d_poolk: layer not supported (see thhip_conv2d_poolk_supported)");
+	const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
+	ConvPoolK pk = { pkH, pkW, pdH, pdW, ppH, ppW, 0, 0 };
+	thhip_pool_outsize(oH, oW, pkH, pkW, pdH, pdW, ppH, ppW, ceil_mode, &pk.oH, &pk.oW);
+	conv_run(x, wpacked, scale, shift, y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, act, thr, val, dtype, 0, 0, 0, 0, 0, &pk);
 }
 
 extern "C" void thhip_conv2d(const void *x, const void *wpacked, const float *bias, void *y,

@@ -207,13 +207,30 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 			hm->in_cl ? "channels-last" : "plane-major");
 	/* conv -> (Threshold) -> 2x2 max pooling in one kernel, where the kernel that
 	 * would run this layer can do it */
-	if (hm->pool_next && thhip_conv2d_pool2_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW,
+	const struct SpatialMaxPooling *pq = hm->pool_next ? &hn->pub.modules[hm->pool_next].SpatialMaxPooling : 0;
+	const int pool22 = pq && pq->kW == 2 && pq->kH == 2 && pq->dW == 2 && pq->dH == 2 && pq->padW == 0 && pq->padH == 0 && !pq->ceil_mode;
+	if (pool22 && thhip_conv2d_pool2_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW,
 			c->dH, c->dW, c->padH, c->padW, dt, hm->x_layout, hm->out_cl)) {
 		void *yp = conv_out(m, dt, &s, c->nOutputPlane, oH / 2, oW / 2);
 		hn->cur_cl = hm->out_cl && (oH / 2) * (oW / 2) > 1;
 		thhip_conv2d_layout_pool2(x, hm->wpacked, hm->scale, hm->bias, yp, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
 			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, hm->fused_act, hm->thr, hm->val, dt, hm->x_layout,
 			hm->out_cl);
+		hn->hm[hm->pool_next].pooled_by_producer = 1;
+		return m->output;
+	}
+	/* fp32, a layer of a few tiles (its K is split and a second kernel adds the parts): that kernel takes
+	 * a max pooling of any window as well */
+	if (pq && dt == THHIP_F32 && !hm->x_layout && !hm->out_cl && s.outnd >= 3 &&
+	    thhip_conv2d_poolk_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW, c->padH, c->padW,
+			pq->kH, pq->kW, pq->dH, pq->dW, pq->padH, pq->padW, pq->ceil_mode, dt)) {
+		int pH, pW;
+		thhip_pool_outsize(oH, oW, pq->kH, pq->kW, pq->dH, pq->dW, pq->padH, pq->padW, pq->ceil_mode, &pH, &pW);
+		void *yp = conv_out(m, dt, &s, c->nOutputPlane, pH, pW);
+		hn->cur_cl = 0;
+		thhip_conv2d_poolk(x, hm->wpacked, hm->scale, hm->bias, yp, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, pq->kH, pq->kW, pq->dH, pq->dW, pq->padH, pq->padW, pq->ceil_mode,
+			hm->fused_act, hm->thr, hm->val, dt);
 		hn->hm[hm->pool_next].pooled_by_producer = 1;
 		return m->output;
 	}
@@ -1381,6 +1398,8 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			continue;
 		const struct SpatialMaxPooling *q = &hn->pub.modules[j].SpatialMaxPooling;
 		if (q->kW == 2 && q->kH == 2 && q->dW == 2 && q->dH == 2 && q->padW == 0 && q->padH == 0 && !q->ceil_mode)
+			hn->hm[i].pool_next = j;
+		else if (dtype == THHIP_F32)	/* any window: by the kernel that adds the parts of a K split (layers of a few tiles) */
 			hn->hm[i].pool_next = j;
 	}
 	/* uint8 engine: the image layer (at most four planes, plane-major), or a convolution between
