@@ -165,6 +165,9 @@ def test_conv_f32_k_split_with_a_pooling_of_any_window(hiplib, oracle):
             assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), ((B, Ci, H, W, Co, k), int((got != ref).sum()))
             want = oracle.maxpool(np.maximum(raw, 0) if act else raw, pkH, pkW, pdH, pdW, ppH, ppW, ceil)
             G.assert_close(got, want, FP32_TOL, str((B, Ci, H, W, Co, k, d, pad)))
+    # a large layer: windows of up to four values only (four lanes per pooled value)
+    assert hiplib.thhip_conv2d_poolk_supported(16, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1, 2, 2, 2, 2, 0, 0, 0, G.F32)
+    assert not hiplib.thhip_conv2d_poolk_supported(16, 512, 14, 14, 512, 3, 3, 1, 1, 1, 1, 3, 3, 2, 2, 0, 0, 0, G.F32)
     # layers of many tiles run without a K split, the half types have their own fused poolings
     assert not hiplib.thhip_conv2d_poolk_supported(16, 64, 112, 112, 64, 3, 3, 1, 1, 1, 1, 3, 3, 2, 2, 0, 0, 0, G.F32)
     assert not hiplib.thhip_conv2d_poolk_supported(1, 64, 27, 27, 192, 5, 5, 1, 1, 2, 2, 3, 3, 2, 2, 0, 0, 0, G.F16)

@@ -2835,20 +2835,21 @@ __global__ void conv_f32_splitk_finish_kernel(const float *ws, const float *bias
 	}
 }
 
-/* The same followed by a max pooling (any window, SpatialMaxPooling.c:6-98): sixteen lanes per pooled
- * value, a lane per value of the window (lane, lane + 16, ... for larger windows).  A lane adds the
- * parts of its values and finishes them as above; the maximum is then taken over the sixteen lanes as
+/* The same followed by a max pooling (any window, SpatialMaxPooling.c:6-98): LPO (four or sixteen) lanes per
+ * pooled value, a lane per value of the window (lane, lane + LPO, ... for larger windows).  A lane adds the
+ * parts of its values and finishes them as above; the maximum is then taken over those lanes as
  * the reference's scan would: the first of equal values wins (+0 and -0), values that are not greater
  * than -FLT_MAX (NaNs) never do.  y is the pooled tensor, plane-major.  For the layers of a few tiles
  * that split K (a batch of one or a few images), where the pooling's own launch costs as much as its
  * work. */
+template <int LPO>
 __global__ __launch_bounds__(256) void conv_f32_splitk_finish_pool_kernel(const float *ws, const float *bias, const float *scale, float *y,
 	int parts, int B, int Co, int N, int oH, int oW, int act, float thr, float val,
 	int kH, int kW, int dH, int dW, int padH, int padW, int pH, int pW)
 {
 	const long total = (long)B * Co * pH * pW, part = (long)Co * N;
-	const long i = ((long)blockIdx.x * 256 + threadIdx.x) >> 4;
-	const int l = threadIdx.x & 15;
+	const long i = ((long)blockIdx.x * 256 + threadIdx.x) / LPO;
+	const int l = threadIdx.x % LPO;
 	float mx = -FLT_MAX;
 	int me = 0x7fffffff;	/* the window element mx came from */
 	if (i < total) {
@@ -2860,7 +2861,7 @@ __global__ __launch_bounds__(256) void conv_f32_splitk_finish_pool_kernel(const 
 		const int hs = py * dH - padH, wst = px * dW - padW;
 		const float sc = scale ? scale[m] : 1.0f, bi = bias ? bias[m] : 0.0f;
 		const float *src = ws + (long)m * N + (long)b * oH * oW;
-		for (int e = l; e < kH * kW; e += 16) {
+		for (int e = l; e < kH * kW; e += LPO) {
 			const int yy = hs + e / kW, xx = wst + e % kW;
 			if (yy < 0 || yy >= oH || xx < 0 || xx >= oW)
 				continue;
@@ -2879,7 +2880,7 @@ __global__ __launch_bounds__(256) void conv_f32_splitk_finish_pool_kernel(const 
 		}
 	}
 #pragma unroll
-	for (int off = 8; off > 0; off >>= 1) {
+	for (int off = LPO / 2; off > 0; off >>= 1) {
 		const float ov = __shfl_xor(mx, off, 64);
 		const int oe = __shfl_xor(me, off, 64);
 		if (ov > mx || (ov == mx && oe < me)) {
@@ -3408,12 +3409,19 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 	const size_t maxcnt = conv_tail_plan(p, resident, nkt, (size_t)BM * BN, 0);
 	conv_f32_direct_kernel<BM, BN, KCH, NST, ROWS><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
 	if (p.pk_kH) {
-		const long blocks = ((long)p.B * p.Co * p.pk_oH * p.pk_oW + 15) / 16;
+		/* four lanes per pooled value for windows of up to four values, else sixteen */
+		const int lpo = p.pk_kH * p.pk_kW <= 4 ? 4 : 16;
+		const long blocks = ((long)p.B * p.Co * p.pk_oH * p.pk_oW * lpo + 255) / 256;
 		if (blocks > 0x7fffffffL)
 			THError("thhip_conv2d: pooled output too large");
-		conv_f32_splitk_finish_pool_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
-			(float *)p.y, p.splitk, p.B, p.Co, p.N, p.oH, p.oW, p.act, p.thr, p.val,
-			p.pk_kH, p.pk_kW, p.pk_dH, p.pk_dW, p.pk_padH, p.pk_padW, p.pk_oH, p.pk_oW);
+		if (lpo == 4)
+			conv_f32_splitk_finish_pool_kernel<4><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
+				(float *)p.y, p.splitk, p.B, p.Co, p.N, p.oH, p.oW, p.act, p.thr, p.val,
+				p.pk_kH, p.pk_kW, p.pk_dH, p.pk_dW, p.pk_padH, p.pk_padW, p.pk_oH, p.pk_oW);
+		else
+			conv_f32_splitk_finish_pool_kernel<16><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
+				(float *)p.y, p.splitk, p.B, p.Co, p.N, p.oH, p.oW, p.act, p.thr, p.val,
+				p.pk_kH, p.pk_kW, p.pk_dH, p.pk_dW, p.pk_padH, p.pk_padW, p.pk_oH, p.pk_oW);
 	} else if (p.splitk > 1) {
 		long blocks = ((long)p.Co * p.N + 255) / 256;
 		if (blocks > 4096)
@@ -4203,6 +4211,11 @@ extern "C" int thhip_conv2d_poolk_supported(int B, int Ci, int H, int W, int Co,
 	if (conv_f32_split_parts(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW) < 2)
 		return 0;
 	const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
+	/* windows of more than four values: where the two launches cost more than their work only (sixteen lanes per
+	 * pooled value and every value of the convolution fetched once per window it lies in; 512->512 @14^2 at
+	 * batch 16 with a 3x3 / stride 2 window would take longer than the two kernels) */
+	if (pkH * pkW > 4 && (long)B * Co * oH * oW > (1L << 18))
+		return 0;
 	int pH, pW;
 	thhip_pool_outsize(oH, oW, pkH, pkW, pdH, pdW, ppH, ppW, ceil_mode, &pH, &pW);
 	return pH >= 1 && pW >= 1;
