@@ -1695,9 +1695,12 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_tail_finish_kernel(C
  *
  * Patch layout: 1 KiB blocks of sixteen pixels x four 16-byte vectors, pixel pp
  * of the patch (row-major, 34 wide) in block pp / 16; vector v of pixel pp sits
- * in slot 4 pp + (v ^ ((pp / 2) % 4)).  A fragment read takes one vector index
- * from 32 consecutive pixels; the swizzle spreads every run of eight over all
- * banks wherever it starts.  Pixels outside the image are fetched out of the
+ * in slot 4 pp + (v ^ ((pp / 4) % 4)).  A fragment read takes one vector index
+ * from 32 consecutive pixels, sixteen lanes (256 bytes, every bank once) a cycle;
+ * pixels four apart share their banks, and the swizzle gives any four such in a
+ * run of sixteen four different slots, wherever the run starts.  (With the key
+ * (pp / 2) % 4, which serves runs of eight, the counters showed conflicts in a
+ * tenth of the cycles.)  Pixels outside the image are fetched out of the
  * buffer's range and arrive as zeros.
  *
  * Four waves; wave w computes all BM planes of tile rows 2w and 2w+1. */
@@ -1753,7 +1756,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 #pragma unroll
 	for (int t = 0; t < BL; t++) {
 		const int pp = (wave + WAVES * t) * 16 + (lane >> 2);
-		const int v = (lane & 3) ^ ((pp >> 1) & 3);
+		const int v = (lane & 3) ^ ((pp >> 2) & 3);
 		const int pr = pp / PW, pc = pp - pr * PW;
 		const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
 		const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
@@ -1800,7 +1803,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 #pragma unroll
 		for (int j = 0; j < TN; j++) {
 			const int pp = pbase_[j] + (tap / 3) * PW + tap % 3;
-			b[j] = (buf ? patch1 : patch0)[pp * 4 + (v ^ ((pp >> 1) & 3))];
+			b[j] = (buf ? patch1 : patch0)[pp * 4 + (v ^ ((pp >> 2) & 3))];
 		}
 	};
 
