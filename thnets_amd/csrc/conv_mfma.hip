@@ -2838,6 +2838,67 @@ __global__ void conv_f32_splitk_finish_kernel(const float *ws, const float *bias
 	}
 }
 
+/* The same for layers whose positions (batch x plane size) are a multiple of four: a thread adds and
+ * finishes four neighbouring positions (16-byte reads of the parts, a quarter of the index arithmetic);
+ * the same values. */
+__global__ void conv_f32_splitk_finish4_kernel(const float *ws, const float *bias, const float *scale, float *y,
+	int parts, int Co, int N, int oHW, int act, float thr, float val, const float *res, int res_mode, float res_c, int res_act)
+{
+	const int N4 = N >> 2;
+	const long total4 = (long)Co * N4, total = (long)Co * N;
+	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+	const long step = (long)gridDim.x * blockDim.x;
+	for (; i < total4; i += step) {
+		const int m = (int)(i / N4), n = (int)(i - (long)m * N4) * 4;
+		floatx4 v = { 0, 0, 0, 0 };
+		for (int s = 0; s < parts; s++) {
+			const floatx4 w = *(const floatx4 *)(ws + (size_t)s * total + (size_t)m * N + n);
+#pragma unroll
+			for (int e = 0; e < 4; e++)
+				v[e] += w[e];
+		}
+		const float bi = bias ? bias[m] : 0.0f, sc = scale ? scale[m] : 1.0f;
+		const int b = n / oHW, rem = n - b * oHW;
+		const size_t at = ((size_t)b * Co + m) * oHW + rem;
+		/* the four lie in one image at an aligned address (always, for plane sizes that are multiples of four):
+		 * 16-byte accesses to the output (and the second tensor) too */
+		const bool together = rem + 3 < oHW && (at & 3) == 0;
+		floatx4 r = { 0, 0, 0, 0 };
+		if (res_mode) {
+			if (together)
+				r = *(const floatx4 *)(res + at);
+			else {
+#pragma unroll
+				for (int e = 0; e < 4; e++) {
+					const int ne = n + e, be = ne / oHW;
+					r[e] = res[((size_t)be * Co + m) * oHW + (ne - be * oHW)];
+				}
+			}
+		}
+#pragma unroll
+		for (int e = 0; e < 4; e++) {
+			float u = scale ? __builtin_fmaf(v[e], sc, bi) : v[e] + bi;
+			if (act)
+				u = u > thr ? u : val;
+			if (res_mode) {
+				u = res_mode == 1 ? u + res_c * r[e] : r[e] + res_c * u;
+				if (res_act)
+					u = u > 0.0f ? u : 0.0f;
+			}
+			v[e] = u;
+		}
+		if (together)
+			*(floatx4 *)(y + at) = v;
+		else {
+#pragma unroll
+			for (int e = 0; e < 4; e++) {
+				const int ne = n + e, be = ne / oHW;
+				y[((size_t)be * Co + m) * oHW + (ne - be * oHW)] = v[e];
+			}
+		}
+	}
+}
+
 /* The same followed by a max pooling (any window, SpatialMaxPooling.c:6-98): LPO (four or sixteen) lanes per
  * pooled value, a lane per value of the window (lane, lane + LPO, ... for larger windows).  A lane adds the
  * parts of its values and finishes them as above; the maximum is then taken over those lanes as
@@ -3425,6 +3486,12 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 			conv_f32_splitk_finish_pool_kernel<16><<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
 				(float *)p.y, p.splitk, p.B, p.Co, p.N, p.oH, p.oW, p.act, p.thr, p.val,
 				p.pk_kH, p.pk_kW, p.pk_dH, p.pk_dW, p.pk_padH, p.pk_padW, p.pk_oH, p.pk_oW);
+	} else if (p.splitk > 1 && p.N % 4 == 0 && ((size_t)p.y & 15) == 0 && ((size_t)p.res & 15) == 0) {
+		long blocks = ((long)p.Co * (p.N / 4) + 255) / 256;
+		if (blocks > 4096)
+			blocks = 4096;
+		conv_f32_splitk_finish4_kernel<<<dim3((unsigned)blocks), dim3(256), 0, thhip_stream()>>>((const float *)p.ws, p.bias, p.scale,
+			(float *)p.y, p.splitk, p.Co, p.N, p.oHW, p.act, p.thr, p.val, p.res, p.res_mode, p.res_c, p.res_act);
 	} else if (p.splitk > 1) {
 		long blocks = ((long)p.Co * p.N + 255) / 256;
 		if (blocks > 4096)
