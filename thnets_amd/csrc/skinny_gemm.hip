@@ -237,11 +237,15 @@ template <int DT, bool SCOPED>
 static void skinny_launch(const void *x, const void *wrow, const float *bias, void *y, float *part,
 	int B, int nIn, int nOut, int rb, int groups, int ksplit, int act, float thr, float val)
 {
-	if (ksplit == 1 && rb == 1 && B <= 16) {
+	if (ksplit == 1 && rb == 1 && B <= 32) {
 		/* a short K (fewer than sixteen K-steps), one row block per workgroup: the workgroup finishes its outputs itself */
 		ThhipLaunchScope scope(SCOPED ? THHIP_FAM_GEMV : -1, (double)thhip_esize(DT) * ((double)nOut * nIn + (double)B * nIn + (double)B * nOut));
-		skinny_kernel<DT, 1, 1, true><<<dim3(groups, 1), dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, 1,
-			bias, y, act, thr, val);
+		if (B <= 16)
+			skinny_kernel<DT, 1, 1, true><<<dim3(groups, 1), dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, 1,
+				bias, y, act, thr, val);
+		else
+			skinny_kernel<DT, 2, 1, true><<<dim3(groups, 1), dim3(SK_THREADS), 0, thhip_stream()>>>(x, wrow, part, B, nIn, nOut, 1,
+				bias, y, act, thr, val);
 		return;
 	}
 	{
