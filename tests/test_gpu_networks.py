@@ -283,6 +283,25 @@ def test_graph_form_networks(hiplib, oracle):
     net = api.HipNetwork(layers)
     G.assert_close(net.process_float(x.copy()), oracle.run_layers(layers, x).ravel(), 1e-4, "two consumers")
     net.free()
+    # a convolution (with its folded Threshold) read by a pooling and by another module: the pooling
+    # must not be taken by the convolution, whose full output the other module needs; and the same
+    # chain with the pooling as its only consumer, where it is (a layer of a few tiles: its K is split)
+    w2 = g.standard_normal((8, 64, 3, 3), dtype=np.float32) * np.float32(0.05)
+    w3 = g.standard_normal((64, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+    b64 = g.standard_normal(64, dtype=np.float32) * np.float32(0.1)
+    for shared in (1, 0):
+        layers = [dict(netbuild.conv(w3, b64, 1, 1), inputs=[]),
+                  dict(netbuild.relu(), inputs=[0]),
+                  dict(netbuild.conv(w2, b(), 1, 1), inputs=[1]),
+                  dict(netbuild.relu(), inputs=[2]),
+                  dict(netbuild.maxpool(3, 2), inputs=[3]),
+                  dict(netbuild.maxpool(3, 2), inputs=[3 if shared else 4])]
+        if shared:
+            layers.append({"type": "caddtable", "inputs": [4, 5]})
+        x = g.uniform(-1, 1, (2, 3, 13, 11)).astype(np.float32)
+        net = api.HipNetwork(layers)
+        G.assert_close(net.process_float(x.copy()), oracle.run_layers(layers, x).ravel(), 1e-4, "pooling, shared %d" % shared)
+        net.free()
 
 
 @pytest.mark.gpu

@@ -1381,8 +1381,6 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 			hn->hm[i + 1].passthrough = 1;
 		}
 	}
-#undef FEEDS_ONLY
-	free(consumers);
 	plan_channels_last(hn, net);
 	/* a 2x2 / stride 2 max pooling right after a convolution (and its folded
 	 * Threshold; half engines: between channels-last tensors) may be done by the
@@ -1391,10 +1389,13 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 		/* (fp32: plane-major tensors, the kernel that loads its tiles straight into LDS) */
 		if (!is_conv_type(hn->pub.modules[i].type) || hn->hm[i].is_linear || (dtype != THHIP_F32 && !hn->hm[i].in_cl))
 			continue;
-		int j = i + 1;
-		while (j < net->nelem && hn->hm[j].passthrough)
+		int j = i + 1, chain = FEEDS_ONLY(i, i + 1);
+		while (j < net->nelem && hn->hm[j].passthrough) {
 			j++;
-		if (j >= net->nelem || hn->pub.modules[j].type != MT_SpatialMaxPooling || hn->hm[j].want_indices)
+			chain = chain && j < net->nelem && FEEDS_ONLY(j - 1, j);
+		}
+		/* (in a graph: the pooling, through the folded modules between, is the convolution's only consumer) */
+		if (j >= net->nelem || !chain || hn->pub.modules[j].type != MT_SpatialMaxPooling || hn->hm[j].want_indices)
 			continue;
 		const struct SpatialMaxPooling *q = &hn->pub.modules[j].SpatialMaxPooling;
 		if (q->kW == 2 && q->kH == 2 && q->dW == 2 && q->dH == 2 && q->padW == 0 && q->padH == 0 && !q->ceil_mode)
@@ -1402,6 +1403,8 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 		else if (dtype == THHIP_F32)	/* any window: by the kernel that adds the parts of a K split (layers of a few tiles) */
 			hn->hm[i].pool_next = j;
 	}
+#undef FEEDS_ONLY
+	free(consumers);
 	/* uint8 engine: the image layer (at most four planes, plane-major), or a convolution between
 	 * channels-last tensors, followed by its folded Threshold and a 3x3 / stride 2 max pooling
 	 * may run as one kernel; whether it does is decided per forward by the layer's shape */
