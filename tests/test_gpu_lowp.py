@@ -501,48 +501,78 @@ def _device_codes(hiplib, net, q):
     return t, (dev, st)
 
 
-def test_alexnet_lowp_full_size_bit_exact_and_batch_property(hiplib, oracle):
-    """Configuration 5 at its real layer shapes.  Two images go through the CPU oracle
-    layer by layer (every code must match); then a batch of 64 must equal the same
-    images run in small batches with the batch's quantisation (the reference itself
-    can only run batch 1)."""
+def _fused_expectation(layers, outs, i, got_shape):
+    """What module i's buffer holds: its own codes, those of the Threshold folded into
+    it, or - when the convolution ran with its Threshold and max pooling as one kernel -
+    the pooled codes.  Returns (index into outs, fused pooling?)."""
+    j = i
+    if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold":
+        j = i + 1
+    if tuple(got_shape[1:]) != tuple(outs[j][0].shape[1:]):
+        j = next(k for k in range(i + 1, len(layers)) if layers[k]["type"] == "maxpool")
+        assert layers[i]["type"] in ("conv", "threshold") and j <= i + 2, (i, got_shape, outs[j][0].shape)
+        return j, True
+    return j, False
+
+
+def test_alexnet_lowp_full_size_bit_exact_all_64_images(hiplib, oracle):
+    """Configuration 5 at its real layer shapes and batch size.  Every code of every
+    module output of ALL 64 images is compared with the CPU oracle (run here, one
+    image at a time with the batch's quantisation, as the reference's engine has to be
+    driven) and with the committed checksums tests/golden/alexnet_lowp_b64_golden.npz;
+    the codes of the last layer also with the fixture's full copy.  Then images 0, 3,
+    40 and 63 as a batch of four must give, module by module, the same codes as their
+    rows of the batch of 64 (a result must not depend on the batch an image is in)."""
+    import os
+    import zlib
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "alexnet_lowp_b64_golden.npz"))
     cfg = configs.alexnet_lowp(batch=64)
+    layers = cfg["layers"]
     x = oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])
-    net = api.HipNetwork(cfg["layers"], lowp_range=cfg["range"])
+    net = api.HipNetwork(layers, lowp_range=cfg["range"])
     xq, im, isub = oracle.lowp_quantize(x)              # one min/max over the whole batch
+    assert (np.float32(im), np.float32(isub)) == tuple(gold["input/quant"])
     G.note("alexnet lowp b64 forward")
     t, keep = _device_codes(hiplib, net, xq)
     assert hiplib.THHipNetwork_setInputQuant(net.handle, im, isub) == 0
     hiplib.THForward(net.handle, C.addressof(t))
     last = net.nelem - 1
-    full = net.module_output(last).astype(np.uint8)
-    assert full.shape == (64, 1000, 1, 1)
-    # oracle on images 3 and 40
-    sel = [3, 40]
-    outs = []
-    q, m, s = oracle.lowp_run_layers(cfg["layers"], xq[sel], im, isub, cfg["range"], collect=outs)
-    assert np.array_equal(full[sel], q)
-    G.note("alexnet lowp b2 forward")
+    got64 = [net.module_output(i).astype(np.uint8) for i in range(net.nelem)]
+    assert got64[last].shape == (64, 1000, 1, 1)
+    # the oracle on all 64 images, eight at a time
+    parts = []
+    for b0 in range(0, 64, 8):
+        outs = []
+        oracle.lowp_run_layers(layers, xq[b0:b0 + 8], im, isub, cfg["range"], collect=outs)
+        parts.append(outs)
+    outs = [(np.concatenate([p[i][0] for p in parts]), parts[0][i][1], parts[0][i][2]) for i in range(len(layers))]
+    fused_pool = False
+    images_checked = np.zeros(64, bool)
+    for i in range(len(layers)):
+        j, fused = _fused_expectation(layers, outs, i, got64[i].shape)
+        fused_pool |= fused
+        want = outs[j][0]
+        differ = (got64[i] != want).reshape(64, -1).sum(axis=1)
+        assert not differ.any(), "module %d (%s): images %s differ in %d codes" % (
+            i, layers[i]["type"], np.flatnonzero(differ).tolist(), differ.sum())
+        # the committed fixture, image by image
+        crc = np.array([zlib.crc32(got64[i][b].tobytes()) for b in range(64)], np.uint32)
+        assert np.array_equal(crc, gold["module%d/crc" % j]), (i, np.flatnonzero(crc != gold["module%d/crc" % j]))
+        assert np.array_equal(got64[i].reshape(64, -1).sum(axis=1, dtype=np.int64), gold["module%d/sum" % j])
+        assert net.module_quant(i) == (np.float32(outs[i][1]), np.float32(outs[i][2])) == tuple(gold["module%d/quant" % i])
+        images_checked |= ~differ.astype(bool)
+    assert images_checked.all() and images_checked.size == 64
+    assert np.array_equal(got64[last].reshape(64, -1), gold["last/codes"])
+    assert fused_pool, "the image layer of AlexNet should take the fused convolution + pooling kernel"
+    # the logits carry information (not saturated everywhere)
+    assert len(np.unique(got64[last])) > 20
+    # the same images in a small batch: the same codes
+    sel = [0, 3, 40, 63]
+    G.note("alexnet lowp b4 forward")
     t2, keep2 = _device_codes(hiplib, net, xq[sel])
     hiplib.THHipNetwork_setInputQuant(net.handle, im, isub)
     hiplib.THForward(net.handle, C.addressof(t2))
-    layers = cfg["layers"]
-    fused_pool = False
-    for i, (qo, mo, so) in enumerate(outs):
-        want = qo
-        if i + 1 < len(layers) and layers[i + 1]["type"] == "threshold":
-            want = outs[i + 1][0]
+    for i in range(len(layers)):
         got = net.module_output(i).astype(np.uint8)
-        if got.shape != want.shape:
-            # the image layer ran with its Threshold and max pooling in one kernel: its buffer
-            # (and the Threshold's view of it) holds the pooled codes
-            j = next(k for k in range(i + 1, len(layers)) if layers[k]["type"] == "maxpool")
-            assert layers[i]["type"] in ("conv", "threshold") and j <= i + 2, (i, got.shape, want.shape)
-            want = outs[j][0]
-            fused_pool = True
-        assert np.array_equal(got, want), "module %d (%s): %d codes differ" % (i, layers[i]["type"], (got != want).sum())
-        assert net.module_quant(i) == (np.float32(mo), np.float32(so))
-    assert fused_pool, "the image layer of AlexNet should take the fused convolution + pooling kernel"
-    # the logits carry information (not saturated everywhere)
-    assert len(np.unique(q)) > 20
+        assert np.array_equal(got, got64[i][sel]), "module %d: a batch of 4 and a batch of 64 differ" % i
     net.free()

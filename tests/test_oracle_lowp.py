@@ -265,3 +265,35 @@ def test_network_executor_matches_layerwise_fp32(oracle):
     relu_code = oracle.lowp_scale_float(m, s, 0.0)
     assert outs[1][0].min() >= relu_code and q.min() >= relu_code
     assert np.array_equal(outs[2][0], oracle.lowp_maxpool(outs[1][0], 2, 2, 2, 2))
+
+
+def test_alexnet_lowp_b64_fixture(oracle):
+    """Configuration 5, all 64 images: the oracle reproduces the committed fixture
+    (checksums per module and image, the last layer's codes in full), and what the
+    codes say is the network's answer: de-quantised, the last layer's codes follow
+    the fp32 network on the same images (correlation > 0.99; they cannot be equal -
+    range 32 saturates at +-16 where the fp32 values reach 20)."""
+    import os
+    import zlib
+    from thnets_amd import configs
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "alexnet_lowp_b64_golden.npz"))
+    cfg = configs.alexnet_lowp(batch=64)
+    layers = cfg["layers"]
+    x = oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])
+    xq, im, isub = oracle.lowp_quantize(x)
+    assert (np.float32(im), np.float32(isub)) == tuple(gold["input/quant"])
+    assert np.array_equal(np.array([zlib.crc32(xq[b].tobytes()) for b in range(64)], np.uint32), gold["input/crc"])
+    last = len(layers) - 1
+    for b0 in range(0, 64, 8):
+        outs = []
+        q, m, s = oracle.lowp_run_layers(layers, xq[b0:b0 + 8], im, isub, cfg["range"], collect=outs)
+        for i, (qi, mi, si) in enumerate(outs):
+            crc = np.array([zlib.crc32(qi[b].tobytes()) for b in range(8)], np.uint32)
+            assert np.array_equal(crc, gold["module%d/crc" % i][b0:b0 + 8]), (i, b0)
+            assert (np.float32(mi), np.float32(si)) == tuple(gold["module%d/quant" % i])
+        assert np.array_equal(q.reshape(8, -1), gold["last/codes"][b0:b0 + 8])
+    sel = [0, 21, 42, 63]
+    yf = oracle.run_layers(layers, x[sel]).reshape(4, -1)
+    yd = oracle.lowp_dequantize(gold["last/codes"][sel], *gold["module%d/quant" % last])
+    for b in range(4):
+        assert np.corrcoef(yf[b], yd[b])[0, 1] > 0.99
