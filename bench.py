@@ -8,7 +8,8 @@ value is whole-job images/second.  The same run also measures the convolution ke
 family with HIP events around every launch inside the timed region (-> "roofline"),
 times the same network through THProcessFloat call by call as the reference's CLI does
 (-> "process_float": best and mean of at least 20 calls after 2 warm-ups, host
-transfers included), times the uint8 AlexNet-OWT batch-64 network (-> "roofline_int8"
+transfers included), THProcessImages on 64 8-bit images beside the same batch as
+floats (-> "process_images"), times the uint8 AlexNet-OWT batch-64 network (-> "roofline_int8"
 and "extra"), the fp16 VGG-16, AlexNet-OWT batch 1 and ResNet-18 networks (-> "extra"),
 what the matrix cores sustain from registers alone (-> "extra"), and the CPU baseline
 on the host cores (-> "cpu_baseline": the reference's own CPU library when oracle/_ref
@@ -306,6 +307,40 @@ def main():
                                  "constructions); parity is against this repository's restatement, image by image"}
         n5.free()
 
+    # ---- THProcessImages on the device: 64 interleaved 8-bit 224 x 224 x 3 images cross the link as bytes and become
+    # normalised planes (float engines) or codes (uint8 engine) there (thapi.c:452-563); beside it the same batch as
+    # floats through THProcessFloat (four times the bytes, normalised by the call) ----
+    process_images = None
+    if not args.no_int8:
+        g = np.random.Generator(np.random.PCG64(77))
+        imgs = [np.ascontiguousarray(g.integers(0, 256, (224, 224, 3), dtype=np.uint8)) for _ in range(64)]
+        ptrs = (C.c_void_p * 64)(*[im.ctypes.data for im in imgs])
+        xf = np.ascontiguousarray(np.stack(imgs).transpose(0, 3, 1, 2).astype(np.float32) / np.float32(255))
+        c6 = configs.alexnet_lowp(batch=1)        # AlexNet-OWT, THMakeSpatial form, no SoftMax
+        process_images = {"workload": "AlexNet-OWT shape, batch 64 of 224x224x3 8-bit images; best / mean images/s of 10 "
+                                      "calls after 2 warm-ups, host transfers included"}
+        res, ow, oh = C.POINTER(C.c_float)(), C.c_int(), C.c_int()
+        for name, kw in (("fp32", {}), ("uint8", {"lowp_range": c6["range"]})):
+            n6 = api.HipNetwork(c6["layers"], c6["mean"], c6["std"], **kw)
+            t_img, t_flt = [], []
+            for i in range(12):
+                t0 = time.perf_counter()
+                lib.THProcessImages(n6.handle, ptrs, 64, 224, 224, 672, C.byref(res), C.byref(ow), C.byref(oh), 0)
+                if i >= 2:
+                    t_img.append(time.perf_counter() - t0)
+            for i in range(12):
+                x = np.array(xf, np.float32, copy=True, order="C")
+                t0 = time.perf_counter()
+                lib.THProcessFloat(n6.handle, x.ctypes.data, 64, 224, 224, 3, C.byref(res), C.byref(ow), C.byref(oh))
+                if i >= 2:
+                    t_flt.append(time.perf_counter() - t0)
+            process_images[name] = {
+                "THProcessImages_images_per_sec_best": round(64.0 / min(t_img), 1),
+                "THProcessImages_images_per_sec_mean": round(64.0 * len(t_img) / sum(t_img), 1),
+                "THProcessFloat_images_per_sec_best": round(64.0 / min(t_flt), 1),
+                "THProcessFloat_images_per_sec_mean": round(64.0 * len(t_flt) / sum(t_flt), 1)}
+            n6.free()
+
     # ---- what the matrix cores sustain from registers alone on this device (no memory traffic), for scale ----
     extra["mfma_register_loop"] = {
         "fp32_32x32x2_TFLOP/s_by_waves_per_simd": {str(w): round(lib.thhip_probe_mfma(0, w, 30.0) / 1e12, 1) for w in (1, 2, 3, 4)},
@@ -327,7 +362,7 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "VGG-16 shape, fp32, batch 16, 3x224x224, THForward with the input resident in HBM "
                                "(BASELINE configs[2])", "batch": 16},
-        "roofline": roofline, "cpu_baseline": cpu, "process_float": process_float, "roofline_int8": roofline_int8,
+        "roofline": roofline, "cpu_baseline": cpu, "process_float": process_float, "process_images": process_images, "roofline_int8": roofline_int8,
         "extra": extra,
     }
     print(json.dumps(line))

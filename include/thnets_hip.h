@@ -389,7 +389,19 @@ void thhip_free(void *p);
 void thhip_memcpy_h2d(void *dst, const void *src, size_t bytes);
 void thhip_memcpy_d2h(void *dst, const void *src, size_t bytes);
 void thhip_memcpy_d2d(void *dst, const void *src, size_t bytes);
+/* Page-locked host memory and copies that are queued on the engine's stream
+ * without waiting for them (the host side must be such memory); what the
+ * ENGINE_HIP branches of THProcessFloat / THProcessImages stage their data
+ * through (the CUDA engine copies from pageable memory, cudnn_basic.c:64-80). */
+void *thhip_host_malloc(size_t bytes);
+void thhip_host_free(void *p);
+void thhip_memcpy_h2d_async(void *dst, const void *src_pinned, size_t bytes);
+void thhip_memcpy_d2h_async(void *dst_pinned, const void *src, size_t bytes);
 void thhip_memset(void *dst, int value, size_t bytes);
+/* How many allocating requests (device or page-locked memory taken or given
+ * back, events created) the library has made of the HIP runtime so far: a test
+ * aid for the entry point that promises none. */
+long thhip_alloc_calls(void);
 void thhip_sync(void);
 /* Events on the engine's stream: slots 0..63. thhip_event_ms(a,b) syncs b. */
 void thhip_event_record(int slot);
@@ -661,6 +673,11 @@ void thhip_normalize(const float *src, void *dst, int B, int C, long HW, const f
  * bytes per row, cp planes) -> normalised planar dst in `dtype`. */
 void thhip_rgb2float(void *dst, const unsigned char *src, int width, int height, int stride, int cp,
 	const float *mean, const float *std, int bgr, int dtype);
+/* The loop over the images of THProcessImages (thapi.c:489-496, 509-515) as one
+ * launch: n images, `src_pitch` bytes apart in src, -> n consecutive planar
+ * tensors in dst. */
+void thhip_rgb2float_batch(void *dst, const unsigned char *src, int n, long src_pitch, int width, int height,
+	int stride, int cp, const float *mean, const float *std, int bgr, int dtype);
 
 /* ---- uint8 (LOWP) path ---- */
 
@@ -789,6 +806,9 @@ void thhip_linear_batched_u8(const unsigned char *x, const unsigned char *wfrag,
  * mean / std; (*mult, *sub) receive that range's quantisation. */
 void thhip_rgb2code(unsigned char *dst, const unsigned char *src_dev, int width, int height, int stride,
 	const float *mean, const float *std, int bgr, float *mult, float *sub);
+/* All n images of Lowp_LoadImages' loop (lowp_basic.c:113-130) in one launch. */
+void thhip_rgb2code_batch(unsigned char *dst, const unsigned char *src_dev, int n, long src_pitch, int width,
+	int height, int stride, const float *mean, const float *std, int bgr, float *mult, float *sub);
 
 /* Replaces Lowp_Threshold_updateOutput (lowp_Threshold.c:3-28) on codes. */
 void thhip_threshold_u8(const unsigned char *x, unsigned char *y, long n, int thr, int val, int inplace);

@@ -84,24 +84,86 @@ def test_golden_layout_is_current_when_reference_is_mounted(tmp_path):
     assert mod.probe(ref, ["-DLOWP"]) == GOLDEN["lowp"]
 
 
+def _object_lists():
+    """The object lists INTEGRATION.md gives a thnets maintainer: the HIP=1 block of the
+    Makefile fragment, and the objects that stand in for gemm8.o under LOWP=1."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    m = re.search(r"LIBOBJS \+= ((?:\w+\.o ?)+)", text)
+    engine = m.group(1).split()
+    m = re.search(r"link `((?:\w+\.o ?)+)` instead", text)
+    lowpgemm = m.group(1).split()
+    return engine, lowpgemm
+
+
+def _nm(path, undefined):
+    out = subprocess.check_output(["nm", "-u" if undefined else "--defined-only", path]).decode()
+    return set(line.split()[-1] for line in out.splitlines() if line.strip())
+
+
+# what the system provides: libc / libm / libstdc++ / compiler runtime / the HIP runtime
+SYSTEM = re.compile(r"^(GOMP_|omp_|hip[A-Z]|__hip|_Z(?!\d+thhip)|__cxa|__gxx|_Unwind|__stack_chk|__dso_handle|_GLOBAL_|__truncsfhf2|"
+                    r"__extendhfsf2|mem(cpy|set|move)$|__mem\w+_chk|malloc$|calloc$|realloc$|free$|exit$|abort$|atexit$|"
+                    r"f?printf$|__\w*printf_chk|v?fprintf$|snprintf$|fputs$|fputc$|fwrite$|fflush$|puts$|stderr$|stdout$|"
+                    r"getenv$|atoi$|strcmp$|strlen$|qsort$|clock_gettime$|log$|logf$|sqrt$|sqrtf$|roundf$|floorf$|ceilf$|"
+                    r"expf$|fmaxf$|fminf$)")
+
+
+def test_makefile_and_integration_name_the_same_kernel_objects():
+    mk = open(os.path.join(ROOT, "thnets_amd", "csrc", "Makefile")).read()
+    hip_srcs = re.search(r"^HIP_SRCS = (.*)$", mk, flags=re.M).group(1).split()
+    engine, _ = _object_lists()
+    assert sorted(o for o in engine if o not in ("th_engine.o", "th_io.o")) == sorted(f[:-4] + ".o" for f in hip_srcs)
+
+
 @pytest.mark.parametrize("flags", [[], ["-DLOWP"]])
-def test_engine_compiles_against_the_reference_header(tmp_path, flags):
-    """With -DTHNETS_IN_TREE the engine's host code takes every structure, module type and
-    tensor helper from the reference's own thnets.h (the way its objects are linked into
-    libthnets with the Makefile's HIP=1 option) instead of this repository's mirror: it must
-    compile, warning-free, against the unmodified header, in the default and the -DLOWP
-    layout; so must a kernel file's host side."""
+def test_in_tree_object_list_links(tmp_path, flags):
+    """The engine as a thnets maintainer would link it (Makefile's HIP=1 option modelled on
+    Makefile:152-178): th_engine.c and th_io.c compile with -DTHNETS_IN_TREE, warning-free,
+    with the reference's flags (-Wall -fopenmp, Makefile:28) against its own unmodified thnets.h (default and -DLOWP layout), and the
+    object list INTEGRATION.md gives is closed - every symbol those objects leave undefined
+    is defined by another of them, by the reference's library (tensor helpers, THError) or
+    by the system.  The same for the objects that replace gemm8.o (lowpgemm,
+    lowp_basic.c:290-297).  The kernel objects are the ones the library was built from."""
     ref = "/root/reference"
     if not os.path.exists(os.path.join(ref, "thnets.h")):
         pytest.skip("reference tree not mounted")
     csrc = os.path.join(ROOT, "thnets_amd", "csrc")
-    r = subprocess.run(["gcc", "-std=gnu11", "-Wall", "-Werror", "-Wno-unused-function", "-c", "-DTHNETS_IN_TREE"] + flags +
-                       ["-I", ref, os.path.join(csrc, "th_engine.c"), "-o", str(tmp_path / "th_engine.o")],
-                       capture_output=True, text=True)
-    assert r.returncode == 0, r.stderr
-    # the object refers to the reference's tensor helpers and to the kernel launchers only
-    syms = subprocess.check_output(["nm", "-u", str(tmp_path / "th_engine.o")]).decode()
-    assert "THFloatTensor_set" in syms and "thhip_conv2d_layout" in syms
+    engine, lowpgemm = _object_lists()
+    assert "th_engine.o" in engine and "th_io.o" in engine and len(engine) == 10
+    paths = {}
+    for o in engine:
+        src = os.path.join(csrc, o[:-2] + ".c")
+        if os.path.exists(src):
+            paths[o] = str(tmp_path / o)
+            r = subprocess.run(["gcc", "-std=gnu11", "-Wall", "-Werror", "-Wno-unused-function", "-fopenmp", "-c",
+                                "-DTHNETS_IN_TREE"] + flags + ["-I", ref, src, "-o", paths[o]], capture_output=True, text=True)
+            assert r.returncode == 0, r.stderr
+        else:
+            assert os.path.exists(os.path.join(csrc, o[:-2] + ".hip")), o
+            paths[o] = os.path.join(csrc, "build", o)
+            if not os.path.exists(paths[o]):
+                pytest.fail("%s missing: build the library first (python __graft_entry__.py)" % paths[o])
+    reflib = os.path.join(ROOT, "oracle", "_ref", "libthnets_ref_lowp.so" if flags else "libthnets_ref.so")
+    if not os.path.exists(reflib):
+        pytest.skip("oracle/_ref not built")
+    provided = _nm(reflib, False)
+    for objs, must_define in ((engine, ["THHip_ToHip", "thhip_forward", "thhip_process_float", "thhip_process_images",
+                                        "THHipTensor_newFromFloatTensor", "THFloatTensor_newFromHipTensor",
+                                        "thhip_free_network", "thhip_free"]),
+                              (lowpgemm, ["lowpgemm"])):
+        defined, undefined = set(), set()
+        for o in objs:
+            defined |= _nm(paths[o], False)
+            undefined |= _nm(paths[o], True)
+        for name in must_define:
+            assert name in defined, name
+        open_ = sorted(u for u in undefined - defined if not SYSTEM.match(u))
+        missing = [u for u in open_ if u not in provided]
+        assert not missing, "%s leave undefined: %s" % (objs, missing)
+        # what does come from the reference's library are its tensor helpers and THError
+        assert all(u.startswith("TH") for u in open_), open_
+    # nothing of the stand-alone host files is needed
+    assert "th_api.o" not in engine and "th_tensor.o" not in engine
 
 
 def declared_functions():

@@ -147,7 +147,12 @@ def test_minmax_kernel(hiplib):
     hiplib.thhip_minmax(d.ptr, q.size, G.U8, C.byref(mn), C.byref(mx))
     assert (mn.value, mx.value) == (float(q.min()), float(q.max()))
     hiplib.thhip_minmax(d.ptr, 0, G.F32, C.byref(mn), C.byref(mx))
-    assert mn.value == np.inf and mx.value == -np.inf      # THInf / -THInf, thapi.c:143-144
+    fmax = float(np.finfo(np.float32).max)
+    assert mn.value == fmax and mx.value == -fmax      # THInf / -THInf (FLT_MAX, thnets.h:463), thapi.c:143-144
+    # values beyond +-FLT_MAX do not move the seeds either (`data[i] > *max` is false for -inf ... FLT_MAX)
+    d = api.DeviceArray(hiplib, np.array([-np.inf, -np.inf], np.float32))
+    hiplib.thhip_minmax(d.ptr, 2, G.F32, C.byref(mn), C.byref(mx))
+    assert mn.value == -np.inf and mx.value == -fmax
 
 
 def test_th_minmax_prints_every_layer(hiplib, oracle):

@@ -27,8 +27,17 @@ def both(lib, oracle, B, nIn, nOut, act, dtype, seed, tol):
     lib.thhip_memset(dy0.ptr, 0xFF, B * nOut * es)
     lib.thhip_memset(dy1.ptr, 0xFF, B * nOut * es)
     lib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy0.ptr, B, nIn, nOut, act, 0.1, -0.5, dtype)
-    rc = lib.thhip_linear_batched_noalloc(dx.ptr, dw.ptr, db.ptr, dy1.ptr, B, nIn, nOut, act, 0.1, -0.5, dtype)
-    assert rc == 0
+    # the property the entry point is named for: not one allocating request (device or page-locked
+    # memory, events) reaches the HIP runtime during the call, with the per-launch profiler off and on
+    for prof in (0, 1):
+        lib.thhip_profile_enable(prof)
+        if prof:        # the profiler's event pool fills on first use; the library's own calls may allocate
+            lib.thhip_linear_batched(dx.ptr, dw.ptr, db.ptr, dy0.ptr, B, nIn, nOut, act, 0.1, -0.5, dtype)
+        before = lib.thhip_alloc_calls()
+        rc = lib.thhip_linear_batched_noalloc(dx.ptr, dw.ptr, db.ptr, dy1.ptr, B, nIn, nOut, act, 0.1, -0.5, dtype)
+        assert rc == 0
+        assert lib.thhip_alloc_calls() == before, "thhip_linear_batched_noalloc allocated (profiling %d)" % prof
+    lib.thhip_profile_enable(0)
     lib.thhip_sync()
     want = api.from_device_dtype(dy0, (B, nOut), dtype)
     got = api.from_device_dtype(dy1, (B, nOut), dtype)

@@ -70,6 +70,11 @@ PROTOTYPES = {
     "thhip_memcpy_h2d": (None, [vp, vp, C.c_size_t]),
     "thhip_memcpy_d2h": (None, [vp, vp, C.c_size_t]),
     "thhip_memcpy_d2d": (None, [vp, vp, C.c_size_t]),
+    "thhip_alloc_calls": (C.c_long, []),
+    "thhip_host_malloc": (vp, [C.c_size_t]),
+    "thhip_host_free": (None, [vp]),
+    "thhip_memcpy_h2d_async": (None, [vp, vp, C.c_size_t]),
+    "thhip_memcpy_d2h_async": (None, [vp, vp, C.c_size_t]),
     "thhip_memset": (None, [vp, C.c_int, C.c_size_t]),
     "thhip_sync": (None, []),
     "thhip_event_record": (None, [C.c_int]),
@@ -115,6 +120,7 @@ PROTOTYPES = {
     "thhip_axpby2": (None, [vp, vp, vp, C.c_long, C.c_long, C.c_float, C.c_int, C.c_int]),
     "thhip_convert": (None, [vp, C.c_int, vp, C.c_int, C.c_long]),
     "thhip_rgb2float": (None, [vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, C.c_int]),
+    "thhip_rgb2float_batch": (None, [vp, vp, C.c_int, C.c_long, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, C.c_int]),
     "thhip_quantize": (None, [vp, vp, C.c_long, c_fp, c_fp]),
     "thhip_dequantize": (None, [vp, vp, C.c_long, C.c_float, C.c_float]),
     "thhip_conv_pack_weight_u8": (vp, [vp, C.c_int, C.c_int, C.c_int]),
@@ -141,6 +147,7 @@ PROTOTYPES = {
     "thhip_linear_pack_weight_u8": (vp, [vp, C.c_int, C.c_int]),
     "thhip_linear_batched_u8": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 3 + [C.c_int] * 5 + [C.c_int] * 3),
     "thhip_rgb2code": (None, [vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, c_fp, c_fp]),
+    "thhip_rgb2code_batch": (None, [vp, vp, C.c_int, C.c_long, C.c_int, C.c_int, C.c_int, vp, vp, C.c_int, c_fp, c_fp]),
     "thhip_threshold_u8": (None, [vp, vp, C.c_long, C.c_int, C.c_int, C.c_int]),
     "thhip_softmax_u8": (C.c_float, [vp, vp, C.c_long, C.c_long, C.c_long, C.c_float, C.c_float]),
 }

@@ -991,10 +991,12 @@ extern "C" void thhip_normalize(const float *src, void *dst, int B, int C, long 
 /* ---------------- 8-bit image -> normalised planar float (thapi.c:20-46) ---------------- */
 
 template <int DT>
-__global__ void rgb2float_kernel(void *dst, const unsigned char *src, int width, int height, int stride, int cp,
+__global__ void rgb2float_kernel(void *dst, const unsigned char *src, long src_pitch, int width, int height, int stride, int cp,
 	floatx4 mean, floatx4 std1, int bgr)
 {
 	const long total = (long)cp * width * height;
+	src += src_pitch * blockIdx.y;		/* one image per blockIdx.y */
+	dst = (char *)dst + (long)blockIdx.y * total * (DT == THHIP_F32 ? 4 : 2);
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
 	const long step = (long)gridDim.x * blockDim.x;
 	for (; i < total; i += step) {
@@ -1010,28 +1012,41 @@ __global__ void rgb2float_kernel(void *dst, const unsigned char *src, int width,
 	}
 }
 
-extern "C" void thhip_rgb2float(void *dst, const unsigned char *src, int width, int height, int stride, int cp,
-	const float *mean, const float *std, int bgr, int dtype)
+/* n images, `src_pitch` bytes apart in src, become n consecutive [cp][height][width] tensors in dst */
+extern "C" void thhip_rgb2float_batch(void *dst, const unsigned char *src, int n, long src_pitch, int width, int height,
+	int stride, int cp, const float *mean, const float *std, int bgr, int dtype)
 {
 	if (cp < 1 || cp > 3)
 		THError("thhip_rgb2float: %d colour planes", cp);
+	if (n < 1 || n > 65535)
+		THError("thhip_rgb2float: %d images", n);
 	floatx4 m = { 0, 0, 0, 0 }, s = { 1, 1, 1, 1 };
 	for (int i = 0; i < cp; i++) {
 		m[i] = mean[i];
 		s[i] = 1 / std[i];
 	}
 	const long total = (long)cp * width * height;
-	ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)total * (1 + thhip_esize(dtype)));
-	THHIP_DISPATCH_FLOAT(dtype, (rgb2float_kernel<DT><<<ew_grid(total), dim3(EW_THREADS), 0, thhip_stream()>>>(
-		dst, src, width, height, stride, cp, m, s, bgr)));
+	ThhipLaunchScope scope(THHIP_FAM_OTHER, (double)n * total * (1 + thhip_esize(dtype)));
+	dim3 grid = ew_grid(total, 4);
+	grid.y = n;
+	THHIP_DISPATCH_FLOAT(dtype, (rgb2float_kernel<DT><<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(
+		dst, src, src_pitch, width, height, stride, cp, m, s, bgr)));
+}
+
+extern "C" void thhip_rgb2float(void *dst, const unsigned char *src, int width, int height, int stride, int cp,
+	const float *mean, const float *std, int bgr, int dtype)
+{
+	thhip_rgb2float_batch(dst, src, 1, 0, width, height, stride, cp, mean, std, bgr, dtype);
 }
 
 /* ---------------- 8-bit image -> planar uint8 codes (lowp/lowp_basic.c:60-131) ---------------- */
 
-__global__ void rgb2code_kernel(unsigned char *dst, const unsigned char *src, int width, int height, int stride,
+__global__ void rgb2code_kernel(unsigned char *dst, const unsigned char *src, long src_pitch, int width, int height, int stride,
 	int sub0, int sub1, int sub2, float mult0, float mult1, float mult2, int bgr)
 {
 	const long total = 3L * width * height;
+	src += src_pitch * blockIdx.y;		/* one image per blockIdx.y */
+	dst += total * blockIdx.y;
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
 	const long step = (long)gridDim.x * blockDim.x;
 	for (; i < total; i += step) {
@@ -1054,9 +1069,11 @@ __global__ void rgb2code_kernel(unsigned char *dst, const unsigned char *src, in
  * derived from mean / std gives the tensor's (mult, sub), returned through the
  * pointers, and per-plane integer offsets and factors.  src is a device copy
  * of the interleaved 8-bit image. */
-extern "C" void thhip_rgb2code(unsigned char *dst, const unsigned char *src, int width, int height, int stride,
-	const float *mean, const float *std, int bgr, float *mult_out, float *sub_out)
+extern "C" void thhip_rgb2code_batch(unsigned char *dst, const unsigned char *src, int n, long src_pitch, int width,
+	int height, int stride, const float *mean, const float *std, int bgr, float *mult_out, float *sub_out)
 {
+	if (n < 1 || n > 65535)
+		THError("thhip_rgb2code: %d images", n);
 	int sub[3];
 	float mult[3], mn = 1e30, mx = -1e30, tmult;
 	/* the kernel reads three bytes of every pixel: the source must hold
@@ -1080,12 +1097,20 @@ extern "C" void thhip_rgb2code(unsigned char *dst, const unsigned char *src, int
 	}
 	const long total = 3L * width * height;
 	if (total > 0) {
-		ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * total);
-		rgb2code_kernel<<<ew_grid(total), dim3(EW_THREADS), 0, thhip_stream()>>>(dst, src, width, height, stride,
+		ThhipLaunchScope scope(THHIP_FAM_OTHER, 2.0 * n * total);
+		dim3 grid = ew_grid(total, 4);
+		grid.y = n;
+		rgb2code_kernel<<<grid, dim3(EW_THREADS), 0, thhip_stream()>>>(dst, src, src_pitch, width, height, stride,
 			sub[0], sub[1], sub[2], mult[0], mult[1], mult[2], bgr);
 	}
 	*mult_out = tmult;
 	*sub_out = mn;
+}
+
+extern "C" void thhip_rgb2code(unsigned char *dst, const unsigned char *src, int width, int height, int stride,
+	const float *mean, const float *std, int bgr, float *mult_out, float *sub_out)
+{
+	thhip_rgb2code_batch(dst, src, 1, 0, width, height, stride, mean, std, bgr, mult_out, sub_out);
 }
 
 /* ---------------- smallest and largest element (FindMinMax, thapi.c:141-154) ---------------- */
@@ -1095,7 +1120,7 @@ __global__ void minmax_any_kernel(const void *x, long n, float *part)
 {
 	long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
 	const long step = (long)gridDim.x * blockDim.x;
-	float mn = INFINITY, mx = -INFINITY;	/* THInf / -THInf; comparisons skip NaN like the reference's */
+	float mn = FLT_MAX, mx = -FLT_MAX;	/* THInf / -THInf (thnets.h:463: FLT_MAX); comparisons skip NaN like the reference's */
 	for (; i < n; i += step) {
 		float v;
 		if constexpr (DT == THHIP_U8)
@@ -1128,7 +1153,7 @@ __global__ void minmax_any_kernel(const void *x, long n, float *part)
 
 extern "C" void thhip_minmax(const void *x, long n, int dtype, float *min_out, float *max_out)
 {
-	float mn = INFINITY, mx = -INFINITY;
+	float mn = FLT_MAX, mx = -FLT_MAX;	/* THInf, thnets.h:463; an empty tensor returns them as they are */
 	if (n > 0) {
 		long blocks = (n + 1023) / 1024;
 		if (blocks > 1024)

@@ -43,20 +43,33 @@ extern "C" int thhip_device_count(void)
 	return n;
 }
 
+/* How often this library has asked the runtime for something that allocates: device and
+ * page-locked memory (taken or given back) and events.  A call that promises to allocate
+ * nothing leaves it unchanged. */
+static long g_alloc_calls;
+
+extern "C" long thhip_alloc_calls(void)
+{
+	return g_alloc_calls;
+}
+
 extern "C" void *thhip_malloc(size_t bytes)
 {
 	void *p = 0;
 	thhip_init_once();
 	if (bytes == 0)
 		bytes = 4;
+	++g_alloc_calls;
 	hipcheck(hipMalloc(&p, bytes));
 	return p;
 }
 
 extern "C" void thhip_free(void *p)
 {
-	if (p)
+	if (p) {
+		++g_alloc_calls;
 		hipcheck(hipFree(p));
+	}
 }
 
 extern "C" void thhip_memcpy_h2d(void *dst, const void *src, size_t bytes)
@@ -69,6 +82,35 @@ extern "C" void thhip_memcpy_d2h(void *dst, const void *src, size_t bytes)
 {
 	hipcheck(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, thhip_stream()));
 	hipcheck(hipStreamSynchronize(thhip_stream()));
+}
+
+/* Page-locked host memory: copies to and from it run at the link's rate and, queued with the
+ * two calls below, return before they have finished. */
+extern "C" void *thhip_host_malloc(size_t bytes)
+{
+	void *p = 0;
+	thhip_init_once();
+	++g_alloc_calls;
+	hipcheck(hipHostMalloc(&p, bytes ? bytes : 4, hipHostMallocDefault));
+	return p;
+}
+
+extern "C" void thhip_host_free(void *p)
+{
+	if (p) {
+		++g_alloc_calls;
+		hipcheck(hipHostFree(p));
+	}
+}
+
+extern "C" void thhip_memcpy_h2d_async(void *dst, const void *src_pinned, size_t bytes)
+{
+	hipcheck(hipMemcpyAsync(dst, src_pinned, bytes, hipMemcpyHostToDevice, thhip_stream()));
+}
+
+extern "C" void thhip_memcpy_d2h_async(void *dst_pinned, const void *src, size_t bytes)
+{
+	hipcheck(hipMemcpyAsync(dst_pinned, src, bytes, hipMemcpyDeviceToHost, thhip_stream()));
 }
 
 extern "C" void thhip_memcpy_d2d(void *dst, const void *src, size_t bytes)
@@ -107,8 +149,10 @@ extern "C" void thhip_event_record(int slot)
 {
 	if (slot < 0 || slot >= THHIP_NSLOTS)
 		THError("thhip_event_record: slot %d out of range", slot);
-	if (!g_slots[slot])
+	if (!g_slots[slot]) {
+		++g_alloc_calls;
 		hipcheck(hipEventCreate(&g_slots[slot]));
+	}
 	hipcheck(hipEventRecord(g_slots[slot], thhip_stream()));
 }
 
@@ -144,6 +188,7 @@ static hipEvent_t prof_event(void)
 		g_evpool.pop_back();
 		return e;
 	}
+	++g_alloc_calls;
 	hipcheck(hipEventCreate(&e));
 	return e;
 }
@@ -327,20 +372,24 @@ extern "C" double thhip_probe_mfma(int dtype, int waves_per_simd, double ms)
 	thhip_memcpy_h2d(in, host, sizeof(host));
 	const double per_mfma = dtype == THHIP_F32 ? 4096.0 : dtype == THHIP_F16 ? 32768.0 : 65536.0;
 	hipEvent_t e0, e1;
+	++g_alloc_calls;
 	hipcheck(hipEventCreate(&e0));
+	++g_alloc_calls;
 	hipcheck(hipEventCreate(&e1));
 	double rate = 0;
 	int iters = 64;
 	for (int pass = 0; pass < 2; pass++) {	/* a short run sizes the long one */
-		hipcheck(hipEventRecord(e0, g_stream));
+		/* (through thhip_stream(), so that the profiler sees the stream in use and starts
+		 * the next profiled launch at an event of its own) */
+		hipcheck(hipEventRecord(e0, thhip_stream()));
 		if (dtype == THHIP_F32)
-			mfma_probe_kernel<THHIP_F32><<<dim3(blocks), dim3(256), 0, g_stream>>>(out, in, iters);
+			mfma_probe_kernel<THHIP_F32><<<dim3(blocks), dim3(256), 0, thhip_stream()>>>(out, in, iters);
 		else if (dtype == THHIP_F16)
-			mfma_probe_kernel<THHIP_F16><<<dim3(blocks), dim3(256), 0, g_stream>>>(out, in, iters);
+			mfma_probe_kernel<THHIP_F16><<<dim3(blocks), dim3(256), 0, thhip_stream()>>>(out, in, iters);
 		else
-			mfma_probe_kernel<THHIP_U8><<<dim3(blocks), dim3(256), 0, g_stream>>>(out, in, iters);
+			mfma_probe_kernel<THHIP_U8><<<dim3(blocks), dim3(256), 0, thhip_stream()>>>(out, in, iters);
 		hipcheck(hipGetLastError());
-		hipcheck(hipEventRecord(e1, g_stream));
+		hipcheck(hipEventRecord(e1, thhip_stream()));
 		hipcheck(hipEventSynchronize(e1));
 		float t;
 		hipcheck(hipEventElapsedTime(&t, e0, e1));

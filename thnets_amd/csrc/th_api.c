@@ -27,8 +27,9 @@ void THInit(void)
 	if (thhip_device_count() < 1)
 		THError("thnets HIP engine: no AMD GPU visible; this library has no CPU fallback");
 	/* the fixed partial-sum array of thhip_linear_batched_noalloc: look its address up now */
-	if (thhip_linear_batched_noalloc_init())
-		THError("thnets HIP engine: the fixed device array of thhip_linear_batched_noalloc could not be resolved");
+	if (thhip_linear_batched_noalloc_init())	/* only that entry point is affected: it then returns -3 */
+		fprintf(stderr, "thnets HIP engine: the fixed device array of thhip_linear_batched_noalloc could not be "
+			"resolved; that call is unavailable\n");
 }
 
 static THNETWORK *create_engine_network(THNETWORK *net, int lowp, float range)
@@ -81,96 +82,13 @@ void THFreeNetwork(THNETWORK *network)
 	free(network);
 }
 
-/* cudnn_basic.c:64-80 is the CUDA analogue: same shape, contiguous device
- * copy in the engine's activation type. */
-static THFloatTensor *device_tensor_like(THFloatTensor *t, int dtype)
-{
-	THFloatTensor *n = malloc(sizeof(*n));
-	memcpy(n, t, sizeof(*n));
-	n->storage = 0;
-	n->storageOffset = 0;
-	if (t->storage) {
-		long stride = 1;
-		for (int i = t->nDimension - 1; i >= 0; i--) {
-			n->stride[i] = stride;
-			stride *= t->size[i];
-		}
-		n->storage = malloc(sizeof(*n->storage));
-		n->storage->nref = 1;
-		n->storage->mustfree = TH_MUSTFREE_HIP_OF(dtype);
-		n->storage->data = thhip_malloc((size_t)THFloatTensor_nElement(t) * (dtype == THHIP_F32 ? 4 : dtype == THHIP_U8 ? 1 : 2));
-	}
-	return n;
-}
-
-static void require_contiguous(THFloatTensor *t)
-{
-	long stride = 1;
-	for (int i = t->nDimension - 1; i >= 0; i--) {
-		if (t->size[i] != 1 && t->stride[i] != stride)
-			THError("tensor is not contiguous");
-		stride *= t->size[i];
-	}
-}
-
-static THFloatTensor *upload_as(THFloatTensor *t, int dtype)
-{
-	THFloatTensor *n = device_tensor_like(t, dtype);
-	if (!t->storage)
-		return n;
-	require_contiguous(t);
-	const long cnt = THFloatTensor_nElement(t);
-	if (dtype == THHIP_F32)
-		thhip_memcpy_h2d(n->storage->data, THFloatTensor_data(t), sizeof(float) * cnt);
-	else {
-		float *tmp = thhip_malloc(sizeof(float) * cnt);
-		thhip_memcpy_h2d(tmp, THFloatTensor_data(t), sizeof(float) * cnt);
-		thhip_convert(tmp, THHIP_F32, n->storage->data, dtype, cnt);
-		thhip_sync();
-		thhip_free(tmp);
-	}
-	return n;
-}
-
-THFloatTensor *THHipTensor_newFromFloatTensor(THFloatTensor *t)
-{
-	return upload_as(t, thhip_engine_dtype());
-}
-
-static THFloatTensor *download_as_float(THFloatTensor *t, int dtype)
-{
-	THFloatTensor *n = malloc(sizeof(*n));
-	memcpy(n, t, sizeof(*n));
-	n->storage = 0;
-	n->storageOffset = 0;
-	if (!t->storage)
-		return n;
-	const long cnt = THFloatTensor_nElement(t);
-	n->storage = THFloatStorage_new(cnt);
-	const void *src = thhip_tensor_ptr(t, dtype);
-	if (dtype == THHIP_F32)
-		thhip_memcpy_d2h(n->storage->data, src, sizeof(float) * cnt);
-	else {
-		float *tmp = thhip_malloc(sizeof(float) * cnt);
-		thhip_convert(src, dtype, tmp, THHIP_F32, cnt);
-		thhip_memcpy_d2h(n->storage->data, tmp, sizeof(float) * cnt);
-		thhip_free(tmp);
-	}
-	return n;
-}
-
-THFloatTensor *THFloatTensor_newFromHipTensor(THFloatTensor *t)
-{
-	return download_as_float(t, thhip_engine_dtype());
-}
-
 THFloatTensor *THForward(THNETWORK *net, THFloatTensor *in)
 {
 	engine_of(net);
 	return thhip_forward(net->net, in);
 }
 
-static int finish(THNETWORK *network, THFloatTensor *out, float **result, int *outwidth, int *outheight)
+static int finish(THFloatTensor *out, float **result, int *outwidth, int *outheight)
 {
 	*result = out->storage->data;
 	if (out->nDimension >= 3) {
@@ -178,193 +96,24 @@ static int finish(THNETWORK *network, THFloatTensor *out, float **result, int *o
 		*outheight = (int)out->size[out->nDimension - 2];
 	} else
 		*outwidth = *outheight = 1;
-	(void)network;
 	return (int)THFloatTensor_nElement(out);
 }
 
-/* uint8 engine: runs a device tensor of codes whose quantisation is in
- * hn->cur_mult / cur_sub, de-quantises the result (lowp_basic.c:40-58) and
- * leaves it in network->out. */
-static THFloatTensor *run_codes(THNETWORK *network, THFloatTensor *q)
-{
-	struct hipnet *hn = (struct hipnet *)network->net;
-	THFloatTensor *out = thhip_forward(network->net, q);
-	THFloatTensor *f = device_tensor_like(out, THHIP_F32);
-	thhip_dequantize(thhip_tensor_ptr(out, THHIP_U8), f->storage->data, THFloatTensor_nElement(out),
-		hn->cur_mult, hn->cur_sub);
-	if (network->out)
-		THFloatTensor_free(network->out);
-	network->out = download_as_float(f, THHIP_F32);
-	THFloatTensor_free(f);
-	return network->out;
-}
-
-/* Runs a device tensor of floats (engine dtype for ENGINE_HIP, fp32 for the
- * uint8 engine, which quantises it first) and leaves the float result in
- * network->out. */
-/* The caller's buffer as THProcessFloat leaves it: planes 0..2 normalised in
- * place (thapi.c:389-403).  mean/std hold three planes: further planes are left
- * untouched here (the reference reads past the arrays for them). */
-struct host_input {
-	float *data;
-	int batchsize, nplanes;
-	long hw;
-	const float *mean, *std;
-};
-
-static void normalize_on_host(const struct host_input *h)
-{
-	for (int b = 0; b < h->batchsize; b++)
-		for (int c = 0; c < h->nplanes && c < 3; c++) {
-			float *p = h->data + ((long)b * h->nplanes + c) * h->hw;
-			const float mean = h->mean[c], std = h->std[c];
-			for (long i = 0; i < h->hw; i++)
-				p[i] = (p[i] - mean) / std;
-		}
-}
-
-/* Runs a device tensor in the engine's float dtype (fp32 for the
- * uint8 engine, which quantises it first) and leaves the float result in
- * network->out.  The kernels of the forward pass are queued without waiting;
- * `host` (if any) is normalised while they run. */
-static THFloatTensor *run_float_input(THNETWORK *network, THFloatTensor *dev_in, const struct host_input *host)
-{
-	struct hipnet *hn = (struct hipnet *)network->net;
-	if (network->net->engine == ENGINE_HIPLOWP) {
-		/* THLowpTensor_newFromFloatTensor on the whole batch (one min/max),
-		 * lowp_basic.c:15-35 */
-		const long cnt = THFloatTensor_nElement(dev_in);
-		THFloatTensor *q = device_tensor_like(dev_in, THHIP_U8);
-		thhip_quantize((const float *)thhip_tensor_ptr(dev_in, THHIP_F32), (unsigned char *)q->storage->data, cnt,
-			&hn->cur_mult, &hn->cur_sub);
-		THFloatTensor *out = thhip_forward(network->net, q);
-		THFloatTensor *f = device_tensor_like(out, THHIP_F32);
-		thhip_dequantize(thhip_tensor_ptr(out, THHIP_U8), f->storage->data, THFloatTensor_nElement(out),
-			hn->cur_mult, hn->cur_sub);
-		if (host)
-			normalize_on_host(host);
-		if (network->out)
-			THFloatTensor_free(network->out);
-		network->out = download_as_float(f, THHIP_F32);
-		THFloatTensor_free(f);
-		THFloatTensor_free(q);
-	} else {
-		THFloatTensor *out = thhip_forward(network->net, dev_in);
-		if (host)
-			normalize_on_host(host);
-		if (network->out)
-			THFloatTensor_free(network->out);
-		network->out = download_as_float(out, hn->dtype);
-	}
-	return network->out;
-}
-
+/* thapi.c:363-450 with the engine's branch (th_io.c) as the only one. */
 int THProcessFloat(THNETWORK *network, float *data, int batchsize, int width, int height, int nplanes,
 	float **result, int *outwidth, int *outheight)
 {
-	const int engine = engine_of(network);
-	struct hipnet *hn = (struct hipnet *)network->net;
-	const long hw = (long)width * height;
-	/* The reference normalises the caller's buffer in place before any engine
-	 * sees it (thapi.c:389-403), and callers observe that.  Here the raw data
-	 * goes to the device first (the copy has finished when the call returns),
-	 * a kernel applies the same arithmetic there, and the host loop over the
-	 * caller's buffer runs while the GPU works on the forward pass: same bits
-	 * on both sides, the host pass off the critical path. */
-	THFloatTensor t;
-	memset(&t, 0, sizeof(t));
-	THFloatStorage st = { data, 1, 0 };
-	t.nDimension = 4;
-	t.size[0] = batchsize; t.size[1] = nplanes; t.size[2] = height; t.size[3] = width;
-	t.stride[3] = 1; t.stride[2] = width; t.stride[1] = hw; t.stride[0] = hw * nplanes;
-	t.storage = &st;
-	const int dt = engine == ENGINE_HIPLOWP ? THHIP_F32 : hn->dtype;
-	THFloatTensor *raw = upload_as(&t, THHIP_F32);
-	THFloatTensor *dev = dt == THHIP_F32 ? raw : device_tensor_like(&t, dt);
-	thhip_normalize(raw->storage->data, dev->storage->data, batchsize, nplanes, hw, network->mean, network->std, dt);
-	const struct host_input host = { data, batchsize, nplanes, hw, network->mean, network->std };
-	THFloatTensor *out = run_float_input(network, dev, &host);
-	if (dev != raw)
-		THFloatTensor_free(raw);
-	THFloatTensor_free(dev);
-	return finish(network, out, result, outwidth, outheight);
+	engine_of(network);
+	return finish(thhip_process_float(network, data, batchsize, width, height, nplanes), result, outwidth, outheight);
 }
 
+/* thapi.c:452-563 likewise. */
 int THProcessImages(THNETWORK *network, unsigned char **images, int batchsize, int width, int height, int stride,
 	float **results, int *outwidth, int *outheight, int bgr)
 {
-	const int engine = engine_of(network);
-	struct hipnet *hn = (struct hipnet *)network->net;
-	int cp = 3;
-	if (stride < width * 3)
-		cp = 1;	/* thapi.c:458-459 */
-	if (engine == ENGINE_HIPLOWP) {
-		/* thapi.c:485-487, 551-558: Lowp_LoadImages (always three planes, always
-		 * 4-D), forward, de-quantise.  It reads three bytes per pixel whatever the
-		 * stride: with stride < 3 * width (what the float engines take as one
-		 * plane, thapi.c:458-459) the reference reads past the image; here that
-		 * would be a device read past the staging copy, so it is refused. */
-		if (cp != 3)
-			THError("THProcessImages: the uint8 engine takes three-plane images only (stride %d < 3 * width %d)",
-				stride, width);
-		THFloatTensor *q = THFloatTensor_new();
-		q->storage = malloc(sizeof(*q->storage));
-		q->storage->nref = 1;
-		q->storage->mustfree = TH_MUSTFREE_HIP_OF(THHIP_U8);
-		q->storage->data = thhip_malloc((size_t)batchsize * 3 * width * height);
-		unsigned char *staging = thhip_malloc((size_t)stride * height);
-		for (int i = 0; i < batchsize; i++) {
-			thhip_memcpy_h2d(staging, images[i], (size_t)stride * height);
-			thhip_rgb2code((unsigned char *)q->storage->data + (size_t)i * 3 * width * height, staging, width, height,
-				stride, network->mean, network->std, bgr, &hn->cur_mult, &hn->cur_sub);
-		}
-		thhip_sync();
-		thhip_free(staging);
-		long s4[4] = { batchsize, 3, height, width };
-		q->nDimension = 4;
-		long st = 1;
-		for (int i = 3; i >= 0; st *= s4[i], i--) {
-			q->size[i] = s4[i];
-			q->stride[i] = st;
-		}
-		THFloatTensor *out = run_codes(network, q);
-		THFloatTensor_free(q);
-		return finish(network, out, results, outwidth, outheight);
-	}
-	const int dt = hn->dtype;
-	const size_t esz = dt == THHIP_F32 ? 4 : 2;
-	THFloatTensor *t = THFloatTensor_new();
-	t->storage = malloc(sizeof(*t->storage));
-	t->storage->nref = 1;
-	t->storage->mustfree = TH_MUSTFREE_HIP_OF(dt);
-	t->storage->data = thhip_malloc((size_t)batchsize * cp * width * height * esz);
-	unsigned char *staging = thhip_malloc((size_t)stride * height);
-	for (int i = 0; i < batchsize; i++) {
-		thhip_memcpy_h2d(staging, images[i], (size_t)stride * height);
-		thhip_rgb2float((char *)t->storage->data + (size_t)i * cp * width * height * esz, staging, width, height,
-			stride, cp, network->mean, network->std, bgr, dt);
-	}
-	thhip_sync();
-	thhip_free(staging);
-	if (batchsize == 1) {	/* thapi.c:497-516 */
-		long s[3] = { cp, height, width };
-		t->nDimension = 3;
-		for (int i = 2, st = 1; i >= 0; st *= s[i], i--) {
-			t->size[i] = s[i];
-			t->stride[i] = st;
-		}
-	} else {
-		long s[4] = { batchsize, cp, height, width };
-		t->nDimension = 4;
-		long st = 1;
-		for (int i = 3; i >= 0; st *= s[i], i--) {
-			t->size[i] = s[i];
-			t->stride[i] = st;
-		}
-	}
-	THFloatTensor *out = run_float_input(network, t, 0);
-	THFloatTensor_free(t);
-	return finish(network, out, results, outwidth, outheight);
+	engine_of(network);
+	return finish(thhip_process_images(network, images, batchsize, width, height, stride, bgr), results, outwidth,
+		outheight);
 }
 
 /* thapi.c:642-690: Views dropped, Linear -> size x size convolution on the host
@@ -442,13 +191,13 @@ long THHipNetwork_copyModuleOutput(THNETWORK *net, int idx, float **dst, long si
 	const int nd = o->nDimension;
 	if (hn->hm[idx].out_cl && nd >= 3 && o->size[nd - 1] * o->size[nd - 2] > 1) {
 		/* kept channels-last inside the engine: hand out the reference's order */
-		THFloatTensor *pm = device_tensor_like(o, hn->dtype);
+		THFloatTensor *pm = thhip_device_tensor_like(o, hn->dtype);
 		thhip_relayout(thhip_tensor_ptr(o, hn->dtype), pm->storage->data, nd == 4 ? (int)o->size[0] : 1,
 			(int)o->size[nd - 3], (int)(o->size[nd - 1] * o->size[nd - 2]), 0, hn->dtype);
-		h = download_as_float(pm, hn->dtype);
+		h = thhip_download_as_float(pm, hn->dtype);
 		THFloatTensor_free(pm);
 	} else
-		h = download_as_float(o, hn->dtype);
+		h = thhip_download_as_float(o, hn->dtype);
 	const long n = THFloatTensor_nElement(h);
 	*ndim = h->nDimension;
 	for (int i = 0; i < 4; i++)
@@ -488,8 +237,8 @@ THFloatTensor *THHipLowpTensor_newFromFloatTensor(THNETWORK *net, THFloatTensor 
 	if (engine_of(net) != ENGINE_HIPLOWP)
 		THError("THHipLowpTensor_newFromFloatTensor needs a network made by THCreateHipLowpNetwork");
 	struct hipnet *hn = (struct hipnet *)net->net;
-	THFloatTensor *f = upload_as(t, THHIP_F32);
-	THFloatTensor *q = device_tensor_like(f, THHIP_U8);
+	THFloatTensor *f = thhip_upload_as(t, THHIP_F32);
+	THFloatTensor *q = thhip_device_tensor_like(f, THHIP_U8);
 	thhip_quantize((const float *)f->storage->data, (unsigned char *)q->storage->data, THFloatTensor_nElement(f),
 		&hn->cur_mult, &hn->cur_sub);
 	thhip_sync();

@@ -1486,6 +1486,7 @@ void thhip_free_network(struct network *net)
 		for (int j = 0; j < 4; j++)
 			thhip_free(hm->bn[j]);
 	}
+	thhip_io_free(hn);
 	free(hn->hm);
 	free(net->modules);
 	free(hn);

@@ -57,6 +57,19 @@ struct hipmod {
 	float q_mult, q_sub;	/* quantisation of this module's output */
 };
 
+/* Staging memory of THProcessFloat / THProcessImages, kept with the top-level network
+ * between calls (th_io.c). */
+struct hipio_buf { THFloatTensor *t; size_t cap; };	/* a device tensor and the bytes behind it */
+struct hipio_pin { void *ptr; size_t cap; };		/* page-locked host memory */
+struct hipio {
+	struct hipio_buf in_raw;	/* the caller's floats as uploaded */
+	struct hipio_buf in_dev;	/* normalised input in a half type; planes made from 8-bit images */
+	struct hipio_buf in_q;		/* uint8 engine: input codes */
+	struct hipio_buf out_f;		/* a half or uint8 result as floats */
+	struct hipio_buf img;		/* 8-bit images as uploaded */
+	struct hipio_pin pin_in, pin_out;
+};
+
 /* A `struct network` with the engine's state behind it. */
 struct hipnet {
 	struct network pub;	/* must be first */
@@ -66,6 +79,7 @@ struct hipnet {
 	float cur_mult, cur_sub;	/* uint8 engine: quantisation of the tensor in flight */
 	int cur_cl;		/* uint8 engine: the tensor in flight is channels-last in memory */
 	int dag;		/* modules name their inputs (ninputs / inputs[]): the list is a graph */
+	struct hipio io;
 };
 
 struct hipnet *hipnet_of(struct module *m);
@@ -75,7 +89,15 @@ int thhip_engine_dtype(void);
 struct network *THHip_ToHip(struct network *net, int lowp, float range);
 THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in);
 void thhip_free_network(struct network *net);
+/* th_io.c */
 void thhip_storage_release(THFloatStorage *s);
+THFloatTensor *thhip_device_tensor_like(THFloatTensor *t, int dtype);
+THFloatTensor *thhip_upload_as(THFloatTensor *t, int dtype);
+THFloatTensor *thhip_download_as_float(THFloatTensor *t, int dtype);
+THFloatTensor *thhip_process_float(THNETWORK *network, float *data, int batchsize, int width, int height, int nplanes);
+THFloatTensor *thhip_process_images(THNETWORK *network, unsigned char **images, int batchsize, int width, int height,
+	int stride, int bgr);
+void thhip_io_free(struct hipnet *hn);
 /* th_load.c */
 int thhip_load_error(void);
 void thhip_free_loaded_network(THNETWORK *n);

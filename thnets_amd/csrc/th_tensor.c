@@ -49,17 +49,6 @@ THFloatStorage *THFloatStorage_newwithbuffer(void *buffer)
 	return s;
 }
 
-void thhip_storage_release(THFloatStorage *s)
-{
-	if (__sync_sub_and_fetch(&s->nref, 1) > 0)
-		return;
-	if (TH_IS_HIP_STORAGE(s->mustfree))
-		thhip_free(s->data);
-	else if (s->mustfree)
-		free(s->data);
-	free(s);
-}
-
 THFloatTensor *THFloatTensor_new(void)
 {
 	return calloc(1, sizeof(THFloatTensor));
