@@ -171,8 +171,21 @@ void thhip_io_free(struct hipnet *hn)
 /* Host memory -> device through the page-locked buffer, in pieces: the host copy
  * of piece i + 1 runs while piece i crosses the link.  When the call returns the
  * caller's memory has been read (the device copy is still on its way). */
+/* (the host copy is memory-bound: one thread moves a fresh 9.6 MB batch in 0.3 ms, the
+ * link takes 0.18 ms) */
+static void copy_to_pinned(char *dst, const char *src, size_t bytes)
+{
+	const size_t blk = (size_t)128 << 10;
+	const long nblk = (long)((bytes + blk - 1) / blk);
+#pragma omp parallel for schedule(static) if (bytes >= ((size_t)1 << 19))
+	for (long i = 0; i < nblk; i++) {
+		const size_t at = (size_t)i * blk;
+		memcpy(dst + at, src + at, bytes - at < blk ? bytes - at : blk);
+	}
+}
+
 #define IO_MIN_PIECE ((size_t)1 << 20)
-#define IO_MAX_PIECES 8
+#define IO_MAX_PIECES 4
 static void io_upload(struct hipnet *hn, void *dst, const void *src, size_t bytes, size_t pin_offset)
 {
 	char *pin = (char *)hn->io.pin_in.ptr + pin_offset;
@@ -182,7 +195,7 @@ static void io_upload(struct hipnet *hn, void *dst, const void *src, size_t byte
 	piece = (piece + 255) & ~(size_t)255;
 	for (size_t at = 0; at < bytes; at += piece) {
 		const size_t n = bytes - at < piece ? bytes - at : piece;
-		memcpy(pin + at, (const char *)src + at, n);
+		copy_to_pinned(pin + at, (const char *)src + at, n);
 		thhip_memcpy_h2d_async((char *)dst + at, pin + at, n);
 	}
 }
@@ -316,6 +329,7 @@ THFloatTensor *thhip_process_images(THNETWORK *network, unsigned char **images, 
 	const int group = batchsize < 8 ? 1 : (batchsize + 7) / 8;
 	for (int i = 0; i < batchsize; i += group) {
 		const int n = batchsize - i < group ? batchsize - i : group;
+#pragma omp parallel for schedule(static) if (ibytes * n >= ((size_t)1 << 19))
 		for (int j = i; j < i + n; j++)
 			memcpy(pin + islot * j, images[j], ibytes);
 		thhip_memcpy_h2d_async(dimg + islot * i, pin + islot * i, islot * n);
