@@ -292,9 +292,10 @@ def test_image_layer_with_pooling_bit_exact(hiplib, oracle):
 def test_conv_u8_patch_bit_exact(hiplib, oracle):
     """thhip_conv2d_u8_patch (input patch kept in LDS, optional 3x3 / stride 2 pooling) against
     the restatement step by step: AlexNet's conv2-5 shapes, several bands per image with and
-    without pooling, kernels of 2x3, 3x3 and 5x5 taps, one to six blocks of 64 input planes
-    (the patch of the next block is fetched while the current one is multiplied), padding codes
-    other than 128, wrapping parameters, and the unclamped last positions of a plane."""
+    without pooling, kernels of 1x1, 2x3, 3x3 and 5x5 taps, one to eight blocks of 64 input
+    planes (the whole patch, every block, is in LDS before the K loop), a last band shorter than
+    the others, padding codes other than 128, wrapping parameters, and the unclamped last
+    positions of a plane."""
     g = cases.rng(2000)
     prms = (dict(a_off=-117, b_off=-128, c_off=32513, c_mult=1028, c_shift=18),
             dict(a_off=-255, b_off=3, c_off=-12345, c_mult=511, c_shift=14),
@@ -307,7 +308,10 @@ def test_conv_u8_patch_bit_exact(hiplib, oracle):
               (1, 128, 9, 20, 64, 2, 3, 0, 1, 0),
               (2, 384, 13, 13, 128, 3, 3, 1, 1, 0),
               (1, 64, 40, 60, 64, 3, 3, 1, 1, 1),
-              (1, 64, 7, 100, 128, 3, 3, 0, 0, 0))
+              (1, 64, 7, 100, 128, 3, 3, 0, 0, 0),
+              (2, 128, 13, 13, 64, 1, 1, 0, 0, 0),
+              (1, 512, 13, 13, 64, 3, 3, 1, 1, 1),
+              (1, 64, 23, 23, 64, 3, 3, 1, 1, 1))
     for ci, (B, Ci, H, W, Co, kH, kW, pH, pW, pool) in enumerate(shapes):
         xq = g.integers(0, 256, (B, Ci, H, W), dtype=np.uint8)
         wq = g.integers(0, 256, (Co, Ci, kH, kW), dtype=np.uint8)
@@ -340,7 +344,7 @@ def test_conv_u8_patch_bit_exact(hiplib, oracle):
         hiplib.thhip_free(wp)
     assert not hiplib.thhip_conv2d_u8_patch_supported(1, 64, 13, 13, 64, 3, 3, 2, 2, 1, 1, 0)    # stride 2
     assert not hiplib.thhip_conv2d_u8_patch_supported(1, 96, 13, 13, 64, 3, 3, 1, 1, 1, 1, 0)    # 96 planes
-    assert not hiplib.thhip_conv2d_u8_patch_supported(1, 64, 13, 13, 64, 1, 1, 1, 1, 0, 0, 0)    # one tap
+    assert not hiplib.thhip_conv2d_u8_patch_supported(1, 4096, 13, 13, 64, 3, 3, 1, 1, 1, 1, 0)  # one output row: a patch of 180 KB
     assert not hiplib.thhip_conv2d_u8_patch_supported(1, 64, 13, 300, 64, 3, 3, 1, 1, 1, 1, 0)   # rows of 300 positions
 
 

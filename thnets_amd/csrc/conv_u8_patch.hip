@@ -11,43 +11,53 @@
  * its own copy of the input from L2 (nine times for a 3x3 layer), and the path from L2
  * to LDS, not the matrix core, sets the time of these layers.  Here a workgroup owns a
  * band of output rows of one image (up to 192 positions, six MFMA tiles of 32) and 64
- * output planes; per block of 64 input planes it copies the band's input patch (with its
- * halo) into LDS once and takes the B fragments of every tap from it; only the weights
- * stream.
+ * output planes.  It copies the band's input patch (with its halo, ALL input planes)
+ * into LDS once, before the K loop; after that the loop has no barrier and writes
+ * nothing to LDS: the B fragments of every tap come from the patch, and the A
+ * fragments - the weights, which thhip_conv_pack_weight_u8_patch stores in exactly the
+ * order the matrix core wants them - go from global memory straight into the registers
+ * the MFMA reads.
  *
  *  - K order: (block of 64 planes, tap, plane in the block); a K-tile is one tap of one
- *    block: 64 codes = two chunks of 32.  thhip_conv_pack_weight_u8_patch stores, per 64
- *    output planes and K-tile, the four 1 KiB fragments (row half i, chunk c) the matrix
- *    core wants, re-centred to signed bytes.
- *  - Four wavefronts: (chunk c, half nh of the position tiles).  A wavefront multiplies
- *    both row halves with three position tiles: 5 fragment reads for 6 MFMAs per K-tile;
- *    the two chunks' partial sums are added through LDS at the end (integers: exact).
- *  - Weights: every wavefront fetches one fragment of a K-tile into registers three
- *    K-tiles ahead and passes it on through one of three LDS stages; one barrier per K-tile.
- *    The patch of the next plane block is fetched at the start of a block and stored a few
- *    K-tiles later into the second patch buffer.
- *  - A patch pixel is 64 bytes = four 16-byte vectors; the patch is kept vector plane by
- *    vector plane, so the 32 positions of a fragment read (neighbouring pixels, one vector
- *    each) are 512 contiguous bytes and a tap is an offset.  Pixels outside the image hold
- *    the padding code.  The codes are re-centred (x ^ 0x80) when the patch is stored, and
- *    the sum of each pixel's 64 codes is kept with it: the column sums of the expanded
- *    offset term are gathered from those, one value per position and tap.
- *  - The fragments of K-tile kt + 1 are requested before K-tile kt is multiplied.
+ *    block: 64 codes = two chunks of 32.  The pack step stores, per 64 output planes and
+ *    K-tile, the four 1 KiB fragments (row half i, chunk c), re-centred to signed bytes.
+ *  - Eight wavefronts: (row half i, half nh of the position tiles, chunk kp).  A wavefront
+ *    multiplies its row half with three position tiles over its chunk of every K-tile:
+ *    one 16-byte load from global memory (a few K-tiles ahead) and three fragment reads
+ *    for three MFMAs.  Two wavefronts per SIMD keep the matrix core issuing (one alone
+ *    gets an MFMA through every 55 cycles of the shader clock counter, two together one every 37).  The two chunks'
+ *    partial sums are added through LDS at the end (integers: exact).
+ *  - A patch pixel is Ci bytes = Ci / 16 vectors; the patch is kept plane block by plane
+ *    block, vector plane by vector plane ([block][vector][pixel][16 bytes]), so the 32
+ *    positions of a fragment read (neighbouring pixels, one vector each) are 512
+ *    contiguous bytes and a tap is an offset.  Pixels outside the image hold the padding
+ *    code.  The codes are re-centred (x ^ 0x80) when the patch is stored.  The sum of
+ *    each pixel's codes (LDS atomics as the vectors are stored) and from those the column
+ *    sums of the expanded offset term (one value per position: the sum over the taps, taken
+ *    along the kernel rows and then down its columns) are made once, before the loop.
  *  - Epilogue as in the other uint8 kernels (expanded offset terms, gemmlowp's output stage
- *    in wrapping int32, bias add with its unclamped tail, threshold); then either 16-byte
- *    channels-last stores, or the codes go to LDS and every thread takes the maximum of a
- *    3x3 window for 16 planes.
+ *    in wrapping int32, bias add with its unclamped tail, threshold), every wavefront
+ *    finishing half of what it and its partner summed; then either 8-byte channels-last
+ *    stores, or the codes go to LDS and every thread takes the maximum of a 3x3 window for
+ *    16 planes.
  */
 #include <stdlib.h>
 #include <string.h>
 #include <type_traits>
 #include "thhip_internal.h"
 
-#define CP_THREADS 256
+#define CP_THREADS 512
 #define CP_MAXPOS 192		/* positions of a workgroup: six tiles of 32 */
-#define CP_MAXPIX 384		/* pixels of a patch (24 KiB) */
-#define CP_PL (CP_MAXPIX * 4 / CP_THREADS)	/* patch vectors per thread */
+#define CP_MAXPIX 1024		/* pixels of a patch */
 #define CP_PLANES 64
+#define CP_DEPTH 6		/* K-tiles of weights on their way to a wavefront's registers */
+#define CP_NB 6			/* patch vectors a thread has on their way at once */
+#define CP_XCH (8 * 24 * 64 * 4)	/* exchange of partial sums: 24 registers of eight wavefronts */
+#define CP_CBUF (CP_MAXPOS * CP_PLANES)	/* codes of a band before the pooling */
+/* column terms, row terms, bias addends, pixel sums, their sums along the kernel rows (reads of up to 3 + 4
+ * sums past a patch's last stay inside) */
+#define CP_TABLES ((CP_MAXPOS + 2 * CP_PLANES + 2 * (CP_MAXPIX + 8)) * 4)
+#define CP_LDS_MAX (150 * 1024)
 
 struct ConvPatchParams {
 	const unsigned char *x;		/* [B][H][W][Ci] codes */
@@ -61,10 +71,14 @@ struct ConvPatchParams {
 	int cwl;			/* convolution columns a workgroup computes */
 	int pw;				/* patch width in pixels: cwl + kW - 1 */
 	int taps, nkt, K;
+	int vp;				/* bytes between the vector planes of a patch */
+	int front;			/* bytes of LDS before the tables */
+	unsigned m_pw, m_cwl, m_pW;	/* x / d == __umulhi(x, m_d) for the small x used here (0: d == 1) */
 	int zero, offA, offB, c_off, c_mult, c_shift, act, ithr, ival;
 };
 
 typedef unsigned short cp_us2 __attribute__((ext_vector_type(2)));
+typedef unsigned uintx2 __attribute__((ext_vector_type(2)));
 
 /* v_permlane32_swap(x, y) exchanges x of lanes 32..63 with y of lanes 0..31. */
 __device__ __forceinline__ void cp_swap32(unsigned &x, unsigned &y)
@@ -74,24 +88,43 @@ __device__ __forceinline__ void cp_swap32(unsigned &x, unsigned &y)
 	y = r[1];
 }
 
-#define CP_VP (CP_MAXPIX * 16 + 64)	/* bytes between the vector planes of a patch: 64 past a multiple of 256 */
-
-/* two workgroups per CU (LDS allows no more): 256 registers per lane */
-template <bool POOL>
-__global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_u8_patch_kernel(ConvPatchParams p)
+__device__ __forceinline__ int cp_div(int x, unsigned magic)
 {
-	/* patch buffers 2 x 4 vector planes | pixel sums 2 x 384 | weight stages 3 x 4 KiB | row terms
-	 * (the front is reused for the exchange of sums and for the codes at the end) */
-	__shared__ __align__(16) unsigned char lds[2 * 4 * CP_VP + 2 * CP_MAXPIX * 4 + 3 * 4096 + 2 * CP_PLANES * 4];
-	unsigned char *const patch0 = lds;
-	int *const psum0 = (int *)(lds + 2 * 4 * CP_VP);
-	unsigned char *const wst = (unsigned char *)(psum0 + 2 * CP_MAXPIX);
-	int *const rowterm = (int *)(wst + 3 * 4096);
+	return magic ? (int)__umulhi((unsigned)x, magic) : x;
+}
+
+/* Sum of n values q[0], q[step], ...: four reads on their way at once, those past the end (which read the
+ * last one again) count nothing. */
+__device__ __forceinline__ int cp_sum_strided(const int *q, int n, int step)
+{
+	int s0 = 0, s1 = 0, s2 = 0, s3 = 0;
+	for (int k = 0; k < n; k += 4) {
+		const int v0 = q[k * step], v1 = q[min(k + 1, n - 1) * step], v2 = q[min(k + 2, n - 1) * step],
+			v3 = q[min(k + 3, n - 1) * step];
+		s0 += v0;
+		s1 += k + 1 < n ? v1 : 0;
+		s2 += k + 2 < n ? v2 : 0;
+		s3 += k + 3 < n ? v3 : 0;
+	}
+	return s0 + s1 + s2 + s3;
+}
+
+/* two workgroups per CU where the patch allows: 128 registers per lane */
+template <bool POOL>
+__global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_u8_patch_kernel(ConvPatchParams p)
+{
+	/* patch: blocks x 4 vector planes                    (the front: later the exchange of sums | the codes)
+	 * column terms | row terms | bias addends | pixel sums | their row sums        (the tables, from p.front on) */
+	extern __shared__ __align__(16) unsigned char lds[];
+	int *const colterm = (int *)(lds + p.front);
+	int *const rowterm = colterm + CP_MAXPOS;
 	int *const rowadd = rowterm + CP_PLANES;
+	int *const psum = rowadd + CP_PLANES;
+	int *const hsum = psum + CP_MAXPIX + 8;
 
 	const int tid = threadIdx.x, lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-	const int kp = wave >> 1, nh = wave & 1;	/* this wavefront's chunk of every K-tile, its half of the position tiles */
+	const int ri = wave & 1, nh = (wave >> 1) & 1, kp = wave >> 2;	/* row half, half of the position tiles, chunk of every K-tile */
 	const int n = lane & 31, h = lane >> 5;
 	const int band = blockIdx.x, mz = blockIdx.y, b = blockIdx.z;
 	/* the band: output rows row0 .. row0 + rows - 1 */
@@ -101,113 +134,116 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
 	const int npos = rows * p.cwl;
 	const int prows = rows + p.kH - 1;
 	const int npix = prows * p.pw;
+	const int nblocks = p.Ci >> 6;
+	const int blk = 4 * p.vp;	/* bytes of a plane block of the patch */
 
-	/* ---- what this thread moves of a patch: vectors s = tid + 256 u = vector s % 4 of pixel s / 4
-	 * (a wavefront's load covers 16 whole pixels: 64 contiguous bytes each) ---- */
-	int psrc[CP_PL];	/* byte offset in x of the vector (without the plane block), or -1: outside the image */
+	/* ---- weights: fragment (row half ri, chunk kp) of every K-tile, CP_DEPTH K-tiles ahead; a base that is
+	 * uniform in the wavefront plus a 32-bit lane offset ---- */
+	const unsigned char *wsrc = p.wp + ((size_t)mz * p.nkt) * 4096 + (ri * 2 + kp) * 1024;
+	const unsigned woff = lane * 16;
+	intx4 wr[CP_DEPTH];
+#define CP_WFETCH(SLOT_, KT_) (wr[SLOT_] = *(const intx4 *)(wsrc + (size_t)min((KT_), p.nkt - 1) * 4096 + woff))
 #pragma unroll
-	for (int u = 0; u < CP_PL; u++) {
-		const int s = tid + CP_THREADS * u, pp = s >> 2;
-		const int pr = pp / p.pw, pc = pp - pr * p.pw;
-		const int iy = row0 - p.padH + pr, ix = pc - p.padW;
-		const bool in = pp < npix && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
-		psrc[u] = in ? (((b * p.H + iy) * p.W + ix) * p.Ci + (s & 3) * 16) : -1;
+	for (int d = 0; d < CP_DEPTH; d++)
+		CP_WFETCH(d, d);
+
+	for (int pp = tid; pp < npix + 8; pp += CP_THREADS)
+		psum[pp] = 0;
+	/* (asked for now, put into LDS once the patch is: nothing waits for memory before the patch's own loads are out) */
+	int rs = 0, ra = 0;
+	if (tid < CP_PLANES) {
+		rs = p.rowsum[mz * CP_PLANES + tid];
+		ra = p.addend ? p.addend[mz * CP_PLANES + tid] : 0;
 	}
-	const int zero4 = p.zero * 0x01010101;
-	intx4 pv[CP_PL];
-	auto patch_fetch = [&](int cb) {
+	__syncthreads();
+
+	/* ---- the patch, plane block by plane block: of a block, vector s = vector s % 4 of pixel s / 4 (a
+	 * wavefront's load covers 16 whole pixels: 64 contiguous bytes each), re-centred (code - 128 as signed
+	 * bytes: x ^ 0x80); with a vector goes its share of the sum of its pixel's codes.  CP_NB loads of a
+	 * thread are on their way before the first is stored. ---- */
+	{
+		const int zero4 = p.zero * 0x01010101;
+		const int nvec = npix * 4 * nblocks;	/* vector s: vector s % 4 of pixel (s / 4) % npix of block s / (4 npix) */
+		const float inv_npix = 1.0f / (float)npix;	/* ((q + 0.5) / npix is at least 0.5 / npix away from an integer: rounding cannot cross it) */
+		for (int s0 = tid; s0 < nvec; s0 += CP_NB * CP_THREADS) {
+			intx4 pv[CP_NB];
+			int dst[CP_NB], pix[CP_NB];
 #pragma unroll
-		for (int u = 0; u < CP_PL; u++)
-			pv[u] = *(const intx4 *)(p.x + (psrc[u] >= 0 ? psrc[u] + cb * 64 : 0));
-	};
-	/* The patch is stored re-centred (code - 128 as signed bytes: x ^ 0x80), vector plane by
-	 * vector plane ([vector][pixel][16 bytes]: the 32 positions of a fragment read are then
-	 * 512 contiguous bytes), and with it the sum of every pixel's 64 re-centred codes, from
-	 * which the column sums of the expanded offset term are gathered tap by tap. */
-	auto patch_store = [&](int buf) {
-#pragma unroll
-		for (int u = 0; u < CP_PL; u++) {
-			const int s = tid + CP_THREADS * u;
-			intx4 v = psrc[u] >= 0 ? pv[u] : intx4{ zero4, zero4, zero4, zero4 };
-			int part = 0;
-#pragma unroll
-			for (int d = 0; d < 4; d++) {
-				v[d] ^= (int)0x80808080;
-				part = __builtin_amdgcn_sdot4(v[d], 0x01010101, part, false);
+			for (int u = 0; u < CP_NB; u++) {
+				const int s = s0 + u * CP_THREADS, q = s >> 2;
+				const int cb = (int)(((float)q + 0.5f) * inv_npix), pp = q - cb * npix;
+				const int pr = cp_div(pp, p.m_pw), pc = pp - pr * p.pw;
+				const int iy = row0 - p.padH + pr, ix = pc - p.padW;
+				const bool in = s < nvec && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
+				dst[u] = s < nvec ? cb * blk + (s & 3) * p.vp + pp * 16 : -1;
+				pix[u] = pp;
+				if (in)
+					pv[u] = *(const intx4 *)(p.x + ((size_t)((b * p.H + iy) * p.W + ix) * p.Ci + cb * 64 + (s & 3) * 16));
+				else
+					pv[u] = intx4{ zero4, zero4, zero4, zero4 };
 			}
-			part += __shfl_xor(part, 1, 64);	/* the four vectors of a pixel sit in four neighbouring lanes */
-			part += __shfl_xor(part, 2, 64);
-			if (s < npix * 4) {
-				*(intx4 *)(patch0 + buf * (4 * CP_VP) + (s & 3) * CP_VP + (s >> 2) * 16) = v;
-				if ((s & 3) == 0)
-					psum0[buf * CP_MAXPIX + (s >> 2)] = part;
+#pragma unroll
+			for (int u = 0; u < CP_NB; u++) {
+				intx4 v = pv[u];
+				int part = 0;
+#pragma unroll
+				for (int d = 0; d < 4; d++) {
+					v[d] ^= (int)0x80808080;
+					part = __builtin_amdgcn_sdot4(v[d], 0x01010101, part, false);
+				}
+				part += __shfl_xor(part, 1, 64);	/* the four vectors of a pixel sit in four neighbouring lanes */
+				part += __shfl_xor(part, 2, 64);
+				if (dst[u] >= 0) {
+					*(intx4 *)(lds + dst[u]) = v;
+					if ((lane & 3) == 0)
+						atomicAdd(&psum[pix[u]], part);
+				}
 			}
 		}
-	};
-
-	/* ---- weights: fragment `wave` (row half wave / 2, chunk wave % 2) of every K-tile ---- */
-	const unsigned char *wsrc = p.wp + ((size_t)mz * p.nkt) * 4096 + wave * 1024 + lane * 16;
-	intx4 wr[3];
-#define CP_WFETCH(SLOT_, KT_) (wr[SLOT_] = *(const intx4 *)(wsrc + (size_t)min((KT_), p.nkt - 1) * 4096))
-#define CP_WSTORE(SLOT_, KT_) (*(intx4 *)(wst + ((KT_) % 3) * 4096 + wave * 1024 + lane * 16) = wr[SLOT_])
-
+	}
+	if (tid < CP_PLANES) {
+		/* (wrapping, like the sum they join; multiplier and rounding term of the output stage folded in:
+		 * (acc + rowterm + colterm) mult + round = acc mult + (rowterm mult + round) + colterm mult) */
+		rowterm[tid] = (p.offB * rs + p.K * p.offA * p.offB + p.c_off) * p.c_mult + (p.c_shift < 1 ? 0 : 1 << (p.c_shift - 1));
+		rowadd[tid] = ra;
+	}
+	__syncthreads();
+	/* the column sums of the expanded offset term: a position's pixel sums under all the taps, in two passes:
+	 * along the kernel rows for every pixel (the sums of pixels whose kernel row leaves the patch are not
+	 * used), then down the kernel columns for every position */
+	for (int pp = tid; pp < npix; pp += CP_THREADS)
+		hsum[pp] = cp_sum_strided(psum + pp, p.kW, 1);
+	__syncthreads();
+	if (tid < CP_MAXPOS) {
+		const int posc = min(tid, npos - 1);
+		const int ly = cp_div(posc, p.m_cwl), lx = posc - ly * p.cwl;
+		colterm[tid] = cp_sum_strided(hsum + ly * p.pw + lx, p.kH, p.pw) * p.offA * p.c_mult;	/* (multiplier folded in) */
+	}
 	/* ---- this lane's positions: tile nh * 3 + j, position n of it ---- */
 	int pp0[3];
 #pragma unroll
 	for (int j = 0; j < 3; j++) {
 		const int pos = min((nh * 3 + j) * 32 + n, npos - 1);
-		const int ly = pos / p.cwl, lx = pos - ly * p.cwl;
-		pp0[j] = ly * p.pw + lx;
+		const int ly = cp_div(pos, p.m_cwl), lx = pos - ly * p.cwl;
+		pp0[j] = (ly * p.pw + lx) * 16 + (2 * kp + h) * p.vp;	/* byte offset in a plane block: the vector plane this lane feeds to the matrix core */
 	}
-	const int vbase = (2 * kp + h) * CP_VP;	/* the vector plane this lane feeds to the matrix core */
-
-	intx16 acc[2][3];
-	int cs[3] = { 0, 0, 0 };
+	/* tiles of this wavefront that hold positions of the band */
+	const int mytiles = min(3, max(0, (npos + 31) / 32 - nh * 3));
+	intx16 acc[3];
 #pragma unroll
-	for (int i = 0; i < 2; i++)
+	for (int j = 0; j < 3; j++)
 #pragma unroll
-		for (int j = 0; j < 3; j++)
-#pragma unroll
-			for (int r = 0; r < 16; r++)
-				acc[i][j][r] = 0;
+		for (int r = 0; r < 16; r++)
+			acc[j][r] = 0;
 
-	/* prologue: patch of block 0, weights of K-tiles 0 and 1 in LDS, 2..4 on their way */
-	patch_fetch(0);
-	CP_WFETCH(0, 0);
-	CP_WFETCH(1, 1);
-	CP_WFETCH(2, 2);
-	if (tid < CP_PLANES) {
-		const int m = mz * CP_PLANES + tid;
-		rowterm[tid] = p.offB * p.rowsum[m] + p.K * p.offA * p.offB + p.c_off;	/* (wrapping, like the sum it joins) */
-		rowadd[tid] = p.addend ? p.addend[m] : 0;
-	}
-	patch_store(0);
-	CP_WSTORE(0, 0);
-	CP_WSTORE(1, 1);
-	CP_WFETCH(0, 3);
-	CP_WFETCH(1, 4);
-	/* ring: K-tile t + 2 is in slot (t + 2) % 3 when step t begins */
-
-	const int nblocks = p.Ci / 64;
-	/* the K-tile whose fragments are requested next: plane block, tap, its offset in the patch */
+	/* the K-tile whose fragments are requested next: plane block, tap */
 	int n_cb = 0, n_tap = 0, n_kh = 0, n_kw = 0;
-	/* the K-tile being multiplied */
-	int c_cb = 0, c_tap = 0, c_toff = 0;
-	intx4 af[2][2], bf[2][3];
-	auto frags = [&](int kt, intx4 (&a)[2], intx4 (&bb)[3]) {
-		const unsigned char *ws = wst + (kt % 3) * 4096 + kp * 1024 + lane * 16;
-#pragma unroll
-		for (int i = 0; i < 2; i++)
-			a[i] = *(const intx4 *)(ws + i * 2048);
-		const unsigned char *pb = patch0 + (n_cb & 1) * (4 * CP_VP) + vbase + (n_kh * p.pw + n_kw) * 16;
+	intx4 bf[2][3];
+	auto frags = [&](intx4 (&bb)[3]) {
+		const unsigned char *pb = lds + n_cb * blk + (n_kh * p.pw + n_kw) * 16;
 #pragma unroll
 		for (int j = 0; j < 3; j++)
-			bb[j] = *(const intx4 *)(pb + pp0[j] * 16);
-	};
-	auto advance = [&]() {		/* current <- next, next <- the K-tile after it */
-		c_cb = n_cb;
-		c_tap = n_tap;
-		c_toff = n_kh * p.pw + n_kw;
+			bb[j] = *(const intx4 *)(pb + pp0[j]);
 		if (++n_kw == p.kW) {
 			n_kw = 0;
 			++n_kh;
@@ -217,150 +253,124 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
 			++n_cb;
 		}
 	};
-	__syncthreads();
-	frags(0, af[0], bf[0]);
-	advance();
-	auto step = [&](int kt, auto slot_, auto par_) {
-		constexpr int slot = decltype(slot_)::value;	/* (kt + 2) % 3 */
-		constexpr int par = decltype(par_)::value;	/* kt % 2: the register set that holds K-tile kt */
-		__syncthreads();	/* K-tile kt + 1 (and a patch stored before) is in LDS; stage (kt + 2) % 3 is free */
-		/* column sums: this tap's pixel of every position (lanes n and n + 32 twice the same);
-		 * requested first and added last, so that nothing this K-tile's MFMAs need waits for LDS */
-		int pst[3] = { 0, 0, 0 };
-		if (kp == 0) {
-			const int *ps = psum0 + (c_cb & 1) * CP_MAXPIX + c_toff;
+	if (mytiles > 0) {
+		/* Every step of the main loop issues the same memory operations whatever its K-tile: the compiler
+		 * sets its waits for the worst of the paths that meet, and an operation on one path only makes
+		 * every step wait for everything (measured: 390 -> 650 cycles a step). */
+		frags(bf[0]);
+		auto step = [&](int kt, auto slot_, auto par_, auto tail_) {
+			constexpr int slot = decltype(slot_)::value;	/* kt % CP_DEPTH */
+			constexpr int par = decltype(par_)::value;	/* kt % 2: the register set that holds K-tile kt */
+			if (!decltype(tail_)::value || kt + 1 < p.nkt)
+				frags(bf[par ^ 1]);	/* requested under this K-tile's MFMAs */
+			const intx4 a = wr[slot];
 #pragma unroll
 			for (int j = 0; j < 3; j++)
-				pst[j] = ps[pp0[j]];
+				acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bf[par][j], acc[j], 0, 0, 0);
+			CP_WFETCH(slot, kt + CP_DEPTH);
+		};
+		typedef std::integral_constant<int, 0> I0;
+		typedef std::integral_constant<int, 1> I1;
+		typedef std::integral_constant<int, 2> I2;
+		typedef std::integral_constant<int, 3> I3;
+		typedef std::integral_constant<int, 4> I4;
+		typedef std::integral_constant<int, 5> I5;
+		int kt = 0;
+		for (; kt + 6 < p.nkt; kt += 6) {	/* (kt + 6 < nkt: the K-tile after these six exists) */
+			step(kt, I0{}, I0{}, I0{});
+			step(kt + 1, I1{}, I1{}, I0{});
+			step(kt + 2, I2{}, I0{}, I0{});
+			step(kt + 3, I3{}, I1{}, I0{});
+			step(kt + 4, I4{}, I0{}, I0{});
+			step(kt + 5, I5{}, I1{}, I0{});
 		}
+		if (kt < p.nkt)
+			step(kt, I0{}, I0{}, I1{});
 		if (kt + 1 < p.nkt)
-			frags(kt + 1, af[par ^ 1], bf[par ^ 1]);	/* requested under this K-tile's MFMAs */
-		/* pass K-tile kt + 2 on, request K-tile kt + 5; the next block's patch early in a block */
-		CP_WSTORE(slot, kt + 2);
-		CP_WFETCH(slot, kt + 5);
-		if (c_tap == 0 && c_cb + 1 < nblocks)
-			patch_fetch(c_cb + 1);
-#pragma unroll
-		for (int j = 0; j < 3; j++)
-#pragma unroll
-			for (int i = 0; i < 2; i++)
-				acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[par][i], bf[par][j], acc[i][j], 0, 0, 0);
-		if (c_tap == 2 && c_cb + 1 < nblocks)
-			patch_store((c_cb + 1) & 1);
-#pragma unroll
-		for (int j = 0; j < 3; j++)
-			cs[j] += pst[j];
-		advance();
-	};
-	typedef std::integral_constant<int, 0> I0;
-	typedef std::integral_constant<int, 1> I1;
-	typedef std::integral_constant<int, 2> I2;
-	int kt = 0;
-	for (; kt + 5 < p.nkt; kt += 6) {
-		step(kt, I2{}, I0{});
-		step(kt + 1, I0{}, I1{});
-		step(kt + 2, I1{}, I0{});
-		step(kt + 3, I2{}, I1{});
-		step(kt + 4, I0{}, I0{});
-		step(kt + 5, I1{}, I1{});
+			step(kt + 1, I1{}, I1{}, I1{});
+		if (kt + 2 < p.nkt)
+			step(kt + 2, I2{}, I0{}, I1{});
+		if (kt + 3 < p.nkt)
+			step(kt + 3, I3{}, I1{}, I1{});
+		if (kt + 4 < p.nkt)
+			step(kt + 4, I4{}, I0{}, I1{});
+		if (kt + 5 < p.nkt)
+			step(kt + 5, I5{}, I1{}, I1{});
 	}
-	if (kt < p.nkt)
-		step(kt, I2{}, I0{});
-	if (kt + 1 < p.nkt)
-		step(kt + 1, I0{}, I1{});
-	if (kt + 2 < p.nkt)
-		step(kt + 2, I1{}, I0{});
-	if (kt + 3 < p.nkt)
-		step(kt + 3, I2{}, I1{});
-	if (kt + 4 < p.nkt)
-		step(kt + 4, I0{}, I0{});
 #undef CP_WFETCH
-#undef CP_WSTORE
-	__syncthreads();	/* everybody is done with the patches and the weight stages */
+	__syncthreads();	/* everybody is done with the patch (and the tables are written) */
 
-	/* ---- the two chunks' sums: wavefront (kp, nh) keeps row half kp, gets it from (1 - kp, nh) ---- */
+	/* ---- the two chunks' sums.  Units u = 2 j + (upper half of the registers): wavefront kp finishes units
+	 * 3 kp .. 3 kp + 2 and hands the other three to its partner (wave ^ 4) ---- */
 	{
-		int *xch = (int *)lds;		/* [wave][3 tiles][16][64 lanes]: 12 KiB per wavefront */
-		int *mine = xch + wave * (3 * 16 * 64);
+		int *mine = (int *)lds + wave * (24 * 64);
 #pragma unroll
-		for (int j = 0; j < 3; j++)
+		for (int u = 0; u < 3; u++)	/* the units the partner finishes (kp is uniform in a wavefront) */
 #pragma unroll
-			for (int r = 0; r < 16; r++)
-				mine[(j * 16 + r) * 64 + lane] = kp ? acc[0][j][r] : acc[1][j][r];	/* the half the other one keeps */
-		int *csx = xch + 4 * (3 * 16 * 64) + wave * (3 * 64);
-#pragma unroll
-		for (int j = 0; j < 3; j++)
-			csx[j * 64 + lane] = cs[j];
+			for (int r = 0; r < 8; r++)
+				mine[(u * 8 + r) * 64 + lane] = kp ? (u == 0 ? acc[0][r] : u == 1 ? acc[0][8 + r] : acc[1][r])
+								   : (u == 0 ? acc[1][8 + r] : u == 1 ? acc[2][r] : acc[2][8 + r]);
 	}
 	__syncthreads();
+	int fin[3][8];	/* the three units this wavefront finishes */
 	{
-		const int *xch = (const int *)lds;
-		const int *other = xch + (wave ^ 2) * (3 * 16 * 64);
+		const int *other = (const int *)lds + (wave ^ 4) * (24 * 64);
 #pragma unroll
-		for (int j = 0; j < 3; j++)
+		for (int u = 0; u < 3; u++)
 #pragma unroll
-			for (int r = 0; r < 16; r++) {
-				const int o = other[(j * 16 + r) * 64 + lane];
-				if (kp)
-					acc[1][j][r] += o;
-				else
-					acc[0][j][r] += o;
+			for (int r = 0; r < 8; r++) {
+				const int own = kp ? (u == 0 ? acc[1][8 + r] : u == 1 ? acc[2][r] : acc[2][8 + r])
+						   : (u == 0 ? acc[0][r] : u == 1 ? acc[0][8 + r] : acc[1][r]);
+				fin[u][r] = own + other[(u * 8 + r) * 64 + lane];
 			}
-		/* column sums: gathered by the wavefront (0, nh), per position */
-		const int *cso = xch + 4 * (3 * 16 * 64);
-#pragma unroll
-		for (int j = 0; j < 3; j++)
-			cs[j] = cso[(nh * 3 + j) * 64 + n];
 	}
-	__syncthreads();	/* the exchange area becomes the code buffer */
 
-	/* ---- requantise: this wavefront's row half kp of its three position tiles ---- */
-	unsigned char *cbuf = lds;	/* pooling: [position][64 planes], 16-byte pieces swapped around by the position */
+	/* ---- requantise ---- */
+	unsigned char *cbuf = lds + CP_XCH;	/* pooling: [position][64 planes], 16-byte pieces swapped around by the position */
 	const int tail0 = (p.oH * p.oW / 8) * 8;	/* lowpadd's unclamped tail starts here */
 	const bool has_add = p.addend != 0;
-	const unsigned round = p.c_shift < 1 ? 0u : 1u << (p.c_shift - 1);
+	const int athr = p.act ? p.ithr : -1;	/* no threshold: every code passes */
 #pragma unroll
-	for (int j = 0; j < 3; j++) {
+	for (int u = 0; u < 3; u++) {
+		const int uu = 3 * kp + u, j = uu >> 1, gh = uu & 1;	/* tile, register half */
 		const int pos = (nh * 3 + j) * 32 + n;
 		const int posc = min(pos, npos - 1);
-		const int ly = posc / p.cwl, lx = posc - ly * p.cwl;
+		const int ly = cp_div(posc, p.m_cwl), lx = posc - ly * p.cwl;
 		const int rem = (row0 + ly) * p.oW + lx;
-		const bool tail = has_add && rem >= tail0;
-		const int colterm = p.offA * cs[j];
-		unsigned word[4];
+		/* lowpadd (lowp_SpatialConvolution.c:71-88): min(sum, 255), then the lower clamp at 0 - except for the
+		 * last oH oW % 8 positions of a plane, whose negative sums wrap (the low byte is taken): a lower bound
+		 * per lane and the mask do both without a branch */
+		const int lo = has_add && rem >= tail0 ? (int)0x80000000 : 0;
+		const int ct = colterm[pos];
+		unsigned word[2];
 #pragma unroll
-		for (int g = 0; g < 4; g++) {
-			const int ml = kp * 32 + 8 * g + 4 * h;
-			const intx4 rt = *(const intx4 *)(rowterm + ml), ra = *(const intx4 *)(rowadd + ml);
+		for (int g2 = 0; g2 < 2; g2++) {
+			const int ml = ri * 32 + 8 * (2 * gh + g2) + 4 * h;
+			const intx4 rt = *(const intx4 *)(rowterm + ml), ra4 = *(const intx4 *)(rowadd + ml);
 			unsigned packed = 0;
 #pragma unroll
 			for (int e = 0; e < 4; e++) {
-				const int a = kp ? acc[1][j][4 * g + e] : acc[0][j][4 * g + e];
-				/* gemmlowp's output stage in wrapping int32 (c_off is in the row term) */
-				const unsigned u = (unsigned)(a + rt[e] + colterm) * (unsigned)p.c_mult + round;
-				int q = (int)u >> p.c_shift;
+				/* gemmlowp's output stage in wrapping int32: (acc + row term + column term) mult + round,
+				 * the constant parts multiplied before */
+				const unsigned uq = (unsigned)fin[u][4 * g2 + e] * (unsigned)p.c_mult + (unsigned)rt[e] + (unsigned)ct;
+				int q = (int)uq >> p.c_shift;
 				q = q < 0 ? 0 : q > 255 ? 255 : q;
-				const int sum = q + ra[e];	/* (no addend: 0, and the clamp changes nothing) */
-				q = tail ? (sum > 255 ? 255 : (sum & 255)) : (sum < 0 ? 0 : sum > 255 ? 255 : sum);	/* lowp_SpatialConvolution.c:71-88 */
-				if (p.act)
-					q = q > p.ithr ? q : p.ival;
+				q = max(min(q + ra4[e], 255), lo) & 255;	/* (no addend: 0, and nothing changes) */
+				q = q > athr ? q : p.ival;
 				packed |= (unsigned)q << (8 * e);
 			}
-			word[g] = packed;
+			word[g2] = packed;
 		}
-		/* lane (n, h) holds planes 8 g + 4 h .. + 3 of the row half; after the swaps lane n holds
-		 * planes 0..15 and lane n + 32 planes 16..31 as 16 bytes */
+		/* lane (n, h) holds planes 16 gh + 4 h .. + 3 and 16 gh + 8 + 4 h .. + 3 of the row half; after the
+		 * swap lane n holds planes 16 gh .. + 7 and lane n + 32 planes 16 gh + 8 .. + 15 as 8 bytes */
 		cp_swap32(word[0], word[1]);
-		cp_swap32(word[2], word[3]);
-		cp_swap32(word[0], word[2]);
-		cp_swap32(word[1], word[3]);
-		const uintx4 v = { word[0], word[1], word[2], word[3] };
-		const int piece = 2 * kp + h;		/* which 16 of the 64 planes */
+		const uintx2 v = { word[0], word[1] };
+		const int piece = 2 * ri + gh;		/* which 16 of the 64 planes */
 		if (pos < npos) {
 			if (POOL)
-				*(uintx4 *)(cbuf + posc * CP_PLANES + ((piece ^ (posc >> 2)) & 3) * 16) = v;
+				*(uintx2 *)(cbuf + posc * CP_PLANES + ((piece ^ (posc >> 2)) & 3) * 16 + h * 8) = v;
 			else
-				*(uintx4 *)(p.y + ((size_t)b * p.oH * p.oW + rem) * p.Co + mz * CP_PLANES + piece * 16) = v;
+				*(uintx2 *)(p.y + ((size_t)b * p.oH * p.oW + rem) * p.Co + mz * CP_PLANES + piece * 16 + h * 8) = v;
 		}
 	}
 	if (!POOL)
@@ -369,7 +379,7 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
 	/* ---- 3x3 / stride 2 maximum, sixteen planes per thread ---- */
 	for (int it = tid; it < pra * p.pW * 4; it += CP_THREADS) {
 		const int c16 = it & 3, t = it >> 2;
-		const int prl = t / p.pW, pcl = t - prl * p.pW;
+		const int prl = cp_div(t, p.m_pW), pcl = t - prl * p.pW;
 		cp_us2 me[4], mo[4];	/* byte-wise maxima as packed 16-bit maxima of the even and of the odd bytes */
 #pragma unroll
 		for (int d = 0; d < 4; d++)
@@ -394,17 +404,39 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2
 	}
 }
 
-/* Geometry of a launch; returns 0 when the kernel does not take the layer. */
+/* x / d == __umulhi(x, cp_magic(d)) for 0 <= x < 2^32 / d (round-up reciprocal); 0 stands for d = 1 */
+static unsigned cp_magic(int d)
+{
+	return d <= 1 ? 0u : (unsigned)((((unsigned long long)1 << 32) + d - 1) / d);
+}
+
+/* Geometry of a launch; returns 0 when the kernel does not take the layer, else the bytes of LDS. */
 static int cp_plan(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int pool,
 	ConvPatchParams *p)
 {
-	if (B < 1 || Ci < 64 || Ci % 64 || Co < 64 || Co % 64 || dH != 1 || dW != 1 || kH < 1 || kW < 1 || kH * kW < 4 ||
+	if (B < 1 || Ci < 64 || Ci % 64 || Co < 64 || Co % 64 || dH != 1 || dW != 1 || kH < 1 || kW < 1 ||
 	    padH < 0 || padW < 0)
-		return 0;	/* (fewer than four taps: the next block's patch would not be stored in time) */
+		return 0;
 	const int oW = W + 2 * padW - kW + 1, oH = H + 2 * padH - kH + 1;
 	if (oW < 1 || oH < 1)
 		return 0;
+	const int nblocks = Ci / 64;
 	int cwl = oW, rb, pH = 0, pW = 0;
+	/* bytes of LDS a band of `rows` output rows needs */
+	auto lds_of = [&](int rows, int *vp_out) {
+		const int npix = (rows + kH - 1) * (cwl + kW - 1);
+		const int vp = (npix * 16 + 255) / 256 * 256 + 64;	/* 64 past a multiple of 256: the two halves of a fragment read fall on different banks */
+		int front = nblocks * 4 * vp;
+		if (npix > CP_MAXPIX)
+			return 1 << 30;
+		const int need = CP_XCH + (pool ? CP_CBUF : 0);
+		if (front < need)
+			front = need;
+		front = (front + 15) / 16 * 16;
+		if (vp_out)
+			*vp_out = vp;
+		return front + CP_TABLES;
+	};
 	if (pool) {
 		if (oW < 3 || oH < 3)
 			return 0;
@@ -416,31 +448,43 @@ static int cp_plan(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, 
 		rb = (CP_MAXPOS / cwl - 1) / 2;		/* pooled rows: 2 rb + 1 convolution rows */
 		if (rb > pH)
 			rb = pH;
-		while (rb > 1 && (2 * rb + kH) * (cwl + kW - 1) > CP_MAXPIX)
+		while (rb > 1 && lds_of(2 * rb + 1, 0) > CP_LDS_MAX)
 			rb--;
-		if ((2 * rb + kH) * (cwl + kW - 1) > CP_MAXPIX)
+		if (lds_of(2 * rb + 1, 0) > CP_LDS_MAX)
 			return 0;
+		/* bands of equal height rather than full ones and a short last one */
+		const int bands = (pH + rb - 1) / rb;
+		rb = (pH + bands - 1) / bands;
 	} else {
 		if (oW > CP_MAXPOS)
 			return 0;
 		rb = CP_MAXPOS / oW;
 		if (rb > oH)
 			rb = oH;
-		while (rb > 1 && (rb + kH - 1) * (oW + kW - 1) > CP_MAXPIX)
+		while (rb > 1 && lds_of(rb, 0) > CP_LDS_MAX)
 			rb--;
-		if ((rb + kH - 1) * (oW + kW - 1) > CP_MAXPIX)
+		if (lds_of(rb, 0) > CP_LDS_MAX)
 			return 0;
+		const int bands = (oH + rb - 1) / rb;
+		rb = (oH + bands - 1) / bands;
 	}
 	if ((double)B * Ci * H * W >= 2147483000.0 || B > 65535 || Co / 64 > 65535)
 		return 0;
+	int vp = 0;
+	const int total = lds_of(pool ? 2 * rb + 1 : rb, &vp);
 	if (p) {
 		p->B = B; p->Ci = Ci; p->H = H; p->W = W; p->Co = Co; p->kH = kH; p->kW = kW; p->padH = padH; p->padW = padW;
 		p->oH = oH; p->oW = oW; p->pH = pH; p->pW = pW; p->pool = pool; p->rb = rb; p->cwl = cwl; p->pw = cwl + kW - 1;
 		p->taps = kH * kW;
 		p->nkt = Ci / 64 * kH * kW;
 		p->K = Ci * kH * kW;
+		p->vp = vp;
+		p->front = total - CP_TABLES;
+		p->m_pw = cp_magic(p->pw);
+		p->m_cwl = cp_magic(cwl);
+		p->m_pW = cp_magic(pW);
 	}
-	return 1;
+	return total;
 }
 
 /* Whether thhip_conv2d_u8_patch takes the layer (pool = 1: together with a 3x3 / stride 2
@@ -448,7 +492,7 @@ static int cp_plan(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, 
 extern "C" int thhip_conv2d_u8_patch_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
 	int padH, int padW, int pool)
 {
-	return cp_plan(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, pool, 0);
+	return cp_plan(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, pool, 0) > 0;
 }
 
 /* Codes [Co][Ci][kH][kW] -> per 64 output planes and K-tile (block of 64 input planes, tap)
@@ -494,7 +538,8 @@ extern "C" void thhip_conv2d_u8_patch(const unsigned char *x, const void *wpatch
 {
 	ConvPatchParams p;
 	memset(&p, 0, sizeof(p));
-	if (!cp_plan(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, pool, &p))
+	const int ldsbytes = cp_plan(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, pool, &p);
+	if (!ldsbytes)
 		THError("thhip_conv2d_u8_patch: layer not supported (see thhip_conv2d_u8_patch_supported)");
 	if (c_shift < 0 || c_shift > 31)
 		THError("thhip_conv2d_u8_patch: shift %d out of range", c_shift);
@@ -511,10 +556,16 @@ extern "C" void thhip_conv2d_u8_patch(const unsigned char *x, const void *wpatch
 	p.c_off = c_off; p.c_mult = c_mult; p.c_shift = c_shift;
 	p.act = act; p.ithr = thr; p.ival = val;
 	const int bands = pool ? (p.pH + p.rb - 1) / p.rb : (p.oH + p.rb - 1) / p.rb;
+	static bool attr_set;
+	if (!attr_set) {	/* more than 64 KiB of dynamic LDS has to be asked for */
+		hipcheck(hipFuncSetAttribute((const void *)conv_u8_patch_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, CP_LDS_MAX));
+		hipcheck(hipFuncSetAttribute((const void *)conv_u8_patch_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, CP_LDS_MAX));
+		attr_set = true;
+	}
 	ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * Co * (double)p.K * B * p.oH * p.oW);
 	const dim3 grid(bands, Co / 64, B);
 	if (pool)
-		conv_u8_patch_kernel<true><<<grid, dim3(CP_THREADS), 0, thhip_stream()>>>(p);
+		conv_u8_patch_kernel<true><<<grid, dim3(CP_THREADS), ldsbytes, thhip_stream()>>>(p);
 	else
-		conv_u8_patch_kernel<false><<<grid, dim3(CP_THREADS), 0, thhip_stream()>>>(p);
+		conv_u8_patch_kernel<false><<<grid, dim3(CP_THREADS), ldsbytes, thhip_stream()>>>(p);
 }

@@ -696,8 +696,7 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 		}
 	}
 	/* small channels-last images followed by a 3x3 / stride 2 pooling: the kernel that keeps the
-	 * input patch in LDS and pools its own codes (without a pooling to fuse, the generic kernel
-	 * below is the faster one: 17 and 21 us against 20 and 25 us on AlexNet's conv3 and conv4) */
+	 * input patch in LDS and pools its own codes */
 	if (hm->wpatch_u8 && hm->pool_next && x_cl == 1 && hm->out_cl && s.outnd >= 3 &&
 	    thhip_conv2d_u8_patch_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW,
 			c->padH, c->padW, 1)) {
@@ -713,6 +712,18 @@ static THFloatTensor *HipLowp_SpatialConvolution_updateOutput(struct module *m, 
 		return m->output;
 	}
 	void *y = conv_out(m, THHIP_U8, &s, c->nOutputPlane, oH, oW);
+	/* the same kernel without a pooling, for images one workgroup holds whole (AlexNet's conv3 and conv4) */
+	if (hm->wpatch_u8 && x_cl == 1 && hm->out_cl && s.outnd >= 3 && oH * oW <= 192 && oH * oW > 1 &&
+	    thhip_conv2d_u8_patch_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW,
+			c->padH, c->padW, 0)) {
+		thhip_conv2d_u8_patch(x, hm->wpatch_u8, hm->addend, y, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, zero, a_off, b_off, offset, mult, shift,
+			hm->fused_act, thr, val, 0);
+		hn->cur_cl = 1;
+		hn->cur_mult = om;
+		hn->cur_sub = osub;
+		return m->output;
+	}
 	if (hm->wrow_u8 && oH == 1 && oW == 1 && c->padH == 0 && c->padW == 0 && c->kH == s.H && c->kW == s.W &&
 	    thhip_linear_batched_u8_supported(s.B, K, c->nOutputPlane))
 		thhip_linear_batched_u8(x, hm->wrow_u8, hm->rowsum_u8, hm->addend, y, s.B, K, c->nOutputPlane,
@@ -1445,11 +1456,6 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 		hn->hm[i].res_target = chm;
 		hn->hm[i].res_from_input = identity;
 	}
-	for (int i = 0; i < net->nelem; i++)
-		if (hn->hm[i].wpatch_u8 && !hn->hm[i].pool_next) {	/* packed for a fusion that is not there */
-			thhip_free(hn->hm[i].wpatch_u8);
-			hn->hm[i].wpatch_u8 = 0;
-		}
 	return &hn->pub;
 }
 
