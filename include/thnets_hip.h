@@ -483,6 +483,19 @@ void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, const float *
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, int x_layout, int y_channels_last);
 
+/* Replaces SpatialConvolutionMM -> (SpatialBatchNormalization, folded) -> Threshold ->
+ * SpatialMaxPooling(3, 3, 2, 2, ppad, ppad) (modules/SpatialConvolutionMM.c:126-225,
+ * modules/SpatialMaxPooling.c:168-247) for an fp32 image layer: at most four
+ * plane-major input planes, whole blocks of 64 output planes, strides up to 4,
+ * pooled rows of whole groups of 14 positions (ResNet-18's 7x7 / stride 2 stem
+ * at 224 x 224).  One kernel; the convolution's output is never written.  y is
+ * [B][Co][pH][pW]. */
+int thhip_conv2d_image_pool_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int pkH, int pkW, int pdH, int pdW, int ppadH, int ppadW, int ceil_mode, int dtype, int x_layout);
+void thhip_conv2d_image_pool(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int ppad,
+	int act, float thr, float val, int dtype);
+
 /* thhip_conv2d_affine followed by a max pooling of any window, stride, padding and
  * rounding (modules/SpatialMaxPooling.c:6-98; the module sequence SpatialConvolutionMM
  * -> Threshold -> SpatialMaxPooling), y = [B][Co][pH][pW] from thhip_pool_outsize of the
@@ -515,39 +528,6 @@ void thhip_conv2d_residual(const void *x, const void *wpacked, const float *scal
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype);
 
-/* Tuning override for tests and experiments: force the convolution's workgroup
- * tile (bm x bn in {64,128}), its split-K factor and the number of workgroups
- * allowed to share a CU; 0 leaves a choice automatic.  A forced tile runs on
- * the kernel that stages its operands through registers, except:
- *   splitk == 9 asks for the kernels that load their operands straight into
- *     LDS (no K split of the whole layer there): half types and uint8 with channels-last input,
- *     tiles 64x64, 128x64, 64x128, 128x128; fp32 plane-major with Ci % 32 == 0,
- *     tiles 64x64 and 128x64, wgs_per_cu == 2 selecting K-tiles of 16 values;
- *   bn == 256 (half types): the 256x256 and 128x256 tiles of the same kernel
- *     (splitk == 4 with bm == 256: K-tiles of 64 values in two stages);
- *   (64, 1): the half-type kernel for 3x3 stride-1 layers of 64, 128, 256 or 512 planes
- *     that keeps an input patch in LDS.
- * A layer the forced kernel cannot take ends in THError. */
-void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu);
-/* fp32 only: force K-tiles of 16 values (chunks = 2) or 32 (4); 0 restores the
- * per-layer choice.  Tests and tuning, like thhip_conv_set_tuning. */
-void thhip_conv_set_ktile(int chunks);
-/* fp32 and half-type tiles loaded straight into LDS, layers without a K split
- * of their own: the tiles an XCD cannot spread evenly over its CUs (its tile
- * count modulo the workgroups it holds at once; half types: only after at
- * least one whole round) are dispatched last and cut along K into up to
- * `parts` parts of at least eight K-tiles, summed in their order by a small
- * kernel (results do not depend on timing).  Default 8, which is also the most
- * that is used; 1 = never cut.  Tests and tuning. */
-void thhip_conv_set_tail_parts(int parts);
-/* Force how the tile grid is cut over the eight XCDs: the M tiles into
- * mparts (1, 2, 4, 8) groups, the N tiles into 8 / mparts ranges; 0 restores
- * the choice by weight size.  Tests and tuning. */
-void thhip_conv_set_xcd_parts(int mparts);
-/* Channels-last inputs whose plane count is a multiple of the K-tile are
- * gathered with the filter tap tracked on the scalar unit; on = 1 forces the
- * per-thread tap decode that serves every plane count.  Tests and tuning. */
-void thhip_conv_set_generic_cl(int on);
 
 /* Replaces nn_Linear_updateOutput's 1-D branch (Linear.c:86-90 ->
  * thbasic.c:713-741 -> sgemv.c:48-105): y = bias + W x, W row-major
@@ -565,9 +545,6 @@ void thhip_gemv(const void *x, const void *w, const float *bias, void *y,
 int thhip_linear_batched_supported(int B, int nIn, int nOut, int dtype);
 void thhip_linear_batched(const void *x, const void *wrow, const float *bias, void *y,
 	int B, int nIn, int nOut, int act, float thr, float val, int dtype);
-/* Tests and tuning: 16-row blocks a wavefront of thhip_linear_batched owns
- * (1 or 4); 0 restores the choice by the layer's width. */
-void thhip_linear_batched_set_tuning(int row_blocks);
 
 /* thhip_linear_batched for callers that cannot allocate device memory (code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has

@@ -129,7 +129,7 @@ def test_in_tree_object_list_links(tmp_path, flags):
         pytest.skip("reference tree not mounted")
     csrc = os.path.join(ROOT, "thnets_amd", "csrc")
     engine, lowpgemm = _object_lists()
-    assert "th_engine.o" in engine and "th_io.o" in engine and len(engine) == 10
+    assert "th_engine.o" in engine and "th_io.o" in engine and len(engine) >= 11
     paths = {}
     for o in engine:
         src = os.path.join(csrc, o[:-2] + ".c")

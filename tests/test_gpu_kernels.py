@@ -128,6 +128,58 @@ def test_conv_f32_last_tiles_cut_along_k(hiplib, oracle):
         hiplib.thhip_conv_set_xcd_parts(0)
 
 
+def test_conv_f32_image_layer_with_pooling(hiplib, oracle):
+    """thhip_conv2d_image_pool (an fp32 image layer, its folded batch norm factor, Threshold and the
+    3x3 / stride 2 max pooling in one kernel) against the oracle's convolution -> factor and shift ->
+    Threshold -> max pooling: ResNet's 7x7 / stride 2 stem at 224 x 224 and 112 x 112, pooling padding 1
+    and 0 (the padding must never win a maximum: all-negative planes without a Threshold), one to four
+    input planes, other kernels and strides, 128 output planes, a last group of pooled rows that is
+    not full; and the layers it leaves to the other kernels."""
+    from thnets_amd import api
+    g = cases.rng(941)
+    #         B  Ci   H    W   Co  k  d pad ppad
+    shapes = [(2, 3, 224, 224, 64, 7, 2, 3, 1), (1, 3, 112, 112, 128, 7, 2, 3, 1), (2, 3, 115, 115, 64, 7, 2, 3, 0),
+              (1, 1, 57, 111, 64, 3, 2, 1, 1), (1, 4, 60, 58, 64, 5, 2, 2, 0), (1, 2, 100, 224, 64, 4, 4, 0, 1),
+              (1, 3, 84, 56, 64, 3, 1, 1, 1)]
+    for (B, Ci, H, W, Co, k, d, pad, ppad) in shapes:
+        x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+        w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+        b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        b[::3] -= np.float32(40)       # whole planes far below zero
+        sc = (g.uniform(0.5, 1.5, Co) * g.choice([-1.0, 1.0], Co)).astype(np.float32)
+        oH, oW = (H + 2 * pad - k) // d + 1, (W + 2 * pad - k) // d + 1
+        pH, pW = oracle.pool_outsize(oH, oW, 3, 3, 2, 2, ppad, ppad, 0)
+        raw = oracle.conv2d(x, w, None, (d, d), (pad, pad))
+        for act, scale in ((1, sc), (0, sc), (1, None)):
+            G.note("image layer + pooling %s act %d scale %s" % ((B, Ci, H, W, Co, k, d, pad, ppad), act, scale is not None))
+            assert hiplib.thhip_conv2d_image_pool_supported(B, Ci, H, W, Co, k, k, d, d, pad, pad, 3, 3, 2, 2, ppad, ppad, 0, G.F32, 0), \
+                (B, Ci, H, W, Co, k, d, pad, ppad)
+            dx = api.DeviceArray(hiplib, x)
+            wp = hiplib.thhip_conv_pack_weight_layout(np.ascontiguousarray(w).ctypes.data, Co, Ci, k, k, G.F32, 0)
+            db = api.DeviceArray(hiplib, b)
+            ds = api.DeviceArray(hiplib, scale) if scale is not None else None
+            dy = api.DeviceArray(hiplib, nbytes=B * Co * pH * pW * 4)
+            hiplib.thhip_memset(dy.ptr, 0x7f, B * Co * pH * pW * 4)
+            hiplib.thhip_conv2d_image_pool(dx.ptr, wp, ds.ptr if ds else None, db.ptr, dy.ptr, B, Ci, H, W, Co, k, k, d, d, pad, pad,
+                                           ppad, act, 0.25, -0.5, G.F32)
+            hiplib.thhip_sync()
+            got = dy.get((B, Co, pH, pW), np.float32)
+            hiplib.thhip_free(wp)
+            v = raw * scale[None, :, None, None] if scale is not None else raw
+            v = v + b[None, :, None, None]
+            if act:
+                v = np.where(v > np.float32(0.25), v, np.float32(-0.5)).astype(np.float32)
+            want = oracle.maxpool(v, 3, 3, 2, 2, ppad, ppad, 0)
+            G.assert_close(got, want, FP32_TOL, str((B, Ci, H, W, Co, k, d, pad, ppad, act)))
+    sup = hiplib.thhip_conv2d_image_pool_supported
+    assert not sup(2, 3, 224, 224, 64, 7, 7, 2, 2, 3, 3, 2, 2, 2, 2, 0, 0, 0, G.F32, 0)       # a 2x2 pooling
+    assert not sup(2, 3, 224, 224, 64, 7, 7, 2, 2, 3, 3, 3, 3, 2, 2, 1, 1, 1, G.F32, 0)       # ceil mode
+    assert not sup(2, 3, 224, 224, 64, 7, 7, 2, 2, 3, 3, 3, 3, 2, 2, 1, 1, 0, G.F16, 0)       # a half type
+    assert not sup(2, 8, 224, 224, 64, 7, 7, 2, 2, 3, 3, 3, 3, 2, 2, 1, 1, 0, G.F32, 0)       # eight planes
+    assert not sup(2, 3, 224, 224, 96, 7, 7, 2, 2, 3, 3, 3, 3, 2, 2, 1, 1, 0, G.F32, 0)       # 96 output planes
+    assert not sup(2, 3, 200, 200, 64, 7, 7, 2, 2, 3, 3, 3, 3, 2, 2, 1, 1, 0, G.F32, 0)       # pooled rows of 50 positions
+
+
 def test_conv_f32_k_split_with_a_pooling_of_any_window(hiplib, oracle):
     """fp32 layers of a few tiles split K and a second kernel adds the parts; that kernel also takes a max
     pooling that follows (any window, stride, padding, rounding): the same bits as the convolution entry

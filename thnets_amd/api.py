@@ -23,6 +23,17 @@ c_fp = C.POINTER(C.c_float)
 c_ip = C.POINTER(C.c_int)
 vp = C.c_void_p
 
+# Test and tuning hooks (process-wide switches of the kernel choice): exported by the library,
+# declared in csrc/thhip_internal.h, not in the installed header.
+TEST_HOOKS = {
+    "thhip_conv_set_ktile": (None, [C.c_int]),
+    "thhip_conv_set_tail_parts": (None, [C.c_int]),
+    "thhip_conv_set_xcd_parts": (None, [C.c_int]),
+    "thhip_conv_set_generic_cl": (None, [C.c_int]),
+    "thhip_linear_batched_set_tuning": (None, [C.c_int]),
+    "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),
+}
+
 # name -> (restype, argtypes); every symbol include/thnets_hip.h declares
 PROTOTYPES = {
     "THError": (None, None),
@@ -91,19 +102,15 @@ PROTOTYPES = {
     "thhip_conv2d_layout": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int, C.c_int, C.c_int]),
     "thhip_relayout": (None, [vp, vp] + [C.c_int] * 5),
     "thhip_maxpool_cl": (None, [vp, vp] + [C.c_int] * 13),
+    "thhip_conv2d_image_pool_supported": (C.c_int, [C.c_int] * 20),
+    "thhip_conv2d_image_pool": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 12 + [C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_conv2d_affine": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 11 + [C.c_int, C.c_float, C.c_float, C.c_int]),
-    "thhip_conv_set_ktile": (None, [C.c_int]),
-    "thhip_conv_set_tail_parts": (None, [C.c_int]),
     "thhip_maxpool_indices": (None, [vp, vp, vp] + [C.c_int] * 13),
     "thhip_maxunpool": (None, [vp, vp, vp] + [C.c_int] * 13),
     "thhip_fullconv_pack_weight": (vp, [vp] + [C.c_int] * 5),
     "thhip_fullconv2d": (None, [vp, vp, vp, C.c_float, vp, vp] + [C.c_int] * 14 + [C.c_float, C.c_float, C.c_int]),
     "thhip_col2im": (None, [vp, vp, C.c_float, vp] + [C.c_int] * 13 + [C.c_float, C.c_float, C.c_int]),
-    "thhip_conv_set_xcd_parts": (None, [C.c_int]),
-    "thhip_conv_set_generic_cl": (None, [C.c_int]),
     "thhip_normalize": (None, [vp, vp, C.c_int, C.c_int, C.c_long, vp, vp, C.c_int]),
-    "thhip_linear_batched_set_tuning": (None, [C.c_int]),
-    "thhip_conv_set_tuning": (None, [C.c_int, C.c_int, C.c_int, C.c_int]),
     "thhip_gemv": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
     "thhip_linear_batched_supported": (C.c_int, [C.c_int] * 4),
     "thhip_linear_batched": (None, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, C.c_int]),
@@ -163,7 +170,7 @@ def load_library(path=LIB_PATH):
             "%s is missing: build it with `make -C thnets_amd/csrc` (or __graft_entry__.build()); "
             "this package has no CPU fallback" % path)
     lib = C.CDLL(path)
-    for name, (res, args) in PROTOTYPES.items():
+    for name, (res, args) in list(PROTOTYPES.items()) + list(TEST_HOOKS.items()):
         fn = getattr(lib, name)
         if args is not None:
             fn.restype = res

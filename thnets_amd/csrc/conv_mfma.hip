@@ -4207,6 +4207,36 @@ extern "C" void thhip_conv2d_layout_pool2(const void *x, const void *wpacked, co
 		x_layout, y_channels_last != 0, 1);
 }
 
+/* Whether thhip_conv2d_image_pool takes the layer: fp32, plane-major, at most four input planes, whole
+ * blocks of 64 output planes, strides up to 4, followed by a 3x3 / stride 2 max pooling (padding 0 or 1,
+ * floor mode) whose output rows are whole groups of 14 positions (ResNet's 7x7 / stride 2 stem and its
+ * pooling at 224 x 224). */
+extern "C" int thhip_conv2d_image_pool_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
+	int padH, int padW, int pkH, int pkW, int pdH, int pdW, int ppadH, int ppadW, int ceil_mode, int dtype, int x_layout)
+{
+	if (x_layout || g_force_bm || g_force_bn || g_force_splitk)
+		return 0;
+	return thhip_conv_image_pool_f32_ok(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, pkH, pkW, pdH, pdW, ppadH, ppadW,
+		ceil_mode, dtype);
+}
+
+/* SpatialConvolutionMM (-> folded batch norm: per-plane factor before the shift) -> Threshold ->
+ * SpatialMaxPooling(3, 3, 2, 2, ppad, ppad) in one kernel for the layers
+ * thhip_conv2d_image_pool_supported accepts (modules/SpatialConvolutionMM.c:126-225,
+ * modules/SpatialMaxPooling.c:168-247): the convolution's output is never written.  y is
+ * [B][Co][pH][pW]; wpacked as thhip_conv_pack_weight_layout(..., x_layout 0) packs it. */
+extern "C" void thhip_conv2d_image_pool(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int ppad,
+	int act, float thr, float val, int dtype)
+{
+	if (!thhip_conv2d_image_pool_supported(B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, 3, 3, 2, 2, ppad, ppad, 0, dtype, 0))
+		THError("thhip_conv2d_image_pool: layer not supported (see thhip_conv2d_image_pool_supported)");
+	const int oW = (W + 2 * padW - kW) / dW + 1, oH = (H + 2 * padH - kH) / dH + 1;
+	ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)Ci * kH * kW * B * oH * oW);
+	thhip_conv_image_pool_f32((const float *)x, (const float *)wpacked, conv_kc(Ci, kH, kW, THHIP_F32, 0), scale, shift,
+		(float *)y, B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, ppad, act, thr, val);
+}
+
 /* Whether thhip_conv2d_residual takes this layer: fp32, plane-major tensors, planes in blocks of 32 (the
  * kernel that loads its tiles straight into LDS), the batch in one slice. */
 extern "C" int thhip_conv2d_residual_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,

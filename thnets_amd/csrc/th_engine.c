@@ -219,6 +219,19 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 		hn->hm[hm->pool_next].pooled_by_producer = 1;
 		return m->output;
 	}
+	/* an fp32 image layer followed by a 3x3 / stride 2 pooling (ResNet's stem): one kernel, no convolution output */
+	if (pq && dt == THHIP_F32 && !hm->x_layout && !hm->out_cl && s.outnd >= 3 &&
+	    thhip_conv2d_image_pool_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW,
+			c->padH, c->padW, pq->kH, pq->kW, pq->dH, pq->dW, pq->padH, pq->padW, pq->ceil_mode, dt, hm->x_layout)) {
+		int pH, pW;
+		thhip_pool_outsize(oH, oW, pq->kH, pq->kW, pq->dH, pq->dW, pq->padH, pq->padW, pq->ceil_mode, &pH, &pW);
+		void *yp = conv_out(m, dt, &s, c->nOutputPlane, pH, pW);
+		hn->cur_cl = 0;
+		thhip_conv2d_image_pool(x, hm->wpacked, hm->scale, hm->bias, yp, s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane,
+			c->kH, c->kW, c->dH, c->dW, c->padH, c->padW, pq->padH, hm->fused_act, hm->thr, hm->val, dt);
+		hn->hm[hm->pool_next].pooled_by_producer = 1;
+		return m->output;
+	}
 	/* fp32, a layer of a few tiles (its K is split and a second kernel adds the parts): that kernel takes
 	 * a max pooling of any window as well */
 	if (pq && dt == THHIP_F32 && !hm->x_layout && !hm->out_cl && s.outnd >= 3 &&
