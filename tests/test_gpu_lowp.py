@@ -293,9 +293,9 @@ def test_conv_u8_patch_bit_exact(hiplib, oracle):
     """thhip_conv2d_u8_patch (input patch kept in LDS, optional 3x3 / stride 2 pooling) against
     the restatement step by step: AlexNet's conv2-5 shapes, several bands per image with and
     without pooling, kernels of 1x1, 2x3, 3x3 and 5x5 taps, one to eight blocks of 64 input
-    planes (the whole patch, every block, is in LDS before the K loop), a last band shorter than
-    the others, padding codes other than 128, wrapping parameters, and the unclamped last
-    positions of a plane."""
+    planes (the whole patch in LDS before the K loop, or streamed block by block with weight
+    rings of three and five K-tiles), a last band shorter than the others, padding codes other
+    than 128, wrapping parameters, and the unclamped last positions of a plane."""
     g = cases.rng(2000)
     prms = (dict(a_off=-117, b_off=-128, c_off=32513, c_mult=1028, c_shift=18),
             dict(a_off=-255, b_off=3, c_off=-12345, c_mult=511, c_shift=14),
@@ -311,7 +311,13 @@ def test_conv_u8_patch_bit_exact(hiplib, oracle):
               (1, 64, 7, 100, 128, 3, 3, 0, 0, 0),
               (2, 128, 13, 13, 64, 1, 1, 0, 0, 0),
               (1, 512, 13, 13, 64, 3, 3, 1, 1, 1),
-              (1, 64, 23, 23, 64, 3, 3, 1, 1, 1))
+              (1, 64, 23, 23, 64, 3, 3, 1, 1, 1),
+              (2, 128, 11, 11, 64, 5, 5, 2, 2, 1),       # streamed patch, weight ring of five
+              (2, 128, 14, 14, 64, 3, 3, 1, 1, 1),       # streamed, ring of three, pooled
+              (1, 192, 6, 6, 64, 3, 3, 0, 0, 0),
+              (1, 128, 9, 9, 64, 3, 5, 1, 2, 0),         # 15 taps: three groups of five
+              (1, 128, 9, 9, 64, 3, 2, 1, 1, 0),         # 6 taps: an even number of groups of three - not streamed
+              (1, 128, 20, 20, 64, 3, 3, 1, 1, 0))       # a patch of more than 256 pixels - not streamed
     for ci, (B, Ci, H, W, Co, kH, kW, pH, pW, pool) in enumerate(shapes):
         xq = g.integers(0, 256, (B, Ci, H, W), dtype=np.uint8)
         wq = g.integers(0, 256, (Co, Ci, kH, kW), dtype=np.uint8)

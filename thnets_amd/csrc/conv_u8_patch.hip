@@ -11,9 +11,10 @@
  * its own copy of the input from L2 (nine times for a 3x3 layer), and the path from L2
  * to LDS, not the matrix core, sets the time of these layers.  Here a workgroup owns a
  * band of output rows of one image (up to 192 positions, six MFMA tiles of 32) and 64
- * output planes.  It copies the band's input patch (with its halo, ALL input planes)
- * into LDS once, before the K loop; after that the loop has no barrier and writes
- * nothing to LDS: the B fragments of every tap come from the patch, and the A
+ * output planes.  The band's input patch (with its halo, ALL input planes) is in LDS
+ * once - before the K loop, or (3x3 and 5x5 kernels on 128 planes and more) plane block by
+ * plane block just ahead of the taps that read it, one barrier a block; the loop itself
+ * has no barrier: the B fragments of every tap come from the patch, and the A
  * fragments - the weights, which thhip_conv_pack_weight_u8_patch stores in exactly the
  * order the matrix core wants them - go from global memory straight into the registers
  * the MFMA reads.
@@ -109,8 +110,23 @@ __device__ __forceinline__ int cp_sum_strided(const int *q, int n, int step)
 	return s0 + s1 + s2 + s3;
 }
 
-/* two workgroups per CU where the patch allows: 128 registers per lane */
-template <bool POOL>
+/* f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>) */
+template <int I, int N, typename F>
+__device__ __forceinline__ void cp_static_for(F &&f)
+{
+	if constexpr (I < N) {
+		f(std::integral_constant<int, I>{});
+		cp_static_for<I + 1, N>(f);
+	}
+}
+
+/* D = 0: the whole patch before the K loop.  D > 0 (3 or 5; the kernel's taps a multiple of it, taps / D odd,
+ * at least two plane blocks, a patch of at most 256 pixels): the patch is streamed - block 0 before the loop,
+ * block cb + 1 requested when block cb's taps begin and stored when they end (one barrier per block), the
+ * weights through a ring of D K-tiles that starts anew with every block, so that every wait count is a
+ * constant of straight-line code.
+ * Two workgroups per CU where the patch allows: 128 registers per lane. */
+template <bool POOL, int D>
 __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4))) void conv_u8_patch_kernel(ConvPatchParams p)
 {
 	/* patch: blocks x 4 vector planes                    (the front: later the exchange of sums | the codes)
@@ -141,10 +157,11 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 	 * uniform in the wavefront plus a 32-bit lane offset ---- */
 	const unsigned char *wsrc = p.wp + ((size_t)mz * p.nkt) * 4096 + (ri * 2 + kp) * 1024;
 	const unsigned woff = lane * 16;
-	intx4 wr[CP_DEPTH];
+	constexpr int RING = D ? D : CP_DEPTH;
+	intx4 wr[RING];
 #define CP_WFETCH(SLOT_, KT_) (wr[SLOT_] = *(const intx4 *)(wsrc + (size_t)min((KT_), p.nkt - 1) * 4096 + woff))
 #pragma unroll
-	for (int d = 0; d < CP_DEPTH; d++)
+	for (int d = 0; d < RING; d++)
 		CP_WFETCH(d, d);
 
 	for (int pp = tid; pp < npix + 8; pp += CP_THREADS)
@@ -161,8 +178,8 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 	 * wavefront's load covers 16 whole pixels: 64 contiguous bytes each), re-centred (code - 128 as signed
 	 * bytes: x ^ 0x80); with a vector goes its share of the sum of its pixel's codes.  CP_NB loads of a
 	 * thread are on their way before the first is stored. ---- */
-	{
-		const int zero4 = p.zero * 0x01010101;
+	const int zero4 = p.zero * 0x01010101;
+	if constexpr (D == 0) {
 		const int nvec = npix * 4 * nblocks;	/* vector s: vector s % 4 of pixel (s / 4) % npix of block s / (4 npix) */
 		const float inv_npix = 1.0f / (float)npix;	/* ((q + 0.5) / npix is at least 0.5 / npix away from an integer: rounding cannot cross it) */
 		for (int s0 = tid; s0 < nvec; s0 += CP_NB * CP_THREADS) {
@@ -201,6 +218,46 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 			}
 		}
 	}
+	/* streamed: of every block this thread moves vectors tid and tid + 512 (vector s % 4 of pixel s / 4) */
+	int psrc[2];	/* byte offset in x of the vector (without the plane block), or -1: outside the image or the patch */
+#pragma unroll
+	for (int u = 0; u < 2; u++) {
+		const int s = tid + u * CP_THREADS, pp = s >> 2;
+		const int pr = cp_div(pp, p.m_pw), pc = pp - pr * p.pw;
+		const int iy = row0 - p.padH + pr, ix = pc - p.padW;
+		const bool in = pp < npix && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
+		psrc[u] = in ? ((b * p.H + iy) * p.W + ix) * p.Ci + (s & 3) * 16 : -1;
+	}
+	intx4 pvn[2];
+	auto patch_fetch = [&](int cb) {	/* (always two loads: what lies outside fetches the tensor's first bytes) */
+#pragma unroll
+		for (int u = 0; u < 2; u++)
+			pvn[u] = *(const intx4 *)(p.x + (psrc[u] >= 0 ? psrc[u] + cb * 64 : 0));
+	};
+	auto patch_store = [&](int cb) {
+#pragma unroll
+		for (int u = 0; u < 2; u++) {
+			const int s = tid + u * CP_THREADS, pp = s >> 2;
+			intx4 v = psrc[u] >= 0 ? pvn[u] : intx4{ zero4, zero4, zero4, zero4 };
+			int part = 0;
+#pragma unroll
+			for (int d = 0; d < 4; d++) {
+				v[d] ^= (int)0x80808080;
+				part = __builtin_amdgcn_sdot4(v[d], 0x01010101, part, false);
+			}
+			part += __shfl_xor(part, 1, 64);
+			part += __shfl_xor(part, 2, 64);
+			if (pp < npix) {
+				*(intx4 *)(lds + cb * blk + (s & 3) * p.vp + pp * 16) = v;
+				if ((lane & 3) == 0)
+					atomicAdd(&psum[pp], part);
+			}
+		}
+	};
+	if constexpr (D != 0) {
+		patch_fetch(0);
+		patch_store(0);
+	}
 	if (tid < CP_PLANES) {
 		/* (wrapping, like the sum they join; multiplier and rounding term of the output stage folded in:
 		 * (acc + rowterm + colterm) mult + round = acc mult + (rowterm mult + round) + colterm mult) */
@@ -210,15 +267,19 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 	__syncthreads();
 	/* the column sums of the expanded offset term: a position's pixel sums under all the taps, in two passes:
 	 * along the kernel rows for every pixel (the sums of pixels whose kernel row leaves the patch are not
-	 * used), then down the kernel columns for every position */
-	for (int pp = tid; pp < npix; pp += CP_THREADS)
-		hsum[pp] = cp_sum_strided(psum + pp, p.kW, 1);
-	__syncthreads();
-	if (tid < CP_MAXPOS) {
-		const int posc = min(tid, npos - 1);
-		const int ly = cp_div(posc, p.m_cwl), lx = posc - ly * p.cwl;
-		colterm[tid] = cp_sum_strided(hsum + ly * p.pw + lx, p.kH, p.pw) * p.offA * p.c_mult;	/* (multiplier folded in) */
-	}
+	 * used), then down the kernel columns for every position.  (Once the whole patch is in LDS.) */
+	auto column_terms = [&]() {
+		for (int pp = tid; pp < npix; pp += CP_THREADS)
+			hsum[pp] = cp_sum_strided(psum + pp, p.kW, 1);
+		__syncthreads();
+		if (tid < CP_MAXPOS) {
+			const int posc = min(tid, npos - 1);
+			const int ly = cp_div(posc, p.m_cwl), lx = posc - ly * p.cwl;
+			colterm[tid] = cp_sum_strided(hsum + ly * p.pw + lx, p.kH, p.pw) * p.offA * p.c_mult;	/* (multiplier folded in) */
+		}
+	};
+	if constexpr (D == 0)
+		column_terms();
 	/* ---- this lane's positions: tile nh * 3 + j, position n of it ---- */
 	int pp0[3];
 #pragma unroll
@@ -227,75 +288,131 @@ __global__ __launch_bounds__(CP_THREADS) __attribute__((amdgpu_waves_per_eu(4, 4
 		const int ly = cp_div(pos, p.m_cwl), lx = pos - ly * p.cwl;
 		pp0[j] = (ly * p.pw + lx) * 16 + (2 * kp + h) * p.vp;	/* byte offset in a plane block: the vector plane this lane feeds to the matrix core */
 	}
-	/* tiles of this wavefront that hold positions of the band */
-	const int mytiles = min(3, max(0, (npos + 31) / 32 - nh * 3));
 	intx16 acc[3];
 #pragma unroll
 	for (int j = 0; j < 3; j++)
 #pragma unroll
 		for (int r = 0; r < 16; r++)
 			acc[j][r] = 0;
-
-	/* the K-tile whose fragments are requested next: plane block, tap */
-	int n_cb = 0, n_tap = 0, n_kh = 0, n_kw = 0;
 	intx4 bf[2][3];
-	auto frags = [&](intx4 (&bb)[3]) {
-		const unsigned char *pb = lds + n_cb * blk + (n_kh * p.pw + n_kw) * 16;
+	if constexpr (D == 0) {
+		/* tiles of this wavefront that hold positions of the band */
+		const int mytiles = min(3, max(0, (npos + 31) / 32 - nh * 3));
+		/* the K-tile whose fragments are requested next: plane block, tap */
+		int n_cb = 0, n_tap = 0, n_kh = 0, n_kw = 0;
+		auto frags = [&](intx4 (&bb)[3]) {
+			const unsigned char *pb = lds + n_cb * blk + (n_kh * p.pw + n_kw) * 16;
 #pragma unroll
-		for (int j = 0; j < 3; j++)
-			bb[j] = *(const intx4 *)(pb + pp0[j]);
-		if (++n_kw == p.kW) {
-			n_kw = 0;
-			++n_kh;
+			for (int j = 0; j < 3; j++)
+				bb[j] = *(const intx4 *)(pb + pp0[j]);
+			if (++n_kw == p.kW) {
+				n_kw = 0;
+				++n_kh;
+			}
+			if (++n_tap == p.taps) {
+				n_tap = n_kh = n_kw = 0;
+				++n_cb;
+			}
+		};
+		if (mytiles > 0) {
+			/* Every step of the main loop issues the same memory operations whatever its K-tile: the compiler
+			 * sets its waits for the worst of the paths that meet, and an operation on one path only makes
+			 * every step wait for everything (measured: 390 -> 650 cycles a step). */
+			frags(bf[0]);
+			auto step = [&](int kt, auto slot_, auto par_, auto tail_) {
+				constexpr int slot = decltype(slot_)::value;	/* kt % CP_DEPTH */
+				constexpr int par = decltype(par_)::value;	/* kt % 2: the register set that holds K-tile kt */
+				if (!decltype(tail_)::value || kt + 1 < p.nkt)
+					frags(bf[par ^ 1]);	/* requested under this K-tile's MFMAs */
+				const intx4 a = wr[slot];
+#pragma unroll
+				for (int j = 0; j < 3; j++)
+					acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bf[par][j], acc[j], 0, 0, 0);
+				CP_WFETCH(slot, kt + CP_DEPTH);
+			};
+			typedef std::integral_constant<int, 0> I0;
+			typedef std::integral_constant<int, 1> I1;
+			typedef std::integral_constant<int, 2> I2;
+			typedef std::integral_constant<int, 3> I3;
+			typedef std::integral_constant<int, 4> I4;
+			typedef std::integral_constant<int, 5> I5;
+			int kt = 0;
+			for (; kt + 6 < p.nkt; kt += 6) {	/* (kt + 6 < nkt: the K-tile after these six exists) */
+				step(kt, I0{}, I0{}, I0{});
+				step(kt + 1, I1{}, I1{}, I0{});
+				step(kt + 2, I2{}, I0{}, I0{});
+				step(kt + 3, I3{}, I1{}, I0{});
+				step(kt + 4, I4{}, I0{}, I0{});
+				step(kt + 5, I5{}, I1{}, I0{});
+			}
+			if (kt < p.nkt)
+				step(kt, I0{}, I0{}, I1{});
+			if (kt + 1 < p.nkt)
+				step(kt + 1, I1{}, I1{}, I1{});
+			if (kt + 2 < p.nkt)
+				step(kt + 2, I2{}, I0{}, I1{});
+			if (kt + 3 < p.nkt)
+				step(kt + 3, I3{}, I1{}, I1{});
+			if (kt + 4 < p.nkt)
+				step(kt + 4, I4{}, I0{}, I1{});
+			if (kt + 5 < p.nkt)
+				step(kt + 5, I5{}, I1{}, I1{});
 		}
-		if (++n_tap == p.taps) {
-			n_tap = n_kh = n_kw = 0;
-			++n_cb;
-		}
-	};
-	if (mytiles > 0) {
-		/* Every step of the main loop issues the same memory operations whatever its K-tile: the compiler
-		 * sets its waits for the worst of the paths that meet, and an operation on one path only makes
-		 * every step wait for everything (measured: 390 -> 650 cycles a step). */
-		frags(bf[0]);
-		auto step = [&](int kt, auto slot_, auto par_, auto tail_) {
-			constexpr int slot = decltype(slot_)::value;	/* kt % CP_DEPTH */
-			constexpr int par = decltype(par_)::value;	/* kt % 2: the register set that holds K-tile kt */
-			if (!decltype(tail_)::value || kt + 1 < p.nkt)
-				frags(bf[par ^ 1]);	/* requested under this K-tile's MFMAs */
+	} else {
+		/* Streamed: a block's taps are groups of D steps, step i of a group on weight slot i; the fragments
+		 * of the next K-tile of the block are requested under a step's MFMAs (past a block's last tap: its
+		 * last tap's again, which nothing uses).  The first group after a block's patch loads went out is
+		 * straight-line code of its own: its waits count the patch loads as younger than the weights they
+		 * wait for; from the second group on the patch loads are older than every weight in flight. */
+		static_assert(D % 2 == 1, "taps / D odd and D odd: a block has an odd number of steps");
+		int c_kh = 0, c_kw = 0;		/* kernel row and column of the K-tile whose fragments were requested last */
+		auto frags = [&](intx4 (&bb)[3], int cb, int kh, int kw) {
+			const unsigned char *pb = lds + cb * blk + (kh * p.pw + kw) * 16;
+#pragma unroll
+			for (int j = 0; j < 3; j++)
+				bb[j] = *(const intx4 *)(pb + pp0[j]);
+		};
+		/* one step: K-tile (cb, tap t) on slot `slot`, its fragments in bf[par] */
+		auto step = [&](int cb, int t, auto slot_, auto par_) {
+			constexpr int slot = decltype(slot_)::value, par = decltype(par_)::value;
+			if (c_kw + 1 < p.kW)
+				++c_kw;
+			else if (c_kh + 1 < p.kH) {
+				c_kw = 0;
+				++c_kh;
+			}
+			frags(bf[par ^ 1], cb, c_kh, c_kw);
 			const intx4 a = wr[slot];
 #pragma unroll
 			for (int j = 0; j < 3; j++)
 				acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bf[par][j], acc[j], 0, 0, 0);
-			CP_WFETCH(slot, kt + CP_DEPTH);
+			CP_WFETCH(slot, cb * p.taps + t + D);
 		};
-		typedef std::integral_constant<int, 0> I0;
-		typedef std::integral_constant<int, 1> I1;
-		typedef std::integral_constant<int, 2> I2;
-		typedef std::integral_constant<int, 3> I3;
-		typedef std::integral_constant<int, 4> I4;
-		typedef std::integral_constant<int, 5> I5;
-		int kt = 0;
-		for (; kt + 6 < p.nkt; kt += 6) {	/* (kt + 6 < nkt: the K-tile after these six exists) */
-			step(kt, I0{}, I0{}, I0{});
-			step(kt + 1, I1{}, I1{}, I0{});
-			step(kt + 2, I2{}, I0{}, I0{});
-			step(kt + 3, I3{}, I1{}, I0{});
-			step(kt + 4, I4{}, I0{}, I0{});
-			step(kt + 5, I5{}, I1{}, I0{});
-		}
-		if (kt < p.nkt)
-			step(kt, I0{}, I0{}, I1{});
-		if (kt + 1 < p.nkt)
-			step(kt + 1, I1{}, I1{}, I1{});
-		if (kt + 2 < p.nkt)
-			step(kt + 2, I2{}, I0{}, I1{});
-		if (kt + 3 < p.nkt)
-			step(kt + 3, I3{}, I1{}, I1{});
-		if (kt + 4 < p.nkt)
-			step(kt + 4, I4{}, I0{}, I1{});
-		if (kt + 5 < p.nkt)
-			step(kt + 5, I5{}, I1{}, I1{});
+		const int groups = p.taps / D;	/* odd */
+		auto block = [&](int cb, auto more_) {
+			constexpr bool more = decltype(more_)::value;	/* another block follows: its patch is streamed */
+			c_kh = c_kw = 0;
+			frags(bf[0], cb, 0, 0);
+			if constexpr (more)
+				patch_fetch(cb + 1);
+			cp_static_for<0, D>([&](auto i_) {
+				constexpr int i = decltype(i_)::value;
+				step(cb, i, i_, std::integral_constant<int, i % 2>{});
+			});
+			for (int g = 1; g < groups; g += 2)
+				cp_static_for<0, 2 * D>([&](auto i_) {
+					constexpr int i = decltype(i_)::value;
+					step(cb, g * D + i, std::integral_constant<int, i % D>{}, std::integral_constant<int, (i + 1) % 2>{});
+				});
+			if constexpr (more) {
+				patch_store(cb + 1);
+				__syncthreads();
+			}
+		};
+		for (int cb = 0; cb + 1 < nblocks; cb++)
+			block(cb, std::true_type{});
+		column_terms();
+		block(nblocks - 1, std::false_type{});
 	}
 #undef CP_WFETCH
 	__syncthreads();	/* everybody is done with the patch (and the tables are written) */
@@ -556,16 +673,35 @@ extern "C" void thhip_conv2d_u8_patch(const unsigned char *x, const void *wpatch
 	p.c_off = c_off; p.c_mult = c_mult; p.c_shift = c_shift;
 	p.act = act; p.ithr = thr; p.ival = val;
 	const int bands = pool ? (p.pH + p.rb - 1) / p.rb : (p.oH + p.rb - 1) / p.rb;
-	static bool attr_set;
-	if (!attr_set) {	/* more than 64 KiB of dynamic LDS has to be asked for */
-		hipcheck(hipFuncSetAttribute((const void *)conv_u8_patch_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, CP_LDS_MAX));
-		hipcheck(hipFuncSetAttribute((const void *)conv_u8_patch_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, CP_LDS_MAX));
-		attr_set = true;
-	}
+	/* the patch streamed block by block where the kernel's taps come in an odd number of groups of 3 or 5,
+	 * there are at least two plane blocks and a thread moves a block in two loads */
+	const int npix_max = ((pool ? 2 * p.rb + 1 : p.rb) + kH - 1) * p.pw;
+	const bool can_stream = Ci >= 128 && npix_max * 4 <= 2 * CP_THREADS;
+	const int D = !can_stream ? 0 : p.taps % 5 == 0 && (p.taps / 5) % 2 ? 5 : p.taps % 3 == 0 && (p.taps / 3) % 2 ? 3 : 0;
 	ThhipLaunchScope scope(THHIP_FAM_CONV_I8, 2.0 * Co * (double)p.K * B * p.oH * p.oW);
 	const dim3 grid(bands, Co / 64, B);
-	if (pool)
-		conv_u8_patch_kernel<true><<<grid, dim3(CP_THREADS), ldsbytes, thhip_stream()>>>(p);
-	else
-		conv_u8_patch_kernel<false><<<grid, dim3(CP_THREADS), ldsbytes, thhip_stream()>>>(p);
+	static bool attr_set[6];
+#define CP_GO(POOL_, D_, I_) do { \
+		if (!attr_set[I_]) {	/* more than 64 KiB of dynamic LDS has to be asked for */ \
+			hipcheck(hipFuncSetAttribute((const void *)conv_u8_patch_kernel<POOL_, D_>, hipFuncAttributeMaxDynamicSharedMemorySize, CP_LDS_MAX)); \
+			attr_set[I_] = true; \
+		} \
+		conv_u8_patch_kernel<POOL_, D_><<<grid, dim3(CP_THREADS), ldsbytes, thhip_stream()>>>(p); \
+	} while (0)
+	if (pool) {
+		if (D == 5)
+			CP_GO(true, 5, 0);
+		else if (D == 3)
+			CP_GO(true, 3, 1);
+		else
+			CP_GO(true, 0, 2);
+	} else {
+		if (D == 5)
+			CP_GO(false, 5, 3);
+		else if (D == 3)
+			CP_GO(false, 3, 4);
+		else
+			CP_GO(false, 0, 5);
+	}
+#undef CP_GO
 }
