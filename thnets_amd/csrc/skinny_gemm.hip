@@ -485,6 +485,19 @@ __global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned ch
 	B = min(B - (int)blockIdx.y * (16 * NCG), 16 * NCG);
 	constexpr int XBUF = NCG * 16 * LU_CHUNK;
 	const int tid = threadIdx.x, lane = tid & 63;
+	/* what this thread needs to finish its outputs (row rr of every row block, batch column bcol), asked
+	 * for now: at the end a trip to memory would be all the kernel waits for */
+	const int rr = tid & 15, bcol = tid >> 4;
+	constexpr bool EARLY = NCG < 4;	/* (four column groups leave no registers for it) */
+	int rsum[RB], radd[RB];
+	if constexpr (EARLY) {
+#pragma unroll
+		for (int rb = 0; rb < RB; rb++) {
+			const int o = min(((int)blockIdx.x * RB + rb) * LU_ROWS + rr, nOut - 1);
+			rsum[rb] = rowsum[o];
+			radd[rb] = addend ? addend[o] : 0;
+		}
+	}
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 	const int m = lane & 15, q = lane >> 4;
 	const int nchunks = (nsteps + LU_WAVES - 1) / LU_WAVES;
@@ -598,8 +611,8 @@ __global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned ch
 	 * Waves 8..15 hand their tiles to waves 0..7, those put the pair sums into LDS,
 	 * and every thread finishes one (row, column).  (The loop's last barrier has
 	 * passed: the activation buffers are free.) */
-	int (*red)[NCG * 4][64] = (int (*)[NCG * 4][64])lds;				/* [8] */
-	int *colsum = (int *)(lds + 8 * NCG * 4 * 64 * sizeof(int));			/* [16 * NCG] */
+	int (*red)[RB][NCG * 4][64] = (int (*)[RB][NCG * 4][64])lds;			/* [8] */
+	int *colsum = (int *)(lds + 8 * RB * NCG * 4 * 64 * sizeof(int));		/* [16 * NCG] */
 	/* a staging thread summed its pieces of rows wave, wave + 16, ...: the lanes of a
 	 * wavefront hold the 64 parts of one column sum */
 #pragma unroll
@@ -611,53 +624,65 @@ __global__ __launch_bounds__(LU_THREADS) void linear_u8_kernel(const unsigned ch
 		if (lane == 0)
 			colsum[g * 16 + wave] = v;
 	}
+	if constexpr (!EARLY) {
+#pragma unroll
+		for (int rb = 0; rb < RB; rb++) {
+			const int o = min(((int)blockIdx.x * RB + rb) * LU_ROWS + rr, nOut - 1);
+			rsum[rb] = rowsum[o];
+			radd[rb] = addend ? addend[o] : 0;
+		}
+	}
+	/* (every row block at once: three barriers whatever RB) */
+	if (wave >= 8) {
+#pragma unroll
+		for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+			for (int gg = 0; gg < NCG; gg++)
+#pragma unroll
+				for (int r = 0; r < 4; r++)
+					red[wave - 8][rb][gg * 4 + r][lane] = acc[rb][gg][r];
+	}
+	__syncthreads();
+	if (wave < 8) {
+#pragma unroll
+		for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+			for (int gg = 0; gg < NCG; gg++)
+#pragma unroll
+				for (int r = 0; r < 4; r++)
+					acc[rb][gg][r] += red[wave][rb][gg * 4 + r][lane];
+	}
+	__syncthreads();
+	if (wave < 8) {
+#pragma unroll
+		for (int rb = 0; rb < RB; rb++)
+#pragma unroll
+			for (int gg = 0; gg < NCG; gg++)
+#pragma unroll
+				for (int r = 0; r < 4; r++)
+					red[wave][rb][gg * 4 + r][lane] = acc[rb][gg][r];
+	}
+	__syncthreads();
 	/* thread -> (row rr, batch column bcol): neighbouring threads write neighbouring bytes of y */
-	const int rr = tid & 15, bcol = tid >> 4;
 	const int g = (bcol >> 4) % NCG, n = bcol & 15;	/* (bcol < 16 NCG is checked before use) */
 	const int src = (rr >> 2) * 16 + n, reg = g * 4 + (rr & 3);
 #pragma unroll
 	for (int rb = 0; rb < RB; rb++) {
-		if (rb)
-			__syncthreads();	/* the previous block's sums have been read */
-		if (wave >= 8) {
-#pragma unroll
-			for (int gg = 0; gg < NCG; gg++)
-#pragma unroll
-				for (int r = 0; r < 4; r++)
-					red[wave - 8][gg * 4 + r][lane] = acc[rb][gg][r];
-		}
-		__syncthreads();
-		if (wave < 8) {
-#pragma unroll
-			for (int gg = 0; gg < NCG; gg++)
-#pragma unroll
-				for (int r = 0; r < 4; r++)
-					acc[rb][gg][r] += red[wave][gg * 4 + r][lane];
-		}
-		__syncthreads();
-		if (wave < 8) {
-#pragma unroll
-			for (int gg = 0; gg < NCG; gg++)
-#pragma unroll
-				for (int r = 0; r < 4; r++)
-					red[wave][gg * 4 + r][lane] = acc[rb][gg][r];
-		}
-		__syncthreads();
 		const int o = ((int)blockIdx.x * RB + rb) * LU_ROWS + rr;
 		if (bcol >= 16 * NCG || bcol >= B || o >= nOut)
 			continue;
 		int sum = 0;
 #pragma unroll
 		for (int wv = 0; wv < 8; wv++)
-			sum += red[wv][reg][src];
+			sum += red[wv][rb][reg][src];
 		const int csum = colsum[bcol];
-		const int t = sum + offB * rowsum[o] + K * offA * offB + offA * csum;
+		const int t = sum + offB * rsum[rb] + K * offA * offB + offA * csum;
 		unsigned u = ((unsigned)t + (unsigned)c_off) * (unsigned)c_mult;
 		u += c_shift < 1 ? 0u : 1u << (c_shift - 1);
 		int code = (int)u >> c_shift;
 		code = code < 0 ? 0 : code > 255 ? 255 : code;
 		if (addend) {
-			const int sa = code + addend[o];
+			const int sa = code + radd[rb];
 			code = sa > 255 ? 255 : (sa & 255);
 		}
 		if (act)
