@@ -823,6 +823,64 @@ def test_conv_half_patch_kernel_with_pooling(hiplib, oracle, dt):
 
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
+def test_conv_half_whole_image_patch_kernel(hiplib, oracle, dt):
+    """3x3 / stride 1 / padding 1 layers of 256 and 512 planes on outputs of at most 14 x 14, one whole
+    image per workgroup (VGG-16's last three convolutions): 32 and 64 planes per workgroup (forced, and as
+    the dispatcher picks them by the number of workgroups), 14 x 14, 13 x 13 and 12 x 14 images, a plane
+    count that leaves a partial block, both output orders; alone against the oracle and the 64 x 64 tile,
+    and with the 2x2 pooling in the epilogue bit for bit the pooled plain result (odd sizes drop the last
+    row and column)."""
+    from thnets_amd import api
+    g = cases.rng(916)
+    shapes = [(16, 512, 14, 14, 512), (4, 256, 13, 13, 1024), (8, 512, 12, 14, 544), (64, 256, 14, 14, 256), (6, 256, 14, 11, 736)]
+    try:
+        for (B, Ci, H, W, Co) in shapes:
+            x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+            w = g.standard_normal((Co, Ci, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * 9)))
+            b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            sc = (g.uniform(0.5, 1.5, Co) * g.choice([-1.0, 1.0], Co)).astype(np.float32)
+            xr = api.from_device_dtype(api.to_device_dtype(hiplib, x, dt), x.shape, dt)
+            wr = api.from_device_dtype(api.to_device_dtype(hiplib, w, dt), w.shape, dt)
+            raw = oracle.conv2d(xr, wr, None, (1, 1), (1, 1))
+            want = np.maximum(raw * sc[None, :, None, None] + b[None, :, None, None], 0)
+            pH, pW = H // 2, W // 2
+            plain = {}
+            for y_cl in (1, 0):
+                hiplib.thhip_conv_set_tuning(64, 64, 0, 0)
+                narrow = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
+                for planes in (3, 4, 0):      # 32 planes, 64 planes, the dispatcher's choice
+                    G.note("whole-image patch kernel %s y_cl %d dtype %d planes %d" % ((B, Ci, H, W, Co), y_cl, dt, planes))
+                    hiplib.thhip_conv_set_tuning(64 if planes else 0, 1 if planes else 0, 0, planes)
+                    got = G.conv2d_layout(hiplib, x, w, b, (1, 1), (1, 1), act=1, dtype=dt, x_cl=1, y_cl=y_cl, scale=sc)
+                    G.assert_close(got, want, HALF_TOL, str((B, Ci, H, W, Co, y_cl, planes)))
+                    G.assert_close(got, narrow, 1e-2, "vs the 64x64 tile " + str((B, Ci, H, W, Co, y_cl, planes)))
+                    if planes == 3:
+                        plain[y_cl] = got
+                    else:
+                        assert np.array_equal(got, plain[y_cl]), (B, Ci, H, W, Co, y_cl, planes)   # (the same sums in the same order)
+            hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+            ref = plain[0][:, :, :2 * pH, :2 * pW].reshape(B, Co, pH, 2, pW, 2).max(axis=(3, 5))
+            for y_cl in (1, 0):
+                G.note("whole-image patch kernel with pooling %s y_cl %d dtype %d" % ((B, Ci, H, W, Co), y_cl, dt))
+                assert hiplib.thhip_conv2d_pool2_supported(B, Ci, H, W, Co, 3, 3, 1, 1, 1, 1, dt, 1, y_cl)
+                dx = api.to_device_dtype(hiplib, np.ascontiguousarray(x.transpose(0, 2, 3, 1)), dt)
+                wp = hiplib.thhip_conv_pack_weight_layout(np.ascontiguousarray(w).ctypes.data, Co, Ci, 3, 3, dt, 1)
+                db, ds = api.DeviceArray(hiplib, b), api.DeviceArray(hiplib, sc)
+                dy = api.DeviceArray(hiplib, nbytes=B * Co * pH * pW * 2)
+                hiplib.thhip_conv2d_layout_pool2(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, B, Ci, H, W, Co, 3, 3, 1, 1, 1, 1,
+                                                 1, 0.0, 0.0, dt, 1, y_cl)
+                hiplib.thhip_sync()
+                if y_cl:
+                    got = np.ascontiguousarray(api.from_device_dtype(dy, (B, pH, pW, Co), dt).transpose(0, 3, 1, 2))
+                else:
+                    got = api.from_device_dtype(dy, (B, Co, pH, pW), dt)
+                hiplib.thhip_free(wp)
+                assert np.array_equal(got, ref), (B, Ci, H, W, Co, y_cl, int((got != ref).sum()))
+    finally:
+        hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
+
+
+@pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_maxpool_and_relayout_half_channels_last(hiplib, oracle, dt):
     from thnets_amd import api
     g = cases.rng(909)

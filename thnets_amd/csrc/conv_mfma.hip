@@ -32,143 +32,7 @@
 #include <vector>
 #include "thhip_internal.h"
 
-#define CONV_THREADS 256
-#define CONV_C4_SLACK 16	/* bytes before and after the four-plane pixel copy of an input */
-
-struct ConvParams {
-	const void *x;
-	const void *wp;
-	const float *bias;
-	const float *scale;	/* float types: per-plane factor applied before the bias (folded batch norm), or NULL */
-	void *y;
-	int B, Ci, H, W, Co, kH, kW, dH, dW, padH, padW, oH, oW;
-	int K, KC, N, oHW, HW, kHW;
-	unsigned magic_khw, magic_kw, magic_ci;	/* low words of floor(2^32/d)+1 */
-	unsigned mhi_khw, mhi_kw, mhi_ci;	/* their bit 32 (set only for d == 1) */
-	int act;
-	float thr, val;
-	int tiles_m, tiles_n;
-	int mparts;		/* the tile grid is cut mparts x (8 / mparts) over the XCDs */
-	unsigned x_bytes;
-	unsigned w_bytes;	/* packed weights (the wide kernel's buffer descriptor) */
-	int pool;		/* the 2x2 / stride 2 max pooling that follows is done in the epilogue (conv_patch_kernel, conv_f32_direct_kernel) */
-	/* conv_f32_direct_kernel: a second tensor of the output's shape combined with the result after the
-	 * (factor,) bias and Threshold: res_mode 1: v + res_c * res, 2: res + res_c * v; then ReLU if res_act
-	 * (the table add of a residual block and the Threshold after it, modules/CAddTable.c:59-70) */
-	const float *res;
-	int res_mode, res_act;
-	float res_c;
-	int cl_shift;		/* channels-last input in whole K-tiles of planes: log2 of the K-tile (K runs block, tap, plane); else 0 */
-	int pW, pHW, npool;	/* pooled width, plane size and positions in all; conv_f32_direct_kernel then walks the
-				 * positions in blocks of 64 = sixteen windows (conv_pool_member), N = 64 ceil(npool / 16) */
-	unsigned x_tail;	/* uint8: bytes of the padding code that follow x (0: none) */
-	/* split-K: S workgroups share an output tile, each over a K range */
-	int splitk;
-	int *ws;		/* [tile][S][BM*BN] partial accumulators (float or int bits) */
-	unsigned *cnt;		/* [tile] arrival counters, zero between launches */
-	/* conv_f32_direct_kernel: K split of the last tiles of every XCD only (0 slots: none) */
-	int tail_slots;		/* workgroups an XCD holds at once */
-	int tail_max;		/* most parts per tile */
-	int tail_cap;		/* scratch blocks (parts of BM*BN sums) reserved per XCD: [xcd][tile][part] */
-	int tail_tiles;		/* most cut tiles of an XCD */
-	int tail_round;		/* 1: an XCD with less than one whole round of tiles is left uncut */
-	/* conv_f32_direct_kernel with a K split of the whole layer: a max pooling that follows, taken by the kernel
-	 * that adds the parts (pk_kH 0: none); pk_oH x pk_oW is the pooled plane */
-	int pk_kH, pk_kW, pk_dH, pk_dW, pk_padH, pk_padW, pk_oH, pk_oW;
-	/* uint8 path only */
-	const int *rowsum;	/* sum_k (w[m][k] - 128), per packed row */
-	const int *addend;	/* per-plane bias addend, or NULL */
-	int zero, offA, offB, c_off, c_mult, c_shift, ithr, ival;
-	int kwv;		/* GM_PIXELS4: vectors (four pixels) per kernel row; magic_kw divides by it */
-	unsigned c4_fill;	/* GM_PIXELS4: one pixel outside the image */
-	/* host side only: memory order of x and y, 0 = [B][C][H][W], 1 = [B][H][W][C] */
-	int x_cl, y_cl;
-};
-
-/* floor(n / d) = (n * m) >> 32 for n*d < 2^32 with the 33-bit m = floor(2^32/d) + 1,
- * evaluated as n*m_hi + umulhi(n, m_lo); m_hi is 1 only for d == 1. */
-static inline unsigned long long conv_magic(unsigned d)
-{
-	return (1ull << 32) / d + 1;
-}
-
-/* Chunks per K-tile (one LDS stage).  An int8 MFMA retires 32 k in the time
- * an fp32 one retires 1, so where the gather is cheap (channels-last codes)
- * deeper K-tiles keep the work per barrier up. */
-#define CONV_KCH_U8_CL 2
-#define CONV_KCH_F32 4
-#define CONV_KCH_HALF_CL 2
-__host__ __device__ constexpr int conv_kch(int dtype, bool x_cl)
-{
-	return dtype == THHIP_U8 ? (x_cl ? CONV_KCH_U8_CL : 2) : dtype == THHIP_F32 ? CONV_KCH_F32 : (x_cl ? CONV_KCH_HALF_CL : 2);
-}
-
-/* Waves per SIMD to ask the register allocator for (what each tile reaches
- * without spilling): more for the small tiles, whose residency matters most. */
-__host__ __device__ constexpr int conv_min_waves(int dtype, int tile_elems, bool generic_gather, int kch)
-{
-	const bool deep = dtype == THHIP_F32 && kch > 2;	/* fp32 K-tiles of 32: LDS limits first */
-	return generic_gather ? 1
-		: tile_elems <= 64 * 64 ? (deep ? 3 : 4)
-		: tile_elems <= 128 * 64 ? (deep ? 2 : 4)
-		: (deep ? 1 : 2);
-}
-
-template <int DT> struct ConvTraits;
-template <> struct ConvTraits<THHIP_F32> {
-	static constexpr int CHUNK = 8;		/* k values per chunk */
-	static constexpr int VEC = 4;		/* elements per 16-byte lane vector */
-	typedef float elem;
-};
-template <> struct ConvTraits<THHIP_F16> {
-	static constexpr int CHUNK = 16;
-	static constexpr int VEC = 8;
-	typedef _Float16 elem;
-};
-template <> struct ConvTraits<THHIP_BF16> {
-	static constexpr int CHUNK = 16;
-	static constexpr int VEC = 8;
-	typedef __bf16 elem;
-};
-
-template <> struct ConvTraits<THHIP_U8> {
-	static constexpr int CHUNK = 32;
-	static constexpr int VEC = 16;
-	typedef unsigned char elem;
-};
-
-template <int DT> struct ConvAcc { typedef floatx16 T; };
-template <> struct ConvAcc<THHIP_U8> { typedef intx16 T; };
-
-template <int DT>
-__device__ __forceinline__ void conv_mma(typename ConvAcc<DT>::T &acc, const floatx4 &a, const floatx4 &b);
-
-template <>
-__device__ __forceinline__ void conv_mma<THHIP_F32>(floatx16 &acc, const floatx4 &a, const floatx4 &b)
-{
-	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[1], b[1], acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[2], b[2], acc, 0, 0, 0);
-	acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[3], b[3], acc, 0, 0, 0);
-}
-
-template <>
-__device__ __forceinline__ void conv_mma<THHIP_F16>(floatx16 &acc, const floatx4 &a, const floatx4 &b)
-{
-	acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), acc, 0, 0, 0);
-}
-
-template <>
-__device__ __forceinline__ void conv_mma<THHIP_BF16>(floatx16 &acc, const floatx4 &a, const floatx4 &b)
-{
-	acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
-}
-
-template <>
-__device__ __forceinline__ void conv_mma<THHIP_U8>(intx16 &acc, const floatx4 &a, const floatx4 &b)
-{
-	acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(intx4, a), __builtin_bit_cast(intx4, b), acc, 0, 0, 0);
-}
+#include "conv_common.h"
 
 /* gemmlowp's legacy output stage as the reference calls it (lowp/gemm8.cc:13-16):
  * ((acc + c_off) * c_mult + rounding) >> c_shift in wrapping 32-bit arithmetic,
@@ -983,75 +847,6 @@ __attribute__((amdgpu_waves_per_eu(conv_min_waves(DT, BM * BN, GM == 0, KCH), 8)
  * fragments of tile kt, after it that stage is free for tile kt+4 and tile
  * kt+1 is complete, so its first fragments are fetched under the second
  * chunk's MFMAs. */
-#define WIDE_LDS(p) ((__attribute__((address_space(3))) void *)(p))
-/* s_waitcnt immediate that waits for all but n vector-memory operations only */
-#define WIDE_VMCNT(n) (0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
-
-/* Waits until at most N vector-memory operations of the wave are outstanding
- * (LGKM0: and no LDS / scalar ones).  The builtin wants a literal: a value that
- * depends on a template parameter makes the host pass drop the kernel. */
-template <int N, bool LGKM0>
-__device__ __forceinline__ void wide_wait()
-{
-	static_assert(N >= 0 && N <= 48, "add the count below");
-#define WIDE_WAIT_CASE(n)                                                          \
-	if constexpr (N == n) {                                                    \
-		if constexpr (LGKM0)                                               \
-			__builtin_amdgcn_s_waitcnt(WIDE_VMCNT(n) & 0xf0ff);        \
-		else                                                               \
-			__builtin_amdgcn_s_waitcnt(WIDE_VMCNT(n));                 \
-	}
-	WIDE_WAIT_CASE(0)
-	WIDE_WAIT_CASE(1)
-	WIDE_WAIT_CASE(2)
-	WIDE_WAIT_CASE(3)
-	WIDE_WAIT_CASE(4)
-	WIDE_WAIT_CASE(5)
-	WIDE_WAIT_CASE(6)
-	WIDE_WAIT_CASE(7)
-	WIDE_WAIT_CASE(8)
-	WIDE_WAIT_CASE(9)
-	WIDE_WAIT_CASE(10)
-	WIDE_WAIT_CASE(11)
-	WIDE_WAIT_CASE(12)
-	WIDE_WAIT_CASE(13)
-	WIDE_WAIT_CASE(14)
-	WIDE_WAIT_CASE(15)
-	WIDE_WAIT_CASE(16)
-	WIDE_WAIT_CASE(17)
-	WIDE_WAIT_CASE(18)
-	WIDE_WAIT_CASE(19)
-	WIDE_WAIT_CASE(20)
-	WIDE_WAIT_CASE(21)
-	WIDE_WAIT_CASE(22)
-	WIDE_WAIT_CASE(23)
-	WIDE_WAIT_CASE(24)
-	WIDE_WAIT_CASE(25)
-	WIDE_WAIT_CASE(26)
-	WIDE_WAIT_CASE(27)
-	WIDE_WAIT_CASE(28)
-	WIDE_WAIT_CASE(29)
-	WIDE_WAIT_CASE(30)
-	WIDE_WAIT_CASE(31)
-	WIDE_WAIT_CASE(32)
-	WIDE_WAIT_CASE(33)
-	WIDE_WAIT_CASE(34)
-	WIDE_WAIT_CASE(35)
-	WIDE_WAIT_CASE(36)
-	WIDE_WAIT_CASE(37)
-	WIDE_WAIT_CASE(38)
-	WIDE_WAIT_CASE(39)
-	WIDE_WAIT_CASE(40)
-	WIDE_WAIT_CASE(41)
-	WIDE_WAIT_CASE(42)
-	WIDE_WAIT_CASE(43)
-	WIDE_WAIT_CASE(44)
-	WIDE_WAIT_CASE(45)
-	WIDE_WAIT_CASE(46)
-	WIDE_WAIT_CASE(47)
-	WIDE_WAIT_CASE(48)
-#undef WIDE_WAIT_CASE
-}
 
 /* XCD x's rectangle of the tile grid (mparts x 8/mparts rectangles): first tile
  * row, rows, first tile column, and the number of tiles. */
@@ -1679,317 +1474,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void conv_wide_tail_finish_kernel(C
 /* 3x3, stride 1, 64 to 512 planes in: taps from an input patch in LDS */
 /* ------------------------------------------------------------------ */
 
-/* With 64 input planes a K-tile of the kernels above moves 64 bytes per
- * position from L2 for 32 multiply-adds per output plane, nine times per
- * pixel (once per tap), and the path from L2 to LDS, not the matrix core, sets
- * their time.  Here a workgroup owns 8 rows x 32 columns of one image's output,
- * copies the 10 x 34 pixel patch those positions read once per block of 32
- * planes (21 KiB, straight to LDS), and takes the B fragments of all nine taps
- * from it: a fragment of tap (kh, kw) is the patch shifted by (kh, kw).  The
- * pipeline is conv_f32_patch_kernel's: two patch buffers, the next block's six
- * loads per wavefront spread over the nine taps of this one, the weights
- * (K-tiles of one tap x 32 planes) through a ring of three stages, the nine
- * steps of a block straight-line code with constant wait counts.  (An earlier
- * form held one patch of 64 planes, 43.5 KiB, and drained the pipeline between
- * blocks: VGG-16 fp16 batch 16 0.735 -> 0.713 ms, batch 64 2.33 -> 2.26 ms.)
- *
- * Patch layout: 1 KiB blocks of sixteen pixels x four 16-byte vectors, pixel pp
- * of the patch (row-major, 34 wide) in block pp / 16; vector v of pixel pp sits
- * in slot 4 pp + (v ^ ((pp / 4) % 4)).  A fragment read takes one vector index
- * from 32 consecutive pixels, sixteen lanes (256 bytes, every bank once) a cycle;
- * pixels four apart share their banks, and the swizzle gives any four such in a
- * run of sixteen four different slots, wherever the run starts.  (With the key
- * (pp / 2) % 4, which serves runs of eight, the counters showed conflicts in a
- * tenth of the cycles.)  Pixels outside the image are fetched out of the
- * buffer's range and arrive as zeros.
- *
- * Four waves; wave w computes all BM planes of tile rows 2w and 2w+1. */
-#define PATCH_TW 32
-#define PATCH_TH 8
-
-template <int DT, bool CLO, int BM, int CI, bool POOL>
-__global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
-{
-#if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
-	typedef ConvTraits<DT> TR;
-	typedef typename TR::elem elem;
-	static_assert(TR::CHUNK == 16 && sizeof(elem) == 2, "a half type");
-	constexpr int TW = PATCH_TW, TH = PATCH_TH, PW = TW + 2, PH = TH + 2, PCI = 32, NB = CI / PCI;
-	constexpr int NPIX = PW * PH, WAVES = 4;
-	constexpr int BL = ((NPIX + 15) / 16 + WAVES - 1) / WAVES;	/* patch loads (sixteen pixels x four vectors) per wave and block */
-	constexpr int B_VECS = BL * WAVES * 64;				/* a buffer: every load's 1 KiB, the unused ones' too */
-	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = 3;
-	constexpr int A_VECS = MB * KCH * 64, A_PW = MB * KCH / WAVES;
-	static_assert(CI % (2 * PCI) == 0 && MB * KCH % WAVES == 0 && TH == 2 * WAVES && BL <= 8, "shape");
-	/* (one array, every stage and buffer at a constant offset: conv_f32_patch_kernel says why) */
-	__shared__ floatx4 lds[NST * A_VECS + 2 * B_VECS];
-	floatx4 *const astage = lds;
-	floatx4 *const patch0 = lds + NST * A_VECS, *const patch1 = patch0 + B_VECS;
-
-	const int tid = threadIdx.x;
-	const int lane = tid & 63;
-	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-
-	/* consecutive tiles (plane block fastest, then along the row) share halo
-	 * pixels: each XCD takes one run of them */
-	const int tx_n = (p.oW + TW - 1) / TW, ty_n = (p.oH + TH - 1) / TH;
-	int tile_m, tx, ty, img;
-	{
-		const int total = p.tiles_m * p.tiles_n, per_xcd = (total + 7) / 8;
-		const int local = blockIdx.x >> 3;
-		const int t = (blockIdx.x & 7) * per_xcd + local;
-		if (local >= per_xcd || t >= total)
-			return;
-		tile_m = t % p.tiles_m;
-		const int sp = t / p.tiles_m;
-		tx = sp % tx_n;
-		ty = (sp / tx_n) % ty_n;
-		img = sp / (tx_n * ty_n);
-	}
-
-	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
-	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
-	/* ---- what this lane fetches of every block of 32 planes: load t of the wave covers pixels
-	 * 16 (wave + 4 t) .. + 15 of the patch, this lane pixel lane / 4 of them, vector lane % 4
-	 * through the swizzle ---- */
-	unsigned voff_[BL];
-#pragma unroll
-	for (int t = 0; t < BL; t++) {
-		const int pp = (wave + WAVES * t) * 16 + (lane >> 2);
-		const int v = (lane & 3) ^ ((pp >> 2) & 3);
-		const int pr = pp / PW, pc = pp - pr * PW;
-		const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
-		const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-		voff_[t] = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + v * 8) * (int)sizeof(elem)) : 0x80000000u;
-	}
-	/* this wave's weight blocks of a K-tile: wave + 4 i counts (chunk, 32-row block) */
-	unsigned a_off_[A_PW];
-	int a_lds_[A_PW];
-#pragma unroll
-	for (int i = 0; i < A_PW; i++) {
-		const int idx = wave + WAVES * i, mbi = idx % MB, kci = idx / MB;
-		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
-		a_lds_[i] = (kci * MB + mbi) * 64;
-	}
-
-	/* the weights of K-tile (block hb of 32 planes, tap): K runs (block, tap, plane) in chunks of 16 */
-	auto issue_a = [&](auto st_, int hb, int tap) {
-		constexpr int st = decltype(st_)::value;
-		const unsigned kc = (unsigned)((hb * 9 + tap) * KCH);
-#pragma unroll
-		for (int i = 0; i < A_PW; i++)
-			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16,
-				hb < NB ? lane * 16 : 0x80000000u, a_off_[i] + kc * 1024u, 0, 0);
-	};
-	auto issue_b = [&](auto t_, int hb, auto buf_) {
-		constexpr int buf = decltype(buf_)::value, t = decltype(t_)::value;
-		__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS((buf ? patch1 : patch0) + (wave + WAVES * t) * 64), 16,
-			hb < NB ? voff_[t] : 0x80000000u, hb < NB ? hb * PCI * (int)sizeof(elem) : 0, 0, 0);
-	};
-
-	/* patch pixel of this lane's position at tap (0, 0), for its two tile rows */
-	int pbase_[TN];
-#pragma unroll
-	for (int j = 0; j < TN; j++)
-		pbase_[j] = (2 * wave + j) * PW + (lane & 31);
-	floatx4 af[2][TM], bf[2][TN];
-	auto read_frags = [&](auto st_, auto buf_, auto tap_, int c, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
-		constexpr int st = decltype(st_)::value, buf = decltype(buf_)::value, tap = decltype(tap_)::value;
-		const floatx4 *la = astage + st * A_VECS;
-#pragma unroll
-		for (int i = 0; i < TM; i++)
-			a[i] = la[(c * MB + i) * 64 + lane];
-		const int v = c * 2 + (lane >> 5);
-#pragma unroll
-		for (int j = 0; j < TN; j++) {
-			const int pp = pbase_[j] + (tap / 3) * PW + tap % 3;
-			b[j] = (buf ? patch1 : patch0)[pp * 4 + (v ^ ((pp >> 2) & 3))];
-		}
-	};
-
-	typename ConvAcc<DT>::T acc[TM][TN];
-#pragma unroll
-	for (int i = 0; i < TM; i++)
-#pragma unroll
-		for (int j = 0; j < TN; j++)
-#pragma unroll
-			for (int r = 0; r < 16; r++)
-				acc[i][j][r] = 0;
-	auto mma = [&](int set) {
-#pragma unroll
-		for (int i = 0; i < TM; i++)
-#pragma unroll
-			for (int j = 0; j < TN; j++)
-				conv_mma<DT>(acc[i][j], af[set][i], bf[set][j]);
-	};
-
-	typedef std::integral_constant<int, 0> C0;
-	typedef std::integral_constant<int, 1> C1;
-	typedef std::integral_constant<int, 2> C2;
-	/* patch loads of the next block: BL of them over the nine steps of this one, step `tap` issues
-	 * numbers [PB(tap), PB(tap + 1)), none in the last */
-#define CONV_PATCH_PB(tap) ((BL * ((tap) < 8 ? (tap) : 8) + 7) / 8)
-	{
-		auto all_b = [&](auto self, auto t_) {
-			constexpr int t = decltype(t_)::value;
-			if constexpr (t < BL) {
-				issue_b(t_, 0, C0{});
-				self(self, std::integral_constant<int, t + 1>{});
-			}
-		};
-		all_b(all_b, C0{});
-	}
-	issue_a(C0{}, 0, 0);
-	issue_a(C1{}, 0, 1);
-	issue_a(C2{}, 0, 2);
-	wide_wait<2 * A_PW, false>();	/* the patch and the first K-tile's weights */
-	__builtin_amdgcn_s_barrier();
-	read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
-	/* The pipeline of conv_f32_patch_kernel: K-tile (hb, tap) has its weights in stage tap % 3; a step issues
-	 * its patch loads first and its weights last, so at most the last step's loads may be outstanding when
-	 * the next K-tile's weights are waited for, and a block's last step waits for the next patch as well. */
-	auto step = [&](int hb, auto buf_, auto tap_) {
-		constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
-		typedef std::integral_constant<int, tap % 3> ST;
-		typedef std::integral_constant<int, (tap + 1) % 3> ST1;
-		typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
-		typedef std::integral_constant<int, buf ^ 1> OTHER;
-		typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
-		constexpr int prev = (tap + 8) % 9;
-		constexpr int last_loads = A_PW + CONV_PATCH_PB(prev + 1) - CONV_PATCH_PB(prev);
-		read_frags(ST{}, buf_, tap_, 1, af[1], bf[1]);
-		__builtin_amdgcn_sched_barrier(0);	/* (the fragments are asked for before the MFMAs that follow in the source) */
-		mma(0);
-		wide_wait<tap == 8 ? A_PW : last_loads, true>();
-		__builtin_amdgcn_s_barrier();
-		read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[0], bf[0]);
-		__builtin_amdgcn_sched_barrier(0);
-		if constexpr (CONV_PATCH_PB(tap + 1) - CONV_PATCH_PB(tap) >= 1)
-			issue_b(std::integral_constant<int, CONV_PATCH_PB(tap)>{}, hb + 1, OTHER{});
-		if constexpr (CONV_PATCH_PB(tap + 1) - CONV_PATCH_PB(tap) >= 2)
-			issue_b(std::integral_constant<int, CONV_PATCH_PB(tap) + 1>{}, hb + 1, OTHER{});
-		if constexpr (tap + 3 < 9)
-			issue_a(ST{}, hb, tap + 3);
-		else
-			issue_a(ST{}, hb + 1, tap + 3 - 9);
-		mma(1);
-	};
-#undef CONV_PATCH_PB
-	auto block = [&](int hb, auto buf_) {
-		step(hb, buf_, std::integral_constant<int, 0>{});
-		step(hb, buf_, std::integral_constant<int, 1>{});
-		step(hb, buf_, std::integral_constant<int, 2>{});
-		step(hb, buf_, std::integral_constant<int, 3>{});
-		step(hb, buf_, std::integral_constant<int, 4>{});
-		step(hb, buf_, std::integral_constant<int, 5>{});
-		step(hb, buf_, std::integral_constant<int, 6>{});
-		step(hb, buf_, std::integral_constant<int, 7>{});
-		step(hb, buf_, std::integral_constant<int, 8>{});
-	};
-	for (int hb = 0; hb < NB; hb += 2) {
-		block(hb, C0{});
-		block(hb + 1, C1{});
-	}
-	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the epilogue reuses it) */
-
-	/* ---- epilogue ---- */
-	elem *y = (elem *)p.y;
-	int *lrow = (int *)astage;
-	__syncthreads();
-	if (tid < BM) {
-		const int mc = min(tile_m * BM + tid, p.Co - 1);
-		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
-		if (p.scale)
-			lrow[BM + tid] = __float_as_int(p.scale[mc]);
-	}
-	__syncthreads();
-	const bool has_scale = p.scale != 0;
-	if constexpr (POOL) {
-		/* The 2x2 / stride 2 max pooling that follows, here: the two rows of a
-		 * window are this wave's two tile rows (the same accumulator index), its
-		 * two columns neighbouring lanes.  Threshold first, as the modules run. */
-		const int pH = p.oH / 2, pW = p.oW / 2;
-		const int py = ty * (TH / 2) + wave, px = tx * (TW / 2) + ((lane & 31) >> 1);
-		const bool store = !(lane & 1) && py < pH && px < pW;
-		const size_t n = ((size_t)img * pH + py) * pW + px;
-		const size_t ybase = (size_t)img * p.Co * pH * pW + (size_t)py * pW + px;
-#pragma unroll
-		for (int i = 0; i < TM; i++) {
-			const int m0 = tile_m * BM + i * 32 + 4 * (lane >> 5);
-#pragma unroll
-			for (int g = 0; g < 4; g++) {
-				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
-				const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
-				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
-				floatx4 rowscale = { 1, 1, 1, 1 };
-				if (has_scale)
-					rowscale = *(const floatx4 *)(lrow + BM + ml);
-#pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int r = 4 * g + e, m = m0 + 8 * g + e;
-					float v0 = has_scale ? acc[i][0][r] * rowscale[e] + rowbias[e] : acc[i][0][r] + rowbias[e];
-					float v1 = has_scale ? acc[i][1][r] * rowscale[e] + rowbias[e] : acc[i][1][r] + rowbias[e];
-					if (p.act) {
-						v0 = v0 > p.thr ? v0 : p.val;
-						v1 = v1 > p.thr ? v1 : p.val;
-					}
-					/* the pooling compares the stored (rounded) values */
-					float v = fmaxf((float)(elem)v0, (float)(elem)v1);
-					v = fmaxf(v, __shfl_xor(v, 1));
-					if constexpr (!CLO) {
-						if (store && m < p.Co)
-							y[ybase + (size_t)m * pH * pW] = (elem)v;
-					}
-					quad.v[e] = (elem)v;
-				}
-				if constexpr (CLO) {
-					if (store && m0 + 8 * g < p.Co)
-						*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
-				}
-			}
-		}
-		return;
-	}
-#pragma unroll
-	for (int j = 0; j < TN; j++) {
-		const int oy = ty * TH + 2 * wave + j, ox = tx * TW + (lane & 31);
-		if (oy >= p.oH || ox >= p.oW)
-			continue;
-		const int rem = oy * p.oW + ox;
-		const size_t n = (size_t)img * p.oHW + rem;
-		const size_t ybase = (size_t)img * p.Co * p.oHW + rem;
-#pragma unroll
-		for (int i = 0; i < TM; i++) {
-			const int m0 = tile_m * BM + i * 32 + 4 * (lane >> 5);
-#pragma unroll
-			for (int g = 0; g < 4; g++) {
-				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
-				const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
-				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
-				floatx4 rowscale = { 1, 1, 1, 1 };
-				if (has_scale)
-					rowscale = *(const floatx4 *)(lrow + BM + ml);
-#pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int r = 4 * g + e, m = m0 + 8 * g + e;
-					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
-					if (p.act)
-						v = v > p.thr ? v : p.val;
-					if constexpr (!CLO) {
-						if (m < p.Co)
-							y[ybase + (size_t)m * p.oHW] = (elem)v;
-					}
-					quad.v[e] = (elem)v;
-				}
-				if constexpr (CLO) {
-					if (m0 + 8 * g < p.Co)
-						*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
-				}
-			}
-		}
-	}
-#endif
-}
 
 /* ------------------------------------------------------------------ */
 /* fp32, plane-major: operands straight into LDS                       */
@@ -3592,53 +3076,18 @@ static void conv_launch_f32_patch(ConvParams &p)
 		conv_f32_patch_tail_finish_kernel<SW, SH><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
-/* Whether conv_patch_kernel can run this layer. */
+/* Whether conv_patch_kernel (conv_half_patch.hip) can run this layer. */
 template <int DT>
 static bool conv_patch_ok(const ConvParams &p)
 {
-	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16)
-		return p.x_cl == 1 && (p.Ci == 64 || p.Ci == 128 || p.Ci == 256 || p.Ci == 512) && p.kH == 3 && p.kW == 3 && p.dH == 1 && p.dW == 1 &&
-			p.x_bytes < 0x7fffffffu && !g_force_generic_cl && (!p.y_cl || p.Co % 4 == 0);
-	return false;
+	return thhip_conv_half_patch_ok(p, DT) && !g_force_generic_cl;
 }
 
-template <int DT, int BM>
-static void conv_launch_patch(ConvParams &p)
+/* ... and in its whole-image form (outputs of at most 14 x 14) */
+template <int DT>
+static bool conv_patch_flat(const ConvParams &p)
 {
-	if constexpr (DT == THHIP_F16 || DT == THHIP_BF16) {
-		p.tiles_m = (p.Co + BM - 1) / BM;
-		p.tiles_n = p.B * ((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH);
-		p.splitk = 1;
-		if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
-			THError("thhip_conv2d: packed weights shorter than the tile grid");
-		const long total = (long)p.tiles_m * p.tiles_n;
-		dim3 grid((unsigned)(8 * ((total + 7) / 8)));
-#define CONV_PATCH_GO(CLO, CI)                                                                               \
-	do {                                                                                                \
-		if (p.pool)                                                                                 \
-			conv_patch_kernel<DT, CLO, BM, CI, true><<<grid, dim3(256), 0, thhip_stream()>>>(p);  \
-		else                                                                                        \
-			conv_patch_kernel<DT, CLO, BM, CI, false><<<grid, dim3(256), 0, thhip_stream()>>>(p); \
-	} while (0)
-		if (p.Ci == 64 && p.y_cl)
-			CONV_PATCH_GO(true, 64);
-		else if (p.Ci == 64)
-			CONV_PATCH_GO(false, 64);
-		else if (p.Ci == 256 && p.y_cl)
-			CONV_PATCH_GO(true, 256);
-		else if (p.Ci == 256)
-			CONV_PATCH_GO(false, 256);
-		else if (p.Ci == 512 && p.y_cl)
-			CONV_PATCH_GO(true, 512);
-		else if (p.Ci == 512)
-			CONV_PATCH_GO(false, 512);
-		else if (p.y_cl)
-			CONV_PATCH_GO(true, 128);
-		else
-			CONV_PATCH_GO(false, 128);
-#undef CONV_PATCH_GO
-	} else
-		THError("thhip_conv2d: the patch kernel is for the half types");
+	return thhip_conv_half_patch_flat_ok(p, DT) && !g_force_generic_cl;
 }
 
 /* Half types, convolution followed by a 2x2 pooling: whether the kernel that keeps an input patch in LDS is
@@ -3652,7 +3101,7 @@ static bool conv_pool_uses_patch(const ConvParams &p)
 		 * 28^2: 31 %, and still faster than the tiles loaded straight into LDS: VGG-16 fp16 batch 16
 		 * 0.712 -> 0.693 ms, batch 64 2.26 -> 2.22 ms; 14^2 would waste three fifths) */
 		const bool fits = (long)((p.oW + PATCH_TW - 1) / PATCH_TW) * ((p.oH + PATCH_TH - 1) / PATCH_TH) * 256 * 100 <= (long)p.oH * p.oW * 132;
-		return conv_patch_ok<DT>(p) && tpatch >= 128 && (fits || p.Ci <= 128);
+		return conv_patch_flat<DT>(p) || (conv_patch_ok<DT>(p) && tpatch >= 128 && (fits || p.Ci <= 128));
 	}
 	return false;
 }
@@ -3860,10 +3309,14 @@ static void conv_dispatch(ConvParams &p)
 	if (bn == 1) {	/* (64, 1): the patch kernel */
 		if (!conv_patch_ok<DT>(p))
 			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64, 128, 256 or 512 planes, 3x3, stride 1");
+		/* a whole image of at most 14 x 14 per workgroup: 64 planes where that makes 256 workgroups, else 32
+		 * (the tuning hook's last argument: 3 forces 32, 4 forces 64, 5 the 32 x 8 tiles) */
+		if (conv_patch_flat<DT>(p) && g_force_wgs != 5 && g_force_wgs != 2) {
+			const bool small = g_force_wgs == 3 || (g_force_wgs != 4 && (long)p.B * (p.Co / 64) < 256);
+			return thhip_conv_half_patch_launch(p, DT, small ? 32 : 64, 1);
+		}
 		/* (the tuning hook's last argument 2: 128 planes per workgroup) */
-		if (g_force_wgs == 2 && p.Co % 128 == 0)
-			return conv_launch_patch<DT, 128>(p);
-		return conv_launch_patch<DT, 64>(p);
+		return thhip_conv_half_patch_launch(p, DT, g_force_wgs == 2 && p.Co % 128 == 0 ? 128 : 64, 0);
 	}
 	if constexpr (DT == THHIP_F32) {
 		if (direct && rows)
