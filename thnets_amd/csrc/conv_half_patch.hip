@@ -12,6 +12,10 @@
 #include <string.h>
 #include "conv_common.h"
 
+#ifndef PATCH_DEEP_TILES
+#define PATCH_DEEP_TILES 1
+#endif
+
 /* With 64 input planes a K-tile of the kernels above moves 64 bytes per
  * position from L2 for 32 multiply-adds per output plane, nine times per
  * pixel (once per tap), and the path from L2 to LDS, not the matrix core, sets
@@ -59,7 +63,8 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	constexpr int NPIX = PW * PH, WAVES = 4;
 	constexpr int BL = ((NPIX + 15) / 16 + WAVES - 1) / WAVES;	/* patch loads (sixteen pixels x four vectors) per wave and block */
 	constexpr int B_VECS = BL * WAVES * 64;				/* a buffer: every load's 1 KiB, the unused ones' too */
-	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = WHOLE ? 9 : 3;	/* NST: weight stages = K-tiles fetched ahead */
+	constexpr bool DEEP = WHOLE || (PATCH_DEEP_TILES && BM <= 64);	/* fragments fetched a whole K-tile ahead (below) */
+	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = WHOLE ? 9 : DEEP ? 6 : 3;	/* NST: weight stages = K-tiles fetched ahead */
 	constexpr int A_VECS = MB * KCH * 64, A_PW = (MB * KCH + WAVES - 1) / WAVES;
 	static_assert(CI % (2 * PCI) == 0 && (MB * KCH % WAVES == 0 || WAVES % (MB * KCH) == 0) && (WHOLE || TH == 2 * WAVES) && BL <= 8, "shape");
 	static_assert(!WHOLE || (NPIX == 256 && WAVES * TN * 32 == 256), "a whole image: 256 patch pixels, 256 position slots");
@@ -169,7 +174,6 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 			oy_[j] = ox_[j] = 0;
 		}
 	}
-	constexpr bool DEEP = WHOLE;	/* fragments fetched a whole K-tile ahead (below) */
 	floatx4 af[DEEP ? 4 : 2][TM], bf[DEEP ? 4 : 2][TN];
 	auto read_frags = [&](auto st_, auto buf_, auto tap_, int c, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
 		constexpr int st = decltype(st_)::value, buf = decltype(buf_)::value, tap = decltype(tap_)::value;
@@ -207,7 +211,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	/* patch loads of the next block: BL of them over the nine steps of this one, step `tap` issues
 	 * numbers [PB(tap), PB(tap + 1)), none in the last (WHOLE, where a workgroup may be alone on its CU
 	 * with nothing to hide a late patch behind: one in each of the first BL steps) */
-#define CONV_PATCH_PB(tap) (WHOLE ? ((tap) < BL ? (tap) : BL) : (BL * ((tap) < 8 ? (tap) : 8) + 7) / 8)
+#define CONV_PATCH_PB(tap) (DEEP ? ((tap) < BL ? (tap) : BL) : (BL * ((tap) < 8 ? (tap) : 8) + 7) / 8)
 #define CONV_PATCH_NB(tap) (CONV_PATCH_PB(((tap) + 9) % 9 + 1) - CONV_PATCH_PB(((tap) + 9) % 9))
 	/* The loads of a wave complete in the order of their issue, and a wait names how many of the latest may
 	 * still be outstanding.  Step t (K-tile t of the layer, tap t % 9) issues its patch loads, then the
@@ -252,7 +256,7 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 		return n;
 	};
 	if constexpr (DEEP) {
-		static_assert(NST == 9, "a stage per tap");
+		static_assert(18 % NST == 0 && NST >= 3, "K-tile k of a pair of blocks in stage k % NST");
 		/* what steps -9 .. -1 would have issued: the first patch, the weights of K-tiles 0 .. NST - 2 */
 		auto virt = [&](auto self, auto v_) {
 			constexpr int v = decltype(v_)::value;	/* step v - 9, tap v */
@@ -261,22 +265,22 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 					issue_b(std::integral_constant<int, CONV_PATCH_PB(v)>{}, 0, C0{});
 				if constexpr (CONV_PATCH_NB(v) >= 2)
 					issue_b(std::integral_constant<int, CONV_PATCH_PB(v) + 1>{}, 0, C0{});
-				if constexpr (v >= 1)
-					issue_a(std::integral_constant<int, v - 1>{}, 0, v - 1);
+				if constexpr (v - 10 + NST >= 0)
+					issue_a(std::integral_constant<int, v - 10 + NST>{}, 0, v - 10 + NST);
 				self(self, std::integral_constant<int, v + 1>{});
 			}
 		};
 		virt(virt, C0{});
-		/* the patch and K-tile 0: what followed the last patch load (the weights of K-tiles BL - 2 .. 7) may be outstanding */
-		wide_wait<(10 - BL) * A_PW, false>();
+		/* the patch (its last load: step BL - 10) and K-tile 0 (step 1 - NST): what the steps after both issued may be outstanding */
+		wide_wait<(BL - 10 > 1 - NST ? 10 - BL : NST - 2) * A_PW, false>();
 		__builtin_amdgcn_s_barrier();
 		read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
 		read_frags(C0{}, C0{}, C0{}, 1, af[1], bf[1]);
 		auto step = [&](int hb, auto buf_, auto tap_) {
 			constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
 			constexpr int par = (tap + buf) & 1;
-			typedef std::integral_constant<int, (tap + 1) % NST> ST1;
-			typedef std::integral_constant<int, (tap + NST - 1) % NST> STP;
+			typedef std::integral_constant<int, (9 * buf + tap + 1) % NST> ST1;
+			typedef std::integral_constant<int, (9 * buf + tap + NST - 1) % NST> STP;
 			typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
 			typedef std::integral_constant<int, buf ^ 1> OTHER;
 			typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;

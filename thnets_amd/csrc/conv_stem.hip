@@ -56,10 +56,11 @@ __global__ __launch_bounds__(STEM_THREADS) __attribute__((amdgpu_waves_per_eu(4,
 	constexpr int NS = F32 ? 14 : 2;	/* MFMAs along K (K padded to 28 / 32) */
 	extern __shared__ __align__(16) unsigned char stem_lds[];
 	float *const rowc = (float *)stem_lds;	/* bias[64], factor[64] */
-	elem *const patch = (elem *)(stem_lds + 512);
+	elem *const patch = (elem *)(stem_lds + 512 + (CLO ? 4 * 4096 : 0));
 
 	const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 	const int n = lane & 31, h = lane >> 5;
+	unsigned char *const stage = stem_lds + 512 + wave * 4096;	/* (channels-last output) */
 	const int b = blockIdx.z, mz = blockIdx.y;
 	const int row0 = blockIdx.x * p.rows;
 	const int rows = min(p.rows, p.H - row0);
@@ -221,14 +222,25 @@ __global__ __launch_bounds__(STEM_THREADS) __attribute__((amdgpu_waves_per_eu(4,
 				}
 			}
 			if constexpr (CLO) {
-				/* the two lanes of a position exchange groups so that each writes 16 bytes */
+				/* into this wave's 4 KiB of LDS, [position][64 planes] with the 16-byte pieces of a
+				 * position exchanged by its number (the 32 positions would otherwise share banks) */
 #pragma unroll
-				for (int hh = 0; hh < 2; hh++) {
-					stem_swap32(lo[2 * hh], lo[2 * hh + 1]);
-					stem_swap32(hi[2 * hh], hi[2 * hh + 1]);
-					const uintx4 v = { lo[2 * hh], hi[2 * hh], lo[2 * hh + 1], hi[2 * hh + 1] };
-					__builtin_amdgcn_raw_buffer_store_b128(v, yrsrc, laneoff, (mb * 32 + 16 * hh) * (int)sizeof(elem), 0);
+				for (int g = 0; g < 4; g++) {
+					const uintx2 v = { lo[g], hi[g] };
+					*(uintx2 *)(stage + n * 128 + (((mb * 4 + g) ^ (n & 7)) * 16) + 8 * h) = v;
 				}
+			}
+		}
+		if constexpr (CLO) {
+			/* ... and out again in memory order: an instruction stores eight positions' 128 bytes each
+			 * (1 KiB in one piece when the layer has 64 planes) */
+			const int obase = ((oy * p.W + tx * 32) * p.Co + mz * 64) * (int)sizeof(elem);
+#pragma unroll
+			for (int i = 0; i < 4; i++) {
+				const int u = i * 64 + lane, px = u >> 3, slot = u & 7;
+				const uintx4 v = *(const uintx4 *)(stage + px * 128 + ((slot ^ (px & 7)) * 16));
+				const int goff = tx * 32 + px < p.W ? obase + px * p.Co * (int)sizeof(elem) + slot * 16 : (int)0x80000000;
+				__builtin_amdgcn_raw_buffer_store_b128(v, yrsrc, goff, 0, 0);
 			}
 		}
 	}
@@ -242,10 +254,10 @@ static int stem_rows(int B, int H)
 	return rows;
 }
 
-static size_t stem_lds_bytes(int rows, int W, int esize)
+static size_t stem_lds_bytes(int rows, int W, int esize, int y_cl)
 {
 	const int tpr = (W + 31) / 32;
-	return 512 + (size_t)3 * (rows + 2) * (32 * tpr + 2) * esize;
+	return 512 + (y_cl ? 4 * 4096 : 0) + (size_t)3 * (rows + 2) * (32 * tpr + 2) * esize;
 }
 
 /* The layers this kernel takes: 3 planes in, whole blocks of 64 planes out, 3x3, stride 1,
@@ -262,7 +274,7 @@ bool thhip_conv_stem_ok(int B, int Ci, int H, int W, int Co, int kH, int kW, int
 		return false;
 	if (B > 65535 || Co / 64 > 65535)
 		return false;
-	return stem_lds_bytes(stem_rows(B, H), W, thhip_esize(dtype)) <= 65536;
+	return stem_lds_bytes(stem_rows(B, H), W, thhip_esize(dtype), y_cl) <= 65536;
 }
 
 template <int DT, bool CLO>
@@ -287,7 +299,7 @@ void thhip_conv_stem(const void *x, const void *wpacked, int KC, const float *sc
 	p.pw = 32 * p.tpr + 2;
 	p.magic_pw = (unsigned)((1ull << 32) / p.pw + 1);
 	p.act = act; p.thr = thr; p.val = val;
-	const size_t lds = stem_lds_bytes(p.rows, W, thhip_esize(dtype));
+	const size_t lds = stem_lds_bytes(p.rows, W, thhip_esize(dtype), y_cl);
 	if (dtype == THHIP_F32)
 		stem_launch<THHIP_F32, false>(p, lds);
 	else if (dtype == THHIP_F16)
