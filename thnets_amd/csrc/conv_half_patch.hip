@@ -12,35 +12,35 @@
 #include <string.h>
 #include "conv_common.h"
 
-#ifndef PATCH_DEEP_TILES
-#define PATCH_DEEP_TILES 1
-#endif
-
-/* With 64 input planes a K-tile of the kernels above moves 64 bytes per
+/* With 64 input planes a K-tile of the generic kernels moves 64 bytes per
  * position from L2 for 32 multiply-adds per output plane, nine times per
  * pixel (once per tap), and the path from L2 to LDS, not the matrix core, sets
  * their time.  Here a workgroup owns 8 rows x 32 columns of one image's output,
  * copies the 10 x 34 pixel patch those positions read once per block of 32
  * planes (21 KiB, straight to LDS), and takes the B fragments of all nine taps
- * from it: a fragment of tap (kh, kw) is the patch shifted by (kh, kw).  The
- * pipeline is conv_f32_patch_kernel's: two patch buffers, the next block's six
- * loads per wavefront spread over the nine taps of this one, the weights
- * (K-tiles of one tap x 32 planes) through a ring of three stages, the nine
- * steps of a block straight-line code with constant wait counts.  (An earlier
- * form held one patch of 64 planes, 43.5 KiB, and drained the pipeline between
- * blocks: VGG-16 fp16 batch 16 0.735 -> 0.713 ms, batch 64 2.33 -> 2.26 ms.)
+ * from it: a fragment of tap (kh, kw) is the patch shifted by (kh, kw).  Two
+ * patch buffers, the next block's loads spread over the first steps of this one,
+ * the weights (K-tiles of one tap x 32 planes) through a ring of NST stages, the
+ * nine steps of a block straight-line code with constant wait counts.
  *
  * Patch layout: 1 KiB blocks of sixteen pixels x four 16-byte vectors, pixel pp
  * of the patch (row-major, 34 wide) in block pp / 16; vector v of pixel pp sits
  * in slot 4 pp + (v ^ ((pp / 4) % 4)).  A fragment read takes one vector index
  * from 32 consecutive pixels, sixteen lanes (256 bytes, every bank once) a cycle;
  * pixels four apart share their banks, and the swizzle gives any four such in a
- * run of sixteen four different slots, wherever the run starts.  (With the key
- * (pp / 2) % 4, which serves runs of eight, the counters showed conflicts in a
- * tenth of the cycles.)  Pixels outside the image are fetched out of the
- * buffer's range and arrive as zeros.
+ * run of sixteen four different slots, wherever the run starts.  Pixels outside
+ * the image are fetched out of the buffer's range and arrive as zeros.
  *
  * Four waves; wave w computes all BM planes of tile rows 2w and 2w+1.
+ *
+ * A workgroup walks several tiles (tile l, l + n, l + 2n, ... of its XCD's run, n
+ * workgroups per XCD) without draining the pipeline: the blocks of its tiles are
+ * one sequence, so the first patch and weights of the next tile are fetched under
+ * the last steps of this one and land while the results are stored.  (One tile per
+ * workgroup and two workgroups per CU, started together, spent as long waiting for
+ * their first patch and storing as multiplying: 64 -> 64 @224^2 kept the matrix
+ * cores 44 % busy.)  The per-plane constants of every plane block sit in LDS from
+ * the start, so that nothing the epilogue needs queues behind those loads.
  *
  * WHOLE: outputs of at most 14 x 14 (VGG-16's last three layers, ResNet's 14 x 14
  * ones), where 32 x 8 tiles would be three fifths empty: a workgroup takes a whole
@@ -52,8 +52,10 @@
  * 16, 512 planes: 128 of 64 planes), so BM may be 32 here: then two of the four
  * waves' weight loads repeat the other two's (same bytes to the same place), which
  * keeps every wave's count of outstanding loads the same. */
+#define PATCH_ROWC 1024	/* output planes (in whole blocks) whose constants the kernel keeps in LDS */
+
 template <int DT, bool CLO, int BM, int CI, bool POOL, bool WHOLE>
-__global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_patch_kernel(ConvParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
 	typedef ConvTraits<DT> TR;
@@ -63,88 +65,126 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	constexpr int NPIX = PW * PH, WAVES = 4;
 	constexpr int BL = ((NPIX + 15) / 16 + WAVES - 1) / WAVES;	/* patch loads (sixteen pixels x four vectors) per wave and block */
 	constexpr int B_VECS = BL * WAVES * 64;				/* a buffer: every load's 1 KiB, the unused ones' too */
-	constexpr bool DEEP = WHOLE || (PATCH_DEEP_TILES && BM <= 64);	/* fragments fetched a whole K-tile ahead (below) */
-	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = WHOLE ? 9 : DEEP ? 6 : 3;	/* NST: weight stages = K-tiles fetched ahead */
+	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = WHOLE ? 9 : 6;	/* NST: weight stages */
 	constexpr int A_VECS = MB * KCH * 64, A_PW = (MB * KCH + WAVES - 1) / WAVES;
 	static_assert(CI % (2 * PCI) == 0 && (MB * KCH % WAVES == 0 || WAVES % (MB * KCH) == 0) && (WHOLE || TH == 2 * WAVES) && BL <= 8, "shape");
 	static_assert(!WHOLE || (NPIX == 256 && WAVES * TN * 32 == 256), "a whole image: 256 patch pixels, 256 position slots");
+	static_assert(18 % NST == 0 && NST >= 3, "K-tile k of a pair of blocks in stage k % NST");
+	/* Walking several tiles pays with 64 input planes, where a tile's eighteen steps are as long as its first
+	 * loads and its stores (64 -> 64 @224^2 with the pooling, batch 64: 264 -> 241 us; 64 -> 128 @112^2:
+	 * 167 -> 156 us); longer K loops lose more to the fixed tile order than they gain (3-7 %) and take one
+	 * tile per workgroup, which the dispatcher hands to the CUs as they come free. */
+	constexpr bool WALK = CI == 64;
+	constexpr int ROWC = WALK ? PATCH_ROWC : BM;	/* planes whose constants sit in LDS */
 	/* (one array, every stage and buffer at a constant offset: conv_f32_patch_kernel says why) */
-	__shared__ floatx4 lds[NST * A_VECS + 2 * B_VECS];
+	__shared__ floatx4 lds[NST * A_VECS + 2 * B_VECS + 2 * ROWC / 4];
 	floatx4 *const astage = lds;
 	floatx4 *const patch0 = lds + NST * A_VECS, *const patch1 = patch0 + B_VECS;
+	float *const rowc = (float *)(patch1 + B_VECS);	/* bias[ROWC], factor[ROWC] */
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
 	const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-	/* consecutive tiles (plane block fastest, then along the row) share halo
-	 * pixels: each XCD takes one run of them */
+	/* ---- this workgroup's tiles: number local0, local0 + nloc, ... of its XCD's.  32 x 8 tiles: consecutive
+	 * tiles (plane block fastest, then along the row) share halo pixels, each XCD takes one run of them.
+	 * WHOLE: every XCD a rectangle of the (plane block, image) grid, mparts x 8 / mparts of them; its
+	 * workgroups run side by side and share the rectangle's weights and images through its L2. ---- */
 	const int tx_n = (p.oW + TW - 1) / TW, ty_n = (p.oH + TH - 1) / TH;
-	int tile_m, tx, ty, img;
-	{
+	const int xcd = blockIdx.x & 7, nloc = gridDim.x >> 3;
+	int first, cnt, mw = 1, m0 = 0, n0 = 0;
+	if constexpr (WHOLE) {
+		const int mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
+		m0 = p.tiles_m * mp / p.mparts;
+		mw = p.tiles_m * (mp + 1) / p.mparts - m0;
+		n0 = p.tiles_n * np / nparts;
+		cnt = mw * (p.tiles_n * (np + 1) / nparts - n0);
+		first = 0;
+	} else {
 		const int total = p.tiles_m * p.tiles_n, per_xcd = (total + 7) / 8;
-		const int local = blockIdx.x >> 3;
-		if constexpr (WHOLE) {
-			/* every XCD a rectangle of the (plane block, image) grid, mparts x 8 / mparts of them: its
-			 * workgroups run side by side and share the rectangle's weights and images through its L2 */
-			const int xcd = blockIdx.x & 7, mp = xcd % p.mparts, np = xcd / p.mparts, nparts = 8 / p.mparts;
-			const int m0 = p.tiles_m * mp / p.mparts, m1 = p.tiles_m * (mp + 1) / p.mparts;
-			const int n0 = p.tiles_n * np / nparts, n1 = p.tiles_n * (np + 1) / nparts;
-			if (local >= (m1 - m0) * (n1 - n0))
-				return;
-			tile_m = m0 + local % (m1 - m0);
-			img = n0 + local / (m1 - m0);
-			tx = ty = 0;
-		} else {
-			const int t = (blockIdx.x & 7) * per_xcd + local;
-			if (local >= per_xcd || t >= total)
-				return;
-			tile_m = t % p.tiles_m;
-			const int sp = t / p.tiles_m;
-			tx = sp % tx_n;
-			ty = (sp / tx_n) % ty_n;
-			img = sp / (tx_n * ty_n);
-		}
+		first = xcd * per_xcd;
+		cnt = min(per_xcd, total - first);
 	}
+	struct Tile { int tile_m, tx, ty, img; bool ok; };
+	auto decode = [&](int local) {
+		Tile T;
+		T.ok = local < cnt;
+		const int l = T.ok ? local : 0;
+		if constexpr (WHOLE) {
+			T.tile_m = m0 + l % mw;
+			T.img = n0 + l / mw;
+			T.tx = T.ty = 0;
+		} else {
+			const int t = first + l;
+			T.tile_m = t % p.tiles_m;
+			const int sp = t / p.tiles_m;
+			T.tx = sp % tx_n;
+			T.ty = (sp / tx_n) % ty_n;
+			T.img = sp / (tx_n * ty_n);
+		}
+		return T;
+	};
+	int nlocal = blockIdx.x >> 3;
+	Tile cur = decode(nlocal);
+	if (!cur.ok)
+		return;
+	nlocal += nloc;
+	Tile nxt = decode(nlocal);
+	if constexpr (!WALK)
+		nxt.ok = false;
 
 	const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.x, 0, p.x_bytes, 0x00020000);
 	const __amdgpu_buffer_rsrc_t wrsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.wp, 0, p.w_bytes, 0x00020000);
-	/* ---- what this lane fetches of every block of 32 planes: load t of the wave covers pixels
-	 * 16 (wave + 4 t) .. + 15 of the patch, this lane pixel lane / 4 of them, vector lane % 4
-	 * through the swizzle ---- */
-	unsigned voff_[BL];
-#pragma unroll
-	for (int t = 0; t < BL; t++) {
-		const int pp = (wave + WAVES * t) * 16 + (lane >> 2);
-		const int v = (lane & 3) ^ ((pp >> 2) & 3);
-		const int pr = pp / PW, pc = pp - pr * PW;
-		const int iy = ty * TH - p.padH + pr, ix = tx * TW - p.padW + pc;
-		const bool ok = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-		voff_[t] = ok ? (unsigned)((((img * p.H + iy) * p.W + ix) * CI + v * 8) * (int)sizeof(elem)) : 0x80000000u;
-	}
-	/* this wave's weight blocks of a K-tile: wave + 4 i counts (chunk, 32-row block) */
-	unsigned a_off_[A_PW];
+	/* ---- what this lane fetches of every block of 32 planes of a tile: load t of the wave covers pixels
+	 * 16 (wave + 4 t) .. + 15 of the patch, this lane pixel lane / 4 of them, vector lane % 4 through the
+	 * swizzle; and the wave's weight blocks of a K-tile: wave + 4 i counts (chunk, 32-row block).  Of a
+	 * tile that does not exist everything is out of range (and arrives as zeros). ---- */
 	int a_lds_[A_PW];
 #pragma unroll
 	for (int i = 0; i < A_PW; i++) {
-		const int idx = (wave + WAVES * i) % (MB * KCH), mbi = idx % MB, kci = idx / MB;
-		a_off_[i] = ((unsigned)(tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
-		a_lds_[i] = (kci * MB + mbi) * 64;
+		const int idx = (wave + WAVES * i) % (MB * KCH);
+		a_lds_[i] = ((idx / MB) * MB + idx % MB) * 64;
 	}
+	auto offsets = [&](const Tile &T, unsigned (&voff)[BL], unsigned (&aoff)[A_PW]) {
+#pragma unroll
+		for (int t = 0; t < BL; t++) {
+			const int pp = (wave + WAVES * t) * 16 + (lane >> 2);
+			const int v = (lane & 3) ^ ((pp >> 2) & 3);
+			const int pr = pp / PW, pc = pp - pr * PW;
+			const int iy = T.ty * TH - p.padH + pr, ix = T.tx * TW - p.padW + pc;
+			const bool ok = T.ok && pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			voff[t] = ok ? (unsigned)((((T.img * p.H + iy) * p.W + ix) * CI + v * 8) * (int)sizeof(elem)) : 0x80000000u;
+		}
+#pragma unroll
+		for (int i = 0; i < A_PW; i++) {
+			const int idx = (wave + WAVES * i) % (MB * KCH), mbi = idx % MB, kci = idx / MB;
+			aoff[i] = ((unsigned)(T.tile_m * MB + mbi) * (unsigned)p.KC + kci) * 1024u;
+		}
+	};
+	unsigned voff_[BL], voffn_[BL], a_off_[A_PW], a_offn_[A_PW];
+	offsets(cur, voff_, a_off_);
+	offsets(nxt, voffn_, a_offn_);
 
-	/* the weights of K-tile (block hb of 32 planes, tap): K runs (block, tap, plane) in chunks of 16 */
+	/* the weights of K-tile (block hb of 32 planes, tap): K runs (block, tap, plane) in chunks of 16.
+	 * Block NB is block 0 of the next tile. */
 	auto issue_a = [&](auto st_, int hb, int tap) {
 		constexpr int st = decltype(st_)::value;
-		const unsigned kc = (unsigned)((hb * 9 + tap) * KCH);
+		const bool here = hb < NB;
+		const unsigned kc = (unsigned)(((here || !WALK ? hb : 0) * 9 + tap) * KCH);
 #pragma unroll
 		for (int i = 0; i < A_PW; i++)
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16,
-				hb < NB ? lane * 16 : 0x80000000u, a_off_[i] + kc * 1024u, 0, 0);
+				here || (WALK && nxt.ok) ? lane * 16 : 0x80000000u, (here || !WALK ? a_off_[i] : a_offn_[i]) + kc * 1024u, 0, 0);
 	};
 	auto issue_b = [&](auto t_, int hb, auto buf_) {
 		constexpr int buf = decltype(buf_)::value, t = decltype(t_)::value;
-		__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS((buf ? patch1 : patch0) + (wave + WAVES * t) * 64), 16,
-			hb < NB ? voff_[t] : 0x80000000u, hb < NB ? hb * PCI * (int)sizeof(elem) : 0, 0, 0);
+		const bool here = hb < NB;
+		if constexpr (WALK)
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS((buf ? patch1 : patch0) + (wave + WAVES * t) * 64), 16,
+				here ? voff_[t] : voffn_[t], here ? hb * PCI * (int)sizeof(elem) : 0, 0, 0);
+		else
+			__builtin_amdgcn_raw_ptr_buffer_load_lds(xrsrc, WIDE_LDS((buf ? patch1 : patch0) + (wave + WAVES * t) * 64), 16,
+				here ? voff_[t] : 0x80000000u, here ? hb * PCI * (int)sizeof(elem) : 0, 0, 0);
 	};
 
 	/* patch pixel of this lane's position at tap (0, 0), for its two tile rows */
@@ -174,7 +214,8 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 			oy_[j] = ox_[j] = 0;
 		}
 	}
-	floatx4 af[DEEP ? 4 : 2][TM], bf[DEEP ? 4 : 2][TN];
+	/* four fragment sets: two chunks each of this K-tile and the next (below) */
+	floatx4 af[4][TM], bf[4][TN];
 	auto read_frags = [&](auto st_, auto buf_, auto tap_, int c, floatx4 (&a)[TM], floatx4 (&b)[TN]) {
 		constexpr int st = decltype(st_)::value, buf = decltype(buf_)::value, tap = decltype(tap_)::value;
 		const floatx4 *la = astage + st * A_VECS;
@@ -190,13 +231,16 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 	};
 
 	typename ConvAcc<DT>::T acc[TM][TN];
+	auto clear = [&]() {
 #pragma unroll
-	for (int i = 0; i < TM; i++)
+		for (int i = 0; i < TM; i++)
 #pragma unroll
-		for (int j = 0; j < TN; j++)
+			for (int j = 0; j < TN; j++)
 #pragma unroll
-			for (int r = 0; r < 16; r++)
-				acc[i][j][r] = 0;
+				for (int r = 0; r < 16; r++)
+					acc[i][j][r] = 0;
+	};
+	clear();
 	auto mma = [&](int set) {
 #pragma unroll
 		for (int i = 0; i < TM; i++)
@@ -207,222 +251,166 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 
 	typedef std::integral_constant<int, 0> C0;
 	typedef std::integral_constant<int, 1> C1;
-	typedef std::integral_constant<int, 2> C2;
-	/* patch loads of the next block: BL of them over the nine steps of this one, step `tap` issues
-	 * numbers [PB(tap), PB(tap + 1)), none in the last (WHOLE, where a workgroup may be alone on its CU
-	 * with nothing to hide a late patch behind: one in each of the first BL steps) */
-#define CONV_PATCH_PB(tap) (DEEP ? ((tap) < BL ? (tap) : BL) : (BL * ((tap) < 8 ? (tap) : 8) + 7) / 8)
+	/* patch loads of the next block: one in each of the first BL steps of this one (step `tap` issues
+	 * numbers [PB(tap), PB(tap + 1))) */
+#define CONV_PATCH_PB(tap) ((tap) < BL ? (tap) : BL)
 #define CONV_PATCH_NB(tap) (CONV_PATCH_PB(((tap) + 9) % 9 + 1) - CONV_PATCH_PB(((tap) + 9) % 9))
-	/* The loads of a wave complete in the order of their issue, and a wait names how many of the latest may
-	 * still be outstanding.  Step t (K-tile t of the layer, tap t % 9) issues its patch loads, then the
-	 * weights of K-tile t + NST.  So when step t waits for the weights of K-tile t + 1, issued in step
-	 * t + 1 - NST, everything steps t + 2 - NST .. t - 1 issued may be outstanding; a block's last step also
-	 * waits for the next patch, whose last load step `lastp` issued before its weights.  The prologue
-	 * issues what steps -NST .. -1 would have, in their order, so the counts hold from the first step. */
+	/* The pipeline.  A wave with the SIMD to itself gets what it asks of LDS before a group of MFMAs only
+	 * after them, so the fragments of a K-tile are fetched a whole step ahead, into four register sets.
+	 * Step t (K-tile t of the workgroup's sequence, tap t % 9) starts with the wait and the barrier: K-tile
+	 * t + 1 is in LDS, and every wave has issued the MFMAs of K-tile t - 1, whose stage the weights of K-tile
+	 * t - 1 + NST now overwrite; then it alternates the reads of K-tile t + 1 with the MFMAs of K-tile t.
+	 * The loads of a wave complete in the order of their issue, and a wait names how many of the latest may
+	 * still be outstanding: the weights of K-tile t + 1 were issued in step t + 2 - NST, what steps
+	 * t + 3 - NST .. t - 1 issued may be; the step that reads the next patch's first fragments (tap 8) needs
+	 * that patch too, whose last load step BL - 1 issued before its weights.  The prologue issues what
+	 * steps -9 .. -1 would have, in their order, so the counts hold from the first step.  (Stores count as
+	 * loads do: after an epilogue the first steps of the next tile wait for most of its stores as well.) */
 	constexpr auto allowed = [](int tap) {
-		int n = 0;
-		for (int t = tap + 2 - NST; t <= tap - 1; t++)
-			n += A_PW + CONV_PATCH_NB(t + 18);
-		if (tap == 8) {
-			int lastp = 0;
-			for (int t = 0; t < 9; t++)
-				if (CONV_PATCH_NB(t) > 0)
-					lastp = t;
-			const int np = (8 - lastp) * A_PW;
-			n = n < np ? n : np;
-		}
-		return n;
-	};
-	/* DEEP.  A workgroup alone on its CU has one wave per SIMD, and what that wave asks of LDS before a group
-	 * of MFMAs it gets only after them: the fragments of a K-tile are then fetched a whole step ahead, into
-	 * four register sets (two chunks each of this K-tile and the next).  A step starts with the wait and the
-	 * barrier (K-tile t + 1 is in LDS, every wave has issued the MFMAs of K-tile t - 1, whose stage the
-	 * weights of K-tile t - 1 + NST now overwrite), then alternates the reads of K-tile t + 1 with the
-	 * MFMAs of K-tile t.  The counts: the weights of K-tile t + 1 were issued in step t + 2 - NST, what
-	 * steps t + 3 - NST .. t - 1 issued may be outstanding; the step that reads the next patch's first
-	 * fragments (tap 8) needs that patch too. */
-	constexpr auto allowed_deep = [](int tap) {
 		int n = 0;
 		for (int t = tap + 3 - NST; t <= tap - 1; t++)
 			n += A_PW + CONV_PATCH_NB(t + 18);
 		if (tap == 8) {
-			int lastp = 0;
-			for (int t = 0; t < 9; t++)
-				if (CONV_PATCH_NB(t) > 0)
-					lastp = t;
-			const int np = (8 - lastp) * A_PW;
+			const int np = (8 - (BL - 1)) * A_PW;
 			n = n < np ? n : np;
 		}
 		return n;
 	};
-	if constexpr (DEEP) {
-		static_assert(18 % NST == 0 && NST >= 3, "K-tile k of a pair of blocks in stage k % NST");
-		/* what steps -9 .. -1 would have issued: the first patch, the weights of K-tiles 0 .. NST - 2 */
+	{
 		auto virt = [&](auto self, auto v_) {
 			constexpr int v = decltype(v_)::value;	/* step v - 9, tap v */
 			if constexpr (v < 9) {
 				if constexpr (CONV_PATCH_NB(v) >= 1)
 					issue_b(std::integral_constant<int, CONV_PATCH_PB(v)>{}, 0, C0{});
-				if constexpr (CONV_PATCH_NB(v) >= 2)
-					issue_b(std::integral_constant<int, CONV_PATCH_PB(v) + 1>{}, 0, C0{});
 				if constexpr (v - 10 + NST >= 0)
 					issue_a(std::integral_constant<int, v - 10 + NST>{}, 0, v - 10 + NST);
 				self(self, std::integral_constant<int, v + 1>{});
 			}
 		};
 		virt(virt, C0{});
-		/* the patch (its last load: step BL - 10) and K-tile 0 (step 1 - NST): what the steps after both issued may be outstanding */
-		wide_wait<(BL - 10 > 1 - NST ? 10 - BL : NST - 2) * A_PW, false>();
-		__builtin_amdgcn_s_barrier();
-		read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
-		read_frags(C0{}, C0{}, C0{}, 1, af[1], bf[1]);
-		auto step = [&](int hb, auto buf_, auto tap_) {
-			constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
-			constexpr int par = (tap + buf) & 1;
-			typedef std::integral_constant<int, (9 * buf + tap + 1) % NST> ST1;
-			typedef std::integral_constant<int, (9 * buf + tap + NST - 1) % NST> STP;
-			typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
-			typedef std::integral_constant<int, buf ^ 1> OTHER;
-			typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
-			wide_wait<allowed_deep(tap), false>();
-			__builtin_amdgcn_s_barrier();
-			if constexpr (CONV_PATCH_NB(tap) >= 1)
-				issue_b(std::integral_constant<int, CONV_PATCH_PB(tap)>{}, hb + 1, OTHER{});
-			if constexpr (CONV_PATCH_NB(tap) >= 2)
-				issue_b(std::integral_constant<int, CONV_PATCH_PB(tap) + 1>{}, hb + 1, OTHER{});
-			issue_a(STP{}, hb + (tap + NST - 1) / 9, (tap + NST - 1) % 9);
-			read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[2 * (par ^ 1)], bf[2 * (par ^ 1)]);
-			__builtin_amdgcn_sched_barrier(0);
-			mma(2 * par);
-			read_frags(ST1{}, BUF1{}, TAP1{}, 1, af[2 * (par ^ 1) + 1], bf[2 * (par ^ 1) + 1]);
-			__builtin_amdgcn_sched_barrier(0);
-			mma(2 * par + 1);
-		};
-		auto block = [&](int hb, auto buf_) {
-			step(hb, buf_, std::integral_constant<int, 0>{});
-			step(hb, buf_, std::integral_constant<int, 1>{});
-			step(hb, buf_, std::integral_constant<int, 2>{});
-			step(hb, buf_, std::integral_constant<int, 3>{});
-			step(hb, buf_, std::integral_constant<int, 4>{});
-			step(hb, buf_, std::integral_constant<int, 5>{});
-			step(hb, buf_, std::integral_constant<int, 6>{});
-			step(hb, buf_, std::integral_constant<int, 7>{});
-			step(hb, buf_, std::integral_constant<int, 8>{});
-		};
-		for (int hb = 0; hb < NB; hb += 2) {
-			block(hb, C0{});
-			block(hb + 1, C1{});
-		}
-	} else {
-		{
-			/* the patch loads steps before -NST would have issued, then steps -NST .. -1 */
-			auto early_b = [&](auto self, auto t_) {
-				constexpr int t = decltype(t_)::value;
-				if constexpr (t < CONV_PATCH_PB(9 - NST)) {
-					issue_b(t_, 0, C0{});
-					self(self, std::integral_constant<int, t + 1>{});
-				}
-			};
-			early_b(early_b, C0{});
-			auto virt = [&](auto self, auto v_) {
-				constexpr int v = decltype(v_)::value, tap = 9 - NST + v;	/* step v - NST */
-				if constexpr (v < NST) {
-					if constexpr (CONV_PATCH_NB(tap) >= 1)
-						issue_b(std::integral_constant<int, CONV_PATCH_PB(tap)>{}, 0, C0{});
-					if constexpr (CONV_PATCH_NB(tap) >= 2)
-						issue_b(std::integral_constant<int, CONV_PATCH_PB(tap) + 1>{}, 0, C0{});
-					issue_a(std::integral_constant<int, v % NST>{}, 0, v);
-					self(self, std::integral_constant<int, v + 1>{});
-				}
-			};
-			virt(virt, C0{});
-		}
-		wide_wait<allowed(8), false>();	/* the patch and the first K-tile's weights */
-		__builtin_amdgcn_s_barrier();
-		read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
-		/* The pipeline of conv_f32_patch_kernel: K-tile (hb, tap) has its weights in stage tap % NST. */
-		auto step = [&](int hb, auto buf_, auto tap_) {
-			constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
-			typedef std::integral_constant<int, tap % NST> ST;
-			typedef std::integral_constant<int, (tap + 1) % NST> ST1;
-			typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
-			typedef std::integral_constant<int, buf ^ 1> OTHER;
-			typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
-			read_frags(ST{}, buf_, tap_, 1, af[1], bf[1]);
-			__builtin_amdgcn_sched_barrier(0);	/* (the fragments are asked for before the MFMAs that follow in the source) */
-			mma(0);
-			wide_wait<allowed(tap), true>();
-			__builtin_amdgcn_s_barrier();
-			read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[0], bf[0]);
-			__builtin_amdgcn_sched_barrier(0);
-			if constexpr (CONV_PATCH_NB(tap) >= 1)
-				issue_b(std::integral_constant<int, CONV_PATCH_PB(tap)>{}, hb + 1, OTHER{});
-			if constexpr (CONV_PATCH_NB(tap) >= 2)
-				issue_b(std::integral_constant<int, CONV_PATCH_PB(tap) + 1>{}, hb + 1, OTHER{});
-			issue_a(ST{}, hb + (tap + NST) / 9, (tap + NST) % 9);
-			mma(1);
-		};
-		auto block = [&](int hb, auto buf_) {
-			step(hb, buf_, std::integral_constant<int, 0>{});
-			step(hb, buf_, std::integral_constant<int, 1>{});
-			step(hb, buf_, std::integral_constant<int, 2>{});
-			step(hb, buf_, std::integral_constant<int, 3>{});
-			step(hb, buf_, std::integral_constant<int, 4>{});
-			step(hb, buf_, std::integral_constant<int, 5>{});
-			step(hb, buf_, std::integral_constant<int, 6>{});
-			step(hb, buf_, std::integral_constant<int, 7>{});
-			step(hb, buf_, std::integral_constant<int, 8>{});
-		};
-		for (int hb = 0; hb < NB; hb += 2) {
-			block(hb, C0{});
-			block(hb + 1, C1{});
-		}
 	}
+	/* the per-plane constants of every plane block, or of this tile's if it is the only one (behind the
+	 * first loads: they are waited for anyway) */
+	const int row0 = WALK ? 0 : cur.tile_m * BM;
+	for (int i = tid; i < (WALK ? p.tiles_m * BM : BM); i += 256) {
+		const int mc = min(row0 + i, p.Co - 1);
+		rowc[i] = p.bias ? p.bias[mc] : 0.0f;
+		rowc[ROWC + i] = p.scale ? p.scale[mc] : 1.0f;
+	}
+	/* the patch (its last load: step BL - 10) and K-tile 0 (step 1 - NST): what the steps after both issued may be outstanding */
+	wide_wait<(BL - 10 > 1 - NST ? 10 - BL : NST - 2) * A_PW, true>();
+	__builtin_amdgcn_s_barrier();
+	read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
+	read_frags(C0{}, C0{}, C0{}, 1, af[1], bf[1]);
+	auto step = [&](int hb, auto buf_, auto tap_) {
+		constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
+		constexpr int par = (tap + buf) & 1;
+		typedef std::integral_constant<int, (9 * buf + tap + 1) % NST> ST1;
+		typedef std::integral_constant<int, (9 * buf + tap + NST - 1) % NST> STP;
+		typedef std::integral_constant<int, (tap + 1) % 9> TAP1;
+		typedef std::integral_constant<int, buf ^ 1> OTHER;
+		typedef std::integral_constant<int, tap == 8 ? buf ^ 1 : buf> BUF1;
+		wide_wait<allowed(tap), false>();
+		__builtin_amdgcn_s_barrier();
+		if constexpr (CONV_PATCH_NB(tap) >= 1)
+			issue_b(std::integral_constant<int, CONV_PATCH_PB(tap)>{}, hb + 1, OTHER{});
+		issue_a(STP{}, hb + (tap + NST - 1) / 9, (tap + NST - 1) % 9);
+		read_frags(ST1{}, BUF1{}, TAP1{}, 0, af[2 * (par ^ 1)], bf[2 * (par ^ 1)]);
+		__builtin_amdgcn_sched_barrier(0);	/* (the fragments are asked for before the MFMAs that follow in the source) */
+		mma(2 * par);
+		read_frags(ST1{}, BUF1{}, TAP1{}, 1, af[2 * (par ^ 1) + 1], bf[2 * (par ^ 1) + 1]);
+		__builtin_amdgcn_sched_barrier(0);
+		mma(2 * par + 1);
+	};
 #undef CONV_PATCH_NB
 #undef CONV_PATCH_PB
-	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the epilogue reuses it) */
+	auto block = [&](int hb, auto buf_) {
+		step(hb, buf_, std::integral_constant<int, 0>{});
+		step(hb, buf_, std::integral_constant<int, 1>{});
+		step(hb, buf_, std::integral_constant<int, 2>{});
+		step(hb, buf_, std::integral_constant<int, 3>{});
+		step(hb, buf_, std::integral_constant<int, 4>{});
+		step(hb, buf_, std::integral_constant<int, 5>{});
+		step(hb, buf_, std::integral_constant<int, 6>{});
+		step(hb, buf_, std::integral_constant<int, 7>{});
+		step(hb, buf_, std::integral_constant<int, 8>{});
+	};
 
-	/* ---- epilogue ---- */
+	/* ---- (factor,) bias, Threshold, (pooling,) store of a finished tile ---- */
 	elem *y = (elem *)p.y;
-	int *lrow = (int *)astage;
-	__syncthreads();
-	if (tid < BM) {
-		const int mc = min(tile_m * BM + tid, p.Co - 1);
-		lrow[tid] = __float_as_int(p.bias ? p.bias[mc] : 0.0f);
-		if (p.scale)
-			lrow[BM + tid] = __float_as_int(p.scale[mc]);
-	}
-	__syncthreads();
 	const bool has_scale = p.scale != 0;
-	if constexpr (POOL && WHOLE) {
-		/* a window's four members in four neighbouring lanes; the first one stores */
-		const int pH = p.oH / 2, pW = p.oW / 2;
+	auto store_tile = [&](const Tile &T) {
+		const float *lrow = rowc + (WALK ? T.tile_m * BM : 0);
+		auto finish = [&](float a, float s, float b) {
+			float v = has_scale ? a * s + b : a + b;
+			if (p.act)
+				v = v > p.thr ? v : p.val;
+			return v;
+		};
+		if constexpr (POOL && WHOLE) {
+			/* a window's four members in four neighbouring lanes; the first one stores */
+			const int pH = p.oH / 2, pW = p.oW / 2;
 #pragma unroll
-		for (int j = 0; j < TN; j++) {
-			const int py = oy_[j] >> 1, px = ox_[j] >> 1;
-			const bool store = !(lane & 3) && oy_[j] >= 0;
-			const size_t n = ((size_t)img * pH + py) * pW + px;
-			const size_t ybase = (size_t)img * p.Co * pH * pW + (size_t)py * pW + px;
+			for (int j = 0; j < TN; j++) {
+				const int py = oy_[j] >> 1, px = ox_[j] >> 1;
+				const bool store = !(lane & 3) && oy_[j] >= 0;
+				const size_t n = ((size_t)T.img * pH + py) * pW + px;
+				const size_t ybase = (size_t)T.img * p.Co * pH * pW + (size_t)py * pW + px;
+#pragma unroll
+				for (int i = 0; i < TM; i++) {
+					const int m0 = T.tile_m * BM + i * 32 + 4 * (lane >> 5);
+#pragma unroll
+					for (int g = 0; g < 4; g++) {
+						struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+						const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
+						const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+						const floatx4 rowscale = *(const floatx4 *)(lrow + ROWC + ml);
+#pragma unroll
+						for (int e = 0; e < 4; e++) {
+							const int m = m0 + 8 * g + e;
+							float v = finish(acc[i][j][4 * g + e], rowscale[e], rowbias[e]);
+							v = (float)(elem)v;	/* the pooling compares the stored (rounded) values */
+							v = fmaxf(v, __shfl_xor(v, 1));
+							v = fmaxf(v, __shfl_xor(v, 2));
+							if constexpr (!CLO) {
+								if (store && m < p.Co)
+									y[ybase + (size_t)m * pH * pW] = (elem)v;
+							}
+							quad.v[e] = (elem)v;
+						}
+						if constexpr (CLO) {
+							if (store && m0 + 8 * g < p.Co)
+								*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
+						}
+					}
+				}
+			}
+		} else if constexpr (POOL) {
+			/* The 2x2 / stride 2 max pooling that follows, here: the two rows of a
+			 * window are this wave's two tile rows (the same accumulator index), its
+			 * two columns neighbouring lanes.  Threshold first, as the modules run. */
+			const int pH = p.oH / 2, pW = p.oW / 2;
+			const int py = T.ty * (TH / 2) + wave, px = T.tx * (TW / 2) + ((lane & 31) >> 1);
+			const bool store = !(lane & 1) && py < pH && px < pW;
+			const size_t n = ((size_t)T.img * pH + py) * pW + px;
+			const size_t ybase = (size_t)T.img * p.Co * pH * pW + (size_t)py * pW + px;
 #pragma unroll
 			for (int i = 0; i < TM; i++) {
-				const int m0 = tile_m * BM + i * 32 + 4 * (lane >> 5);
+				const int m0 = T.tile_m * BM + i * 32 + 4 * (lane >> 5);
 #pragma unroll
 				for (int g = 0; g < 4; g++) {
 					struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
 					const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
 					const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
-					floatx4 rowscale = { 1, 1, 1, 1 };
-					if (has_scale)
-						rowscale = *(const floatx4 *)(lrow + BM + ml);
+					const floatx4 rowscale = *(const floatx4 *)(lrow + ROWC + ml);
 #pragma unroll
 					for (int e = 0; e < 4; e++) {
-						const int r = 4 * g + e, m = m0 + 8 * g + e;
-						float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
-						if (p.act)
-							v = v > p.thr ? v : p.val;
-						v = (float)(elem)v;	/* the pooling compares the stored (rounded) values */
+						const int m = m0 + 8 * g + e;
+						const float v0 = finish(acc[i][0][4 * g + e], rowscale[e], rowbias[e]);
+						const float v1 = finish(acc[i][1][4 * g + e], rowscale[e], rowbias[e]);
+						/* the pooling compares the stored (rounded) values */
+						float v = fmaxf((float)(elem)v0, (float)(elem)v1);
 						v = fmaxf(v, __shfl_xor(v, 1));
-						v = fmaxf(v, __shfl_xor(v, 2));
 						if constexpr (!CLO) {
 							if (store && m < p.Co)
 								y[ybase + (size_t)m * pH * pW] = (elem)v;
@@ -435,93 +423,65 @@ __global__ __launch_bounds__(256) void conv_patch_kernel(ConvParams p)
 					}
 				}
 			}
-		}
-		return;
-	}
-	if constexpr (POOL) {
-		/* The 2x2 / stride 2 max pooling that follows, here: the two rows of a
-		 * window are this wave's two tile rows (the same accumulator index), its
-		 * two columns neighbouring lanes.  Threshold first, as the modules run. */
-		const int pH = p.oH / 2, pW = p.oW / 2;
-		const int py = ty * (TH / 2) + wave, px = tx * (TW / 2) + ((lane & 31) >> 1);
-		const bool store = !(lane & 1) && py < pH && px < pW;
-		const size_t n = ((size_t)img * pH + py) * pW + px;
-		const size_t ybase = (size_t)img * p.Co * pH * pW + (size_t)py * pW + px;
+		} else {
 #pragma unroll
-		for (int i = 0; i < TM; i++) {
-			const int m0 = tile_m * BM + i * 32 + 4 * (lane >> 5);
+			for (int j = 0; j < TN; j++) {
+				const int oy = WHOLE ? oy_[j] : T.ty * TH + 2 * wave + j, ox = WHOLE ? ox_[j] : T.tx * TW + (lane & 31);
+				if (oy < 0 || oy >= p.oH || ox >= p.oW)
+					continue;
+				const int rem = oy * p.oW + ox;
+				const size_t n = (size_t)T.img * p.oHW + rem;
+				const size_t ybase = (size_t)T.img * p.Co * p.oHW + rem;
 #pragma unroll
-			for (int g = 0; g < 4; g++) {
-				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
-				const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
-				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
-				floatx4 rowscale = { 1, 1, 1, 1 };
-				if (has_scale)
-					rowscale = *(const floatx4 *)(lrow + BM + ml);
+				for (int i = 0; i < TM; i++) {
+					const int m0 = T.tile_m * BM + i * 32 + 4 * (lane >> 5);
 #pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int r = 4 * g + e, m = m0 + 8 * g + e;
-					float v0 = has_scale ? acc[i][0][r] * rowscale[e] + rowbias[e] : acc[i][0][r] + rowbias[e];
-					float v1 = has_scale ? acc[i][1][r] * rowscale[e] + rowbias[e] : acc[i][1][r] + rowbias[e];
-					if (p.act) {
-						v0 = v0 > p.thr ? v0 : p.val;
-						v1 = v1 > p.thr ? v1 : p.val;
+					for (int g = 0; g < 4; g++) {
+						struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
+						const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
+						const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
+						const floatx4 rowscale = *(const floatx4 *)(lrow + ROWC + ml);
+#pragma unroll
+						for (int e = 0; e < 4; e++) {
+							const int m = m0 + 8 * g + e;
+							const float v = finish(acc[i][j][4 * g + e], rowscale[e], rowbias[e]);
+							if constexpr (!CLO) {
+								if (m < p.Co)
+									y[ybase + (size_t)m * p.oHW] = (elem)v;
+							}
+							quad.v[e] = (elem)v;
+						}
+						if constexpr (CLO) {
+							if (m0 + 8 * g < p.Co)
+								*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
+						}
 					}
-					/* the pooling compares the stored (rounded) values */
-					float v = fmaxf((float)(elem)v0, (float)(elem)v1);
-					v = fmaxf(v, __shfl_xor(v, 1));
-					if constexpr (!CLO) {
-						if (store && m < p.Co)
-							y[ybase + (size_t)m * pH * pW] = (elem)v;
-					}
-					quad.v[e] = (elem)v;
-				}
-				if constexpr (CLO) {
-					if (store && m0 + 8 * g < p.Co)
-						*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
 				}
 			}
 		}
-		return;
-	}
-#pragma unroll
-	for (int j = 0; j < TN; j++) {
-		const int oy = WHOLE ? oy_[j] : ty * TH + 2 * wave + j, ox = WHOLE ? ox_[j] : tx * TW + (lane & 31);
-		if (oy < 0 || oy >= p.oH || ox >= p.oW)
-			continue;
-		const int rem = oy * p.oW + ox;
-		const size_t n = (size_t)img * p.oHW + rem;
-		const size_t ybase = (size_t)img * p.Co * p.oHW + rem;
-#pragma unroll
-		for (int i = 0; i < TM; i++) {
-			const int m0 = tile_m * BM + i * 32 + 4 * (lane >> 5);
-#pragma unroll
-			for (int g = 0; g < 4; g++) {
-				struct alignas(4 * sizeof(elem)) Quad { elem v[4]; } quad;
-				const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
-				const floatx4 rowbias = *(const floatx4 *)(lrow + ml);
-				floatx4 rowscale = { 1, 1, 1, 1 };
-				if (has_scale)
-					rowscale = *(const floatx4 *)(lrow + BM + ml);
-#pragma unroll
-				for (int e = 0; e < 4; e++) {
-					const int r = 4 * g + e, m = m0 + 8 * g + e;
-					float v = has_scale ? acc[i][j][r] * rowscale[e] + rowbias[e] : acc[i][j][r] + rowbias[e];
-					if (p.act)
-						v = v > p.thr ? v : p.val;
-					if constexpr (!CLO) {
-						if (m < p.Co)
-							y[ybase + (size_t)m * p.oHW] = (elem)v;
-					}
-					quad.v[e] = (elem)v;
-				}
-				if constexpr (CLO) {
-					if (m0 + 8 * g < p.Co)
-						*(Quad *)(y + n * p.Co + m0 + 8 * g) = quad;
-				}
-			}
+	};
+
+	for (;;) {
+		for (int hb = 0; hb < NB; hb += 2) {
+			block(hb, C0{});
+			block(hb + 1, C1{});
 		}
+		store_tile(cur);
+		if (!WALK || !nxt.ok)
+			break;
+		cur = nxt;
+#pragma unroll
+		for (int t = 0; t < BL; t++)
+			voff_[t] = voffn_[t];
+#pragma unroll
+		for (int i = 0; i < A_PW; i++)
+			a_off_[i] = a_offn_[i];
+		nlocal += nloc;
+		nxt = decode(nlocal);
+		offsets(nxt, voffn_, a_offn_);
+		clear();
 	}
+	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS) */
 #endif
 }
 
@@ -531,7 +491,7 @@ bool thhip_conv_half_patch_ok(const ConvParams &p, int dtype)
 	if (dtype != THHIP_F16 && dtype != THHIP_BF16)
 		return false;
 	return p.x_cl == 1 && (p.Ci == 64 || p.Ci == 128 || p.Ci == 256 || p.Ci == 512) && p.kH == 3 && p.kW == 3 && p.dH == 1 && p.dW == 1 &&
-		p.x_bytes < 0x7fffffffu && (!p.y_cl || p.Co % 4 == 0);
+		p.x_bytes < 0x7fffffffu && (!p.y_cl || p.Co % 4 == 0) && (p.Ci != 64 || p.Co <= PATCH_ROWC);
 }
 
 /* Whether the whole-image form is the one to run: an output of at most 14 x 14 that fills at least five of
@@ -547,6 +507,46 @@ bool thhip_conv_half_patch_flat_ok(const ConvParams &p, int dtype)
 	return slots > 128 && (long)p.B * (p.Co / 32) >= 128;
 }
 
+/* Workgroups of a kernel that one CU holds at once (by its registers and LDS), asked once per kernel. */
+template <void (*kernel)(ConvParams)>
+static int patch_residents()
+{
+	static int n;
+	if (!n) {
+		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, 256, 0));
+		if (n < 1)
+			THError("thhip_conv2d: the patch kernel does not fit a CU");
+	}
+	return n;
+}
+
+static int patch_cus()
+{
+	static int n;
+	if (!n) {
+		int dev;
+		hipcheck(hipGetDevice(&dev));
+		hipcheck(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+	}
+	return n;
+}
+
+template <void (*kernel)(ConvParams)>
+static void patch_go(ConvParams &p, long per_xcd, bool walk)
+{
+	/* walk: as many workgroups per XCD as it holds at once, or fewer when that spreads its tiles as evenly:
+	 * each then walks rounds = ceil(tiles / workgroups) tiles or one less.  Else one workgroup per tile,
+	 * which the dispatcher hands to the CUs as they come free. */
+	long n = per_xcd;
+	if (walk) {
+		const long slots = (long)(patch_cus() / 8) * patch_residents<kernel>();
+		n = per_xcd < slots ? per_xcd : slots;
+		const long rounds = (per_xcd + n - 1) / n;
+		n = (per_xcd + rounds - 1) / rounds;
+	}
+	kernel<<<dim3((unsigned)(8 * n)), dim3(256), 0, thhip_stream()>>>(p);
+}
+
 template <int DT, int BM, bool WHOLE>
 static void conv_launch_patch(ConvParams &p)
 {
@@ -555,6 +555,9 @@ static void conv_launch_patch(ConvParams &p)
 	p.splitk = 1;
 	if ((size_t)p.tiles_m * BM / 32 * p.KC * 1024 > p.w_bytes)
 		THError("thhip_conv2d: packed weights shorter than the tile grid");
+	const bool walk = p.Ci == 64;	/* (the kernel's WALK) */
+	if (walk && p.tiles_m * BM > PATCH_ROWC)
+		THError("thhip_conv2d: the patch kernel keeps the constants of at most %d planes", PATCH_ROWC);
 	const long total = (long)p.tiles_m * p.tiles_n;
 	long per_xcd = (total + 7) / 8;
 	if constexpr (WHOLE) {
@@ -578,13 +581,12 @@ static void conv_launch_patch(ConvParams &p)
 			per_xcd = cnt > per_xcd ? cnt : per_xcd;
 		}
 	}
-	dim3 grid((unsigned)(8 * per_xcd));
-#define CONV_PATCH_GO(CLO, CI)                                                                                      \
-	do {                                                                                                       \
-		if (p.pool)                                                                                        \
-			conv_patch_kernel<DT, CLO, BM, CI, true, WHOLE><<<grid, dim3(256), 0, thhip_stream()>>>(p);  \
-		else                                                                                               \
-			conv_patch_kernel<DT, CLO, BM, CI, false, WHOLE><<<grid, dim3(256), 0, thhip_stream()>>>(p); \
+#define CONV_PATCH_GO(CLO, CI)                                                              \
+	do {                                                                               \
+		if (p.pool)                                                                \
+			patch_go<conv_patch_kernel<DT, CLO, BM, CI, true, WHOLE>>(p, per_xcd, walk);  \
+		else                                                                       \
+			patch_go<conv_patch_kernel<DT, CLO, BM, CI, false, WHOLE>>(p, per_xcd, walk); \
 	} while (0)
 	if constexpr (!WHOLE) {
 		if (p.Ci == 64 && p.y_cl)
@@ -607,19 +609,20 @@ static void conv_launch_patch(ConvParams &p)
 #undef CONV_PATCH_GO
 }
 
-/* bm: output planes per workgroup (64 or 128; the whole-image form: 32 or 64) */
+/* flat: the whole-image form, with bm = 32 or 64 output planes per workgroup (the 32 x 8 tiles: always 64) */
 void thhip_conv_half_patch_launch(ConvParams &p, int dtype, int bm, int flat)
 {
 	if (!thhip_conv_half_patch_ok(p, dtype))
-		THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64, 128, 256 or 512 planes, 3x3, stride 1");
+		THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64, 128, 256 or 512 planes, 3x3, stride 1, at most %d output planes",
+			PATCH_ROWC);
 	if (flat && !thhip_conv_half_patch_flat_ok(p, dtype))
 		THError("thhip_conv2d: the whole-image patch kernel needs 256 or 512 input planes, padding 1 and an output of at most 14 x 14");
 	if (dtype == THHIP_F16) {
 		if (flat)
 			return bm == 32 ? conv_launch_patch<THHIP_F16, 32, true>(p) : conv_launch_patch<THHIP_F16, 64, true>(p);
-		return bm == 128 ? conv_launch_patch<THHIP_F16, 128, false>(p) : conv_launch_patch<THHIP_F16, 64, false>(p);
+		return conv_launch_patch<THHIP_F16, 64, false>(p);
 	}
 	if (flat)
 		return bm == 32 ? conv_launch_patch<THHIP_BF16, 32, true>(p) : conv_launch_patch<THHIP_BF16, 64, true>(p);
-	return bm == 128 ? conv_launch_patch<THHIP_BF16, 128, false>(p) : conv_launch_patch<THHIP_BF16, 64, false>(p);
+	return conv_launch_patch<THHIP_BF16, 64, false>(p);
 }

@@ -3311,12 +3311,11 @@ static void conv_dispatch(ConvParams &p)
 			THError("thhip_conv2d: the patch kernel needs a half type, channels-last input of 64, 128, 256 or 512 planes, 3x3, stride 1");
 		/* a whole image of at most 14 x 14 per workgroup: 64 planes where that makes 256 workgroups, else 32
 		 * (the tuning hook's last argument: 3 forces 32, 4 forces 64, 5 the 32 x 8 tiles) */
-		if (conv_patch_flat<DT>(p) && g_force_wgs != 5 && g_force_wgs != 2) {
+		if (conv_patch_flat<DT>(p) && g_force_wgs != 5) {
 			const bool small = g_force_wgs == 3 || (g_force_wgs != 4 && (long)p.B * (p.Co / 64) < 256);
 			return thhip_conv_half_patch_launch(p, DT, small ? 32 : 64, 1);
 		}
-		/* (the tuning hook's last argument 2: 128 planes per workgroup) */
-		return thhip_conv_half_patch_launch(p, DT, g_force_wgs == 2 && p.Co % 128 == 0 ? 128 : 64, 0);
+		return thhip_conv_half_patch_launch(p, DT, 64, 0);
 	}
 	if constexpr (DT == THHIP_F32) {
 		if (direct && rows)
