@@ -216,6 +216,38 @@ __device__ __forceinline__ void wide_wait()
 #undef WIDE_WAIT_CASE
 }
 
+/* Channels-last stores of a 32x32 accumulator.  Lane l holds, for position
+ * l % 32, the four planes 4 (l / 32) + 8 g + e of group g = 0..3: stored as it
+ * lies, an instruction writes 64 separate pieces of four values.
+ * v_permlane32_swap(x, y) exchanges x of lanes 32..63 with y of lanes 0..31, so
+ * after it the low lane owns both halves of x's group and the high lane both
+ * halves of y's: every lane then writes 16 bytes, in half (uint8: a quarter)
+ * as many instructions, and lanes l and l + 32 write neighbouring pieces.
+ * Every lane of the wave must take part (no divergence around the calls). */
+__device__ __forceinline__ void conv_swap32(unsigned &x, unsigned &y)
+{
+	const auto r = __builtin_amdgcn_permlane32_swap(x, y, false, false);
+	x = r[0];
+	y = r[1];
+}
+
+/* Half types: lo[g], hi[g] = planes 0..1 and 2..3 of group g as packed pairs.
+ * yn points at the position's plane 0 of this accumulator's 32 planes; planes
+ * from `left` on do not exist (left % 8 == 0, rows 16-byte aligned). */
+__device__ __forceinline__ void conv_store_cl_half(unsigned short *yn, int left, bool valid, unsigned (&lo)[4], unsigned (&hi)[4], int lane)
+{
+#pragma unroll
+	for (int h = 0; h < 2; h++) {
+		conv_swap32(lo[2 * h], lo[2 * h + 1]);
+		conv_swap32(hi[2 * h], hi[2 * h + 1]);
+		const int m = 16 * h + 8 * (lane >> 5);
+		if (valid && m < left) {
+			uintx4 v = { lo[2 * h], hi[2 * h], lo[2 * h + 1], hi[2 * h + 1] };
+			*(uintx4 *)(yn + m) = v;
+		}
+	}
+}
+
 /* conv_patch_kernel's output tile (positions of one image) */
 #define PATCH_TW 32
 #define PATCH_TH 8

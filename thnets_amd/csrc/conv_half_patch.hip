@@ -338,11 +338,94 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 	/* ---- (factor,) bias, Threshold, (pooling,) store of a finished tile ---- */
 	elem *y = (elem *)p.y;
-	const bool has_scale = p.scale != 0;
 	auto store_tile = [&](const Tile &T) {
 		const float *lrow = rowc + (WALK ? T.tile_m * BM : 0);
+		/* The usual case, channels-last output after a ReLU (Threshold(0, 0)), on packed pairs: a rounded
+		 * value at or above zero orders as its bits do, and a negative one is a negative 16-bit integer, so
+		 * the pooling is an integer maximum and the ReLU one more against zero afterwards (the results are
+		 * those of the general code below; a finished tile costs a quarter of its instructions, which with
+		 * 64 input planes was two fifths of a tile's time).  The two lanes of a position then exchange groups
+		 * and each writes 16 bytes (conv_store_cl_half). */
+		if constexpr (CLO) {
+			if (p.act && p.thr == 0.0f && p.val == 0.0f && p.Co % 8 == 0) {
+				typedef short shortx2 __attribute__((ext_vector_type(2)));
+				typedef elem elemx2 __attribute__((ext_vector_type(2)));
+				auto pack2 = [](float a, float b) {
+					const elemx2 v = { (elem)a, (elem)b };
+					return __builtin_bit_cast(unsigned, v);
+				};
+				auto max2 = [](unsigned a, unsigned b) {
+					return __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(shortx2, a), __builtin_bit_cast(shortx2, b)));
+				};
+				/* accumulator i of tile row / slot block j as eight packed pairs: lo[g], hi[g] = planes 0..1, 2..3 of group g */
+				auto packed = [&](int i, int j, unsigned (&lo)[4], unsigned (&hi)[4]) {
+#pragma unroll
+					for (int g = 0; g < 4; g++) {
+						const int ml = i * 32 + 4 * (lane >> 5) + 8 * g;
+						const floatx4 rb = *(const floatx4 *)(lrow + ml), rs = *(const floatx4 *)(lrow + ROWC + ml);
+						lo[g] = pack2(__builtin_fmaf(acc[i][j][4 * g], rs[0], rb[0]), __builtin_fmaf(acc[i][j][4 * g + 1], rs[1], rb[1]));
+						hi[g] = pack2(__builtin_fmaf(acc[i][j][4 * g + 2], rs[2], rb[2]), __builtin_fmaf(acc[i][j][4 * g + 3], rs[3], rb[3]));
+					}
+				};
+				unsigned short *const yh = (unsigned short *)y;
+#pragma unroll
+				for (int i = 0; i < TM; i++) {
+					const int mt = T.tile_m * BM + i * 32;
+					if constexpr (POOL && WHOLE) {
+						const int pH = p.oH / 2, pW = p.oW / 2;
+#pragma unroll
+						for (int j = 0; j < TN; j++) {
+							unsigned lo[4], hi[4];
+							packed(i, j, lo, hi);
+#pragma unroll
+							for (int g = 0; g < 4; g++) {
+								lo[g] = max2(lo[g], (unsigned)__builtin_amdgcn_update_dpp(0, (int)lo[g], 0xB1, 0xF, 0xF, false));
+								hi[g] = max2(hi[g], (unsigned)__builtin_amdgcn_update_dpp(0, (int)hi[g], 0xB1, 0xF, 0xF, false));
+								lo[g] = max2(max2(lo[g], (unsigned)__builtin_amdgcn_update_dpp(0, (int)lo[g], 0x4E, 0xF, 0xF, false)), 0u);
+								hi[g] = max2(max2(hi[g], (unsigned)__builtin_amdgcn_update_dpp(0, (int)hi[g], 0x4E, 0xF, 0xF, false)), 0u);
+							}
+							const int py = oy_[j] >> 1, px = ox_[j] >> 1;
+							const size_t n = ((size_t)T.img * pH + py) * pW + px;
+							conv_store_cl_half(yh + n * p.Co + mt, p.Co - mt, !(lane & 3) && oy_[j] >= 0, lo, hi, lane);
+						}
+					} else if constexpr (POOL) {
+						const int pH = p.oH / 2, pW = p.oW / 2;
+						const int py = T.ty * (TH / 2) + wave, px = T.tx * (TW / 2) + ((lane & 31) >> 1);
+						const size_t n = ((size_t)T.img * pH + py) * pW + px;
+						unsigned lo[4], hi[4], lo1[4], hi1[4];
+						packed(i, 0, lo, hi);
+						packed(i, 1, lo1, hi1);
+#pragma unroll
+						for (int g = 0; g < 4; g++) {
+							lo[g] = max2(lo[g], lo1[g]);
+							hi[g] = max2(hi[g], hi1[g]);
+							lo[g] = max2(max2(lo[g], (unsigned)__builtin_amdgcn_update_dpp(0, (int)lo[g], 0xB1, 0xF, 0xF, false)), 0u);
+							hi[g] = max2(max2(hi[g], (unsigned)__builtin_amdgcn_update_dpp(0, (int)hi[g], 0xB1, 0xF, 0xF, false)), 0u);
+						}
+						conv_store_cl_half(yh + n * p.Co + mt, p.Co - mt, !(lane & 1) && py < pH && px < pW, lo, hi, lane);
+					} else {
+#pragma unroll
+						for (int j = 0; j < TN; j++) {
+							const int oy = WHOLE ? oy_[j] : T.ty * TH + 2 * wave + j, ox = WHOLE ? ox_[j] : T.tx * TW + (lane & 31);
+							const bool valid = oy >= 0 && oy < p.oH && ox < p.oW;
+							const size_t n = (size_t)T.img * p.oHW + (valid ? oy * p.oW + ox : 0);
+							unsigned lo[4], hi[4];
+							packed(i, j, lo, hi);
+#pragma unroll
+							for (int g = 0; g < 4; g++) {
+								lo[g] = max2(lo[g], 0u);
+								hi[g] = max2(hi[g], 0u);
+							}
+							conv_store_cl_half(yh + n * p.Co + mt, p.Co - mt, valid, lo, hi, lane);
+						}
+					}
+				}
+				return;
+			}
+		}
+		/* (one fused multiply-add in both forms of the epilogue: they must round alike; the factor is 1 without a batch norm) */
 		auto finish = [&](float a, float s, float b) {
-			float v = has_scale ? a * s + b : a + b;
+			float v = __builtin_fmaf(a, s, b);
 			if (p.act)
 				v = v > p.thr ? v : p.val;
 			return v;
