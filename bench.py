@@ -296,8 +296,9 @@ def main():
             "bound": "mfma", "achieved": round(i8_tops, 3), "peak": PEAK_TOPS_INT8_MFMA, "unit": "TOP/s",
             "frac": round(i8_tops / PEAK_TOPS_INT8_MFMA, 4),
             "traffic": counter_traffic("conv_u8_alexnet_owt_b64_counters.md", "conv_hbm_bytes_per_launch"),
-            "kernel": "conv_u8_image_pool_kernel, conv_u8_patch_kernel<pool>, conv_wide_kernel<uint8>, linear_u8_kernel "
-                      "(uint8 AlexNet-OWT batch 64: eight launches per step)",
+            "kernel": "conv_u8_image_pool_kernel (conv1 with its pooling), conv_u8_patch_kernel (conv2-5: the input patch of a band "
+                      "resident in LDS or streamed plane block by plane block, pooling in the epilogue where one follows), "
+                      "linear_u8_kernel (fc6-8) (uint8 AlexNet-OWT batch 64: eight launches per step)",
             "launches_per_step": i8_n / max(args.steps, 20), "avg_launch_ms": round(i8_ms / max(i8_n, 1), 5),
             "ops_per_launch": i8_ops / max(i8_n, 1),
             "cpu_baseline": None,
