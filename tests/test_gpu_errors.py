@@ -178,3 +178,44 @@ C.CDLL(None).fflush(None)
         want = outs[i + 1] if cfg["layers"][i]["type"] == "conv" and cfg["layers"][i + 1]["type"] == "threshold" else outs[i]
         assert abs(mn - float(want.min())) <= 2e-5 * max(1, abs(float(want.min()))) + 1e-6, (i, line)
         assert abs(mx - float(want.max())) <= 2e-5 * max(1, abs(float(want.max()))) + 1e-6, (i, line)
+
+
+def test_th_minmax_where_threshold_and_pooling_run_in_the_convolution(hiplib, oracle):
+    """A convolution that takes the Threshold and the 2x2 pooling after it into its epilogue writes the
+    pooled tensor only, so its line (and the lines of the two modules it absorbed, which pass that tensor
+    on) shows the pooled tensor's range: the maximum is the convolution's own, the minimum that of the
+    window maxima.  One line per module all the same (thapi.c:197-202)."""
+    r = child(r"""
+g = cases.rng(77)
+from thnets_amd import configs
+w1 = g.standard_normal((32, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+w2 = g.standard_normal((64, 32, 3, 3), dtype=np.float32) * np.float32(0.08)
+layers = [configs.conv(w1, g.standard_normal(32, dtype=np.float32) * np.float32(0.1), 1, 1), configs.relu(),
+          configs.conv(w2, g.standard_normal(64, dtype=np.float32) * np.float32(0.1), 1, 1), configs.relu(), configs.maxpool(2, 2)]
+x = g.uniform(0, 1, (3, 3, 128, 128)).astype(np.float32)
+assert lib.thhip_conv2d_pool2_supported(3, 32, 128, 128, 64, 3, 3, 1, 1, 1, 1, 0, 0, 0)
+C.c_int.in_dll(lib, "th_minmax").value = 1
+net = api.HipNetwork(layers, cfg["mean"], cfg["std"])
+net.process_float(x.copy())
+C.CDLL(None).fflush(None)
+""")
+    assert r.returncode == 0, r.stderr
+    lines = [l for l in r.stdout.splitlines() if l.startswith("Layer ")]
+    assert len(lines) == 5, lines
+    from thnets_amd import configs
+    g = cases.rng(77)
+    w1 = g.standard_normal((32, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+    w2 = g.standard_normal((64, 32, 3, 3), dtype=np.float32) * np.float32(0.08)
+    layers = [configs.conv(w1, g.standard_normal(32, dtype=np.float32) * np.float32(0.1), 1, 1), configs.relu(),
+              configs.conv(w2, g.standard_normal(64, dtype=np.float32) * np.float32(0.1), 1, 1), configs.relu(), configs.maxpool(2, 2)]
+    x = g.uniform(0, 1, (3, 3, 128, 128)).astype(np.float32)
+    cfg = cases.small_networks()["tiny_cnn"]
+    outs = []
+    oracle.run_layers(layers, oracle.normalize(x, cfg["mean"], cfg["std"]), collect=outs)
+    want = [outs[1], outs[1], outs[4], outs[4], outs[4]]      # (thresholded; thresholded and pooled)
+    for i, line in enumerate(lines):
+        assert line.startswith("Layer %d output: min=" % (i + 1))
+        mn = float(line.split("min=")[1].split(",")[0])
+        mx = float(line.split("max=")[1])
+        assert abs(mn - float(want[i].min())) <= 2e-5 * max(1, abs(float(want[i].min()))) + 1e-6, (i, line, float(want[i].min()))
+        assert abs(mx - float(want[i].max())) <= 2e-5 * max(1, abs(float(want[i].max()))) + 1e-6, (i, line, float(want[i].max()))

@@ -3074,6 +3074,21 @@ static bool conv_pool_uses_patch(const ConvParams &p)
 	return false;
 }
 
+/* fp32 layers of at most 512 tiles of 64 x 64 (a long K, few positions): the K parts their whole K range is cut
+ * into -- about 1024 workgroups' worth, at least eight K-tiles each, at most sixteen; 1: no split.  The one rule
+ * both conv_dispatch and the entry points that must know the split beforehand (thhip_conv2d_poolk_supported) use. */
+static int conv_f32_ksplit(long t64, int nkt)
+{
+	if (t64 > 512)
+		return 1;
+	int parts = (int)((1024 + t64 - 1) / t64);
+	if (parts > nkt / 8)
+		parts = nkt / 8;
+	if (parts > 16)
+		parts = 16;
+	return parts > 1 ? parts : 1;
+}
+
 /* conv_f32_patch_kernel takes layers of at least this many 64 x 64 tiles (below, conv_dispatch splits K
  * of the whole layer) */
 #define CONV_F32_PATCH_MIN 513
@@ -3189,14 +3204,7 @@ static void conv_dispatch(ConvParams &p)
 			 * 181 -> 161 us (3 parts), @7^2 batch 32 108 -> 96 us; AlexNet batch 1,
 			 * against the other kernel's in-kernel split: conv2 32 -> 15, conv3
 			 * 25 -> 14, conv4 27 -> 16, conv5 31 -> 15 us. */
-			const int nkt = p.KC / kch;
-			int parts = (int)((1024 + t64 - 1) / t64);
-			if (parts > nkt / 8)
-				parts = nkt / 8;
-			if (parts > 16)
-				parts = 16;
-			if (parts > 1)
-				splitk = parts;
+			splitk = conv_f32_ksplit(t64, p.KC / kch);
 		}
 	} else if (DT == THHIP_F32 && conv_f32_rows_ok(p) && (p.dW == 1 || t64 <= 512) && !g_force_kch && !g_force_bm && !g_force_bn) {
 		/* any other number of planes (image layers with larger kernels): the same kernel with a tap of
@@ -3206,16 +3214,8 @@ static void conv_dispatch(ConvParams &p)
 		 * a few tiles with a K split: 17 -> 11 us). */
 		direct = rows = true;
 		kch = 2;
-		if (t64 <= 512) {
-			const int nkt = p.KC / kch;
-			int parts = (int)((1024 + t64 - 1) / t64);
-			if (parts > nkt / 8)
-				parts = nkt / 8;
-			if (parts > 16)
-				parts = 16;
-			if (parts > 1)
-				splitk = parts;
-		}
+		if (t64 <= 512)
+			splitk = conv_f32_ksplit(t64, p.KC / kch);
 	} else if (DT == THHIP_F32 && t128 >= 300) {
 		kch = 2;
 		if (p.Co > 64 && t128 >= 700)
@@ -3714,12 +3714,7 @@ static int conv_f32_split_parts(int B, int Ci, int H, int W, int Co, int kH, int
 		kch = 2;	/* a (plane, tap) per K row */
 	else
 		return 0;
-	const int nkt = conv_kc(Ci, kH, kW, THHIP_F32, 0) / kch;
-	int parts = (int)((1024 + t64 - 1) / t64);
-	if (parts > nkt / 8)
-		parts = nkt / 8;
-	if (parts > 16)
-		parts = 16;
+	const int parts = conv_f32_ksplit(t64, conv_kc(Ci, kH, kW, THHIP_F32, 0) / kch);
 	return parts > 1 ? parts : 0;
 }
 
