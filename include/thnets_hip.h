@@ -496,6 +496,23 @@ void thhip_conv2d_image_pool(const void *x, const void *wpacked, const float *sc
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW, int ppad,
 	int act, float thr, float val, int dtype);
 
+/* Replaces two modules and what is folded into them: the image layer
+ * SpatialConvolutionMM(3 -> 64, 3x3, stride 1, padding 1) (-> batch norm, folded) -> Threshold,
+ * and the 3x3 / stride 1 / padding 1 layer of 64 input planes that follows with its own
+ * (-> SpatialMaxPooling(2, 2, 2, 2) when pool2 is set), for the half types
+ * (modules/SpatialConvolutionMM.c:126-225 twice, modules/Threshold.c:38-63,
+ * modules/SpatialMaxPooling.c:6-98).  One kernel: the first layer's output, 64 planes a
+ * pixel, is computed patch by patch in LDS and never written.  img: [B][3][H][W]
+ * plane-major, W even; wfront: the first layer's [64][3][3][3] weights from
+ * thhip_conv_pack_weight_image_front (6 KiB on the device, thhip_free); wpacked: the second
+ * layer's weights as for thhip_conv2d_layout with channels-last input; y: channels-last,
+ * [B][H][W][Co] or [B][H/2][W/2][Co]; Co at most 256, a multiple of 8. */
+void *thhip_conv_pack_weight_image_front(const float *w, int dtype);
+int thhip_conv2d_image_pair_supported(int B, int H, int W, int Co1, int Co2, int dtype, int y_channels_last);
+void thhip_conv2d_image_pair(const void *img, const void *wfront, const float *scale1, const float *shift1,
+	int act1, float thr1, float val1, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int H, int W, int Co, int act, float thr, float val, int pool2, int dtype);
+
 /* thhip_conv2d_affine followed by a max pooling of any window, stride, padding and
  * rounding (modules/SpatialMaxPooling.c:6-98; the module sequence SpatialConvolutionMM
  * -> Threshold -> SpatialMaxPooling), y = [B][Co][pH][pW] from thhip_pool_outsize of the

@@ -883,6 +883,61 @@ def test_conv_half_whole_image_patch_kernel(hiplib, oracle, dt):
 
 
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
+def test_conv_half_image_layer_in_front(hiplib, oracle, dt):
+    """The network's image layer (3 -> 64 planes, 3x3 / stride 1 / padding 1, factor, shift, Threshold) computed
+    inside the 3x3 layer of 64 input planes that follows it, with and without that layer's 2x2 pooling: against
+    the oracle run on the values the device holds (the first layer's output rounded to the half type, as the
+    separate kernel stores it), and against the two layers run one after the other on the device; images
+    smaller than a tile, partial tiles on both axes, several tiles per workgroup, a Threshold other than ReLU
+    after the first layer, plane counts of the second layer with a partial block."""
+    from thnets_amd import api
+    g = cases.rng(918)
+    shapes = [(2, 8, 32, 64, 1), (3, 19, 46, 72, 1), (1, 5, 6, 64, 0), (40, 16, 64, 128, 1), (2, 37, 70, 136, 0), (1, 224, 224, 64, 1)]
+    for (B, H, W, Co, relu1) in shapes:
+        x = g.uniform(-1, 1, (B, 3, H, W)).astype(np.float32)
+        w1 = g.standard_normal((64, 3, 3, 3), dtype=np.float32) * np.float32(0.3)
+        b1 = g.standard_normal(64, dtype=np.float32) * np.float32(0.1)
+        s1 = (g.uniform(0.5, 1.5, 64) * g.choice([-1.0, 1.0], 64)).astype(np.float32)
+        w2 = g.standard_normal((Co, 64, 3, 3), dtype=np.float32) * np.float32(np.sqrt(2.0 / (64 * 9)))
+        b2 = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+        s2 = g.uniform(0.5, 1.5, Co).astype(np.float32)
+        thr1, val1 = (0.0, 0.0) if relu1 else (0.05, -0.02)
+        rd = lambda a: api.from_device_dtype(api.to_device_dtype(hiplib, a, dt), a.shape, dt)
+        raw1 = oracle.conv2d(rd(x), rd(w1), None, (1, 1), (1, 1)) * s1[None, :, None, None] + b1[None, :, None, None]
+        mid = rd(np.where(raw1 > thr1, raw1, np.float32(val1)).astype(np.float32))
+        raw2 = oracle.conv2d(mid, rd(w2), None, (1, 1), (1, 1)) * s2[None, :, None, None] + b2[None, :, None, None]
+        want = np.maximum(raw2, 0)
+        # the two layers one after the other on the device
+        first = G.conv2d_layout(hiplib, x, w1, b1, (1, 1), (1, 1), act=1, thr=thr1, val=val1, dtype=dt, x_cl=0, y_cl=1, scale=s1)
+        G.assert_close(first, mid, HALF_TOL, "image layer alone " + str((B, H, W)))
+        second = G.conv2d_layout(hiplib, first, w2, b2, (1, 1), (1, 1), act=1, dtype=dt, x_cl=1, y_cl=1, scale=s2)
+        assert hiplib.thhip_conv2d_image_pair_supported(B, H, W, 64, Co, dt, 1)
+        dx = api.to_device_dtype(hiplib, x, dt)
+        wf = hiplib.thhip_conv_pack_weight_image_front(np.ascontiguousarray(w1).ctypes.data, dt)
+        wp = hiplib.thhip_conv_pack_weight_layout(np.ascontiguousarray(w2).ctypes.data, Co, 64, 3, 3, dt, 1)
+        d1b, d1s, d2b, d2s = (api.DeviceArray(hiplib, a) for a in (b1, s1, b2, s2))
+        for pool in (0, 1):
+            if pool and (H < 2 or W < 2):
+                continue
+            G.note("image layer in front %s pool %d dtype %d" % ((B, H, W, Co, relu1), pool, dt))
+            oH, oW = (H // 2, W // 2) if pool else (H, W)
+            dy = api.DeviceArray(hiplib, nbytes=B * Co * oH * oW * 2)
+            hiplib.thhip_conv2d_image_pair(dx.ptr, wf, d1s.ptr, d1b.ptr, 1, thr1, val1, wp, d2s.ptr, d2b.ptr, dy.ptr,
+                                           B, H, W, Co, 1, 0.0, 0.0, pool, dt)
+            hiplib.thhip_sync()
+            got = np.ascontiguousarray(api.from_device_dtype(dy, (B, oH, oW, Co), dt).transpose(0, 3, 1, 2))
+            pooled = lambda a: a[:, :, :2 * oH, :2 * oW].reshape(B, Co, oH, 2, oW, 2).max(axis=(3, 5)) if pool else a
+            G.assert_close(got, pooled(want), HALF_TOL, str((B, H, W, Co, pool)))
+            G.assert_close(got, pooled(second), 1e-2, "vs the two layers one after the other " + str((B, H, W, Co, pool)))
+        hiplib.thhip_free(wf)
+        hiplib.thhip_free(wp)
+    assert not hiplib.thhip_conv2d_image_pair_supported(2, 8, 31, 64, 64, dt, 1)      # odd width
+    assert not hiplib.thhip_conv2d_image_pair_supported(2, 8, 32, 32, 64, dt, 1)      # the image layer makes 64 planes
+    assert not hiplib.thhip_conv2d_image_pair_supported(2, 8, 32, 64, 512, dt, 1)
+    assert not hiplib.thhip_conv2d_image_pair_supported(2, 8, 32, 64, 64, G.F32, 1)
+
+
+@pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_maxpool_and_relayout_half_channels_last(hiplib, oracle, dt):
     from thnets_amd import api
     g = cases.rng(909)

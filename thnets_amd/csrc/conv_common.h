@@ -57,6 +57,13 @@ struct ConvParams {
 	int zero, offA, offB, c_off, c_mult, c_shift, ithr, ival;
 	int kwv;		/* GM_PIXELS4: vectors (four pixels) per kernel row; magic_kw divides by it */
 	unsigned c4_fill;	/* GM_PIXELS4: one pixel outside the image */
+	/* conv_patch_kernel with the network's image layer in front (img != 0): the three-plane image, plane-major,
+	 * that layer's weights as thhip_conv_pack_weight_image_front packs them, its shift, factor and Threshold */
+	const void *img, *wstem;
+	const float *sbias, *sscale;
+	int sact;
+	float sthr, sval;
+	unsigned img_bytes;
 	/* host side only: memory order of x and y, 0 = [B][C][H][W], 1 = [B][H][W][C] */
 	int x_cl, y_cl;
 };

@@ -51,10 +51,22 @@
  * again and store nothing.  With few images such a layer has few workgroups (batch
  * 16, 512 planes: 128 of 64 planes), so BM may be 32 here: then two of the four
  * waves' weight loads repeat the other two's (same bytes to the same place), which
- * keeps every wave's count of outstanding loads the same. */
+ * keeps every wave's count of outstanding loads the same.
+ *
+ * STEM: the layer in front is the network's image layer (3 planes -> 64, 3x3 / stride 1 / padding 1, with its
+ * factor, bias and Threshold), whose output would be written by one kernel only to be read back by this one
+ * (128 bytes a pixel: 411 MB for a batch of 64 at 224 x 224).  Here a workgroup computes the two 32-plane
+ * patches of a tile from the image instead of loading them: the 12 x 36 pixels of the three image planes
+ * under the patch go to LDS (a fourth plane of zeros beside them), a wave takes blocks of 32 patch pixels,
+ * builds its B operand from 24 two-byte reads at constant offsets (lane half h reads planes 2h and 2h + 1, so
+ * that the halves differ by a constant: K = 2 x 18 taps in three chunks, packed that way by
+ * thhip_conv_pack_weight_image_front), multiplies with the 64 x 48 weights kept in LDS, applies factor, bias
+ * and Threshold, writes zeros for pixels outside the image (this layer's padding) and puts the rounded
+ * values where the loads would have put them.  The image pixels of the next tile are requested before the
+ * stores of this one.  Every tile then starts its own weight ring (the patch computation covers its latency). */
 #define PATCH_ROWC 1024	/* output planes (in whole blocks) whose constants the kernel keeps in LDS */
 
-template <int DT, bool CLO, int BM, int CI, bool POOL, bool WHOLE>
+template <int DT, bool CLO, int BM, int CI, bool POOL, bool WHOLE, bool STEM = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void conv_patch_kernel(ConvParams p)
 {
 #if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
@@ -64,7 +76,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	constexpr int TW = WHOLE ? 14 : PATCH_TW, TH = WHOLE ? 14 : PATCH_TH, PW = TW + 2, PH = TH + 2, PCI = 32, NB = CI / PCI;
 	constexpr int NPIX = PW * PH, WAVES = 4;
 	constexpr int BL = ((NPIX + 15) / 16 + WAVES - 1) / WAVES;	/* patch loads (sixteen pixels x four vectors) per wave and block */
-	constexpr int B_VECS = BL * WAVES * 64;				/* a buffer: every load's 1 KiB, the unused ones' too */
+	constexpr int B_VECS = STEM ? 22 * 64 : BL * WAVES * 64;	/* a buffer: every load's 1 KiB, the unused ones' too (STEM: 22 blocks of 16 pixels) */
 	constexpr int MB = BM / 32, TM = MB, TN = 2, KCH = 2, NST = WHOLE ? 9 : 6;	/* NST: weight stages */
 	constexpr int A_VECS = MB * KCH * 64, A_PW = (MB * KCH + WAVES - 1) / WAVES;
 	static_assert(CI % (2 * PCI) == 0 && (MB * KCH % WAVES == 0 || WAVES % (MB * KCH) == 0) && (WHOLE || TH == 2 * WAVES) && BL <= 8, "shape");
@@ -75,12 +87,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	 * 167 -> 156 us); longer K loops lose more to the fixed tile order than they gain (3-7 %) and take one
 	 * tile per workgroup, which the dispatcher hands to the CUs as they come free. */
 	constexpr bool WALK = CI == 64;
-	constexpr int ROWC = WALK ? PATCH_ROWC : BM;	/* planes whose constants sit in LDS */
+	constexpr int ROWC = STEM ? 256 : WALK ? PATCH_ROWC : BM;	/* planes whose constants sit in LDS */
+	static_assert(!STEM || (CI == 64 && !WHOLE && BM == 64), "the image layer in front: 64 planes into 32 x 8 tiles");
+	/* STEM: the image patch (four planes of 12 x 36 halfs), the image layer's weights (2 x 3 fragments of 1 KiB) and constants */
+	constexpr int IMG_ROWS = PH + 2, IMG_W = PW + 2, IMG_PLANE = IMG_ROWS * IMG_W;
+	constexpr int IMG_VECS = (4 * IMG_PLANE * 2 + 15) / 16, WST_VECS = 2 * 3 * 64, SC_VECS = 2 * 64 / 4;
 	/* (one array, every stage and buffer at a constant offset: conv_f32_patch_kernel says why) */
-	__shared__ floatx4 lds[NST * A_VECS + 2 * B_VECS + 2 * ROWC / 4];
+	__shared__ floatx4 lds[NST * A_VECS + 2 * B_VECS + 2 * ROWC / 4 + (STEM ? IMG_VECS + WST_VECS + SC_VECS : 0)];
 	floatx4 *const astage = lds;
 	floatx4 *const patch0 = lds + NST * A_VECS, *const patch1 = patch0 + B_VECS;
 	float *const rowc = (float *)(patch1 + B_VECS);	/* bias[ROWC], factor[ROWC] */
+	unsigned short *const imgl = (unsigned short *)(rowc + 2 * ROWC);	/* (STEM) */
+	floatx4 *const wstl = (floatx4 *)imgl + IMG_VECS;
+	float *const stemc = (float *)(wstl + WST_VECS);
 
 	const int tid = threadIdx.x;
 	const int lane = tid & 63;
@@ -174,7 +193,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
 		for (int i = 0; i < A_PW; i++)
 			__builtin_amdgcn_raw_ptr_buffer_load_lds(wrsrc, WIDE_LDS(astage + st * A_VECS + a_lds_[i]), 16,
-				here || (WALK && nxt.ok) ? lane * 16 : 0x80000000u, (here || !WALK ? a_off_[i] : a_offn_[i]) + kc * 1024u, 0, 0);
+				here || (WALK && !STEM && nxt.ok) ? lane * 16 : 0x80000000u, (here || !WALK ? a_off_[i] : a_offn_[i]) + kc * 1024u, 0, 0);
 	};
 	auto issue_b = [&](auto t_, int hb, auto buf_) {
 		constexpr int buf = decltype(buf_)::value, t = decltype(t_)::value;
@@ -253,7 +272,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	typedef std::integral_constant<int, 1> C1;
 	/* patch loads of the next block: one in each of the first BL steps of this one (step `tap` issues
 	 * numbers [PB(tap), PB(tap + 1))) */
-#define CONV_PATCH_PB(tap) ((tap) < BL ? (tap) : BL)
+#define CONV_PATCH_PB(tap) (STEM ? 0 : (tap) < BL ? (tap) : BL)
 #define CONV_PATCH_NB(tap) (CONV_PATCH_PB(((tap) + 9) % 9 + 1) - CONV_PATCH_PB(((tap) + 9) % 9))
 	/* The pipeline.  A wave with the SIMD to itself gets what it asks of LDS before a group of MFMAs only
 	 * after them, so the fragments of a K-tile are fetched a whole step ahead, into four register sets.
@@ -270,13 +289,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 		int n = 0;
 		for (int t = tap + 3 - NST; t <= tap - 1; t++)
 			n += A_PW + CONV_PATCH_NB(t + 18);
-		if (tap == 8) {
+		if (tap == 8 && !STEM) {
 			const int np = (8 - (BL - 1)) * A_PW;
 			n = n < np ? n : np;
 		}
 		return n;
 	};
-	{
+	/* what steps -9 .. -1 would have issued: the first patch, the weights of K-tiles 0 .. NST - 2 */
+	auto ring_start = [&]() {
 		auto virt = [&](auto self, auto v_) {
 			constexpr int v = decltype(v_)::value;	/* step v - 9, tap v */
 			if constexpr (v < 9) {
@@ -288,20 +308,160 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 			}
 		};
 		virt(virt, C0{});
-	}
+	};
+	/* ... and once the patch (its last load: step BL - 10) and K-tile 0 (step 1 - NST) are there (what the steps
+	 * after both issued may be outstanding), the first fragments */
+	auto ring_first = [&]() {
+		wide_wait<(!STEM && BL - 10 > 1 - NST ? 10 - BL : NST - 2) * A_PW, true>();
+		__builtin_amdgcn_s_barrier();
+		read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
+		read_frags(C0{}, C0{}, C0{}, 1, af[1], bf[1]);
+	};
 	/* the per-plane constants of every plane block, or of this tile's if it is the only one (behind the
 	 * first loads: they are waited for anyway) */
-	const int row0 = WALK ? 0 : cur.tile_m * BM;
-	for (int i = tid; i < (WALK ? p.tiles_m * BM : BM); i += 256) {
-		const int mc = min(row0 + i, p.Co - 1);
-		rowc[i] = p.bias ? p.bias[mc] : 0.0f;
-		rowc[ROWC + i] = p.scale ? p.scale[mc] : 1.0f;
+	auto fill_rowc = [&]() {
+		const int row0 = WALK ? 0 : cur.tile_m * BM;
+		for (int i = tid; i < (WALK ? p.tiles_m * BM : BM); i += 256) {
+			const int mc = min(row0 + i, p.Co - 1);
+			rowc[i] = p.bias ? p.bias[mc] : 0.0f;
+			rowc[ROWC + i] = p.scale ? p.scale[mc] : 1.0f;
+		}
+	};
+
+	/* ---- STEM: the image pixels a tile's patch is computed from, three dwords a thread ---- */
+	const __amdgpu_buffer_rsrc_t irsrc = __builtin_amdgcn_make_buffer_rsrc((void *)(STEM ? p.img : p.x), 0, STEM ? p.img_bytes : 0, 0x00020000);
+	unsigned imgv[3];
+	auto image_request = [&](const Tile &T) {
+#pragma unroll
+		for (int u = 0; u < 3; u++) {
+			const int idx = tid + 256 * u, c = idx / (IMG_ROWS * (IMG_W / 2)), r = (idx / (IMG_W / 2)) % IMG_ROWS, d = idx % (IMG_W / 2);
+			const int iy = T.ty * TH - p.padH - 1 + r, ix = T.tx * TW - p.padW - 1 + 2 * d;
+			const bool ok = c < 3 && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+			imgv[u] = __builtin_amdgcn_raw_buffer_load_b32(irsrc, ok ? (((T.img * 3 + c) * p.H + iy) * p.W + ix) * 2 : (int)0x80000000, 0, 0);
+		}
+	};
+	/* A tile's start with the image layer in front: image pixels to LDS, the weight ring started, the two
+	 * patches computed, the first fragments read. */
+	auto stem_tile = [&](const Tile &T) {
+#pragma unroll
+		for (int u = 0; u < 3; u++) {
+			const int idx = tid + 256 * u;
+			if (idx < 3 * IMG_ROWS * (IMG_W / 2))
+				((unsigned *)imgl)[idx] = imgv[u];
+		}
+		wide_wait<48, true>();	/* (the LDS writes; every wave is past its last tile's reads of stages and patches) */
+		__builtin_amdgcn_s_barrier();
+		ring_start();
+		/* Three blocks of 32 patch pixels a wave (the last wave: two).  Everything the blocks read from LDS is
+		 * requested before the first MFMA -- the other workgroup of the CU keeps LDS busy with its K loop, and
+		 * a wave that asks for a block's operands, waits, multiplies, asks for the constants, waits, ... spent
+		 * 12 000 cycles here where its instructions need 2 000. */
+		const int n = lane & 31, h = lane >> 5;
+		constexpr int NBW = ((NPIX + 31) / 32 + WAVES - 1) / WAVES;
+		uintx4 bw[NBW][3];
+		int pp_[NBW];
+		bool inside_[NBW];
+#pragma unroll
+		for (int t = 0; t < NBW; t++) {
+			const int pp = (wave + WAVES * t) * 32 + n, ppc = min(pp, NPIX - 1);
+			const int pr = ppc / PW, pc = ppc - pr * PW;
+			const unsigned short *src = imgl + pr * IMG_W + pc + h * (2 * IMG_PLANE);
+#pragma unroll
+			for (int sc = 0; sc < 3; sc++)
+#pragma unroll
+				for (int d = 0; d < 4; d++) {
+					unsigned two[2];
+#pragma unroll
+					for (int e = 0; e < 2; e++) {
+						const int j = 8 * sc + 2 * d + e;	/* tap j of this lane half's two planes: (plane, kh, kw) = (j / 9, j % 9 / 3, j % 3) */
+						two[e] = src[j < 18 ? ((j / 9) * IMG_ROWS + (j % 9) / 3) * IMG_W + j % 3 : 0];
+					}
+					bw[t][sc][d] = two[0] | (two[1] << 16);
+				}
+			const int iy = T.ty * TH - p.padH + pr, ix = T.tx * TW - p.padW + pc;
+			pp_[t] = pp;
+			inside_[t] = pp < NPIX && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+		}
+		const bool relu = p.sact && p.sthr == 0.0f && p.sval == 0.0f;
+#pragma unroll
+		for (int mb = 0; mb < 2; mb++) {
+			floatx4 wa[3], rb[4], rs[4];
+#pragma unroll
+			for (int sc = 0; sc < 3; sc++)
+				wa[sc] = wstl[(mb * 3 + sc) * 64 + lane];
+#pragma unroll
+			for (int g = 0; g < 4; g++) {
+				const int ml = mb * 32 + 8 * g + 4 * h;
+				rb[g] = *(const floatx4 *)(stemc + ml);
+				rs[g] = *(const floatx4 *)(stemc + 64 + ml);
+			}
+			floatx16 sacc[NBW];
+#pragma unroll
+			for (int t = 0; t < NBW; t++)
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					sacc[t][r] = 0.0f;
+#pragma unroll
+			for (int sc = 0; sc < 3; sc++)
+#pragma unroll
+				for (int t = 0; t < NBW; t++)
+					conv_mma<DT>(sacc[t], wa[sc], __builtin_bit_cast(floatx4, bw[t][sc]));
+			/* register 4 g + e of block mb is plane 32 mb + 8 g + 4 h + e of pixel pp: half of vector g */
+#pragma unroll
+			for (int t = 0; t < NBW; t++) {
+				if (wave + WAVES * t >= (NPIX + 31) / 32)
+					continue;	/* (the last wave's third block does not exist) */
+				const int pp = pp_[t];
+				const bool inside = inside_[t];
+#pragma unroll
+				for (int g = 0; g < 4; g++) {
+					char *const dst = (char *)(mb ? patch1 : patch0) + (4 * pp + (g ^ ((pp >> 2) & 3))) * 16 + 8 * h;
+					if (relu) {
+						/* on packed pairs: a ReLU of rounded values is an integer maximum with zero */
+						typedef short shortx2 __attribute__((ext_vector_type(2)));
+						typedef elem elemx2 __attribute__((ext_vector_type(2)));
+						uintx2 out;
+#pragma unroll
+						for (int e2 = 0; e2 < 2; e2++) {
+							const elemx2 v = { (elem)__builtin_fmaf(sacc[t][4 * g + 2 * e2], rs[g][2 * e2], rb[g][2 * e2]),
+								(elem)__builtin_fmaf(sacc[t][4 * g + 2 * e2 + 1], rs[g][2 * e2 + 1], rb[g][2 * e2 + 1]) };
+							const shortx2 zero = { 0, 0 };
+							const unsigned u = __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(shortx2, v), zero));
+							out[e2] = inside ? u : 0u;
+						}
+						*(uintx2 *)dst = out;
+					} else {
+						struct alignas(8) Quad { elem v[4]; } quad;
+#pragma unroll
+						for (int e = 0; e < 4; e++) {
+							float v = __builtin_fmaf(sacc[t][4 * g + e], rs[g][e], rb[g][e]);
+							if (p.sact)
+								v = v > p.sthr ? v : p.sval;
+							quad.v[e] = inside ? (elem)v : (elem)0.0f;
+						}
+						*(Quad *)dst = quad;
+					}
+				}
+			}
+		}
+		ring_first();
+	};
+	if constexpr (STEM) {
+		for (int i = tid; i < WST_VECS; i += 256)
+			wstl[i] = ((const floatx4 *)p.wstem)[i];
+		if (tid < 64) {
+			stemc[tid] = p.sbias ? p.sbias[tid] : 0.0f;
+			stemc[64 + tid] = p.sscale ? p.sscale[tid] : 1.0f;
+		}
+		for (int i = tid; i < IMG_PLANE / 2; i += 256)
+			((unsigned *)imgl)[3 * IMG_PLANE / 2 + i] = 0;	/* the fourth plane */
+		image_request(cur);
+		fill_rowc();
+	} else {
+		ring_start();
+		fill_rowc();
+		ring_first();
 	}
-	/* the patch (its last load: step BL - 10) and K-tile 0 (step 1 - NST): what the steps after both issued may be outstanding */
-	wide_wait<(BL - 10 > 1 - NST ? 10 - BL : NST - 2) * A_PW, true>();
-	__builtin_amdgcn_s_barrier();
-	read_frags(C0{}, C0{}, C0{}, 0, af[0], bf[0]);
-	read_frags(C0{}, C0{}, C0{}, 1, af[1], bf[1]);
 	auto step = [&](int hb, auto buf_, auto tap_) {
 		constexpr int tap = decltype(tap_)::value, buf = decltype(buf_)::value;
 		constexpr int par = (tap + buf) & 1;
@@ -545,10 +705,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 	};
 
 	for (;;) {
+		if constexpr (STEM)
+			stem_tile(cur);
 		for (int hb = 0; hb < NB; hb += 2) {
 			block(hb, C0{});
 			block(hb + 1, C1{});
 		}
+		if constexpr (STEM)
+			if (nxt.ok)
+				image_request(nxt);
 		store_tile(cur);
 		if (!WALK || !nxt.ok)
 			break;
@@ -671,6 +836,17 @@ static void conv_launch_patch(ConvParams &p)
 		else                                                                       \
 			patch_go<conv_patch_kernel<DT, CLO, BM, CI, false, WHOLE>>(p, per_xcd, walk); \
 	} while (0)
+	if constexpr (!WHOLE && BM == 64) {
+		if (p.img) {	/* the image layer in front */
+			if (p.Ci != 64 || !p.y_cl || p.tiles_m * BM > 256 || p.W % 2 || p.padH != 1 || p.padW != 1 || !p.wstem)
+				THError("thhip_conv2d: the image layer goes in front of a 3x3 / padding 1 layer of 64 input and at most 256 output planes, channels-last, on images of even width");
+			if (p.pool)
+				patch_go<conv_patch_kernel<DT, true, BM, 64, true, false, true>>(p, per_xcd, true);
+			else
+				patch_go<conv_patch_kernel<DT, true, BM, 64, false, false, true>>(p, per_xcd, true);
+			return;
+		}
+	}
 	if constexpr (!WHOLE) {
 		if (p.Ci == 64 && p.y_cl)
 			CONV_PATCH_GO(true, 64);

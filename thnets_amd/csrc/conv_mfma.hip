@@ -3429,10 +3429,18 @@ struct ConvResidual {
 	float c;
 };
 
+/* the network's image layer (3 planes -> 64, 3x3 / stride 1 / padding 1) in front of the convolution */
+struct ConvImageFront {
+	const void *img, *wfront;
+	const float *scale, *shift;
+	int act;
+	float thr, val;
+};
+
 static void conv_run(const void *x, const void *wpacked, const float *scale, const float *bias, void *y,
 	int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW, int padH, int padW,
 	int act, float thr, float val, int dtype, const ConvU8Args *u8, int f_x_layout = 0, int f_y_cl = 0, int f_pool2 = 0,
-	const ConvResidual *f_res = 0, const ConvPoolK *f_pk = 0)
+	const ConvResidual *f_res = 0, const ConvPoolK *f_pk = 0, const ConvImageFront *f_front = 0)
 {
 	if (B < 1 || Ci < 1 || Co < 1 || kH < 1 || kW < 1 || dH < 1 || dW < 1 || padH < 0 || padW < 0)
 		THError("thhip_conv2d: bad geometry");
@@ -3544,6 +3552,24 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 				p.res_mode = f_res->mode;
 				p.res_c = f_res->c;
 				p.res_act = f_res->act;
+			}
+			if (f_front) {
+				/* (x is not read: the kernel computes its input patches from the image) */
+				if (bn != B)
+					THError("thhip_conv2d_image_pair: the batch must fit one slice");
+				p.x = 0;
+				p.x_bytes = 0;
+				p.img = f_front->img;
+				p.img_bytes = (unsigned)((size_t)bn * 3 * H * W * esize);
+				p.wstem = f_front->wfront;
+				p.sscale = f_front->scale;
+				p.sbias = f_front->shift;
+				p.sact = f_front->act;
+				p.sthr = f_front->thr;
+				p.sval = f_front->val;
+				ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N + 2.0 * 64 * 27 * p.N);
+				thhip_conv_half_patch_launch(p, dtype, 64, 0);
+				continue;
 			}
 			ThhipLaunchScope scope(THHIP_FAM_CONV, 2.0 * Co * (double)K * p.N);
 			/* a 3x3 image layer: whole rows from a patch in LDS (conv_stem.hip), unless a test forces a tile */
@@ -3659,6 +3685,59 @@ extern "C" void thhip_conv2d_image_pool(const void *x, const void *wpacked, cons
 
 /* Whether thhip_conv2d_residual takes this layer: fp32, plane-major tensors, planes in blocks of 32 (the
  * kernel that loads its tiles straight into LDS), the batch in one slice. */
+/* The image layer's weights [64][3][3][3] in the order the kernel of thhip_conv2d_image_pair multiplies them:
+ * [32-row block][chunk of 16][lane half h][row][8 values], value e of chunk s being tap j = 8 s + e of the
+ * eighteen of planes 2 h and 2 h + 1 (plane j / 9, kernel row j % 9 / 3, column j % 3; zero beyond and for the
+ * fourth plane).  A device buffer of 6 KiB (thhip_free). */
+extern "C" void *thhip_conv_pack_weight_image_front(const float *w, int dtype)
+{
+	if (dtype != THHIP_F16 && dtype != THHIP_BF16)
+		THError("thhip_conv_pack_weight_image_front: a half dtype");
+	std::vector<unsigned short> host(2 * 3 * 64 * 8, 0);
+	for (int mb = 0; mb < 2; mb++)
+		for (int s = 0; s < 3; s++)
+			for (int lane = 0; lane < 64; lane++)
+				for (int e = 0; e < 8; e++) {
+					const int m = mb * 32 + (lane & 31), h = lane >> 5, j = 8 * s + e, c = 2 * h + j / 9;
+					float v = 0.0f;
+					if (j < 18 && c < 3)
+						v = w[(m * 3 + c) * 9 + j % 9];
+					host[(((size_t)mb * 3 + s) * 64 + lane) * 8 + e] = dtype == THHIP_F16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v);
+				}
+	void *d = thhip_malloc(host.size() * 2);
+	thhip_memcpy_h2d(d, host.data(), host.size() * 2);
+	return d;
+}
+
+/* Whether thhip_conv2d_image_pair takes the two layers: half type; the first 3 -> 64 planes, the second 64 ->
+ * at most 256 planes, both 3x3 / stride 1 / padding 1; channels-last output; an even image width. */
+extern "C" int thhip_conv2d_image_pair_supported(int B, int H, int W, int Co1, int Co2, int dtype, int y_channels_last)
+{
+	if (dtype != THHIP_F16 && dtype != THHIP_BF16)
+		return 0;
+	if (Co1 != 64 || Co2 < 1 || Co2 > 256 || Co2 % 8 || !y_channels_last || W % 2 || H < 1 || W < 2 || B < 1)
+		return 0;
+	if ((double)B * 64 * H * W * 2 >= 2147483000.0 || (double)B * Co2 * H * W * 2 >= 2147483000.0)
+		return 0;
+	return !g_force_generic_cl && !g_force_bm && !g_force_bn;
+}
+
+/* Two modules' worth in one kernel: the image layer SpatialConvolutionMM(3 -> 64, 3x3, 1, 1) with its factor /
+ * shift and Threshold, and the 3x3 layer that follows it with its own (and optionally the 2x2 max pooling after
+ * that): the first layer's output (64 planes a pixel) is computed patch by patch in LDS and never written
+ * (modules/SpatialConvolutionMM.c:126-225 twice, Threshold.c:38-63, SpatialMaxPooling.c:6-98).  img: [B][3][H][W]
+ * plane-major; wfront from thhip_conv_pack_weight_image_front; wpacked as for thhip_conv2d_layout with
+ * channels-last input; y channels-last. */
+extern "C" void thhip_conv2d_image_pair(const void *img, const void *wfront, const float *scale1, const float *shift1,
+	int act1, float thr1, float val1, const void *wpacked, const float *scale, const float *shift, void *y,
+	int B, int H, int W, int Co, int act, float thr, float val, int pool2, int dtype)
+{
+	if (!thhip_conv2d_image_pair_supported(B, H, W, 64, Co, dtype, 1))
+		THError("thhip_conv2d_image_pair: layers not supported (see thhip_conv2d_image_pair_supported)");
+	const ConvImageFront f = { img, wfront, scale1, shift1, act1, thr1, val1 };
+	conv_run(img, wpacked, scale, shift, y, B, 64, H, W, Co, 3, 3, 1, 1, 1, 1, act, thr, val, dtype, 0, 1, 1, pool2 != 0, 0, 0, &f);
+}
+
 extern "C" int thhip_conv2d_residual_supported(int B, int Ci, int H, int W, int Co, int kH, int kW, int dH, int dW,
 	int padH, int padW, int dtype)
 {

@@ -186,6 +186,7 @@ long THHipNetwork_copyModuleOutput(THNETWORK *net, int idx, float **dst, long si
 	THFloatTensor *o = net->net->modules[idx].output;
 	if (net->net->modules[idx].type == MT_ConcatTable || !o || !o->storage)
 		THError("THHipNetwork_copyModuleOutput: module %d has no tensor output", idx);
+	thhip_materialize_output(net->net, idx);	/* (a module that left its work to its consumer) */
 	thhip_sync();
 	THFloatTensor *h;
 	const int nd = o->nDimension;

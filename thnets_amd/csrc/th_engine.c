@@ -209,6 +209,35 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 	 * would run this layer can do it */
 	const struct SpatialMaxPooling *pq = hm->pool_next ? &hn->pub.modules[hm->pool_next].SpatialMaxPooling : 0;
 	const int pool22 = pq && pq->kW == 2 && pq->kH == 2 && pq->dW == 2 && pq->dH == 2 && pq->padW == 0 && pq->padH == 0 && !pq->ceil_mode;
+	/* the image layer of a half network: left to the convolution after it, which computes this layer's
+	 * output patch by patch in LDS; nothing is written here (the output tensor keeps its shape and memory, and
+	 * is filled on demand: thhip_materialize_output).  Not while th_minmax wants every tensor's range. */
+	hm->deferred = 0;
+	if (hm->front_of && !th_minmax && s.outnd == 4 &&
+	    thhip_conv2d_image_pair_supported(s.B, s.H, s.W, c->nOutputPlane,
+			hn->pub.modules[hm->front_of].SpatialConvolution.nOutputPlane, dt, 1)) {
+		conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
+		hn->cur_cl = hm->out_cl;
+		hm->deferred = 1;
+		hm->front_img = x;
+		hm->front_B = s.B; hm->front_H = s.H; hm->front_W = s.W;
+		return m->output;
+	}
+	if (hm->front && hn->hm[hm->front - 1].deferred) {
+		struct hipmod *fm = &hn->hm[hm->front - 1];
+		const int pool = pool22 && oH >= 2 && oW >= 2;
+		if (fm->front_B == s.B && fm->front_H == s.H && fm->front_W == s.W) {
+			void *yp = conv_out(m, dt, &s, c->nOutputPlane, pool ? oH / 2 : oH, pool ? oW / 2 : oW);
+			hn->cur_cl = hm->out_cl && (pool ? (oH / 2) * (oW / 2) : oH * oW) > 1;
+			thhip_conv2d_image_pair(fm->front_img, fm->wfront, fm->scale, fm->bias, fm->fused_act, fm->thr, fm->val,
+				hm->wpacked, hm->scale, hm->bias, yp, s.B, s.H, s.W, c->nOutputPlane, hm->fused_act, hm->thr, hm->val,
+				pool, dt);
+			if (pool)
+				hn->hm[hm->pool_next].pooled_by_producer = 1;
+			return m->output;
+		}
+		thhip_materialize_output(&hn->pub, hm->front - 1);	/* (another shape than the image layer saw: never in a list of modules) */
+	}
 	if (pool22 && thhip_conv2d_pool2_supported(s.B, c->nInputPlane, s.H, s.W, c->nOutputPlane, c->kH, c->kW,
 			c->dH, c->dW, c->padH, c->padW, dt, hm->x_layout, hm->out_cl)) {
 		void *yp = conv_out(m, dt, &s, c->nOutputPlane, oH / 2, oW / 2);
@@ -868,6 +897,22 @@ static int is_conv_type(int type)
 	return type == MT_SpatialConvolutionMM || type == MT_SpatialConvolutionVirtMM || type == MT_SpatialConvolution;
 }
 
+/* The output of a module that left its work to its consumer in the last forward (the image layer of a half
+ * network, above), computed now by the module's own kernel: for callers that read module outputs. */
+void thhip_materialize_output(struct network *net, int idx)
+{
+	struct hipnet *hn = (struct hipnet *)net;
+	struct hipmod *hm = &hn->hm[idx];
+	if (!hm->deferred)
+		return;
+	struct module *m = &net->modules[idx];
+	struct SpatialConvolution *c = &m->SpatialConvolution;
+	thhip_conv2d_layout(hm->front_img, hm->wpacked, hm->scale, hm->bias, thhip_tensor_ptr(m->output, hn->dtype), hm->front_B,
+		c->nInputPlane, hm->front_H, hm->front_W, c->nOutputPlane, c->kH, c->kW, c->dH, c->dW, c->padH, c->padW,
+		hm->fused_act, hm->thr, hm->val, hn->dtype, hm->x_layout, hm->out_cl);
+	hm->deferred = 0;
+}
+
 /* forward(), thapi.c:158-235, without the per-layer frees; with th_profile
  * the stream is drained around each module the way the OpenCL engine calls
  * clFinish (thapi.c:213-216), so the printed seconds are kernel time. */
@@ -1427,6 +1472,31 @@ static struct network *to_hip(struct network *net, int engine, int dtype, float 
 		else if (dtype == THHIP_F32)	/* any window: by the kernel that adds the parts of a K split (layers of a few tiles) */
 			hn->hm[i].pool_next = j;
 	}
+	/* half engines, a list of modules: the image layer (3 -> 64 planes, 3x3 / stride 1 / padding 1, plane-major
+	 * in, channels-last out) followed, through its folded Threshold, by a 3x3 / stride 1 / padding 1 layer of at
+	 * most 256 planes between channels-last tensors: that layer may compute the image layer's output itself */
+	for (int i = 0; i + 1 < net->nelem && engine == ENGINE_HIP && dtype != THHIP_F32 && !dag; i++) {
+		if (!is_conv_type(hn->pub.modules[i].type) || hn->hm[i].is_linear || hn->hm[i].in_cl || !hn->hm[i].out_cl || hn->hm[i].pool_next)
+			continue;
+		const struct SpatialConvolution *a = &hn->pub.modules[i].SpatialConvolution;
+		if (a->nInputPlane != 3 || a->nOutputPlane != 64 || a->kW != 3 || a->kH != 3 || a->dW != 1 || a->dH != 1 || a->padW != 1 || a->padH != 1)
+			continue;
+		int j = i + 1;
+		while (j < net->nelem && hn->hm[j].passthrough)
+			j++;
+		if (j >= net->nelem || !is_conv_type(hn->pub.modules[j].type) || hn->hm[j].is_linear || !hn->hm[j].in_cl || !hn->hm[j].out_cl)
+			continue;
+		const struct SpatialConvolution *b = &hn->pub.modules[j].SpatialConvolution;
+		if (b->nInputPlane != 64 || b->nOutputPlane > 256 || b->nOutputPlane % 8 || b->kW != 3 || b->kH != 3 || b->dW != 1 || b->dH != 1 ||
+		    b->padW != 1 || b->padH != 1)
+			continue;
+		const THFloatTensor *w = net->modules[i].SpatialConvolution.weight;
+		if (!w || !w->storage || THFloatTensor_nElement((THFloatTensor *)w) != 64 * 27)
+			continue;
+		hn->hm[i].wfront = thhip_conv_pack_weight_image_front(w->storage->data + w->storageOffset, dtype);
+		hn->hm[i].front_of = j;
+		hn->hm[j].front = i + 1;
+	}
 #undef FEEDS_ONLY
 	free(consumers);
 	/* uint8 engine: the image layer (at most four planes, plane-major), or a convolution between
@@ -1494,6 +1564,7 @@ void thhip_free_network(struct network *net)
 		THFloatTensor_free(m->output);
 		thhip_free(hm->wpacked);
 		thhip_free(hm->wrow);
+		thhip_free(hm->wfront);
 		thhip_free(hm->bias);
 		thhip_free(hm->scale);
 		thhip_free(hm->addend);

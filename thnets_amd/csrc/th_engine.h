@@ -51,6 +51,14 @@ struct hipmod {
 	size_t pool_ind_cap;
 	int want_indices;	/* a SpatialMaxUnpooling of this network reads this pooling's indices */
 	int pool_index;		/* SpatialMaxUnpooling: position of its pooling in the network */
+	/* half engines: the network's image layer (3 -> 64 planes, 3x3 / stride 1 / padding 1) may be computed by the
+	 * 3x3 layer that follows it, patch by patch in LDS, and then writes nothing (thhip_conv2d_image_pair) */
+	int front_of;		/* image layer: position of that following convolution (0: none) */
+	int front;		/* that convolution: position of the image layer + 1 (0: none) */
+	void *wfront;		/* image layer: its weights packed for that kernel (device) */
+	int deferred;		/* image layer: in this forward its output was left to the convolution after it (not written) */
+	const void *front_img;	/* image layer: its input of this forward, [B][3][H][W] */
+	int front_B, front_H, front_W;
 	int in_cl, out_cl;	/* input / output codes are channels-last [B][H][W][C] in memory */
 	int x_layout;		/* how the convolution reads its input: thhip_conv_pack_weight_u8_layout */
 	float wm, wsub;		/* weight quantisation */
@@ -89,6 +97,7 @@ int thhip_engine_dtype(void);
 struct network *THHip_ToHip(struct network *net, int lowp, float range);
 THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in);
 void thhip_free_network(struct network *net);
+void thhip_materialize_output(struct network *net, int idx);
 /* th_io.c */
 void thhip_storage_release(THFloatStorage *s);
 THFloatTensor *thhip_device_tensor_like(THFloatTensor *t, int dtype);
