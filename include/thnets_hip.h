@@ -335,6 +335,13 @@ int THHipHalfFloat(int enable);
  * nn_SpatialBatchNormalization_updateOutput.  Applies to engines created
  * afterwards; returns the previous setting. */
 int THHipFoldBatchNorm(int enable);
+/* Half engines: whether the image layer (3 -> 64 planes, 3x3 / stride 1 / padding 1) is computed by the
+ * 3x3 layer after it instead of by a kernel of its own (thhip_conv2d_image_pair; nothing in the reference:
+ * its engines run module by module, cudnn/cudnn_basic.c:189-303).  0: never; 2: always; 1 (default): for
+ * batches of up to 2048 of that layer's 32 x 8 tiles, where one launch beats two.  The results are the same
+ * within the last bit of a half value (another order of the 27 products' sum).  Read at every forward;
+ * returns the previous setting. */
+int THHipImageLayerInFront(int mode);
 /* 0 (default): CAddTable / CSubTable compute what the reference's shipped modules
  * compute (modules/CAddTable.c:59-84: with two inputs CAddTable gives a - b and
  * CSubTable a + b; with more, 2a + b + c + ... and 0 - b - c - ...).  1: what the

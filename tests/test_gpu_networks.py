@@ -173,6 +173,52 @@ def test_half_engine_small_vgg(hiplib, oracle, half):
         n2.free()
 
 
+@pytest.mark.parametrize("half", [1, 2])
+def test_half_engine_image_layer_in_front(hiplib, oracle, half):
+    """A half network whose image layer (3 -> 64, 3x3 / stride 1 / padding 1, ReLU) is followed by a 3x3 layer of
+    64 planes: with THHipImageLayerInFront(2) the second layer computes the first one's output itself (one
+    launch, nothing written), with 0 both run their own kernels, with 1 (the default) the batch decides.  Every
+    module output against the oracle in each mode -- the image layer's is then filled on demand -- the modes
+    against each other, and a second forward of another batch through the same network."""
+    from thnets_amd.netbuild import conv, relu, maxpool
+    g = cases.rng(1300)
+    def wgt(*shape):
+        return g.standard_normal(shape, dtype=np.float32) * np.float32(np.sqrt(2.0 / np.prod(shape[1:])))
+    layers = [conv(wgt(64, 3, 3, 3), wgt(64) * np.float32(0.1), 1, 1), relu(),
+              conv(wgt(72, 64, 3, 3), wgt(72) * np.float32(0.1), 1, 1), relu(), maxpool(2, 2),
+              conv(wgt(32, 72, 3, 3), wgt(32) * np.float32(0.1), 1, 1), relu()]
+    mean, std = (0.485, 0.456, 0.406), (0.229, 0.224, 0.225)
+    tol = 2e-2 if half == 1 else 6e-2
+    old = hiplib.THHipImageLayerInFront(1)
+    try:
+        for mode in (0, 2, 1):
+            hiplib.THHipImageLayerInFront(mode)
+            net = api.HipNetwork(layers, mean, std, half=half)
+            for (B, H, W) in ((3, 40, 66), (5, 17, 32)):
+                x = g.uniform(0, 1, (B, 3, H, W)).astype(np.float32)
+                cfg = {"layers": layers, "mean": mean, "std": std, "input": x}
+                net.process_float(x.copy())
+                layerwise(net, oracle, cfg, tol)
+            net.free()
+    finally:
+        hiplib.THHipImageLayerInFront(old)
+    # the two forms on one input
+    g2 = cases.rng(1301)
+    x = g2.uniform(0, 1, (4, 3, 24, 64)).astype(np.float32)
+    ys = []
+    try:
+        for mode in (0, 2):
+            hiplib.THHipImageLayerInFront(mode)
+            net = api.HipNetwork(layers, mean, std, half=half)
+            ys.append((net.process_float(x.copy()), net.module_output(0), net.module_output(2)))
+            net.free()
+    finally:
+        hiplib.THHipImageLayerInFront(old)
+    assert np.array_equal(ys[0][1], ys[1][1])          # the image layer's own kernel either way
+    G.assert_close(ys[1][2], ys[0][2], 1e-2, "second layer, image layer in front against behind")
+    G.assert_close(ys[1][0], ys[0][0], 2e-2, "network output, image layer in front against behind")
+
+
 def test_process_images_matches_process_float(hiplib, oracle):
     cfg = cases.small_networks()["tiny_cnn"]
     g = cases.rng(1200)

@@ -66,6 +66,7 @@ PROTOTYPES = {
     "THCreateHipNetwork": (vp, [vp]),
     "THHipHalfFloat": (C.c_int, [C.c_int]),
     "THHipFoldBatchNorm": (C.c_int, [C.c_int]),
+    "THHipImageLayerInFront": (C.c_int, [C.c_int]),
     "THHipTableArithmetic": (C.c_int, [C.c_int]),
     "THCreateHipLowpNetwork": (vp, [vp, C.c_float]),
     "THHipTensor_newFromFloatTensor": (vp, [vp]),

@@ -40,6 +40,15 @@ static int g_fold_bn = 1;
  * is folded into that convolution's epilogue when the engine is created;
  * 0: it runs as its own kernel, as in the reference's CPU path.  Returns the
  * previous setting. */
+int THHipImageLayerInFront(int mode)
+{
+	extern int thhip_image_layer_in_front;
+	const int old = thhip_image_layer_in_front;
+	if (mode >= 0 && mode <= 2)
+		thhip_image_layer_in_front = mode;
+	return old;
+}
+
 int THHipFoldBatchNorm(int enable)
 {
 	const int old = g_fold_bn;
@@ -152,6 +161,13 @@ static void out_alias(struct module *m, THFloatTensor *in)
 /* fp32 / fp16 / bf16 modules                                          */
 /* ------------------------------------------------------------------ */
 
+/* Whether the image layer of a half network is left to the convolution after it (Hip_SpatialConvolution_updateOutput):
+ * 0 never, 2 always, 1 (default) for batches of up to 2048 of that convolution's 32 x 8 tiles -- measured on
+ * VGG-16 fp16 at 224 x 224, one kernel against two: batch 1 -1.6 %, 2 -4 %, 4 -3.3 %, 8 -1 % of the forward,
+ * batch 16 and 64 +0.8 % (there the patch computation of a tile costs more than the image layer's own kernel,
+ * which runs at the rate its stores allow). */
+int thhip_image_layer_in_front = 1;	/* (THHipImageLayerInFront) */
+
 struct convshape { int B, H, W, outnd; };
 
 /* Input shapes a convolution accepts: 3-D (one image) and 4-D as
@@ -214,6 +230,9 @@ static THFloatTensor *Hip_SpatialConvolution_updateOutput(struct module *m, THFl
 	 * is filled on demand: thhip_materialize_output).  Not while th_minmax wants every tensor's range. */
 	hm->deferred = 0;
 	if (hm->front_of && !th_minmax && s.outnd == 4 &&
+	    (thhip_image_layer_in_front == 2 ||
+	     (thhip_image_layer_in_front == 1 && (long)s.B * ((oH + 7) / 8) * ((oW + 31) / 32) *
+			((hn->pub.modules[hm->front_of].SpatialConvolution.nOutputPlane + 63) / 64) <= 2048)) &&
 	    thhip_conv2d_image_pair_supported(s.B, s.H, s.W, c->nOutputPlane,
 			hn->pub.modules[hm->front_of].SpatialConvolution.nOutputPlane, dt, 1)) {
 		conv_out(m, dt, &s, c->nOutputPlane, oH, oW);
