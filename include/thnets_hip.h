@@ -520,6 +520,15 @@ void thhip_conv2d_image_pair(const void *img, const void *wfront, const float *s
 	int act1, float thr1, float val1, const void *wpacked, const float *scale, const float *shift, void *y,
 	int B, int H, int W, int Co, int act, float thr, float val, int pool2, int dtype);
 
+/* Two convolutions that do not depend on each other as one launch (nothing in the reference, whose
+ * modules run one after the other, thapi.c:158-235: the shortcut's 1x1 projection of a residual block
+ * beside the block's first convolution, modules/ConcatTable.c).  The convolution call right after _begin
+ * is held back if its kernel can run it whole (fp32, no K split, no cut tiles) and goes out in one grid
+ * with the next call if that runs on the same kernel; otherwise right after that call, or at _end.  The
+ * caller guarantees that neither of the two layers reads the other's output. */
+void thhip_conv_pair_begin(void);
+void thhip_conv_pair_end(void);
+
 /* thhip_conv2d_affine followed by a max pooling of any window, stride, padding and
  * rounding (modules/SpatialMaxPooling.c:6-98; the module sequence SpatialConvolutionMM
  * -> Threshold -> SpatialMaxPooling), y = [B][Co][pH][pW] from thhip_pool_outsize of the

@@ -105,6 +105,8 @@ PROTOTYPES = {
     "thhip_maxpool_cl": (None, [vp, vp] + [C.c_int] * 13),
     "thhip_conv2d_image_pool_supported": (C.c_int, [C.c_int] * 20),
     "thhip_conv2d_image_pool": (None, [vp, vp, vp, vp, vp] + [C.c_int] * 12 + [C.c_int, C.c_float, C.c_float, C.c_int]),
+    "thhip_conv_pair_begin": (None, []),
+    "thhip_conv_pair_end": (None, []),
     "thhip_conv_pack_weight_image_front": (vp, [vp, C.c_int]),
     "thhip_conv2d_image_pair_supported": (C.c_int, [C.c_int] * 7),
     "thhip_conv2d_image_pair": (None, [vp, vp, vp, vp, C.c_int, C.c_float, C.c_float, vp, vp, vp, vp] + [C.c_int] * 5 +

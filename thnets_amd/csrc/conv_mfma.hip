@@ -1539,10 +1539,10 @@ __device__ __forceinline__ void conv_f32_direct_store(const ConvParams &p, float
  * (n, k): step s of a chunk reads rows 8 c + s (lanes 0..31) and 8 c + 4 + s
  * (lanes 32..63); rows are BN + 8 floats apart, so the two halves use different
  * banks.  Needs Ci % 32 == 0. */
-template <int BM, int BN, int KCH, int NST, bool ROWS = false>
-__global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
+#if defined(__HIP_DEVICE_COMPILE__)
+template <int BM, int BN, int KCH, int NST, bool ROWS>
+__device__ __forceinline__ void conv_f32_direct_body(const ConvParams &p, const int bid)
 {
-#if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
 	constexpr int CHUNK = 8, KT = KCH * CHUNK, SUB = 4 / KCH, WAVES = 4, WGM = 2, WGN = 2;
 	static_assert(KCH == 2 || KCH == 4, "the packed blocks of 32 planes are walked in one or two K-tiles");
 	constexpr int MB = BM / 32, TM = BM / WGM / 32, TN = BN / WGN / 32;
@@ -1564,7 +1564,7 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 	int tile_m, tile_n, split = 0, nsplit = p.splitk > 1 ? p.splitk : 1;
 	long tail_blk = -1;
 	{	/* every XCD gets a rectangle of the tile grid, as in conv_mfma_kernel */
-		const int bid = blockIdx.x;
+		
 		const int xcd = bid & 7;
 		int local = bid >> 3;
 		if (p.splitk > 1) {	/* the parts of a tile are neighbours in the order */
@@ -1862,6 +1862,26 @@ __global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
 	}
 	__syncthreads();
 	conv_f32_direct_store<BM, BN, TM, TN>(p, acc, tile_m, tile_n, (int *)lds);
+}
+#endif
+
+template <int BM, int BN, int KCH, int NST, bool ROWS = false>
+__global__ __launch_bounds__(256) void conv_f32_direct_kernel(ConvParams p)
+{
+#if defined(__HIP_DEVICE_COMPILE__)	/* as for conv_wide_kernel: the host pass gets the stub only */
+	conv_f32_direct_body<BM, BN, KCH, NST, ROWS>(p, (int)blockIdx.x);
+#endif
+}
+
+/* Two layers that do not depend on each other in one launch (workgroups 0 .. na - 1 run a, the others b): a
+ * short layer beside a longer one fills the CUs the longer one leaves idle at its end, and costs no launch
+ * of its own (the 1x1 shortcut projection of a residual block beside the block's first convolution). */
+template <int BM, int BN, int KCH, int NST, bool ROWS = false>
+__global__ __launch_bounds__(256) void conv_f32_direct_pair_kernel(ConvParams a, ConvParams b, int na)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+	const bool first = (int)blockIdx.x < na;
+	conv_f32_direct_body<BM, BN, KCH, NST, ROWS>(first ? a : b, first ? (int)blockIdx.x : (int)blockIdx.x - na);
 #endif
 }
 
@@ -2893,6 +2913,35 @@ static bool conv_f32_rows_ok(const ConvParams &p)
 	return !p.x_cl && !p.y_cl && p.Ci % 32 != 0 && p.x_bytes < 0x7fffffffu && p.kHW <= 4096;
 }
 
+/* Pairing (thhip_conv_pair_begin / _end): the launch of a layer that conv_f32_direct_kernel<64, 64, 4, 3> runs whole
+ * (no K split, no cut tiles, no pooling) is held back, and goes out together with the next launch of that kernel
+ * as one grid (conv_f32_direct_pair_kernel); any other convolution call, or _end, sends it out alone. */
+static int g_pair_mode;		/* 1: the launch of the next convolution call is held back if it can be */
+static int g_pair_have;		/* a launch is held back */
+static int g_pair_fresh;	/* ... by the convolution call that is running */
+static ConvParams g_pair_p;
+static unsigned g_pair_grid;
+
+static void conv_pair_flush(void)
+{
+	if (!g_pair_have)
+		return;
+	g_pair_have = 0;
+	conv_f32_direct_kernel<64, 64, 4, 3, false><<<dim3(g_pair_grid), dim3(256), 0, thhip_stream()>>>(g_pair_p);
+}
+
+extern "C" void thhip_conv_pair_begin(void)
+{
+	conv_pair_flush();
+	g_pair_mode = 1;
+}
+
+extern "C" void thhip_conv_pair_end(void)
+{
+	g_pair_mode = 0;
+	conv_pair_flush();
+}
+
 template <int BM, int BN, int KCH, int NST, bool ROWS = false>
 static void conv_launch_f32_direct(ConvParams &p, int splitk)
 {
@@ -2923,7 +2972,26 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 			resident = 1;
 	}
 	const size_t maxcnt = conv_tail_plan(p, resident, nkt, (size_t)BM * BN, 0);
-	conv_f32_direct_kernel<BM, BN, KCH, NST, ROWS><<<dim3((unsigned)(8 * maxcnt * p.splitk)), dim3(256), 0, thhip_stream()>>>(p);
+	const unsigned grid = (unsigned)(8 * maxcnt * p.splitk);
+	bool launched = false;
+	if constexpr (BM == 64 && BN == 64 && KCH == 4 && NST == 3 && !ROWS) {
+		if (g_pair_mode && !g_pair_have && p.splitk == 1 && !p.tail_slots && !p.pk_kH) {
+			g_pair_p = p;	/* held back: goes out with the next launch of this kernel */
+			g_pair_grid = grid;
+			g_pair_have = g_pair_fresh = 1;
+			g_pair_mode = 0;
+			return;
+		}
+		if (g_pair_have) {
+			g_pair_have = 0;
+			conv_f32_direct_pair_kernel<BM, BN, KCH, NST, ROWS><<<dim3(grid + g_pair_grid), dim3(256), 0, thhip_stream()>>>(p, g_pair_p, (int)grid);
+			launched = true;
+		}
+	}
+	if (!launched) {
+		conv_pair_flush();
+		conv_f32_direct_kernel<BM, BN, KCH, NST, ROWS><<<dim3(grid), dim3(256), 0, thhip_stream()>>>(p);
+	}
 	if (p.pk_kH) {
 		/* four lanes per pooled value for windows of up to four values, else sixteen */
 		const int lpo = p.pk_kH * p.pk_kW <= 4 ? 4 : 16;
@@ -3579,6 +3647,11 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 			else
 				THHIP_DISPATCH_FLOAT(dtype, conv_dispatch<DT>(p));
 		}
+		/* a launch held back by an earlier call that this call did not take along goes out now */
+		if (g_pair_have && !g_pair_fresh)
+			conv_pair_flush();
+		g_pair_fresh = 0;
+		g_pair_mode = 0;	/* (only the call right after thhip_conv_pair_begin may be held back) */
 	}
 }
 

@@ -26,6 +26,8 @@ struct hipmod {
 	long res_n;
 	struct hipmod *res_target;	/* ConcatTable: the convolution planned to do the add, or NULL */
 	int res_from_input;	/* ConcatTable: the other branch is the identity (the table's input), else branch 0's output */
+	int shortcut_first;	/* ConcatTable: the shortcut (one convolution) runs first, in one launch with the main branch's first
+				 * convolution, and the main branch's last convolution adds its output */
 	int added_by_producer;	/* table add: 1 + the branch whose convolution did the add in this forward */
 	int table_named;	/* table add / subtract: what the module's name says instead of the shipped arithmetic (THHipTableArithmetic) */
 	int is_linear;		/* MT_Linear in the source network */
