@@ -882,6 +882,63 @@ def test_conv_half_whole_image_patch_kernel(hiplib, oracle, dt):
         hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
 
 
+def test_conv_f32_two_layers_in_one_launch(hiplib, oracle):
+    """thhip_conv_pair_begin / _end: the call right after _begin is held back and shares a launch with the
+    next one where both run whole on the kernel that loads its tiles straight into LDS; bit for bit the two
+    calls made one after the other.  The shapes of a residual block with a projection (1x1 / stride 2
+    beside 3x3 / stride 2), a first call that cannot be held back (a K split), a second call on another
+    kernel (the held launch then follows it), and nothing after the held call but _end."""
+    from thnets_amd import api
+    g = cases.rng(930)
+
+    class Layer:
+        def __init__(self, B, Ci, H, W, Co, k, d, pad, x=None):
+            self.shape = (B, Ci, H, W, Co, k, d, pad)
+            self.x = x if x is not None else api.DeviceArray(hiplib, g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32))
+            w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+            self.w = w
+            self.b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            self.db = api.DeviceArray(hiplib, self.b)
+            self.wp = hiplib.thhip_conv_pack_weight(np.ascontiguousarray(w).ctypes.data, Co, Ci, k * k, G.F32)
+            self.o = ((H + 2 * pad - k) // d + 1, (W + 2 * pad - k) // d + 1)
+            self.y = api.DeviceArray(hiplib, nbytes=B * Co * self.o[0] * self.o[1] * 4)
+
+        def run(self):
+            B, Ci, H, W, Co, k, d, pad = self.shape
+            hiplib.thhip_conv2d(self.x.ptr, self.wp, self.db.ptr, self.y.ptr, B, Ci, H, W, Co, k, k, d, d, pad, pad, 1, 0.0, 0.0, G.F32)
+
+        def read(self):
+            hiplib.thhip_sync()
+            out = api.from_device_dtype(self.y, (self.shape[0], self.shape[4]) + self.o, G.F32).copy()
+            hiplib.thhip_memset(self.y.ptr, 0, self.y.nbytes)
+            return out
+
+    cases_ = []
+    for (B, Ci, S, Co) in ((8, 64, 56, 128), (8, 128, 28, 256), (3, 32, 30, 64)):
+        a = Layer(B, Ci, S, S, Co, 1, 2, 0)
+        cases_.append((a, Layer(B, Ci, S, S, Co, 3, 2, 1, x=a.x), "projection beside the first convolution"))
+    a = Layer(2, 256, 14, 14, 256, 3, 1, 1)                       # few tiles, long K: split, not held back
+    cases_.append((a, Layer(2, 256, 14, 14, 64, 1, 1, 0, x=a.x), "a first call with a K split"))
+    a = Layer(16, 64, 28, 28, 64, 1, 1, 0)
+    cases_.append((a, Layer(16, 64, 56, 56, 64, 3, 1, 1), "a second call on the patch kernel"))
+    for (first, second, what) in cases_:
+        G.note("two layers in one launch: " + what + " " + str(first.shape) + " " + str(second.shape))
+        first.run(); second.run()
+        want = (first.read(), second.read())
+        hiplib.thhip_conv_pair_begin()
+        first.run(); second.run()
+        hiplib.thhip_conv_pair_end()
+        got = (first.read(), second.read())
+        assert np.array_equal(got[0], want[0]) and np.array_equal(got[1], want[1]), what
+        G.assert_close(got[0], np.maximum(oracle.conv2d(api.from_device_dtype(first.x, first.shape[:4], G.F32), first.w, first.b,
+                                                        (first.shape[6],) * 2, (first.shape[7],) * 2), 0), FP32_TOL, what)
+        hiplib.thhip_conv_pair_begin()
+        first.run()
+        hiplib.thhip_conv_pair_end()
+        assert np.array_equal(first.read(), want[0]), what + ", alone"
+        hiplib.thhip_free(first.wp); hiplib.thhip_free(second.wp)
+
+
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_conv_half_image_layer_in_front(hiplib, oracle, dt):
     """The network's image layer (3 -> 64 planes, 3x3 / stride 1 / padding 1, factor, shift, Threshold) computed
