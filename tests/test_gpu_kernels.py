@@ -549,7 +549,7 @@ def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
                 hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
             G.assert_close(got, want, FP32_TOL, "fp32 patch kernel " + str((B, Ci, H, W, Co, act)))
     # seeded random shapes (all three patch shapes, last tiles of one to three 4x4 patches): against the kernel
-    # that fetches every tap with a load of its own (another order of the sums)
+    # that fetches every tap with a load of its own (another order of the sums) and against the restatement
     for it in range(16):
         B, Ci, Co = int(g.integers(1, 6)), int(g.choice([32, 64, 96, 160])), int(g.choice([64, 128, 192]))
         H, W = 4 * int(g.integers(1, 13)), 4 * int(g.integers(1, 13))
@@ -565,6 +565,8 @@ def test_conv_f32_taps_from_a_patch_in_lds(hiplib, oracle):
             finally:
                 hiplib.thhip_conv_set_tuning(0, 0, 0, 0)
         G.assert_close(outs[0], outs[1], FP32_TOL, "fp32 patch kernel against the other " + str((B, Ci, H, W, Co)))
+        want = np.maximum(oracle.conv2d(x, w, b, (1, 1), (1, 1)), np.float32(0))
+        G.assert_close(outs[0], want, FP32_TOL, "fp32 patch kernel, random shape, against the restatement " + str((B, Ci, H, W, Co)))
     # as dispatched: 2048 tiles of 64 planes x 64 pixels
     for (B, Ci, H, W, Co) in ((32, 32, 64, 64, 64), (24, 64, 56, 56, 128), (44, 64, 28, 28, 256), (140, 32, 24, 40, 64)):
         x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)

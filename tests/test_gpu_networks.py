@@ -379,9 +379,12 @@ def test_vgg16_full_size_half_engines(hiplib, oracle, half):
 def test_loaded_model_directory_runs_like_the_layer_list(hiplib, oracle, tmp_path, name):
     """THLoadNetwork -> THCreateHipNetwork -> THProcessFloat on a Torch7 model
     directory gives, bit for bit, what the same weights give when the module array
-    is assembled by hand, in fp32, fp16 and uint8 form."""
+    is assembled by hand, in fp32, fp16 and uint8 form; the fp32 and fp16 results are
+    also held against the golden vector of the reference's CPU library and against the
+    oracle on the same weights."""
     from thnets_amd import t7
     cfg = cases.small_networks()[name]
+    ref = np.asarray(oracle.run_layers(cfg["layers"], oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])))
     t7.save_model_dir(str(tmp_path), cfg["layers"], cfg["mean"], cfg["std"], longsize=4 if name == "tiny_cnn" else 8)
     G.note("model directory %s" % name)
     for kw in ({}, {"half": 1}) + (({"lowp_range": 16.0, "make_spatial": 8},) if name == "tiny_cnn" else ()):
@@ -391,6 +394,11 @@ def test_loaded_model_directory_runs_like_the_layer_list(hiplib, oracle, tmp_pat
         a.free()
         b.free()
         assert got.shape == want.shape and np.array_equal(got, want), kw
+        if not kw:
+            G.assert_close(got, GOLD["net_" + name], NET_TOL, "model directory against the golden vector")
+            G.assert_close(got.ravel(), ref.ravel(), NET_TOL, "model directory against the oracle")
+        elif "half" in kw:
+            G.assert_close(got.ravel(), ref.ravel(), 3e-2, "model directory, fp16, against the oracle")
 
 
 @pytest.mark.gpu
@@ -408,12 +416,14 @@ def test_command_line_driver(hiplib, oracle, tmp_path):
     assert os.path.exists(exe), "build it with make -C thnets_amd/csrc"
     net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
     want = net.process_float(np.stack([x, x]))
+    ref = np.asarray(oracle.run_layers(cfg["layers"], oracle.normalize(np.stack([x, x]), cfg["mean"], cfg["std"])))
     G.note("thnets-hip-test fp32 batch 2")
     r = subprocess.run([exe, "-m", str(tmp_path), "-i", str(tmp_path / "in.t7"), "-p", "-b", "2", "-r", "2"],
                        capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stderr
     vals = [float(l.split(":")[1]) for l in r.stdout.splitlines() if l.startswith("(")]
     assert len(vals) == want.size and np.allclose(vals, want, rtol=0, atol=5e-7)
+    G.assert_close(np.asarray(vals, np.float32), ref.ravel(), NET_TOL, "printed values against the oracle")
     assert "1 run processing time:" in r.stdout
     # an 8-bit image through THProcessImages
     g = cases.rng(91)
@@ -428,6 +438,9 @@ def test_command_line_driver(hiplib, oracle, tmp_path):
     assert r.returncode == 0, r.stderr
     vals = [float(l.split(":")[1]) for l in r.stdout.splitlines() if l.startswith("(")]
     assert len(vals) == 4 and np.allclose(vals, want[:4], rtol=0, atol=5e-7)
+    ximg = oracle.rgb2float(img, cfg["mean"], cfg["std"], 0)[None]
+    ref = np.asarray(oracle.run_layers(cfg["layers"], ximg)).ravel()
+    G.assert_close(np.asarray(vals, np.float32), ref[:4], NET_TOL, "printed values of the image against the oracle")
     # a model directory that does not exist: the reference's message, exit code 0 (thnets-test.c:199)
     r = subprocess.run([exe, "-m", str(tmp_path / "none"), "-i", "random"], capture_output=True, text=True, timeout=120)
     assert "The network could not be loaded: -1" in r.stdout
