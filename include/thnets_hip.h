@@ -342,6 +342,14 @@ int THHipFoldBatchNorm(int enable);
  * within the last bit of a half value (another order of the 27 products' sum).  Read at every forward;
  * returns the previous setting. */
 int THHipImageLayerInFront(int mode);
+/* fp32 convolutions cut the tiles an XCD could not spread evenly over its CUs into parts along K, computed
+ * by several workgroups of that XCD (nothing in the reference: its GEMM is one sgemm call per image,
+ * modules/SpatialConvolutionMM.c:136-150).  1 (default): the workgroup whose part is ready last adds the
+ * parts, in their order, and finishes the tile; the parts meet in the XCD's L2, and every such workgroup
+ * checks that it runs on the XCD its position in the grid implies (a violation is reported as an error at
+ * the next synchronisation, never as a silently wrong sum).  0: a second launch adds the parts.  The same
+ * bits either way.  Read at every launch; returns the previous setting. */
+int THHipSumPartsInKernel(int enable);
 /* 0 (default): CAddTable / CSubTable compute what the reference's shipped modules
  * compute (modules/CAddTable.c:59-84: with two inputs CAddTable gives a - b and
  * CSubTable a + b; with more, 2a + b + c + ... and 0 - b - c - ...).  1: what the

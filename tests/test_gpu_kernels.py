@@ -941,6 +941,72 @@ def test_conv_f32_two_layers_in_one_launch(hiplib, oracle):
         hiplib.thhip_free(first.wp); hiplib.thhip_free(second.wp)
 
 
+def test_conv_f32_cut_tiles_added_in_the_kernel(hiplib, oracle):
+    """THHipSumPartsInKernel: the tiles an XCD cuts along K, added by the workgroup whose part is ready last
+    (the parts meet in the XCD's L2) against the same launch followed by the kernel that adds them: the same
+    bits, on both fp32 kernels that cut tiles (3x3 / stride 1 from a patch in LDS; strided and 1x1 layers with
+    tiles loaded straight into LDS), with the folded factor and Threshold, with a table add, with the 2x2
+    pooling; every case three times in a row (the arrival counters are left at zero).  One case against the
+    restatement.  The workgroups of every residue of blockIdx.x % 8 were seen on one XCD."""
+    from thnets_amd import api
+    g = cases.rng(7700)
+    assert hiplib.thhip_xcd_map() >> 31, "workgroups of one residue of blockIdx.x % 8 on different XCDs"
+    shapes = [(32, 64, 56, 56, 64, 3, 1, 1), (24, 64, 56, 56, 128, 3, 1, 1), (44, 64, 28, 28, 256, 3, 1, 1), (12, 128, 64, 32, 128, 3, 1, 1),
+              (32, 64, 56, 56, 128, 3, 2, 1), (16, 64, 40, 40, 128, 5, 1, 2), (9, 64, 75, 77, 64, 3, 1, 1), (32, 128, 56, 56, 128, 3, 2, 1)]
+    cut = [0, 0]        # launches with cut tiles: tiles loaded straight into LDS, taps from a patch
+    try:
+        for (B, Ci, H, W, Co, k, d, pad) in shapes:
+            oH, oW = (H + 2 * pad - k) // d + 1, (W + 2 * pad - k) // d + 1
+            x = g.uniform(-1, 1, (B, Ci, H, W)).astype(np.float32)
+            w = g.standard_normal((Co, Ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (Ci * k * k)))
+            b = g.standard_normal(Co, dtype=np.float32) * np.float32(0.1)
+            sc = g.uniform(0.5, 1.5, Co).astype(np.float32)
+            r = g.standard_normal((B, Co, oH, oW), dtype=np.float32)
+            args = (B, Ci, H, W, Co, k, k, d, d, pad, pad)
+            wp = hiplib.thhip_conv_pack_weight_layout(w.ctypes.data, Co, Ci, k, k, G.F32, 0)
+            dx, db, ds, dr = (api.DeviceArray(hiplib, a) for a in (x, b, sc, r))
+            n = B * Co * oH * oW
+            dy = api.DeviceArray(hiplib, nbytes=n * 4)
+            pool = oH % 2 == 0 and oW % 2 == 0 and hiplib.thhip_conv2d_pool2_supported(*args, G.F32, 0, 0)
+            res = hiplib.thhip_conv2d_residual_supported(*args, G.F32)
+            outs = {}
+            for mode in (0, 1, 1, 1, 0):
+                G.note("cut tiles, added in the kernel %d, %s" % (mode, args))
+                hiplib.THHipSumPartsInKernel(mode)
+                before = hiplib.thhip_conv_cut_launches(0), hiplib.thhip_conv_cut_launches(1)
+                got = []
+                hiplib.thhip_memset(dy.ptr, 0xFF, n * 4)
+                hiplib.thhip_conv2d_layout(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, *args, 1, 0.05, 0.05, G.F32, 0, 0)
+                hiplib.thhip_sync()
+                got.append(dy.get((B, Co, oH, oW), np.float32))
+                after = hiplib.thhip_conv_cut_launches(0), hiplib.thhip_conv_cut_launches(1)
+                assert after[mode] == before[mode] and after[1 - mode] - before[1 - mode] in (0, 1), (args, mode, before, after)
+                cut[(k, d) == (3, 1)] += after[1 - mode] - before[1 - mode]
+                if res:
+                    hiplib.thhip_memset(dy.ptr, 0xFF, n * 4)
+                    hiplib.thhip_conv2d_residual(dx.ptr, wp, None, db.ptr, dr.ptr, 2, -1.0, 1, dy.ptr, *args, 0, 0.0, 0.0, G.F32)
+                    hiplib.thhip_sync()
+                    got.append(dy.get((B, Co, oH, oW), np.float32))
+                if pool:
+                    hiplib.thhip_memset(dy.ptr, 0xFF, n * 4)
+                    hiplib.thhip_conv2d_layout_pool2(dx.ptr, wp, ds.ptr, db.ptr, dy.ptr, *args, 1, 0.05, 0.05, G.F32, 0, 0)
+                    hiplib.thhip_sync()
+                    got.append(dy.get((B, Co, oH // 2, oW // 2), np.float32))
+                if mode in outs:
+                    assert all(np.array_equal(a, c) for a, c in zip(got, outs[mode])), ("not the same twice", args, mode)
+                outs[mode] = got
+            assert len(outs[0]) == len(outs[1]) == 1 + int(bool(res)) + int(bool(pool))
+            for a, c in zip(outs[0], outs[1]):
+                assert np.array_equal(a, c), (args, np.abs(a - c).max())
+            if (B, Ci, H) == (9, 64, 75):
+                raw = oracle.conv2d(x, w, None, (d, d), (pad, pad)) * sc[None, :, None, None] + b[None, :, None, None]
+                G.assert_close(outs[1][0], np.where(raw > 0.05, raw, np.float32(0.05)), FP32_TOL, "cut tiles added in the kernel " + str(args))
+            hiplib.thhip_free(wp)
+        assert cut[0] >= 10 and cut[1] >= 15, cut     # (five launches a shape)
+    finally:
+        hiplib.THHipSumPartsInKernel(1)
+
+
 @pytest.mark.parametrize("dt", [G.F16, G.BF16])
 def test_conv_half_image_layer_in_front(hiplib, oracle, dt):
     """The network's image layer (3 -> 64 planes, 3x3 / stride 1 / padding 1, factor, shift, Threshold) computed

@@ -28,6 +28,8 @@ vp = C.c_void_p
 TEST_HOOKS = {
     "thhip_conv_set_ktile": (None, [C.c_int]),
     "thhip_conv_set_tail_parts": (None, [C.c_int]),
+    "thhip_xcd_map": (C.c_uint, []),
+    "thhip_conv_cut_launches": (C.c_long, [C.c_int]),
     "thhip_conv_set_xcd_parts": (None, [C.c_int]),
     "thhip_conv_set_generic_cl": (None, [C.c_int]),
     "thhip_linear_batched_set_tuning": (None, [C.c_int]),
@@ -67,6 +69,7 @@ PROTOTYPES = {
     "THHipHalfFloat": (C.c_int, [C.c_int]),
     "THHipFoldBatchNorm": (C.c_int, [C.c_int]),
     "THHipImageLayerInFront": (C.c_int, [C.c_int]),
+    "THHipSumPartsInKernel": (C.c_int, [C.c_int]),
     "THHipTableArithmetic": (C.c_int, [C.c_int]),
     "THCreateHipLowpNetwork": (vp, [vp, C.c_float]),
     "THHipTensor_newFromFloatTensor": (vp, [vp]),

@@ -48,6 +48,9 @@ struct ConvParams {
 	int tail_cap;		/* scratch blocks (parts of BM*BN sums) reserved per XCD: [xcd][tile][part] */
 	int tail_tiles;		/* most cut tiles of an XCD */
 	int tail_round;		/* 1: an XCD with less than one whole round of tiles is left uncut */
+	int tail_inline;	/* 1: the part of a cut tile that arrives last adds the parts and finishes the tile (cnt) */
+	unsigned xcd_map;	/* thhip_xcd_map() */
+	int *fault;		/* thhip_fault_flag() */
 	/* conv_f32_direct_kernel with a K split of the whole layer: a max pooling that follows, taken by the kernel
 	 * that adds the parts (pk_kH 0: none); pk_oH x pk_oW is the pooled plane */
 	int pk_kH, pk_kW, pk_dH, pk_dW, pk_padH, pk_padW, pk_oH, pk_oW;

@@ -829,6 +829,40 @@ __device__ inline void conv_xcd_rect(const ConvParams &p, int xcd, int &m0, int 
 	cnt = mw * (n1 - n0);
 }
 
+/* The parts of a cut tile are computed by workgroups of one XCD (workgroup b runs on XCD b % 8), which
+ * share that XCD's L2: a part's sums need only reach L2 (the vector caches write through; the wait for
+ * the stores' acknowledgement is the release) before the ticket is drawn there (an atomic without the
+ * device-scope bit executes in the XCD's L2), and the workgroup that draws the last ticket reads them
+ * from L2.  No L2 write-back or invalidate as a device-scope fence would do (measured with those, and
+ * with device-scope loads and stores of the parts: slower than a second launch; this way ResNet-18 batch
+ * 32 1.269 -> 1.239 ms and VGG-16 batch 16 3.825 -> 3.803 ms against the second launch.  The parts of a
+ * layer whose whole K is split stay with their second launch: every tile's last workgroup adding parts
+ * cost 8 us a layer more than it).  Returns whether this
+ * workgroup drew the last of `parts` tickets (and has reset the counter for the next launch); `slot`
+ * is one int of LDS nobody else uses until the next barrier after the call. */
+__device__ __forceinline__ bool conv_xcd_last_arriver(const ConvParams &p, unsigned *counter, int parts, int *slot)
+{
+	/* (on the XCD the map names for this residue of blockIdx.x, or the host hears of it) */
+	if (threadIdx.x == 0 && (int)__builtin_amdgcn_s_getreg(THHIP_GETREG_XCC_ID) != (int)((p.xcd_map >> (4 * (blockIdx.x & 7))) & 7u))
+		__hip_atomic_store(p.fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+	__syncthreads();
+	if (threadIdx.x == 0)
+		*slot = (int)__hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+	__syncthreads();
+	const bool last = *slot == parts - 1;
+	if (last && threadIdx.x == 0)
+		*counter = 0;
+	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+	return last;
+}
+
+/* One fp32 sum of another workgroup's part, from L2 (sc0: not from this CU's vector cache). */
+__device__ __forceinline__ float conv_load_part(const float *p)
+{
+	return __builtin_bit_cast(float, __hip_atomic_load((const int *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP));
+}
+
 /* The tiles an XCD cannot spread evenly: of its cnt tiles the last cnt % slots
  * would run a few to a CU (or alone) while the other CUs idle.  Those are cut
  * along K into as many parts as fill the slots once, at most smax; *full is
@@ -1825,10 +1859,10 @@ __device__ __forceinline__ void conv_f32_direct_body(const ConvParams &p, const 
 	}
 
 	if (tail_blk >= 0) {
-		/* a part of one of the XCD's last tiles: the accumulators as they lie in
-		 * the registers, [register][thread]; conv_f32_tail_finish_kernel adds the
-		 * parts in their order */
-		float *part = (float *)p.ws + tail_blk * (BM * BN);
+		/* a part of one of the XCD's last tiles: the accumulators as they lie in the registers,
+		 * [register][thread], in block tail_blk of scratch */
+		const long blk0 = tail_blk - split;
+		float *part = (float *)p.ws + (blk0 + split) * (BM * BN);
 #pragma unroll
 		for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -1836,6 +1870,35 @@ __device__ __forceinline__ void conv_f32_direct_body(const ConvParams &p, const 
 #pragma unroll
 				for (int r = 0; r < 16; r++)
 					part[((i * TN + j) * 16 + r) * 256 + tid] = acc[i][j][r];
+		if (!p.tail_inline)
+			return;		/* conv_f32_tail_finish_kernel adds the parts */
+		/* the part that arrives last adds them all in their order (four on their way at a time) */
+		if (!conv_xcd_last_arriver(p, p.cnt + blk0, nsplit, (int *)lds))
+			return;
+		const float *all = (const float *)p.ws + blk0 * (BM * BN) + tid;
+#pragma unroll
+		for (int i = 0; i < TM; i++)
+#pragma unroll
+			for (int j = 0; j < TN; j++)
+				for (int q0 = 0; q0 < nsplit; q0 += 4) {
+					float in[4][16];
+#pragma unroll
+					for (int q = 0; q < 4; q++)
+						if (q0 + q < nsplit) {
+#pragma unroll
+							for (int r = 0; r < 16; r++)
+								in[q][r] = conv_load_part(all + (long)(q0 + q) * (BM * BN) + ((i * TN + j) * 16 + r) * 256);
+						}
+#pragma unroll
+					for (int q = 0; q < 4; q++)
+						if (q0 + q < nsplit) {
+#pragma unroll
+							for (int r = 0; r < 16; r++)
+								acc[i][j][r] = q0 + q == 0 ? in[q][r] : acc[i][j][r] + in[q][r];
+						}
+				}
+		__syncthreads();
+		conv_f32_direct_store<BM, BN, TM, TN>(p, acc, tile_m, tile_n, (int *)lds);
 		return;
 	}
 	if (p.splitk > 1) {
@@ -2009,7 +2072,8 @@ __device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx
  * next half block's loads spread over this one's taps), the weights' 1 KiB blocks go through a ring
  * of three K-tiles as in conv_f32_direct_kernel.  The nine taps of a half block are straight-line
  * code: every LDS offset and wait count a constant.  The last tiles of an XCD are cut along K as
- * there (conv_tail_parts; a part is whole blocks of 32 planes), summed by
+ * there (conv_tail_parts; a part is whole blocks of 32 planes) and added by the workgroup whose part
+ * is ready last (conv_xcd_last_arriver), or, with THHipSumPartsInKernel(0), by
  * conv_f32_patch_tail_finish_kernel. */
 template <int SW, int SH>
 __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
@@ -2192,12 +2256,34 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the workgroup ends or the epilogue reuses it) */
 	if (tail_blk >= 0) {
 		/* a part of one of the XCD's last tiles: the accumulator as it lies in the registers,
-		 * [register][thread]; conv_f32_patch_tail_finish_kernel adds the parts in their order */
+		 * [register][thread] */
 		float *part = (float *)p.ws + tail_blk * (64 * 64);
 #pragma unroll
 		for (int r = 0; r < 16; r++)
 			part[r * 256 + tid] = acc[r];
-		return;
+		if (!p.tail_inline)
+			return;		/* conv_f32_patch_tail_finish_kernel adds the parts */
+		/* the part that arrives last adds them all in their order (four on their way at a time) */
+		if (!conv_xcd_last_arriver(p, p.cnt + (tail_blk - split), nsplit, (int *)lds_a))
+			return;
+		const float *all = (const float *)p.ws + (tail_blk - split) * (64 * 64) + tid;
+		for (int q0 = 0; q0 < nsplit; q0 += 4) {
+			float in[4][16];
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				if (q0 + q < nsplit) {
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						in[q][r] = conv_load_part(all + (long)(q0 + q) * (64 * 64) + r * 256);
+				}
+#pragma unroll
+			for (int q = 0; q < 4; q++)
+				if (q0 + q < nsplit) {
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						acc[r] = q0 + q == 0 ? in[q][r] : acc[r] + in[q][r];
+				}
+		}
 	}
 	__syncthreads();
 	conv_f32_patch_store<SW, SH>(p, acc, tile_m, tile_n, (int *)lds_a);
@@ -2605,6 +2691,22 @@ extern "C" void thhip_conv_set_xcd_parts(int mparts)
 /* fp32 and half-type tiles loaded straight into LDS: the most K parts for the
  * tiles an XCD cannot spread evenly over its CUs (1: never cut them). */
 static int g_tail_parts = 8;
+/* Whether the parts of a cut tile are added by the part that arrives last (conv_xcd_last_arriver) or by a
+ * second launch; the first only where the workgroups of a residue of blockIdx.x % 8 were seen on one XCD. */
+static int g_tail_inline = 1;
+/* launches so far whose cut tiles were added in the kernel / by a second launch (for the tests) */
+static long g_tail_launches[2];
+extern "C" long thhip_conv_cut_launches(int second_launch)
+{
+	return g_tail_launches[second_launch != 0];
+}
+
+extern "C" int THHipSumPartsInKernel(int on)
+{
+	const int was = g_tail_inline;
+	g_tail_inline = on != 0;
+	return was;
+}
 extern "C" void thhip_conv_set_tail_parts(int parts)
 {
 	if (parts < 1 || parts > 64)
@@ -2634,6 +2736,20 @@ static size_t g_ws_bytes;
 static unsigned *g_cnt;
 static size_t g_cnt_n;
 
+/* Points p.cnt at `tiles` arrival counters, zero between launches (the workgroup that draws a tile's last
+ * ticket resets it). */
+static void conv_counters(ConvParams &p, size_t tiles)
+{
+	if (tiles > g_cnt_n) {
+		hipcheck(hipStreamSynchronize(thhip_stream()));
+		thhip_free(g_cnt);
+		g_cnt_n = tiles < 4096 ? 4096 : tiles;
+		g_cnt = (unsigned *)thhip_malloc(g_cnt_n * sizeof(unsigned));
+		thhip_memset(g_cnt, 0, g_cnt_n * sizeof(unsigned));
+	}
+	p.cnt = g_cnt;
+}
+
 static void conv_scratch(ConvParams &p, size_t tiles, size_t tile_words)
 {
 	const size_t need = tiles * p.splitk * tile_words * sizeof(int);
@@ -2643,15 +2759,8 @@ static void conv_scratch(ConvParams &p, size_t tiles, size_t tile_words)
 		g_ws = (int *)thhip_malloc(need);
 		g_ws_bytes = need;
 	}
-	if (tiles > g_cnt_n) {
-		hipcheck(hipStreamSynchronize(thhip_stream()));
-		thhip_free(g_cnt);
-		g_cnt_n = tiles < 4096 ? 4096 : tiles;
-		g_cnt = (unsigned *)thhip_malloc(g_cnt_n * sizeof(unsigned));
-		thhip_memset(g_cnt, 0, g_cnt_n * sizeof(unsigned));
-	}
 	p.ws = g_ws;
-	p.cnt = g_cnt;
+	conv_counters(p, tiles);
 }
 
 #define CONV_LDS_PER_CU (160 * 1024)
@@ -2788,7 +2897,7 @@ static void conv_f32_scratch(ConvParams &p, size_t need)
  * holds `resident` workgroups per CU and walks nkt K-tiles per tile: sets
  * p.tail_*, points p.ws at scratch for the parts and returns the largest
  * number of workgroups an XCD needs (its whole tiles plus the parts). */
-static size_t conv_tail_plan(ConvParams &p, int resident, int nkt, size_t tile_floats, int need_round)
+static size_t conv_tail_plan(ConvParams &p, int resident, int nkt, size_t tile_floats, int need_round, bool inline_ok = false)
 {
 	static int cus;
 	if (!cus) {
@@ -2796,11 +2905,11 @@ static size_t conv_tail_plan(ConvParams &p, int resident, int nkt, size_t tile_f
 		hipcheck(hipGetDevice(&dev));
 		hipcheck(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
 	}
-	p.tail_slots = p.tail_max = p.tail_cap = p.tail_tiles = 0;
+	p.tail_slots = p.tail_max = p.tail_cap = p.tail_tiles = p.tail_inline = 0;
 	p.tail_round = need_round;
 	if (p.splitk == 1 && g_tail_parts != 1) {
 		p.tail_slots = cus / 8 * (resident < 1 ? 1 : resident);
-		p.tail_max = nkt / 8 < g_tail_parts ? nkt / 8 : g_tail_parts;	/* at least eight K-tiles a part */
+		p.tail_max = nkt / 8 < g_tail_parts ? nkt / 8 : g_tail_parts;	/* at least eight K-tiles a part (four and two: slower) */
 		if (p.tail_max > 8)
 			p.tail_max = 8;	/* the finishing kernels hold eight parts in registers */
 		if (p.tail_max < 2)
@@ -2825,8 +2934,15 @@ static size_t conv_tail_plan(ConvParams &p, int resident, int nkt, size_t tile_f
 	}
 	if (!p.tail_cap)
 		p.tail_slots = 0;
-	else
+	else {
 		conv_f32_scratch(p, (size_t)8 * p.tail_cap * tile_floats * sizeof(float));
+		p.tail_inline = inline_ok && g_tail_inline && (thhip_xcd_map() >> 31);
+		if (p.tail_inline) {
+			conv_counters(p, (size_t)8 * p.tail_cap);
+			p.xcd_map = thhip_xcd_map();
+			p.fault = thhip_fault_flag();
+		}
+	}
 	return maxwgs;
 }
 
@@ -2971,7 +3087,7 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 		if (resident < 1)
 			resident = 1;
 	}
-	const size_t maxcnt = conv_tail_plan(p, resident, nkt, (size_t)BM * BN, 0);
+	const size_t maxcnt = conv_tail_plan(p, resident, nkt, (size_t)BM * BN, 0, true);
 	const unsigned grid = (unsigned)(8 * maxcnt * p.splitk);
 	bool launched = false;
 	if constexpr (BM == 64 && BN == 64 && KCH == 4 && NST == 3 && !ROWS) {
@@ -3020,6 +3136,8 @@ static void conv_launch_f32_direct(ConvParams &p, int splitk)
 			(float *)p.y, p.splitk, p.Co, p.N, p.oHW, p.act, p.thr, p.val, p.res, p.res_mode, p.res_c, p.res_act);
 	}
 	if (p.tail_slots)
+		g_tail_launches[!p.tail_inline]++;
+	if (p.tail_slots && !p.tail_inline)
 		conv_f32_tail_finish_kernel<BM, BN><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
 
@@ -3106,9 +3224,11 @@ static void conv_launch_f32_patch(ConvParams &p)
 		if (dyn < 0)
 			dyn = 0;
 	}
-	const size_t maxcnt = conv_tail_plan(p, use, p.Ci / 32 * 8, 64 * 64, 0);
+	const size_t maxcnt = conv_tail_plan(p, use, p.Ci / 32 * 8, 64 * 64, 0, true);
 	conv_f32_patch_kernel<SW, SH><<<dim3((unsigned)(8 * maxcnt)), dim3(256), dyn, thhip_stream()>>>(p);
 	if (p.tail_slots)
+		g_tail_launches[!p.tail_inline]++;
+	if (p.tail_slots && !p.tail_inline)
 		conv_f32_patch_tail_finish_kernel<SW, SH><<<dim3((unsigned)(8 * p.tail_tiles)), dim3(256), 0, thhip_stream()>>>(p);
 }
 

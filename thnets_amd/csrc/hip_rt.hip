@@ -78,10 +78,13 @@ extern "C" void thhip_memcpy_h2d(void *dst, const void *src, size_t bytes)
 	hipcheck(hipStreamSynchronize(thhip_stream()));
 }
 
+static void fault_check(void);
+
 extern "C" void thhip_memcpy_d2h(void *dst, const void *src, size_t bytes)
 {
 	hipcheck(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, thhip_stream()));
 	hipcheck(hipStreamSynchronize(thhip_stream()));
+	fault_check();
 }
 
 /* Page-locked host memory: copies to and from it run at the link's rate and, queued with the
@@ -139,6 +142,72 @@ extern "C" void thhip_memset(void *dst, int value, size_t bytes)
 extern "C" void thhip_sync(void)
 {
 	hipcheck(hipStreamSynchronize(thhip_stream()));
+	fault_check();
+}
+
+/* ---- which XCD a workgroup runs on ----
+ * The convolution kernels let the workgroups that compute the parts of one tile meet in their XCD's L2
+ * (conv_xcd_last_arriver), which is right only if those workgroups -- all of one residue of
+ * blockIdx.x modulo 8 -- run on one XCD.  The hardware hands workgroup b to XCD b % 8; this is checked
+ * once per process on a grid of 4096 workgroups (thhip_xcd_map), and again by every such workgroup
+ * against the map (a mismatch raises the flag below, which the next synchronisation turns into an
+ * error). */
+__global__ void xcd_probe_kernel(int *out)
+{
+	if (threadIdx.x == 0)
+		out[blockIdx.x] = __builtin_amdgcn_s_getreg(THHIP_GETREG_XCC_ID);
+}
+
+/* 0x80000000 | the XCC id (0 .. 7) of residue r in bits 4 r .. 4 r + 2; 0 if the workgroups of a residue were
+ * seen on different XCDs (then nothing may rely on it). */
+extern "C" unsigned thhip_xcd_map(void)
+{
+	static unsigned map;
+	static int done;
+	if (done)
+		return map;
+	const int n = 4096;
+	int *dev = (int *)thhip_malloc(n * sizeof(int));
+	std::vector<int> host(n);
+	xcd_probe_kernel<<<dim3(n), dim3(64), 0, thhip_stream()>>>(dev);
+	hipcheck(hipGetLastError());
+	hipcheck(hipMemcpyAsync(host.data(), dev, n * sizeof(int), hipMemcpyDeviceToHost, thhip_stream()));
+	hipcheck(hipStreamSynchronize(thhip_stream()));
+	thhip_free(dev);
+	bool ok = true;
+	for (int b = 0; b < n; b++)
+		ok = ok && host[b] == host[b & 7] && (unsigned)host[b] < 8u;
+	map = 0;
+	if (ok) {
+		map = 0x80000000u;
+		for (int r = 0; r < 8; r++)
+			map |= (unsigned)host[r] << (4 * r);
+	}
+	done = 1;
+	return map;
+}
+
+/* One int in page-locked host memory that kernels set when they find themselves where they must not
+ * be; thhip_sync and the copies to the host look at it. */
+static int *g_fault;
+
+extern "C" int *thhip_fault_flag(void)
+{
+	if (!g_fault) {
+		g_fault = (int *)thhip_host_malloc(sizeof(int));
+		*g_fault = 0;
+	}
+	return g_fault;
+}
+
+static void fault_check(void)
+{
+	if (g_fault && *(volatile int *)g_fault) {
+		const int code = *(volatile int *)g_fault;
+		*g_fault = 0;
+		THError("thnets HIP engine: a kernel reported fault %d (1: workgroups that share partial sums through "
+			"their XCD's L2 ran on different XCDs; THHipSumPartsInKernel(0) turns that path off)", code);
+	}
 }
 
 /* ---- events ---- */

@@ -12,6 +12,11 @@
 
 hipStream_t thhip_stream(void);
 
+/* s_getreg operand of the XCC id (hardware register 20, bits 0 .. 3): the XCD this wave runs on */
+#define THHIP_GETREG_XCC_ID ((3 << 11) | 20)
+extern "C" unsigned thhip_xcd_map(void);	/* hip_rt.hip: which XCD the workgroups of a residue of blockIdx.x % 8 run on */
+extern "C" int *thhip_fault_flag(void);		/* hip_rt.hip: set by a kernel, turned into an error at the next synchronisation */
+
 /* Profiling hooks: bracket one kernel launch.  `work` is the algorithmic
  * work of the launch (flops for GEMM-like kernels, bytes otherwise). */
 int thhip_prof_begin(int family);
@@ -56,6 +61,8 @@ void thhip_conv_set_ktile(int chunks);
  * kernel (results do not depend on timing).  Default 8, which is also the most
  * that is used; 1 = never cut.  Tests and tuning. */
 void thhip_conv_set_tail_parts(int parts);
+/* launches so far whose cut tiles were added in the kernel (0) / by a second launch (1) */
+long thhip_conv_cut_launches(int second_launch);
 /* Force how the tile grid is cut over the eight XCDs: the M tiles into
  * mparts (1, 2, 4, 8) groups, the N tiles into 8 / mparts ranges; 0 restores
  * the choice by weight size.  Tests and tuning. */
