@@ -179,7 +179,7 @@ def main():
                 "traffic": counter_traffic("conv_f32_vgg16_fp32_b16_counters.md", "conv_hbm_bytes_per_launch"),
                 "kernel": "conv_f32_patch_kernel (implicit-GEMM convolution, every tap of a 3x3 layer read from one input patch "
                           "per plane in LDS: nine of the 13 convolutions of a step, four of them with the 2x2 max pooling that "
-                          "follows in their epilogue, six with the kernel that sums the K parts of their last tiles) and "
+                          "follows in their epilogue; the K parts of an XCD's last tiles added in the kernel) and "
                           "conv_f32_direct_kernel (operands loaded straight into LDS: the three 14x14 layers, K split in three, with "
                           "the kernel that sums the parts); the image layer on conv_stem_kernel<fp32>",
                 "launches_per_step": conv_n / args.steps, "avg_launch_ms": round(conv_ms / max(conv_n, 1), 5),

@@ -2072,7 +2072,7 @@ __device__ __forceinline__ void conv_f32_patch_store(const ConvParams &p, floatx
  * next half block's loads spread over this one's taps), the weights' 1 KiB blocks go through a ring
  * of three K-tiles as in conv_f32_direct_kernel.  The nine taps of a half block are straight-line
  * code: every LDS offset and wait count a constant.  The last tiles of an XCD are cut along K as
- * there (conv_tail_parts; a part is whole blocks of 32 planes) and added by the workgroup whose part
+ * there (conv_tail_parts; a part is whole half blocks of 16 planes) and added by the workgroup whose part
  * is ready last (conv_xcd_last_arriver), or, with THHipSumPartsInKernel(0), by
  * conv_f32_patch_tail_finish_kernel. */
 template <int SW, int SH>
@@ -2119,9 +2119,9 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 		tile_m = m0 + local % mw;
 		tile_n = n0 + local / mw;
 	}
-	/* this workgroup's half blocks [hb0, hb1): whole blocks of 32 planes */
-	const int blocks32 = p.Ci / 32;
-	const int hb0 = 2 * (int)((long)blocks32 * split / nsplit), hb1 = 2 * (int)((long)blocks32 * (split + 1) / nsplit);
+	/* this workgroup's half blocks of 16 planes [hb0, hb1) */
+	const int blocks16 = p.Ci / 16;
+	const int hb0 = (int)((long)blocks16 * split / nsplit), hb1 = (int)((long)blocks16 * (split + 1) / nsplit);
 
 	/* ---- what this lane fetches of every plane: elements lane + 64 j of the tile's patches ---- */
 	unsigned voff_[NL];
@@ -2249,9 +2249,10 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 		step(hb, buf_, std::integral_constant<int, 7>{});
 		step(hb, buf_, std::integral_constant<int, 8>{});
 	};
-	for (int hb = hb0; hb < hb1; hb += 2) {	/* (whole blocks of 32 planes: an even number of half blocks) */
+	for (int hb = hb0; hb < hb1; hb += 2) {	/* (a part may be an odd number of half blocks; the first goes to buffer 0) */
 		half_block(hb, C0{});
-		half_block(hb + 1, C1{});
+		if (hb + 1 < hb1)
+			half_block(hb + 1, C1{});
 	}
 	wide_wait<0, false>();	/* (the loads past the end bring zeros into LDS: done before the workgroup ends or the epilogue reuses it) */
 	if (tail_blk >= 0) {
@@ -3174,8 +3175,8 @@ static void conv_launch_f32_patch(ConvParams &p)
 		p.mparts *= 2;
 	if (g_force_mparts)
 		p.mparts = g_force_mparts <= p.tiles_m ? g_force_mparts : 1;
-	/* the tiles an XCD cannot spread evenly over its CUs are cut along K into parts of whole blocks of
-	 * 32 planes (conv_tail_parts; `8 blocks` K-tiles so that conv_tail_plan allows at most one part a block) */
+	/* the tiles an XCD cannot spread evenly over its CUs are cut along K into parts of whole half blocks of
+	 * 16 planes (conv_tail_parts; `8 half blocks` K-tiles so that conv_tail_plan allows at most one part a half block) */
 	static int resident, static_lds, cus;
 	if (!resident) {
 		hipcheck(hipOccupancyMaxActiveBlocksPerMultiprocessor(&resident, conv_f32_patch_kernel<SW, SH>, 256, 0));
@@ -3194,7 +3195,7 @@ static void conv_launch_f32_patch(ConvParams &p)
 	 * eight).  Rounds an XCD needs: whole rounds, plus 1 / parts for the cut tiles or 1 if they cannot be cut. */
 	int use = resident;
 	{
-		const int smax = p.Ci / 32 < g_tail_parts ? p.Ci / 32 : g_tail_parts;
+		const int smax = p.Ci / 16 < g_tail_parts ? p.Ci / 16 : g_tail_parts;
 		double best = 0;
 		for (int r = resident; r >= 3 && r >= resident - 2; r--) {
 			double worst = 1.0;
@@ -3224,7 +3225,7 @@ static void conv_launch_f32_patch(ConvParams &p)
 		if (dyn < 0)
 			dyn = 0;
 	}
-	const size_t maxcnt = conv_tail_plan(p, use, p.Ci / 32 * 8, 64 * 64, 0, true);
+	const size_t maxcnt = conv_tail_plan(p, use, p.Ci / 16 * 8, 64 * 64, 0, true);
 	conv_f32_patch_kernel<SW, SH><<<dim3((unsigned)(8 * maxcnt)), dim3(256), dyn, thhip_stream()>>>(p);
 	if (p.tail_slots)
 		g_tail_launches[!p.tail_inline]++;
