@@ -111,6 +111,10 @@ THFloatTensor *thhip_process_images(THNETWORK *network, unsigned char **images, 
 void thhip_io_free(struct hipnet *hn);
 /* th_load.c */
 int thhip_load_error(void);
+/* hip_rt.hip: which XCD the workgroups of a residue of blockIdx.x % 8 run on (probed once); the flag a
+ * kernel raises when it runs where it must not (an error at the next synchronisation) */
+unsigned thhip_xcd_map(void);
+int *thhip_fault_flag(void);
 void thhip_free_loaded_network(THNETWORK *n);
 
 #endif
