@@ -5,7 +5,8 @@
 One "step" is one THForward of the VGG-16-shape network (fp32, batch 16, 3x224x224,
 synthetic seeded input and weights) with the input already resident in HBM; the
 value is whole-job images/second.  The same run also measures the convolution kernel
-family with HIP events around every launch inside the timed region (-> "roofline"),
+family with HIP events inside the timed region, on the engine's stream: one pair around every run of
+convolution launches that nothing else on the stream interrupts (-> "roofline"),
 times the same network through THProcessFloat call by call as the reference's CLI does
 (-> "process_float": best and mean of at least 20 calls after 2 warm-ups, host
 transfers included), THProcessImages on 64 8-bit images beside the same batch as
@@ -56,11 +57,11 @@ def profile_get(lib, fam):
 
 def timed_forward(lib, net, steps, warmup, families, profiled=True, timed_families=None, reps=1):
     """W untimed + K timed THForward calls; returns ms/step and per-family
-    (ms, launches, work) measured with events around each launch.  profiled=True: the
-    launches of `timed_families` (default: all of `families`) carry their events in the
-    timed steps themselves; the other families, and every family with profiled=False,
-    are measured in K further steps (an event pair costs a few microseconds of stream
-    time per launch, which shows on networks of short kernels).  reps > 1 (the legs under
+    (ms, launches, work) measured with an event pair around every run of launches of one family
+    (no event between two launches of a run: one there costs 3-5 us of stream time, which shows on
+    networks of short kernels).  profiled=True: the launches of `timed_families` (default: all of
+    `families`) carry their events in the timed steps themselves; the other families, and every
+    family with profiled=False, are measured in K further steps.  reps > 1 (the legs under
     "extra" only, never the headline): the K timed steps are run that many times and the
     fastest run counts (a 15 ms run right after a network was built sees the clocks ramp)."""
     if timed_families is None:
@@ -189,7 +190,7 @@ def main():
              "vgg16_other_kernels_ms_per_step": round(fam[3][0] / args.steps, 4),
              "method_of_the_other_networks": "each of the networks below: at least twenty warm-up steps (ten at batch 64), then the fastest of three "
                                              "runs of K steps without events; kernel-family rates from K further "
-                                             "steps with an event around every launch"}
+                                             "steps with an event pair around every run of launches of a family"}
     # the HBM-bound kernels of the same step against the 8 TB/s peak: batched Linear (weights read once)
     # and max pooling (input read + output written once)
     if fam[1][0] > 0:
@@ -291,7 +292,7 @@ def main():
             "conv_i8_TOP/s": round(i8_tops, 2), "frac_of_int8_mfma_peak": round(i8_tops / PEAK_TOPS_INT8_MFMA, 4),
             "dtype": "u8 x u8 -> i32", "workload": "AlexNet-OWT THMakeSpatial form, range 32 (BASELINE configs[4])"}
         # the uint8 convolution family (the eight layers of a step, fc6-8 as one-position convolutions) like `roofline`:
-        # ops = 2 M K N B per launch over the time of the launches (events around each, in a second pass of K steps)
+        # ops = 2 M K N B per launch over the time of the launches (events around the run of them, in a second pass of K steps)
         roofline_int8 = {
             "bound": "mfma", "achieved": round(i8_tops, 3), "peak": PEAK_TOPS_INT8_MFMA, "unit": "TOP/s",
             "frac": round(i8_tops / PEAK_TOPS_INT8_MFMA, 4),

@@ -27,10 +27,15 @@ static void thhip_init_once(void)
 /* (counts how often the stream was handed out: the profiler uses it to see that nothing was put on
  * the stream between two of its launches) */
 static unsigned long g_stream_uses;
+/* the profiler's open run of launches (below): anything else that asks for the stream ends it first */
+static int g_prof_open = -1, g_prof_in_scope;
+static void prof_close_run(void);
 
 hipStream_t thhip_stream(void)
 {
 	thhip_init_once();
+	if (g_prof_open >= 0 && !g_prof_in_scope)
+		prof_close_run();
 	++g_stream_uses;
 	return g_stream;
 }
@@ -236,16 +241,20 @@ extern "C" float thhip_event_ms(int a, int b)
 }
 
 /* ---- per-launch profiler ---- */
-struct ProfRec { int family; hipEvent_t start, stop; double work; bool shared_start; };
+/* One record per run of launches of one family with nothing else on the stream between them: a start event
+ * before the first, a stop event after the last (recorded when something else asks for the stream, or a
+ * launch of another family begins).  No event sits between the launches of a run -- an event between two
+ * dependent kernels costs 3-5 us of stream time, which showed on networks of short kernels -- so a
+ * family's time is what its kernels take as the stream runs them, gaps between them included. */
+struct ProfRec { int family; hipEvent_t start, stop; double work; bool shared_start; long n; };
 static std::vector<ProfRec> g_recs;
 static std::vector<hipEvent_t> g_evpool;
 static int g_prof_on;
 static double g_fam_ms[THHIP_FAM_COUNT], g_fam_work[THHIP_FAM_COUNT];
 static long g_fam_n[THHIP_FAM_COUNT];
 
-/* A launch that follows another profiled launch with nothing put on the stream between them starts
- * at that launch's stop event: one event per launch instead of two (an event costs a few
- * microseconds of stream time, which shows on networks of short kernels). */
+/* A run that follows another run with nothing put on the stream between them starts at that run's stop
+ * event. */
 static hipEvent_t g_last_stop;
 static unsigned long g_last_stop_uses;	/* g_stream_uses right after that event was recorded; 0: none */
 
@@ -262,8 +271,20 @@ static hipEvent_t prof_event(void)
 	return e;
 }
 
+static void prof_close_run(void)
+{
+	if (g_prof_open < 0)
+		return;
+	ProfRec &r = g_recs[g_prof_open];
+	hipcheck(hipEventRecord(r.stop, g_stream));
+	g_last_stop = r.stop;
+	g_last_stop_uses = g_stream_uses;
+	g_prof_open = -1;
+}
+
 static void prof_drain(void)
 {
+	prof_close_run();
 	if (g_recs.empty())
 		return;
 	hipcheck(hipStreamSynchronize(thhip_stream()));
@@ -272,7 +293,7 @@ static void prof_drain(void)
 		hipcheck(hipEventElapsedTime(&ms, g_recs[i].start, g_recs[i].stop));
 		g_fam_ms[g_recs[i].family] += ms;
 		g_fam_work[g_recs[i].family] += g_recs[i].work;
-		g_fam_n[g_recs[i].family]++;
+		g_fam_n[g_recs[i].family] += g_recs[i].n;
 		if (!g_recs[i].shared_start)
 			g_evpool.push_back(g_recs[i].start);
 		g_evpool.push_back(g_recs[i].stop);
@@ -287,6 +308,15 @@ int thhip_prof_begin(int family)
 	/* a negative family: a launch that must not be bracketed (no events made) */
 	if (family < 0 || !g_prof_on || (g_prof_on != 1 && !(g_prof_on & (2 << family))))
 		return -1;
+	if (g_prof_in_scope)
+		return -1;	/* (a bracket inside a bracket is part of the outer one) */
+	if (g_prof_open >= 0 && g_recs[g_prof_open].family == family) {
+		/* the run goes on (anything else on the stream since its last launch would have closed it) */
+		g_recs[g_prof_open].n++;
+		g_prof_in_scope = 1;
+		return g_prof_open;
+	}
+	prof_close_run();
 	if (g_recs.size() >= 4096)
 		prof_drain();
 	ProfRec r;
@@ -300,7 +330,9 @@ int thhip_prof_begin(int family)
 	}
 	r.stop = prof_event();
 	r.work = 0;
+	r.n = 1;
 	g_recs.push_back(r);
+	g_prof_in_scope = 1;
 	return (int)g_recs.size() - 1;
 }
 
@@ -308,10 +340,9 @@ void thhip_prof_end(int token, double work)
 {
 	if (token < 0)
 		return;
-	g_recs[token].work = work;
-	hipcheck(hipEventRecord(g_recs[token].stop, thhip_stream()));
-	g_last_stop = g_recs[token].stop;
-	g_last_stop_uses = g_stream_uses;
+	g_recs[token].work += work;
+	g_prof_in_scope = 0;
+	g_prof_open = token;	/* its stop event: when the run ends */
 }
 
 extern "C" void thhip_profile_enable(int on)
