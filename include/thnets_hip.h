@@ -346,9 +346,13 @@ int THHipImageLayerInFront(int mode);
  * by several workgroups of that XCD (nothing in the reference: its GEMM is one sgemm call per image,
  * modules/SpatialConvolutionMM.c:136-150).  1 (default): the workgroup whose part is ready last adds the
  * parts, in their order, and finishes the tile; the parts meet in the XCD's L2, and every such workgroup
- * checks that it runs on the XCD its position in the grid implies (a violation is reported as an error at
- * the next synchronisation, never as a silently wrong sum).  0: a second launch adds the parts.  The same
- * bits either way.  Read at every launch; returns the previous setting. */
+ * checks that it runs on the XCD its position in the grid implies.  That holds while the engine's kernels
+ * have the GPU's dispatcher to themselves; kernels of another process or stream dispatched at the same time
+ * can break it.  A violation is never a silently wrong sum: it switches this setting to 0 for the rest of
+ * the process, and THProcessFloat / THProcessImages then run their forward pass once more and return the
+ * right values, while a plain synchronisation after THForward reports it as an error (the forward pass
+ * has to be run again by the caller).  0: a second launch adds the parts.  The same bits either way.  Read
+ * at every launch; returns the previous setting. */
 int THHipSumPartsInKernel(int enable);
 /* 0 (default): CAddTable / CSubTable compute what the reference's shipped modules
  * compute (modules/CAddTable.c:59-84: with two inputs CAddTable gives a - b and

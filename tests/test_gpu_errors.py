@@ -99,6 +99,44 @@ lib.THProcessFloat(C.addressof(host.thnet), x.ctypes.data, 1, 8, 8, 3, C.byref(r
 """, "it carries no CPU path")
 
 
+def test_a_fault_reported_by_a_kernel_is_fatal_where_nothing_can_be_repeated():
+    """A kernel that adds the K parts of cut tiles through its XCD's L2 reports, through a flag in page-locked
+    host memory, when it runs on another XCD than its place in the grid implies (hip_rt.hip).  The report is
+    forced from the host here (no kernel misbehaves): at a plain synchronisation it is a fatal error that says
+    what to do."""
+    fatal(r"""
+lib.thhip_fault_flag()[0] = 1
+lib.thhip_sync()
+""", "a kernel reported fault 1")
+
+
+def test_a_fault_reported_by_a_kernel_makes_THProcessFloat_repeat_the_forward(hiplib, oracle):
+    """The same report during THProcessFloat / THProcessImages: the path that raised it is switched off
+    (THHipSumPartsInKernel reads 0 afterwards), the forward pass runs once more and the call returns the
+    same values as without the report."""
+    cfg = cases.small_networks()["tiny_cnn"]
+    net = api.HipNetwork(cfg["layers"], cfg["mean"], cfg["std"])
+    g = cases.rng(4100)
+    imgs = [g.integers(0, 256, (8, 8, 3), dtype=np.uint8) for _ in range(2)]
+    try:
+        want = net.process_float(cfg["input"])
+        want_img = net.process_images(imgs)
+        for call in ("float", "images"):
+            assert hiplib.THHipSumPartsInKernel(1) == 1
+            G.note("a reported fault during THProcess" + call)
+            hiplib.thhip_fault_flag()[0] = 1
+            got = net.process_float(cfg["input"]) if call == "float" else net.process_images(imgs)
+            assert hiplib.thhip_fault_flag()[0] == 0
+            assert np.array_equal(got, want if call == "float" else want_img)
+            assert hiplib.THHipSumPartsInKernel(1) == 0, "the report did not switch the path off"
+        hiplib.thhip_sync()         # nothing is left over for the next synchronisation
+        ref = np.asarray(oracle.run_layers(cfg["layers"], oracle.normalize(cfg["input"], cfg["mean"], cfg["std"])))
+        G.assert_close(got if call == "float" else want, ref.ravel(), 1e-4, "after the repeat")
+    finally:
+        hiplib.THHipSumPartsInKernel(1)
+        net.free()
+
+
 def test_batchnorm_with_too_few_variances_is_fatal():
     body = r"""
 g = cases.rng(5)

@@ -2751,6 +2751,22 @@ static void conv_counters(ConvParams &p, size_t tiles)
 	p.cnt = g_cnt;
 }
 
+/* A workgroup that adds parts in the kernel found itself on another XCD than its place in the grid implies
+ * (kernels of another stream or process were being dispatched beside this one): from now on the parts
+ * are added by the second launch, and the arrival counters, which such a launch may have left anywhere,
+ * start from zero again. */
+extern "C" void thhip_conv_parts_fault(void)
+{
+	static int told;
+	g_tail_inline = 0;
+	if (g_cnt)
+		thhip_memset(g_cnt, 0, g_cnt_n * sizeof(unsigned));
+	if (!told)
+		fprintf(stderr, "thnets HIP engine: the workgroups of a convolution were not spread over the XCDs in grid "
+			"order (other work on this GPU); the K parts of cut tiles are added by a second launch from now on\n");
+	told = 1;
+}
+
 static void conv_scratch(ConvParams &p, size_t tiles, size_t tile_words)
 {
 	const size_t need = tiles * p.splitk * tile_words * sizeof(int);

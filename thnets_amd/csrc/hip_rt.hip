@@ -205,14 +205,40 @@ extern "C" int *thhip_fault_flag(void)
 	return g_fault;
 }
 
+/* A caller that can run its work again (THProcessFloat, THProcessImages) holds the error back, asks
+ * with thhip_fault_take() whether a kernel reported a fault meanwhile and, if so, repeats the forward
+ * pass; everywhere else the report is fatal.  Either way the path that raised it is switched off first
+ * (thhip_conv_parts_fault: the K parts of cut tiles go back to their second launch), so the repeat, or
+ * the caller's next attempt, cannot meet it again. */
+static int g_fault_hold, g_fault_seen;
+
+extern "C" void thhip_fault_hold(int on)
+{
+	g_fault_hold = on != 0;
+}
+
+extern "C" int thhip_fault_take(void)
+{
+	const int code = g_fault_seen;
+	g_fault_seen = 0;
+	return code;
+}
+
 static void fault_check(void)
 {
-	if (g_fault && *(volatile int *)g_fault) {
-		const int code = *(volatile int *)g_fault;
-		*g_fault = 0;
-		THError("thnets HIP engine: a kernel reported fault %d (1: workgroups that share partial sums through "
-			"their XCD's L2 ran on different XCDs; THHipSumPartsInKernel(0) turns that path off)", code);
+	if (!g_fault || !*(volatile int *)g_fault)
+		return;
+	const int code = *(volatile int *)g_fault;
+	*g_fault = 0;
+	thhip_conv_parts_fault();
+	if (g_fault_hold) {
+		g_fault_seen = code;
+		return;
 	}
+	THError("thnets HIP engine: a kernel reported fault %d (1: workgroups that share partial sums through their "
+		"XCD's L2 ran on different XCDs -- other work was running on this GPU; the results since the last "
+		"synchronisation are not valid.  The engine now adds such sums with a second launch, as after "
+		"THHipSumPartsInKernel(0): run the forward pass again)", code);
 }
 
 /* ---- events ---- */

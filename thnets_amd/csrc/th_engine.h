@@ -115,6 +115,10 @@ int thhip_load_error(void);
  * kernel raises when it runs where it must not (an error at the next synchronisation) */
 unsigned thhip_xcd_map(void);
 int *thhip_fault_flag(void);
+/* hip_rt.hip: a caller that can repeat its forward pass holds the error of such a report back (1 / 0) and
+ * asks afterwards whether one came (the fault's code, 0: none) */
+void thhip_fault_hold(int on);
+int thhip_fault_take(void);
 void thhip_free_loaded_network(THNETWORK *n);
 
 #endif

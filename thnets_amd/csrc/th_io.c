@@ -258,10 +258,19 @@ static void normalize_on_host(float *data, int batchsize, int nplanes, long hw, 
 static THFloatTensor *run_and_download(THNETWORK *network, THFloatTensor *dev_in)
 {
 	struct hipnet *hn = (struct hipnet *)network->net;
+	const int lowp = network->net->engine == ENGINE_HIPLOWP;
+	/* A kernel may report that it ran where its results cannot be trusted (hip_rt.hip: thhip_fault_flag;
+	 * the path that depends on it is switched off by the report): the input is still on the device, so the
+	 * forward pass is simply run once more. */
+	thhip_fault_hold(1);
 	THFloatTensor *out = thhip_forward(network->net, dev_in);
-	if (network->net->engine == ENGINE_HIPLOWP)
-		return io_download_result(network, out, THHIP_U8, 1);
-	return io_download_result(network, out, hn->dtype, 0);
+	THFloatTensor *res = io_download_result(network, out, lowp ? THHIP_U8 : hn->dtype, lowp);
+	thhip_fault_hold(0);
+	if (thhip_fault_take()) {
+		out = thhip_forward(network->net, dev_in);
+		res = io_download_result(network, out, lowp ? THHIP_U8 : hn->dtype, lowp);
+	}
+	return res;
 }
 
 /* The engine's body of THProcessFloat (thapi.c:363-450): `data` is [batchsize][nplanes]
@@ -293,9 +302,16 @@ THFloatTensor *thhip_process_float(THNETWORK *network, float *data, int batchsiz
 		thhip_quantize((const float *)dev->storage->data, (unsigned char *)in->storage->data, cnt,
 			&hn->cur_mult, &hn->cur_sub);
 	}
+	thhip_fault_hold(1);	/* (as in run_and_download) */
 	THFloatTensor *out = thhip_forward(network->net, in);
 	normalize_on_host(data, batchsize, nplanes, hw, network->mean, network->std);
-	return io_download_result(network, out, lowp ? THHIP_U8 : hn->dtype, lowp);
+	THFloatTensor *res = io_download_result(network, out, lowp ? THHIP_U8 : hn->dtype, lowp);
+	thhip_fault_hold(0);
+	if (thhip_fault_take()) {
+		out = thhip_forward(network->net, in);
+		res = io_download_result(network, out, lowp ? THHIP_U8 : hn->dtype, lowp);
+	}
+	return res;
 }
 
 /* The engine's body of THProcessImages (thapi.c:452-563): interleaved 8-bit images

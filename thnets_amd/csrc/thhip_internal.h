@@ -16,6 +16,9 @@ hipStream_t thhip_stream(void);
 #define THHIP_GETREG_XCC_ID ((3 << 11) | 20)
 extern "C" unsigned thhip_xcd_map(void);	/* hip_rt.hip: which XCD the workgroups of a residue of blockIdx.x % 8 run on */
 extern "C" int *thhip_fault_flag(void);		/* hip_rt.hip: set by a kernel, turned into an error at the next synchronisation */
+extern "C" void thhip_fault_hold(int on);	/* hip_rt.hip: 1: the error is held back for thhip_fault_take() */
+extern "C" int thhip_fault_take(void);		/* hip_rt.hip: the fault reported while errors were held back (0: none); clears it */
+extern "C" void thhip_conv_parts_fault(void);	/* conv_mfma.hip: what a report of fault 1 switches off */
 
 /* Profiling hooks: bracket one kernel launch.  `work` is the algorithmic
  * work of the launch (flops for GEMM-like kernels, bytes otherwise). */
