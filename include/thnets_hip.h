@@ -345,11 +345,12 @@ int THHipImageLayerInFront(int mode);
 /* fp32 convolutions cut the tiles an XCD could not spread evenly over its CUs into parts along K, computed
  * by several workgroups of that XCD (nothing in the reference: its GEMM is one sgemm call per image,
  * modules/SpatialConvolutionMM.c:136-150).  1 (default): the workgroup whose part is ready last adds the
- * parts, in their order, and finishes the tile; the parts meet in the XCD's L2, and every such workgroup
- * checks that it runs on the XCD its position in the grid implies.  That holds while the engine's kernels
- * have the GPU's dispatcher to themselves; kernels of another process or stream dispatched at the same time
- * can break it.  A violation is never a silently wrong sum: it switches this setting to 0 for the rest of
- * the process, and THProcessFloat / THProcessImages then run their forward pass once more and return the
+ * parts, in their order, and finishes the tile; the parts meet in the XCD's L2.  That is right while the
+ * hardware hands workgroup b of a launch to XCD (b + r) % 8 with one r for the whole launch (r itself
+ * changes as queues come and go: other streams, other processes), which every launch checks for itself:
+ * its part workgroups record the r they see, and the one that finishes a tile looks at the record.  A
+ * launch that saw two is never a silently wrong sum: it switches this setting to 0 for the rest of the
+ * process, and THProcessFloat / THProcessImages then run their forward pass once more and return the
  * right values, while a plain synchronisation after THForward reports it as an error (the forward pass
  * has to be run again by the caller).  0: a second launch adds the parts.  The same bits either way.  Read
  * at every launch; returns the previous setting. */

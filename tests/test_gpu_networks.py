@@ -234,6 +234,52 @@ def test_process_images_matches_process_float(hiplib, oracle):
     net.free()
 
 
+def test_process_float_uploads_a_large_batch_in_windows(hiplib, oracle):
+    """THProcessFloat on eight images of 4.8 MB: the batch goes up in three pieces and the first two
+    convolutions (with their Threshold and pooling) work on a piece while the next one crosses the link
+    (thhip_forward_windows).  Against the oracle, fp32 and fp16; a network whose first modules run a
+    kernel that knows no window (a 3x3 / stride 2 pooling after the image layer) is noticed: that call, and
+    the ones after it, run on the whole batch and give the right values too."""
+    g = cases.rng(8800)
+    def w(co, ci, k):
+        return g.standard_normal((co, ci, k, k), dtype=np.float32) * np.float32(np.sqrt(2.0 / (ci * k * k)))
+    def b(n):
+        return g.standard_normal(n, dtype=np.float32) * np.float32(0.1)
+    bn = dict(type="bn", weight=g.uniform(0.5, 1.5, 64).astype(np.float32), bias=b(64),
+              running_mean=b(64), running_var=g.uniform(0.5, 1.5, 64).astype(np.float32), eps=1e-5)
+    layers = [netbuild.conv(w(32, 3, 3), b(32), 1, 1), netbuild.relu(),
+              netbuild.conv(w(64, 32, 3), b(64), 1, 1), bn, netbuild.relu(), netbuild.maxpool(2, 2),
+              netbuild.conv(w(8, 64, 3), b(8), 1, 1), netbuild.relu(), netbuild.maxpool(2, 2)]
+    mean, std = [0.485, 0.456, 0.406], [0.229, 0.224, 0.225]
+    x = g.uniform(0, 1, (8, 3, 224, 224)).astype(np.float32)
+    want = np.asarray(oracle.run_layers(layers, oracle.normalize(x, mean, std))).ravel()
+    for kw, tol in (({}, 1e-4), ({"half": 1}, 3e-2)):
+        net = api.HipNetwork(layers, mean, std, **kw)
+        before = hiplib.thhip_windowed_forwards()
+        G.note("THProcessFloat in windows %s" % (kw,))
+        x0 = x.copy()
+        got = net.process_float(x0)
+        assert hiplib.thhip_windowed_forwards() == before + 1, "the batch was not run in windows"
+        G.assert_close(got, want, tol, "in windows %s" % (kw,))
+        again = net.process_float(x)
+        assert np.array_equal(got, again)
+        net.free()
+    # a 3x3 / stride 2 pooling after the image layer: its kernels take no window
+    layers = [netbuild.conv(w(32, 3, 3), b(32), 1, 1), netbuild.relu(), netbuild.maxpool(3, 2),
+              netbuild.conv(w(64, 32, 3), b(64), 1, 1), netbuild.relu(), netbuild.maxpool(2, 2),
+              netbuild.conv(w(8, 64, 3), b(8), 1, 1), netbuild.relu()]
+    want = np.asarray(oracle.run_layers(layers, oracle.normalize(x, mean, std))).ravel()
+    for kw, tol in (({}, 1e-4), ({"half": 1}, 3e-2)):
+        net = api.HipNetwork(layers, mean, std, **kw)
+        before = hiplib.thhip_windowed_forwards()
+        G.note("THProcessFloat, a module of the prefix without a window %s" % (kw,))
+        got = net.process_float(x)
+        G.assert_close(got, want, tol, "whole batch after the window was ignored %s" % (kw,))
+        assert np.array_equal(net.process_float(x), got)
+        assert hiplib.thhip_windowed_forwards() == before
+        net.free()
+
+
 def test_vgg16_full_size_properties(hiplib, oracle):
     """Full configuration 3 (batch 16, 224x224): too large for the CPU checker inside a
     test, so check size-independent properties: batch == images one by one, and the

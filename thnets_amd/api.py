@@ -29,6 +29,7 @@ TEST_HOOKS = {
     "thhip_conv_set_ktile": (None, [C.c_int]),
     "thhip_conv_set_tail_parts": (None, [C.c_int]),
     "thhip_xcd_map": (C.c_uint, []),
+    "thhip_windowed_forwards": (C.c_long, []),
     "thhip_fault_flag": (C.POINTER(C.c_int), []),
     "thhip_conv_cut_launches": (C.c_long, [C.c_int]),
     "thhip_conv_set_xcd_parts": (None, [C.c_int]),

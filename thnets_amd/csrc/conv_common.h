@@ -49,7 +49,8 @@ struct ConvParams {
 	int tail_tiles;		/* most cut tiles of an XCD */
 	int tail_round;		/* 1: an XCD with less than one whole round of tiles is left uncut */
 	int tail_inline;	/* 1: the part of a cut tile that arrives last adds the parts and finishes the tile (cnt) */
-	unsigned xcd_map;	/* thhip_xcd_map() */
+	unsigned *rot;		/* [64] device words, one per launch in flight: the set of (XCC id - blockIdx.x) % 8 its part workgroups saw */
+	int rot_slot, rot_clear;	/* this launch's word, and the word a later launch will use (cleared by this one) */
 	int *fault;		/* thhip_fault_flag() */
 	/* conv_f32_direct_kernel with a K split of the whole layer: a max pooling that follows, taken by the kernel
 	 * that adds the parts (pk_kH 0: none); pk_oH x pk_oW is the pooled plane */

@@ -829,30 +829,51 @@ __device__ inline void conv_xcd_rect(const ConvParams &p, int xcd, int &m0, int 
 	cnt = mw * (n1 - n0);
 }
 
-/* The parts of a cut tile are computed by workgroups of one XCD (workgroup b runs on XCD b % 8), which
- * share that XCD's L2: a part's sums need only reach L2 (the vector caches write through; the wait for
- * the stores' acknowledgement is the release) before the ticket is drawn there (an atomic without the
- * device-scope bit executes in the XCD's L2), and the workgroup that draws the last ticket reads them
- * from L2.  No L2 write-back or invalidate as a device-scope fence would do (measured with those, and
- * with device-scope loads and stores of the parts: slower than a second launch; this way ResNet-18 batch
- * 32 1.269 -> 1.239 ms and VGG-16 batch 16 3.825 -> 3.803 ms against the second launch.  The parts of a
- * layer whose whole K is split stay with their second launch: every tile's last workgroup adding parts
- * cost 8 us a layer more than it).  Returns whether this
- * workgroup drew the last of `parts` tickets (and has reset the counter for the next launch); `slot`
- * is one int of LDS nobody else uses until the next barrier after the call. */
+/* The parts of a cut tile are computed by workgroups whose blockIdx.x agree modulo 8, and the hardware
+ * hands workgroup b of a launch to XCD (b + r) % 8 -- r is the same for every workgroup of a launch, but
+ * changes from launch to launch when queues are created or mapped anew (another stream, another process)
+ * -- so they run on one XCD and share its L2: a part's sums need only reach L2 (the vector caches write
+ * through; the wait for the stores' acknowledgement is the release) before the ticket is drawn there (an
+ * atomic without the device-scope bit executes in the XCD's L2), and the workgroup that draws the last
+ * ticket reads them from L2.  No L2 write-back or invalidate as a device-scope fence would do (measured with
+ * those, and with device-scope loads and stores of the parts: slower than a second launch; this way
+ * ResNet-18 batch 32 1.269 -> 1.239 ms and VGG-16 batch 16 3.825 -> 3.803 ms against the second launch.
+ * The parts of a layer whose whole K is split stay with their second launch: every tile's last workgroup
+ * adding parts cost 8 us a layer more than it).
+ *
+ * That every part workgroup of the launch saw the same r is checked, not assumed: each of them ORs
+ * 1 << r into the launch's word of p.rot when it starts (conv_xcd_report: a device-scope atomic nobody waits
+ * for; it is complete before the workgroup draws its ticket, whose release waits for everything the
+ * wavefront has outstanding), and the workgroup that draws a tile's last ticket reads the word: more than
+ * one bit, and the host hears of it (p.fault; hip_rt.hip turns that into a repeat or an error). */
+__device__ __forceinline__ void conv_xcd_report(const ConvParams &p, bool part)
+{
+	if (threadIdx.x != 0)
+		return;
+	if (part) {
+		const unsigned r = ((unsigned)__builtin_amdgcn_s_getreg(THHIP_GETREG_XCC_ID) - blockIdx.x) & 7u;
+		__hip_atomic_fetch_or(p.rot + p.rot_slot, 1u << r, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+	}
+	if (blockIdx.x == 0)	/* the word of a launch to come (this launch's was cleared as long ago) */
+		__hip_atomic_store(p.rot + p.rot_clear, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+/* Returns whether this workgroup drew the last of `parts` tickets (and has reset the counter for the next
+ * launch); `slot` is one int of LDS nobody else uses until the next barrier after the call. */
 __device__ __forceinline__ bool conv_xcd_last_arriver(const ConvParams &p, unsigned *counter, int parts, int *slot)
 {
-	/* (on the XCD the map names for this residue of blockIdx.x, or the host hears of it) */
-	if (threadIdx.x == 0 && (int)__builtin_amdgcn_s_getreg(THHIP_GETREG_XCC_ID) != (int)((p.xcd_map >> (4 * (blockIdx.x & 7))) & 7u))
-		__hip_atomic_store(p.fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
 	__builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
 	__syncthreads();
 	if (threadIdx.x == 0)
 		*slot = (int)__hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 	__syncthreads();
 	const bool last = *slot == parts - 1;
-	if (last && threadIdx.x == 0)
+	if (last && threadIdx.x == 0) {
 		*counter = 0;
+		const unsigned seen = __hip_atomic_load(p.rot + p.rot_slot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		if (seen & (seen - 1))
+			__hip_atomic_store(p.fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+	}
 	__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 	return last;
 }
@@ -1618,6 +1639,8 @@ __device__ __forceinline__ void conv_f32_direct_body(const ConvParams &p, const 
 				tail_blk = (long)xcd * p.tail_cap + t * s + split;
 			}
 		}
+		if (p.tail_inline)
+			conv_xcd_report(p, tail_blk >= 0);
 		if (local >= cnt)
 			return;
 		tile_m = m0 + local % mw;
@@ -2114,6 +2137,8 @@ __global__ __launch_bounds__(256) void conv_f32_patch_kernel(ConvParams p)
 				tail_blk = (long)xcd * p.tail_cap + t * s + split;
 			}
 		}
+		if (p.tail_inline)
+			conv_xcd_report(p, tail_blk >= 0);
 		if (local >= cnt)
 			return;
 		tile_m = m0 + local % mw;
@@ -2734,7 +2759,7 @@ extern "C" void thhip_conv_set_tuning(int bm, int bn, int splitk, int wgs_per_cu
 /* Split-K scratch: partial tiles and arrival counters (grow-only). */
 static int *g_ws;
 static size_t g_ws_bytes;
-static unsigned *g_cnt;
+static unsigned *g_cnt, *g_cnt_rot;
 static size_t g_cnt_n;
 
 /* Points p.cnt at `tiles` arrival counters, zero between launches (the workgroup that draws a tile's last
@@ -2748,22 +2773,27 @@ static void conv_counters(ConvParams &p, size_t tiles)
 		g_cnt = (unsigned *)thhip_malloc(g_cnt_n * sizeof(unsigned));
 		thhip_memset(g_cnt, 0, g_cnt_n * sizeof(unsigned));
 	}
+	if (!g_cnt_rot) {	/* (conv_xcd_report's words, one per launch in flight) */
+		g_cnt_rot = (unsigned *)thhip_malloc(64 * sizeof(unsigned));
+		thhip_memset(g_cnt_rot, 0, 64 * sizeof(unsigned));
+	}
 	p.cnt = g_cnt;
 }
 
-/* A workgroup that adds parts in the kernel found itself on another XCD than its place in the grid implies
- * (kernels of another stream or process were being dispatched beside this one): from now on the parts
- * are added by the second launch, and the arrival counters, which such a launch may have left anywhere,
- * start from zero again. */
+/* The part workgroups of a launch did not all see the same offset between their place in the grid and the
+ * XCD they ran on: from now on the parts are added by the second launch, and the arrival counters, which
+ * such a launch may have left anywhere, start from zero again. */
 extern "C" void thhip_conv_parts_fault(void)
 {
 	static int told;
 	g_tail_inline = 0;
 	if (g_cnt)
 		thhip_memset(g_cnt, 0, g_cnt_n * sizeof(unsigned));
+	if (g_cnt_rot)
+		thhip_memset(g_cnt_rot, 0, 64 * sizeof(unsigned));
 	if (!told)
-		fprintf(stderr, "thnets HIP engine: the workgroups of a convolution were not spread over the XCDs in grid "
-			"order (other work on this GPU); the K parts of cut tiles are added by a second launch from now on\n");
+		fprintf(stderr, "thnets HIP engine: the workgroups of a convolution were not handed to the XCDs in one "
+			"order; the K parts of cut tiles are added by a second launch from now on\n");
 	told = 1;
 }
 
@@ -2955,8 +2985,12 @@ static size_t conv_tail_plan(ConvParams &p, int resident, int nkt, size_t tile_f
 		conv_f32_scratch(p, (size_t)8 * p.tail_cap * tile_floats * sizeof(float));
 		p.tail_inline = inline_ok && g_tail_inline && (thhip_xcd_map() >> 31);
 		if (p.tail_inline) {
+			static unsigned seq;
 			conv_counters(p, (size_t)8 * p.tail_cap);
-			p.xcd_map = thhip_xcd_map();
+			p.rot = g_cnt_rot;
+			p.rot_slot = (int)(seq & 63);
+			p.rot_clear = (int)((seq + 32) & 63);
+			seq++;
 			p.fault = thhip_fault_flag();
 		}
 	}
@@ -3669,8 +3703,17 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 		THError("thhip_conv2d: one image exceeds 2 GiB");
 	if ((long)oH * oW * bmax > (1L << 30))
 		bmax = (1L << 30) / ((long)oH * oW);
-	for (int b0 = 0; b0 < B; b0 += (int)bmax) {
-		const int bn = B - b0 < bmax ? B - b0 : (int)bmax;
+	/* a window of the batch (hip_rt.hip: thhip_batch_window): the images of the window only */
+	int win0 = 0;
+	int winn = thhip_batch_window_get(&win0);
+	if (winn && (f_pk || f_front || u8)) {	/* (these take the batch in one piece: the caller hears of it) */
+		thhip_batch_window_violate();
+		winn = 0;
+	}
+	const int bfirst = winn ? (win0 < B ? win0 : B) : 0, bend = winn ? (win0 + winn < B ? win0 + winn : B) : B;
+	thhip_batch_window_scope(1);
+	for (int b0 = bfirst; b0 < bend; b0 += (int)bmax) {
+		const int bn = bend - b0 < bmax ? bend - b0 : (int)bmax;
 		ConvParams p;
 		memset(&p, 0, sizeof(p));
 		p.x = (const char *)x + (size_t)b0 * in_img * esize;
@@ -3790,6 +3833,7 @@ static void conv_run(const void *x, const void *wpacked, const float *scale, con
 		g_pair_fresh = 0;
 		g_pair_mode = 0;	/* (only the call right after thhip_conv_pair_begin may be held back) */
 	}
+	thhip_batch_window_scope(0);
 }
 
 extern "C" void thhip_conv2d_affine(const void *x, const void *wpacked, const float *scale, const float *shift, void *y,

@@ -31,13 +31,55 @@ static unsigned long g_stream_uses;
 static int g_prof_open = -1, g_prof_in_scope;
 static void prof_close_run(void);
 
+/* The batch window (below): a launch made while one is set, outside the code that honours it, is noted */
+static int g_win_b0, g_win_n, g_win_scope, g_win_violated;
+
 hipStream_t thhip_stream(void)
 {
 	thhip_init_once();
 	if (g_prof_open >= 0 && !g_prof_in_scope)
 		prof_close_run();
+	if (g_win_n && !g_win_scope)
+		g_win_violated = 1;
 	++g_stream_uses;
 	return g_stream;
+}
+
+/* ---- a window of the batch ----
+ * THProcessFloat uploads a large batch in pieces and lets the first modules of the network run on the
+ * images of a piece while the next one crosses the link.  Those modules run on the tensors of the whole
+ * batch; while a window [b0, b0 + n) is set, the convolution entry points (conv_run, conv_mfma.hip) launch
+ * their kernels on those images only.  Anything else that puts work on the stream while a window is set
+ * would have processed the whole batch: it is noted, and the caller then runs the modules again on the
+ * whole batch, without a window. */
+extern "C" void thhip_batch_window(int b0, int n)
+{
+	g_win_b0 = b0;
+	g_win_n = n > 0 ? n : 0;
+	g_win_scope = 0;
+}
+
+extern "C" int thhip_batch_window_get(int *b0)
+{
+	*b0 = g_win_b0;
+	return g_win_n;
+}
+
+extern "C" void thhip_batch_window_scope(int on)
+{
+	g_win_scope = on != 0;
+}
+
+extern "C" void thhip_batch_window_violate(void)
+{
+	g_win_violated = 1;
+}
+
+extern "C" int thhip_batch_window_violated(void)
+{
+	const int v = g_win_violated;
+	g_win_violated = 0;
+	return v;
 }
 
 extern "C" int thhip_device_count(void)
@@ -121,6 +163,37 @@ extern "C" void thhip_memcpy_d2h_async(void *dst_pinned, const void *src, size_t
 	hipcheck(hipMemcpyAsync(dst_pinned, src, bytes, hipMemcpyDeviceToHost, thhip_stream()));
 }
 
+/* Host -> device copies on a stream of their own, each followed by an event the engine's stream can be
+ * made to wait for: a piece of a batch crosses the link while kernels work on the piece before it.  The
+ * caller keeps the destination away from the engine's stream until that stream has waited for the event. */
+#define THHIP_COPY_EVENTS 8
+static hipStream_t g_copy_stream;
+static hipEvent_t g_copy_events[THHIP_COPY_EVENTS];
+
+extern "C" void thhip_memcpy_h2d_piece(void *dst, const void *src_pinned, size_t bytes, int event)
+{
+	thhip_init_once();
+	if (event < 0 || event >= THHIP_COPY_EVENTS)
+		THError("thhip_memcpy_h2d_piece: event %d out of range", event);
+	if (!g_copy_stream) {
+		++g_alloc_calls;
+		hipcheck(hipStreamCreate(&g_copy_stream));
+	}
+	if (!g_copy_events[event]) {
+		++g_alloc_calls;
+		hipcheck(hipEventCreateWithFlags(&g_copy_events[event], hipEventDisableTiming));
+	}
+	hipcheck(hipMemcpyAsync(dst, src_pinned, bytes, hipMemcpyHostToDevice, g_copy_stream));
+	hipcheck(hipEventRecord(g_copy_events[event], g_copy_stream));
+}
+
+extern "C" void thhip_wait_h2d_piece(int event)
+{
+	if (event < 0 || event >= THHIP_COPY_EVENTS || !g_copy_events[event])
+		THError("thhip_wait_h2d_piece: event %d not recorded", event);
+	hipcheck(hipStreamWaitEvent(thhip_stream(), g_copy_events[event], 0));
+}
+
 extern "C" void thhip_memcpy_d2d(void *dst, const void *src, size_t bytes)
 {
 	hipcheck(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, thhip_stream()));
@@ -152,19 +225,20 @@ extern "C" void thhip_sync(void)
 
 /* ---- which XCD a workgroup runs on ----
  * The convolution kernels let the workgroups that compute the parts of one tile meet in their XCD's L2
- * (conv_xcd_last_arriver), which is right only if those workgroups -- all of one residue of
- * blockIdx.x modulo 8 -- run on one XCD.  The hardware hands workgroup b to XCD b % 8; this is checked
- * once per process on a grid of 4096 workgroups (thhip_xcd_map), and again by every such workgroup
- * against the map (a mismatch raises the flag below, which the next synchronisation turns into an
- * error). */
+ * (conv_xcd_last_arriver), which is right only if those workgroups -- all of one residue of blockIdx.x
+ * modulo 8 -- run on one XCD.  The hardware hands workgroup b of a launch to XCD (b + r) % 8, with r fixed
+ * for the launch (it changes when queues are created: measured on one stream, 0, then 7, 6, 5 as three more
+ * streams were made).  Whether the GPU does so at all is checked here once per process on a grid of 4096
+ * workgroups; that every launch did is checked by its own workgroups (conv_xcd_report), and a launch that
+ * did not raises the flag below, which the next synchronisation turns into a repeat or an error. */
 __global__ void xcd_probe_kernel(int *out)
 {
 	if (threadIdx.x == 0)
 		out[blockIdx.x] = __builtin_amdgcn_s_getreg(THHIP_GETREG_XCC_ID);
 }
 
-/* 0x80000000 | the XCC id (0 .. 7) of residue r in bits 4 r .. 4 r + 2; 0 if the workgroups of a residue were
- * seen on different XCDs (then nothing may rely on it). */
+/* 0x80000000 | r if workgroup b of the probe ran on XCD (b + r) % 8 for every b; 0 if not (then nothing
+ * may rely on it). */
 extern "C" unsigned thhip_xcd_map(void)
 {
 	static unsigned map;
@@ -179,15 +253,10 @@ extern "C" unsigned thhip_xcd_map(void)
 	hipcheck(hipMemcpyAsync(host.data(), dev, n * sizeof(int), hipMemcpyDeviceToHost, thhip_stream()));
 	hipcheck(hipStreamSynchronize(thhip_stream()));
 	thhip_free(dev);
-	bool ok = true;
+	bool ok = (unsigned)host[0] < 8u;
 	for (int b = 0; b < n; b++)
-		ok = ok && host[b] == host[b & 7] && (unsigned)host[b] < 8u;
-	map = 0;
-	if (ok) {
-		map = 0x80000000u;
-		for (int r = 0; r < 8; r++)
-			map |= (unsigned)host[r] << (4 * r);
-	}
+		ok = ok && host[b] == ((host[0] + b) & 7);
+	map = ok ? 0x80000000u | (unsigned)host[0] : 0;
 	done = 1;
 	return map;
 }
@@ -235,8 +304,8 @@ static void fault_check(void)
 		g_fault_seen = code;
 		return;
 	}
-	THError("thnets HIP engine: a kernel reported fault %d (1: workgroups that share partial sums through their "
-		"XCD's L2 ran on different XCDs -- other work was running on this GPU; the results since the last "
+	THError("thnets HIP engine: a kernel reported fault %d (1: the workgroups of a launch that share partial sums "
+		"through their XCD's L2 were not handed to the XCDs in one order; the results since the last "
 		"synchronisation are not valid.  The engine now adds such sums with a second launch, as after "
 		"THHipSumPartsInKernel(0): run the forward pass again)", code);
 }

@@ -949,12 +949,20 @@ void thhip_materialize_output(struct network *net, int idx)
  * clFinish (thapi.c:213-216), so the printed seconds are kernel time. */
 static int g_run_depth;	/* 1 while the top-level module list runs, more inside containers */
 
+static THFloatTensor *run_modules(struct network *net, THFloatTensor *in, int first, int last);
+
 static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
 {
-	double t = 0;
 	((struct hipnet *)net)->cur_cl = 0;	/* inputs arrive in the reference's plane-major order */
+	return run_modules(net, in, 0, net->nelem);
+}
+
+/* modules [first, last) of the list, the first of them on `in` */
+static THFloatTensor *run_modules(struct network *net, THFloatTensor *in, int first, int last)
+{
+	double t = 0;
 	g_run_depth++;
-	for (int i = 0; i < net->nelem; i++) {
+	for (int i = first; i < last; i++) {
 		struct module *m = &net->modules[i];
 		if (th_profile) {
 			thhip_sync();
@@ -1017,6 +1025,72 @@ static THFloatTensor *run_network(struct network *net, THFloatTensor *in)
 	}
 	g_run_depth--;
 	return in;
+}
+
+/* How many leading modules of the list work image by image on kernels that honour a window of the batch
+ * (thhip_batch_window): the first two convolutions with what follows each of them up to the third.  0:
+ * none (a graph, a list that does not start that way, or nothing after them). */
+static int window_prefix(struct network *net)
+{
+	int convs = 0, i;
+	if (((struct hipnet *)net)->dag || net->engine != ENGINE_HIP)
+		return 0;
+	for (i = 0; i < net->nelem; i++) {
+		const int type = net->modules[i].type;
+		if (net->modules[i].ninputs)
+			return 0;
+		if (is_conv_type(type)) {
+			if (convs == 2)
+				break;
+			convs++;
+		} else if (type != MT_Threshold && type != MT_SpatialMaxPooling && type != MT_SpatialBatchNormalization &&
+			   type != MT_Dropout)
+			break;
+	}
+	return convs && i < net->nelem ? i : 0;
+}
+
+/* forward passes so far whose first modules ran window by window (for the tests) */
+static long g_windowed_forwards;
+long thhip_windowed_forwards(void)
+{
+	return g_windowed_forwards;
+}
+
+/* thhip_forward, the first modules window by window: before(ctx, w) makes the images of window w ready
+ * (their upload may still be on its way while the window before is worked on).  Where the list does not
+ * allow it, or a module of the prefix turns out to launch something that works on the whole batch (noted
+ * by hip_rt.hip; remembered for the network), every window is made ready first and the list runs on the
+ * whole batch as thhip_forward runs it: what the first window's launches wrote is written again. */
+THFloatTensor *thhip_forward_windows(struct network *net, THFloatTensor *in, int nwin, const int *b0, const int *bn,
+	void (*before)(void *ctx, int w), void *ctx)
+{
+	struct hipnet *hn = (struct hipnet *)net;
+	const int prefix = nwin > 1 && !hn->no_windows && !th_profile && !th_minmax && !th_debug ? window_prefix(net) : 0;
+	int w = 0;
+	if (prefix) {
+		THFloatTensor *x = in;
+		thhip_batch_window_violated();
+		for (; w < nwin; w++) {
+			before(ctx, w);
+			thhip_batch_window(b0[w], bn[w]);
+			hn->cur_cl = 0;
+			x = run_modules(net, in, 0, prefix);
+			thhip_batch_window(0, 0);
+			if (thhip_batch_window_violated()) {
+				hn->no_windows = 1;
+				w++;
+				break;
+			}
+		}
+		if (!hn->no_windows) {
+			g_windowed_forwards++;
+			return run_modules(net, x, prefix, net->nelem);
+		}
+	}
+	for (; w < nwin; w++)
+		before(ctx, w);
+	return thhip_forward(net, in);
 }
 
 THFloatTensor *thhip_forward(struct network *net, THFloatTensor *in)

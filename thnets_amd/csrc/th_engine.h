@@ -89,6 +89,7 @@ struct hipnet {
 	float cur_mult, cur_sub;	/* uint8 engine: quantisation of the tensor in flight */
 	int cur_cl;		/* uint8 engine: the tensor in flight is channels-last in memory */
 	int dag;		/* modules name their inputs (ninputs / inputs[]): the list is a graph */
+	int no_windows;		/* the first modules do not all honour a window of the batch (found on the first try) */
 	struct hipio io;
 };
 
@@ -119,6 +120,17 @@ int *thhip_fault_flag(void);
  * asks afterwards whether one came (the fault's code, 0: none) */
 void thhip_fault_hold(int on);
 int thhip_fault_take(void);
+/* hip_rt.hip: a window of the batch for the convolution entry points (0 images: none); whether anything
+ * was launched outside them while one was set (clears the note); a host -> device copy on the copy stream
+ * followed by event `event`, and the engine's stream made to wait for that event */
+void thhip_batch_window(int b0, int n);
+int thhip_batch_window_violated(void);
+void thhip_memcpy_h2d_piece(void *dst, const void *src_pinned, size_t bytes, int event);
+void thhip_wait_h2d_piece(int event);
+/* th_engine.c: thhip_forward with the first modules run window by window; before(ctx, w) is called
+ * before the modules see window w (to make its images ready) */
+THFloatTensor *thhip_forward_windows(struct network *net, THFloatTensor *in, int nwin, const int *b0, const int *bn,
+	void (*before)(void *ctx, int w), void *ctx);
 void thhip_free_loaded_network(THNETWORK *n);
 
 #endif

@@ -19,6 +19,9 @@ extern "C" int *thhip_fault_flag(void);		/* hip_rt.hip: set by a kernel, turned 
 extern "C" void thhip_fault_hold(int on);	/* hip_rt.hip: 1: the error is held back for thhip_fault_take() */
 extern "C" int thhip_fault_take(void);		/* hip_rt.hip: the fault reported while errors were held back (0: none); clears it */
 extern "C" void thhip_conv_parts_fault(void);	/* conv_mfma.hip: what a report of fault 1 switches off */
+extern "C" int thhip_batch_window_get(int *b0);	/* hip_rt.hip: the images [b0, b0 + n) the convolutions are to work on (n = 0: all) */
+extern "C" void thhip_batch_window_scope(int on);	/* hip_rt.hip: 1 while code that honours the window launches */
+extern "C" void thhip_batch_window_violate(void);	/* hip_rt.hip: this call works on the whole batch in spite of a window */
 
 /* Profiling hooks: bracket one kernel launch.  `work` is the algorithmic
  * work of the launch (flops for GEMM-like kernels, bytes otherwise). */
@@ -64,6 +67,8 @@ void thhip_conv_set_ktile(int chunks);
  * kernel (results do not depend on timing).  Default 8, which is also the most
  * that is used; 1 = never cut.  Tests and tuning. */
 void thhip_conv_set_tail_parts(int parts);
+/* th_engine.c: forward passes so far whose first modules ran window by window under THProcessFloat */
+long thhip_windowed_forwards(void);
 /* launches so far whose cut tiles were added in the kernel (0) / by a second launch (1) */
 long thhip_conv_cut_launches(int second_launch);
 /* Force how the tile grid is cut over the eight XCDs: the M tiles into
