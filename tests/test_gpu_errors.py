@@ -101,7 +101,7 @@ lib.THProcessFloat(C.addressof(host.thnet), x.ctypes.data, 1, 8, 8, 3, C.byref(r
 
 def test_a_fault_reported_by_a_kernel_is_fatal_where_nothing_can_be_repeated():
     """A kernel that adds the K parts of cut tiles through its XCD's L2 reports, through a flag in page-locked
-    host memory, when it runs on another XCD than its place in the grid implies (hip_rt.hip).  The report is
+    host memory, when the workgroups of its launch were not handed to the XCDs in one order (hip_rt.hip).  The report is
     forced from the host here (no kernel misbehaves): at a plain synchronisation it is a fatal error that says
     what to do."""
     fatal(r"""

@@ -947,10 +947,10 @@ def test_conv_f32_cut_tiles_added_in_the_kernel(hiplib, oracle):
     bits, on both fp32 kernels that cut tiles (3x3 / stride 1 from a patch in LDS; strided and 1x1 layers with
     tiles loaded straight into LDS), with the folded factor and Threshold, with a table add, with the 2x2
     pooling; every case three times in a row (the arrival counters are left at zero).  One case against the
-    restatement.  The workgroups of every residue of blockIdx.x % 8 were seen on one XCD."""
+    restatement.  The probe launch saw workgroup b on XCD (b + r) % 8 for every b."""
     from thnets_amd import api
     g = cases.rng(7700)
-    assert hiplib.thhip_xcd_map() >> 31, "workgroups of one residue of blockIdx.x % 8 on different XCDs"
+    assert hiplib.thhip_xcd_map() >> 31, "the workgroups of the probe launch were not handed to the XCDs in order"
     shapes = [(32, 64, 56, 56, 64, 3, 1, 1), (24, 64, 56, 56, 128, 3, 1, 1), (44, 64, 28, 28, 256, 3, 1, 1), (12, 128, 64, 32, 128, 3, 1, 1),
               (32, 64, 56, 56, 128, 3, 2, 1), (16, 64, 40, 40, 128, 5, 1, 2), (9, 64, 75, 77, 64, 3, 1, 1), (32, 128, 56, 56, 128, 3, 2, 1)]
     cut = [0, 0]        # launches with cut tiles: tiles loaded straight into LDS, taps from a patch

@@ -112,8 +112,8 @@ THFloatTensor *thhip_process_images(THNETWORK *network, unsigned char **images, 
 void thhip_io_free(struct hipnet *hn);
 /* th_load.c */
 int thhip_load_error(void);
-/* hip_rt.hip: which XCD the workgroups of a residue of blockIdx.x % 8 run on (probed once); the flag a
- * kernel raises when it runs where it must not (an error at the next synchronisation) */
+/* hip_rt.hip: whether the GPU hands the workgroups of a launch to the XCDs in order (probed once); the flag
+ * a kernel raises when it finds that its launch was not (a repeat or an error at the next synchronisation) */
 unsigned thhip_xcd_map(void);
 int *thhip_fault_flag(void);
 /* hip_rt.hip: a caller that can repeat its forward pass holds the error of such a report back (1 / 0) and

@@ -14,7 +14,7 @@ hipStream_t thhip_stream(void);
 
 /* s_getreg operand of the XCC id (hardware register 20, bits 0 .. 3): the XCD this wave runs on */
 #define THHIP_GETREG_XCC_ID ((3 << 11) | 20)
-extern "C" unsigned thhip_xcd_map(void);	/* hip_rt.hip: which XCD the workgroups of a residue of blockIdx.x % 8 run on */
+extern "C" unsigned thhip_xcd_map(void);	/* hip_rt.hip: 0x80000000 | r where workgroup b of a probe launch ran on XCD (b + r) % 8 for every b; 0 otherwise */
 extern "C" int *thhip_fault_flag(void);		/* hip_rt.hip: set by a kernel, turned into an error at the next synchronisation */
 extern "C" void thhip_fault_hold(int on);	/* hip_rt.hip: 1: the error is held back for thhip_fault_take() */
 extern "C" int thhip_fault_take(void);		/* hip_rt.hip: the fault reported while errors were held back (0: none); clears it */
