@@ -26,12 +26,12 @@ void THInit(void)
 	 * no GPU is visible */
 	if (thhip_device_count() < 1)
 		THError("thnets HIP engine: no AMD GPU visible; this library has no CPU fallback");
-	/* the fixed partial-sum array of thhip_linear_batched_noalloc: look its address up now */
-	/* which XCD the workgroups of a grid run on (the convolutions add the K parts of cut tiles inside the
-	 * kernel only where that is as expected), and the flag kernels raise: probed and allocated now, not in
-	 * the first forward */
+	/* whether the GPU hands the workgroups of a launch to the XCDs in order (the convolutions add the K
+	 * parts of cut tiles inside the kernel only where it does), and the flag kernels raise: probed and
+	 * allocated now, not in the first forward */
 	thhip_xcd_map();
 	thhip_fault_flag();
+	/* the fixed partial-sum array of thhip_linear_batched_noalloc: look its address up now */
 	if (thhip_linear_batched_noalloc_init())	/* only that entry point is affected: it then returns -3 */
 		fprintf(stderr, "thnets HIP engine: the fixed device array of thhip_linear_batched_noalloc could not be "
 			"resolved; that call is unavailable\n");
